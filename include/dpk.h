@@ -1,0 +1,229 @@
+/*
+ * dpk.h - C ABI of libdpsgd_hip.so: the DP-SGD hot path (per-sample gradients,
+ * ghost-clipping per-sample norms, clip + accumulate + Gaussian noise) as
+ * hand-written HIP kernels for gfx950 (MI355X).
+ *
+ * Conventions shared by every entry point
+ *   - Plain C: pointers, sizes, scalars. No C++ or torch types cross the boundary.
+ *   - Every pointer is a DEVICE pointer unless its comment says "host".
+ *   - All tensors are dense, row-major, batch first; float tensors are 16-byte
+ *     aligned (bf16 too), id tensors are int64 and 8-byte aligned.
+ *   - Work is enqueued on `stream` (a hipStream_t passed as void*; NULL = the
+ *     null stream) and the call returns without waiting for it.
+ *   - The library never allocates or frees device memory: the caller passes
+ *     outputs and, where an entry point needs scratch, a workspace whose size
+ *     the matching dpk_*_workspace_bytes() query returns.
+ *   - Return value: DPK_OK (0) or a negative DPK_E_* code; dpk_last_error()
+ *     then holds a message for the calling thread. Nothing is launched when an
+ *     argument check fails. n == 0 returns DPK_OK without launching.
+ *   - `scale` multiplies the backprops on the fly. The reference multiplies the
+ *     backprops tensor by the batch size for a mean-reduced loss in a pass of
+ *     its own (opacus/grad_sample/grad_sample_module.py:402-406); pass 1.0f for
+ *     a sum-reduced loss.
+ *   - Reductions use a fixed order: the same inputs give the same bits.
+ */
+#ifndef DPK_H
+#define DPK_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* dpk_stream_t;
+
+enum dpk_status {
+  DPK_OK = 0,
+  DPK_E_SHAPE = -1,     /* a size is negative, zero where it may not be, or too large */
+  DPK_E_DTYPE = -2,     /* dtype code not supported by this entry point */
+  DPK_E_ALIGN = -3,     /* pointer not aligned as the conventions above require */
+  DPK_E_LAUNCH = -4,    /* the HIP runtime refused the launch */
+  DPK_E_WORKSPACE = -5, /* workspace missing or smaller than the query says */
+  DPK_E_ARG = -6        /* NULL where a pointer is required, or a bad flag */
+};
+
+enum dpk_dtype { DPK_F32 = 0, DPK_BF16 = 1 };
+
+#define DPK_MULTI_MAX 48 /* tensors per call of the *_multi entry points */
+
+/* ABI revision; bumped when a signature changes. */
+int dpk_abi_version(void);
+/* Message of the last failing call on this host thread ("" if none). */
+const char* dpk_last_error(void);
+/* Number of compute units of the current device (host query, cached per device). */
+int dpk_device_cus(void);
+
+/* ------------------------------------------------------------------------- *
+ * Per-sample gradients of nn.Linear
+ * replaces opacus/grad_sample/linear.py:29-51 (compute_linear_grad_sample)
+ * ------------------------------------------------------------------------- */
+
+/* gs[n,i,j] = scale * sum_t b[n,t,i] * a[n,t,j]          (linear.py:47)
+ * b: [n,T,out], a: [n,T,in] of `in_dtype`; gs: [n,out,in] of `gs_dtype`.
+ * sumsq (nullable, float[n]) receives sum_ij gs[n,i,j]^2 of the values as
+ * written (fp32 accumulators before any down-cast), so that the optimizer's
+ * norm pass (optimizers/optimizer.py:444-446) need not re-read gs.
+ * T == 1 takes a store-bound outer-product kernel; T > 1 an MFMA kernel.
+ * ws is needed only when sumsq != NULL. */
+size_t dpk_linear_gs_workspace_bytes(int64_t n, int64_t T, int64_t out, int64_t in);
+int dpk_linear_gs(const void* b, const void* a, int in_dtype, void* gs, int gs_dtype,
+                  float* sumsq, int64_t n, int64_t T, int64_t out, int64_t in, float scale,
+                  void* ws, size_t ws_bytes, dpk_stream_t stream);
+
+/* gs_bias[n,k] = scale * sum_t b[n,t,k]                   (linear.py:50) */
+int dpk_linear_bias_gs(const void* b, int in_dtype, void* gs_bias, int gs_dtype, int64_t n,
+                       int64_t T, int64_t out, float scale, dpk_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
+ * Ghost-clipping per-sample norms of nn.Linear
+ * replaces opacus/grad_sample/linear.py:54-93 (compute_linear_norm_sample)
+ * ------------------------------------------------------------------------- */
+
+/* norm_w[n] = sqrt(max(0, sum_{t,t'} (b_t.b_t')(a_t.a_t')))   (linear.py:83-89)
+ * norm_b[n] = sqrt(max(0, sum_{t,t'} b_t.b_t'))              (linear.py:91-92)
+ * For T == 1 these are the closed forms of linear.py:71-79.
+ * Either output may be NULL (parameter without requires_grad). Outputs are
+ * fp32 whatever `dtype` the inputs have. The T x T Gram matrices are never
+ * written to memory: matching tiles of b b^T and a a^T are formed in MFMA
+ * accumulators, multiplied and reduced in registers. */
+size_t dpk_linear_ghost_norm_workspace_bytes(int64_t n, int64_t T, int64_t out, int64_t in);
+int dpk_linear_ghost_norm(const void* b, const void* a, int dtype, float* norm_w, float* norm_b,
+                          int64_t n, int64_t T, int64_t out, int64_t in, float scale, void* ws,
+                          size_t ws_bytes, dpk_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
+ * Per-sample gradients of nn.Conv2d
+ * replaces opacus/grad_sample/conv.py:28-119 (compute_conv_grad_sample, the
+ * Conv2d branch) together with opacus/utils/tensor_utils.py:116-172 (unfold2d)
+ * ------------------------------------------------------------------------- */
+
+/* gs[n,o,c,kh,kw] = scale * sum_{oh,ow} b[n,o,oh,ow] *
+ *        xpad[n, g(o)*C/groups + c, oh*sh + kh*dh, ow*sw + kw*dw]
+ * x: [n,C,H,W], b: [n,O,OH,OW] (OH, OW follow from the geometry exactly as
+ * unfold2d computes H_effective/W_effective), gs: [n,O,C/groups,KH,KW].
+ * The unfolded activation matrix is never materialised. Padding is given per
+ * side so that padding="same" (asymmetric, tensor_utils.py:128-134) is
+ * expressible. sumsq as for dpk_linear_gs. fp32 only. */
+size_t dpk_conv2d_gs_workspace_bytes(int64_t n, int64_t C, int64_t O, int64_t KH, int64_t KW,
+                                     int64_t groups);
+int dpk_conv2d_gs(const void* x, const void* b, int in_dtype, void* gs, int gs_dtype, float* sumsq,
+                  int64_t n, int64_t C, int64_t H, int64_t W, int64_t O, int64_t KH, int64_t KW,
+                  int64_t sh, int64_t sw, int64_t ph_lo, int64_t ph_hi, int64_t pw_lo,
+                  int64_t pw_hi, int64_t dh, int64_t dw, int64_t groups, float scale, void* ws,
+                  size_t ws_bytes, dpk_stream_t stream);
+
+/* gs_bias[n,o] = scale * sum_q b[n,o,q]                    (conv.py:117)
+ * b: [n,O,q]. */
+int dpk_conv_bias_gs(const void* b, int in_dtype, void* gs_bias, int gs_dtype, int64_t n,
+                     int64_t O, int64_t q, float scale, dpk_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
+ * nn.Embedding
+ * replaces opacus/grad_sample/embedding.py:25-64 (compute_embedding_grad_sample)
+ * and opacus/grad_sample/embedding_norm_sample.py:27-151
+ * ------------------------------------------------------------------------- */
+
+/* The integer stage of embedding_norm_sample.py:116-129, bit-exact:
+ * the (row, id) pairs of ids[n,T] made unique in sorted order.
+ *   inverse[n*T]      position of pair (row(t), ids[t]) in the sorted unique list
+ *   unique_pairs[U,2] the list itself (only the first U rows are written)
+ *   n_unique[1]       U
+ * ids need not lie in any range here. */
+size_t dpk_embedding_workspace_bytes(int64_t n, int64_t T);
+int dpk_embedding_unique_pairs(const int64_t* ids, int64_t n, int64_t T, int64_t* inverse,
+                               int64_t* unique_pairs, int64_t* n_unique, void* ws,
+                               size_t ws_bytes, dpk_stream_t stream);
+
+/* gs[n,v,:] = scale * sum_{t : ids[n,t]==v} b[n,t,:]        (embedding.py:48-61)
+ * gs: [n,V,D] of gs_dtype, fully written (rows no id names are zero).
+ * Ids outside [0,V) make the call fail with DPK_E_ARG after a device-side
+ * check (the one entry point that waits for the stream). */
+int dpk_embedding_gs(const int64_t* ids, const void* b, int in_dtype, void* gs, int gs_dtype,
+                     int64_t n, int64_t T, int64_t V, int64_t D, float scale, void* ws,
+                     size_t ws_bytes, dpk_stream_t stream);
+
+/* norm[n] = sqrt(sum_{v} || scale * sum_{t : ids[n,t]==v} b[n,t,:] ||^2)
+ * (embedding_norm_sample.py:131-150). fp32 output. */
+int dpk_embedding_ghost_norm(const int64_t* ids, const void* b, int dtype, float* norm, int64_t n,
+                             int64_t T, int64_t D, float scale, void* ws, size_t ws_bytes,
+                             dpk_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
+ * Normalisation layers with an affine weight
+ * replaces opacus/grad_sample/group_norm.py:26-47 and rms_norm.py:27-47
+ * ------------------------------------------------------------------------- */
+
+/* gs_w[n,c] = scale * sum_s group_norm(x)[n,c,s] * b[n,c,s]   (group_norm.py:43-44)
+ * gs_b[n,c] = scale * sum_s b[n,c,s]                          (group_norm.py:46)
+ * x, b: [n,C,S]; normalisation without affine over each (n, group). Either
+ * output may be NULL. */
+int dpk_group_norm_gs(const void* x, const void* b, int in_dtype, void* gs_w, void* gs_b,
+                      int gs_dtype, int64_t n, int64_t C, int64_t S, int64_t groups, float eps,
+                      float scale, dpk_stream_t stream);
+
+/* gs_w[n,d] = scale * sum_t x[n,t,d] * rsqrt(mean_d x[n,t,:]^2 + eps) * b[n,t,d]
+ * (rms_norm.py:44-47). x, b: [n,T,D], D = number of normalised elements. */
+size_t dpk_rms_norm_gs_workspace_bytes(int64_t n, int64_t T, int64_t D);
+int dpk_rms_norm_gs(const void* x, const void* b, int in_dtype, void* gs_w, int gs_dtype,
+                    int64_t n, int64_t T, int64_t D, float eps, float scale, void* ws,
+                    size_t ws_bytes, dpk_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
+ * DPOptimizer.clip_and_accumulate, add_noise, scale_grad
+ * replaces opacus/optimizers/optimizer.py:432-504
+ * ------------------------------------------------------------------------- */
+
+/* sumsq[n] = sum_p gs[n,p]^2                                (optimizer.py:444-446)
+ * gs: [n,P]. */
+size_t dpk_sumsq_rows_workspace_bytes(int64_t n, int64_t P);
+int dpk_sumsq_rows(const void* gs, int dtype, int64_t n, int64_t P, float* sumsq, void* ws,
+                   size_t ws_bytes, dpk_stream_t stream);
+
+/* norm[n] = sqrt(sum_k sumsq[k,n]); clip[n] = min(1, C / (norm[n] + 1e-6))
+ * (optimizer.py:452-455; grad_sample_module_fast_gradient_clipping.py:137-150)
+ * sumsq: [K,n] squared per-parameter norms. With `is_norm` != 0 the input
+ * holds norms instead of squared norms (the ghost path stores norms).
+ * norm (nullable) and clip (nullable) are float[n]. */
+int dpk_clip_factor(const float* sumsq, int64_t K, int64_t n, int is_norm, float max_grad_norm,
+                    float* norm, float* clip, dpk_stream_t stream);
+
+/* summed[p] (+)= sum_n clip[n] * gs[n,p]                    (optimizer.py:464-473)
+ * gs: [n,P] of gs_dtype; summed: [P] of out_dtype; `accumulate` != 0 adds to
+ * what summed holds (optimizer.py:470-471), else overwrites. The n x P tensor
+ * is read exactly once. */
+int dpk_clip_accumulate(const void* gs, int gs_dtype, const float* clip, void* summed,
+                        int out_dtype, int64_t n, int64_t P, int accumulate, dpk_stream_t stream);
+
+/* The same two passes over up to DPK_MULTI_MAX parameters in one launch each:
+ * the per-parameter Python loop of optimizer.py:457-475 folded into the grid.
+ * Host arrays of K device pointers / sizes. All tensors share n and dtypes.
+ * dpk_sumsq_rows_multi writes sumsq[k*n + i]. */
+size_t dpk_sumsq_rows_multi_workspace_bytes(int64_t n, const int64_t* P /*host*/, int64_t K);
+int dpk_sumsq_rows_multi(const void* const* gs /*host*/, const int64_t* P /*host*/, int64_t K,
+                         int dtype, int64_t n, float* sumsq, void* ws, size_t ws_bytes,
+                         dpk_stream_t stream);
+int dpk_clip_accumulate_multi(const void* const* gs /*host*/, void* const* summed /*host*/,
+                              const int64_t* P /*host*/, int64_t K, int gs_dtype, int out_dtype,
+                              const float* clip, int64_t n, int accumulate, dpk_stream_t stream);
+
+/* grad[p] = (summed[p] + std * z[p]) / denom,  z ~ N(0,1)   (optimizer.py:485-504)
+ * Folds _generate_noise (optimizer.py:104-169), the add (:491) and scale_grad's
+ * division (:502-504) into one pass. std == 0 adds exact zeros and draws
+ * nothing (optimizer.py:139-140). z comes from Philox4x32-10 keyed by `seed`
+ * with counter (element index / 4, offset); `draws` = 1, or 4 for the
+ * reference's secure mode (sum of four normals halved, optimizer.py:150-160).
+ * A call consumes `draws` units of offset. grad may alias summed. */
+int dpk_add_noise(const void* summed, int in_dtype, void* grad, int out_dtype, int64_t P,
+                  float std, float denom, uint64_t seed, uint64_t offset, int draws,
+                  dpk_stream_t stream);
+
+/* out[p] = std * z[p]: the bare generator, for statistical tests. */
+int dpk_fill_normal(float* out, int64_t P, float std, uint64_t seed, uint64_t offset,
+                    dpk_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DPK_H */

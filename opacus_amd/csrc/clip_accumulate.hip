@@ -1,0 +1,357 @@
+// Streaming kernels behind DPOptimizer.clip_and_accumulate
+// (opacus/optimizers/optimizer.py:432-475): per-sample squared norms, the clip
+// factor, and the clip-weighted sum over the batch. All HBM-bound; each reads
+// the n x P per-sample gradient tensor exactly once, with 16-byte accesses that
+// are contiguous across a wavefront, and reduces in a fixed order.
+#include "dpk_common.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / DPK_WAVE;
+// Elements of one row handled by one block of the sum-of-squares kernel.
+constexpr int64_t kSumsqChunk = 8192;
+
+struct MultiArgs {
+  const void* gs[DPK_MULTI_MAX];
+  void* out[DPK_MULTI_MAX];
+  int64_t P[DPK_MULTI_MAX];
+  int64_t prefix[DPK_MULTI_MAX + 1];  // blocks (per row for sumsq) before tensor k
+  int K;
+};
+
+__device__ __forceinline__ int find_tensor(const MultiArgs& a, int64_t c) {
+  int k = 0;
+  while (k + 1 < a.K && c >= a.prefix[k + 1]) ++k;
+  return k;
+}
+
+// ---- sum of squares per row --------------------------------------------------
+// grid.x = n * CT where CT = prefix[K] = chunks per row summed over the tensors.
+// Block (row, c) reduces chunk c of that row to one float:
+//   ws[n * prefix[k] + row * nchunk_k + (c - prefix[k])].
+template <typename T, bool VEC>
+__global__ __launch_bounds__(kThreads) void sumsq_partial_kernel(MultiArgs a, int64_t n, float* ws) {
+  __shared__ float red[kWaves];
+  const int64_t CT = a.prefix[a.K];
+  const int64_t row = blockIdx.x / CT;
+  const int64_t c = blockIdx.x % CT;
+  const int k = find_tensor(a, c);
+  const int64_t P = a.P[k];
+  const int64_t nchunk = a.prefix[k + 1] - a.prefix[k];
+  const int64_t chunk = c - a.prefix[k];
+  const T* rowp = static_cast<const T*>(a.gs[k]) + row * P;
+  const int64_t lo = chunk * kSumsqChunk;
+  const int64_t hi = (lo + kSumsqChunk < P) ? lo + kSumsqChunk : P;
+  float acc0 = 0.f, acc1 = 0.f, acc2 = 0.f, acc3 = 0.f;
+  if (VEC) {
+    for (int64_t i = lo + threadIdx.x * 4; i < hi; i += kThreads * 4) {
+      float4 v = dpk_io<T>::load4(rowp + i);
+      acc0 += v.x * v.x;
+      acc1 += v.y * v.y;
+      acc2 += v.z * v.z;
+      acc3 += v.w * v.w;
+    }
+  } else {
+    for (int64_t i = lo + threadIdx.x; i < hi; i += kThreads) {
+      float v = dpk_io<T>::load(rowp + i);
+      acc0 += v * v;
+    }
+  }
+  float s = block_sum<kWaves>((acc0 + acc1) + (acc2 + acc3), red);
+  if (threadIdx.x == 0) ws[n * a.prefix[k] + row * nchunk + chunk] = s;
+}
+
+// One wave per (tensor, row): sumsq[k*n + row] = sum of that row's partials.
+__global__ __launch_bounds__(kThreads) void sumsq_final_kernel(MultiArgs a, int64_t n,
+                                                                 const float* ws, float* sumsq) {
+  const int64_t w = (static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x) / DPK_WAVE;
+  const int lane = threadIdx.x & (DPK_WAVE - 1);
+  if (w >= static_cast<int64_t>(a.K) * n) return;
+  const int k = static_cast<int>(w / n);
+  const int64_t row = w % n;
+  const int64_t nchunk = a.prefix[k + 1] - a.prefix[k];
+  const float* p = ws + n * a.prefix[k] + row * nchunk;
+  float s = 0.f;
+  for (int64_t i = lane; i < nchunk; i += DPK_WAVE) s += p[i];
+  s = wave_sum(s);
+  if (lane == 0) sumsq[w] = s;
+}
+
+// ---- clip factor -----------------------------------------------------------
+__global__ void clip_factor_kernel(const float* __restrict__ v, int64_t K, int64_t n, int is_norm,
+                                   float C, float* __restrict__ norm, float* __restrict__ clip) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  float s = 0.f;
+  for (int64_t k = 0; k < K; ++k) {
+    float x = v[k * n + i];
+    s += is_norm ? x * x : x;
+  }
+  const float nr = sqrtf(s);
+  if (norm) norm[i] = nr;
+  if (clip) clip[i] = fminf(C / (nr + 1e-6f), 1.0f);
+}
+
+// ---- clip-weighted sum over the batch ----------------------------------------
+// A block owns (kThreads / RS) * W consecutive columns of one tensor (W = 4
+// with VEC, else 1). Thread (cx, ry) walks rows ry, ry+RS, ... of its columns;
+// the RS partial sums meet in LDS in a fixed order. RS = 1 is the streaming
+// shape for large P; RS > 1 keeps the chip busy when P is small and n large.
+template <typename TG, typename TO, bool VEC, int RS>
+__global__ __launch_bounds__(kThreads) void clip_accumulate_kernel(MultiArgs a, int64_t n,
+                                                                     const float* __restrict__ clip,
+                                                                     int accumulate) {
+  constexpr int W = VEC ? 4 : 1;
+  constexpr int CX = kThreads / RS;
+  __shared__ float4 part[RS > 1 ? kThreads : 1];
+  const int k = find_tensor(a, blockIdx.x);
+  const int64_t P = a.P[k];
+  const int64_t blk = blockIdx.x - a.prefix[k];
+  const int cx = threadIdx.x % CX;
+  const int ry = threadIdx.x / CX;
+  const int64_t col = (blk * CX + cx) * W;
+  const bool live = col < P;
+  const TG* base = static_cast<const TG*>(a.gs[k]) + col;
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (live) {
+    constexpr int U = 8;
+    int64_t r = ry;
+    for (; r + (U - 1) * RS < n; r += U * RS) {
+      float4 v[U];
+      float c[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const TG* p = base + (r + u * RS) * P;
+        if (VEC) {
+          v[u] = dpk_io<TG>::load4(p);
+        } else {
+          v[u] = make_float4(dpk_io<TG>::load(p), 0.f, 0.f, 0.f);
+        }
+        c[u] = clip[r + u * RS];
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        acc.x = fmaf(c[u], v[u].x, acc.x);
+        if (VEC) {
+          acc.y = fmaf(c[u], v[u].y, acc.y);
+          acc.z = fmaf(c[u], v[u].z, acc.z);
+          acc.w = fmaf(c[u], v[u].w, acc.w);
+        }
+      }
+    }
+    for (; r < n; r += RS) {
+      const TG* p = base + r * P;
+      const float c = clip[r];
+      if (VEC) {
+        float4 v = dpk_io<TG>::load4(p);
+        acc.x = fmaf(c, v.x, acc.x);
+        acc.y = fmaf(c, v.y, acc.y);
+        acc.z = fmaf(c, v.z, acc.z);
+        acc.w = fmaf(c, v.w, acc.w);
+      } else {
+        acc.x = fmaf(c, dpk_io<TG>::load(p), acc.x);
+      }
+    }
+  }
+  if (RS > 1) {
+    part[threadIdx.x] = acc;
+    __syncthreads();
+    if (ry != 0) return;
+#pragma unroll
+    for (int j = 1; j < RS; ++j) {
+      float4 o = part[j * CX + cx];
+      acc.x += o.x;
+      acc.y += o.y;
+      acc.z += o.z;
+      acc.w += o.w;
+    }
+  }
+  if (!live) return;
+  TO* out = static_cast<TO*>(a.out[k]) + col;
+  if (VEC) {
+    if (accumulate) {
+      float4 o = dpk_io<TO>::load4(out);
+      acc.x += o.x;
+      acc.y += o.y;
+      acc.z += o.z;
+      acc.w += o.w;
+    }
+    dpk_io<TO>::store4(out, acc);
+  } else {
+    if (accumulate) acc.x += dpk_io<TO>::load(out);
+    dpk_io<TO>::store(out, acc.x);
+  }
+}
+
+template <typename TG, typename TO, bool VEC, int RS>
+void launch_clip_accumulate(const MultiArgs& a, int64_t blocks, int64_t n, const float* clip,
+                            int accumulate, hipStream_t s) {
+  hipLaunchKernelGGL((clip_accumulate_kernel<TG, TO, VEC, RS>), dim3(static_cast<unsigned>(blocks)),
+                     dim3(kThreads), 0, s, a, n, clip, accumulate);
+}
+
+template <typename TG, typename TO>
+void dispatch_clip_accumulate(MultiArgs& a, const int64_t* P, int K, int64_t n, const float* clip,
+                              int accumulate, bool vec, int rs, hipStream_t s, int64_t* blocks_out) {
+  const int W = vec ? 4 : 1;
+  const int64_t cols_per_block = static_cast<int64_t>(kThreads / rs) * W;
+  a.prefix[0] = 0;
+  for (int k = 0; k < K; ++k) a.prefix[k + 1] = a.prefix[k] + dpk_cdiv(P[k], cols_per_block);
+  const int64_t blocks = a.prefix[K];
+  *blocks_out = blocks;
+  if (blocks == 0 || blocks > DPK_MAX_GRID_X) return;
+  if (vec) {
+    if (rs == 1) launch_clip_accumulate<TG, TO, true, 1>(a, blocks, n, clip, accumulate, s);
+    else launch_clip_accumulate<TG, TO, true, 16>(a, blocks, n, clip, accumulate, s);
+  } else {
+    if (rs == 1) launch_clip_accumulate<TG, TO, false, 1>(a, blocks, n, clip, accumulate, s);
+    else launch_clip_accumulate<TG, TO, false, 16>(a, blocks, n, clip, accumulate, s);
+  }
+}
+
+int fill_sumsq_args(MultiArgs& a, const void* const* gs, const int64_t* P, int64_t K, int dtype,
+                    bool* vec, const char* who) {
+  DPK_REQUIRE(gs && P, DPK_E_ARG, "%s: NULL pointer table", who);
+  DPK_REQUIRE(K >= 1 && K <= DPK_MULTI_MAX, DPK_E_SHAPE, "%s: K=%lld not in [1,%d]", who,
+              (long long)K, DPK_MULTI_MAX);
+  DPK_REQUIRE(dpk_dtype_ok(dtype), DPK_E_DTYPE, "%s: dtype %d", who, dtype);
+  const size_t need = dtype == DPK_BF16 ? 8 : 16;
+  *vec = true;
+  a.K = static_cast<int>(K);
+  a.prefix[0] = 0;
+  for (int k = 0; k < K; ++k) {
+    DPK_REQUIRE(P[k] >= 1, DPK_E_SHAPE, "%s: P[%d]=%lld", who, k, (long long)P[k]);
+    DPK_REQUIRE(gs[k], DPK_E_ARG, "%s: gs[%d] is NULL", who, k);
+    DPK_REQUIRE(dpk_aligned(gs[k], dpk_elsize(dtype)), DPK_E_ALIGN, "%s: gs[%d] misaligned", who, k);
+    if (P[k] % 4 != 0 || !dpk_aligned(gs[k], need)) *vec = false;
+    a.gs[k] = gs[k];
+    a.out[k] = nullptr;
+    a.P[k] = P[k];
+    a.prefix[k + 1] = a.prefix[k] + dpk_cdiv(P[k], kSumsqChunk);
+  }
+  return DPK_OK;
+}
+
+}  // namespace
+
+extern "C" size_t dpk_sumsq_rows_multi_workspace_bytes(int64_t n, const int64_t* P, int64_t K) {
+  if (n <= 0 || !P || K <= 0) return 0;
+  int64_t ct = 0;
+  for (int64_t k = 0; k < K; ++k) ct += dpk_cdiv(P[k] > 0 ? P[k] : 0, kSumsqChunk);
+  return dpk_align_up(static_cast<size_t>(n) * ct * sizeof(float), 256);
+}
+
+extern "C" size_t dpk_sumsq_rows_workspace_bytes(int64_t n, int64_t P) {
+  return dpk_sumsq_rows_multi_workspace_bytes(n, &P, 1);
+}
+
+extern "C" int dpk_sumsq_rows_multi(const void* const* gs, const int64_t* P, int64_t K, int dtype,
+                                    int64_t n, float* sumsq, void* ws, size_t ws_bytes,
+                                    dpk_stream_t stream) {
+  const char* who = "dpk_sumsq_rows_multi";
+  DPK_REQUIRE(n >= 0, DPK_E_SHAPE, "%s: n=%lld", who, (long long)n);
+  if (n == 0) return DPK_OK;
+  MultiArgs a;
+  bool vec;
+  int rc = fill_sumsq_args(a, gs, P, K, dtype, &vec, who);
+  if (rc != DPK_OK) return rc;
+  DPK_REQUIRE(sumsq, DPK_E_ARG, "%s: sumsq is NULL", who);
+  const size_t need = dpk_sumsq_rows_multi_workspace_bytes(n, P, K);
+  DPK_REQUIRE(ws && ws_bytes >= need, DPK_E_WORKSPACE, "%s: workspace %zu < %zu bytes", who,
+              ws_bytes, need);
+  DPK_REQUIRE(dpk_aligned(ws, 4), DPK_E_ALIGN, "%s: workspace misaligned", who);
+  const int64_t blocks = n * a.prefix[K];
+  DPK_REQUIRE(blocks <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: %lld blocks exceed the grid limit", who,
+              (long long)blocks);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  float* wsf = static_cast<float*>(ws);
+  dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
+  if (dtype == DPK_F32) {
+    if (vec) hipLaunchKernelGGL((sumsq_partial_kernel<float, true>), grid, block, 0, s, a, n, wsf);
+    else hipLaunchKernelGGL((sumsq_partial_kernel<float, false>), grid, block, 0, s, a, n, wsf);
+  } else {
+    if (vec) hipLaunchKernelGGL((sumsq_partial_kernel<bf16_t, true>), grid, block, 0, s, a, n, wsf);
+    else hipLaunchKernelGGL((sumsq_partial_kernel<bf16_t, false>), grid, block, 0, s, a, n, wsf);
+  }
+  DPK_LAUNCH_CHECK(who);
+  const int64_t waves = K * n;
+  hipLaunchKernelGGL(sumsq_final_kernel, dim3(static_cast<unsigned>(dpk_cdiv(waves, kWaves))), block,
+                     0, s, a, n, wsf, sumsq);
+  DPK_LAUNCH_CHECK(who);
+  return DPK_OK;
+}
+
+extern "C" int dpk_sumsq_rows(const void* gs, int dtype, int64_t n, int64_t P, float* sumsq,
+                              void* ws, size_t ws_bytes, dpk_stream_t stream) {
+  return dpk_sumsq_rows_multi(&gs, &P, 1, dtype, n, sumsq, ws, ws_bytes, stream);
+}
+
+extern "C" int dpk_clip_factor(const float* sumsq, int64_t K, int64_t n, int is_norm,
+                               float max_grad_norm, float* norm, float* clip, dpk_stream_t stream) {
+  const char* who = "dpk_clip_factor";
+  DPK_REQUIRE(n >= 0 && K >= 1, DPK_E_SHAPE, "%s: K=%lld n=%lld", who, (long long)K, (long long)n);
+  if (n == 0) return DPK_OK;
+  DPK_REQUIRE(sumsq, DPK_E_ARG, "%s: input is NULL", who);
+  DPK_REQUIRE(norm || clip, DPK_E_ARG, "%s: both outputs are NULL", who);
+  hipLaunchKernelGGL(clip_factor_kernel, dim3(static_cast<unsigned>(dpk_cdiv(n, 256))), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), sumsq, K, n, is_norm, max_grad_norm, norm, clip);
+  DPK_LAUNCH_CHECK(who);
+  return DPK_OK;
+}
+
+extern "C" int dpk_clip_accumulate_multi(const void* const* gs, void* const* summed,
+                                         const int64_t* P, int64_t K, int gs_dtype, int out_dtype,
+                                         const float* clip, int64_t n, int accumulate,
+                                         dpk_stream_t stream) {
+  const char* who = "dpk_clip_accumulate_multi";
+  DPK_REQUIRE(n >= 0, DPK_E_SHAPE, "%s: n=%lld", who, (long long)n);
+  DPK_REQUIRE(gs && summed && P, DPK_E_ARG, "%s: NULL pointer table", who);
+  DPK_REQUIRE(K >= 1 && K <= DPK_MULTI_MAX, DPK_E_SHAPE, "%s: K=%lld not in [1,%d]", who,
+              (long long)K, DPK_MULTI_MAX);
+  DPK_REQUIRE(dpk_dtype_ok(gs_dtype) && dpk_dtype_ok(out_dtype), DPK_E_DTYPE, "%s: dtypes %d,%d",
+              who, gs_dtype, out_dtype);
+  DPK_REQUIRE(n == 0 || clip, DPK_E_ARG, "%s: clip is NULL", who);
+  MultiArgs a;
+  a.K = static_cast<int>(K);
+  bool vec = true;
+  int64_t ptotal = 0;
+  const size_t gneed = gs_dtype == DPK_BF16 ? 8 : 16, oneed = out_dtype == DPK_BF16 ? 8 : 16;
+  for (int k = 0; k < K; ++k) {
+    DPK_REQUIRE(P[k] >= 1, DPK_E_SHAPE, "%s: P[%d]=%lld", who, k, (long long)P[k]);
+    DPK_REQUIRE(summed[k] && (n == 0 || gs[k]), DPK_E_ARG, "%s: tensor %d is NULL", who, k);
+    DPK_REQUIRE(dpk_aligned(gs[k], dpk_elsize(gs_dtype)) && dpk_aligned(summed[k], dpk_elsize(out_dtype)),
+                DPK_E_ALIGN, "%s: tensor %d misaligned", who, k);
+    if (P[k] % 4 != 0 || !dpk_aligned(gs[k], gneed) || !dpk_aligned(summed[k], oneed)) vec = false;
+    a.gs[k] = gs[k];
+    a.out[k] = summed[k];
+    a.P[k] = P[k];
+    ptotal += P[k];
+  }
+  // An empty batch contributes a zero sum: with accumulate nothing changes,
+  // without it the kernel's row loop runs zero times and writes zeros.
+  if (n == 0 && accumulate) return DPK_OK;
+  // Split the rows inside a block when the columns alone cannot fill the chip.
+  const int rs = (ptotal / (vec ? 4 : 1) < 256LL * 1024 && n >= 64) ? 16 : 1;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  int64_t blocks = 0;
+  if (gs_dtype == DPK_F32 && out_dtype == DPK_F32)
+    dispatch_clip_accumulate<float, float>(a, P, (int)K, n, clip, accumulate, vec, rs, s, &blocks);
+  else if (gs_dtype == DPK_BF16 && out_dtype == DPK_F32)
+    dispatch_clip_accumulate<bf16_t, float>(a, P, (int)K, n, clip, accumulate, vec, rs, s, &blocks);
+  else if (gs_dtype == DPK_F32 && out_dtype == DPK_BF16)
+    dispatch_clip_accumulate<float, bf16_t>(a, P, (int)K, n, clip, accumulate, vec, rs, s, &blocks);
+  else
+    dispatch_clip_accumulate<bf16_t, bf16_t>(a, P, (int)K, n, clip, accumulate, vec, rs, s, &blocks);
+  DPK_REQUIRE(blocks <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: %lld blocks exceed the grid limit", who,
+              (long long)blocks);
+  DPK_LAUNCH_CHECK(who);
+  return DPK_OK;
+}
+
+extern "C" int dpk_clip_accumulate(const void* gs, int gs_dtype, const float* clip, void* summed,
+                                   int out_dtype, int64_t n, int64_t P, int accumulate,
+                                   dpk_stream_t stream) {
+  return dpk_clip_accumulate_multi(&gs, &summed, &P, 1, gs_dtype, out_dtype, clip, n, accumulate,
+                                   stream);
+}

@@ -1,0 +1,319 @@
+// Per-sample gradients of nn.Linear (opacus/grad_sample/linear.py:29-51).
+//   weight: gs[n,i,j] = scale * sum_t b[n,t,i] * a[n,t,j]     (linear.py:47)
+//   bias:   gs[n,k]   = scale * sum_t b[n,t,k]                (linear.py:50)
+// T == 1 is a rank-1 outer product per sample: no contraction, the kernel is
+// bound by the n*out*in store stream. T > 1 is a batched GEMM with K = T on the
+// fp32 MFMA path (bf16 inputs are widened on the way into LDS, which is exact).
+// Both kernels also emit the per-sample sum of squares of what they wrote, as
+// one partial per block reduced in a fixed order, so the optimizer's norm pass
+// over the n*out*in tensor disappears.
+#include "dpk_common.h"
+#include "mfma_f32.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / DPK_WAVE;
+constexpr int kOuterRows = 64;  // rows of one sample's gs written by one block (T == 1)
+
+// ---- T == 1 ------------------------------------------------------------------
+// Block = CX column threads x (256 / CX) row groups; a thread keeps its 4 (or 1)
+// activations in registers and walks the block's rows. Each row of the block is
+// a contiguous run of CX*W floats.
+template <typename TIN, typename TOUT, bool VEC>
+__global__ __launch_bounds__(kThreads) void linear_outer_kernel(
+    const TIN* __restrict__ b, const TIN* __restrict__ a, TOUT* __restrict__ gs,
+    float* __restrict__ partials, int64_t M, int64_t N, float scale, int cx_log2, int64_t tiles_m,
+    int64_t tiles_n) {
+  constexpr int W = VEC ? 4 : 1;
+  __shared__ float red[kWaves];
+  const int CX = 1 << cx_log2, RY = kThreads >> cx_log2;
+  const int cx = threadIdx.x & (CX - 1), ry = threadIdx.x >> cx_log2;
+  const int64_t per_sample = tiles_m * tiles_n;
+  const int64_t sample = blockIdx.x / per_sample;
+  const int64_t rem = blockIdx.x % per_sample;
+  const int64_t i0 = (rem / tiles_n) * kOuterRows;
+  const int64_t j = ((rem % tiles_n) * CX + cx) * W;
+  const TIN* bs = b + sample * M;
+  TOUT* out = gs + sample * M * N;
+  float ss = 0.f;
+  if (j < N) {
+    float4 av = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (VEC) av = dpk_io<TIN>::load4(a + sample * N + j);
+    else av.x = dpk_io<TIN>::load(a + sample * N + j);
+    const float a2 = VEC ? (av.x * av.x + av.y * av.y) + (av.z * av.z + av.w * av.w) : av.x * av.x;
+    const int64_t iend = (i0 + kOuterRows < M) ? i0 + kOuterRows : M;
+    float b2 = 0.f;
+    for (int64_t i = i0 + ry; i < iend; i += RY) {
+      const float bv = scale * dpk_io<TIN>::load(bs + i);
+      b2 = fmaf(bv, bv, b2);
+      if (VEC) dpk_io<TOUT>::store4(out + i * N + j, make_float4(bv * av.x, bv * av.y, bv * av.z, bv * av.w));
+      else dpk_io<TOUT>::store(out + i * N + j, bv * av.x);
+    }
+    ss = a2 * b2;
+  }
+  if (partials) {
+    const float s = block_sum<kWaves>(ss, red);
+    if (threadIdx.x == 0) partials[blockIdx.x] = s;
+  }
+}
+
+// ---- T > 1 -------------------------------------------------------------------
+template <int BM, int BN, typename TIN, typename TOUT, bool VEC>
+__global__ __launch_bounds__(kThreads) void linear_mfma_kernel(
+    const TIN* __restrict__ b, const TIN* __restrict__ a, TOUT* __restrict__ gs,
+    float* __restrict__ partials, int64_t T, int64_t M, int64_t N, float scale, int64_t tiles_m,
+    int64_t tiles_n) {
+  __shared__ mf32::Smem<BM, BN> sm;
+  __shared__ float red[kWaves];
+  const int64_t per_sample = tiles_m * tiles_n;
+  const int64_t sample = blockIdx.x / per_sample;
+  const int64_t rem = blockIdx.x % per_sample;
+  const int64_t m0 = (rem / tiles_n) * BM, n0 = (rem % tiles_n) * BN;
+  mf32::LoaderMContig<BM, TIN, VEC> la(b + sample * T * M, M, m0, M, T);
+  mf32::LoaderMContig<BN, TIN, VEC> lb(a + sample * T * N, N, n0, N, T);
+  mf32::Tile<BM, BN> tile;
+  tile.clear();
+  mf32::mainloop<BM, BN>(tile, sm, la, lb, T);
+  TOUT* out = gs + sample * M * N;
+  float ss = 0.f;
+  tile.for_each([&](int r, int c, float v) {
+    const int64_t i = m0 + r, j = n0 + c;
+    if (i < M && j < N) {
+      const float x = v * scale;
+      dpk_io<TOUT>::store(out + i * N + j, x);
+      ss = fmaf(x, x, ss);
+    }
+  });
+  if (partials) {
+    const float s = block_sum<kWaves>(ss, red);
+    if (threadIdx.x == 0) partials[blockIdx.x] = s;
+  }
+}
+
+// ---- bias / row sums -----------------------------------------------------------
+// out[n,k] = scale * sum_t b[n,t,k]; threads along k, RS row groups along t.
+template <typename TIN, typename TOUT, int RS>
+__global__ __launch_bounds__(kThreads) void colsum_kernel(const TIN* __restrict__ b,
+                                                            TOUT* __restrict__ out, int64_t T,
+                                                            int64_t Kdim, float scale,
+                                                            int64_t blocks_per_sample) {
+  constexpr int CX = kThreads / RS;
+  __shared__ float part[kThreads];
+  const int64_t sample = blockIdx.x / blocks_per_sample;
+  const int64_t k = (blockIdx.x % blocks_per_sample) * CX + threadIdx.x % CX;
+  const int ry = threadIdx.x / CX;
+  float acc = 0.f;
+  if (k < Kdim) {
+    const TIN* p = b + sample * T * Kdim + k;
+    for (int64_t t = ry; t < T; t += RS) acc += dpk_io<TIN>::load(p + t * Kdim);
+  }
+  if (RS > 1) {
+    part[threadIdx.x] = acc;
+    __syncthreads();
+    if (ry != 0) return;
+#pragma unroll
+    for (int j = 1; j < RS; ++j) acc += part[j * CX + threadIdx.x];
+  }
+  if (k < Kdim) dpk_io<TOUT>::store(out + sample * Kdim + k, acc * scale);
+}
+
+// out[r] = scale * sum_q b[r,q]: one wave per row (conv bias, conv.py:117).
+template <typename TIN, typename TOUT>
+__global__ __launch_bounds__(kThreads) void rowsum_kernel(const TIN* __restrict__ b,
+                                                            TOUT* __restrict__ out, int64_t rows,
+                                                            int64_t q, float scale) {
+  const int64_t w = (static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x) / DPK_WAVE;
+  const int lane = threadIdx.x & (DPK_WAVE - 1);
+  if (w >= rows) return;
+  const TIN* p = b + w * q;
+  float s = 0.f;
+  for (int64_t i = lane; i < q; i += DPK_WAVE) s += dpk_io<TIN>::load(p + i);
+  s = wave_sum(s);
+  if (lane == 0) dpk_io<TOUT>::store(out + w, s * scale);
+}
+
+struct Plan {
+  bool outer;
+  int cx_log2;
+  int bm;
+  int64_t tiles_m, tiles_n;
+};
+
+Plan make_plan(int64_t T, int64_t M, int64_t N, bool vec) {
+  Plan p;
+  p.outer = (T == 1);
+  if (p.outer) {
+    const int64_t cols = dpk_cdiv(N, vec ? 4 : 1);
+    int lg = 3;  // at least 8 column threads
+    while (lg < 8 && (1LL << lg) < cols) ++lg;
+    p.cx_log2 = lg;
+    p.bm = 0;
+    p.tiles_m = dpk_cdiv(M, kOuterRows);
+    p.tiles_n = dpk_cdiv(cols, 1LL << lg);
+  } else {
+    p.cx_log2 = 0;
+    p.bm = (M > 64 && N > 64) ? 128 : 64;
+    p.tiles_m = dpk_cdiv(M, p.bm);
+    p.tiles_n = dpk_cdiv(N, p.bm);
+  }
+  return p;
+}
+
+template <typename TIN, typename TOUT>
+void launch_linear(const Plan& p, bool vec, const void* b, const void* a, void* gs, float* partials,
+                   int64_t n, int64_t T, int64_t M, int64_t N, float scale, hipStream_t s) {
+  const dim3 grid(static_cast<unsigned>(n * p.tiles_m * p.tiles_n)), block(kThreads);
+  const TIN* bp = static_cast<const TIN*>(b);
+  const TIN* ap = static_cast<const TIN*>(a);
+  TOUT* gp = static_cast<TOUT*>(gs);
+  if (p.outer) {
+    if (vec)
+      hipLaunchKernelGGL((linear_outer_kernel<TIN, TOUT, true>), grid, block, 0, s, bp, ap, gp,
+                         partials, M, N, scale, p.cx_log2, p.tiles_m, p.tiles_n);
+    else
+      hipLaunchKernelGGL((linear_outer_kernel<TIN, TOUT, false>), grid, block, 0, s, bp, ap, gp,
+                         partials, M, N, scale, p.cx_log2, p.tiles_m, p.tiles_n);
+  } else if (p.bm == 128) {
+    if (vec)
+      hipLaunchKernelGGL((linear_mfma_kernel<128, 128, TIN, TOUT, true>), grid, block, 0, s, bp, ap,
+                         gp, partials, T, M, N, scale, p.tiles_m, p.tiles_n);
+    else
+      hipLaunchKernelGGL((linear_mfma_kernel<128, 128, TIN, TOUT, false>), grid, block, 0, s, bp, ap,
+                         gp, partials, T, M, N, scale, p.tiles_m, p.tiles_n);
+  } else {
+    if (vec)
+      hipLaunchKernelGGL((linear_mfma_kernel<64, 64, TIN, TOUT, true>), grid, block, 0, s, bp, ap,
+                         gp, partials, T, M, N, scale, p.tiles_m, p.tiles_n);
+    else
+      hipLaunchKernelGGL((linear_mfma_kernel<64, 64, TIN, TOUT, false>), grid, block, 0, s, bp, ap,
+                         gp, partials, T, M, N, scale, p.tiles_m, p.tiles_n);
+  }
+}
+
+bool linear_vec(const void* b, const void* a, const void* gs, int in_dtype, int gs_dtype, int64_t M,
+                int64_t N) {
+  const size_t ia = in_dtype == DPK_BF16 ? 8 : 16, oa = gs_dtype == DPK_BF16 ? 8 : 16;
+  return M % 4 == 0 && N % 4 == 0 && dpk_aligned(b, ia) && dpk_aligned(a, ia) && dpk_aligned(gs, oa);
+}
+
+}  // namespace
+
+extern "C" size_t dpk_linear_gs_workspace_bytes(int64_t n, int64_t T, int64_t out, int64_t in) {
+  if (n <= 0 || T <= 0 || out <= 0 || in <= 0) return 0;
+  // The scalar plan never has fewer blocks than the vector plan.
+  const Plan p = make_plan(T, out, in, false);
+  return dpk_align_up(static_cast<size_t>(n * p.tiles_m * p.tiles_n) * sizeof(float), 256);
+}
+
+extern "C" int dpk_linear_gs(const void* b, const void* a, int in_dtype, void* gs, int gs_dtype,
+                             float* sumsq, int64_t n, int64_t T, int64_t out, int64_t in,
+                             float scale, void* ws, size_t ws_bytes, dpk_stream_t stream) {
+  const char* who = "dpk_linear_gs";
+  DPK_REQUIRE(n >= 0 && T >= 1 && out >= 1 && in >= 1, DPK_E_SHAPE,
+              "%s: n=%lld T=%lld out=%lld in=%lld", who, (long long)n, (long long)T, (long long)out,
+              (long long)in);
+  if (n == 0) return DPK_OK;
+  DPK_REQUIRE(b && a && gs, DPK_E_ARG, "%s: NULL tensor", who);
+  DPK_REQUIRE(dpk_dtype_ok(in_dtype) && dpk_dtype_ok(gs_dtype), DPK_E_DTYPE, "%s: dtypes %d,%d", who,
+              in_dtype, gs_dtype);
+  DPK_REQUIRE(dpk_aligned(b, dpk_elsize(in_dtype)) && dpk_aligned(a, dpk_elsize(in_dtype)) &&
+                  dpk_aligned(gs, dpk_elsize(gs_dtype)),
+              DPK_E_ALIGN, "%s: misaligned tensor", who);
+  const bool vec = linear_vec(b, a, gs, in_dtype, gs_dtype, out, in);
+  const Plan p = make_plan(T, out, in, vec);
+  const int64_t blocks = n * p.tiles_m * p.tiles_n;
+  DPK_REQUIRE(blocks <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: %lld blocks exceed the grid limit", who,
+              (long long)blocks);
+  float* partials = nullptr;
+  if (sumsq) {
+    const size_t need = static_cast<size_t>(blocks) * sizeof(float);
+    DPK_REQUIRE(ws && ws_bytes >= need, DPK_E_WORKSPACE, "%s: workspace %zu < %zu bytes", who,
+                ws_bytes, need);
+    DPK_REQUIRE(dpk_aligned(ws, 4), DPK_E_ALIGN, "%s: workspace misaligned", who);
+    partials = static_cast<float*>(ws);
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (in_dtype == DPK_F32 && gs_dtype == DPK_F32)
+    launch_linear<float, float>(p, vec, b, a, gs, partials, n, T, out, in, scale, s);
+  else if (in_dtype == DPK_BF16 && gs_dtype == DPK_BF16)
+    launch_linear<bf16_t, bf16_t>(p, vec, b, a, gs, partials, n, T, out, in, scale, s);
+  else if (in_dtype == DPK_BF16 && gs_dtype == DPK_F32)
+    launch_linear<bf16_t, float>(p, vec, b, a, gs, partials, n, T, out, in, scale, s);
+  else
+    launch_linear<float, bf16_t>(p, vec, b, a, gs, partials, n, T, out, in, scale, s);
+  DPK_LAUNCH_CHECK(who);
+  if (sumsq) {
+    dpk_launch_reduce_rows(partials, n, p.tiles_m * p.tiles_n, sumsq, 0, 1.f, s);
+    DPK_LAUNCH_CHECK(who);
+  }
+  return DPK_OK;
+}
+
+namespace {
+template <typename TIN, typename TOUT>
+void launch_colsum(const void* b, void* out, int64_t n, int64_t T, int64_t K, float scale,
+                   hipStream_t s) {
+  // Split the t loop inside the block when there are few columns to go round.
+  if (n * K < 64 * 1024 && T >= 32) {
+    const int64_t bps = dpk_cdiv(K, kThreads / 16);
+    hipLaunchKernelGGL((colsum_kernel<TIN, TOUT, 16>), dim3(static_cast<unsigned>(n * bps)),
+                       dim3(kThreads), 0, s, static_cast<const TIN*>(b), static_cast<TOUT*>(out), T,
+                       K, scale, bps);
+  } else {
+    const int64_t bps = dpk_cdiv(K, kThreads);
+    hipLaunchKernelGGL((colsum_kernel<TIN, TOUT, 1>), dim3(static_cast<unsigned>(n * bps)),
+                       dim3(kThreads), 0, s, static_cast<const TIN*>(b), static_cast<TOUT*>(out), T,
+                       K, scale, bps);
+  }
+}
+template <typename TIN, typename TOUT>
+void launch_rowsum(const void* b, void* out, int64_t rows, int64_t q, float scale, hipStream_t s) {
+  hipLaunchKernelGGL((rowsum_kernel<TIN, TOUT>), dim3(static_cast<unsigned>(dpk_cdiv(rows, kWaves))),
+                     dim3(kThreads), 0, s, static_cast<const TIN*>(b), static_cast<TOUT*>(out), rows,
+                     q, scale);
+}
+}  // namespace
+
+extern "C" int dpk_linear_bias_gs(const void* b, int in_dtype, void* gs_bias, int gs_dtype,
+                                  int64_t n, int64_t T, int64_t out, float scale,
+                                  dpk_stream_t stream) {
+  const char* who = "dpk_linear_bias_gs";
+  DPK_REQUIRE(n >= 0 && T >= 1 && out >= 1, DPK_E_SHAPE, "%s: n=%lld T=%lld out=%lld", who,
+              (long long)n, (long long)T, (long long)out);
+  if (n == 0) return DPK_OK;
+  DPK_REQUIRE(b && gs_bias, DPK_E_ARG, "%s: NULL tensor", who);
+  DPK_REQUIRE(dpk_dtype_ok(in_dtype) && dpk_dtype_ok(gs_dtype), DPK_E_DTYPE, "%s: dtypes %d,%d", who,
+              in_dtype, gs_dtype);
+  DPK_REQUIRE(dpk_aligned(b, dpk_elsize(in_dtype)) && dpk_aligned(gs_bias, dpk_elsize(gs_dtype)),
+              DPK_E_ALIGN, "%s: misaligned tensor", who);
+  DPK_REQUIRE(n * dpk_cdiv(out, 16) <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: too many blocks", who);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (in_dtype == DPK_F32 && gs_dtype == DPK_F32) launch_colsum<float, float>(b, gs_bias, n, T, out, scale, s);
+  else if (in_dtype == DPK_BF16 && gs_dtype == DPK_BF16) launch_colsum<bf16_t, bf16_t>(b, gs_bias, n, T, out, scale, s);
+  else if (in_dtype == DPK_BF16 && gs_dtype == DPK_F32) launch_colsum<bf16_t, float>(b, gs_bias, n, T, out, scale, s);
+  else launch_colsum<float, bf16_t>(b, gs_bias, n, T, out, scale, s);
+  DPK_LAUNCH_CHECK(who);
+  return DPK_OK;
+}
+
+extern "C" int dpk_conv_bias_gs(const void* b, int in_dtype, void* gs_bias, int gs_dtype, int64_t n,
+                                int64_t O, int64_t q, float scale, dpk_stream_t stream) {
+  const char* who = "dpk_conv_bias_gs";
+  DPK_REQUIRE(n >= 0 && O >= 1 && q >= 1, DPK_E_SHAPE, "%s: n=%lld O=%lld q=%lld", who,
+              (long long)n, (long long)O, (long long)q);
+  if (n == 0) return DPK_OK;
+  DPK_REQUIRE(b && gs_bias, DPK_E_ARG, "%s: NULL tensor", who);
+  DPK_REQUIRE(dpk_dtype_ok(in_dtype) && dpk_dtype_ok(gs_dtype), DPK_E_DTYPE, "%s: dtypes %d,%d", who,
+              in_dtype, gs_dtype);
+  DPK_REQUIRE(dpk_aligned(b, dpk_elsize(in_dtype)) && dpk_aligned(gs_bias, dpk_elsize(gs_dtype)),
+              DPK_E_ALIGN, "%s: misaligned tensor", who);
+  DPK_REQUIRE(dpk_cdiv(n * O, kWaves) <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: too many rows", who);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (in_dtype == DPK_F32 && gs_dtype == DPK_F32) launch_rowsum<float, float>(b, gs_bias, n * O, q, scale, s);
+  else if (in_dtype == DPK_BF16 && gs_dtype == DPK_BF16) launch_rowsum<bf16_t, bf16_t>(b, gs_bias, n * O, q, scale, s);
+  else if (in_dtype == DPK_BF16 && gs_dtype == DPK_F32) launch_rowsum<bf16_t, float>(b, gs_bias, n * O, q, scale, s);
+  else launch_rowsum<float, bf16_t>(b, gs_bias, n * O, q, scale, s);
+  DPK_LAUNCH_CHECK(who);
+  return DPK_OK;
+}

@@ -1,0 +1,534 @@
+"""Tensor-level wrappers over the C ABI of ``libdpsgd_hip.so``.
+
+Each function checks devices, dtypes and shapes, makes inputs dense, allocates the
+outputs (and the workspace the entry point asks for) with torch, and enqueues the
+HIP kernels on torch's current stream of the tensors' device. Tensors must live on
+the GPU: there is no CPU implementation behind these calls.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from contextlib import contextmanager
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import DPK_BF16, DPK_F32, DPK_MULTI_MAX, check, lib
+
+_DTYPES = {torch.float32: DPK_F32, torch.bfloat16: DPK_BF16}
+
+
+def supported_dtype(dtype: torch.dtype) -> bool:
+    return dtype in _DTYPES
+
+
+def _code(t_or_dtype) -> int:
+    dt = t_or_dtype.dtype if isinstance(t_or_dtype, torch.Tensor) else t_or_dtype
+    try:
+        return _DTYPES[dt]
+    except KeyError:
+        raise TypeError(f"dpk kernels take float32 or bfloat16 tensors, got {dt}") from None
+
+
+def _need_gpu(*tensors: torch.Tensor) -> torch.device:
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError(
+                "opacus_amd runs on the GPU only (HIP kernels, no CPU fallback); got a tensor on "
+                f"{t.device}"
+            )
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise RuntimeError(f"tensors on different devices: {dev} and {t.device}")
+    return dev
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream(dev: torch.device):
+    return ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+
+def _ws(nbytes: int, dev: torch.device) -> Tuple[Optional[torch.Tensor], int]:
+    if nbytes == 0:
+        return None, 0
+    t = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    return t, nbytes
+
+
+# ---- optional per-kernel timing (HIP events on the launch stream) -------------------
+_TIMING: Optional[Dict[str, List[Tuple[torch.cuda.Event, torch.cuda.Event]]]] = None
+
+
+@contextmanager
+def record_kernel_times():
+    """Collects (start, end) event pairs around every wrapper call made inside the block.
+
+    Yields a dict ``name -> [(start, end), ...]``; after a device synchronize,
+    ``start.elapsed_time(end)`` is the duration in ms of that call's kernels.
+    """
+    global _TIMING
+    prev, _TIMING = _TIMING, {}
+    try:
+        yield _TIMING
+    finally:
+        _TIMING = prev
+
+
+@contextmanager
+def _timed(name: str, dev: torch.device):
+    if _TIMING is None:
+        yield
+        return
+    with torch.cuda.device(dev):
+        s = torch.cuda.Event(enable_timing=True)
+        e = torch.cuda.Event(enable_timing=True)
+        s.record()
+        yield
+        e.record()
+    _TIMING.setdefault(name, []).append((s, e))
+
+
+def _dense(t: torch.Tensor) -> torch.Tensor:
+    return t if t.is_contiguous() else t.contiguous()
+
+
+# ---- nn.Linear ----------------------------------------------------------------------
+def linear_grad_sample(
+    backprops: torch.Tensor,
+    activations: torch.Tensor,
+    scale: float = 1.0,
+    want_sumsq: bool = True,
+    out_dtype: Optional[torch.dtype] = None,
+) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """``gs[n,i,j] = scale * sum_t b[n,t,i] a[n,t,j]`` and ``sum_ij gs[n]^2``.
+
+    ``backprops`` is ``[n, *, out]``, ``activations`` ``[n, *, in]`` with the same middle dims.
+    """
+    dev = _need_gpu(backprops, activations)
+    if activations.dtype != backprops.dtype:
+        activations = activations.to(backprops.dtype)
+    n, out_f, in_f = backprops.shape[0], backprops.shape[-1], activations.shape[-1]
+    b = _dense(backprops).reshape(n, -1, out_f) if n else backprops.reshape(0, 1, out_f)
+    a = _dense(activations).reshape(n, -1, in_f) if n else activations.reshape(0, 1, in_f)
+    T = b.shape[1]
+    if a.shape[1] != T:
+        raise ValueError(f"activations {tuple(activations.shape)} and backprops {tuple(backprops.shape)} disagree")
+    out_dtype = out_dtype or backprops.dtype
+    gs = torch.empty((n, out_f, in_f), dtype=out_dtype, device=dev)
+    sumsq = torch.empty((n,), dtype=torch.float32, device=dev) if want_sumsq else None
+    if n == 0:
+        return gs, sumsq
+    L = lib()
+    ws, wsb = _ws(L.dpk_linear_gs_workspace_bytes(n, T, out_f, in_f) if want_sumsq else 0, dev)
+    with _timed("linear_gs", dev):
+        check(
+            "dpk_linear_gs",
+            L.dpk_linear_gs(
+                _ptr(b), _ptr(a), _code(b), _ptr(gs), _code(gs), _ptr(sumsq), n, T, out_f, in_f,
+                float(scale), _ptr(ws), wsb, _stream(dev),
+            ),
+        )
+    return gs, sumsq
+
+
+def linear_bias_grad_sample(
+    backprops: torch.Tensor, scale: float = 1.0, out_dtype: Optional[torch.dtype] = None
+) -> torch.Tensor:
+    """``gs[n,k] = scale * sum over middle dims of b[n,*,k]``."""
+    dev = _need_gpu(backprops)
+    n, out_f = backprops.shape[0], backprops.shape[-1]
+    gs = torch.empty((n, out_f), dtype=out_dtype or backprops.dtype, device=dev)
+    if n == 0:
+        return gs
+    b = _dense(backprops).reshape(n, -1, out_f)
+    with _timed("linear_bias_gs", dev):
+        check(
+            "dpk_linear_bias_gs",
+            lib().dpk_linear_bias_gs(
+                _ptr(b), _code(b), _ptr(gs), _code(gs), n, b.shape[1], out_f, float(scale), _stream(dev)
+            ),
+        )
+    return gs
+
+
+def linear_ghost_norm(
+    backprops: torch.Tensor,
+    activations: torch.Tensor,
+    scale: float = 1.0,
+    want_weight: bool = True,
+    want_bias: bool = False,
+) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
+    """Per-sample norms (fp32) of the Linear weight and bias gradients without forming them."""
+    dev = _need_gpu(backprops, activations)
+    if activations.dtype != backprops.dtype:
+        activations = activations.to(backprops.dtype)
+    n, out_f, in_f = backprops.shape[0], backprops.shape[-1], activations.shape[-1]
+    nw = torch.empty((n,), dtype=torch.float32, device=dev) if want_weight else None
+    nb = torch.empty((n,), dtype=torch.float32, device=dev) if want_bias else None
+    if n == 0 or not (want_weight or want_bias):
+        return nw, nb
+    b = _dense(backprops).reshape(n, -1, out_f)
+    a = _dense(activations).reshape(n, -1, in_f)
+    T = b.shape[1]
+    if a.shape[1] != T:
+        raise ValueError(f"activations {tuple(activations.shape)} and backprops {tuple(backprops.shape)} disagree")
+    L = lib()
+    ws, wsb = _ws(L.dpk_linear_ghost_norm_workspace_bytes(n, T, out_f, in_f), dev)
+    with _timed("linear_ghost_norm", dev):
+        check(
+            "dpk_linear_ghost_norm",
+            L.dpk_linear_ghost_norm(
+                _ptr(b), _ptr(a), _code(b), _ptr(nw), _ptr(nb), n, T, out_f, in_f, float(scale),
+                _ptr(ws), wsb, _stream(dev),
+            ),
+        )
+    return nw, nb
+
+
+# ---- nn.Conv2d ----------------------------------------------------------------------
+def conv2d_grad_sample(
+    x: torch.Tensor,
+    backprops: torch.Tensor,
+    kernel_size: Tuple[int, int],
+    stride: Tuple[int, int],
+    padding: Tuple[int, int, int, int],
+    dilation: Tuple[int, int],
+    groups: int,
+    scale: float = 1.0,
+    want_sumsq: bool = True,
+) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """Per-sample weight gradients ``[n, O, C/groups, KH, KW]`` of a 2-d convolution.
+
+    ``padding`` is ``(top, bottom, left, right)``; ``backprops`` is ``[n, O, OH, OW]``.
+    """
+    dev = _need_gpu(x, backprops)
+    if x.dtype != backprops.dtype:
+        x = x.to(backprops.dtype)
+    n, C, H, W = x.shape
+    O = backprops.shape[1]
+    KH, KW = kernel_size
+    gs = torch.empty((n, O, C // groups, KH, KW), dtype=backprops.dtype, device=dev)
+    sumsq = torch.empty((n,), dtype=torch.float32, device=dev) if want_sumsq else None
+    if n == 0:
+        return gs, sumsq
+    x = _dense(x)
+    b = _dense(backprops)
+    L = lib()
+    ws, wsb = _ws(L.dpk_conv2d_gs_workspace_bytes(n, C, O, KH, KW, groups) if want_sumsq else 0, dev)
+    oh = (H + padding[0] + padding[1] - (dilation[0] * (KH - 1) + 1)) // stride[0] + 1
+    ow = (W + padding[2] + padding[3] - (dilation[1] * (KW - 1) + 1)) // stride[1] + 1
+    if b.numel() != n * O * oh * ow:
+        raise ValueError(
+            f"backprops {tuple(backprops.shape)} do not match the output geometry [{n},{O},{oh},{ow}]"
+        )
+    with _timed("conv2d_gs", dev):
+        check(
+            "dpk_conv2d_gs",
+            L.dpk_conv2d_gs(
+                _ptr(x), _ptr(b), _code(b), _ptr(gs), _code(gs), _ptr(sumsq), n, C, H, W, O, KH, KW,
+                stride[0], stride[1], padding[0], padding[1], padding[2], padding[3], dilation[0],
+                dilation[1], groups, float(scale), _ptr(ws), wsb, _stream(dev),
+            ),
+        )
+    return gs, sumsq
+
+
+def conv_bias_grad_sample(backprops: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """``gs[n,o] = scale * sum over the spatial dims of b[n,o,...]``."""
+    dev = _need_gpu(backprops)
+    n, O = backprops.shape[0], backprops.shape[1]
+    gs = torch.empty((n, O), dtype=backprops.dtype, device=dev)
+    if n == 0:
+        return gs
+    b = _dense(backprops).reshape(n, O, -1)
+    with _timed("conv_bias_gs", dev):
+        check(
+            "dpk_conv_bias_gs",
+            lib().dpk_conv_bias_gs(
+                _ptr(b), _code(b), _ptr(gs), _code(gs), n, O, b.shape[2], float(scale), _stream(dev)
+            ),
+        )
+    return gs
+
+
+# ---- nn.Embedding -------------------------------------------------------------------
+def _ids_2d(ids: torch.Tensor) -> torch.Tensor:
+    if ids.dtype != torch.int64:
+        ids = ids.to(torch.int64)
+    return _dense(ids).reshape(ids.shape[0], -1)
+
+
+def embedding_unique_pairs(ids: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``(unique_pairs [U,2], inverse [n*T])`` of the (row, id) pairs, sorted: the integer stage."""
+    dev = _need_gpu(ids)
+    ids2 = _ids_2d(ids)
+    n, T = ids2.shape
+    inverse = torch.empty((n * T,), dtype=torch.int64, device=dev)
+    pairs = torch.empty((n * T, 2), dtype=torch.int64, device=dev)
+    count = torch.zeros((1,), dtype=torch.int64, device=dev)
+    if n * T == 0:
+        return pairs[:0], inverse
+    L = lib()
+    ws, wsb = _ws(L.dpk_embedding_workspace_bytes(n, T), dev)
+    with _timed("embedding_unique_pairs", dev):
+        check(
+            "dpk_embedding_unique_pairs",
+            L.dpk_embedding_unique_pairs(
+                _ptr(ids2), n, T, _ptr(inverse), _ptr(pairs), _ptr(count), _ptr(ws), wsb, _stream(dev)
+            ),
+        )
+    return pairs[: int(count.item())], inverse
+
+
+def embedding_grad_sample(
+    ids: torch.Tensor, backprops: torch.Tensor, num_embeddings: int, scale: float = 1.0
+) -> torch.Tensor:
+    """``gs[n,v,:] = scale * sum_{t: ids[n,t]==v} b[n,t,:]`` as a dense ``[n, V, D]`` tensor."""
+    dev = _need_gpu(ids, backprops)
+    ids2 = _ids_2d(ids)
+    n, T = ids2.shape
+    D = backprops.shape[-1]
+    gs = torch.empty((n, num_embeddings, D), dtype=backprops.dtype, device=dev)
+    if n == 0:
+        return gs
+    b = _dense(backprops).reshape(n, -1, D)
+    if b.shape[1] != T:
+        raise ValueError(f"ids {tuple(ids.shape)} and backprops {tuple(backprops.shape)} disagree")
+    L = lib()
+    ws, wsb = _ws(L.dpk_embedding_workspace_bytes(n, T), dev)
+    with _timed("embedding_gs", dev):
+        check(
+            "dpk_embedding_gs",
+            L.dpk_embedding_gs(
+                _ptr(ids2), _ptr(b), _code(b), _ptr(gs), _code(gs), n, T, num_embeddings, D,
+                float(scale), _ptr(ws), wsb, _stream(dev),
+            ),
+        )
+    return gs
+
+
+def embedding_ghost_norm(ids: torch.Tensor, backprops: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """Per-sample norm (fp32) of the Embedding weight gradient without forming it."""
+    dev = _need_gpu(ids, backprops)
+    ids2 = _ids_2d(ids)
+    n, T = ids2.shape
+    D = backprops.shape[-1]
+    norm = torch.empty((n,), dtype=torch.float32, device=dev)
+    if n == 0:
+        return norm
+    b = _dense(backprops).reshape(n, -1, D)
+    if b.shape[1] != T:
+        raise ValueError(f"ids {tuple(ids.shape)} and backprops {tuple(backprops.shape)} disagree")
+    L = lib()
+    ws, wsb = _ws(L.dpk_embedding_workspace_bytes(n, T), dev)
+    with _timed("embedding_ghost_norm", dev):
+        check(
+            "dpk_embedding_ghost_norm",
+            L.dpk_embedding_ghost_norm(
+                _ptr(ids2), _ptr(b), _code(b), _ptr(norm), n, T, D, float(scale), _ptr(ws), wsb,
+                _stream(dev),
+            ),
+        )
+    return norm
+
+
+# ---- normalisation layers -----------------------------------------------------------
+def group_norm_grad_sample(
+    x: torch.Tensor,
+    backprops: torch.Tensor,
+    num_groups: int,
+    eps: float,
+    scale: float = 1.0,
+    want_weight: bool = True,
+    want_bias: bool = True,
+) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
+    """Per-sample gradients ``[n, C]`` of GroupNorm's weight and bias."""
+    dev = _need_gpu(x, backprops)
+    if x.dtype != backprops.dtype:
+        x = x.to(backprops.dtype)
+    n, C = x.shape[0], x.shape[1]
+    gw = torch.empty((n, C), dtype=backprops.dtype, device=dev) if want_weight else None
+    gb = torch.empty((n, C), dtype=backprops.dtype, device=dev) if want_bias else None
+    if n == 0 or not (want_weight or want_bias):
+        return gw, gb
+    xd = _dense(x).reshape(n, C, -1)
+    bd = _dense(backprops).reshape(n, C, -1)
+    with _timed("group_norm_gs", dev):
+        check(
+            "dpk_group_norm_gs",
+            lib().dpk_group_norm_gs(
+                _ptr(xd), _ptr(bd), _code(bd), _ptr(gw), _ptr(gb), _code(backprops.dtype), n, C,
+                xd.shape[2], num_groups, float(eps), float(scale), _stream(dev),
+            ),
+        )
+    return gw, gb
+
+
+def rms_norm_grad_sample(
+    x: torch.Tensor, backprops: torch.Tensor, normalized_numel: int, eps: float, scale: float = 1.0
+) -> torch.Tensor:
+    """Per-sample gradient ``[n, D]`` of RMSNorm's weight (``D = normalized_numel``)."""
+    dev = _need_gpu(x, backprops)
+    if x.dtype != backprops.dtype:
+        x = x.to(backprops.dtype)
+    n, D = x.shape[0], normalized_numel
+    gw = torch.empty((n, D), dtype=backprops.dtype, device=dev)
+    if n == 0:
+        return gw
+    xd = _dense(x).reshape(n, -1, D)
+    bd = _dense(backprops).reshape(n, -1, D)
+    T = xd.shape[1]
+    L = lib()
+    ws, wsb = _ws(L.dpk_rms_norm_gs_workspace_bytes(n, T, D), dev)
+    with _timed("rms_norm_gs", dev):
+        check(
+            "dpk_rms_norm_gs",
+            L.dpk_rms_norm_gs(
+                _ptr(xd), _ptr(bd), _code(bd), _ptr(gw), _code(gw), n, T, D, float(eps), float(scale),
+                _ptr(ws), wsb, _stream(dev),
+            ),
+        )
+    return gw
+
+
+# ---- optimizer: norms, clip factor, clip-weighted sum, noise ---------------------------
+def _flat2d(gs: torch.Tensor) -> torch.Tensor:
+    g = _dense(gs)
+    return g.reshape(g.shape[0], -1)
+
+
+def sumsq_rows(gs_list: Sequence[torch.Tensor]) -> torch.Tensor:
+    """``out[k, i] = sum of squares of sample i of tensor k`` (fp32), one pass over each tensor."""
+    dev = _need_gpu(*gs_list)
+    K = len(gs_list)
+    n = gs_list[0].shape[0]
+    out = torch.empty((K, n), dtype=torch.float32, device=dev)
+    if n == 0 or K == 0:
+        return out
+    flats = [_flat2d(g) for g in gs_list]
+    dt = flats[0].dtype
+    if any(f.dtype != dt or f.shape[0] != n for f in flats):
+        raise ValueError("per-sample gradient tensors must share the batch size and dtype")
+    L = lib()
+    for lo in range(0, K, DPK_MULTI_MAX):
+        chunk = flats[lo : lo + DPK_MULTI_MAX]
+        k = len(chunk)
+        ptrs = (ctypes.c_void_p * k)(*[f.data_ptr() for f in chunk])
+        sizes = (ctypes.c_int64 * k)(*[f.shape[1] for f in chunk])
+        ws, wsb = _ws(L.dpk_sumsq_rows_multi_workspace_bytes(n, sizes, k), dev)
+        with _timed("sumsq_rows", dev):
+            check(
+                "dpk_sumsq_rows_multi",
+                L.dpk_sumsq_rows_multi(
+                    ptrs, sizes, k, _code(dt), n, _ptr(out[lo : lo + k]), _ptr(ws), wsb, _stream(dev)
+                ),
+            )
+    return out
+
+
+def clip_factor(
+    values: torch.Tensor, max_grad_norm: float, is_norm: bool = False
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``(norm[n], clip[n])`` from ``values[K, n]`` (squared norms, or norms with ``is_norm``)."""
+    dev = _need_gpu(values)
+    v = _dense(values.to(torch.float32)).reshape(-1, values.shape[-1])
+    K, n = v.shape
+    norm = torch.empty((n,), dtype=torch.float32, device=dev)
+    clip = torch.empty((n,), dtype=torch.float32, device=dev)
+    if n == 0:
+        return norm, clip
+    check(
+        "dpk_clip_factor",
+        lib().dpk_clip_factor(
+            _ptr(v), K, n, int(is_norm), float(max_grad_norm), _ptr(norm), _ptr(clip), _stream(dev)
+        ),
+    )
+    return norm, clip
+
+
+def clip_accumulate(
+    gs_list: Sequence[torch.Tensor],
+    clip: torch.Tensor,
+    summed_list: Sequence[torch.Tensor],
+    accumulate: bool,
+) -> None:
+    """``summed_k (+)= sum_n clip[n] * gs_k[n]`` for every k, reading each gs once."""
+    dev = _need_gpu(clip, *gs_list, *summed_list)
+    K = len(gs_list)
+    if K == 0:
+        return
+    n = gs_list[0].shape[0]
+    flats = [_flat2d(g) for g in gs_list]
+    gdt, odt = flats[0].dtype, summed_list[0].dtype
+    for f, s in zip(flats, summed_list):
+        if f.dtype != gdt or s.dtype != odt or f.shape[0] != n:
+            raise ValueError("tensors of one clip_accumulate call must share batch size and dtypes")
+        if not s.is_contiguous() or s.numel() != f.shape[1]:
+            raise ValueError("summed tensors must be dense and match the per-sample gradient size")
+    if clip.dtype != torch.float32 or clip.numel() != n:
+        raise ValueError("clip must be a float32 tensor with one entry per sample")
+    clip = _dense(clip)
+    L = lib()
+    for lo in range(0, K, DPK_MULTI_MAX):
+        fs, ss = flats[lo : lo + DPK_MULTI_MAX], summed_list[lo : lo + DPK_MULTI_MAX]
+        k = len(fs)
+        gptrs = (ctypes.c_void_p * k)(*[f.data_ptr() for f in fs])
+        sptrs = (ctypes.c_void_p * k)(*[s.data_ptr() for s in ss])
+        sizes = (ctypes.c_int64 * k)(*[f.shape[1] for f in fs])
+        with _timed("clip_accumulate", dev):
+            check(
+                "dpk_clip_accumulate_multi",
+                L.dpk_clip_accumulate_multi(
+                    gptrs, sptrs, sizes, k, _code(gdt), _code(odt), _ptr(clip), n, int(accumulate),
+                    _stream(dev),
+                ),
+            )
+
+
+def add_noise(
+    summed: torch.Tensor,
+    grad: torch.Tensor,
+    std: float,
+    denom: float,
+    seed: int,
+    offset: int,
+    draws: int = 1,
+) -> None:
+    """``grad = (summed + std * z) / denom`` with ``z ~ N(0,1)`` from Philox(seed, offset)."""
+    dev = _need_gpu(summed, grad)
+    if not summed.is_contiguous() or not grad.is_contiguous() or summed.numel() != grad.numel():
+        raise ValueError("summed and grad must be dense and of equal size")
+    with _timed("add_noise", dev):
+        check(
+            "dpk_add_noise",
+            lib().dpk_add_noise(
+                _ptr(summed), _code(summed), _ptr(grad), _code(grad), summed.numel(), float(std),
+                float(denom), seed & 0xFFFFFFFFFFFFFFFF, offset & 0xFFFFFFFFFFFFFFFF, draws, _stream(dev),
+            ),
+        )
+
+
+def fill_normal(out: torch.Tensor, std: float, seed: int, offset: int) -> None:
+    dev = _need_gpu(out)
+    if out.dtype != torch.float32 or not out.is_contiguous():
+        raise ValueError("fill_normal needs a dense float32 tensor")
+    check(
+        "dpk_fill_normal",
+        lib().dpk_fill_normal(
+            _ptr(out), out.numel(), float(std), seed & 0xFFFFFFFFFFFFFFFF, offset & 0xFFFFFFFFFFFFFFFF,
+            _stream(dev),
+        ),
+    )
+
+
+def device_cus() -> int:
+    return lib().dpk_device_cus()

@@ -1,0 +1,222 @@
+"""GPU parity: every HIP kernel, called through the C ABI, against the CPU oracle.
+
+Tolerances follow the stated bar: fp32 within rel 1e-5 (of the tensor's scale), bf16
+within rel 2e-2 with fp32 accumulation, integer outputs bit-exact.
+"""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import dp_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+FP32_REL = 1e-5
+BF16_REL = 2e-2
+
+
+@pytest.fixture(scope="module")
+def K():
+    from opacus_amd import kernels
+
+    return kernels
+
+
+def dev(t):
+    return t.to("cuda")
+
+
+def assert_rel(got, want, rel, what=""):
+    """max |got - want| <= rel * max |want| (tensor-scale relative error), plus exact shape."""
+    got = got.detach().float().cpu()
+    want = want.detach().float().cpu()
+    assert got.shape == want.shape, f"{what}: shape {tuple(got.shape)} != {tuple(want.shape)}"
+    if want.numel() == 0:
+        return
+    scale = want.abs().max().item()
+    err = (got - want).abs().max().item()
+    assert err <= rel * max(scale, 1e-30), f"{what}: max err {err:.3e} vs scale {scale:.3e} (rel {err / max(scale, 1e-30):.2e})"
+
+
+# ---- Linear per-sample gradients ---------------------------------------------------------
+LINEAR_SHAPES = [
+    # (n, middle dims, in, out)
+    (4, (), 8, 4),  # T = 1, tiny
+    (3, (), 130, 67),  # T = 1, odd sizes -> scalar path
+    (16, (), 512, 32),  # C1 fc1 shape
+    (5, (1,), 256, 96),  # 3-d with T = 1
+    (3, (7,), 64, 64),  # MFMA 64x64 tiles, K smaller than one k tile
+    (2, (50,), 200, 136),  # MFMA 128 tiles with ragged edges
+    (2, (33,), 70, 30),  # MFMA small tile, odd sizes -> scalar loads
+    (2, (4, 9), 132, 260),  # two middle dims
+    (1, (300,), 128, 128),  # long K
+]
+
+
+@pytest.mark.parametrize("n,mid,fin,fout", LINEAR_SHAPES)
+@pytest.mark.parametrize("scale", [1.0, 3.0])
+def test_linear_grad_sample_f32(K, n, mid, fin, fout, scale):
+    torch.manual_seed(n * 1000 + fin)
+    a = torch.randn(n, *mid, fin)
+    b = torch.randn(n, *mid, fout)
+    want_w, want_b = O.linear_grad_sample(a, b * scale)
+    gs, sumsq = K.linear_grad_sample(dev(b), dev(a), scale=scale)
+    gb = K.linear_bias_grad_sample(dev(b), scale=scale)
+    assert_rel(gs, want_w, FP32_REL, "weight")
+    assert_rel(gb, want_b, FP32_REL, "bias")
+    assert_rel(sumsq, want_w.double().flatten(1).pow(2).sum(1), 2e-5, "sumsq")
+
+
+@pytest.mark.parametrize("n,mid,fin,fout", [(4, (), 64, 32), (2, (40,), 136, 200), (3, (5,), 30, 18)])
+def test_linear_grad_sample_bf16(K, n, mid, fin, fout):
+    torch.manual_seed(7)
+    a = torch.randn(n, *mid, fin).bfloat16()
+    b = torch.randn(n, *mid, fout).bfloat16()
+    want_w, want_b = O.linear_grad_sample(a.float(), b.float())
+    gs, sumsq = K.linear_grad_sample(dev(b), dev(a))
+    assert gs.dtype == torch.bfloat16
+    assert_rel(gs, want_w, BF16_REL, "weight bf16")
+    assert_rel(K.linear_bias_grad_sample(dev(b)), want_b, BF16_REL, "bias bf16")
+    assert_rel(sumsq, want_w.double().flatten(1).pow(2).sum(1), 1e-4, "sumsq (fp32 accumulators)")
+    gs32, _ = K.linear_grad_sample(dev(b), dev(a), out_dtype=torch.float32)
+    assert_rel(gs32, want_w, FP32_REL, "weight bf16 in, fp32 out")
+
+
+def test_linear_grad_sample_mixed_activation_dtype_and_views(K):
+    torch.manual_seed(8)
+    a = torch.randn(6, 5, 40)
+    b = torch.randn(5, 6, 24).transpose(0, 1)  # not contiguous
+    want_w, _ = O.linear_grad_sample(a, b)
+    gs, _ = K.linear_grad_sample(dev(b), dev(a).double())  # activations are cast to backprops' dtype
+    assert_rel(gs, want_w, FP32_REL)
+
+
+def test_linear_empty_batch(K):
+    gs, sumsq = K.linear_grad_sample(torch.zeros(0, 4, device="cuda"), torch.zeros(0, 6, device="cuda"))
+    assert gs.shape == (0, 4, 6) and sumsq.shape == (0,)
+
+
+def test_linear_is_deterministic(K):
+    torch.manual_seed(9)
+    a, b = dev(torch.randn(8, 33, 200)), dev(torch.randn(8, 33, 136))
+    g1, s1 = K.linear_grad_sample(b, a)
+    g2, s2 = K.linear_grad_sample(b, a)
+    assert torch.equal(g1, g2) and torch.equal(s1, s2)
+
+
+# ---- Optimizer kernels ---------------------------------------------------------------
+GS_SETS = [
+    [(5, (3, 4)), (5, (7,))],  # tiny, odd -> scalar path
+    [(64, (32, 512)), (64, (32,)), (64, (10, 32)), (64, (10,))],  # C1-like tail
+    [(9, (40000,))],  # several chunks per row
+    [(130, (16, 1, 8, 8)), (130, (16,))],  # n not a multiple of the unroll, row split
+]
+
+
+@pytest.mark.parametrize("spec", GS_SETS)
+@pytest.mark.parametrize("C", [0.5, 1e20])
+def test_clip_and_accumulate_f32(K, spec, C):
+    torch.manual_seed(len(spec))
+    gs = [torch.randn(n, *shape) * (0.01 if i % 2 else 1.0) for i, (n, shape) in enumerate(spec)]
+    gs[0][0] *= 50.0
+    norms, clip, summed = O.clip_and_accumulate(gs, C)
+    dgs = [dev(g) for g in gs]
+    ss = K.sumsq_rows(dgs)
+    want_ss = torch.stack([g.double().flatten(1).pow(2).sum(1) for g in gs])
+    assert_rel(ss, want_ss, FP32_REL, "sumsq")
+    gnorm, gclip = K.clip_factor(ss, C)
+    assert_rel(gnorm, norms, FP32_REL, "norm")
+    assert_rel(gclip, clip, FP32_REL, "clip")
+    outs = [torch.full(g.shape[1:], 7.0, device="cuda") for g in gs]
+    K.clip_accumulate(dgs, gclip, outs, accumulate=False)
+    for o, s in zip(outs, summed):
+        assert_rel(o, s, FP32_REL, "summed")
+    K.clip_accumulate(dgs, gclip, outs, accumulate=True)
+    for o, s in zip(outs, summed):
+        assert_rel(o, 2 * s, FP32_REL, "summed twice")
+
+
+def test_clip_accumulate_bf16_in_fp32_out(K):
+    torch.manual_seed(3)
+    gs = [torch.randn(33, 24, 40).bfloat16(), torch.randn(33, 7).bfloat16()]
+    _, clip, summed = O.clip_and_accumulate([g.float() for g in gs], 1.0)
+    dgs = [dev(g) for g in gs]
+    ss = K.sumsq_rows(dgs)
+    _, gclip = K.clip_factor(ss, 1.0)
+    assert_rel(gclip, clip, 1e-5)
+    outs = [torch.empty(g.shape[1:], device="cuda") for g in gs]
+    K.clip_accumulate(dgs, gclip, outs, accumulate=False)
+    for o, s in zip(outs, summed):
+        assert_rel(o, s, FP32_REL)
+    outs16 = [torch.empty(g.shape[1:], device="cuda", dtype=torch.bfloat16) for g in gs]
+    K.clip_accumulate(dgs, gclip, outs16, accumulate=False)
+    for o, s in zip(outs16, summed):
+        assert_rel(o, s, BF16_REL)
+
+
+def test_clip_factor_from_norms(K):
+    ns = torch.tensor([[3.0, 0.0, 0.3], [4.0, 0.0, 0.4]])
+    norm, clip = K.clip_factor(dev(ns), 1.0, is_norm=True)
+    assert_rel(norm, O.per_sample_norm(list(ns)), 1e-6)
+    assert_rel(clip, O.clipping_coef(list(ns), 1.0), 1e-6)
+
+
+def test_clip_accumulate_many_tensors(K):
+    torch.manual_seed(4)
+    gs = [torch.randn(6, 3 + i) for i in range(60)]  # more than one launch's worth
+    _, clip, summed = O.clip_and_accumulate(gs, 2.0)
+    dgs = [dev(g) for g in gs]
+    _, gclip = K.clip_factor(K.sumsq_rows(dgs), 2.0)
+    outs = [torch.empty(g.shape[1:], device="cuda") for g in gs]
+    K.clip_accumulate(dgs, gclip, outs, accumulate=False)
+    for o, s in zip(outs, summed):
+        assert_rel(o, s, FP32_REL)
+
+
+# ---- Noise ---------------------------------------------------------------------------
+def test_add_noise_zero_std_is_exact(K):
+    torch.manual_seed(5)
+    s = torch.randn(1003)
+    out = torch.empty(1003, device="cuda")
+    K.add_noise(dev(s), out, std=0.0, denom=1.0, seed=1, offset=0)
+    assert torch.equal(out.cpu(), s)
+    K.add_noise(dev(s), out, std=0.0, denom=256.0, seed=1, offset=0)
+    assert torch.equal(out.cpu(), s / 256.0)
+
+
+def test_noise_stream_matches_philox_restatement(K):
+    P = 4099
+    out = torch.empty(P, device="cuda")
+    K.fill_normal(out, std=1.0, seed=0xDEADBEEFCAFE, offset=12345678901)
+    want = O.philox_normal(P, seed=0xDEADBEEFCAFE, offset=12345678901)
+    np.testing.assert_allclose(out.cpu().numpy(), want, rtol=0, atol=2e-5)
+
+
+def test_noise_statistics(K):
+    P = 1 << 22
+    out = torch.empty(P, device="cuda")
+    K.fill_normal(out, std=1.7, seed=42, offset=0)
+    z = out.double()
+    se = 1.7 / math.sqrt(P)
+    assert abs(z.mean().item()) < 5 * se
+    assert abs(z.std().item() - 1.7) < 5 * 1.7 / math.sqrt(2 * P)
+    assert abs(((z / 1.7) ** 4).mean().item() - 3.0) < 0.03
+    out2 = torch.empty(P, device="cuda")
+    K.fill_normal(out2, std=1.7, seed=42, offset=1)
+    assert abs(torch.corrcoef(torch.stack([out, out2]))[0, 1].item()) < 5 / math.sqrt(P)
+    K.fill_normal(out2, std=1.7, seed=42, offset=0)
+    assert torch.equal(out, out2)  # same (seed, offset) -> same bits
+
+
+def test_add_noise_secure_draws_and_dtypes(K):
+    P = 1 << 20
+    s = torch.zeros(P, device="cuda")
+    g = torch.empty(P, device="cuda")
+    K.add_noise(s, g, std=2.0, denom=4.0, seed=3, offset=10, draws=4)
+    assert abs(g.double().std().item() - 0.5) < 5e-3 and abs(g.double().mean().item()) < 5e-3
+    gb = torch.empty(P, device="cuda", dtype=torch.bfloat16)
+    K.add_noise(s.bfloat16(), gb, std=1.0, denom=1.0, seed=3, offset=10)
+    assert abs(gb.double().std().item() - 1.0) < 1e-2
