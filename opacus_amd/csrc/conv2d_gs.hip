@@ -1,0 +1,218 @@
+// Per-sample gradients of nn.Conv2d (opacus/grad_sample/conv.py:28-119, Conv2d
+// branch) as an implicit-GEMM on the fp32 MFMA path:
+//   gs[n, g*Og + m, p] = scale * sum_q b[n, g*Og + m, q] * U[n, g, p, q]
+// with q = (oh, ow) running over output positions and p = (c, kh, kw) over one
+// group's kernel elements. U is the unfolded activation of
+// opacus/utils/tensor_utils.py:116-172,
+//   U[n, g, (c,kh,kw), (oh,ow)] = xpad[n, g*Cg + c, oh*sh + kh*dh, ow*sw + kw*dw],
+// which is gathered straight from x into the LDS tile (zero where the padding
+// is): the n x C*KH*KW x OH*OW matrix the reference writes and re-reads never
+// exists. Only the group-diagonal blocks are computed, where the reference forms
+// the full O x p product and discards the rest (conv.py:102-112).
+#include "dpk_common.h"
+#include "mfma_f32.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / DPK_WAVE;
+
+struct ConvGeom {
+  int H, W, OW, Q;      // input rows/cols, output cols, output positions
+  int KH, KW, Pg;       // kernel, kernel elements per group (Cg*KH*KW)
+  int sh, sw, dh, dw;   // stride, dilation
+  int ph, pw;           // top / left padding
+};
+
+// Element (k = q, col = p) of the unfolded activation, staged as S[k][p].
+template <int BN, typename T>
+struct LoaderIm2col {
+  static constexpr int R = mf32::BK * BN / mf32::NTHREADS;
+  static constexpr int PSTEP = mf32::NTHREADS / mf32::BK;
+  const T* x;  // first channel of this sample's group
+  ConvGeom g;
+  int kq, pl0;
+  int off[R], dy[R], dx[R];
+  float st[R];
+  __device__ __forceinline__ LoaderIm2col(const T* x_, const ConvGeom& g_, int p0) : x(x_), g(g_) {
+    kq = threadIdx.x % mf32::BK;
+    pl0 = threadIdx.x / mf32::BK;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int p = p0 + pl0 + r * PSTEP;
+      if (p < g.Pg) {
+        const int c = p / (g.KH * g.KW), rem = p % (g.KH * g.KW);
+        off[r] = c * g.H * g.W;
+        dy[r] = (rem / g.KW) * g.dh - g.ph;
+        dx[r] = (rem % g.KW) * g.dw - g.pw;
+      } else {
+        off[r] = -1;
+        dy[r] = dx[r] = 0;
+      }
+    }
+  }
+  __device__ __forceinline__ void fetch(int64_t k0) {
+    const int q = static_cast<int>(k0) + kq;
+    const int oh = q / g.OW, ow = q - oh * g.OW;
+    const int iy0 = oh * g.sh, ix0 = ow * g.sw;
+    const bool inq = q < g.Q;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int iy = iy0 + dy[r], ix = ix0 + dx[r];
+      const bool ok = inq && off[r] >= 0 && static_cast<unsigned>(iy) < static_cast<unsigned>(g.H) &&
+                      static_cast<unsigned>(ix) < static_cast<unsigned>(g.W);
+      st[r] = ok ? dpk_io<T>::load(x + off[r] + iy * g.W + ix) : 0.f;
+    }
+  }
+  __device__ __forceinline__ void commit(float (*S)[BN + mf32::PAD]) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) S[kq][pl0 + r * PSTEP] = st[r];
+  }
+};
+
+template <int BM, int BN, typename TIN, typename TOUT, bool VEC>
+__global__ __launch_bounds__(kThreads) void conv2d_gs_kernel(
+    const TIN* __restrict__ x, const TIN* __restrict__ b, TOUT* __restrict__ gs,
+    float* __restrict__ partials, ConvGeom g, int C, int O, int groups, float scale, int tiles_m,
+    int tiles_n) {
+  __shared__ mf32::Smem<BM, BN> sm;
+  __shared__ float red[kWaves];
+  const int Og = O / groups, Cg = C / groups;
+  int64_t bid = blockIdx.x;
+  const int tn = static_cast<int>(bid % tiles_n);
+  bid /= tiles_n;
+  const int tm = static_cast<int>(bid % tiles_m);
+  bid /= tiles_m;
+  const int grp = static_cast<int>(bid % groups);
+  const int64_t sample = bid / groups;
+  const int m0 = tm * BM, p0 = tn * BN;
+  const TIN* bg = b + (sample * O + static_cast<int64_t>(grp) * Og) * g.Q;
+  const TIN* xg = x + (sample * C + static_cast<int64_t>(grp) * Cg) * g.H * g.W;
+  mf32::LoaderKContig<BM, TIN, VEC> la(bg, g.Q, m0, Og, g.Q);
+  LoaderIm2col<BN, TIN> lb(xg, g, p0);
+  mf32::Tile<BM, BN> tile;
+  tile.clear();
+  mf32::mainloop<BM, BN>(tile, sm, la, lb, g.Q);
+  TOUT* out = gs + (sample * O + static_cast<int64_t>(grp) * Og) * g.Pg;
+  float ss = 0.f;
+  tile.for_each([&](int r, int c, float v) {
+    const int m = m0 + r, p = p0 + c;
+    if (m < Og && p < g.Pg) {
+      const float val = v * scale;
+      dpk_io<TOUT>::store(out + static_cast<int64_t>(m) * g.Pg + p, val);
+      ss = fmaf(val, val, ss);
+    }
+  });
+  if (partials) {
+    const float s = block_sum<kWaves>(ss, red);
+    if (threadIdx.x == 0) partials[blockIdx.x] = s;
+  }
+}
+
+struct Plan {
+  int bm, bn, tiles_m, tiles_n;
+};
+
+Plan make_plan(int64_t Og, int64_t Pg) {
+  Plan p;
+  p.bm = Og > 64 ? 128 : 64;
+  p.bn = (Pg > 64 && p.bm == 128) ? 128 : 64;
+  if (p.bn == 64) p.bm = 64;
+  p.tiles_m = static_cast<int>(dpk_cdiv(Og, p.bm));
+  p.tiles_n = static_cast<int>(dpk_cdiv(Pg, p.bn));
+  return p;
+}
+
+template <typename TIN, typename TOUT>
+void launch(const Plan& p, bool vec, const void* x, const void* b, void* gs, float* partials,
+            const ConvGeom& g, int64_t n, int C, int O, int groups, float scale, hipStream_t s) {
+  const dim3 grid(static_cast<unsigned>(n * groups * p.tiles_m * p.tiles_n)), block(kThreads);
+  const TIN* xp = static_cast<const TIN*>(x);
+  const TIN* bp = static_cast<const TIN*>(b);
+  TOUT* gp = static_cast<TOUT*>(gs);
+#define DPK_CONV_LAUNCH(BM, BN, V)                                                              \
+  hipLaunchKernelGGL((conv2d_gs_kernel<BM, BN, TIN, TOUT, V>), grid, block, 0, s, xp, bp, gp,   \
+                     partials, g, C, O, groups, scale, p.tiles_m, p.tiles_n)
+  if (p.bm == 128) {
+    if (vec) DPK_CONV_LAUNCH(128, 128, true);
+    else DPK_CONV_LAUNCH(128, 128, false);
+  } else {
+    if (vec) DPK_CONV_LAUNCH(64, 64, true);
+    else DPK_CONV_LAUNCH(64, 64, false);
+  }
+#undef DPK_CONV_LAUNCH
+}
+
+}  // namespace
+
+extern "C" size_t dpk_conv2d_gs_workspace_bytes(int64_t n, int64_t C, int64_t O, int64_t KH,
+                                                int64_t KW, int64_t groups) {
+  if (n <= 0 || C <= 0 || O <= 0 || KH <= 0 || KW <= 0 || groups <= 0) return 0;
+  if (C % groups != 0 || O % groups != 0) return 0;
+  const Plan p = make_plan(O / groups, (C / groups) * KH * KW);
+  return dpk_align_up(static_cast<size_t>(n * groups * p.tiles_m * p.tiles_n) * sizeof(float), 256);
+}
+
+extern "C" int dpk_conv2d_gs(const void* x, const void* b, int in_dtype, void* gs, int gs_dtype,
+                             float* sumsq, int64_t n, int64_t C, int64_t H, int64_t W, int64_t O,
+                             int64_t KH, int64_t KW, int64_t sh, int64_t sw, int64_t ph_lo,
+                             int64_t ph_hi, int64_t pw_lo, int64_t pw_hi, int64_t dh, int64_t dw,
+                             int64_t groups, float scale, void* ws, size_t ws_bytes,
+                             dpk_stream_t stream) {
+  const char* who = "dpk_conv2d_gs";
+  DPK_REQUIRE(n >= 0 && C >= 1 && H >= 1 && W >= 1 && O >= 1 && KH >= 1 && KW >= 1, DPK_E_SHAPE,
+              "%s: bad tensor sizes", who);
+  DPK_REQUIRE(sh >= 1 && sw >= 1 && dh >= 1 && dw >= 1 && ph_lo >= 0 && ph_hi >= 0 && pw_lo >= 0 &&
+                  pw_hi >= 0 && groups >= 1,
+              DPK_E_SHAPE, "%s: bad geometry", who);
+  DPK_REQUIRE(C % groups == 0 && O % groups == 0, DPK_E_SHAPE,
+              "%s: groups=%lld does not divide C=%lld and O=%lld", who, (long long)groups,
+              (long long)C, (long long)O);
+  if (n == 0) return DPK_OK;
+  const int64_t eh = H + ph_lo + ph_hi - (dh * (KH - 1) + 1), ew = W + pw_lo + pw_hi - (dw * (KW - 1) + 1);
+  DPK_REQUIRE(eh >= 0 && ew >= 0, DPK_E_SHAPE, "%s: kernel larger than the padded input", who);
+  const int64_t OH = eh / sh + 1, OW = ew / sw + 1;
+  const int64_t Q = OH * OW, Pg = (C / groups) * KH * KW;
+  DPK_REQUIRE(C * H * W < (1LL << 31) && O * Q < (1LL << 31) && O * Pg < (1LL << 31), DPK_E_SHAPE,
+              "%s: one sample exceeds 2^31 elements", who);
+  DPK_REQUIRE(x && b && gs, DPK_E_ARG, "%s: NULL tensor", who);
+  DPK_REQUIRE(dpk_dtype_ok(in_dtype) && dpk_dtype_ok(gs_dtype), DPK_E_DTYPE, "%s: dtypes %d,%d", who,
+              in_dtype, gs_dtype);
+  DPK_REQUIRE(dpk_aligned(x, dpk_elsize(in_dtype)) && dpk_aligned(b, dpk_elsize(in_dtype)) &&
+                  dpk_aligned(gs, dpk_elsize(gs_dtype)),
+              DPK_E_ALIGN, "%s: misaligned tensor", who);
+  const Plan p = make_plan(O / groups, Pg);
+  const int64_t blocks = n * groups * p.tiles_m * p.tiles_n;
+  DPK_REQUIRE(blocks <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: %lld blocks exceed the grid limit", who,
+              (long long)blocks);
+  float* partials = nullptr;
+  if (sumsq) {
+    const size_t need = static_cast<size_t>(blocks) * sizeof(float);
+    DPK_REQUIRE(ws && ws_bytes >= need, DPK_E_WORKSPACE, "%s: workspace %zu < %zu bytes", who,
+                ws_bytes, need);
+    DPK_REQUIRE(dpk_aligned(ws, 4), DPK_E_ALIGN, "%s: workspace misaligned", who);
+    partials = static_cast<float*>(ws);
+  }
+  ConvGeom g;
+  g.H = (int)H; g.W = (int)W; g.OW = (int)OW; g.Q = (int)Q;
+  g.KH = (int)KH; g.KW = (int)KW; g.Pg = (int)Pg;
+  g.sh = (int)sh; g.sw = (int)sw; g.dh = (int)dh; g.dw = (int)dw;
+  g.ph = (int)ph_lo; g.pw = (int)pw_lo;
+  const bool vec = Q % 4 == 0 && dpk_aligned(b, in_dtype == DPK_BF16 ? 8 : 16);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (in_dtype == DPK_F32 && gs_dtype == DPK_F32)
+    launch<float, float>(p, vec, x, b, gs, partials, g, n, (int)C, (int)O, (int)groups, scale, s);
+  else if (in_dtype == DPK_BF16 && gs_dtype == DPK_BF16)
+    launch<bf16_t, bf16_t>(p, vec, x, b, gs, partials, g, n, (int)C, (int)O, (int)groups, scale, s);
+  else if (in_dtype == DPK_BF16 && gs_dtype == DPK_F32)
+    launch<bf16_t, float>(p, vec, x, b, gs, partials, g, n, (int)C, (int)O, (int)groups, scale, s);
+  else
+    launch<float, bf16_t>(p, vec, x, b, gs, partials, g, n, (int)C, (int)O, (int)groups, scale, s);
+  DPK_LAUNCH_CHECK(who);
+  if (sumsq) {
+    dpk_launch_reduce_rows(partials, n, static_cast<int64_t>(groups) * p.tiles_m * p.tiles_n, sumsq, 0,
+                           1.f, s);
+    DPK_LAUNCH_CHECK(who);
+  }
+  return DPK_OK;
+}

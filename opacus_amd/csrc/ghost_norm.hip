@@ -1,0 +1,229 @@
+// Ghost-clipping per-sample gradient norms of nn.Linear
+// (opacus/grad_sample/linear.py:54-93) without forming the gradients:
+//   |gs_w[n]|_F^2 = sum_{t,t'} (b_t . b_t') (a_t . a_t'),   |gs_b[n]|^2 = sum_{t,t'} b_t . b_t'
+// The reference writes both T x T Gram matrices to memory and reads them back for
+// the elementwise contraction. Here a block owns one (ti, tj) tile pair of one
+// sample: it forms the b b^T tile in MFMA accumulators (k loop over out), then
+// the a a^T tile (k loop over in) - same accumulator layout - multiplies them
+// element by element and reduces. The Grams are symmetric, so only tiles with
+// ti <= tj are visited and off-diagonal ones count twice. One float per block
+// goes to the workspace; a fixed-order reduction applies clamp(min=0) and sqrt
+// (linear.py:87-89, :92).
+#include "dpk_common.h"
+#include "mfma_bf16.h"
+#include "mfma_f32.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / DPK_WAVE;
+
+__device__ __forceinline__ void decode_pair(int pair, int nt, int& ti, int& tj) {
+  ti = 0;
+  while (pair >= nt - ti) {
+    pair -= nt - ti;
+    ++ti;
+  }
+  tj = ti + pair;
+}
+
+// Sums acc_g (.) acc_a and acc_g over the block; thread 0 writes the partials.
+template <class TileT>
+__device__ __forceinline__ void contract_and_store(const TileT& tg, const TileT& ta, bool have_a,
+                                                   float weight, float* pw, float* pb, float* red) {
+  float sw = 0.f, sb = 0.f;
+#pragma unroll
+  for (int i = 0; i < TileT::TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TileT::TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const float g = tg.acc[i][j][v];
+        sb += g;
+        if (have_a) sw = fmaf(g, ta.acc[i][j][v], sw);
+      }
+  if (pw) {
+    const float s = block_sum<kWaves>(sw, red);
+    if (threadIdx.x == 0) pw[blockIdx.x] = s * weight;
+  }
+  if (pb) {
+    const float s = block_sum<kWaves>(sb, red);
+    if (threadIdx.x == 0) pb[blockIdx.x] = s * weight;
+  }
+}
+
+template <int B, bool VEC>
+__global__ __launch_bounds__(kThreads) void ghost_norm_f32_kernel(
+    const float* __restrict__ b, const float* __restrict__ a, float* __restrict__ pw,
+    float* __restrict__ pb, int64_t T, int64_t Dout, int64_t Din, int nt, int npairs) {
+  __shared__ mf32::Smem<B, B> sm;
+  __shared__ float red[kWaves];
+  const int64_t sample = blockIdx.x / npairs;
+  int ti, tj;
+  decode_pair(static_cast<int>(blockIdx.x % npairs), nt, ti, tj);
+  mf32::Tile<B, B> tg, ta;
+  tg.clear();
+  ta.clear();
+  {
+    const float* bs = b + sample * T * Dout;
+    mf32::LoaderKContig<B, float, VEC> la(bs, Dout, static_cast<int64_t>(ti) * B, T, Dout);
+    mf32::LoaderKContig<B, float, VEC> lb(bs, Dout, static_cast<int64_t>(tj) * B, T, Dout);
+    mf32::mainloop<B, B>(tg, sm, la, lb, Dout);
+  }
+  if (pw) {
+    const float* as = a + sample * T * Din;
+    mf32::LoaderKContig<B, float, VEC> la(as, Din, static_cast<int64_t>(ti) * B, T, Din);
+    mf32::LoaderKContig<B, float, VEC> lb(as, Din, static_cast<int64_t>(tj) * B, T, Din);
+    mf32::mainloop<B, B>(ta, sm, la, lb, Din);
+  }
+  contract_and_store(tg, ta, pw != nullptr, ti == tj ? 1.f : 2.f, pw, pb, red);
+}
+
+template <int B, bool VEC>
+__global__ __launch_bounds__(kThreads) void ghost_norm_bf16_kernel(
+    const bf16_t* __restrict__ b, const bf16_t* __restrict__ a, float* __restrict__ pw,
+    float* __restrict__ pb, int64_t T, int64_t Dout, int64_t Din, int nt, int npairs) {
+  __shared__ mb16::Smem<B, B> sm;
+  __shared__ float red[kWaves];
+  const int64_t sample = blockIdx.x / npairs;
+  int ti, tj;
+  decode_pair(static_cast<int>(blockIdx.x % npairs), nt, ti, tj);
+  mb16::Tile<B, B> tg, ta;
+  tg.clear();
+  ta.clear();
+  {
+    const bf16_t* bs = b + sample * T * Dout;
+    mb16::Loader<B, VEC> la(bs, Dout, static_cast<int64_t>(ti) * B, T, Dout);
+    mb16::Loader<B, VEC> lb(bs, Dout, static_cast<int64_t>(tj) * B, T, Dout);
+    mb16::mainloop<B, B>(tg, sm, la, lb, Dout);
+  }
+  if (pw) {
+    const bf16_t* as = a + sample * T * Din;
+    mb16::Loader<B, VEC> la(as, Din, static_cast<int64_t>(ti) * B, T, Din);
+    mb16::Loader<B, VEC> lb(as, Din, static_cast<int64_t>(tj) * B, T, Din);
+    mb16::mainloop<B, B>(ta, sm, la, lb, Din);
+  }
+  contract_and_store(tg, ta, pw != nullptr, ti == tj ? 1.f : 2.f, pw, pb, red);
+}
+
+// T == 1: closed forms of linear.py:71-79. One block per sample.
+template <typename T_>
+__global__ __launch_bounds__(kThreads) void ghost_norm_rank1_kernel(
+    const T_* __restrict__ b, const T_* __restrict__ a, float* __restrict__ nw,
+    float* __restrict__ nb, int64_t Dout, int64_t Din, float absscale) {
+  __shared__ float red[kWaves];
+  const int64_t sample = blockIdx.x;
+  float sb = 0.f, sa = 0.f;
+  for (int64_t i = threadIdx.x; i < Dout; i += kThreads) {
+    const float v = dpk_io<T_>::load(b + sample * Dout + i);
+    sb = fmaf(v, v, sb);
+  }
+  if (nw)
+    for (int64_t i = threadIdx.x; i < Din; i += kThreads) {
+      const float v = dpk_io<T_>::load(a + sample * Din + i);
+      sa = fmaf(v, v, sa);
+    }
+  const float tb = block_sum<kWaves>(sb, red);
+  const float ta = block_sum<kWaves>(sa, red);
+  if (threadIdx.x == 0) {
+    if (nw) nw[sample] = sqrtf(tb * ta) * absscale;
+    if (nb) nb[sample] = sqrtf(tb) * absscale;
+  }
+}
+
+int tile_edge(int64_t T) { return T > 64 ? 128 : 64; }
+
+}  // namespace
+
+extern "C" size_t dpk_linear_ghost_norm_workspace_bytes(int64_t n, int64_t T, int64_t out,
+                                                        int64_t in) {
+  (void)out;
+  (void)in;
+  if (n <= 0 || T <= 1) return 0;
+  // Sized for the smallest tile edge, which has the most tile pairs.
+  const int64_t nt = dpk_cdiv(T, 64);
+  return dpk_align_up(static_cast<size_t>(2 * n * (nt * (nt + 1) / 2)) * sizeof(float), 256);
+}
+
+extern "C" int dpk_linear_ghost_norm(const void* b, const void* a, int dtype, float* norm_w,
+                                     float* norm_b, int64_t n, int64_t T, int64_t out, int64_t in,
+                                     float scale, void* ws, size_t ws_bytes, dpk_stream_t stream) {
+  const char* who = "dpk_linear_ghost_norm";
+  DPK_REQUIRE(n >= 0 && T >= 1 && out >= 1 && in >= 1, DPK_E_SHAPE,
+              "%s: n=%lld T=%lld out=%lld in=%lld", who, (long long)n, (long long)T, (long long)out,
+              (long long)in);
+  if (n == 0 || (!norm_w && !norm_b)) return DPK_OK;
+  DPK_REQUIRE(b && (a || !norm_w), DPK_E_ARG, "%s: NULL tensor", who);
+  DPK_REQUIRE(dpk_dtype_ok(dtype), DPK_E_DTYPE, "%s: dtype %d", who, dtype);
+  DPK_REQUIRE(dpk_aligned(b, dpk_elsize(dtype)) && dpk_aligned(a, dpk_elsize(dtype)), DPK_E_ALIGN,
+              "%s: misaligned tensor", who);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const float absscale = fabsf(scale);
+  if (T == 1) {
+    DPK_REQUIRE(n <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: n too large", who);
+    if (dtype == DPK_F32)
+      hipLaunchKernelGGL(ghost_norm_rank1_kernel<float>, dim3((unsigned)n), dim3(kThreads), 0, s,
+                         static_cast<const float*>(b), static_cast<const float*>(a), norm_w, norm_b,
+                         out, in, absscale);
+    else
+      hipLaunchKernelGGL(ghost_norm_rank1_kernel<bf16_t>, dim3((unsigned)n), dim3(kThreads), 0, s,
+                         static_cast<const bf16_t*>(b), static_cast<const bf16_t*>(a), norm_w, norm_b,
+                         out, in, absscale);
+    DPK_LAUNCH_CHECK(who);
+    return DPK_OK;
+  }
+  const int B = tile_edge(T);
+  const int64_t nt = dpk_cdiv(T, B);
+  const int64_t npairs = nt * (nt + 1) / 2;
+  const int64_t blocks = n * npairs;
+  DPK_REQUIRE(nt < 32768 && blocks <= DPK_MAX_GRID_X, DPK_E_SHAPE,
+              "%s: %lld blocks exceed the grid limit", who, (long long)blocks);
+  const size_t need = static_cast<size_t>(2 * blocks) * sizeof(float);
+  DPK_REQUIRE(ws && ws_bytes >= need, DPK_E_WORKSPACE, "%s: workspace %zu < %zu bytes", who, ws_bytes,
+              need);
+  DPK_REQUIRE(dpk_aligned(ws, 4), DPK_E_ALIGN, "%s: workspace misaligned", who);
+  float* pw = norm_w ? static_cast<float*>(ws) : nullptr;
+  float* pb = norm_b ? static_cast<float*>(ws) + blocks : nullptr;
+  const dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
+  if (dtype == DPK_F32) {
+    const bool vec = out % 4 == 0 && in % 4 == 0 && dpk_aligned(b, 16) && dpk_aligned(a, 16);
+    const float* bp = static_cast<const float*>(b);
+    const float* ap = static_cast<const float*>(a);
+#define DPK_GN_LAUNCH(B_, V_)                                                                 \
+  hipLaunchKernelGGL((ghost_norm_f32_kernel<B_, V_>), grid, block, 0, s, bp, ap, pw, pb, T, out, \
+                     in, (int)nt, (int)npairs)
+    if (B == 128) {
+      if (vec) DPK_GN_LAUNCH(128, true);
+      else DPK_GN_LAUNCH(128, false);
+    } else {
+      if (vec) DPK_GN_LAUNCH(64, true);
+      else DPK_GN_LAUNCH(64, false);
+    }
+#undef DPK_GN_LAUNCH
+  } else {
+    const bool vec = out % 8 == 0 && in % 8 == 0 && dpk_aligned(b, 16) && dpk_aligned(a, 16);
+    const bf16_t* bp = static_cast<const bf16_t*>(b);
+    const bf16_t* ap = static_cast<const bf16_t*>(a);
+#define DPK_GN_LAUNCH(B_, V_)                                                                  \
+  hipLaunchKernelGGL((ghost_norm_bf16_kernel<B_, V_>), grid, block, 0, s, bp, ap, pw, pb, T, out, \
+                     in, (int)nt, (int)npairs)
+    if (B == 128) {
+      if (vec) DPK_GN_LAUNCH(128, true);
+      else DPK_GN_LAUNCH(128, false);
+    } else {
+      if (vec) DPK_GN_LAUNCH(64, true);
+      else DPK_GN_LAUNCH(64, false);
+    }
+#undef DPK_GN_LAUNCH
+  }
+  DPK_LAUNCH_CHECK(who);
+  if (pw) {
+    dpk_launch_reduce_rows(pw, n, npairs, norm_w, 1, absscale, s);
+    DPK_LAUNCH_CHECK(who);
+  }
+  if (pb) {
+    dpk_launch_reduce_rows(pb, n, npairs, norm_b, 1, absscale, s);
+    DPK_LAUNCH_CHECK(who);
+  }
+  return DPK_OK;
+}

@@ -1,0 +1,138 @@
+// bf16 MFMA block-tile machinery for gfx950 (wave64): C[m][n] = sum_k A[m][k] * B[n][k]
+// with both operands stored with k contiguous (rows of a [T, d] matrix), fp32
+// accumulation. A block of 256 threads (4 waves, 2 x 2) owns a BM x BN tile.
+//
+// v_mfma_f32_32x32x16_bf16 operand layout (lane l of 64):
+//   a = A[m = l % 32][k = (l / 32) * 8 .. + 7]   (8 bf16 = 16 bytes, k contiguous)
+//   b = B[n = l % 32][k = (l / 32) * 8 .. + 7]
+//   c[v], v = 0..15: row = (v / 4) * 8 + (l / 32) * 4 + (v % 4), col = l % 32
+// so a k-contiguous row-major tile in LDS feeds the instruction with one 16-byte
+// read per operand and no transposition. LDS rows are padded by 16 bytes to
+// spread the 32 rows a half-wave reads over the banks.
+#pragma once
+
+#include "dpk_common.h"
+
+namespace mb16 {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int BK = 64;        // k extent of a staged tile (bf16 elements)
+constexpr int LDK = BK + 8;   // padded LDS row, in bf16 elements (144 bytes)
+constexpr int NTHREADS = 256;
+
+template <int BM, int BN>
+struct Smem {
+  bf16_t a[2][BM][LDK];
+  bf16_t b[2][BN][LDK];
+};
+
+template <int BM, int BN>
+struct Tile {
+  static constexpr int WM = BM / 2, WN = BN / 2;
+  static constexpr int TM = WM / 32, TN = WN / 32;
+  static_assert(TM >= 1 && TN >= 1, "block tile must be at least 64 x 64");
+  floatx16 acc[TM][TN];
+
+  __device__ __forceinline__ void clear() {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+  }
+
+  __device__ __forceinline__ void mma(const bf16_t (*As)[LDK], const bf16_t (*Bs)[LDK]) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
+    const int kg = (lane >> 5) * 8, l32 = lane & 31;
+#pragma unroll
+    for (int k0 = 0; k0 < BK; k0 += 16) {
+      bf16x8 av[TM], bv[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        av[i] = *reinterpret_cast<const bf16x8*>(&As[wm0 + i * 32 + l32][k0 + kg]);
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        bv[j] = *reinterpret_cast<const bf16x8*>(&Bs[wn0 + j * 32 + l32][k0 + kg]);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[i], bv[j], acc[i][j], 0, 0, 0);
+    }
+  }
+};
+
+// Rows of the source run along k: element (m, k) at base[m * ld + k].
+// VEC: ld % 8 == 0 and base 16-byte aligned, so every 8-element group is one
+// 16-byte load; otherwise elements are fetched one by one with bounds checks.
+template <int BMN, bool VEC>
+struct Loader {
+  static constexpr int R = BMN * BK / 8 / NTHREADS;
+  static_assert(R >= 1, "tile too small for this loader");
+  const bf16_t* base;
+  int64_t ld, m0, M, K;
+  uint4 st[R];
+  __device__ __forceinline__ Loader(const bf16_t* base_, int64_t ld_, int64_t m0_, int64_t M_,
+                                    int64_t K_)
+      : base(base_), ld(ld_), m0(m0_), M(M_), K(K_) {}
+  __device__ __forceinline__ void fetch(int64_t k0) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int idx = threadIdx.x + r * NTHREADS;
+      const int64_t m = m0 + idx / (BK / 8);
+      const int64_t k = k0 + (idx % (BK / 8)) * 8;
+      uint4 v = make_uint4(0u, 0u, 0u, 0u);
+      if (m < M && k < K) {
+        const bf16_t* p = base + m * ld + k;
+        if (VEC) {
+          v = *reinterpret_cast<const uint4*>(p);
+        } else {
+          uint32_t w[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (k + e < K) w[e >> 1] |= static_cast<uint32_t>(p[e]) << ((e & 1) * 16);
+          v = make_uint4(w[0], w[1], w[2], w[3]);
+        }
+      }
+      st[r] = v;
+    }
+  }
+  __device__ __forceinline__ void commit(bf16_t (*S)[LDK]) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int idx = threadIdx.x + r * NTHREADS;
+      *reinterpret_cast<uint4*>(&S[idx / (BK / 8)][(idx % (BK / 8)) * 8]) = st[r];
+    }
+  }
+};
+
+template <int BM, int BN, class LA, class LB>
+__device__ __forceinline__ void mainloop(Tile<BM, BN>& t, Smem<BM, BN>& sm, LA& la, LB& lb,
+                                         int64_t K) {
+  const int64_t nk = (K + BK - 1) / BK;
+  la.fetch(0);
+  lb.fetch(0);
+  la.commit(sm.a[0]);
+  lb.commit(sm.b[0]);
+  __syncthreads();
+  for (int64_t kt = 0; kt < nk; ++kt) {
+    const int cur = static_cast<int>(kt & 1);
+    const bool more = kt + 1 < nk;
+    if (more) {
+      la.fetch((kt + 1) * BK);
+      lb.fetch((kt + 1) * BK);
+    }
+    t.mma(sm.a[cur], sm.b[cur]);
+    if (more) {
+      la.commit(sm.a[cur ^ 1]);
+      lb.commit(sm.b[cur ^ 1]);
+    }
+    __syncthreads();
+  }
+}
+
+}  // namespace mb16

@@ -220,3 +220,100 @@ def test_add_noise_secure_draws_and_dtypes(K):
     gb = torch.empty(P, device="cuda", dtype=torch.bfloat16)
     K.add_noise(s.bfloat16(), gb, std=1.0, denom=1.0, seed=3, offset=10)
     assert abs(gb.double().std().item() - 1.0) < 1e-2
+
+
+# ---- Linear ghost norms --------------------------------------------------------------
+GHOST_SHAPES = [
+    # (n, T, in, out)
+    (5, 1, 40, 24),  # closed form
+    (3, 2, 8, 4),
+    (4, 9, 33, 17),  # odd everything -> scalar loads
+    (2, 64, 128, 64),  # exactly one 64-tile
+    (3, 100, 72, 200),  # 128-tiles, ragged T, one tile pair
+    (2, 300, 136, 264),  # 3 x 3 tile pairs, off-diagonal weights
+    (1, 512, 1024, 256),
+]
+
+
+@pytest.mark.parametrize("n,T,fin,fout", GHOST_SHAPES)
+@pytest.mark.parametrize("scale", [1.0, 4.0])
+def test_linear_ghost_norm_f32(K, n, T, fin, fout, scale):
+    torch.manual_seed(T * 7 + fin)
+    a = torch.randn(n, T, fin)
+    b = torch.randn(n, T, fout) * 0.1
+    # float64 oracle on the 3-d Gram path, and its identity with the materialised gradient
+    want_w, want_b = O.linear_norm_sample(a.double(), (b * scale).double())
+    gs_w, gs_b = O.linear_grad_sample(a.double(), (b * scale).double())
+    torch.testing.assert_close(want_w, gs_w.flatten(1).norm(dim=1), rtol=1e-9, atol=1e-12)
+    nw, nb = K.linear_ghost_norm(dev(b), dev(a), scale=scale, want_weight=True, want_bias=True)
+    assert nw.dtype == torch.float32
+    assert_rel(nw, want_w, FP32_REL, "weight norm")
+    assert_rel(nb, want_b, FP32_REL, "bias norm")
+    only_b = K.linear_ghost_norm(dev(b), dev(a), scale=scale, want_weight=False, want_bias=True)
+    assert only_b[0] is None
+    assert_rel(only_b[1], want_b, FP32_REL, "bias norm alone")
+
+
+def test_linear_ghost_norm_2d_inputs(K):
+    torch.manual_seed(21)
+    a, b = torch.randn(6, 50), torch.randn(6, 30)
+    want_w, want_b = O.linear_norm_sample(a, b)
+    nw, nb = K.linear_ghost_norm(dev(b), dev(a), want_bias=True)
+    assert_rel(nw, want_w, FP32_REL)
+    assert_rel(nb, want_b, FP32_REL)
+
+
+@pytest.mark.parametrize("n,T,fin,fout", [(3, 2, 8, 16), (2, 70, 40, 24), (2, 200, 136, 264), (2, 256, 1024, 512), (3, 33, 30, 18)])
+def test_linear_ghost_norm_bf16(K, n, T, fin, fout):
+    torch.manual_seed(T)
+    a = torch.randn(n, T, fin).bfloat16()
+    b = (torch.randn(n, T, fout) * 0.02).bfloat16()
+    want_w, want_b = O.linear_norm_sample(a.double(), b.double())
+    nw, nb = K.linear_ghost_norm(dev(b), dev(a), want_weight=True, want_bias=True)
+    # inputs are exact in bf16 and accumulation is fp32: far inside the bf16 bar
+    assert_rel(nw, want_w, 1e-4, "weight norm bf16")
+    assert_rel(nb, want_b, 1e-4, "bias norm bf16")
+
+
+# ---- Conv2d ---------------------------------------------------------------------------
+CONV_CASES = [
+    dict(n=3, C=3, O=4, k=(3, 3), stride=(1, 1), padding=(1, 1), dilation=(1, 1), groups=1, H=6, W=7),
+    dict(n=3, C=4, O=6, k=(3, 2), stride=(2, 1), padding=(0, 2), dilation=(1, 2), groups=2, H=9, W=8),
+    dict(n=2, C=2, O=2, k=(2, 3), stride=(1, 2), padding="same", dilation=(2, 1), groups=1, H=7, W=9),
+    dict(n=2, C=6, O=3, k=(1, 1), stride=(1, 1), padding="valid", dilation=(1, 1), groups=3, H=4, W=4),
+    dict(n=4, C=1, O=16, k=(8, 8), stride=(2, 2), padding=(3, 3), dilation=(1, 1), groups=1, H=28, W=28),  # C1 conv1
+    dict(n=4, C=16, O=32, k=(4, 4), stride=(2, 2), padding=(0, 0), dilation=(1, 1), groups=1, H=13, W=13),  # C1 conv2
+    dict(n=2, C=64, O=64, k=(3, 3), stride=(1, 1), padding=(1, 1), dilation=(1, 1), groups=1, H=32, W=32),  # C4
+    dict(n=2, C=24, O=160, k=(3, 3), stride=(1, 1), padding=(1, 1), dilation=(1, 1), groups=1, H=10, W=12),  # 128-tiles
+    dict(n=2, C=16, O=16, k=(3, 3), stride=(1, 1), padding=(1, 1), dilation=(1, 1), groups=16, H=8, W=8),  # depthwise
+]
+
+
+@pytest.mark.parametrize("case", CONV_CASES)
+@pytest.mark.parametrize("scale", [1.0, 2.0])
+def test_conv2d_grad_sample_f32(K, case, scale):
+    torch.manual_seed(case["C"] * 31 + case["O"])
+    n = case["n"]
+    x = torch.randn(n, case["C"], case["H"], case["W"])
+    pad = O.conv2d_padding(case["padding"], case["k"], case["dilation"])
+    oh = (case["H"] + pad[0] + pad[1] - (case["dilation"][0] * (case["k"][0] - 1) + 1)) // case["stride"][0] + 1
+    ow = (case["W"] + pad[2] + pad[3] - (case["dilation"][1] * (case["k"][1] - 1) + 1)) // case["stride"][1] + 1
+    b = torch.randn(n, case["O"], oh, ow)
+    want_w, want_b = O.conv2d_grad_sample(
+        x.double(), (b * scale).double(), kernel_size=case["k"], padding=case["padding"], stride=case["stride"],
+        dilation=case["dilation"], groups=case["groups"],
+    )
+    gs, sumsq = K.conv2d_grad_sample(dev(x), dev(b), case["k"], case["stride"], pad, case["dilation"], case["groups"], scale=scale)
+    assert_rel(gs, want_w, FP32_REL, "conv weight")
+    assert_rel(sumsq, want_w.flatten(1).pow(2).sum(1), 2e-5, "conv sumsq")
+    assert_rel(K.conv_bias_grad_sample(dev(b), scale=scale), want_b, FP32_REL, "conv bias")
+
+
+def test_conv2d_grad_sample_bf16(K):
+    torch.manual_seed(77)
+    x = torch.randn(2, 8, 9, 9).bfloat16()
+    b = torch.randn(2, 12, 9, 9).bfloat16()
+    want_w, _ = O.conv2d_grad_sample(x.double(), b.double(), kernel_size=(3, 3), padding=(1, 1), stride=(1, 1), dilation=(1, 1), groups=1)
+    gs, _ = K.conv2d_grad_sample(dev(x), dev(b), (3, 3), (1, 1), (1, 1, 1, 1), (1, 1), 1)
+    assert gs.dtype == torch.bfloat16
+    assert_rel(gs, want_w, BF16_REL)
