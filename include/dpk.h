@@ -105,7 +105,7 @@ int dpk_linear_ghost_norm(const void* b, const void* a, int dtype, float* norm_w
  * unfold2d computes H_effective/W_effective), gs: [n,O,C/groups,KH,KW].
  * The unfolded activation matrix is never materialised. Padding is given per
  * side so that padding="same" (asymmetric, tensor_utils.py:128-134) is
- * expressible. sumsq as for dpk_linear_gs. fp32 only. */
+ * expressible. sumsq as for dpk_linear_gs. */
 size_t dpk_conv2d_gs_workspace_bytes(int64_t n, int64_t C, int64_t O, int64_t KH, int64_t KW,
                                      int64_t groups);
 int dpk_conv2d_gs(const void* x, const void* b, int in_dtype, void* gs, int gs_dtype, float* sumsq,
@@ -131,7 +131,9 @@ int dpk_conv_bias_gs(const void* b, int in_dtype, void* gs_bias, int gs_dtype, i
  *   unique_pairs[U,2] the list itself (only the first U rows are written)
  *   n_unique[1]       U
  * ids need not lie in any range here. */
-size_t dpk_embedding_workspace_bytes(int64_t n, int64_t T);
+/* One workspace layout serves the three entry points below; pass D = 0 when only
+ * dpk_embedding_unique_pairs is called. The workspace must be 256-byte aligned. */
+size_t dpk_embedding_workspace_bytes(int64_t n, int64_t T, int64_t D);
 int dpk_embedding_unique_pairs(const int64_t* ids, int64_t n, int64_t T, int64_t* inverse,
                                int64_t* unique_pairs, int64_t* n_unique, void* ws,
                                size_t ws_bytes, dpk_stream_t stream);

@@ -1,0 +1,374 @@
+// nn.Embedding on the DP-SGD hot path:
+//   per-sample gradients      opacus/grad_sample/embedding.py:25-64
+//   ghost-clipping norms      opacus/grad_sample/embedding_norm_sample.py:27-151
+// Both need, per sample, the positions grouped by id. The reference sorts
+// (row, id) pairs with torch.unique and scatters with atomics; here each sample
+// gets a linked list per distinct id, built by integer comparisons only:
+//   leader[t] = 1 iff no t' < t in the sample has the same id
+//   next[t]   = the smallest t' > t with the same id, or -1
+// A leader then walks its list in increasing t and sums the backprop rows in
+// registers - a fixed order, no atomics, each row of b read exactly once. The
+// sorted-unique view the reference exposes (unique pairs + inverse index) is
+// derived from the same flags: rank[t] = number of distinct ids below ids[t].
+#include "dpk_common.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / DPK_WAVE;
+constexpr int kIdTile = 2048;  // ids staged in LDS per step of the pairwise scan
+constexpr int kLeadersPerBlock = 16;
+
+struct EmbWs {
+  int32_t* next;
+  int32_t* leader;
+  int32_t* rank;
+  int32_t* count;  // [n] distinct ids per sample
+  int64_t* base;   // [n + 1] exclusive prefix of count
+  int32_t* flag;   // [1] set when an id is outside [0, V)
+  float* partials;
+};
+
+size_t ws_layout(int64_t n, int64_t T, int64_t D, void* ws, EmbWs* out) {
+  const int64_t nt = n * T;
+  size_t off = 0;
+  auto take = [&](size_t bytes) {
+    size_t o = off;
+    off += dpk_align_up(bytes, 256);
+    return o;
+  };
+  const size_t o_next = take(nt * 4), o_leader = take(nt * 4), o_rank = take(nt * 4);
+  const size_t o_count = take(n * 4), o_base = take((n + 1) * 8), o_flag = take(4);
+  const int64_t tch = dpk_cdiv(T, kLeadersPerBlock), dch = dpk_cdiv(D > 0 ? D : 1, kThreads * 4);
+  const size_t o_part = take(n * tch * dch * 4);
+  if (out && ws) {
+    char* p = static_cast<char*>(ws);
+    out->next = reinterpret_cast<int32_t*>(p + o_next);
+    out->leader = reinterpret_cast<int32_t*>(p + o_leader);
+    out->rank = reinterpret_cast<int32_t*>(p + o_rank);
+    out->count = reinterpret_cast<int32_t*>(p + o_count);
+    out->base = reinterpret_cast<int64_t*>(p + o_base);
+    out->flag = reinterpret_cast<int32_t*>(p + o_flag);
+    out->partials = reinterpret_cast<float*>(p + o_part);
+  }
+  return off;
+}
+
+// grid = n * ceil(T / 256); thread <-> one position t of one sample.
+__global__ __launch_bounds__(kThreads) void emb_link_kernel(const int64_t* __restrict__ ids,
+                                                             int64_t T, int64_t V, int blocks_per_sample,
+                                                             int32_t* __restrict__ next,
+                                                             int32_t* __restrict__ leader,
+                                                             int32_t* __restrict__ flag) {
+  __shared__ int64_t tile[kIdTile];
+  const int64_t sample = blockIdx.x / blocks_per_sample;
+  const int64_t t = static_cast<int64_t>(blockIdx.x % blocks_per_sample) * kThreads + threadIdx.x;
+  const int64_t* row = ids + sample * T;
+  const bool live = t < T;
+  const int64_t mine = live ? row[t] : 0;
+  bool seen_before = false;
+  int64_t nxt = -1;
+  for (int64_t c0 = 0; c0 < T; c0 += kIdTile) {
+    const int64_t cn = (T - c0 < kIdTile) ? T - c0 : kIdTile;
+    __syncthreads();
+    for (int64_t i = threadIdx.x; i < cn; i += kThreads) tile[i] = row[c0 + i];
+    __syncthreads();
+    if (live) {
+      for (int64_t i = 0; i < cn; ++i) {
+        const int64_t u = c0 + i;
+        if (tile[i] == mine) {
+          if (u < t) seen_before = true;
+          else if (u > t && nxt < 0) nxt = u;
+        }
+      }
+    }
+  }
+  if (live) {
+    next[sample * T + t] = static_cast<int32_t>(nxt);
+    leader[sample * T + t] = seen_before ? 0 : 1;
+    if (V > 0 && (mine < 0 || mine >= V)) *flag = 1;
+  }
+}
+
+// rank[t] = #{leaders t' of the sample with ids[t'] < ids[t]}; count[sample] = #leaders.
+__global__ __launch_bounds__(kThreads) void emb_rank_kernel(const int64_t* __restrict__ ids, int64_t T,
+                                                             int blocks_per_sample,
+                                                             const int32_t* __restrict__ leader,
+                                                             int32_t* __restrict__ rank,
+                                                             int32_t* __restrict__ count) {
+  __shared__ int64_t tile[kIdTile];
+  __shared__ int32_t lead[kIdTile];
+  const int64_t sample = blockIdx.x / blocks_per_sample;
+  const int bps = static_cast<int>(blockIdx.x % blocks_per_sample);
+  const int64_t t = static_cast<int64_t>(bps) * kThreads + threadIdx.x;
+  const int64_t* row = ids + sample * T;
+  const int32_t* lrow = leader + sample * T;
+  const bool live = t < T;
+  const int64_t mine = live ? row[t] : 0;
+  int32_t below = 0, total = 0;
+  for (int64_t c0 = 0; c0 < T; c0 += kIdTile) {
+    const int64_t cn = (T - c0 < kIdTile) ? T - c0 : kIdTile;
+    __syncthreads();
+    for (int64_t i = threadIdx.x; i < cn; i += kThreads) {
+      tile[i] = row[c0 + i];
+      lead[i] = lrow[c0 + i];
+    }
+    __syncthreads();
+    for (int64_t i = 0; i < cn; ++i) {
+      total += lead[i];
+      if (lead[i] && tile[i] < mine) ++below;
+    }
+  }
+  if (live) rank[sample * T + t] = below;
+  if (bps == 0 && threadIdx.x == 0) count[sample] = total;
+}
+
+// One block: base = exclusive prefix of count over samples (sequential: n is a batch size).
+__global__ void emb_prefix_kernel(const int32_t* __restrict__ count, int64_t n,
+                                  int64_t* __restrict__ base, int64_t* __restrict__ n_unique) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  int64_t acc = 0;
+  for (int64_t i = 0; i < n; ++i) {
+    base[i] = acc;
+    acc += count[i];
+  }
+  base[n] = acc;
+  *n_unique = acc;
+}
+
+__global__ __launch_bounds__(kThreads) void emb_emit_pairs_kernel(
+    const int64_t* __restrict__ ids, int64_t n, int64_t T, const int32_t* __restrict__ leader,
+    const int32_t* __restrict__ rank, const int64_t* __restrict__ base, int64_t* __restrict__ inverse,
+    int64_t* __restrict__ pairs) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (i >= n * T) return;
+  const int64_t sample = i / T;
+  const int64_t pos = base[sample] + rank[i];
+  inverse[i] = pos;
+  if (leader[i]) {
+    pairs[2 * pos] = sample;
+    pairs[2 * pos + 1] = ids[i];
+  }
+}
+
+// grid = n * tch * dch. A block owns kLeadersPerBlock positions and 1024 columns;
+// thread <-> 4 columns. MODE 0: sum of squares of the per-id sums (ghost norm).
+// MODE 1: write scale * sum into gs[sample, id, :].
+template <typename TIN, typename TOUT, int MODE, bool VEC>
+__global__ __launch_bounds__(kThreads) void emb_walk_kernel(
+    const int64_t* __restrict__ ids, const TIN* __restrict__ b, const int32_t* __restrict__ next,
+    const int32_t* __restrict__ leader, int64_t T, int64_t D, int64_t V, int tch, int dch,
+    float scale, float* __restrict__ partials, TOUT* __restrict__ gs) {
+  __shared__ float red[kWaves];
+  int64_t bid = blockIdx.x;
+  const int dc = static_cast<int>(bid % dch);
+  bid /= dch;
+  const int tc = static_cast<int>(bid % tch);
+  const int64_t sample = bid / tch;
+  const int64_t d = (static_cast<int64_t>(dc) * kThreads + threadIdx.x) * 4;
+  const int64_t t0 = static_cast<int64_t>(tc) * kLeadersPerBlock;
+  const int64_t t1 = (t0 + kLeadersPerBlock < T) ? t0 + kLeadersPerBlock : T;
+  const TIN* bs = b + sample * T * D;
+  const int32_t* nx = next + sample * T;
+  const int32_t* ld = leader + sample * T;
+  float ss = 0.f;
+  for (int64_t t = t0; t < t1; ++t) {
+    if (!ld[t]) continue;  // uniform over the block
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (d < D) {
+      for (int64_t u = t; u >= 0; u = nx[u]) {
+        const TIN* p = bs + u * D + d;
+        if (VEC) {
+          const float4 v = dpk_io<TIN>::load4(p);
+          acc.x += v.x;
+          acc.y += v.y;
+          acc.z += v.z;
+          acc.w += v.w;
+        } else {
+          acc.x += dpk_io<TIN>::load(p);
+          if (d + 1 < D) acc.y += dpk_io<TIN>::load(p + 1);
+          if (d + 2 < D) acc.z += dpk_io<TIN>::load(p + 2);
+          if (d + 3 < D) acc.w += dpk_io<TIN>::load(p + 3);
+        }
+      }
+    }
+    if (MODE == 0) {
+      ss += (acc.x * acc.x + acc.y * acc.y) + (acc.z * acc.z + acc.w * acc.w);
+    } else if (d < D) {
+      const int64_t id = ids[sample * T + t];
+      if (id >= 0 && id < V) {
+        TOUT* o = gs + (sample * V + id) * D + d;
+        acc.x *= scale;
+        acc.y *= scale;
+        acc.z *= scale;
+        acc.w *= scale;
+        if (VEC) {
+          dpk_io<TOUT>::store4(o, acc);
+        } else {
+          dpk_io<TOUT>::store(o, acc.x);
+          if (d + 1 < D) dpk_io<TOUT>::store(o + 1, acc.y);
+          if (d + 2 < D) dpk_io<TOUT>::store(o + 2, acc.z);
+          if (d + 3 < D) dpk_io<TOUT>::store(o + 3, acc.w);
+        }
+      }
+    }
+  }
+  if (MODE == 0) {
+    const float s = block_sum<kWaves>(ss, red);
+    if (threadIdx.x == 0) partials[blockIdx.x] = s;
+  }
+}
+
+// Zero fill with 16-byte stores (a kernel rather than a memset node, so that a
+// caller may capture the stream into a graph).
+__global__ __launch_bounds__(kThreads) void zero_fill_kernel(uint4* __restrict__ p, int64_t n16,
+                                                              unsigned char* __restrict__ tail,
+                                                              int64_t ntail) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < n16; i += stride)
+    p[i] = make_uint4(0u, 0u, 0u, 0u);
+  if (blockIdx.x == 0 && threadIdx.x < ntail) tail[threadIdx.x] = 0;
+}
+
+__global__ void zero_flag_kernel(int32_t* flag) { *flag = 0; }
+
+int check_common(const char* who, const int64_t* ids, int64_t n, int64_t T, int64_t D, void* ws,
+                 size_t ws_bytes, EmbWs* w) {
+  DPK_REQUIRE(ids, DPK_E_ARG, "%s: ids is NULL", who);
+  DPK_REQUIRE(dpk_aligned(ids, 8), DPK_E_ALIGN, "%s: ids misaligned", who);
+  DPK_REQUIRE(T < (1LL << 31) && n * dpk_cdiv(T, kThreads) <= DPK_MAX_GRID_X, DPK_E_SHAPE,
+              "%s: n=%lld T=%lld too large", who, (long long)n, (long long)T);
+  const size_t need = ws_layout(n, T, D, nullptr, nullptr);
+  DPK_REQUIRE(ws && ws_bytes >= need, DPK_E_WORKSPACE, "%s: workspace %zu < %zu bytes", who, ws_bytes,
+              need);
+  DPK_REQUIRE(dpk_aligned(ws, 256), DPK_E_ALIGN, "%s: workspace must be 256-byte aligned", who);
+  ws_layout(n, T, D, ws, w);
+  return DPK_OK;
+}
+
+void launch_link(const int64_t* ids, int64_t n, int64_t T, int64_t V, const EmbWs& w, hipStream_t s) {
+  const int bps = static_cast<int>(dpk_cdiv(T, kThreads));
+  hipLaunchKernelGGL(zero_flag_kernel, dim3(1), dim3(1), 0, s, w.flag);
+  hipLaunchKernelGGL(emb_link_kernel, dim3(static_cast<unsigned>(n * bps)), dim3(kThreads), 0, s, ids, T,
+                     V, bps, w.next, w.leader, w.flag);
+}
+
+template <typename TIN, typename TOUT, int MODE>
+void launch_walk(bool vec, const int64_t* ids, const void* b, const EmbWs& w, int64_t n, int64_t T,
+                 int64_t D, int64_t V, float scale, void* gs, hipStream_t s) {
+  const int tch = static_cast<int>(dpk_cdiv(T, kLeadersPerBlock));
+  const int dch = static_cast<int>(dpk_cdiv(D, kThreads * 4));
+  const dim3 grid(static_cast<unsigned>(n * tch * dch)), block(kThreads);
+  if (vec)
+    hipLaunchKernelGGL((emb_walk_kernel<TIN, TOUT, MODE, true>), grid, block, 0, s, ids,
+                       static_cast<const TIN*>(b), w.next, w.leader, T, D, V, tch, dch, scale,
+                       w.partials, static_cast<TOUT*>(gs));
+  else
+    hipLaunchKernelGGL((emb_walk_kernel<TIN, TOUT, MODE, false>), grid, block, 0, s, ids,
+                       static_cast<const TIN*>(b), w.next, w.leader, T, D, V, tch, dch, scale,
+                       w.partials, static_cast<TOUT*>(gs));
+}
+
+}  // namespace
+
+extern "C" size_t dpk_embedding_workspace_bytes(int64_t n, int64_t T, int64_t D) {
+  if (n <= 0 || T <= 0) return 0;
+  return ws_layout(n, T, D, nullptr, nullptr);
+}
+
+extern "C" int dpk_embedding_unique_pairs(const int64_t* ids, int64_t n, int64_t T,
+                                          int64_t* inverse, int64_t* unique_pairs,
+                                          int64_t* n_unique, void* ws, size_t ws_bytes,
+                                          dpk_stream_t stream) {
+  const char* who = "dpk_embedding_unique_pairs";
+  DPK_REQUIRE(n >= 0 && T >= 0, DPK_E_SHAPE, "%s: n=%lld T=%lld", who, (long long)n, (long long)T);
+  if (n == 0 || T == 0) return DPK_OK;
+  DPK_REQUIRE(inverse && unique_pairs && n_unique, DPK_E_ARG, "%s: NULL output", who);
+  EmbWs w;
+  int rc = check_common(who, ids, n, T, 0, ws, ws_bytes, &w);
+  if (rc != DPK_OK) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  launch_link(ids, n, T, 0, w, s);
+  DPK_LAUNCH_CHECK(who);
+  const int bps = static_cast<int>(dpk_cdiv(T, kThreads));
+  hipLaunchKernelGGL(emb_rank_kernel, dim3(static_cast<unsigned>(n * bps)), dim3(kThreads), 0, s, ids, T,
+                     bps, w.leader, w.rank, w.count);
+  hipLaunchKernelGGL(emb_prefix_kernel, dim3(1), dim3(64), 0, s, w.count, n, w.base, n_unique);
+  hipLaunchKernelGGL(emb_emit_pairs_kernel, dim3(static_cast<unsigned>(dpk_cdiv(n * T, kThreads))),
+                     dim3(kThreads), 0, s, ids, n, T, w.leader, w.rank, w.base, inverse, unique_pairs);
+  DPK_LAUNCH_CHECK(who);
+  return DPK_OK;
+}
+
+extern "C" int dpk_embedding_ghost_norm(const int64_t* ids, const void* b, int dtype, float* norm,
+                                        int64_t n, int64_t T, int64_t D, float scale, void* ws,
+                                        size_t ws_bytes, dpk_stream_t stream) {
+  const char* who = "dpk_embedding_ghost_norm";
+  DPK_REQUIRE(n >= 0 && T >= 1 && D >= 1, DPK_E_SHAPE, "%s: n=%lld T=%lld D=%lld", who, (long long)n,
+              (long long)T, (long long)D);
+  if (n == 0) return DPK_OK;
+  DPK_REQUIRE(b && norm, DPK_E_ARG, "%s: NULL tensor", who);
+  DPK_REQUIRE(dpk_dtype_ok(dtype), DPK_E_DTYPE, "%s: dtype %d", who, dtype);
+  DPK_REQUIRE(dpk_aligned(b, dpk_elsize(dtype)), DPK_E_ALIGN, "%s: misaligned tensor", who);
+  EmbWs w;
+  int rc = check_common(who, ids, n, T, D, ws, ws_bytes, &w);
+  if (rc != DPK_OK) return rc;
+  const int64_t tch = dpk_cdiv(T, kLeadersPerBlock), dch = dpk_cdiv(D, kThreads * 4);
+  DPK_REQUIRE(n * tch * dch <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: too many blocks", who);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  launch_link(ids, n, T, 0, w, s);
+  DPK_LAUNCH_CHECK(who);
+  const bool vec = D % 4 == 0 && dpk_aligned(b, dtype == DPK_BF16 ? 8 : 16);
+  if (dtype == DPK_F32) launch_walk<float, float, 0>(vec, ids, b, w, n, T, D, 0, scale, nullptr, s);
+  else launch_walk<bf16_t, float, 0>(vec, ids, b, w, n, T, D, 0, scale, nullptr, s);
+  DPK_LAUNCH_CHECK(who);
+  dpk_launch_reduce_rows(w.partials, n, tch * dch, norm, 1, fabsf(scale), s);
+  DPK_LAUNCH_CHECK(who);
+  return DPK_OK;
+}
+
+extern "C" int dpk_embedding_gs(const int64_t* ids, const void* b, int in_dtype, void* gs,
+                                int gs_dtype, int64_t n, int64_t T, int64_t V, int64_t D,
+                                float scale, void* ws, size_t ws_bytes, dpk_stream_t stream) {
+  const char* who = "dpk_embedding_gs";
+  DPK_REQUIRE(n >= 0 && T >= 1 && V >= 1 && D >= 1, DPK_E_SHAPE, "%s: n=%lld T=%lld V=%lld D=%lld", who,
+              (long long)n, (long long)T, (long long)V, (long long)D);
+  if (n == 0) return DPK_OK;
+  DPK_REQUIRE(b && gs, DPK_E_ARG, "%s: NULL tensor", who);
+  DPK_REQUIRE(dpk_dtype_ok(in_dtype) && in_dtype == gs_dtype, DPK_E_DTYPE,
+              "%s: dtypes %d,%d (must be equal)", who, in_dtype, gs_dtype);
+  DPK_REQUIRE(dpk_aligned(b, dpk_elsize(in_dtype)) && dpk_aligned(gs, dpk_elsize(gs_dtype)),
+              DPK_E_ALIGN, "%s: misaligned tensor", who);
+  EmbWs w;
+  int rc = check_common(who, ids, n, T, D, ws, ws_bytes, &w);
+  if (rc != DPK_OK) return rc;
+  const int64_t tch = dpk_cdiv(T, kLeadersPerBlock), dch = dpk_cdiv(D, kThreads * 4);
+  DPK_REQUIRE(n * tch * dch <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: too many blocks", who);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  launch_link(ids, n, T, V, w, s);
+  DPK_LAUNCH_CHECK(who);
+  // Ids outside [0, V) would address memory outside gs: find out before writing.
+  int32_t flag = 0;
+  hipError_t e = hipMemcpyAsync(&flag, w.flag, sizeof(flag), hipMemcpyDeviceToHost, s);
+  if (e == hipSuccess) e = hipStreamSynchronize(s);
+  DPK_REQUIRE(e == hipSuccess, DPK_E_LAUNCH, "%s: %s", who, hipGetErrorString(e));
+  DPK_REQUIRE(flag == 0, DPK_E_ARG, "%s: an id lies outside [0, %lld)", who, (long long)V);
+  const size_t bytes = static_cast<size_t>(n) * V * D * dpk_elsize(gs_dtype);
+  const int64_t n16 = dpk_aligned(gs, 16) ? static_cast<int64_t>(bytes / 16) : 0;
+  const int64_t ntail = static_cast<int64_t>(bytes - static_cast<size_t>(n16) * 16);
+  if (n16 > 0 || ntail > 0) {
+    DPK_REQUIRE(ntail < kThreads, DPK_E_ALIGN, "%s: gs must be 16-byte aligned", who);
+    int64_t blocks = dpk_cdiv(n16 > 0 ? n16 : 1, kThreads * 4);
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL(zero_fill_kernel, dim3(static_cast<unsigned>(blocks)), dim3(kThreads), 0, s,
+                       static_cast<uint4*>(gs), n16,
+                       static_cast<unsigned char*>(gs) + static_cast<size_t>(n16) * 16, ntail);
+    DPK_LAUNCH_CHECK(who);
+  }
+  const bool vec = D % 4 == 0 && dpk_aligned(b, in_dtype == DPK_BF16 ? 8 : 16) &&
+                   dpk_aligned(gs, gs_dtype == DPK_BF16 ? 8 : 16);
+  if (in_dtype == DPK_F32) launch_walk<float, float, 1>(vec, ids, b, w, n, T, D, V, scale, gs, s);
+  else launch_walk<bf16_t, bf16_t, 1>(vec, ids, b, w, n, T, D, V, scale, gs, s);
+  DPK_LAUNCH_CHECK(who);
+  return DPK_OK;
+}

@@ -278,7 +278,7 @@ def embedding_unique_pairs(ids: torch.Tensor) -> Tuple[torch.Tensor, torch.Tenso
     if n * T == 0:
         return pairs[:0], inverse
     L = lib()
-    ws, wsb = _ws(L.dpk_embedding_workspace_bytes(n, T), dev)
+    ws, wsb = _ws(L.dpk_embedding_workspace_bytes(n, T, 0), dev)
     with _timed("embedding_unique_pairs", dev):
         check(
             "dpk_embedding_unique_pairs",
@@ -304,7 +304,7 @@ def embedding_grad_sample(
     if b.shape[1] != T:
         raise ValueError(f"ids {tuple(ids.shape)} and backprops {tuple(backprops.shape)} disagree")
     L = lib()
-    ws, wsb = _ws(L.dpk_embedding_workspace_bytes(n, T), dev)
+    ws, wsb = _ws(L.dpk_embedding_workspace_bytes(n, T, D), dev)
     with _timed("embedding_gs", dev):
         check(
             "dpk_embedding_gs",
@@ -329,7 +329,7 @@ def embedding_ghost_norm(ids: torch.Tensor, backprops: torch.Tensor, scale: floa
     if b.shape[1] != T:
         raise ValueError(f"ids {tuple(ids.shape)} and backprops {tuple(backprops.shape)} disagree")
     L = lib()
-    ws, wsb = _ws(L.dpk_embedding_workspace_bytes(n, T), dev)
+    ws, wsb = _ws(L.dpk_embedding_workspace_bytes(n, T, D), dev)
     with _timed("embedding_ghost_norm", dev):
         check(
             "dpk_embedding_ghost_norm",

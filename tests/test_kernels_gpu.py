@@ -317,3 +317,104 @@ def test_conv2d_grad_sample_bf16(K):
     gs, _ = K.conv2d_grad_sample(dev(x), dev(b), (3, 3), (1, 1), (1, 1, 1, 1), (1, 1), 1)
     assert gs.dtype == torch.bfloat16
     assert_rel(gs, want_w, BF16_REL)
+
+
+# ---- Embedding ------------------------------------------------------------------------
+def test_embedding_golden_vectors(K, embedding_norm_cases):
+    """The reference's own known-answer triples and docstring intermediates, on the GPU."""
+    for c in embedding_norm_cases:
+        norm = K.embedding_ghost_norm(dev(c["ids"]), dev(c["backprops"]))
+        torch.testing.assert_close(norm.cpu(), c["expected"], atol=1e-4, rtol=1e-4, msg=c["name"])
+        if c["intermediates"]:
+            pairs, inverse = K.embedding_unique_pairs(dev(c["ids"]))
+            assert pairs.cpu().tolist() == c["intermediates"]["unique_paired_indices"]
+            assert inverse.cpu().tolist() == c["intermediates"]["new_index_positions"]
+
+
+@pytest.mark.parametrize("n,T,V", [(1, 1, 1), (7, 10, 6), (3, 300, 50), (2, 2500, 4000), (4, 513, 3)])
+def test_embedding_unique_pairs_bit_exact(K, n, T, V):
+    torch.manual_seed(n * T)
+    ids = torch.randint(0, V, (n, T))
+    want_pairs, want_inv = O.embedding_unique_pairs(ids)
+    pairs, inverse = K.embedding_unique_pairs(dev(ids))
+    assert torch.equal(pairs.cpu(), want_pairs)
+    assert torch.equal(inverse.cpu(), want_inv)
+
+
+def test_embedding_unique_pairs_any_integer_ids(K):
+    ids = torch.tensor([[-5, 2**40, -5, 7], [7, 7, -(2**50), 0]])
+    want_pairs, want_inv = O.embedding_unique_pairs(ids)
+    pairs, inverse = K.embedding_unique_pairs(dev(ids))
+    assert torch.equal(pairs.cpu(), want_pairs) and torch.equal(inverse.cpu(), want_inv)
+
+
+@pytest.mark.parametrize("n,Tshape,V,D", [(5, (3, 2), 9, 4), (3, (40,), 7, 17), (2, (300,), 5000, 64), (2, (64,), 10, 1030)])
+@pytest.mark.parametrize("scale", [1.0, 5.0])
+def test_embedding_grad_sample_and_norm_f32(K, n, Tshape, V, D, scale):
+    torch.manual_seed(V + D)
+    ids = torch.randint(0, V, (n, *Tshape))
+    b = torch.randn(n, *Tshape, D)
+    want = O.embedding_grad_sample(ids, b * scale, V)
+    gs = K.embedding_grad_sample(dev(ids), dev(b), V, scale=scale)
+    assert_rel(gs, want, FP32_REL, "embedding gs")
+    # which rows are touched is integer work: exact
+    assert torch.equal((gs != 0).any(dim=2).cpu(), (want != 0).any(dim=2))
+    want_norm = O.embedding_norm_sample(ids, (b * scale).double())["result_sqrt"]
+    norm = K.embedding_ghost_norm(dev(ids), dev(b), scale=scale)
+    assert_rel(norm, want_norm, FP32_REL, "embedding norm")
+
+
+def test_embedding_bf16(K):
+    torch.manual_seed(5)
+    ids = torch.randint(0, 11, (3, 50))
+    b = torch.randn(3, 50, 24).bfloat16()
+    want = O.embedding_grad_sample(ids, b.double(), 11)
+    gs = K.embedding_grad_sample(dev(ids), dev(b), 11)
+    assert gs.dtype == torch.bfloat16
+    assert_rel(gs, want, BF16_REL)
+    norm = K.embedding_ghost_norm(dev(ids), dev(b))
+    assert_rel(norm, want.flatten(1).norm(dim=1), 1e-4)
+
+
+def test_embedding_out_of_range_id_is_an_error(K):
+    from opacus_amd._lib import DpkError
+
+    ids = torch.tensor([[0, 3, 9]])
+    with pytest.raises(DpkError, match="outside"):
+        K.embedding_grad_sample(dev(ids), torch.zeros(1, 3, 4, device="cuda"), 9)
+
+
+# ---- Normalisation layers ---------------------------------------------------------------
+@pytest.mark.parametrize("n,C,G,spatial", [(4, 6, 2, (3, 5)), (3, 64, 32, (32, 32)), (2, 8, 1, (7,)), (2, 10, 10, (4, 4)), (2, 256, 4, ())])
+@pytest.mark.parametrize("scale", [1.0, 3.0])
+def test_group_norm_grad_sample_f32(K, n, C, G, spatial, scale):
+    torch.manual_seed(C + G)
+    x = torch.randn(n, C, *spatial) * 2 + 0.5
+    b = torch.randn(n, C, *spatial)
+    want_w, want_b = O.group_norm_grad_sample(x.double(), (b * scale).double(), G, 1e-5)
+    gw, gb = K.group_norm_grad_sample(dev(x), dev(b), G, 1e-5, scale=scale)
+    assert_rel(gw, want_w, FP32_REL, "gn weight")
+    assert_rel(gb, want_b, FP32_REL, "gn bias")
+
+
+@pytest.mark.parametrize("shape,D", [((4, 8), 8), ((3, 5, 8), 8), ((2, 3, 4, 16), 16), ((2, 200, 260), 260), ((2, 130, 33), 33)])
+def test_rms_norm_grad_sample_f32(K, shape, D):
+    torch.manual_seed(D)
+    x = torch.randn(*shape) + 0.3
+    b = torch.randn(*shape)
+    want = O.rms_norm_grad_sample(x.double(), b.double(), (D,), 1e-6)
+    got = K.rms_norm_grad_sample(dev(x), dev(b), D, 1e-6)
+    assert_rel(got, want, FP32_REL, "rms weight")
+
+
+def test_norm_layers_bf16(K):
+    torch.manual_seed(3)
+    x = torch.randn(2, 70, 64).bfloat16()
+    b = torch.randn(2, 70, 64).bfloat16()
+    want = O.rms_norm_grad_sample(x.double(), b.double(), (64,), 1e-6)
+    assert_rel(K.rms_norm_grad_sample(dev(x), dev(b), 64, 1e-6), want, BF16_REL)
+    x4, b4 = torch.randn(2, 8, 6, 6).bfloat16(), torch.randn(2, 8, 6, 6).bfloat16()
+    want_w, want_b = O.group_norm_grad_sample(x4.double(), b4.double(), 4, 1e-5)
+    gw, gb = K.group_norm_grad_sample(dev(x4), dev(b4), 4, 1e-5)
+    assert_rel(gw, want_w, BF16_REL)
+    assert_rel(gb, want_b, BF16_REL)
