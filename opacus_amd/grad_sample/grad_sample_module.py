@@ -1,0 +1,310 @@
+"""Hooks-based per-sample-gradient engine (mirror of opacus/grad_sample/grad_sample_module.py).
+
+Forward hooks keep the detached inputs of every layer that owns trainable parameters;
+full-backward hooks hand those inputs and the layer's output gradient to the layer's
+registered sampler, which launches the HIP kernels, and file the result under
+``p.grad_sample``.
+
+Two passes of the reference over per-sample data are gone here:
+  * the multiplication of the backprops by the batch size for a mean-reduced loss
+    (grad_sample_module.py:402-406) is passed to the kernels as a scalar when the
+    sampler accepts one (``fused_scale``);
+  * the zero-filled ``[max_batch_len, ...]`` buffer and the copy into it
+    (grad_sample_module.py:61-66) are skipped when the sampler's tensor already has that
+    batch length and is the sampler's own fresh output (``owns_output``).
+"""
+
+from __future__ import annotations
+
+import logging
+import warnings
+from functools import partial
+from typing import Callable, Iterable, List, Tuple
+
+import torch
+import torch.nn as nn
+
+from ..utils.module_utils import has_trainable_params, requires_grad, trainable_modules, trainable_parameters
+from .functorch import ft_compute_per_sample_gradient, prepare_layer
+from .gsm_base import AbstractGradSampleHooks, AbstractGradSampleModule
+
+logger = logging.getLogger(__name__)
+logger.disabled = True
+
+
+def fused_scale(fn: Callable) -> Callable:
+    """Marks a sampler that takes ``scale=`` and applies it to the backprops inside its kernels."""
+    fn.accepts_scale = True
+    return fn
+
+
+def owns_output(fn: Callable) -> Callable:
+    """Marks a sampler whose returned tensors are fresh allocations nobody else refers to."""
+    fn.owns_output = True
+    return fn
+
+
+def call_sampler(fn: Callable, module: nn.Module, activations, backprops: torch.Tensor, scale: float):
+    """Calls a grad or norm sampler, folding ``scale`` into it if it can take it."""
+    if getattr(fn, "accepts_scale", False):
+        return fn(module, activations, backprops, scale=scale)
+    if scale != 1.0:
+        backprops = backprops * scale
+    return fn(module, activations, backprops)
+
+
+def create_or_accumulate_grad_sample(
+    *, param: torch.Tensor, grad_sample: torch.Tensor, max_batch_len: int, adopt: bool = False
+) -> None:
+    """Starts or continues ``param._current_grad_sample`` for the backward pass in flight.
+
+    A later result for the same parameter in the same pass (tied weights, recurrent steps)
+    is added into the first ``len(grad_sample)`` rows (grad_sample_module.py:58-59). The
+    first result is copied into a zero-filled ``[max_batch_len, ...]`` buffer (:61-66),
+    unless ``adopt`` says the tensor may be kept as it is.
+    """
+    if not param.requires_grad:
+        return
+    if hasattr(param, "_current_grad_sample"):
+        param._current_grad_sample[: grad_sample.shape[0]] += grad_sample
+    elif adopt and grad_sample.shape[0] == max_batch_len:
+        param._current_grad_sample = grad_sample
+    else:
+        buf = torch.zeros(
+            torch.Size([max_batch_len]) + grad_sample.shape[1:], device=grad_sample.device, dtype=grad_sample.dtype
+        )
+        buf[: grad_sample.shape[0]] = grad_sample
+        param._current_grad_sample = buf
+
+
+def promote_current_grad_sample(p: nn.Parameter) -> None:
+    """Moves the finished pass's tensor to ``p.grad_sample``; a second pass makes it a list (:69-79)."""
+    if not p.requires_grad:
+        return
+    if p.grad_sample is None:
+        p.grad_sample = p._current_grad_sample
+    elif isinstance(p.grad_sample, list):
+        p.grad_sample.append(p._current_grad_sample)
+    else:
+        p.grad_sample = [p.grad_sample, p._current_grad_sample]
+    del p._current_grad_sample
+
+
+def _get_batch_size(*, module: nn.Module, batch_dim: int) -> int:
+    """Largest batch length among the pending activations of ``module`` (:552-573)."""
+    return max((acts[-1].shape[batch_dim] for acts in module.activations), default=0)
+
+
+def _batch_first_view(t: torch.Tensor, batch_dim: int) -> torch.Tensor:
+    return t.permute([batch_dim] + [d for d in range(t.dim()) if d != batch_dim])
+
+
+class GradSampleHooks(AbstractGradSampleHooks):
+    """Attaches per-sample-gradient hooks to a module without wrapping it."""
+
+    GRAD_SAMPLERS = {}
+
+    def __init__(
+        self,
+        m: nn.Module,
+        *,
+        batch_first=True,
+        loss_reduction="mean",
+        strict: bool = True,
+        force_functorch=False,
+    ):
+        super().__init__(m, batch_first=batch_first, loss_reduction=loss_reduction)
+        errors = self.validate(module=m, strict=strict)
+        if errors and not strict:
+            logger.info(f"Validation found the following errors: {errors}. Using non-strict mode, continuing")
+        self.hooks_enabled = False
+        self.grad_accumulation_allowed = True
+        self.force_functorch = force_functorch
+        self.add_hooks(loss_reduction=loss_reduction, batch_first=batch_first, force_functorch=force_functorch)
+
+    # ---- hook installation -----------------------------------------------------------
+    def _get_module_type(self, module: nn.Module):
+        return type(module)
+
+    def iterate_submodules(self, module: nn.Module) -> Iterable[nn.Module]:
+        """Modules that get hooks: every one with trainable parameters of its own. Below a
+        module that has them but no registered sampler nothing is visited: the generic
+        fallback differentiates that whole subtree (grad_sample_module.py:152-165)."""
+        own = has_trainable_params(module)
+        if own:
+            yield module
+            if self._get_module_type(module) not in self.GRAD_SAMPLERS:
+                return
+        for child in module.children():
+            yield from self.iterate_submodules(child)
+
+    def add_hooks(self, *, loss_reduction: str = "mean", batch_first: bool = True, force_functorch: bool = False) -> None:
+        if hasattr(self._module, "autograd_grad_sample_hooks"):
+            raise ValueError("Trying to add hooks twice to the same model")
+        self._module.autograd_grad_sample_hooks = []
+        self.autograd_grad_sample_hooks = self._module.autograd_grad_sample_hooks
+        for module in self.iterate_submodules(self._module):
+            if force_functorch or self._get_module_type(module) not in self.GRAD_SAMPLERS:
+                prepare_layer(module, batch_first=batch_first)
+            self.autograd_grad_sample_hooks.append(module.register_forward_hook(self.capture_activations_hook))
+            self.autograd_grad_sample_hooks.append(
+                module.register_full_backward_hook(
+                    partial(self.capture_backprops_hook, loss_reduction=loss_reduction, batch_first=batch_first)
+                )
+            )
+        self.enable_hooks()
+
+    def remove_hooks(self) -> None:
+        self.disable_hooks()
+        for p in self._module.parameters():
+            if hasattr(p, "ddp_hooks"):
+                while p.ddp_hooks:
+                    p.ddp_hooks.pop().remove()
+                delattr(p, "ddp_hooks")
+        if hasattr(self, "autograd_grad_sample_hooks"):
+            while self.autograd_grad_sample_hooks:
+                self.autograd_grad_sample_hooks.pop().remove()
+            delattr(self, "autograd_grad_sample_hooks")
+            if hasattr(self._module, "autograd_grad_sample_hooks"):
+                delattr(self._module, "autograd_grad_sample_hooks")
+        for _, module in trainable_modules(self._module):
+            if hasattr(module, "ft_compute_sample_grad"):
+                delattr(module, "ft_compute_sample_grad")
+
+    def disable_hooks(self) -> None:
+        """Hooks stay installed (autograd keeps those of a built graph anyway) but do nothing."""
+        self.hooks_enabled = False
+
+    def enable_hooks(self) -> None:
+        self.hooks_enabled = True
+
+    # ---- the hooks ----------------------------------------------------------------------
+    def capture_activations_hook(self, module: nn.Module, forward_input: List[torch.Tensor], _forward_output):
+        if not requires_grad(module) or not module.training or not torch.is_grad_enabled():
+            return
+        if not self.hooks_enabled:
+            return
+        if not hasattr(module, "activations"):
+            module.activations = []
+        module.activations.append([t.detach() for t in forward_input])
+        for _, p in trainable_parameters(module):
+            p._forward_counter += 1
+
+    def _sampler_for(self, module: nn.Module) -> Callable:
+        if not self.force_functorch and self._get_module_type(module) in self.GRAD_SAMPLERS:
+            return self.GRAD_SAMPLERS[self._get_module_type(module)]
+        return ft_compute_per_sample_gradient
+
+    def capture_backprops_hook(
+        self, module: nn.Module, _forward_input, forward_output, loss_reduction: str, batch_first: bool
+    ):
+        """Per-sample gradients of ``module`` from its stored input and its output gradient.
+
+        Results of one backward pass accumulate in ``p._current_grad_sample``; when the
+        parameter's forward counter is back at zero the pass is over for it and the tensor
+        moves to ``p.grad_sample`` (grad_sample_module.py:291-365).
+        """
+        if not self.hooks_enabled:
+            return
+        backprops = forward_output[0].detach()
+        activations, backprops, scale = self._take_activations(
+            module=module, backprops=backprops, loss_reduction=loss_reduction, batch_first=batch_first
+        )
+        sampler = self._sampler_for(module)
+        grad_samples = call_sampler(sampler, module, activations, backprops, scale)
+        adopt = getattr(sampler, "owns_output", False)
+        for param, gs in grad_samples.items():
+            create_or_accumulate_grad_sample(
+                param=param, grad_sample=gs, max_batch_len=module.max_batch_len, adopt=adopt
+            )
+        for _, p in trainable_parameters(module):
+            p._forward_counter -= 1
+            if p._forward_counter == 0:
+                promote_current_grad_sample(p)
+            if not self.grad_accumulation_allowed:
+                if isinstance(p.grad_sample, list) and len(p.grad_sample) > 1:
+                    raise ValueError(
+                        "Poisson sampling is not compatible with grad accumulation. "
+                        "You need to call optimizer.step() after every forward/backward pass "
+                        "or consider using BatchMemoryManager"
+                    )
+        if len(module.activations) == 0 and hasattr(module, "max_batch_len"):
+            del module.max_batch_len
+
+    def _take_activations(
+        self, *, module: nn.Module, backprops: torch.Tensor, loss_reduction: str, batch_first: bool
+    ) -> Tuple[List[torch.Tensor], torch.Tensor, float]:
+        """Pops the matching activations and returns them batch-first with the backprops
+        (not yet scaled) and the factor that turns them into sum-loss backprops."""
+        if not hasattr(module, "activations"):
+            raise ValueError(f"No activations detected for {type(module)}, run forward after add_hooks(model)")
+        batch_dim = 0 if batch_first else 1
+        if not hasattr(module, "max_batch_len"):
+            module.max_batch_len = _get_batch_size(module=module, batch_dim=batch_dim)
+        activations = module.activations.pop()
+        if loss_reduction == "mean":
+            scale = float(module.max_batch_len)
+        elif loss_reduction == "sum":
+            scale = 1.0
+        else:
+            raise ValueError(f"loss_reduction = {loss_reduction}. Only 'sum' and 'mean' losses are supported")
+        if batch_dim != 0:
+            activations = [_batch_first_view(t, batch_dim) for t in activations]
+            backprops = _batch_first_view(backprops, batch_dim)
+        return activations, backprops, scale
+
+    def rearrange_grad_samples(
+        self, *, module: nn.Module, backprops: torch.Tensor, loss_reduction: str, batch_first: bool
+    ) -> Tuple[List[torch.Tensor], torch.Tensor]:
+        """Activations and backprops as a plain sampler expects them: batch first, backprops
+        multiplied by the batch size for a mean loss (grad_sample_module.py:367-422)."""
+        activations, backprops, scale = self._take_activations(
+            module=module, backprops=backprops, loss_reduction=loss_reduction, batch_first=batch_first
+        )
+        if scale != 1.0:
+            backprops = backprops * scale
+        return activations, backprops
+
+    # ---- validation ----------------------------------------------------------------------
+    @classmethod
+    def is_supported(cls, module: nn.Module) -> bool:
+        warnings.warn(
+            "GradSampleModule.is_supported is deprecated, as all layers can now be used with functorch.",
+            DeprecationWarning,
+        )
+        return True
+
+    @classmethod
+    def validate(cls, module: nn.Module, *, strict: bool = False) -> List[NotImplementedError]:
+        """Trainable modules that own buffers (BatchNorm and the like) cannot have per-sample
+        gradients: the buffers mix samples (grad_sample_module.py:446-485)."""
+        errors = [
+            NotImplementedError(
+                f"Model contains a trainable layer with buffers that Opacus doesn't currently support({name}:{m}). "
+            )
+            for name, m in trainable_modules(module)
+            if len(list(m.buffers())) > 0
+        ]
+        if strict and errors:
+            raise NotImplementedError(errors)
+        return errors
+
+    def forbid_grad_accumulation(self):
+        self.grad_accumulation_allowed = False
+
+    def allow_grad_accumulation(self):
+        self.grad_accumulation_allowed = True
+
+
+class GradSampleModule(GradSampleHooks, AbstractGradSampleModule):
+    """``nn.Module`` wrapper whose parameters carry ``.grad_sample`` after ``backward``."""
+
+    def __init__(self, m: nn.Module, *, batch_first=True, loss_reduction="mean", strict: bool = True, force_functorch=False):
+        nn.Module.__init__(self)
+        GradSampleHooks.__init__(
+            self, m, batch_first=batch_first, loss_reduction=loss_reduction, strict=strict, force_functorch=force_functorch
+        )
+        self.grad_accumulation_hook = None
+
+    def forward(self, *args, **kwargs):
+        return self._module(*args, **kwargs)

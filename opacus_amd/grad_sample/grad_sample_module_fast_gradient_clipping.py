@@ -1,0 +1,209 @@
+"""Ghost clipping / fast gradient clipping hooks.
+
+Mirror of opacus/grad_sample/grad_sample_module_fast_gradient_clipping.py: on the first
+backward pass every parameter receives a per-sample gradient NORM (``p._norm_sample``)
+instead of a per-sample gradient. Layers with a registered norm sampler (Linear,
+Embedding) get it from the ghost-norm kernels without the gradient ever existing; other
+layers have their per-sample gradient formed by the grad sampler, reduced to a norm and
+dropped at once. ``get_clipping_coef`` then yields ``min(1, C / (norm + 1e-6))``.
+
+Norm samples are kept in float32 whatever the dtype of the backprops (the kernels
+accumulate in fp32; rounding a norm to bf16 before it meets the other parameters' norms
+would only lose bits).
+"""
+
+from __future__ import annotations
+
+import logging
+from typing import List
+
+import torch
+import torch.nn as nn
+
+from .. import kernels
+from ..utils.module_utils import requires_grad, trainable_modules, trainable_parameters
+from .grad_sample_module import (
+    GradSampleHooks,
+    call_sampler,
+    create_or_accumulate_grad_sample,
+    promote_current_grad_sample,
+)
+from .gsm_base import AbstractGradSampleModule
+
+logger = logging.getLogger(__name__)
+logger.disabled = True
+
+
+def _cached_sumsq(gs: torch.Tensor):
+    """The per-sample sum of squares a sampler's kernel left on ``gs``, if still valid."""
+    ss = getattr(gs, "_dpk_sumsq", None)
+    if ss is not None and getattr(gs, "_dpk_sumsq_version", None) == gs._version:
+        return ss
+    return None
+
+
+def create_norm_sample(*, param: torch.Tensor, grad_sample: torch.Tensor, max_batch_len: int) -> None:
+    """``param._norm_sample`` = per-sample 2-norm of ``grad_sample``; an empty tensor for an
+    empty batch (grad_sample_module_fast_gradient_clipping.py:42-70)."""
+    if not param.requires_grad:
+        return
+    if max_batch_len == 0:
+        param._norm_sample = torch.zeros((0,), device=grad_sample.device, dtype=torch.float32)
+        return
+    ss = _cached_sumsq(grad_sample)
+    if ss is None:
+        ss = kernels.sumsq_rows([grad_sample])[0]
+    param._norm_sample, _ = kernels.clip_factor(ss.reshape(1, -1), 1.0)
+
+
+class GradSampleHooksFastGradientClipping(GradSampleHooks):
+    """Hooks object computing per-sample gradient norms (ghost clipping where a norm
+    sampler exists, fast gradient clipping elsewhere)."""
+
+    NORM_SAMPLERS = {}
+
+    def __init__(
+        self,
+        m: nn.Module,
+        *,
+        batch_first=True,
+        loss_reduction="mean",
+        strict: bool = True,
+        force_functorch=False,
+        max_grad_norm=1,
+        use_ghost_clipping=True,
+    ):
+        super().__init__(
+            m, batch_first=batch_first, loss_reduction=loss_reduction, strict=strict, force_functorch=force_functorch
+        )
+        self.trainable_parameters = [p for _, p in trainable_parameters(self._module)]
+        self.max_grad_norm = max_grad_norm
+        self.use_ghost_clipping = use_ghost_clipping
+        self._per_sample_gradient_norms = None
+
+    # ---- clipping coefficient ----------------------------------------------------------
+    def get_norm_sample(self) -> torch.Tensor:
+        """Per-sample norm over all parameters: 2-norm of the stacked per-parameter norms
+        (grad_sample_module_fast_gradient_clipping.py:142-150)."""
+        norm, _ = self._norm_and_coef()
+        return norm
+
+    def get_clipping_coef(self) -> torch.Tensor:
+        """``min(1, C / (norm + 1e-6))`` per sample (:137-140)."""
+        _, coef = self._norm_and_coef()
+        return coef
+
+    def _norm_and_coef(self):
+        norm_samples = [p._norm_sample for p in self.trainable_parameters]
+        if not norm_samples:
+            raise ValueError("no trainable parameter carries a norm sample")
+        dev = norm_samples[0].device
+        stacked = torch.stack([ns.to(device=dev, dtype=torch.float32).reshape(-1) for ns in norm_samples], dim=0)
+        norm, coef = kernels.clip_factor(stacked, float(self.max_grad_norm), is_norm=True)
+        self.per_sample_gradient_norms = norm
+        return norm, coef
+
+    # ---- hooks ------------------------------------------------------------------------------
+    def capture_activations_hook(self, module: nn.Module, forward_input: List[torch.Tensor], _forward_output):
+        if (
+            not requires_grad(module)
+            or not module.training
+            or not torch.is_grad_enabled()
+            or not self.hooks_enabled
+        ):
+            return
+        if not hasattr(module, "activations"):
+            module.activations = []
+        module.activations.append([t.detach() for t in forward_input])
+        for _, p in trainable_parameters(module):
+            p._forward_counter += 1
+            if self.use_ghost_clipping and p._forward_counter > 1 and type(module) in self.NORM_SAMPLERS:
+                # the norm of a sum of two layers' gradients is not a function of their norms
+                raise NotImplementedError("Parameter tying is not supported with Ghost Clipping")
+
+    def capture_backprops_hook(
+        self, module: nn.Module, _forward_input, forward_output, loss_reduction: str, batch_first: bool
+    ):
+        """Fills ``p._norm_sample`` for the parameters of ``module`` (:181-253)."""
+        if not self.hooks_enabled:
+            return
+        backprops = forward_output[0].detach()
+        activations, backprops, scale = self._take_activations(
+            module=module, backprops=backprops, loss_reduction=loss_reduction, batch_first=batch_first
+        )
+        if self.use_ghost_clipping and type(module) in self.NORM_SAMPLERS:
+            norm_samples = call_sampler(self.NORM_SAMPLERS[type(module)], module, activations, backprops, scale)
+            for param, ns in norm_samples.items():
+                if param.requires_grad:
+                    param._norm_sample = ns
+                    param._forward_counter -= 1
+        else:
+            sampler = self._sampler_for(module)
+            grad_samples = call_sampler(sampler, module, activations, backprops, scale)
+            adopt = getattr(sampler, "owns_output", False)
+            for param, gs in grad_samples.items():
+                create_or_accumulate_grad_sample(
+                    param=param, grad_sample=gs, max_batch_len=module.max_batch_len, adopt=adopt
+                )
+            del grad_samples
+            for _, p in trainable_parameters(module):
+                p._forward_counter -= 1
+                if p._forward_counter == 0:
+                    promote_current_grad_sample(p)
+                    create_norm_sample(param=p, grad_sample=p.grad_sample, max_batch_len=module.max_batch_len)
+                    p.grad_sample = None
+        if len(module.activations) == 0 and hasattr(module, "max_batch_len"):
+            del module.max_batch_len
+
+    def log_module_gradient_sample_mode(self, module: nn.Module, *, force_functorch=False, use_ghost_clipping=True):
+        """Logs, per trainable module, which of the three paths it takes (:255-290)."""
+        for name, m in trainable_modules(module):
+            if use_ghost_clipping and type(m) in self.NORM_SAMPLERS:
+                how = "under Ghost Clipping."
+            elif not force_functorch and type(m) in self.GRAD_SAMPLERS:
+                how = "under Fast Gradient Clipping (hook mode)."
+            else:
+                how = "under Fast Gradient Clipping (functorch mode)."
+            logger.info(f"Module name: {name}, module type: {type(m)}, {how}")
+
+    @property
+    def per_sample_gradient_norms(self) -> torch.Tensor:
+        """Per-sample gradient norms of the last ``get_norm_sample``/``get_clipping_coef`` call."""
+        if self._per_sample_gradient_norms is None:
+            raise AttributeError("per_sample_gradient_norms is not set. Please call forward and backward on the model before accessing this property.")
+        return self._per_sample_gradient_norms
+
+    @per_sample_gradient_norms.setter
+    def per_sample_gradient_norms(self, value):
+        self._per_sample_gradient_norms = value
+
+
+class GradSampleModuleFastGradientClipping(GradSampleHooksFastGradientClipping, AbstractGradSampleModule):
+    """``nn.Module`` wrapper flavour of :class:`GradSampleHooksFastGradientClipping`."""
+
+    def __init__(
+        self,
+        m: nn.Module,
+        *,
+        batch_first=True,
+        loss_reduction="mean",
+        strict: bool = True,
+        force_functorch=False,
+        max_grad_norm=1,
+        use_ghost_clipping=True,
+    ):
+        nn.Module.__init__(self)
+        GradSampleHooksFastGradientClipping.__init__(
+            self,
+            m,
+            batch_first=batch_first,
+            loss_reduction=loss_reduction,
+            strict=strict,
+            force_functorch=force_functorch,
+            max_grad_norm=max_grad_norm,
+            use_ghost_clipping=use_ghost_clipping,
+        )
+        self.grad_accumulation_hook = None
+
+    def forward(self, *args, **kwargs):
+        return self._module(*args, **kwargs)

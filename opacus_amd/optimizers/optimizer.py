@@ -1,0 +1,358 @@
+"""``DPOptimizer`` on the HIP kernels (mirror of opacus/optimizers/optimizer.py).
+
+Same life cycle as the reference: ``step()`` -> ``pre_step()`` -> ``clip_and_accumulate()``
+-> ``add_noise()`` -> ``scale_grad()`` -> step hook -> the wrapped optimizer's ``step()``.
+What changes is how many times the per-sample gradients cross HBM:
+
+  * per-sample squared norms come for free from the sampler kernels that wrote the
+    per-sample gradients (they ride on the tensor); only tensors without a valid one are
+    read, all of them in one multi-tensor launch;
+  * the clip factor is one tiny kernel;
+  * ``sum_n clip[n] * gs[n]`` reads every per-sample gradient exactly once, all parameters
+    of a dtype in one launch;
+  * noise, the add and the division by the batch size are one kernel per parameter that
+    draws Philox normals in registers, instead of zeros + normal + add + div.
+"""
+
+from __future__ import annotations
+
+import logging
+from collections import defaultdict
+from typing import Callable, Dict, List, Optional, Tuple, Union
+
+import torch
+from torch import nn
+from torch.optim import Optimizer
+
+from .. import kernels
+from ..grad_sample._common import cached_sumsq
+from .utils import params
+
+logger = logging.getLogger(__name__)
+logger.disabled = True
+
+# Units of generator offset one noise call consumes (torch wants multiples of 4).
+_OFFSET_PER_CALL = 4
+
+
+def _mark_as_processed(obj: Union[torch.Tensor, List[torch.Tensor]]):
+    """Flags gradients as consumed by a step so that using them twice is caught (optimizer.py:32-58)."""
+    if isinstance(obj, torch.Tensor):
+        obj._processed = True
+    elif isinstance(obj, list):
+        for x in obj:
+            x._processed = True
+
+
+def _check_processed_flag_tensor(x: torch.Tensor):
+    if hasattr(x, "_processed"):
+        raise ValueError(
+            "Gradients haven't been cleared since the last optimizer step. "
+            "In order to obtain privacy guarantees you must call optimizer.zero_grad()"
+            "on each step"
+        )
+
+
+def _check_processed_flag(obj: Union[torch.Tensor, List[torch.Tensor]]):
+    if isinstance(obj, torch.Tensor):
+        _check_processed_flag_tensor(obj)
+    elif isinstance(obj, list):
+        for x in obj:
+            _check_processed_flag_tensor(x)
+
+
+def philox_stream(generator: Optional[torch.Generator], device: torch.device) -> Tuple[int, int]:
+    """``(seed, offset)`` for one noise kernel call, advancing the generator.
+
+    A generator on the GPU (the default one when ``generator`` is None) is used the way
+    torch's own Philox kernels use it: its seed is the key and its offset moves on, so
+    ``torch.manual_seed`` / ``generator.manual_seed`` make runs repeat. A CPU generator
+    cannot share an offset with the device; two 63-bit draws from it become the key and
+    the offset, which keeps the same determinism.
+    """
+    if generator is None:
+        generator = torch.cuda.default_generators[device.index if device.index is not None else torch.cuda.current_device()]
+    if generator.device.type == "cuda":
+        seed = generator.initial_seed()
+        offset = generator.get_offset()
+        generator.set_offset(offset + _OFFSET_PER_CALL)
+        return seed, offset
+    draws = torch.randint(0, 2**62, (2,), generator=generator, dtype=torch.int64)
+    return int(draws[0]), int(draws[1]) * _OFFSET_PER_CALL
+
+
+def _generate_noise(std: float, reference: torch.Tensor, generator=None, secure_mode: bool = False) -> torch.Tensor:
+    """Gaussian noise of ``reference``'s shape and dtype (optimizer.py:104-169).
+
+    ``std == 0`` gives exact zeros without touching the generator. ``secure_mode`` sums
+    four draws and halves, as the reference does against floating-point attacks.
+    """
+    out = torch.zeros(reference.shape, device=reference.device, dtype=reference.dtype)
+    if std == 0:
+        return out
+    seed, offset = philox_stream(generator, reference.device)
+    kernels.add_noise(out, out, std, 1.0, seed, offset, draws=4 if secure_mode else 1)
+    return out
+
+
+class DPOptimizer(Optimizer):
+    """Wraps a ``torch.optim.Optimizer``: clips per-sample gradients to ``max_grad_norm``,
+    sums them, adds ``N(0, (noise_multiplier * max_grad_norm)^2)`` and rescales
+    (optimizer.py:172-581). Per-sample gradients are read from ``p.grad_sample``."""
+
+    def __init__(
+        self,
+        optimizer: Optimizer,
+        *,
+        noise_multiplier: float,
+        max_grad_norm: float,
+        expected_batch_size: Optional[int],
+        loss_reduction: str = "mean",
+        generator=None,
+        secure_mode: bool = False,
+        **kwargs,
+    ):
+        if loss_reduction not in ("mean", "sum"):
+            raise ValueError(f"Unexpected value for loss_reduction: {loss_reduction}")
+        if loss_reduction == "mean" and expected_batch_size is None:
+            raise ValueError("You must provide expected batch size of the loss reduction is mean")
+        self.original_optimizer = optimizer
+        self.noise_multiplier = noise_multiplier
+        self.max_grad_norm = max_grad_norm
+        self.loss_reduction = loss_reduction
+        self.expected_batch_size = expected_batch_size
+        self.step_hook = None
+        self.generator = generator
+        self.secure_mode = secure_mode
+        self._step_skip_queue = []
+        self._is_last_step_skipped = False
+        for p in self.params:
+            p.summed_grad = None
+
+    # ---- per-sample gradient access -----------------------------------------------------
+    def _get_flat_grad_sample(self, p: torch.Tensor):
+        """``p.grad_sample`` as one tensor; a list from several backward passes is
+        concatenated along the batch (optimizer.py:252-292)."""
+        if not hasattr(p, "grad_sample"):
+            raise ValueError("Per sample gradient not found. Are you using GradSampleModule?")
+        if p.grad_sample is None:
+            raise ValueError("Per sample gradient is not initialized. Not updated in backward pass?")
+        if isinstance(p.grad_sample, torch.Tensor):
+            return p.grad_sample
+        if isinstance(p.grad_sample, list):
+            return torch.cat(p.grad_sample, dim=0)
+        raise ValueError(f"Unexpected grad_sample type: {type(p.grad_sample)}")
+
+    def signal_skip_step(self, do_skip=True):
+        """Queues whether the next ``step`` only clips and accumulates (virtual batches,
+        optimizer.py:294-329)."""
+        self._step_skip_queue.append(do_skip)
+
+    def _check_skip_next_step(self, pop_next=True):
+        if self._step_skip_queue:
+            return self._step_skip_queue.pop(0) if pop_next else self._step_skip_queue[0]
+        return False
+
+    @property
+    def params(self) -> List[nn.Parameter]:
+        return params(self)
+
+    @property
+    def grad_samples(self) -> List[torch.Tensor]:
+        return [self._get_flat_grad_sample(p) for p in self.params]
+
+    @property
+    def accumulated_iterations(self) -> int:
+        """Backward passes accumulated in ``grad_sample`` (1 for a tensor, the length of a
+        list); must agree across parameters (optimizer.py:348-376)."""
+        vals = set()
+        for p in self.params:
+            if not hasattr(p, "grad_sample"):
+                raise ValueError("Per sample gradient not found. Are you using GradSampleModule?")
+            if isinstance(p.grad_sample, torch.Tensor):
+                vals.add(1)
+            elif isinstance(p.grad_sample, list):
+                vals.add(len(p.grad_sample))
+            else:
+                raise ValueError(f"Unexpected grad_sample type: {type(p.grad_sample)}")
+        if len(vals) > 1:
+            raise ValueError("Number of accumulated steps is inconsistent across parameters")
+        return vals.pop()
+
+    # ---- delegation to the wrapped optimizer ------------------------------------------------
+    @property
+    def param_groups(self) -> List[dict]:
+        return self.original_optimizer.param_groups
+
+    @param_groups.setter
+    def param_groups(self, param_groups: List[dict]):
+        self.original_optimizer.param_groups = param_groups
+
+    @property
+    def state(self) -> defaultdict:
+        return self.original_optimizer.state
+
+    @state.setter
+    def state(self, state: defaultdict):
+        self.original_optimizer.state = state
+
+    @property
+    def defaults(self) -> dict:
+        return self.original_optimizer.defaults
+
+    @defaults.setter
+    def defaults(self, defaults: dict):
+        self.original_optimizer.defaults = defaults
+
+    def attach_step_hook(self, fn: Callable[["DPOptimizer"], None]):
+        """``fn(optimizer)`` runs after noise and scaling, before the wrapped step (privacy accounting)."""
+        self.step_hook = fn
+
+    # ---- the hot path ---------------------------------------------------------------------
+    def _per_param_sumsq(self, plist: List[nn.Parameter], flats: List[torch.Tensor]) -> torch.Tensor:
+        """``[K, n]`` squared norms: cached ones from the sampler kernels where they are still
+        valid, one multi-tensor pass over the rest."""
+        n = flats[0].shape[0]
+        dev = flats[0].device
+        rows: List[Optional[torch.Tensor]] = []
+        missing: Dict[Tuple[torch.dtype, torch.device], List[int]] = {}
+        for k, (p, g) in enumerate(zip(plist, flats)):
+            ss = cached_sumsq(p.grad_sample) if isinstance(p.grad_sample, torch.Tensor) else None
+            rows.append(ss)
+            if ss is None:
+                missing.setdefault((g.dtype, g.device), []).append(k)
+        for (_, _), idxs in missing.items():
+            got = kernels.sumsq_rows([flats[k] for k in idxs])
+            for j, k in enumerate(idxs):
+                rows[k] = got[j]
+        return torch.stack([r.to(dev) for r in rows], dim=0) if len(rows) > 1 else rows[0].to(dev).reshape(1, n)
+
+    def clip_and_accumulate(self):
+        """Clips every sample's gradient to ``max_grad_norm`` and adds the clipped gradients
+        into ``p.summed_grad`` (optimizer.py:432-475)."""
+        plist = self.params
+        flats = []
+        for p in plist:
+            _check_processed_flag(p.grad_sample)
+            g = self._get_flat_grad_sample(p)
+            if not kernels.supported_dtype(g.dtype):
+                raise TypeError(f"per-sample gradients must be float32 or bfloat16 on this path, got {g.dtype}")
+            flats.append(g)
+        n = len(flats[0])
+        if n == 0:
+            clip = torch.zeros((0,), device=flats[0].device, dtype=torch.float32)
+        else:
+            sumsq = self._per_param_sumsq(plist, flats)
+            _, clip = kernels.clip_factor(sumsq, float(self.max_grad_norm))
+        # one launch per (device, per-sample dtype, parameter dtype, fresh/accumulate) group
+        groups: Dict[tuple, List[int]] = {}
+        for k, (p, g) in enumerate(zip(plist, flats)):
+            out_dtype = p.dtype if kernels.supported_dtype(p.dtype) else torch.float32
+            if p.summed_grad is None:
+                p.summed_grad = torch.empty(g.shape[1:], device=g.device, dtype=out_dtype)
+                fresh = True
+            else:
+                fresh = False
+                if not p.summed_grad.is_contiguous() or p.summed_grad.dtype != out_dtype:
+                    raise ValueError("summed_grad must be a dense tensor of the parameter's dtype")
+            groups.setdefault((g.device, g.dtype, out_dtype, fresh), []).append(k)
+        for (dev, _, _, fresh), idxs in groups.items():
+            kernels.clip_accumulate(
+                [flats[k] for k in idxs], clip.to(dev), [plist[k].summed_grad for k in idxs], accumulate=not fresh
+            )
+        for p in plist:
+            if p.summed_grad.dtype != p.dtype:
+                p.summed_grad = p.summed_grad.to(p.dtype)
+            _mark_as_processed(p.grad_sample)
+
+    def _noise_std(self) -> float:
+        return self.noise_multiplier * self.max_grad_norm
+
+    def _add_noise_scaled(self, denom: float):
+        std = self._noise_std()
+        for p in self.params:
+            _check_processed_flag(p.summed_grad)
+            summed = p.summed_grad
+            if not kernels.supported_dtype(summed.dtype):
+                raise TypeError(f"summed_grad must be float32 or bfloat16 on this path, got {summed.dtype}")
+            if not summed.is_contiguous():
+                summed = summed.contiguous()
+            grad = torch.empty(p.shape, device=summed.device, dtype=summed.dtype)
+            if std == 0:
+                seed = offset = 0  # nothing is drawn and the generator stays where it is
+            else:
+                seed, offset = philox_stream(self.generator, summed.device)
+            kernels.add_noise(summed, grad, std, denom, seed, offset, draws=4 if self.secure_mode else 1)
+            p.grad = grad
+            _mark_as_processed(p.summed_grad)
+
+    def add_noise(self):
+        """``p.grad = (p.summed_grad + N(0, std^2)).view_as(p)`` (optimizer.py:477-493)."""
+        self._add_noise_scaled(1.0)
+
+    def scale_grad(self):
+        """Divides ``p.grad`` by ``expected_batch_size * accumulated_iterations`` for a
+        mean-reduced loss; nothing for a sum (optimizer.py:495-504)."""
+        if self.loss_reduction == "mean":
+            denom = float(self.expected_batch_size * self.accumulated_iterations)
+            for p in self.params:
+                g = p.grad
+                if g.is_cuda and g.is_contiguous() and kernels.supported_dtype(g.dtype):
+                    kernels.add_noise(g, g, 0.0, denom, 0, 0)
+                else:
+                    p.grad /= denom
+
+    def _noise_and_scale(self):
+        """``add_noise`` then ``scale_grad``; one kernel per parameter when neither method
+        has been overridden by a subclass."""
+        cls = type(self)
+        fused = cls.add_noise is DPOptimizer.add_noise and cls.scale_grad is DPOptimizer.scale_grad
+        if fused:
+            denom = 1.0
+            if self.loss_reduction == "mean":
+                denom = float(self.expected_batch_size * self.accumulated_iterations)
+            self._add_noise_scaled(denom)
+        else:
+            self.add_noise()
+            self.scale_grad()
+
+    def zero_grad(self, set_to_none: bool = False):
+        """Clears ``p.grad``, ``p.grad_sample`` and, unless the last step was a skipped
+        (virtual) one, ``p.summed_grad`` (optimizer.py:506-537)."""
+        for p in self.params:
+            p.grad_sample = None
+            if not self._is_last_step_skipped:
+                p.summed_grad = None
+        self.original_optimizer.zero_grad(set_to_none)
+
+    def pre_step(self, closure: Optional[Callable[[], float]] = None) -> Optional[float]:
+        """Everything before the wrapped optimizer's step; returns False when this step is
+        a skipped one that only accumulated (optimizer.py:539-563)."""
+        if len(self.params) == 0:
+            return True
+        self.clip_and_accumulate()
+        if self._check_skip_next_step():
+            self._is_last_step_skipped = True
+            return False
+        self._noise_and_scale()
+        if self.step_hook:
+            self.step_hook(self)
+        self._is_last_step_skipped = False
+        return True
+
+    def step(self, closure: Optional[Callable[[], float]] = None) -> Optional[float]:
+        if closure is not None:
+            with torch.enable_grad():
+                closure()
+        if self.pre_step():
+            return self.original_optimizer.step()
+        return None
+
+    def __repr__(self):
+        return self.original_optimizer.__repr__()
+
+    def state_dict(self):
+        return self.original_optimizer.state_dict()
+
+    def load_state_dict(self, state_dict) -> None:
+        self.original_optimizer.load_state_dict(state_dict)
