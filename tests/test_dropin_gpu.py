@@ -1,0 +1,554 @@
+"""GPU integration: the drop-in API (GradSampleModule, ghost clipping, DPOptimizer,
+PrivacyEngine.make_private) against the CPU oracle and plain autograd, on down-scaled
+versions of the five benchmark configurations. Modelled on the reference's own tests
+(opacus/tests/grad_samples/common.py, privacy_engine_test.py,
+grad_sample_module_fast_gradient_clipping_test.py, randomness_test.py)."""
+
+import copy
+import math
+
+import pytest
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+from torch.utils.data import DataLoader, TensorDataset
+
+from oracle import dp_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+
+
+@pytest.fixture(scope="module")
+def A():
+    import opacus_amd
+
+    return opacus_amd
+
+
+def per_sample_grads_cpu(model, x, y, loss_fn, batch_dim=0):
+    """Batch-of-one autograd on the CPU: the reference's microbatch oracle."""
+    names = [k for k, p in model.named_parameters() if p.requires_grad]
+    out = {k: [] for k in names}
+    for i in range(x.shape[batch_dim]):
+        model.zero_grad()
+        xi = x.narrow(batch_dim, i, 1)
+        loss_fn(model(xi), y[i : i + 1]).backward()
+        for k, p in model.named_parameters():
+            if p.requires_grad:
+                out[k].append(p.grad.clone())
+    model.zero_grad()
+    return {k: torch.stack(v) for k, v in out.items()}
+
+
+def close(got, want, rtol, atol, msg=""):
+    torch.testing.assert_close(got.detach().float().cpu(), want.detach().float().cpu(), rtol=rtol, atol=atol, msg=lambda m: f"{msg}: {m}")
+
+
+# ---- models (down-scaled versions of the benchmark configurations) -----------------------------
+class SmallCNN(nn.Module):
+    """Config 1: Conv(1,16,8,2,3) ReLU MaxPool Conv(16,32,4,2) ReLU MaxPool Linear(512,32) ReLU Linear(32,10)."""
+
+    def __init__(self):
+        super().__init__()
+        self.conv1 = nn.Conv2d(1, 16, 8, 2, padding=3)
+        self.conv2 = nn.Conv2d(16, 32, 4, 2)
+        self.fc1 = nn.Linear(32 * 4 * 4, 32)
+        self.fc2 = nn.Linear(32, 10)
+
+    def forward(self, x):
+        x = F.max_pool2d(F.relu(self.conv1(x)), 2, 1)
+        x = F.max_pool2d(F.relu(self.conv2(x)), 2, 1)
+        return self.fc2(F.relu(self.fc1(x.flatten(1))))
+
+
+class ResBlock(nn.Module):
+    """Config 4: two 3x3 convolutions with GroupNorm and a skip, then a small head."""
+
+    def __init__(self, ch=16, groups=8):
+        super().__init__()
+        self.c1, self.g1 = nn.Conv2d(ch, ch, 3, padding=1), nn.GroupNorm(groups, ch)
+        self.c2, self.g2 = nn.Conv2d(ch, ch, 3, padding=1), nn.GroupNorm(groups, ch)
+        self.head = nn.Linear(ch, 10)
+
+    def forward(self, x):
+        h = F.relu(self.g1(self.c1(x)))
+        h = F.relu(self.g2(self.c2(h)) + x)
+        return self.head(h.mean(dim=(2, 3)))
+
+
+class TinyLlama(nn.Module):
+    """Config 5, down-scaled: embedding, RMSNorm, grouped-query attention with rotary
+    embedding (no parameters), SwiGLU, untied LM head; all bias-free."""
+
+    def __init__(self, vocab=50, d=32, heads=4, kv=2, ffn=48, layers=2):
+        super().__init__()
+        self.emb = nn.Embedding(vocab, d)
+        self.heads, self.kv, self.hd = heads, kv, d // heads
+        self.blocks = nn.ModuleList()
+        for _ in range(layers):
+            self.blocks.append(
+                nn.ModuleDict(
+                    dict(
+                        n1=nn.RMSNorm(d, eps=1e-5),
+                        q=nn.Linear(d, d, bias=False),
+                        k=nn.Linear(d, kv * self.hd, bias=False),
+                        v=nn.Linear(d, kv * self.hd, bias=False),
+                        o=nn.Linear(d, d, bias=False),
+                        n2=nn.RMSNorm(d, eps=1e-5),
+                        gate=nn.Linear(d, ffn, bias=False),
+                        up=nn.Linear(d, ffn, bias=False),
+                        down=nn.Linear(ffn, d, bias=False),
+                    )
+                )
+            )
+        self.norm = nn.RMSNorm(d, eps=1e-5)
+        self.lm_head = nn.Linear(d, vocab, bias=False)
+
+    @staticmethod
+    def rope(x):
+        B, H, T, D = x.shape
+        pos = torch.arange(T, device=x.device, dtype=torch.float32)
+        inv = 1.0 / (10000 ** (torch.arange(0, D, 2, device=x.device, dtype=torch.float32) / D))
+        ang = pos[:, None] * inv[None, :]
+        cos, sin = ang.cos().to(x.dtype), ang.sin().to(x.dtype)
+        x1, x2 = x[..., 0::2], x[..., 1::2]
+        return torch.stack([x1 * cos - x2 * sin, x1 * sin + x2 * cos], dim=-1).flatten(-2)
+
+    def forward(self, ids):
+        h = self.emb(ids)
+        B, T, _ = h.shape
+        for blk in self.blocks:
+            a = blk["n1"](h)
+            q = blk["q"](a).view(B, T, self.heads, self.hd).transpose(1, 2)
+            k = blk["k"](a).view(B, T, self.kv, self.hd).transpose(1, 2)
+            v = blk["v"](a).view(B, T, self.kv, self.hd).transpose(1, 2)
+            q, k = self.rope(q), self.rope(k)
+            rep = self.heads // self.kv
+            k, v = k.repeat_interleave(rep, dim=1), v.repeat_interleave(rep, dim=1)
+            att = F.scaled_dot_product_attention(q, k, v, is_causal=True)
+            h = h + blk["o"](att.transpose(1, 2).reshape(B, T, -1))
+            m = blk["n2"](h)
+            h = h + blk["down"](F.silu(blk["gate"](m)) * blk["up"](m))
+        return self.lm_head(self.norm(h))
+
+
+def ce_sum(out, y):
+    return F.cross_entropy(out, y, reduction="sum")
+
+
+# ---- per-sample gradients through the hooks --------------------------------------------------
+@pytest.mark.parametrize("loss_reduction", ["mean", "sum"])
+def test_small_cnn_grad_samples(A, loss_reduction):
+    torch.manual_seed(0)
+    net = SmallCNN()
+    n = 8
+    x, y = torch.randn(n, 1, 28, 28), torch.randint(0, 10, (n,))
+    want = per_sample_grads_cpu(net, x, y, ce_sum)
+    gsm = A.GradSampleModule(copy.deepcopy(net).to(DEV), loss_reduction=loss_reduction)
+    F.cross_entropy(gsm(x.to(DEV)), y.to(DEV), reduction=loss_reduction).backward()
+    for k, p in gsm._module.named_parameters():
+        assert p.grad_sample.shape == (n, *p.shape)
+        close(p.grad_sample, want[k], 1e-4, 1e-5, k)  # the reference's own tolerance (common.py:50-51)
+        # and the stricter bar of this build: relative to the tensor's scale
+        assert (p.grad_sample.cpu() - want[k]).abs().max() <= 2e-5 * want[k].abs().max()
+
+
+def test_res_block_grad_samples(A):
+    torch.manual_seed(1)
+    net = ResBlock()
+    n = 5
+    x, y = torch.randn(n, 16, 8, 8), torch.randint(0, 10, (n,))
+    want = per_sample_grads_cpu(net, x, y, ce_sum)
+    gsm = A.GradSampleModule(copy.deepcopy(net).to(DEV), loss_reduction="mean")
+    F.cross_entropy(gsm(x.to(DEV)), y.to(DEV)).backward()
+    for k, p in gsm._module.named_parameters():
+        close(p.grad_sample, want[k], 1e-3, 1e-4, k)  # conv tolerance of the reference (conv2d_test.py:84-85)
+        assert (p.grad_sample.cpu() - want[k]).abs().max() <= 5e-5 * want[k].abs().max(), k
+
+
+@pytest.mark.parametrize("batch_first", [True, False])
+def test_sequence_model_grad_samples(A, batch_first):
+    """Embedding -> Linear over [batch, seq]; also with the batch in dimension 1."""
+    torch.manual_seed(2)
+
+    class Seq(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.emb = nn.Embedding(20, 12)
+            self.fc = nn.Linear(12, 7)
+
+        def forward(self, ids):
+            return self.fc(torch.tanh(self.emb(ids)))
+
+    net = Seq()
+    n, T = 6, 9
+    ids = torch.randint(0, 20, (n, T) if batch_first else (T, n))
+    tgt = torch.randn(n, T, 7) if batch_first else torch.randn(T, n, 7)
+    bdim = 0 if batch_first else 1
+
+    def loss_i(out, t):
+        return (out - t).pow(2).sum()
+
+    names = [k for k, _ in net.named_parameters()]
+    want = {k: [] for k in names}
+    for i in range(n):
+        net.zero_grad()
+        loss_i(net(ids.narrow(bdim, i, 1)), tgt.narrow(bdim, i, 1)).backward()
+        for k, p in net.named_parameters():
+            want[k].append(p.grad.clone())
+    want = {k: torch.stack(v) for k, v in want.items()}
+    gsm = A.GradSampleModule(copy.deepcopy(net).to(DEV), loss_reduction="sum", batch_first=batch_first)
+    loss_i(gsm(ids.to(DEV)), tgt.to(DEV)).backward()
+    for k, p in gsm._module.named_parameters():
+        close(p.grad_sample, want[k], 1e-4, 1e-5, k)
+
+
+def test_accumulation_tied_parameters_and_functorch_fallback(A):
+    torch.manual_seed(3)
+
+    class Tied(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.fc = nn.Linear(6, 6)
+            self.ln = nn.LayerNorm(6)  # no kernel here: generic fallback
+
+        def forward(self, x):
+            return self.ln(self.fc(torch.relu(self.fc(x))))
+
+    net = Tied()
+    x, y = torch.randn(4, 6), torch.randn(4, 6)
+
+    def mse(out, t):
+        return (out - t).pow(2).sum()
+
+    want = per_sample_grads_cpu(net, x, y, mse)
+    gsm = A.GradSampleModule(copy.deepcopy(net).to(DEV), loss_reduction="sum")
+    mse(gsm(x.to(DEV)), y.to(DEV)).backward()
+    for k, p in gsm._module.named_parameters():
+        assert isinstance(p.grad_sample, torch.Tensor)
+        close(p.grad_sample, want[k], 1e-4, 1e-5, k)
+    # a second backward without zero_grad stacks a list; the optimizer concatenates it
+    mse(gsm(x.to(DEV)), y.to(DEV)).backward()
+    assert all(isinstance(p.grad_sample, list) and len(p.grad_sample) == 2 for p in gsm.parameters())
+    opt = A.DPOptimizer(torch.optim.SGD(gsm.parameters(), lr=0.0), noise_multiplier=0.0, max_grad_norm=1e20, expected_batch_size=4)
+    assert opt.accumulated_iterations == 2
+    opt.step()
+    for k, p in gsm._module.named_parameters():
+        close(p.grad, 2 * want[k].sum(0) / (4 * 2), 1e-4, 1e-5, k)
+
+
+# ---- DPOptimizer ------------------------------------------------------------------------------
+def _train(A, net, batches, *, private, sigma=0.0, C=1e20, lr=0.1, seed=None, generator=None, secure=False):
+    net = copy.deepcopy(net).to(DEV)
+    opt = torch.optim.SGD(net.parameters(), lr=lr)
+    model = net
+    if private:
+        model = A.GradSampleModule(net, loss_reduction="mean")
+        opt = A.DPOptimizer(opt, noise_multiplier=sigma, max_grad_norm=C, expected_batch_size=batches[0][0].shape[0], generator=generator, secure_mode=secure)
+    if seed is not None:
+        torch.manual_seed(seed)
+    for x, y in batches:
+        opt.zero_grad()
+        F.cross_entropy(model(x.to(DEV)), y.to(DEV)).backward()
+        opt.step()
+    return [p.detach().cpu() for p in net.parameters()]
+
+
+def test_private_equals_vanilla_when_nothing_clips(A):
+    """sigma = 0, C = 1e20 (privacy_engine_test.py:220-273: atol 1e-7 one step, 1e-4 three, rtol 1e-3)."""
+    torch.manual_seed(4)
+    net = SmallCNN()
+    batches = [(torch.randn(8, 1, 28, 28), torch.randint(0, 10, (8,))) for _ in range(3)]
+    for steps, atol in ((1, 1e-7), (3, 1e-4)):
+        van = _train(A, net, batches[:steps], private=False)
+        prv = _train(A, net, batches[:steps], private=True)
+        for v, p in zip(van, prv):
+            torch.testing.assert_close(p, v, atol=atol, rtol=1e-3)
+    clipped = _train(A, net, batches[:1], private=True, C=0.01)
+    noised = _train(A, net, batches[:1], private=True, sigma=1.0, C=1.0)
+    assert not torch.allclose(clipped[0], van[0]) and not torch.allclose(noised[0], van[0])
+
+
+def test_flat_clipping_batch_of_one_has_norm_C(A):
+    """privacy_engine_test.py:302-327."""
+    torch.manual_seed(5)
+    C = 0.5
+    gsm = A.GradSampleModule(SmallCNN().to(DEV), loss_reduction="mean")
+    opt = A.DPOptimizer(torch.optim.SGD(gsm.parameters(), lr=0.1), noise_multiplier=0.0, max_grad_norm=C, expected_batch_size=1)
+    F.cross_entropy(gsm(torch.randn(1, 1, 28, 28, device=DEV)), torch.tensor([3], device=DEV)).backward()
+    opt.clip_and_accumulate()
+    total = math.sqrt(sum(p.summed_grad.double().pow(2).sum().item() for p in gsm.parameters()))
+    assert round(total, 3) == C
+
+
+def test_clipped_sum_matches_oracle_and_sumsq_cache_is_guarded(A):
+    torch.manual_seed(6)
+    net = ResBlock()
+    n, C = 6, 0.3
+    x, y = torch.randn(n, 16, 8, 8), torch.randint(0, 10, (n,))
+    want_gs = per_sample_grads_cpu(net, x, y, ce_sum)
+    names = list(want_gs)
+    norms, clip, summed = O.clip_and_accumulate([want_gs[k] for k in names], C)
+    gsm = A.GradSampleModule(copy.deepcopy(net).to(DEV), loss_reduction="sum")
+    opt = A.DPOptimizer(torch.optim.SGD(gsm.parameters(), lr=0.1), noise_multiplier=0.0, max_grad_norm=C, expected_batch_size=n, loss_reduction="sum")
+    ce_sum(gsm(x.to(DEV)), y.to(DEV)).backward()
+    # tamper with one per-sample gradient in place: the squared norms its kernel left behind
+    # are stale now and must not be used
+    w = gsm._module.c1.weight
+    assert getattr(w.grad_sample, "_dpk_sumsq", None) is not None
+    w.grad_sample.mul_(3.0)
+    want_gs["c1.weight"] = want_gs["c1.weight"] * 3.0
+    norms, clip, summed = O.clip_and_accumulate([want_gs[k] for k in names], C)
+    opt.clip_and_accumulate()
+    for (k, p), s in zip(gsm._module.named_parameters(), summed):
+        assert (p.summed_grad.cpu() - s).abs().max() <= 5e-5 * s.abs().max(), k
+    with pytest.raises(ValueError, match="haven't been cleared"):
+        opt.clip_and_accumulate()  # same grad samples twice
+
+
+def test_virtual_steps_accumulate_summed_grad(A):
+    torch.manual_seed(7)
+    net = nn.Linear(10, 4)
+    xs = [torch.randn(5, 10) for _ in range(2)]
+    ys = [torch.randint(0, 4, (5,)) for _ in range(2)]
+    C = 0.2
+    gsm = A.GradSampleModule(copy.deepcopy(net).to(DEV), loss_reduction="mean")
+    opt = A.DPOptimizer(torch.optim.SGD(gsm.parameters(), lr=1.0), noise_multiplier=0.0, max_grad_norm=C, expected_batch_size=10)
+    opt.signal_skip_step(True)
+    opt.signal_skip_step(False)
+    results = []
+    for x, y in zip(xs, ys):
+        opt.zero_grad()
+        F.cross_entropy(gsm(x.to(DEV)), y.to(DEV)).backward()
+        results.append(opt.step())
+    assert results[0] is None
+    total = None
+    for x, y in zip(xs, ys):
+        gs = per_sample_grads_cpu(net, x, y, ce_sum)
+        _, _, summed = O.clip_and_accumulate([gs["weight"], gs["bias"]], C)
+        total = summed if total is None else [a + b for a, b in zip(total, summed)]
+    close(gsm._module.weight.grad, total[0] / 10, 1e-4, 1e-6)
+    close(gsm._module.bias.grad, total[1] / 10, 1e-4, 1e-6)
+
+
+def test_noise_level(A):
+    """privacy_engine_test.py:676-739: with zero gradients, after k steps sum p^2 ~ k P (sigma C lr / B)^2."""
+    torch.manual_seed(8)
+    net = nn.Linear(300, 200)
+    P = sum(p.numel() for p in net.parameters())
+    for p in net.parameters():
+        p.data.zero_()
+    sigma, C, lr, B, k = 1.5, 0.8, 0.5, 4, 3
+    gsm = A.GradSampleModule(net.to(DEV), loss_reduction="mean")
+    opt = A.DPOptimizer(torch.optim.SGD(gsm.parameters(), lr=lr), noise_multiplier=sigma, max_grad_norm=C, expected_batch_size=B)
+    for _ in range(k):
+        opt.zero_grad()
+        (gsm(torch.zeros(B, 300, device=DEV)).sum() * 0.0).backward()
+        opt.step()
+    energy = sum(p.double().pow(2).sum().item() for p in net.parameters())
+    expected = k * P * (sigma * C * lr / B) ** 2
+    assert abs(energy / expected - 1) < 0.05
+
+
+def test_noise_determinism_rules(A):
+    """randomness_test.py:199-255: same global seed or same generator seed => same weights; else different."""
+    torch.manual_seed(9)
+    net = nn.Linear(20, 5)
+    batches = [(torch.randn(4, 20), torch.randint(0, 5, (4,))) for _ in range(2)]
+    a = _train(A, net, batches, private=True, sigma=1.0, C=1.0, seed=123)
+    b = _train(A, net, batches, private=True, sigma=1.0, C=1.0, seed=123)
+    c = _train(A, net, batches, private=True, sigma=1.0, C=1.0, seed=124)
+    assert all(torch.equal(x, y) for x, y in zip(a, b))
+    assert not torch.equal(a[0], c[0])
+    for gdev in ("cuda", "cpu"):
+        g1 = torch.Generator(device=gdev).manual_seed(7)
+        g2 = torch.Generator(device=gdev).manual_seed(7)
+        g3 = torch.Generator(device=gdev).manual_seed(8)
+        d = _train(A, net, batches, private=True, sigma=1.0, C=1.0, generator=g1)
+        e = _train(A, net, batches, private=True, sigma=1.0, C=1.0, generator=g2)
+        f = _train(A, net, batches, private=True, sigma=1.0, C=1.0, generator=g3)
+        assert all(torch.equal(x, y) for x, y in zip(d, e)), gdev
+        assert not torch.equal(d[0], f[0]), gdev
+    s = _train(A, net, batches, private=True, sigma=1.0, C=1.0, seed=123, secure=True)
+    assert not torch.equal(a[0], s[0])
+    # noise per parameter is independent of the other parameters' noise
+    torch.manual_seed(1)
+    n1 = A.optimizers.optimizer._generate_noise(1.0, torch.zeros(100000, device=DEV))
+    n2 = A.optimizers.optimizer._generate_noise(1.0, torch.zeros(100000, device=DEV))
+    assert abs(torch.corrcoef(torch.stack([n1, n2]))[0, 1].item()) < 0.02
+    assert A.optimizers.optimizer._generate_noise(0.0, torch.ones(5, device=DEV)).abs().sum() == 0
+
+
+def test_zero_std_leaves_the_generator_alone(A):
+    net = nn.Linear(4, 2).to(DEV)
+    gsm = A.GradSampleModule(net, loss_reduction="mean")
+    gen = torch.Generator(device="cuda").manual_seed(11)
+    opt = A.DPOptimizer(torch.optim.SGD(gsm.parameters(), lr=0.1), noise_multiplier=0.0, max_grad_norm=1.0, expected_batch_size=2, generator=gen)
+    before = gen.get_offset()
+    gsm(torch.randn(2, 4, device=DEV)).sum().backward()
+    opt.step()
+    assert gen.get_offset() == before
+
+
+# ---- ghost clipping ----------------------------------------------------------------------------
+class PerSampleMSE(nn.Module):
+    def __init__(self, reduction="mean"):
+        super().__init__()
+        self.reduction = reduction
+
+    def forward(self, out, tgt):
+        l = (out - tgt).pow(2).flatten(1).mean(1)
+        if self.reduction == "none":
+            return l
+        return l.mean() if self.reduction == "mean" else l.sum()
+
+
+@pytest.mark.parametrize("loss_reduction", ["mean", "sum"])
+def test_ghost_norms_and_step_match_hooks_mode(A, loss_reduction):
+    """grad_sample_module_fast_gradient_clipping_test.py:129-280: per-parameter norms and the
+    weights after one step agree between ghost clipping and materialised clipping."""
+    torch.manual_seed(10)
+    mlp = nn.Sequential(nn.Linear(24, 40), nn.GELU(), nn.Linear(40, 12))  # config 3, down-scaled
+    n, T, C = 6, 33, 0.05
+    x, y = torch.randn(n, T, 24), torch.randn(n, T, 12)
+    crit = PerSampleMSE(loss_reduction)
+
+    hooks = A.GradSampleModule(copy.deepcopy(mlp).to(DEV), loss_reduction=loss_reduction)
+    hopt = A.DPOptimizer(torch.optim.SGD(hooks.parameters(), lr=0.5), noise_multiplier=0.0, max_grad_norm=C, expected_batch_size=n, loss_reduction=loss_reduction)
+    crit(hooks(x.to(DEV)), y.to(DEV)).backward()
+    want_norms = [p.grad_sample.double().flatten(1).norm(dim=1).cpu() for p in hooks.parameters()]
+    hopt.step()
+
+    ghost = A.GradSampleModuleFastGradientClipping(copy.deepcopy(mlp).to(DEV), loss_reduction=loss_reduction, max_grad_norm=C)
+    gopt = A.DPOptimizerFastGradientClipping(torch.optim.SGD(ghost.parameters(), lr=0.5), noise_multiplier=0.0, max_grad_norm=C, expected_batch_size=n, loss_reduction=loss_reduction)
+    dpl = A.DPLossFastGradientClipping(ghost, gopt, PerSampleMSE(loss_reduction), loss_reduction)
+    gopt.zero_grad()
+    dpl(ghost(x.to(DEV)), y.to(DEV)).backward()
+    for p, w in zip(ghost.parameters(), want_norms):
+        assert p.grad_sample is None
+        close(p._norm_sample, w, 1e-4, 1e-7)
+    total = torch.stack(want_norms).norm(dim=0)
+    close(ghost.per_sample_gradient_norms, total, 1e-4, 1e-7)
+    assert (total > C).all()  # the test clips every sample
+    gopt.step()
+    for pg, ph in zip(ghost.parameters(), hooks.parameters()):
+        close(pg, ph, 1e-4, 1e-6)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_ghost_tiny_llama_norms(A, dtype):
+    """Config 5, down-scaled: Embedding (ghost, id dedupe), RMSNorm (gradient formed and reduced
+    at once), Linear (Gram contraction), sequence-level loss via shape=."""
+    torch.manual_seed(11)
+    net = TinyLlama()
+    n, T, V = 4, 16, 50
+    ids = torch.randint(0, V, (n, T))
+    ids[0, :8] = 3  # repeated ids inside a sample
+    tgt = torch.randint(0, V, (n, T))
+
+    def seq_loss(logits, t):
+        return F.cross_entropy(logits.flatten(0, 1).float(), t.flatten(), reduction="none").view(1, -1).mean(1).sum()
+
+    want = per_sample_grads_cpu(net, ids, tgt, seq_loss)
+    want_norm = torch.sqrt(sum(v.double().flatten(1).pow(2).sum(1) for v in want.values()))
+
+    gnet = copy.deepcopy(net).to(DEV).to(dtype)
+    ghost = A.GradSampleModuleFastGradientClipping(gnet, loss_reduction="mean", max_grad_norm=1.0)
+    gopt = A.DPOptimizerFastGradientClipping(torch.optim.SGD(ghost.parameters(), lr=0.1), noise_multiplier=0.0, max_grad_norm=1.0, expected_batch_size=n)
+    dpl = A.DPLossFastGradientClipping(ghost, gopt, nn.CrossEntropyLoss(), "mean")
+    logits = ghost(ids.to(DEV))
+    loss = dpl(logits.flatten(0, 1).float(), tgt.flatten().to(DEV), shape=(n, T, V))
+    loss.backward()
+    rtol = 1e-3 if dtype == torch.float32 else 5e-2
+    close(ghost.per_sample_gradient_norms, want_norm, rtol, 1e-6)
+    if dtype == torch.float32:
+        coef = (1.0 / (want_norm + 1e-6)).clamp(max=1.0).float()
+        gopt.step()  # lr 0.1, mean over n
+        for (k, p0), p1 in zip(net.named_parameters(), gnet.parameters()):
+            g = (coef.view(-1, *[1] * (want[k].dim() - 1)) * want[k]).sum(0) / n
+            close(p1, p0 - 0.1 * g, 1e-3, 1e-5, k)
+
+
+def test_ghost_bf16_mlp(A):
+    """Config 3, down-scaled, bf16 parameters with fp32 accumulation inside the kernels."""
+    torch.manual_seed(12)
+    mlp = nn.Sequential(nn.Linear(64, 128), nn.GELU(), nn.Linear(128, 64))
+    n, T = 4, 70
+    x, y = torch.randn(n, T, 64), torch.randn(n, T, 64)
+    ghost = A.GradSampleModuleFastGradientClipping(copy.deepcopy(mlp).to(DEV).bfloat16(), loss_reduction="mean", max_grad_norm=1.0)
+    gopt = A.DPOptimizerFastGradientClipping(torch.optim.SGD(ghost.parameters(), lr=0.1), noise_multiplier=0.0, max_grad_norm=1.0, expected_batch_size=n)
+    dpl = A.DPLossFastGradientClipping(ghost, gopt, PerSampleMSE("mean"), "mean")
+    dpl(ghost(x.to(DEV).bfloat16()), y.to(DEV).bfloat16()).backward()
+    # oracle: the same bf16 model evaluated sample by sample with autograd (bf16 forward)
+    ref = copy.deepcopy(mlp).bfloat16()
+    norms = []
+    for i in range(n):
+        ref.zero_grad()
+        PerSampleMSE("sum")(ref(x[i : i + 1].bfloat16()), y[i : i + 1].bfloat16()).backward()
+        norms.append(torch.sqrt(sum(p.grad.double().pow(2).sum() for p in ref.parameters())))
+    close(ghost.per_sample_gradient_norms, torch.stack(norms), 2e-2, 1e-6)
+    for p in ghost.parameters():
+        assert p._norm_sample.dtype == torch.float32 and p.grad.dtype == torch.bfloat16
+    gopt.step()
+
+
+def test_ghost_tied_parameters_raise(A):
+    class Tied(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.fc = nn.Linear(6, 6)
+
+        def forward(self, x):
+            return self.fc(self.fc(x))
+
+    ghost = A.GradSampleModuleFastGradientClipping(Tied().to(DEV))
+    with pytest.raises(NotImplementedError, match="tying"):
+        ghost(torch.randn(2, 6, device=DEV))
+
+
+# ---- make_private end to end ----------------------------------------------------------------------
+@pytest.mark.parametrize("mode", ["hooks", "ghost"])
+def test_make_private_trains(A, mode):
+    torch.manual_seed(13)
+    net = ResBlock().to(DEV)
+    ds = TensorDataset(torch.randn(16, 16, 8, 8), torch.randint(0, 10, (16,)))
+    dl = DataLoader(ds, batch_size=8)
+    engine = A.PrivacyEngine()
+    out = engine.make_private(
+        module=net, optimizer=torch.optim.SGD(net.parameters(), lr=0.05), data_loader=dl, noise_multiplier=1.0,
+        max_grad_norm=1.0, poisson_sampling=False, grad_sample_mode=mode,
+    )
+    model, opt = out[0], out[1]
+    crit = out[2] if mode == "ghost" else nn.CrossEntropyLoss()
+    before = [p.detach().clone() for p in net.parameters()]
+    for x, y in dl:
+        opt.zero_grad()
+        crit(model(x.to(DEV)), y.to(DEV)).backward()
+        opt.step()
+    assert len(engine.accountant) == 2 and engine.accountant.history[0][:2] == (1.0, 0.5)
+    assert all(not torch.equal(b, p) for b, p in zip(before, net.parameters()))
+    assert all(torch.isfinite(p).all() for p in net.parameters())
+
+
+def test_mixed_precision_dtypes(A):
+    """mixed_precision_test.py:107-213 checks dtypes only: fp32 parameters under bf16 autocast keep
+    fp32 grads; bf16 parameters give bf16 grads."""
+    net = nn.Sequential(nn.Linear(16, 32), nn.ReLU(), nn.Linear(32, 4)).to(DEV)
+    gsm = A.GradSampleModule(net, loss_reduction="mean")
+    opt = A.DPOptimizer(torch.optim.SGD(gsm.parameters(), lr=0.1), noise_multiplier=1.0, max_grad_norm=1.0, expected_batch_size=4)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        out = gsm(torch.randn(4, 16, device=DEV))
+        assert out.dtype == torch.bfloat16
+        out.float().sum().backward()
+    opt.step()
+    for p in net.parameters():
+        assert p.grad.dtype == torch.float32 and p.summed_grad.dtype == torch.float32
+    low = nn.Linear(16, 4).to(DEV).bfloat16()
+    gl = A.GradSampleModule(low, loss_reduction="mean")
+    ol = A.DPOptimizer(torch.optim.SGD(gl.parameters(), lr=0.1), noise_multiplier=1.0, max_grad_norm=1.0, expected_batch_size=4)
+    gl(torch.randn(4, 16, device=DEV).bfloat16()).sum().backward()
+    ol.step()
+    for p in low.parameters():
+        assert p.grad.dtype == torch.bfloat16 and p.grad_sample.dtype == torch.bfloat16

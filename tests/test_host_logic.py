@@ -1,0 +1,514 @@
+"""Host-side behaviour of the drop-in layer that needs no GPU: registry, hook bookkeeping,
+guards and error paths. Arithmetic is not tested here (it has no CPU implementation: the
+tests below assert that it fails loudly instead)."""
+
+from unittest.mock import MagicMock
+
+import pytest
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+from torch.utils.data import DataLoader, TensorDataset
+
+import opacus_amd
+from opacus_amd import (
+    DPOptimizer,
+    DPOptimizerFastGradientClipping,
+    GradSampleHooks,
+    GradSampleHooksFastGradientClipping,
+    GradSampleModule,
+    GradSampleModuleFastGradientClipping,
+    PrivacyEngine,
+    register_grad_sampler,
+    register_norm_sampler,
+)
+from opacus_amd.grad_sample import get_gsm_class, get_hooks_class, prepare_module
+from opacus_amd.optimizers import get_optimizer_class
+from opacus_amd.utils.fast_gradient_clipping_utils import DPLossFastGradientClipping, DPTensorFastGradientClipping
+
+
+class Scale(nn.Module):
+    """A custom layer with a torch-only sampler: lets the hook machinery run on the CPU."""
+
+    def __init__(self, d):
+        super().__init__()
+        self.w = nn.Parameter(torch.ones(d))
+
+    def forward(self, x):
+        return x * self.w
+
+
+@register_grad_sampler(Scale)
+def scale_grad_sample(layer, activations, backprops):
+    prod = activations[0] * backprops
+    return {layer.w: prod.reshape(prod.shape[0], -1, prod.shape[-1]).sum(1)}
+
+
+@register_norm_sampler(Scale)
+def scale_norm_sample(layer, activations, backprops):
+    prod = activations[0] * backprops
+    return {layer.w: prod.reshape(prod.shape[0], -1, prod.shape[-1]).sum(1).norm(dim=1)}
+
+
+# ---- registry ---------------------------------------------------------------------------
+def test_registry_writes_both_engines_and_last_wins():
+    assert GradSampleHooks.GRAD_SAMPLERS[Scale] is scale_grad_sample
+    assert GradSampleHooksFastGradientClipping.GRAD_SAMPLERS[Scale] is scale_grad_sample
+    assert GradSampleHooksFastGradientClipping.NORM_SAMPLERS[Scale] is scale_norm_sample
+    assert Scale not in getattr(GradSampleHooks, "NORM_SAMPLERS", {})
+
+    class Tmp(nn.Module):
+        pass
+
+    @register_grad_sampler([Tmp])
+    def first(layer, a, b):
+        return {}
+
+    @register_grad_sampler(Tmp)
+    def second(layer, a, b):
+        return {}
+
+    assert GradSampleHooks.GRAD_SAMPLERS[Tmp] is second
+    GradSampleHooks.GRAD_SAMPLERS.pop(Tmp, None)
+    GradSampleHooksFastGradientClipping.GRAD_SAMPLERS.pop(Tmp, None)
+
+
+def test_builtin_samplers_are_registered():
+    for cls in (nn.Linear, nn.Conv1d, nn.Conv2d, nn.Embedding, nn.GroupNorm, nn.RMSNorm):
+        assert cls in GradSampleHooks.GRAD_SAMPLERS
+    assert set(GradSampleHooksFastGradientClipping.NORM_SAMPLERS) >= {nn.Linear, nn.Embedding}
+
+
+def test_mode_tables():
+    assert get_gsm_class("hooks") is GradSampleModule
+    assert get_gsm_class("ghost") is GradSampleModuleFastGradientClipping
+    assert get_hooks_class("hooks") is GradSampleHooks
+    assert get_hooks_class("ghost") is GradSampleHooksFastGradientClipping
+    with pytest.raises(NotImplementedError):
+        get_gsm_class("ew")
+    with pytest.raises(ValueError):
+        get_gsm_class("nonsense")
+    assert get_optimizer_class("flat", False, "hooks") is DPOptimizer
+    assert get_optimizer_class("flat", False, "ghost") is DPOptimizerFastGradientClipping
+    with pytest.raises(NotImplementedError):
+        get_optimizer_class("per_layer", False, "hooks")
+    with pytest.raises(NotImplementedError):
+        get_optimizer_class("flat", True, "hooks")
+    with pytest.raises(ValueError):
+        get_optimizer_class("weird", False, "hooks")
+
+
+# ---- wrapper behaviour --------------------------------------------------------------------
+def test_wrapper_surface():
+    net = nn.Sequential(nn.Linear(4, 3), nn.ReLU(), nn.Linear(3, 2))
+    gsm = GradSampleModule(net)
+    assert all(k.startswith("_module.") for k in gsm.state_dict())
+    assert gsm._module[0] is net[0]
+    assert len(net.autograd_grad_sample_hooks) == 4  # forward + backward hook for each Linear
+    for p in net.parameters():
+        assert p.grad_sample is None and p._forward_counter == 0
+    with pytest.raises(ValueError, match="twice"):
+        GradSampleModule(net)
+    back = gsm.to_standard_module()
+    assert back is net and not hasattr(net, "autograd_grad_sample_hooks")
+    for p in net.parameters():
+        assert not hasattr(p, "grad_sample") and not hasattr(p, "_forward_counter")
+    GradSampleModule(net)  # can be wrapped again after cleanup
+
+
+def test_submodule_passthrough_and_repr():
+    class Net(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.fc1 = nn.Linear(2, 2)
+
+        def forward(self, x):
+            return self.fc1(x)
+
+    gsm = GradSampleModule(Net())
+    assert isinstance(gsm.fc1, nn.Linear)
+    with pytest.raises(AttributeError):
+        gsm.nothing_here
+    assert repr(gsm).startswith("GradSampleModule(Net(")
+
+
+def test_buffers_are_rejected_in_strict_mode():
+    net = nn.Sequential(nn.Linear(4, 4), nn.BatchNorm1d(4))
+    with pytest.raises(NotImplementedError):
+        GradSampleModule(net)
+    errors = GradSampleModule.validate(net, strict=False)
+    assert len(errors) == 1
+
+
+def test_wrap_model_false_returns_hooks_object():
+    net = nn.Linear(3, 3)
+    hooks = prepare_module(net, grad_sample_mode="hooks", wrap_model=False)
+    assert isinstance(hooks, GradSampleHooks) and not isinstance(hooks, nn.Module)
+    hooks.cleanup()
+    assert not hasattr(net.weight, "grad_sample")
+
+
+def test_no_capture_in_eval_or_no_grad_or_disabled():
+    net = Scale(3)
+    gsm = GradSampleModule(net)
+    x = torch.randn(2, 3)
+    gsm.eval()
+    gsm(x)
+    assert not hasattr(net, "activations")
+    gsm.train()
+    with torch.no_grad():
+        gsm(x)
+    assert not hasattr(net, "activations")
+    gsm.disable_hooks()
+    gsm(x)
+    assert not hasattr(net, "activations")
+    gsm.enable_hooks()
+    gsm(x)
+    assert len(net.activations) == 1 and net.w._forward_counter == 1
+
+
+# ---- hook machinery on the CPU, through a torch-only custom sampler ----------------------------
+@pytest.mark.parametrize("loss_reduction", ["mean", "sum"])
+@pytest.mark.parametrize("batch_first", [True, False])
+def test_hook_flow_with_custom_sampler(loss_reduction, batch_first):
+    torch.manual_seed(0)
+    net = Scale(5)
+    gsm = GradSampleModule(net, loss_reduction=loss_reduction, batch_first=batch_first)
+    x = torch.randn(4, 3, 5) if batch_first else torch.randn(3, 4, 5)  # batch of 4 either way
+    out = gsm(x)
+    loss = out.pow(2).mean() if loss_reduction == "mean" else out.pow(2).sum()
+    loss.backward()
+    gs = net.w.grad_sample
+    assert gs.shape == (4, 5)
+    # per-sample gradients of a mean loss are those of the sum loss: they add up to n * grad
+    factor = 4 if loss_reduction == "mean" else 1
+    torch.testing.assert_close(gs.sum(0), net.w.grad * factor, rtol=1e-5, atol=1e-6)
+    assert not hasattr(net, "max_batch_len") and net.activations == []
+
+
+def test_second_backward_makes_a_list_and_zero_grad_clears():
+    net = Scale(3)
+    gsm = GradSampleModule(net, loss_reduction="sum")
+    for _ in range(2):
+        gsm(torch.randn(2, 3)).sum().backward()
+    assert isinstance(net.w.grad_sample, list) and len(net.w.grad_sample) == 2
+    gsm(torch.randn(2, 3)).sum().backward()
+    assert len(net.w.grad_sample) == 3
+    gsm.zero_grad()
+    assert net.w.grad_sample is None
+
+
+def test_forbid_grad_accumulation():
+    net = Scale(3)
+    gsm = GradSampleModule(net, loss_reduction="sum")
+    gsm.forbid_grad_accumulation()
+    gsm(torch.randn(2, 3)).sum().backward()
+    with pytest.raises(ValueError, match="Poisson sampling is not compatible"):
+        gsm(torch.randn(2, 3)).sum().backward()
+
+
+def test_tied_layer_used_twice_accumulates_within_a_pass():
+    net = Scale(3)
+
+    class Twice(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.s = net
+
+        def forward(self, x):
+            return self.s(self.s(x))
+
+    gsm = GradSampleModule(Twice(), loss_reduction="sum")
+    x = torch.randn(4, 3)
+    gsm(x).sum().backward()
+    gs = net.w.grad_sample
+    assert isinstance(gs, torch.Tensor) and gs.shape == (4, 3)
+    torch.testing.assert_close(gs.sum(0), net.w.grad)
+
+
+def test_ghost_hooks_with_custom_norm_sampler_and_tying_guard():
+    net = Scale(3)
+    gsm = GradSampleModuleFastGradientClipping(net, loss_reduction="sum", max_grad_norm=1.0)
+    x = torch.randn(4, 3)
+    gsm(x).sum().backward()
+    torch.testing.assert_close(net.w._norm_sample, x.norm(dim=1))
+    assert net.w.grad_sample is None
+
+    class Twice(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.s = Scale(3)
+
+        def forward(self, x):
+            return self.s(self.s(x))
+
+    tied = GradSampleModuleFastGradientClipping(Twice(), loss_reduction="sum")
+    with pytest.raises(NotImplementedError, match="tying"):
+        tied(torch.randn(2, 3))
+    with pytest.raises(AttributeError):
+        tied.per_sample_gradient_norms
+
+
+# ---- no CPU fallback ------------------------------------------------------------------------
+def test_builtin_samplers_fail_loudly_on_cpu_tensors():
+    gsm = GradSampleModule(nn.Linear(4, 3), loss_reduction="sum")
+    out = gsm(torch.randn(2, 4))
+    with pytest.raises(RuntimeError, match="GPU only"):
+        out.sum().backward()
+
+
+def test_optimizer_fails_loudly_on_cpu_tensors():
+    lin = nn.Linear(2, 2)
+    opt = DPOptimizer(torch.optim.SGD(lin.parameters(), lr=0.1), noise_multiplier=0.0, max_grad_norm=1.0, expected_batch_size=2)
+    for p in lin.parameters():
+        p.grad_sample = torch.randn(2, *p.shape)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        opt.step()
+
+
+def test_missing_library_is_an_error(monkeypatch, tmp_path):
+    from opacus_amd import _lib
+
+    monkeypatch.setattr(_lib, "_LIB", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", tmp_path / "libdpsgd_hip.so")
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        _lib.lib()
+
+
+# ---- DPOptimizer bookkeeping ------------------------------------------------------------------
+def _opt(lin, **kw):
+    args = dict(noise_multiplier=1.0, max_grad_norm=1.0, expected_batch_size=4)
+    args.update(kw)
+    return DPOptimizer(torch.optim.SGD(lin.parameters(), lr=0.1), **args)
+
+
+def test_optimizer_constructor_checks_and_delegation():
+    lin = nn.Linear(2, 2)
+    lin.bias.requires_grad_(False)
+    with pytest.raises(ValueError):
+        _opt(lin, loss_reduction="max")
+    with pytest.raises(ValueError):
+        _opt(lin, expected_batch_size=None)
+    opt = _opt(lin, expected_batch_size=None, loss_reduction="sum")
+    assert opt.params == [lin.weight] and lin.weight.summed_grad is None
+    assert opt.param_groups is opt.original_optimizer.param_groups
+    assert opt.state is opt.original_optimizer.state and opt.defaults["lr"] == 0.1
+    assert repr(opt) == repr(opt.original_optimizer)
+    assert opt.state_dict() == opt.original_optimizer.state_dict()
+
+
+def test_grad_sample_access_errors_and_accumulated_iterations():
+    lin = nn.Linear(2, 2)
+    opt = _opt(lin)
+    with pytest.raises(ValueError, match="Are you using GradSampleModule"):
+        opt.grad_samples
+    for p in lin.parameters():
+        p.grad_sample = None
+    with pytest.raises(ValueError, match="not initialized"):
+        opt.grad_samples
+    lin.weight.grad_sample = [torch.zeros(1, 2, 2), torch.zeros(3, 2, 2)]
+    lin.bias.grad_sample = torch.zeros(4, 2)
+    assert opt._get_flat_grad_sample(lin.weight).shape == (4, 2, 2)
+    with pytest.raises(ValueError, match="inconsistent"):
+        opt.accumulated_iterations
+    lin.bias.grad_sample = [torch.zeros(1, 2), torch.zeros(3, 2)]
+    assert opt.accumulated_iterations == 2
+    lin.bias.grad_sample = "bad"
+    with pytest.raises(ValueError, match="Unexpected grad_sample type"):
+        opt.grad_samples
+
+
+def test_processed_flag_guard():
+    from opacus_amd.optimizers.optimizer import _check_processed_flag, _mark_as_processed
+
+    t = [torch.zeros(1), torch.zeros(1)]
+    _check_processed_flag(t)
+    _mark_as_processed(t)
+    with pytest.raises(ValueError, match="haven't been cleared"):
+        _check_processed_flag(t)
+    lin = nn.Linear(2, 2)
+    opt = _opt(lin)
+    for p in lin.parameters():
+        p.grad_sample = torch.zeros(4, *p.shape)
+        _mark_as_processed(p.grad_sample)
+    with pytest.raises(ValueError, match="haven't been cleared"):
+        opt.clip_and_accumulate()
+
+
+def test_skip_queue_and_zero_grad():
+    lin = nn.Linear(2, 2)
+    opt = _opt(lin)
+    assert opt._check_skip_next_step() is False
+    opt.signal_skip_step(True)
+    opt.signal_skip_step(False)
+    assert opt._check_skip_next_step(pop_next=False) is True
+    assert opt._check_skip_next_step() is True and opt._check_skip_next_step() is False
+    for p in lin.parameters():
+        p.grad_sample = torch.zeros(4, *p.shape)
+        p.summed_grad = torch.zeros_like(p)
+    opt._is_last_step_skipped = True
+    opt.zero_grad()
+    assert lin.weight.grad_sample is None and lin.weight.summed_grad is not None
+    opt._is_last_step_skipped = False
+    opt.zero_grad()
+    assert lin.weight.summed_grad is None
+
+
+def test_no_trainable_parameters_is_a_plain_step():
+    lin = nn.Linear(2, 2)
+    for p in lin.parameters():
+        p.requires_grad_(False)
+    opt = DPOptimizer(torch.optim.SGD(lin.parameters(), lr=0.1), noise_multiplier=1.0, max_grad_norm=1.0, expected_batch_size=1)
+    assert opt.pre_step() is True
+
+
+def test_ghost_optimizer_is_always_one_iteration():
+    lin = nn.Linear(2, 2)
+    opt = DPOptimizerFastGradientClipping(
+        torch.optim.SGD(lin.parameters(), lr=0.1), noise_multiplier=0.0, max_grad_norm=1.0, expected_batch_size=2
+    )
+    assert opt.accumulated_iterations == 1
+    assert opt.clip_and_accumulate() is None and opt._get_flat_grad_sample(lin.weight) is None
+    # accumulate: summed_grad shares p.grad unless a skipped step is queued
+    for p in lin.parameters():
+        p.grad = torch.ones_like(p)
+    opt.accumulate()
+    assert lin.weight.summed_grad.data_ptr() == lin.weight.grad.data_ptr()
+    opt.accumulate()
+    assert torch.all(lin.weight.summed_grad == 2)
+    opt.zero_grad()
+    opt.signal_skip_step(True)
+    for p in lin.parameters():
+        p.grad = torch.ones_like(p)
+    assert opt.pre_step() is False and opt._is_last_step_skipped
+    assert lin.weight.summed_grad.data_ptr() != lin.weight.grad.data_ptr()
+    opt.zero_grad()
+    assert torch.all(lin.weight.summed_grad == 1)  # survives the zero_grad of a skipped step
+
+
+# ---- ghost-clipping loss wrappers ---------------------------------------------------------------
+def _mock_pair(loss_reduction="mean"):
+    module, optimizer = MagicMock(), MagicMock()
+    module.loss_reduction = optimizer.loss_reduction = loss_reduction
+    return module, optimizer
+
+
+def test_dp_tensor_arithmetic_and_scalars():
+    module, optimizer = _mock_pair()
+    t = DPTensorFastGradientClipping(module, optimizer, torch.tensor([1.0, 2.0, 3.0]), "mean")
+    assert t.item() == 2.0 and (t * 2).item() == 4.0 and (2 * t).item() == 4.0
+    assert (t / 2).item() == 1.0 and (t + 1).item() == 3.0 and (1 + t).item() == 3.0
+    assert (t - 1).item() == 1.0 and (5 - t).item() == 3.0 and (-t).item() == -2.0
+    assert (t + t).item() == 4.0 and (t - t).item() == 0.0
+    assert "DPTensorFastGradientClipping(2.0000)" == str(t) and "shape" in repr(t)
+    other = DPTensorFastGradientClipping(module, optimizer, torch.tensor([1.0, 2.0, 3.0]), "sum")
+    assert other.item() == 6.0
+    with pytest.raises(ValueError):
+        t + other
+
+
+def test_dp_tensor_backward_order():
+    module, optimizer = _mock_pair("sum")
+    calls = []
+    optimizer.zero_grad.side_effect = lambda: calls.append("zero_grad")
+    module.get_clipping_coef.side_effect = lambda: (calls.append("coef"), torch.tensor([0.5, 1.0]))[1]
+    module.disable_hooks.side_effect = lambda: calls.append("off")
+    module.enable_hooks.side_effect = lambda: calls.append("on")
+    w = torch.tensor([1.0, 1.0], requires_grad=True)
+    loss = DPTensorFastGradientClipping(module, optimizer, w * torch.tensor([2.0, 3.0]), "sum")
+    loss.backward()
+    assert calls == ["zero_grad", "coef", "off", "on"]
+    # first backward left [2, 3]; it was not zeroed by the mock; second adds coef * [2, 3]
+    torch.testing.assert_close(w.grad, torch.tensor([2.0 + 1.0, 3.0 + 3.0]))
+
+
+def test_dp_loss_requires_consistent_reductions_and_restores_reduction():
+    module, optimizer = _mock_pair("mean")
+    crit = nn.CrossEntropyLoss(reduction="mean")
+    with pytest.raises(AssertionError):
+        DPLossFastGradientClipping(module, optimizer, nn.CrossEntropyLoss(reduction="sum"), "mean")
+    with pytest.raises(AssertionError):
+        DPLossFastGradientClipping(module, optimizer, crit, "max")
+    dpl = DPLossFastGradientClipping(module, optimizer, crit, "mean")
+    logits, y = torch.randn(6, 5), torch.randint(0, 5, (6,))
+    out = dpl(logits, y)
+    assert crit.reduction == "mean" and out.loss_per_sample.shape == (6,)
+    torch.testing.assert_close(out.detach(), F.cross_entropy(logits, y))
+
+
+@pytest.mark.parametrize("loss_reduction", ["mean", "sum"])
+def test_dp_loss_sequence_shape_and_ignore_index(loss_reduction):
+    module, optimizer = _mock_pair(loss_reduction)
+    crit = nn.CrossEntropyLoss(reduction=loss_reduction, ignore_index=-100)
+    dpl = DPLossFastGradientClipping(module, optimizer, crit, loss_reduction)
+    B, T, V = 3, 4, 7
+    logits = torch.randn(B * T, V)
+    y = torch.randint(0, V, (B * T,))
+    y[1] = y[5] = y[6] = -100
+    out = dpl(logits, y, shape=(B, T, V))
+    assert out.loss_per_sample.shape == (B,)
+    tok = F.cross_entropy(logits, y, reduction="none", ignore_index=-100).view(B, T)
+    if loss_reduction == "sum":
+        want = tok.sum(1)
+    else:
+        want = tok.sum(1) / (y.view(B, T) != -100).sum(1).clamp(min=1)
+    torch.testing.assert_close(out.loss_per_sample, want)
+
+
+# ---- PrivacyEngine wiring -----------------------------------------------------------------------
+def _loader(n=8, bs=4):
+    return DataLoader(TensorDataset(torch.randn(n, 4), torch.randint(0, 2, (n,))), batch_size=bs)
+
+
+def test_make_private_arity_and_wiring():
+    with pytest.warns(UserWarning, match="Secure RNG turned off"):
+        engine = PrivacyEngine()
+    net = nn.Linear(4, 2)
+    sgd = torch.optim.SGD(net.parameters(), lr=0.1)
+    model, opt, dl = engine.make_private(
+        module=net, optimizer=sgd, data_loader=_loader(), noise_multiplier=1.1, max_grad_norm=1.0, poisson_sampling=False
+    )
+    assert isinstance(model, GradSampleModule) and type(opt) is DPOptimizer
+    assert opt.expected_batch_size == 4 and opt.noise_multiplier == 1.1 and opt.step_hook is not None
+    opt.step_hook(MagicMock(noise_multiplier=1.1, accumulated_iterations=1))
+    opt.step_hook(MagicMock(noise_multiplier=1.1, accumulated_iterations=1))
+    assert engine.accountant.history == [(1.1, 0.5, 2)] and len(engine.accountant) == 2
+
+    net2 = nn.Linear(4, 2)
+    out = PrivacyEngine().make_private(
+        module=net2,
+        optimizer=torch.optim.SGD(net2.parameters(), lr=0.1),
+        data_loader=_loader(),
+        noise_multiplier=1.0,
+        max_grad_norm=2.0,
+        poisson_sampling=False,
+        grad_sample_mode="ghost",
+    )
+    assert len(out) == 4
+    model, opt, crit, dl = out
+    assert isinstance(model, GradSampleModuleFastGradientClipping) and model.max_grad_norm == 2.0
+    assert type(opt) is DPOptimizerFastGradientClipping and isinstance(crit, DPLossFastGradientClipping)
+
+
+def test_make_private_errors():
+    net, other = nn.Linear(4, 2), nn.Linear(4, 2)
+    engine = PrivacyEngine()
+    common = dict(data_loader=_loader(), noise_multiplier=1.0, max_grad_norm=1.0)
+    with pytest.raises(ValueError, match="Module parameters are different"):
+        engine.make_private(module=net, optimizer=torch.optim.SGD(other.parameters(), lr=0.1), poisson_sampling=False, **common)
+    with pytest.raises(NotImplementedError, match="Poisson"):
+        engine.make_private(module=net, optimizer=torch.optim.SGD(net.parameters(), lr=0.1), **common)
+    assert not hasattr(net, "autograd_grad_sample_hooks")  # refused before anything was attached
+    wrapped = GradSampleModule(net, loss_reduction="sum")
+    with pytest.raises(ValueError, match="Pre-existing GradSampleModule"):
+        engine.make_private(module=wrapped, optimizer=torch.optim.SGD(net.parameters(), lr=0.1), poisson_sampling=False, **common)
+    wrapped.to_standard_module()
+    hooks_obj, opt, _ = engine.make_private(
+        module=net, optimizer=torch.optim.SGD(net.parameters(), lr=0.1), poisson_sampling=False, wrap_model=False, **common
+    )
+    assert isinstance(hooks_obj, GradSampleHooks) and not isinstance(hooks_obj, nn.Module)
+
+
+def test_package_surface():
+    for name in opacus_amd.__all__:
+        assert hasattr(opacus_amd, name)
