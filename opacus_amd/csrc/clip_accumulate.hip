@@ -33,9 +33,9 @@ __device__ __forceinline__ int find_tensor(const MultiArgs& a, int64_t c) {
 template <typename T, bool VEC>
 __global__ __launch_bounds__(kThreads) void sumsq_partial_kernel(MultiArgs a, int64_t n, float* ws) {
   __shared__ float red[kWaves];
-  const int64_t CT = a.prefix[a.K];
+  const uint32_t CT = static_cast<uint32_t>(a.prefix[a.K]);  // grid.x = n * CT fits 31 bits
   const int64_t row = blockIdx.x / CT;
-  const int64_t c = blockIdx.x % CT;
+  const int64_t c = blockIdx.x - static_cast<uint32_t>(row) * CT;
   const int k = find_tensor(a, c);
   const int64_t P = a.P[k];
   const int64_t nchunk = a.prefix[k + 1] - a.prefix[k];
@@ -94,17 +94,20 @@ __global__ void clip_factor_kernel(const float* __restrict__ v, int64_t K, int64
 }
 
 // ---- clip-weighted sum over the batch ----------------------------------------
-// A block owns (kThreads / RS) * W consecutive columns of one tensor (W = 4
-// with VEC, else 1). Thread (cx, ry) walks rows ry, ry+RS, ... of its columns;
-// the RS partial sums meet in LDS in a fixed order. RS = 1 is the streaming
-// shape for large P; RS > 1 keeps the chip busy when P is small and n large.
-template <typename TG, typename TO, bool VEC, int RS>
-__global__ __launch_bounds__(kThreads) void clip_accumulate_kernel(MultiArgs a, int64_t n,
-                                                                     const float* __restrict__ clip,
-                                                                     int accumulate) {
+// A block of NT threads owns (NT / RS) * W consecutive columns of one tensor
+// (W = 4 with VEC, else 1). Thread (cx, ry) walks rows ry, ry+RS, ... of its
+// columns; the RS partial sums meet in LDS in a fixed order. RS = 1 with one
+// wave per block is the streaming shape for large P: every lane keeps U
+// independent 16-byte non-temporal loads in flight (the tensor is read once and
+// never again), and many one-wave blocks measured closest to the HBM read
+// ceiling. RS > 1 keeps the chip busy when P is small and n large.
+template <typename TG, typename TO, bool VEC, int RS, int NT, int U>
+__global__ __launch_bounds__(NT) void clip_accumulate_kernel(MultiArgs a, int64_t n,
+                                                               const float* __restrict__ clip,
+                                                               int accumulate) {
   constexpr int W = VEC ? 4 : 1;
-  constexpr int CX = kThreads / RS;
-  __shared__ float4 part[RS > 1 ? kThreads : 1];
+  constexpr int CX = NT / RS;
+  __shared__ float4 part[RS > 1 ? NT : 1];
   const int k = find_tensor(a, blockIdx.x);
   const int64_t P = a.P[k];
   const int64_t blk = blockIdx.x - a.prefix[k];
@@ -115,7 +118,6 @@ __global__ __launch_bounds__(kThreads) void clip_accumulate_kernel(MultiArgs a, 
   const TG* base = static_cast<const TG*>(a.gs[k]) + col;
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
   if (live) {
-    constexpr int U = 8;
     int64_t r = ry;
     for (; r + (U - 1) * RS < n; r += U * RS) {
       float4 v[U];
@@ -124,7 +126,7 @@ __global__ __launch_bounds__(kThreads) void clip_accumulate_kernel(MultiArgs a, 
       for (int u = 0; u < U; ++u) {
         const TG* p = base + (r + u * RS) * P;
         if (VEC) {
-          v[u] = dpk_io<TG>::load4(p);
+          v[u] = dpk_io<TG>::load4_nt(p);
         } else {
           v[u] = make_float4(dpk_io<TG>::load(p), 0.f, 0.f, 0.f);
         }
@@ -184,18 +186,23 @@ __global__ __launch_bounds__(kThreads) void clip_accumulate_kernel(MultiArgs a, 
   }
 }
 
+constexpr int kStreamThreads = 64;  // block size of the RS = 1 streaming shape
+constexpr int kStreamUnroll = 16;
+
 template <typename TG, typename TO, bool VEC, int RS>
 void launch_clip_accumulate(const MultiArgs& a, int64_t blocks, int64_t n, const float* clip,
                             int accumulate, hipStream_t s) {
-  hipLaunchKernelGGL((clip_accumulate_kernel<TG, TO, VEC, RS>), dim3(static_cast<unsigned>(blocks)),
-                     dim3(kThreads), 0, s, a, n, clip, accumulate);
+  constexpr int NT = RS == 1 ? kStreamThreads : kThreads;
+  constexpr int U = RS == 1 ? kStreamUnroll : 8;
+  hipLaunchKernelGGL((clip_accumulate_kernel<TG, TO, VEC, RS, NT, U>),
+                     dim3(static_cast<unsigned>(blocks)), dim3(NT), 0, s, a, n, clip, accumulate);
 }
 
 template <typename TG, typename TO>
 void dispatch_clip_accumulate(MultiArgs& a, const int64_t* P, int K, int64_t n, const float* clip,
                               int accumulate, bool vec, int rs, hipStream_t s, int64_t* blocks_out) {
   const int W = vec ? 4 : 1;
-  const int64_t cols_per_block = static_cast<int64_t>(kThreads / rs) * W;
+  const int64_t cols_per_block = static_cast<int64_t>((rs == 1 ? kStreamThreads : kThreads) / rs) * W;
   a.prefix[0] = 0;
   for (int k = 0; k < K; ++k) a.prefix[k + 1] = a.prefix[k] + dpk_cdiv(P[k], cols_per_block);
   const int64_t blocks = a.prefix[K];

@@ -55,8 +55,16 @@ __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
   return static_cast<bf16_t>(u >> 16);
 }
 
+typedef float dpk_vf4 __attribute__((ext_vector_type(4)));
+typedef uint32_t dpk_vu2 __attribute__((ext_vector_type(2)));
+
 template <typename T> struct dpk_io;
 template <> struct dpk_io<float> {
+  // load4 with a non-temporal hint: for data that is streamed through exactly once
+  static __device__ __forceinline__ float4 load4_nt(const float* p) {
+    const dpk_vf4 v = __builtin_nontemporal_load(reinterpret_cast<const dpk_vf4*>(p));
+    return make_float4(v.x, v.y, v.z, v.w);
+  }
   static __device__ __forceinline__ float load(const float* p) { return *p; }
   static __device__ __forceinline__ void store(float* p, float v) { *p = v; }
   // 4 consecutive elements, p 16-byte aligned
@@ -68,6 +76,15 @@ template <> struct dpk_io<float> {
   }
 };
 template <> struct dpk_io<bf16_t> {
+  static __device__ __forceinline__ float4 load4_nt(const bf16_t* p) {
+    const dpk_vu2 r = __builtin_nontemporal_load(reinterpret_cast<const dpk_vu2*>(p));
+    float4 v;
+    v.x = __uint_as_float(r.x << 16);
+    v.y = __uint_as_float(r.x & 0xffff0000u);
+    v.z = __uint_as_float(r.y << 16);
+    v.w = __uint_as_float(r.y & 0xffff0000u);
+    return v;
+  }
   static __device__ __forceinline__ float load(const bf16_t* p) { return bf16_to_f32(*p); }
   static __device__ __forceinline__ void store(bf16_t* p, float v) { *p = f32_to_bf16(v); }
   // 4 consecutive elements, p 8-byte aligned

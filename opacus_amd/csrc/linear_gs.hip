@@ -4,9 +4,10 @@
 // T == 1 is a rank-1 outer product per sample: no contraction, the kernel is
 // bound by the n*out*in store stream. T > 1 is a batched GEMM with K = T on the
 // fp32 MFMA path (bf16 inputs are widened on the way into LDS, which is exact).
-// Both kernels also emit the per-sample sum of squares of what they wrote, as
-// one partial per block reduced in a fixed order, so the optimizer's norm pass
-// over the n*out*in tensor disappears.
+// Both paths also deliver the per-sample sum of squares of what they wrote (the
+// MFMA kernel as one partial per block reduced in a fixed order, the rank-one
+// case from its closed form), so the optimizer's norm pass over the n*out*in
+// tensor disappears.
 #include "dpk_common.h"
 #include "mfma_f32.h"
 
@@ -14,48 +15,74 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / DPK_WAVE;
-constexpr int kOuterRows = 64;  // rows of one sample's gs written by one block (T == 1)
+constexpr int kOuterRowsPerThread = 8;  // rows of gs each thread writes (T == 1)
 
 // ---- T == 1 ------------------------------------------------------------------
-// Block = CX column threads x (256 / CX) row groups; a thread keeps its 4 (or 1)
-// activations in registers and walks the block's rows. Each row of the block is
-// a contiguous run of CX*W floats.
-template <typename TIN, typename TOUT, bool VEC>
+// Block = CX column threads x RY = 256 / CX row groups; a thread keeps its 4 (or
+// 1) activations in registers and writes kOuterRowsPerThread rows, so a block
+// covers 8 * RY rows of CX * W contiguous elements each. With CX = 256 that is 8
+// rows of 4 KB: few rows per block (many small blocks in flight) is what keeps
+// the store stream closest to the HBM write ceiling.
+template <typename TIN, typename TOUT, bool VEC, int CXLOG2>
 __global__ __launch_bounds__(kThreads) void linear_outer_kernel(
-    const TIN* __restrict__ b, const TIN* __restrict__ a, TOUT* __restrict__ gs,
-    float* __restrict__ partials, int64_t M, int64_t N, float scale, int cx_log2, int64_t tiles_m,
-    int64_t tiles_n) {
+    const TIN* __restrict__ b, const TIN* __restrict__ a, TOUT* __restrict__ gs, int64_t M, int64_t N,
+    float scale, uint32_t tiles_m, uint32_t tiles_n) {
   constexpr int W = VEC ? 4 : 1;
-  __shared__ float red[kWaves];
-  const int CX = 1 << cx_log2, RY = kThreads >> cx_log2;
-  const int cx = threadIdx.x & (CX - 1), ry = threadIdx.x >> cx_log2;
-  const int64_t per_sample = tiles_m * tiles_n;
-  const int64_t sample = blockIdx.x / per_sample;
-  const int64_t rem = blockIdx.x % per_sample;
-  const int64_t i0 = (rem / tiles_n) * kOuterRows;
-  const int64_t j = ((rem % tiles_n) * CX + cx) * W;
+  constexpr int CX = 1 << CXLOG2, RY = kThreads >> CXLOG2;
+  constexpr int ROWS = kOuterRowsPerThread * RY;
+  const int cx = threadIdx.x & (CX - 1), ry = threadIdx.x >> CXLOG2;
+  // 32-bit index arithmetic: a block only issues a handful of stores, so 64-bit
+  // divisions here would cost more instructions than the work itself
+  const uint32_t per_sample = tiles_m * tiles_n;
+  const uint32_t sample32 = blockIdx.x / per_sample;
+  const uint32_t rem = blockIdx.x - sample32 * per_sample;
+  const uint32_t tm = rem / tiles_n, tn = rem - tm * tiles_n;
+  const int64_t sample = sample32;
+  const int64_t i0 = static_cast<int64_t>(tm) * ROWS + ry;
+  const int64_t j = (static_cast<int64_t>(tn) * CX + cx) * W;
+  if (j >= N) return;
   const TIN* bs = b + sample * M;
-  TOUT* out = gs + sample * M * N;
-  float ss = 0.f;
-  if (j < N) {
-    float4 av = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (VEC) av = dpk_io<TIN>::load4(a + sample * N + j);
-    else av.x = dpk_io<TIN>::load(a + sample * N + j);
-    const float a2 = VEC ? (av.x * av.x + av.y * av.y) + (av.z * av.z + av.w * av.w) : av.x * av.x;
-    const int64_t iend = (i0 + kOuterRows < M) ? i0 + kOuterRows : M;
-    float b2 = 0.f;
-    for (int64_t i = i0 + ry; i < iend; i += RY) {
-      const float bv = scale * dpk_io<TIN>::load(bs + i);
-      b2 = fmaf(bv, bv, b2);
-      if (VEC) dpk_io<TOUT>::store4(out + i * N + j, make_float4(bv * av.x, bv * av.y, bv * av.z, bv * av.w));
-      else dpk_io<TOUT>::store(out + i * N + j, bv * av.x);
+  TOUT* out = gs + sample * M * N + j;
+  float4 av = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (VEC) av = dpk_io<TIN>::load4(a + sample * N + j);
+  else av.x = dpk_io<TIN>::load(a + sample * N + j);
+  float bv[kOuterRowsPerThread];
+#pragma unroll
+  for (int r = 0; r < kOuterRowsPerThread; ++r) {
+    const int64_t i = i0 + r * RY;
+    bv[r] = i < M ? scale * dpk_io<TIN>::load(bs + i) : 0.f;
+  }
+#pragma unroll
+  for (int r = 0; r < kOuterRowsPerThread; ++r) {
+    const int64_t i = i0 + r * RY;
+    if (i < M) {
+      if (VEC) dpk_io<TOUT>::store4(out + i * N, make_float4(bv[r] * av.x, bv[r] * av.y, bv[r] * av.z, bv[r] * av.w));
+      else dpk_io<TOUT>::store(out + i * N, bv[r] * av.x);
     }
-    ss = a2 * b2;
   }
-  if (partials) {
-    const float s = block_sum<kWaves>(ss, red);
-    if (threadIdx.x == 0) partials[blockIdx.x] = s;
+}
+
+// Sum of squares of a rank-one matrix: sum_ij (s b_i a_j)^2 = (sum_i (s b_i)^2)(sum_j a_j^2).
+// One block per sample; keeps the reduction out of the store-bound kernel above.
+template <typename TIN>
+__global__ __launch_bounds__(kThreads) void rank1_sumsq_kernel(const TIN* __restrict__ b,
+                                                                 const TIN* __restrict__ a,
+                                                                 float* __restrict__ sumsq, int64_t M,
+                                                                 int64_t N, float scale) {
+  __shared__ float red[kWaves];
+  const int64_t sample = blockIdx.x;
+  float sb = 0.f, sa = 0.f;
+  for (int64_t i = threadIdx.x; i < M; i += kThreads) {
+    const float v = scale * dpk_io<TIN>::load(b + sample * M + i);
+    sb = fmaf(v, v, sb);
   }
+  for (int64_t i = threadIdx.x; i < N; i += kThreads) {
+    const float v = dpk_io<TIN>::load(a + sample * N + i);
+    sa = fmaf(v, v, sa);
+  }
+  const float tb = block_sum<kWaves>(sb, red);
+  const float ta = block_sum<kWaves>(sa, red);
+  if (threadIdx.x == 0) sumsq[sample] = tb * ta;
 }
 
 // ---- T > 1 -------------------------------------------------------------------
@@ -136,6 +163,7 @@ __global__ __launch_bounds__(kThreads) void rowsum_kernel(const TIN* __restrict_
 struct Plan {
   bool outer;
   int cx_log2;
+  int rows_pb;
   int bm;
   int64_t tiles_m, tiles_n;
 };
@@ -145,14 +173,16 @@ Plan make_plan(int64_t T, int64_t M, int64_t N, bool vec) {
   p.outer = (T == 1);
   if (p.outer) {
     const int64_t cols = dpk_cdiv(N, vec ? 4 : 1);
-    int lg = 3;  // at least 8 column threads
-    while (lg < 8 && (1LL << lg) < cols) ++lg;
+    // column threads per block: 8, 32, 128 or 256 (the instantiated shapes)
+    const int lg = cols > 128 ? 8 : cols > 32 ? 7 : cols > 8 ? 5 : 3;
     p.cx_log2 = lg;
     p.bm = 0;
-    p.tiles_m = dpk_cdiv(M, kOuterRows);
+    p.rows_pb = kOuterRowsPerThread * (kThreads >> lg);
+    p.tiles_m = dpk_cdiv(M, p.rows_pb);
     p.tiles_n = dpk_cdiv(cols, 1LL << lg);
   } else {
     p.cx_log2 = 0;
+    p.rows_pb = 0;
     p.bm = (M > 64 && N > 64) ? 128 : 64;
     p.tiles_m = dpk_cdiv(M, p.bm);
     p.tiles_n = dpk_cdiv(N, p.bm);
@@ -168,12 +198,21 @@ void launch_linear(const Plan& p, bool vec, const void* b, const void* a, void* 
   const TIN* ap = static_cast<const TIN*>(a);
   TOUT* gp = static_cast<TOUT*>(gs);
   if (p.outer) {
-    if (vec)
-      hipLaunchKernelGGL((linear_outer_kernel<TIN, TOUT, true>), grid, block, 0, s, bp, ap, gp,
-                         partials, M, N, scale, p.cx_log2, p.tiles_m, p.tiles_n);
-    else
-      hipLaunchKernelGGL((linear_outer_kernel<TIN, TOUT, false>), grid, block, 0, s, bp, ap, gp,
-                         partials, M, N, scale, p.cx_log2, p.tiles_m, p.tiles_n);
+#define DPK_OUTER(V, LG)                                                                          \
+  hipLaunchKernelGGL((linear_outer_kernel<TIN, TOUT, V, LG>), grid, block, 0, s, bp, ap, gp, M, N, \
+                     scale, static_cast<uint32_t>(p.tiles_m), static_cast<uint32_t>(p.tiles_n))
+    if (vec) {
+      if (p.cx_log2 == 8) DPK_OUTER(true, 8);
+      else if (p.cx_log2 == 7) DPK_OUTER(true, 7);
+      else if (p.cx_log2 == 5) DPK_OUTER(true, 5);
+      else DPK_OUTER(true, 3);
+    } else {
+      if (p.cx_log2 == 8) DPK_OUTER(false, 8);
+      else if (p.cx_log2 == 7) DPK_OUTER(false, 7);
+      else if (p.cx_log2 == 5) DPK_OUTER(false, 5);
+      else DPK_OUTER(false, 3);
+    }
+#undef DPK_OUTER
   } else if (p.bm == 128) {
     if (vec)
       hipLaunchKernelGGL((linear_mfma_kernel<128, 128, TIN, TOUT, true>), grid, block, 0, s, bp, ap,
@@ -200,7 +239,7 @@ bool linear_vec(const void* b, const void* a, const void* gs, int in_dtype, int 
 }  // namespace
 
 extern "C" size_t dpk_linear_gs_workspace_bytes(int64_t n, int64_t T, int64_t out, int64_t in) {
-  if (n <= 0 || T <= 0 || out <= 0 || in <= 0) return 0;
+  if (n <= 0 || T <= 1 || out <= 0 || in <= 0) return 0;  // the rank-one path needs none
   // The scalar plan never has fewer blocks than the vector plan.
   const Plan p = make_plan(T, out, in, false);
   return dpk_align_up(static_cast<size_t>(n * p.tiles_m * p.tiles_n) * sizeof(float), 256);
@@ -226,7 +265,7 @@ extern "C" int dpk_linear_gs(const void* b, const void* a, int in_dtype, void* g
   DPK_REQUIRE(blocks <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: %lld blocks exceed the grid limit", who,
               (long long)blocks);
   float* partials = nullptr;
-  if (sumsq) {
+  if (sumsq && !p.outer) {
     const size_t need = static_cast<size_t>(blocks) * sizeof(float);
     DPK_REQUIRE(ws && ws_bytes >= need, DPK_E_WORKSPACE, "%s: workspace %zu < %zu bytes", who,
                 ws_bytes, need);
@@ -243,7 +282,15 @@ extern "C" int dpk_linear_gs(const void* b, const void* a, int in_dtype, void* g
   else
     launch_linear<float, bf16_t>(p, vec, b, a, gs, partials, n, T, out, in, scale, s);
   DPK_LAUNCH_CHECK(who);
-  if (sumsq) {
+  if (sumsq && p.outer) {
+    if (in_dtype == DPK_F32)
+      hipLaunchKernelGGL(rank1_sumsq_kernel<float>, dim3(static_cast<unsigned>(n)), dim3(kThreads), 0, s,
+                         static_cast<const float*>(b), static_cast<const float*>(a), sumsq, out, in, scale);
+    else
+      hipLaunchKernelGGL(rank1_sumsq_kernel<bf16_t>, dim3(static_cast<unsigned>(n)), dim3(kThreads), 0, s,
+                         static_cast<const bf16_t*>(b), static_cast<const bf16_t*>(a), sumsq, out, in, scale);
+    DPK_LAUNCH_CHECK(who);
+  } else if (sumsq) {
     dpk_launch_reduce_rows(partials, n, p.tiles_m * p.tiles_n, sumsq, 0, 1.f, s);
     DPK_LAUNCH_CHECK(who);
   }

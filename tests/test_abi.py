@@ -73,7 +73,8 @@ def test_workspace_queries_and_argument_errors_without_a_gpu():
     from opacus_amd import _lib
 
     lib = _lib.lib()
-    assert lib.dpk_linear_gs_workspace_bytes(128, 1, 4096, 4096) >= 128 * 64 * 4
+    assert lib.dpk_linear_gs_workspace_bytes(128, 1, 4096, 4096) == 0
+    assert lib.dpk_linear_gs_workspace_bytes(16, 256, 1024, 1024) >= 16 * 8 * 8 * 4
     assert lib.dpk_sumsq_rows_workspace_bytes(4, 8192 * 3) >= 4 * 3 * 4
     assert lib.dpk_linear_ghost_norm_workspace_bytes(2, 512, 8, 8) >= 2 * 2 * 36 * 4
     assert lib.dpk_embedding_workspace_bytes(2, 100, 64) > 0
