@@ -11,6 +11,7 @@
 // (linear.py:87-89, :92).
 #include "dpk_common.h"
 #include "mfma_bf16.h"
+#include "mfma_bf16_dlds.h"
 #include "mfma_f32.h"
 
 namespace {
@@ -106,6 +107,90 @@ __global__ __launch_bounds__(kThreads) void ghost_norm_bf16_kernel(
   contract_and_store(tg, ta, pw != nullptr, ti == tj ? 1.f : 2.f, pw, pb, red);
 }
 
+// Workgroups are handed to the 8 XCDs round-robin by hardware id. Renumbering
+// them so that each XCD works through one contiguous range of (sample, tile pair)
+// keeps the rows of a sample in that XCD's L2 while its tile pairs are computed.
+__device__ __forceinline__ uint32_t xcd_contiguous_id(uint32_t bid, uint32_t nb) {
+  const uint32_t x = bid & 7u, idx = bid >> 3;
+  const uint32_t base = nb >> 3, rem = nb & 7u;
+  return x * base + (x < rem ? x : rem) + idx;
+}
+
+// Fast path: operand tiles go global -> LDS directly through a ring of stages
+// (mfma_bf16_dlds.h). Needs Dout % 64 == Din % 64 == 0 and 16-byte aligned rows.
+// The block tile is BM x BN with BM = R * BN: row blocks I, column blocks J, and
+// the block-triangle J >= R * I is visited. Column blocks inside the row block's
+// own diagonal square (J < R * (I + 1)) count once - together they cover that
+// square completely - the ones beyond it twice.
+template <class C>
+__global__ __launch_bounds__(C::kThreads) void ghost_norm_bf16_dlds_kernel(
+    const bf16_t* __restrict__ b, const bf16_t* __restrict__ a, float* __restrict__ pw,
+    float* __restrict__ pb, int64_t T, int64_t Dout, int64_t Din, int nJ, int npairs) {
+  constexpr int R = C::BM / C::BN;
+  __shared__ mb16d::Smem<C> sm;
+  __shared__ float red[C::kWaves];
+  const uint32_t lid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  const int64_t sample = lid / static_cast<uint32_t>(npairs);
+  int pair = static_cast<int>(lid % static_cast<uint32_t>(npairs));
+  int I = 0;
+  while (pair >= nJ - R * I) {
+    pair -= nJ - R * I;
+    ++I;
+  }
+  const int J = R * I + pair;
+  const int64_t m0a = static_cast<int64_t>(I) * C::BM, m0b = static_cast<int64_t>(J) * C::BN;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wm0 = (wave / C::kWaveCols) * 64, wn0 = (wave % C::kWaveCols) * 64;
+  mb16d::Tile tg, ta;
+  tg.clear();
+  ta.clear();
+  const bf16_t* bs = b + sample * T * Dout;
+  mb16d::mainloop<C>(tg, sm, bs, bs, Dout, m0a, m0b, T, Dout, wm0, wn0);
+  if (pw) {
+    const bf16_t* as = a + sample * T * Din;
+    mb16d::mainloop<C>(ta, sm, as, as, Din, m0a, m0b, T, Din, wm0, wn0);
+  }
+  // rows past T hold copies of row T - 1: leave them out
+  const int rmax = static_cast<int>(T - m0a < C::BM ? T - m0a : C::BM);
+  const int cmax = static_cast<int>(T - m0b < C::BN ? T - m0b : C::BN);
+  float sw = 0.f, sb = 0.f;
+  const int kh = lane >> 5, l32 = lane & 31;
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int row = wm0 + i * 32 + (v >> 2) * 8 + kh * 4 + (v & 3), col = wn0 + j * 32 + l32;
+        if (row < rmax && col < cmax) {
+          const float g = tg.acc[i][j][v];
+          sb += g;
+          sw = fmaf(g, ta.acc[i][j][v], sw);
+        }
+      }
+  const float weight = J < R * (I + 1) ? 1.f : 2.f;
+  if (pw) {
+    const float s = block_sum<C::kWaves>(sw, red);
+    if (threadIdx.x == 0) pw[lid] = s * weight;
+  }
+  if (pb) {
+    const float s = block_sum<C::kWaves>(sb, red);
+    if (threadIdx.x == 0) pb[lid] = s * weight;
+  }
+}
+
+// 128 x 128 tile, 4 waves, two 32 KB stages: two blocks fit a CU, which measured
+// better than one block with a deeper ring or a 256 x 128 tile (8 waves, 3 stages).
+using GhostCfg = mb16d::Config<2, 2, 2>;
+
+// Tile pairs per sample for a BM x BN tiling of the T x T block-triangle.
+int64_t ghost_pairs(int64_t T, int bm, int bn) {
+  const int64_t nI = dpk_cdiv(T, bm), nJ = dpk_cdiv(T, bn), R = bm / bn;
+  int64_t p = 0;
+  for (int64_t I = 0; I < nI; ++I) p += nJ - R * I;
+  return p;
+}
+
 // T == 1: closed forms of linear.py:71-79. One block per sample.
 template <typename T_>
 __global__ __launch_bounds__(kThreads) void ghost_norm_rank1_kernel(
@@ -174,7 +259,10 @@ extern "C" int dpk_linear_ghost_norm(const void* b, const void* a, int dtype, fl
   }
   const int B = tile_edge(T);
   const int64_t nt = dpk_cdiv(T, B);
-  const int64_t npairs = nt * (nt + 1) / 2;
+  // bf16 with 64-aligned feature sizes takes the direct-to-LDS kernel
+  const bool dlds = dtype == DPK_BF16 && B == 128 && out % 64 == 0 && (in % 64 == 0 || !norm_w) &&
+                    dpk_aligned(b, 16) && dpk_aligned(a, 16);
+  const int64_t npairs = dlds ? ghost_pairs(T, GhostCfg::BM, GhostCfg::BN) : nt * (nt + 1) / 2;
   const int64_t blocks = n * npairs;
   DPK_REQUIRE(nt < 32768 && blocks <= DPK_MAX_GRID_X, DPK_E_SHAPE,
               "%s: %lld blocks exceed the grid limit", who, (long long)blocks);
@@ -204,6 +292,12 @@ extern "C" int dpk_linear_ghost_norm(const void* b, const void* a, int dtype, fl
     const bool vec = out % 8 == 0 && in % 8 == 0 && dpk_aligned(b, 16) && dpk_aligned(a, 16);
     const bf16_t* bp = static_cast<const bf16_t*>(b);
     const bf16_t* ap = static_cast<const bf16_t*>(a);
+    if (dlds) {
+      hipLaunchKernelGGL((ghost_norm_bf16_dlds_kernel<GhostCfg>), dim3(static_cast<unsigned>(blocks)),
+                         dim3(GhostCfg::kThreads), 0, s, bp, ap, pw, pb, T, out, in,
+                         (int)dpk_cdiv(T, GhostCfg::BN), (int)npairs);
+      DPK_LAUNCH_CHECK(who);
+    } else {
 #define DPK_GN_LAUNCH(B_, V_)                                                                  \
   hipLaunchKernelGGL((ghost_norm_bf16_kernel<B_, V_>), grid, block, 0, s, bp, ap, pw, pb, T, out, \
                      in, (int)nt, (int)npairs)
@@ -215,6 +309,7 @@ extern "C" int dpk_linear_ghost_norm(const void* b, const void* a, int dtype, fl
       else DPK_GN_LAUNCH(64, false);
     }
 #undef DPK_GN_LAUNCH
+    }
   }
   DPK_LAUNCH_CHECK(who);
   if (pw) {

@@ -69,16 +69,19 @@ struct Tile {
 // Rows of the source run along k: element (m, k) at base[m * ld + k].
 // VEC: ld % 8 == 0 and base 16-byte aligned, so every 8-element group is one
 // 16-byte load; otherwise elements are fetched one by one with bounds checks.
+// Two register slots, so that the tile after next is already in flight while
+// the next one waits in registers for its LDS buffer to become free.
 template <int BMN, bool VEC>
 struct Loader {
   static constexpr int R = BMN * BK / 8 / NTHREADS;
   static_assert(R >= 1, "tile too small for this loader");
   const bf16_t* base;
   int64_t ld, m0, M, K;
-  uint4 st[R];
+  uint4 st[2][R];
   __device__ __forceinline__ Loader(const bf16_t* base_, int64_t ld_, int64_t m0_, int64_t M_,
                                     int64_t K_)
       : base(base_), ld(ld_), m0(m0_), M(M_), K(K_) {}
+  template <int SLOT>
   __device__ __forceinline__ void fetch(int64_t k0) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
@@ -98,38 +101,58 @@ struct Loader {
           v = make_uint4(w[0], w[1], w[2], w[3]);
         }
       }
-      st[r] = v;
+      st[SLOT][r] = v;
     }
   }
+  template <int SLOT>
   __device__ __forceinline__ void commit(bf16_t (*S)[LDK]) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const int idx = threadIdx.x + r * NTHREADS;
-      *reinterpret_cast<uint4*>(&S[idx / (BK / 8)][(idx % (BK / 8)) * 8]) = st[r];
+      *reinterpret_cast<uint4*>(&S[idx / (BK / 8)][(idx % (BK / 8)) * 8]) = st[SLOT][r];
     }
   }
 };
 
+// Software pipeline over k, two tiles per trip so that every register slot and
+// LDS buffer index is a compile-time constant:
+//   LDS buffer (kt & 1) holds tile kt, register slot ((kt + 1) & 1) holds tile
+//   kt + 1 (loaded during the previous step), and the loads of tile kt + 2 are
+//   issued before the MFMAs of tile kt start. Global-memory latency is thus
+//   covered by a whole step of MFMAs rather than by a fraction of one.
 template <int BM, int BN, class LA, class LB>
 __device__ __forceinline__ void mainloop(Tile<BM, BN>& t, Smem<BM, BN>& sm, LA& la, LB& lb,
                                          int64_t K) {
   const int64_t nk = (K + BK - 1) / BK;
-  la.fetch(0);
-  lb.fetch(0);
-  la.commit(sm.a[0]);
-  lb.commit(sm.b[0]);
+  la.template fetch<0>(0);
+  lb.template fetch<0>(0);
+  if (nk > 1) {
+    la.template fetch<1>(BK);
+    lb.template fetch<1>(BK);
+  }
+  la.template commit<0>(sm.a[0]);
+  lb.template commit<0>(sm.b[0]);
   __syncthreads();
-  for (int64_t kt = 0; kt < nk; ++kt) {
-    const int cur = static_cast<int>(kt & 1);
-    const bool more = kt + 1 < nk;
-    if (more) {
-      la.fetch((kt + 1) * BK);
-      lb.fetch((kt + 1) * BK);
+  for (int64_t kt = 0; kt < nk; kt += 2) {
+    if (kt + 2 < nk) {
+      la.template fetch<0>((kt + 2) * BK);
+      lb.template fetch<0>((kt + 2) * BK);
     }
-    t.mma(sm.a[cur], sm.b[cur]);
-    if (more) {
-      la.commit(sm.a[cur ^ 1]);
-      lb.commit(sm.b[cur ^ 1]);
+    t.mma(sm.a[0], sm.b[0]);
+    if (kt + 1 < nk) {
+      la.template commit<1>(sm.a[1]);
+      lb.template commit<1>(sm.b[1]);
+    }
+    __syncthreads();
+    if (kt + 1 >= nk) break;
+    if (kt + 3 < nk) {
+      la.template fetch<1>((kt + 3) * BK);
+      lb.template fetch<1>((kt + 3) * BK);
+    }
+    t.mma(sm.a[1], sm.b[1]);
+    if (kt + 2 < nk) {
+      la.template commit<0>(sm.a[0]);
+      lb.template commit<0>(sm.b[0]);
     }
     __syncthreads();
   }

@@ -1,0 +1,190 @@
+// bf16 MFMA Gram tiles fed by direct global->LDS loads (gfx950).
+//
+// Same contraction as mfma_bf16.h (C[m][n] = sum_k A[m][k] B[n][k], operands with
+// k contiguous), but the operand tiles never pass through VGPRs: each lane issues
+// global_load_lds_dwordx4, which drops its 16 bytes at LDS[base + lane * 16], and
+// an NS-deep ring of LDS stages keeps NS - 1 k-tiles in flight behind the MFMAs.
+// A block is NWR x NWC waves, each owning a 64 x 64 piece (2 x 2 MFMA tiles of
+// 32 x 32) of the (64 NWR) x (64 NWC) block tile.
+// Requirements of this path (the caller falls back to mfma_bf16.h otherwise):
+// K % 64 == 0, row stride % 8 == 0, 16-byte aligned base.
+//
+// LDS stage layout: row-major [rows][64 bf16] = 128 bytes per row, no padding
+// (a wave's 64 lanes must land contiguously), 16-byte chunks XOR-swizzled:
+//   physical chunk = logical chunk ^ ((row >> 1) & 7).
+// For the MFMA operand read (16 consecutive rows, one logical chunk, 16 bytes
+// per lane) the 16 lanes then hit 16 distinct 16-byte slots of the 256-byte bank
+// space: conflict-free. Rows beyond the matrix are fetched from the last valid
+// row instead (no fault, finite values); the caller masks them out of its
+// reduction.
+#pragma once
+
+#include "dpk_common.h"
+#include "mfma_bf16.h"
+
+namespace mb16d {
+
+using mb16::bf16x8;
+using mb16::floatx16;
+
+constexpr int BK = 64;
+constexpr int ROW_BYTES = BK * 2;  // 128
+
+typedef __attribute__((address_space(3))) void* lptr_t;
+
+template <int NWR, int NWC, int NS>
+struct Config {
+  static constexpr int kWaveRows = NWR, kWaveCols = NWC;
+  static constexpr int kWaves = NWR * NWC;
+  static constexpr int kThreads = 64 * kWaves;
+  static constexpr int BM = 64 * NWR, BN = 64 * NWC;
+  static constexpr int kStages = NS;
+  static constexpr int kStageBytes = (BM + BN) * ROW_BYTES;
+  // global->LDS instructions per thread and k-tile: one per 1 KB of tile per wave
+  static constexpr int kLoadsA = BM * ROW_BYTES / 1024 / kWaves;
+  static constexpr int kLoadsB = BN * ROW_BYTES / 1024 / kWaves;
+  static constexpr int kLoadsPerTile = kLoadsA + kLoadsB;
+  static_assert(BM * ROW_BYTES % (1024 * kWaves) == 0 && BN * ROW_BYTES % (1024 * kWaves) == 0,
+                "tile rows must split evenly over the waves");
+};
+
+template <class C>
+struct Smem {
+  alignas(1024) unsigned char stage[C::kStages][C::kStageBytes];  // per stage: A tile, then B tile
+};
+
+__device__ __forceinline__ int swz(int row, int chunk) { return chunk ^ ((row >> 1) & 7); }
+
+// One direct global->LDS load of 16 bytes per lane: lane l's bytes land at
+// LDS[lds_base + l * 16]. Written as inline assembly so that waiting for it stays
+// in this file's hands: the ring below wants loads of later tiles to remain in
+// flight across the barrier and across the LDS reads of the current tile.
+__device__ __forceinline__ void load16_to_lds(const void* gptr, uint32_t lds_base) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, off\n\t"
+      :
+      : "s"(lds_base), "v"(gptr)
+      : "memory", "m0");
+}
+
+__device__ __forceinline__ uint32_t lds_offset(const void* p) {
+  return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lptr_t)p));
+}
+
+// Issues the loads of one tile of 8 * NLOADS * NWAVES rows (rows m0.., k offset
+// k0) into LDS at byte offset `dst`.
+template <int NLOADS, int NWAVES>
+__device__ __forceinline__ void issue_tile(const bf16_t* base, int64_t ld, int64_t m0, int64_t M,
+                                           int64_t k0, uint32_t dst) {
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+#pragma unroll
+  for (int r = 0; r < NLOADS; ++r) {
+    const int grp = r * NWAVES + wave;  // 8 rows of 128 bytes = 1 KB per wave instruction
+    const int row = grp * 8 + (lane >> 3);
+    const int lc = swz(row, lane & 7);  // which logical chunk lives at this physical slot
+    int64_t m = m0 + row;
+    m = m < M ? m : M - 1;
+    load16_to_lds(base + m * ld + k0 + lc * 8, dst + grp * 1024);
+  }
+}
+
+// Waits until at most N of this wave's loads are outstanding, then meets the
+// other waves. No fence beyond that: the LDS reads of the previous tile were
+// consumed by MFMAs already, and nothing else is shared.
+template <int N>
+__device__ __forceinline__ void wait_and_barrier() {
+  static_assert(N == 0 || N == 6 || N == 8 || N == 12 || N == 16 || N == 18 || N == 24,
+                "add the vmcnt value to the switch below");
+  switch (N) {
+    case 0: asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory"); break;
+    case 6: asm volatile("s_waitcnt vmcnt(6)\n\ts_barrier" ::: "memory"); break;
+    case 8: asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory"); break;
+    case 12: asm volatile("s_waitcnt vmcnt(12)\n\ts_barrier" ::: "memory"); break;
+    case 16: asm volatile("s_waitcnt vmcnt(16)\n\ts_barrier" ::: "memory"); break;
+    case 18: asm volatile("s_waitcnt vmcnt(18)\n\ts_barrier" ::: "memory"); break;
+    default: asm volatile("s_waitcnt vmcnt(24)\n\ts_barrier" ::: "memory"); break;
+  }
+}
+
+// The 64 x 64 accumulator piece of one wave.
+struct Tile {
+  floatx16 acc[2][2];
+
+  __device__ __forceinline__ void clear() {
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+  }
+
+  // As / Bs: the stage's operand tiles; (wm0, wn0): this wave's corner in the block tile.
+  __device__ __forceinline__ void mma(const unsigned char* As, const unsigned char* Bs, int wm0, int wn0) {
+    const int lane = threadIdx.x & 63;
+    const int kh = lane >> 5, l32 = lane & 31;
+    // All operand fragments of the k-tile are requested up front (16 reads of 16
+    // bytes per lane); the MFMAs of step ks then only wait for their own four,
+    // so LDS latency is paid once per tile instead of once per step.
+    constexpr int KS = BK / 16;
+    bf16x8 av[KS][2], bv[KS][2];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int row = wm0 + i * 32 + l32;
+        av[ks][i] = *reinterpret_cast<const bf16x8*>(As + row * ROW_BYTES + swz(row, ks * 2 + kh) * 16);
+      }
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int row = wn0 + j * 32 + l32;
+        bv[ks][j] = *reinterpret_cast<const bf16x8*>(Bs + row * ROW_BYTES + swz(row, ks * 2 + kh) * 16);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);  // keep the reads ahead of the MFMAs
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[ks][i], bv[ks][j], acc[i][j], 0, 0, 0);
+  }
+};
+
+// C tile += A[m0a.., :K] . B[m0b.., :K]^T with an NS-stage ring. Every iteration
+// issues exactly one tile's worth of loads (past the end the last tile is
+// fetched again into a stage nobody reads), so the number of loads that may
+// stay outstanding while tile kt is awaited is the constant
+// kLoadsPerTile * (NS - 2).
+template <class C>
+__device__ __forceinline__ void mainloop(Tile& t, Smem<C>& sm, const bf16_t* abase,
+                                         const bf16_t* bbase, int64_t ld, int64_t m0a, int64_t m0b,
+                                         int64_t M, int64_t K, int wm0, int wn0) {
+  constexpr int NS = C::kStages;
+  const int64_t nk = K / BK;
+  const uint32_t lds0 = lds_offset(&sm.stage[0][0]);
+  auto issue = [&](int64_t kt, int stage) {
+    const int64_t kc = kt < nk ? kt : nk - 1;
+    const uint32_t st = lds0 + stage * C::kStageBytes;
+    issue_tile<C::kLoadsA, C::kWaves>(abase, ld, m0a, M, kc * BK, st);
+    issue_tile<C::kLoadsB, C::kWaves>(bbase, ld, m0b, M, kc * BK, st + C::BM * ROW_BYTES);
+  };
+#pragma unroll
+  for (int s = 0; s < NS - 1; ++s) issue(s, s);
+  int stage = 0;  // stage of tile kt
+  for (int64_t kt = 0; kt < nk; ++kt) {
+    // tile kt has landed for every wave, and the stage of tile kt - 1 is free again
+    wait_and_barrier<C::kLoadsPerTile*(NS - 2)>();
+    issue(kt + NS - 1, stage == 0 ? NS - 1 : stage - 1);
+    const unsigned char* st = sm.stage[stage];
+    t.mma(st, st + C::BM * ROW_BYTES, wm0, wn0);
+    stage = stage + 1 == NS ? 0 : stage + 1;
+  }
+  wait_and_barrier<0>();  // the ring may be reused by the caller's next main loop
+}
+
+}  // namespace mb16d
