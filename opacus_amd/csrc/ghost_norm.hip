@@ -181,7 +181,10 @@ __global__ __launch_bounds__(C::kThreads) void ghost_norm_bf16_dlds_kernel(
 
 // 128 x 128 tile, 4 waves, two 32 KB stages: two blocks fit a CU, which measured
 // better than one block with a deeper ring or a 256 x 128 tile (8 waves, 3 stages).
-using GhostCfg = mb16d::Config<2, 2, 2>;
+#ifndef DPK_GHOST_CFG
+#define DPK_GHOST_CFG 2, 2, 2, 64
+#endif
+using GhostCfg = mb16d::Config<DPK_GHOST_CFG>;
 
 // Tile pairs per sample for a BM x BN tiling of the T x T block-triangle.
 int64_t ghost_pairs(int64_t T, int bm, int bn) {

@@ -27,13 +27,16 @@ namespace mb16d {
 using mb16::bf16x8;
 using mb16::floatx16;
 
-constexpr int BK = 64;
-constexpr int ROW_BYTES = BK * 2;  // 128
 
 typedef __attribute__((address_space(3))) void* lptr_t;
 
-template <int NWR, int NWC, int NS>
+template <int NWR, int NWC, int NS, int BK_ = 64>
 struct Config {
+  static_assert(BK_ == 64 || BK_ == 32, "k extent of a stage: 64 or 32 bf16");
+  static constexpr int BK = BK_;
+  static constexpr int ROW_BYTES = BK * 2;          // 128 or 64
+  static constexpr int kChunks = ROW_BYTES / 16;    // 16-byte chunks per row: 8 or 4
+  static constexpr int kRowsPerKB = 1024 / ROW_BYTES;  // rows covered by one wave instruction
   static constexpr int kWaveRows = NWR, kWaveCols = NWC;
   static constexpr int kWaves = NWR * NWC;
   static constexpr int kThreads = 64 * kWaves;
@@ -53,7 +56,12 @@ struct Smem {
   alignas(1024) unsigned char stage[C::kStages][C::kStageBytes];  // per stage: A tile, then B tile
 };
 
-__device__ __forceinline__ int swz(int row, int chunk) { return chunk ^ ((row >> 1) & 7); }
+// 8 chunks per row: chunk ^ ((row >> 1) & 7); 4 chunks per row: chunk ^ ((row >> 2) & 3).
+// Either way 16 consecutive rows at one logical chunk cover the 256-byte bank space once.
+template <class C>
+__device__ __forceinline__ int swz(int row, int chunk) {
+  return C::kChunks == 8 ? chunk ^ ((row >> 1) & 7) : chunk ^ ((row >> 2) & 3);
+}
 
 // One direct global->LDS load of 16 bytes per lane: lane l's bytes land at
 // LDS[lds_base + l * 16]. Written as inline assembly so that waiting for it stays
@@ -73,22 +81,26 @@ __device__ __forceinline__ uint32_t lds_offset(const void* p) {
   return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lptr_t)p));
 }
 
-// Issues the loads of one tile of 8 * NLOADS * NWAVES rows (rows m0.., k offset
-// k0) into LDS at byte offset `dst`.
-template <int NLOADS, int NWAVES>
-__device__ __forceinline__ void issue_tile(const bf16_t* base, int64_t ld, int64_t m0, int64_t M,
-                                           int64_t k0, uint32_t dst) {
+// issue_one: the r-th global->LDS load of a tile (rows m0.., k offset k0) whose
+// LDS image starts at byte offset `dst`; issue_tile: all NLOADS of them.
+template <class C>
+__device__ __forceinline__ void issue_one(const bf16_t* base, int64_t ld, int64_t m0, int64_t M,
+                                          int64_t k0, uint32_t dst, int r) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int grp = r * C::kWaves + wave;  // 1 KB of consecutive rows per wave instruction
+  const int row = grp * C::kRowsPerKB + lane / C::kChunks;
+  const int lc = swz<C>(row, lane % C::kChunks);  // which logical chunk lives at this physical slot
+  int64_t m = m0 + row;
+  m = m < M ? m : M - 1;
+  load16_to_lds(base + m * ld + k0 + lc * 8, dst + grp * 1024);
+}
+
+template <class C, int NLOADS>
+__device__ __forceinline__ void issue_tile(const bf16_t* base, int64_t ld, int64_t m0, int64_t M,
+                                           int64_t k0, uint32_t dst) {
 #pragma unroll
-  for (int r = 0; r < NLOADS; ++r) {
-    const int grp = r * NWAVES + wave;  // 8 rows of 128 bytes = 1 KB per wave instruction
-    const int row = grp * 8 + (lane >> 3);
-    const int lc = swz(row, lane & 7);  // which logical chunk lives at this physical slot
-    int64_t m = m0 + row;
-    m = m < M ? m : M - 1;
-    load16_to_lds(base + m * ld + k0 + lc * 8, dst + grp * 1024);
-  }
+  for (int r = 0; r < NLOADS; ++r) issue_one<C>(base, ld, m0, M, k0, dst, r);
 }
 
 // Waits until at most N of this wave's loads are outstanding, then meets the
@@ -96,10 +108,11 @@ __device__ __forceinline__ void issue_tile(const bf16_t* base, int64_t ld, int64
 // consumed by MFMAs already, and nothing else is shared.
 template <int N>
 __device__ __forceinline__ void wait_and_barrier() {
-  static_assert(N == 0 || N == 6 || N == 8 || N == 12 || N == 16 || N == 18 || N == 24,
+  static_assert(N == 0 || N == 4 || N == 6 || N == 8 || N == 12 || N == 16 || N == 18 || N == 24,
                 "add the vmcnt value to the switch below");
   switch (N) {
     case 0: asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory"); break;
+    case 4: asm volatile("s_waitcnt vmcnt(4)\n\ts_barrier" ::: "memory"); break;
     case 6: asm volatile("s_waitcnt vmcnt(6)\n\ts_barrier" ::: "memory"); break;
     case 8: asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory"); break;
     case 12: asm volatile("s_waitcnt vmcnt(12)\n\ts_barrier" ::: "memory"); break;
@@ -122,36 +135,46 @@ struct Tile {
         for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
   }
 
-  // As / Bs: the stage's operand tiles; (wm0, wn0): this wave's corner in the block tile.
-  __device__ __forceinline__ void mma(const unsigned char* As, const unsigned char* Bs, int wm0, int wn0) {
+  // As / Bs: the stage's operand tiles; (wm0, wn0): this wave's corner in the block tile;
+  // issue(q), q < NLOADS: issues the q-th load of the tile being prefetched.
+  template <class C, int NLOADS, class IssueFn>
+  __device__ __forceinline__ void mma(const unsigned char* As, const unsigned char* Bs, int wm0, int wn0,
+                                      IssueFn issue) {
     const int lane = threadIdx.x & 63;
     const int kh = lane >> 5, l32 = lane & 31;
     // All operand fragments of the k-tile are requested up front (16 reads of 16
     // bytes per lane); the MFMAs of step ks then only wait for their own four,
     // so LDS latency is paid once per tile instead of once per step.
-    constexpr int KS = BK / 16;
+    constexpr int KS = C::BK / 16, ROW_BYTES = C::ROW_BYTES;
     bf16x8 av[KS][2], bv[KS][2];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         const int row = wm0 + i * 32 + l32;
-        av[ks][i] = *reinterpret_cast<const bf16x8*>(As + row * ROW_BYTES + swz(row, ks * 2 + kh) * 16);
+        av[ks][i] = *reinterpret_cast<const bf16x8*>(As + row * ROW_BYTES + swz<C>(row, ks * 2 + kh) * 16);
       }
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         const int row = wn0 + j * 32 + l32;
-        bv[ks][j] = *reinterpret_cast<const bf16x8*>(Bs + row * ROW_BYTES + swz(row, ks * 2 + kh) * 16);
+        bv[ks][j] = *reinterpret_cast<const bf16x8*>(Bs + row * ROW_BYTES + swz<C>(row, ks * 2 + kh) * 16);
       }
     }
     __builtin_amdgcn_sched_barrier(0);  // keep the reads ahead of the MFMAs
+    // MFMAs execute asynchronously: the global->LDS loads of the tile after next
+    // (and their address arithmetic) are issued in their shadow, a few per step.
+    constexpr int PER_STEP = (NLOADS + KS - 1) / KS;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
+    for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[ks][i], bv[ks][j], acc[i][j], 0, 0, 0);
+#pragma unroll
+      for (int q = ks * PER_STEP; q < (ks + 1) * PER_STEP && q < NLOADS; ++q) issue(q);
+      __builtin_amdgcn_sched_barrier(0);
+    }
   }
 };
 
@@ -165,13 +188,14 @@ __device__ __forceinline__ void mainloop(Tile& t, Smem<C>& sm, const bf16_t* aba
                                          const bf16_t* bbase, int64_t ld, int64_t m0a, int64_t m0b,
                                          int64_t M, int64_t K, int wm0, int wn0) {
   constexpr int NS = C::kStages;
+  constexpr int BK = C::BK, ROW_BYTES = C::ROW_BYTES;
   const int64_t nk = K / BK;
   const uint32_t lds0 = lds_offset(&sm.stage[0][0]);
   auto issue = [&](int64_t kt, int stage) {
     const int64_t kc = kt < nk ? kt : nk - 1;
     const uint32_t st = lds0 + stage * C::kStageBytes;
-    issue_tile<C::kLoadsA, C::kWaves>(abase, ld, m0a, M, kc * BK, st);
-    issue_tile<C::kLoadsB, C::kWaves>(bbase, ld, m0b, M, kc * BK, st + C::BM * ROW_BYTES);
+    issue_tile<C, C::kLoadsA>(abase, ld, m0a, M, kc * BK, st);
+    issue_tile<C, C::kLoadsB>(bbase, ld, m0b, M, kc * BK, st + C::BM * ROW_BYTES);
   };
 #pragma unroll
   for (int s = 0; s < NS - 1; ++s) issue(s, s);
@@ -179,9 +203,13 @@ __device__ __forceinline__ void mainloop(Tile& t, Smem<C>& sm, const bf16_t* aba
   for (int64_t kt = 0; kt < nk; ++kt) {
     // tile kt has landed for every wave, and the stage of tile kt - 1 is free again
     wait_and_barrier<C::kLoadsPerTile*(NS - 2)>();
-    issue(kt + NS - 1, stage == 0 ? NS - 1 : stage - 1);
+    const int64_t kn = kt + NS - 1 < nk ? kt + NS - 1 : nk - 1;
+    const uint32_t dst = lds0 + (stage == 0 ? NS - 1 : stage - 1) * C::kStageBytes;
     const unsigned char* st = sm.stage[stage];
-    t.mma(st, st + C::BM * ROW_BYTES, wm0, wn0);
+    t.template mma<C, C::kLoadsPerTile>(st, st + C::BM * ROW_BYTES, wm0, wn0, [&](int q) {
+      if (q < C::kLoadsA) issue_one<C>(abase, ld, m0a, M, kn * BK, dst, q);
+      else issue_one<C>(bbase, ld, m0b, M, kn * BK, dst + C::BM * ROW_BYTES, q - C::kLoadsA);
+    });
     stage = stage + 1 == NS ? 0 : stage + 1;
   }
   wait_and_barrier<0>();  // the ring may be reused by the caller's next main loop
