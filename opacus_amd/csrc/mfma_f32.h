@@ -47,19 +47,24 @@ struct Tile {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
     const int kk = lane >> 5, l32 = lane & 31;
+    // all operand reads of the k-tile first, then its MFMAs: LDS latency is paid
+    // once per tile instead of once per k step
+    float av[BK / 2][TM], bv[BK / 2][TN];
 #pragma unroll
-    for (int k0 = 0; k0 < BK; k0 += 2) {
-      float av[TM], bv[TN];
+    for (int k2 = 0; k2 < BK / 2; ++k2) {
 #pragma unroll
-      for (int i = 0; i < TM; ++i) av[i] = As[k0 + kk][wm0 + i * 32 + l32];
+      for (int i = 0; i < TM; ++i) av[k2][i] = As[2 * k2 + kk][wm0 + i * 32 + l32];
 #pragma unroll
-      for (int j = 0; j < TN; ++j) bv[j] = Bs[k0 + kk][wn0 + j * 32 + l32];
+      for (int j = 0; j < TN; ++j) bv[k2][j] = Bs[2 * k2 + kk][wn0 + j * 32 + l32];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int k2 = 0; k2 < BK / 2; ++k2)
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], bv[j], acc[i][j], 0, 0, 0);
-    }
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[k2][i], bv[k2][j], acc[i][j], 0, 0, 0);
   }
 
   // f(row, col, value) for every accumulator element this thread owns; row and
