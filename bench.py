@@ -1,16 +1,20 @@
 """DP-SGD step throughput on one MI355X: ``python bench.py --gpus 1 --steps K --warmup W``.
 
-Default workload (the one the headline metric is quoted on): a single
+Default workload (the one the headline metric is quoted on, ``--workload c2``): a single
 ``nn.Linear(4096, 4096, bias=True)`` in fp32, batch 128, one position per sample, hooks
 mode: forward, backward (per-sample gradients, 128 x 4096 x 4096 fp32 = 8.59 GB), then
 ``DPOptimizer.step`` (clip at C = 1, accumulate, noise sigma = 1, SGD update) and
-``zero_grad``. Inputs are synthetic N(0,1) tensors resident in HBM before the clock starts.
+``zero_grad``. Inputs are synthetic tensors resident in HBM before the clock starts.
 
-Prints ONE JSON line. ``roofline`` describes the dominant kernel of the step (the
-clip-weighted sum over the batch, which streams the per-sample gradients once), timed
-with HIP events on the launch stream inside the timed region. ``cpu_baseline`` is the
-CPU oracle (a restatement of the reference's einsum path, allocation pattern included)
-timed on this box's host cores on a bounded sample of the same workload.
+Prints ONE JSON line. ``roofline`` describes the dominant kernel of the step, timed with
+HIP events on the launch stream inside the timed region. ``cpu_baseline`` (default
+workload only) is the CPU oracle - a restatement of the reference's einsum path,
+allocation pattern included - timed on this box's host cores on a bounded sample of the
+same workload.
+
+The other four benchmark configurations can be timed with ``--workload c1|c3|c4|c5``
+(same JSON shape, no CPU baseline); they are parity-test shapes first and bench lines
+second.
 """
 
 from __future__ import annotations
@@ -24,53 +28,282 @@ from pathlib import Path
 
 import torch
 import torch.nn as nn
+import torch.nn.functional as F
 
 ROOT = Path(__file__).resolve().parent
 if str(ROOT) not in sys.path:
     sys.path.insert(0, str(ROOT))
 
-HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
-N, D_IN, D_OUT = 128, 4096, 4096
-SIGMA, CLIP, LR = 1.0, 1.0, 0.05
+# MI355X published peaks
+HBM_PEAK_GBS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+MFMA_FP32_PEAK_TFLOPS = 157.3
 
 
-def gpu_step_factory(dev):
+# ---- models of the five configurations -------------------------------------------------
+class SmallCNN(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.conv1 = nn.Conv2d(1, 16, 8, 2, padding=3)
+        self.conv2 = nn.Conv2d(16, 32, 4, 2)
+        self.fc1 = nn.Linear(32 * 4 * 4, 32)
+        self.fc2 = nn.Linear(32, 10)
+
+    def forward(self, x):
+        x = F.max_pool2d(F.relu(self.conv1(x)), 2, 1)
+        x = F.max_pool2d(F.relu(self.conv2(x)), 2, 1)
+        return self.fc2(F.relu(self.fc1(x.flatten(1))))
+
+
+class ResBlock(nn.Module):
+    def __init__(self, ch=64, groups=32):
+        super().__init__()
+        self.c1, self.g1 = nn.Conv2d(ch, ch, 3, padding=1), nn.GroupNorm(groups, ch)
+        self.c2, self.g2 = nn.Conv2d(ch, ch, 3, padding=1), nn.GroupNorm(groups, ch)
+        self.head = nn.Linear(ch, 10)
+
+    def forward(self, x):
+        h = F.relu(self.g1(self.c1(x)))
+        h = F.relu(self.g2(self.c2(h)) + x)
+        return self.head(h.mean(dim=(2, 3)))
+
+
+class Llama(nn.Module):
+    """Decoder stack: RMSNorm, grouped-query attention with rotary embedding, SwiGLU; untied
+    embedding and LM head (ghost clipping does not support tied parameters); bias-free."""
+
+    def __init__(self, vocab=32000, d=2048, heads=16, kv=4, ffn=5632, layers=4):
+        super().__init__()
+        self.emb = nn.Embedding(vocab, d)
+        self.heads, self.kv, self.hd = heads, kv, d // heads
+        self.blocks = nn.ModuleList(
+            nn.ModuleDict(
+                dict(
+                    n1=nn.RMSNorm(d, eps=1e-5),
+                    q=nn.Linear(d, d, bias=False),
+                    k=nn.Linear(d, kv * (d // heads), bias=False),
+                    v=nn.Linear(d, kv * (d // heads), bias=False),
+                    o=nn.Linear(d, d, bias=False),
+                    n2=nn.RMSNorm(d, eps=1e-5),
+                    gate=nn.Linear(d, ffn, bias=False),
+                    up=nn.Linear(d, ffn, bias=False),
+                    down=nn.Linear(ffn, d, bias=False),
+                )
+            )
+            for _ in range(layers)
+        )
+        self.norm = nn.RMSNorm(d, eps=1e-5)
+        self.lm_head = nn.Linear(d, vocab, bias=False)
+
+    @staticmethod
+    def rope(x):
+        T, D = x.shape[-2], x.shape[-1]
+        pos = torch.arange(T, device=x.device, dtype=torch.float32)
+        inv = 1.0 / (10000 ** (torch.arange(0, D, 2, device=x.device, dtype=torch.float32) / D))
+        ang = pos[:, None] * inv[None, :]
+        cos, sin = ang.cos().to(x.dtype), ang.sin().to(x.dtype)
+        x1, x2 = x[..., 0::2], x[..., 1::2]
+        return torch.stack([x1 * cos - x2 * sin, x1 * sin + x2 * cos], dim=-1).flatten(-2)
+
+    def forward(self, ids):
+        h = self.emb(ids)
+        B, T, _ = h.shape
+        for blk in self.blocks:
+            a = blk["n1"](h)
+            q = blk["q"](a).view(B, T, self.heads, self.hd).transpose(1, 2)
+            k = blk["k"](a).view(B, T, self.kv, self.hd).transpose(1, 2)
+            v = blk["v"](a).view(B, T, self.kv, self.hd).transpose(1, 2)
+            q, k = self.rope(q), self.rope(k)
+            att = F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)
+            h = h + blk["o"](att.transpose(1, 2).reshape(B, T, -1))
+            m = blk["n2"](h)
+            h = h + blk["down"](F.silu(blk["gate"](m)) * blk["up"](m))
+        return self.lm_head(self.norm(h))
+
+
+class PerSampleMSE(nn.Module):
+    """Mean squared error against zeros, one value per sample (mean over positions and features)."""
+
+    def __init__(self, reduction="mean"):
+        super().__init__()
+        self.reduction = reduction
+
+    def forward(self, out, _target=None):
+        l = out.float().pow(2).flatten(1).mean(1)
+        if self.reduction == "none":
+            return l
+        return l.mean() if self.reduction == "mean" else l.sum()
+
+
+def ghost_executed_flops(model: nn.Module, n: int, T: int) -> float:
+    """MFMA FLOPs the ghost-norm kernel executes per step: 128 x 128 tiles of the upper
+    block-triangle of both Gram matrices of every Linear layer."""
+    nt = (T + 127) // 128
+    pairs = nt * (nt + 1) // 2
+    total = 0.0
+    for m in model.modules():
+        if isinstance(m, nn.Linear):
+            total += n * pairs * 2.0 * 128 * 128 * (m.in_features + m.out_features)
+    return total
+
+
+# ---- workloads ----------------------------------------------------------------------------
+def workload_c2(dev):
     from opacus_amd import GradSampleModule
     from opacus_amd.optimizers import DPOptimizer
 
+    N, D_IN, D_OUT = 128, 4096, 4096
     torch.manual_seed(0)
     lin = nn.Linear(D_IN, D_OUT, bias=True)
-    x = torch.randn(N, D_IN)
-    b = torch.randn(N, D_OUT)
+    x, b = torch.randn(N, D_IN).to(dev), torch.randn(N, D_OUT).to(dev)
     model = GradSampleModule(lin.to(dev), loss_reduction="sum")
     opt = DPOptimizer(
-        torch.optim.SGD(model.parameters(), lr=LR),
-        noise_multiplier=SIGMA,
-        max_grad_norm=CLIP,
-        expected_batch_size=N,
-        loss_reduction="sum",
+        torch.optim.SGD(model.parameters(), lr=0.05), noise_multiplier=1.0, max_grad_norm=1.0,
+        expected_batch_size=N, loss_reduction="sum",
     )
-    x, b = x.to(dev), b.to(dev)
 
     def step():
         opt.zero_grad(set_to_none=True)
-        y = model(x)
-        y.backward(b)  # backprops ~ N(0,1) injected at the layer output
+        model(x).backward(b)  # backprops ~ N(0,1) injected at the layer output
         opt.step()
 
-    return step, model
+    P = D_OUT * D_IN + D_OUT
+    return dict(
+        step=step, n=N, dtype="f32",
+        workload="Linear(4096->4096, bias) fp32, batch 128, T=1, hooks per-sample grad + clip(C=1) + noise(sigma=1) + SGD",
+        extra={"per_sample_grad_bytes": N * P * 4},
+        # one launch covers weight and bias: reads n * P * 4 bytes, writes P * 4 bytes
+        roofline=dict(
+            kernel="clip_accumulate_kernel<float,float,vec,RS=1,64 threads,U=16>", timer="clip_accumulate",
+            bound="hbm", work_per_launch=float(N * P * 4 + P * 4), unit="GB/s", peak=HBM_PEAK_GBS,
+            # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (KiB per
+            # dispatch), each scaled by what the counter reads for a 1 GiB device copy
+            # (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000): 8,390,854 + 65,552 KiB.
+            traffic=8456406 * 1024,
+        ),
+    )
+
+
+def _hooks_workload(dev, net, x, y, n, sigma, desc, roofline, dtype="f32"):
+    from opacus_amd import GradSampleModule
+    from opacus_amd.optimizers import DPOptimizer
+
+    model = GradSampleModule(net.to(dev), loss_reduction="mean")
+    opt = DPOptimizer(
+        torch.optim.SGD(model.parameters(), lr=0.1), noise_multiplier=sigma, max_grad_norm=1.0, expected_batch_size=n
+    )
+    x, y = x.to(dev), y.to(dev)
+
+    def step():
+        opt.zero_grad(set_to_none=True)
+        F.cross_entropy(model(x), y).backward()
+        opt.step()
+
+    return dict(step=step, n=n, dtype=dtype, workload=desc, extra={}, roofline=roofline)
+
+
+def workload_c1(dev):
+    torch.manual_seed(0)
+    n = 256
+    P = 26010
+    return _hooks_workload(
+        dev, SmallCNN(), torch.randn(n, 1, 28, 28), torch.randint(0, 10, (n,)), n, 1.1,
+        "Small CNN (conv 1->16 k8 s2 p3, conv 16->32 k4 s2, fc 512->32, fc 32->10) fp32, batch 256, hooks, C=1, sigma=1.1",
+        dict(kernel="clip_accumulate_kernel<float,float,*,RS=16> (8 tensors, one launch)", timer="clip_accumulate",
+             bound="hbm", work_per_launch=float(n * P * 4 + P * 4), unit="GB/s", peak=HBM_PEAK_GBS, traffic=None),
+    )
+
+
+def workload_c4(dev):
+    torch.manual_seed(0)
+    n = 256
+    flops = 2.0 * n * 64 * 576 * 1024  # per conv launch
+    return _hooks_workload(
+        dev, ResBlock(), torch.randn(n, 64, 32, 32), torch.randint(0, 10, (n,)), n, 1.0,
+        "ResNet basic block: 2 x Conv2d(64->64, 3x3, p1) + GroupNorm(32), 32x32 images, fp32, batch 256, hooks, C=1, sigma=1",
+        dict(kernel="conv2d_gs_patch_kernel<64,64,float,float>", timer="conv2d_gs", bound="mfma",
+             work_per_launch=flops, unit="TFLOP/s", peak=MFMA_FP32_PEAK_TFLOPS, traffic=None),
+    )
+
+
+def _ghost_workload(dev, net, make_inputs, loss_call, n, T, sigma, desc):
+    from opacus_amd import GradSampleModuleFastGradientClipping
+    from opacus_amd.optimizers import DPOptimizerFastGradientClipping
+
+    net = net.to(dev).bfloat16()
+    model = GradSampleModuleFastGradientClipping(net, loss_reduction="mean", max_grad_norm=1.0)
+    opt = DPOptimizerFastGradientClipping(
+        torch.optim.SGD(model.parameters(), lr=0.01), noise_multiplier=sigma, max_grad_norm=1.0, expected_batch_size=n
+    )
+    inputs = make_inputs()
+
+    def step():
+        opt.zero_grad(set_to_none=True)
+        loss_call(model, opt, inputs).backward()
+        opt.step()
+
+    flops = ghost_executed_flops(net, n, T)
+    return dict(
+        step=step, n=n, dtype="bf16", workload=desc, extra={"ghost_norm_executed_flops_per_step": flops},
+        roofline=dict(kernel="ghost_norm_bf16_dlds_kernel<128x128, 2 stages> (all Linear layers of a step)",
+                      timer="linear_ghost_norm", bound="mfma", work_per_step=flops, unit="TFLOP/s",
+                      peak=MFMA_BF16_PEAK_TFLOPS, traffic=None),
+    )
+
+
+def workload_c3(dev):
+    from opacus_amd import DPLossFastGradientClipping
+
+    torch.manual_seed(0)
+    n, T = 32, 512
+    net = nn.Sequential(nn.Linear(1024, 4096), nn.GELU(), nn.Linear(4096, 1024))
+    crit = {}
+
+    def loss_call(model, opt, x):
+        if "c" not in crit:
+            crit["c"] = DPLossFastGradientClipping(model, opt, PerSampleMSE("mean"), "mean")
+        return crit["c"](model(x), None)
+
+    return _ghost_workload(
+        dev, net, lambda: torch.randn(n, T, 1024).to(dev).bfloat16(), loss_call, n, T, 1.0,
+        "MLP Linear(1024->4096) GELU Linear(4096->1024), bf16, batch 32, T=512, ghost clipping, C=1, sigma=1",
+    )
+
+
+def workload_c5(dev):
+    from opacus_amd import DPLossFastGradientClipping
+
+    torch.manual_seed(0)
+    n, T, V = 16, 1024, 32000
+    net = Llama()
+    crit = {}
+
+    def loss_call(model, opt, ids):
+        if "c" not in crit:
+            crit["c"] = DPLossFastGradientClipping(model, opt, nn.CrossEntropyLoss(), "mean")
+        logits = model(ids)[:, :-1]
+        return crit["c"](logits.reshape(-1, V).float(), ids[:, 1:].reshape(-1), shape=(n, T - 1, V))
+
+    return _ghost_workload(
+        dev, net, lambda: torch.randint(0, V, (n, T)).to(dev), loss_call, n, T, 0.8,
+        "4-layer Llama-style decoder (d 2048, 16 heads / 4 KV, SwiGLU 5632, vocab 32000, untied), bf16, batch 16, seq 1024, ghost clipping, C=1, sigma=0.8",
+    )
+
+
+WORKLOADS = {"c1": workload_c1, "c2": workload_c2, "c3": workload_c3, "c4": workload_c4, "c5": workload_c5}
 
 
 def cpu_baseline(n_sample: int = 16, steps: int = 3) -> dict:
-    """The oracle's DP-SGD step for the same layer on the host cores, on ``n_sample`` of the
-    128 samples (every pass over per-sample data is linear in the batch size)."""
+    """The oracle's DP-SGD step for the default workload on the host cores, on ``n_sample`` of
+    the 128 samples (every pass over per-sample data is linear in the batch size)."""
     from oracle import dp_oracle as O
 
+    N, D_IN, D_OUT = 128, 4096, 4096
     torch.manual_seed(0)
     lin = nn.Linear(D_IN, D_OUT, bias=True)
     x = torch.randn(n_sample, D_IN)
     b = torch.randn(n_sample, D_OUT)
-    sgd = torch.optim.SGD(lin.parameters(), lr=LR)
+    sgd = torch.optim.SGD(lin.parameters(), lr=0.05)
 
     def step():
         sgd.zero_grad(set_to_none=True)
@@ -79,8 +312,8 @@ def cpu_baseline(n_sample: int = 16, steps: int = 3) -> dict:
         bp = O.scale_backprops(b, n_sample, "sum")
         gs_w, gs_b = O.linear_grad_sample(x, bp)
         gs = [O.store_grad_sample(gs_w, n_sample), O.store_grad_sample(gs_b, n_sample)]
-        _, _, summed = O.clip_and_accumulate(gs, CLIP)
-        grads = O.add_noise_and_scale(summed, [lin.weight.shape, lin.bias.shape], SIGMA, CLIP, n_sample, "sum")
+        _, _, summed = O.clip_and_accumulate(gs, 1.0)
+        grads = O.add_noise_and_scale(summed, [lin.weight.shape, lin.bias.shape], 1.0, 1.0, n_sample, "sum")
         lin.weight.grad, lin.bias.grad = grads
         sgd.step()
 
@@ -104,6 +337,7 @@ def main() -> None:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="c2")
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing")
     ap.add_argument(
         "--calibrate-copy",
@@ -120,7 +354,8 @@ def main() -> None:
     from opacus_amd import kernels
 
     dev = torch.device("cuda:0")
-    step, model = gpu_step_factory(dev)
+    w = WORKLOADS[args.workload](dev)
+    step = w["step"]
     for _ in range(args.warmup):
         step()
     if args.calibrate_copy:
@@ -137,16 +372,24 @@ def main() -> None:
         elapsed = time.perf_counter() - t0
 
     ms_per_step = elapsed / args.steps * 1e3
-    value = N * args.steps / elapsed
-
-    # dominant kernel: the clip-weighted sum. One launch covers weight and bias:
-    # reads n * P * 4 bytes, writes P * 4 bytes, P = 4096 * 4096 + 4096.
-    P = D_OUT * D_IN + D_OUT
-    algo_bytes = N * P * 4 + P * 4
-    ca = [s.elapsed_time(e) for s, e in times.get("clip_accumulate", [])]
-    ca_ms = sum(ca) / max(len(ca), 1)
-    achieved = algo_bytes / (ca_ms * 1e-3) / 1e9 if ca_ms > 0 else 0.0
+    value = w["n"] * args.steps / elapsed
     kernel_ms = {k: sum(s.elapsed_time(e) for s, e in v) / args.steps for k, v in times.items()}
+
+    r = dict(w["roofline"])
+    spans = [s.elapsed_time(e) for s, e in times.get(r.pop("timer"), [])]
+    if "work_per_step" in r:  # several launches per step share the work figure
+        work, ms = r.pop("work_per_step"), sum(spans) / args.steps
+        r["launches_per_step"] = len(spans) // args.steps
+    else:
+        work, ms = r.pop("work_per_launch"), sum(spans) / max(len(spans), 1)
+    scale = 1e9 if r["unit"] == "GB/s" else 1e12
+    achieved = work / (ms * 1e-3) / scale if ms > 0 else 0.0
+    roofline = {
+        "kernel": r["kernel"], "bound": r["bound"], "achieved": achieved, "peak": r["peak"], "unit": r["unit"],
+        "frac": achieved / r["peak"], "traffic": r["traffic"], "algorithmic_work": work, "kernel_ms": ms,
+    }
+    if "launches_per_step" in r:
+        roofline["launches_per_step"] = r["launches_per_step"]
 
     out = {
         "metric": "dp_sgd_step_samples_per_sec",
@@ -159,30 +402,12 @@ def main() -> None:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
+        "dtype": w["dtype"],
         "data": "synthetic",
-        "config": {
-            "workload": "Linear(4096->4096, bias) fp32, batch 128, T=1, hooks per-sample grad + clip(C=1) + noise(sigma=1) + SGD",
-            "global_batch": N,
-            "per_sample_grad_bytes": N * P * 4,
-            "kernel_ms_per_step": kernel_ms,
-        },
-        "roofline": {
-            "kernel": "clip_accumulate_kernel<float,float,vec,RS=1>",
-            "bound": "hbm",
-            "achieved": achieved,
-            "peak": HBM_PEAK_GBS,
-            "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS,
-            # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (KiB per
-            # dispatch), each scaled by what the counter reads for a 1 GiB device copy
-            # (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000): 8,390,854 + 65,552 KiB.
-            "traffic": 8456406 * 1024,
-            "algorithmic_bytes_per_launch": algo_bytes,
-            "avg_launch_ms": ca_ms,
-        },
+        "config": {"workload": w["workload"], "global_batch": w["n"], "kernel_ms_per_step": kernel_ms, **w["extra"]},
+        "roofline": roofline,
     }
-    if not args.no_cpu_baseline:
+    if args.workload == "c2" and not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
 

@@ -221,6 +221,15 @@ int dpk_add_noise(const void* summed, int in_dtype, void* grad, int out_dtype, i
                   float std, float denom, uint64_t seed, uint64_t offset, int draws,
                   dpk_stream_t stream);
 
+/* The same for up to DPK_MULTI_MAX parameters in one launch (the Python loop of
+ * optimizer.py:482-493 folded into the grid). Host arrays of K device pointers and
+ * sizes; all tensors share the dtypes. The tensors draw from ONE Philox stream laid
+ * end to end: element i of tensor k uses counter (sum_{j<k} ceil(P[j]/4) + i/4, offset).
+ * The call consumes `draws` units of offset in total. */
+int dpk_add_noise_multi(const void* const* summed /*host*/, void* const* grad /*host*/,
+                        const int64_t* P /*host*/, int64_t K, int in_dtype, int out_dtype, float std,
+                        float denom, uint64_t seed, uint64_t offset, int draws, dpk_stream_t stream);
+
 /* out[p] = std * z[p]: the bare generator, for statistical tests. */
 int dpk_fill_normal(float* out, int64_t P, float std, uint64_t seed, uint64_t offset,
                     dpk_stream_t stream);

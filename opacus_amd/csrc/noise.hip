@@ -112,6 +112,59 @@ void launch(const void* summed, void* grad, int64_t P, float std, float denom, u
                        offset, draws);
 }
 
+struct NoiseMulti {
+  const void* summed[DPK_MULTI_MAX];
+  void* grad[DPK_MULTI_MAX];
+  int64_t P[DPK_MULTI_MAX];
+  int64_t gprefix[DPK_MULTI_MAX + 1];  // 4-element groups before tensor k: block and counter base
+  int K;
+};
+
+// All parameters of an optimizer in one launch. Tensor k's element i uses Philox
+// group gprefix[k] + i / 4, i.e. the tensors draw from one stream laid end to end.
+// Blocks never straddle tensors (each tensor's groups are padded to whole blocks
+// in the grid, not in the counter space).
+template <typename TI, typename TO>
+__global__ __launch_bounds__(kThreads) void add_noise_multi_kernel(NoiseMulti a, float std, float denom,
+                                                                     uint64_t seed, uint64_t offset,
+                                                                     int draws) {
+  // Which tensor this block belongs to: tensor k owns ceil(groups_k / kThreads) blocks.
+  int k = 0;
+  int64_t b0 = 0;
+  for (;;) {
+    const int64_t nb = ((a.gprefix[k + 1] - a.gprefix[k]) + kThreads - 1) / kThreads;
+    if (static_cast<int64_t>(blockIdx.x) < b0 + nb || k + 1 >= a.K) break;
+    b0 += nb;
+    ++k;
+  }
+  const int64_t g = (static_cast<int64_t>(blockIdx.x) - b0) * kThreads + threadIdx.x;
+  const int64_t i = g * 4, P = a.P[k];
+  if (i >= P) return;
+  const TI* summed = static_cast<const TI*>(a.summed[k]);
+  TO* grad = static_cast<TO*>(a.grad[k]);
+  float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (std != 0.f) {
+    z = noise4(static_cast<uint64_t>(a.gprefix[k] + g), seed, offset, draws);
+    z.x *= std;
+    z.y *= std;
+    z.z *= std;
+    z.w *= std;
+  }
+  const bool vec = i + 4 <= P && ((reinterpret_cast<uintptr_t>(summed) | reinterpret_cast<uintptr_t>(grad)) & 15) == 0;
+  if (vec) {
+    float4 v = dpk_io<TI>::load4(summed + i);
+    v.x = (v.x + z.x) / denom;
+    v.y = (v.y + z.y) / denom;
+    v.z = (v.z + z.z) / denom;
+    v.w = (v.w + z.w) / denom;
+    dpk_io<TO>::store4(grad + i, v);
+  } else {
+    const float zz[4] = {z.x, z.y, z.z, z.w};
+    for (int e = 0; e < 4 && i + e < P; ++e)
+      dpk_io<TO>::store(grad + i + e, (dpk_io<TI>::load(summed + i + e) + zz[e]) / denom);
+  }
+}
+
 }  // namespace
 
 extern "C" int dpk_add_noise(const void* summed, int in_dtype, void* grad, int out_dtype, int64_t P,
@@ -154,6 +207,47 @@ extern "C" int dpk_fill_normal(float* out, int64_t P, float std, uint64_t seed, 
   DPK_REQUIRE(dpk_cdiv(dpk_cdiv(P, 4), kThreads) <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: P too large", who);
   launch<float, float>(nullptr, out, P, std, 1.0f, seed, offset, 1, dpk_aligned(out, 16),
                        static_cast<hipStream_t>(stream));
+  DPK_LAUNCH_CHECK(who);
+  return DPK_OK;
+}
+
+extern "C" int dpk_add_noise_multi(const void* const* summed, void* const* grad, const int64_t* P,
+                                   int64_t K, int in_dtype, int out_dtype, float std, float denom,
+                                   uint64_t seed, uint64_t offset, int draws, dpk_stream_t stream) {
+  const char* who = "dpk_add_noise_multi";
+  DPK_REQUIRE(summed && grad && P, DPK_E_ARG, "%s: NULL pointer table", who);
+  DPK_REQUIRE(K >= 1 && K <= DPK_MULTI_MAX, DPK_E_SHAPE, "%s: K=%lld not in [1,%d]", who, (long long)K,
+              DPK_MULTI_MAX);
+  DPK_REQUIRE(dpk_dtype_ok(in_dtype) && dpk_dtype_ok(out_dtype), DPK_E_DTYPE, "%s: dtypes %d,%d", who,
+              in_dtype, out_dtype);
+  DPK_REQUIRE(draws == 1 || draws == 4, DPK_E_ARG, "%s: draws=%d (1 or 4)", who, draws);
+  DPK_REQUIRE(std >= 0.f && denom != 0.f, DPK_E_ARG, "%s: std=%g denom=%g", who, (double)std, (double)denom);
+  NoiseMulti a;
+  a.K = static_cast<int>(K);
+  a.gprefix[0] = 0;
+  int64_t blocks = 0;
+  for (int k = 0; k < K; ++k) {
+    DPK_REQUIRE(P[k] >= 1, DPK_E_SHAPE, "%s: P[%d]=%lld", who, k, (long long)P[k]);
+    DPK_REQUIRE(summed[k] && grad[k], DPK_E_ARG, "%s: tensor %d is NULL", who, k);
+    DPK_REQUIRE(dpk_aligned(summed[k], dpk_elsize(in_dtype)) && dpk_aligned(grad[k], dpk_elsize(out_dtype)),
+                DPK_E_ALIGN, "%s: tensor %d misaligned", who, k);
+    a.summed[k] = summed[k];
+    a.grad[k] = grad[k];
+    a.P[k] = P[k];
+    const int64_t groups = dpk_cdiv(P[k], 4);
+    a.gprefix[k + 1] = a.gprefix[k] + groups;
+    blocks += dpk_cdiv(groups, kThreads);
+  }
+  DPK_REQUIRE(blocks <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: too many blocks", who);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
+#define DPK_NM(TI, TO) \
+  hipLaunchKernelGGL((add_noise_multi_kernel<TI, TO>), grid, block, 0, s, a, std, denom, seed, offset, draws)
+  if (in_dtype == DPK_F32 && out_dtype == DPK_F32) DPK_NM(float, float);
+  else if (in_dtype == DPK_F32 && out_dtype == DPK_BF16) DPK_NM(float, bf16_t);
+  else if (in_dtype == DPK_BF16 && out_dtype == DPK_F32) DPK_NM(bf16_t, float);
+  else DPK_NM(bf16_t, bf16_t);
+#undef DPK_NM
   DPK_LAUNCH_CHECK(who);
   return DPK_OK;
 }

@@ -517,6 +517,49 @@ def add_noise(
         )
 
 
+def add_noise_multi(
+    summed_list: Sequence[torch.Tensor],
+    grad_list: Sequence[torch.Tensor],
+    std: float,
+    denom: float,
+    seed: int,
+    offset: int,
+    draws: int = 1,
+) -> int:
+    """``grad_k = (summed_k + std * z) / denom`` for every k; one Philox stream laid across the
+    tensors in order, one launch per ``DPK_MULTI_MAX`` tensors. Returns the number of offset units
+    consumed (``draws`` per launch), by which the caller advances its generator."""
+    K = len(summed_list)
+    if K == 0:
+        return 0
+    dev = _need_gpu(*summed_list, *grad_list)
+    idt, odt = summed_list[0].dtype, grad_list[0].dtype
+    for s, g in zip(summed_list, grad_list):
+        if s.dtype != idt or g.dtype != odt:
+            raise ValueError("tensors of one add_noise_multi call must share dtypes")
+        if not s.is_contiguous() or not g.is_contiguous() or s.numel() != g.numel():
+            raise ValueError("summed and grad tensors must be dense and of equal size")
+    L = lib()
+    used = 0
+    for lo in range(0, K, DPK_MULTI_MAX):
+        ss, gg = summed_list[lo : lo + DPK_MULTI_MAX], grad_list[lo : lo + DPK_MULTI_MAX]
+        k = len(ss)
+        sptrs = (ctypes.c_void_p * k)(*[t.data_ptr() for t in ss])
+        gptrs = (ctypes.c_void_p * k)(*[t.data_ptr() for t in gg])
+        sizes = (ctypes.c_int64 * k)(*[t.numel() for t in ss])
+        with _timed("add_noise", dev):
+            check(
+                "dpk_add_noise_multi",
+                L.dpk_add_noise_multi(
+                    sptrs, gptrs, sizes, k, _code(idt), _code(odt), float(std), float(denom),
+                    seed & 0xFFFFFFFFFFFFFFFF, (offset + used) & 0xFFFFFFFFFFFFFFFF, draws,
+                    _stream(dev),
+                ),
+            )
+        used += draws
+    return used
+
+
 def fill_normal(out: torch.Tensor, std: float, seed: int, offset: int) -> None:
     dev = _need_gpu(out)
     if out.dtype != torch.float32 or not out.is_contiguous():

@@ -10,8 +10,8 @@ What changes is how many times the per-sample gradients cross HBM:
   * the clip factor is one tiny kernel;
   * ``sum_n clip[n] * gs[n]`` reads every per-sample gradient exactly once, all parameters
     of a dtype in one launch;
-  * noise, the add and the division by the batch size are one kernel per parameter that
-    draws Philox normals in registers, instead of zeros + normal + add + div.
+  * noise, the add and the division by the batch size are one kernel over all parameters
+    that draws Philox normals in registers, instead of zeros + normal + add + div each.
 """
 
 from __future__ import annotations
@@ -61,8 +61,9 @@ def _check_processed_flag(obj: Union[torch.Tensor, List[torch.Tensor]]):
             _check_processed_flag_tensor(x)
 
 
-def philox_stream(generator: Optional[torch.Generator], device: torch.device) -> Tuple[int, int]:
-    """``(seed, offset)`` for one noise kernel call, advancing the generator.
+def philox_stream(generator: Optional[torch.Generator], device: torch.device, calls: int = 1) -> Tuple[int, int]:
+    """``(seed, offset)`` for ``calls`` noise kernel launches (each may use up to four
+    consecutive offsets), advancing the generator.
 
     A generator on the GPU (the default one when ``generator`` is None) is used the way
     torch's own Philox kernels use it: its seed is the key and its offset moves on, so
@@ -75,7 +76,7 @@ def philox_stream(generator: Optional[torch.Generator], device: torch.device) ->
     if generator.device.type == "cuda":
         seed = generator.initial_seed()
         offset = generator.get_offset()
-        generator.set_offset(offset + _OFFSET_PER_CALL)
+        generator.set_offset(offset + _OFFSET_PER_CALL * calls)
         return seed, offset
     draws = torch.randint(0, 2**62, (2,), generator=generator, dtype=torch.int64)
     return int(draws[0]), int(draws[1]) * _OFFSET_PER_CALL
@@ -270,6 +271,9 @@ class DPOptimizer(Optimizer):
 
     def _add_noise_scaled(self, denom: float):
         std = self._noise_std()
+        draws = 4 if self.secure_mode else 1
+        # one launch per (device, dtype) group of parameters, all drawing from one stream
+        groups: Dict[tuple, Tuple[list, list]] = {}
         for p in self.params:
             _check_processed_flag(p.summed_grad)
             summed = p.summed_grad
@@ -277,14 +281,23 @@ class DPOptimizer(Optimizer):
                 raise TypeError(f"summed_grad must be float32 or bfloat16 on this path, got {summed.dtype}")
             if not summed.is_contiguous():
                 summed = summed.contiguous()
+            if summed.numel() == 0:
+                p.grad = torch.empty(p.shape, device=summed.device, dtype=summed.dtype)
+                _mark_as_processed(p.summed_grad)
+                continue
             grad = torch.empty(p.shape, device=summed.device, dtype=summed.dtype)
+            ss, gg = groups.setdefault((summed.device, summed.dtype), ([], []))
+            ss.append(summed)
+            gg.append(grad)
+            p.grad = grad
+            _mark_as_processed(p.summed_grad)
+        for (dev, _), (ss, gg) in groups.items():
+            launches = -(-len(ss) // kernels.DPK_MULTI_MAX)
             if std == 0:
                 seed = offset = 0  # nothing is drawn and the generator stays where it is
             else:
-                seed, offset = philox_stream(self.generator, summed.device)
-            kernels.add_noise(summed, grad, std, denom, seed, offset, draws=4 if self.secure_mode else 1)
-            p.grad = grad
-            _mark_as_processed(p.summed_grad)
+                seed, offset = philox_stream(self.generator, dev, calls=launches)
+            kernels.add_noise_multi(ss, gg, std, denom, seed, offset, draws=draws)
 
     def add_noise(self):
         """``p.grad = (p.summed_grad + N(0, std^2)).view_as(p)`` (optimizer.py:477-493)."""
@@ -303,8 +316,8 @@ class DPOptimizer(Optimizer):
                     p.grad /= denom
 
     def _noise_and_scale(self):
-        """``add_noise`` then ``scale_grad``; one kernel per parameter when neither method
-        has been overridden by a subclass."""
+        """``add_noise`` then ``scale_grad``; one kernel when neither method has been
+        overridden by a subclass."""
         cls = type(self)
         fused = cls.add_noise is DPOptimizer.add_noise and cls.scale_grad is DPOptimizer.scale_grad
         if fused:

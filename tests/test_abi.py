@@ -35,6 +35,7 @@ def test_header_declares_the_expected_surface():
         "dpk_clip_accumulate",
         "dpk_clip_accumulate_multi",
         "dpk_add_noise",
+        "dpk_add_noise_multi",
     ]:
         assert must in names
 

@@ -222,6 +222,40 @@ def test_add_noise_secure_draws_and_dtypes(K):
     assert abs(gb.double().std().item() - 1.0) < 1e-2
 
 
+def test_add_noise_multi_is_one_stream_laid_across_the_tensors(K):
+    """Tensor k's element i draws group (groups before k) + i // 4 of the restated stream; odd
+    sizes (scalar tails), a 1-element tensor and a misaligned view are in the mix."""
+    torch.manual_seed(11)
+    sizes = [1030, 1, 7, 4096, 513]
+    base = torch.randn(sum(sizes) + 64, device="cuda")
+    summed, lo = [], 0
+    for k, P in enumerate(sizes):
+        start = lo + (1 if k == 2 else 0)  # tensor 2 starts 4 bytes off a 16-byte boundary
+        summed.append(base[start : start + P])
+        lo += P + 8 - (P % 4)
+    grads = [torch.empty(P, device="cuda") for P in sizes]
+    used = K.add_noise_multi(summed, grads, std=1.5, denom=8.0, seed=77, offset=40, draws=1)
+    assert used == 1
+    total_groups = sum((P + 3) // 4 for P in sizes)
+    z = O.philox_normal(4 * total_groups, seed=77, offset=40)
+    g0 = 0
+    for P, s, g in zip(sizes, summed, grads):
+        want = (s.cpu().numpy() + np.float32(1.5) * z[4 * g0 : 4 * g0 + P]) / np.float32(8.0)
+        np.testing.assert_allclose(g.cpu().numpy(), want, rtol=0, atol=1e-5)
+        g0 += (P + 3) // 4
+    # more tensors than one launch holds: later launches move on by `draws` offsets
+    many = [torch.zeros(5, device="cuda") for _ in range(50)]
+    outs = [torch.empty(5, device="cuda") for _ in range(50)]
+    assert K.add_noise_multi(many, outs, std=1.0, denom=1.0, seed=1, offset=8, draws=1) == 2
+    z8, z9 = O.philox_normal(8 * 48, seed=1, offset=8), O.philox_normal(16, seed=1, offset=9)
+    np.testing.assert_allclose(outs[47].cpu().numpy(), z8[8 * 47 : 8 * 47 + 5], rtol=0, atol=2e-5)
+    np.testing.assert_allclose(outs[49].cpu().numpy(), z9[8:13], rtol=0, atol=2e-5)
+    # std == 0 is exact
+    K.add_noise_multi(summed, grads, std=0.0, denom=1.0, seed=0, offset=0)
+    for s, g in zip(summed, grads):
+        assert torch.equal(s, g)
+
+
 # ---- Linear ghost norms --------------------------------------------------------------
 GHOST_SHAPES = [
     # (n, T, in, out)
