@@ -273,6 +273,17 @@ extern "C" int dpk_linear_gs(const void* b, const void* a, int in_dtype, void* g
     partials = static_cast<float*>(ws);
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (sumsq && p.outer) {
+    // Ahead of the store-bound kernel: the operands are still warm from the backward
+    // pass, and the pass leaves them in the cache for the kernel that follows.
+    if (in_dtype == DPK_F32)
+      hipLaunchKernelGGL(rank1_sumsq_kernel<float>, dim3(static_cast<unsigned>(n)), dim3(kThreads), 0, s,
+                         static_cast<const float*>(b), static_cast<const float*>(a), sumsq, out, in, scale);
+    else
+      hipLaunchKernelGGL(rank1_sumsq_kernel<bf16_t>, dim3(static_cast<unsigned>(n)), dim3(kThreads), 0, s,
+                         static_cast<const bf16_t*>(b), static_cast<const bf16_t*>(a), sumsq, out, in, scale);
+    DPK_LAUNCH_CHECK(who);
+  }
   if (in_dtype == DPK_F32 && gs_dtype == DPK_F32)
     launch_linear<float, float>(p, vec, b, a, gs, partials, n, T, out, in, scale, s);
   else if (in_dtype == DPK_BF16 && gs_dtype == DPK_BF16)
@@ -282,15 +293,7 @@ extern "C" int dpk_linear_gs(const void* b, const void* a, int in_dtype, void* g
   else
     launch_linear<float, bf16_t>(p, vec, b, a, gs, partials, n, T, out, in, scale, s);
   DPK_LAUNCH_CHECK(who);
-  if (sumsq && p.outer) {
-    if (in_dtype == DPK_F32)
-      hipLaunchKernelGGL(rank1_sumsq_kernel<float>, dim3(static_cast<unsigned>(n)), dim3(kThreads), 0, s,
-                         static_cast<const float*>(b), static_cast<const float*>(a), sumsq, out, in, scale);
-    else
-      hipLaunchKernelGGL(rank1_sumsq_kernel<bf16_t>, dim3(static_cast<unsigned>(n)), dim3(kThreads), 0, s,
-                         static_cast<const bf16_t*>(b), static_cast<const bf16_t*>(a), sumsq, out, in, scale);
-    DPK_LAUNCH_CHECK(who);
-  } else if (sumsq) {
+  if (sumsq && !p.outer) {
     dpk_launch_reduce_rows(partials, n, p.tiles_m * p.tiles_n, sumsq, 0, 1.f, s);
     DPK_LAUNCH_CHECK(who);
   }

@@ -1,7 +1,8 @@
 // DPOptimizer.add_noise + scale_grad (opacus/optimizers/optimizer.py:477-504)
 // with _generate_noise (optimizer.py:104-169) folded in: one pass that reads
 // summed_grad, draws Gaussian noise from a counter-based generator in registers,
-// adds, divides and writes grad. HBM-bound: 2 * P * elsize bytes.
+// adds, divides and writes grad: 2 * P * elsize bytes of HBM traffic, against about a
+// hundred ALU instructions per four elements for the generator.
 //
 // Generator: Philox4x32-10 (Salmon et al., SC'11), key = seed, counter =
 // (group index lo, hi, offset lo, hi) where a group is 4 consecutive elements.
@@ -37,12 +38,15 @@ __device__ __forceinline__ float4 normal4(uint64_t group, uint64_t seed, uint64_
       make_uint4(static_cast<uint32_t>(group), static_cast<uint32_t>(group >> 32),
                  static_cast<uint32_t>(offset), static_cast<uint32_t>(offset >> 32)),
       make_uint2(static_cast<uint32_t>(seed), static_cast<uint32_t>(seed >> 32)));
-  const float r0 = sqrtf(-2.0f * logf(u01(r.x)));
-  const float r1 = sqrtf(-2.0f * logf(u01(r.z)));
-  float s0, c0, s1, c1;
-  sincosf(6.2831853071795865f * u01(r.y), &s0, &c0);
-  sincosf(6.2831853071795865f * u01(r.w), &s1, &c1);
-  return make_float4(r0 * c0, r0 * s0, r1 * c1, r1 * s1);
+  // Box-Muller on the hardware transcendentals: v_log_f32 is log2, v_sin/v_cos take
+  // their argument in revolutions, so cos(2 pi u) is one instruction. The kernel is
+  // otherwise bound by these, not by memory.
+  constexpr float kNeg2Ln2 = -1.3862943611198906f;
+  const float r0 = __builtin_amdgcn_sqrtf(kNeg2Ln2 * __builtin_amdgcn_logf(u01(r.x)));
+  const float r1 = __builtin_amdgcn_sqrtf(kNeg2Ln2 * __builtin_amdgcn_logf(u01(r.z)));
+  const float t0 = u01(r.y), t1 = u01(r.w);
+  return make_float4(r0 * __builtin_amdgcn_cosf(t0), r0 * __builtin_amdgcn_sinf(t0),
+                     r1 * __builtin_amdgcn_cosf(t1), r1 * __builtin_amdgcn_sinf(t1));
 }
 
 __device__ __forceinline__ float4 noise4(uint64_t group, uint64_t seed, uint64_t offset, int draws) {
@@ -65,104 +69,99 @@ __device__ __forceinline__ float4 noise4(uint64_t group, uint64_t seed, uint64_t
   return z;
 }
 
-template <typename TI, typename TO, bool VEC>
-__global__ __launch_bounds__(kThreads) void add_noise_kernel(const TI* __restrict__ summed,
-                                                               TO* __restrict__ grad, int64_t P,
-                                                               float std, float denom,
+// A block covers kGroupsPerBlock consecutive 4-element groups of one tensor, thread t
+// taking groups t, t + 256, ... so that a wave's accesses stay contiguous.
+constexpr int kUnroll = 4;
+constexpr int kGroupsPerBlock = kThreads * kUnroll;
+
+struct NoiseArgs {
+  const void* summed[DPK_MULTI_MAX];  // NULL: the tensor counts as zeros
+  void* grad[DPK_MULTI_MAX];
+  int64_t P[DPK_MULTI_MAX];
+  int64_t gprefix[DPK_MULTI_MAX + 1];   // groups before tensor k: its base in the counter space
+  uint32_t bprefix[DPK_MULTI_MAX + 1];  // blocks before tensor k
+  int K;
+};
+
+// Tensor k's element i uses Philox group gprefix[k] + i / 4: the tensors draw from one
+// stream laid end to end, whatever the launch shape. Blocks never straddle tensors.
+template <typename TI, typename TO>
+__global__ __launch_bounds__(kThreads) void add_noise_kernel(NoiseArgs a, float std, float denom,
                                                                uint64_t seed, uint64_t offset,
                                                                int draws) {
-  const int64_t g = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  const int64_t i = g * 4;
-  if (i >= P) return;
-  float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
-  if (std != 0.f) {
-    z = noise4(static_cast<uint64_t>(g), seed, offset, draws);
-    z.x *= std;
-    z.y *= std;
-    z.z *= std;
-    z.w *= std;
+  // the tensor this block belongs to: last k with bprefix[k] <= blockIdx.x (uniform, scalar)
+  int lo = 0, hi = a.K - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (a.bprefix[mid] <= blockIdx.x) lo = mid;
+    else hi = mid - 1;
   }
-  if (VEC && i + 4 <= P) {
-    float4 v = summed ? dpk_io<TI>::load4(summed + i) : make_float4(0.f, 0.f, 0.f, 0.f);
-    v.x = (v.x + z.x) / denom;
-    v.y = (v.y + z.y) / denom;
-    v.z = (v.z + z.z) / denom;
-    v.w = (v.w + z.w) / denom;
-    dpk_io<TO>::store4(grad + i, v);
-  } else {
-    const float zz[4] = {z.x, z.y, z.z, z.w};
-    for (int e = 0; e < 4 && i + e < P; ++e) {
-      const float v = summed ? dpk_io<TI>::load(summed + i + e) : 0.f;
-      dpk_io<TO>::store(grad + i + e, (v + zz[e]) / denom);
+  const int k = lo;
+  const int64_t P = a.P[k];
+  const TI* summed = static_cast<const TI*>(a.summed[k]);
+  TO* grad = static_cast<TO*>(a.grad[k]);
+  const uint64_t gbase = static_cast<uint64_t>(a.gprefix[k]);
+  const bool aligned =
+      ((reinterpret_cast<uintptr_t>(summed) | reinterpret_cast<uintptr_t>(grad)) & 15) == 0;
+  const float inv = 1.0f / denom;
+  const bool exact_div = std == 0.f;  // a pure rescale stays a correctly rounded division
+  const int64_t g0 = static_cast<int64_t>(blockIdx.x - a.bprefix[k]) * kGroupsPerBlock + threadIdx.x;
+#pragma unroll
+  for (int u = 0; u < kUnroll; ++u) {
+    const int64_t g = g0 + u * kThreads;
+    const int64_t i = g * 4;
+    if (i >= P) break;
+    float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (std != 0.f) {
+      z = noise4(gbase + static_cast<uint64_t>(g), seed, offset, draws);
+      z.x *= std;
+      z.y *= std;
+      z.z *= std;
+      z.w *= std;
+    }
+    if (aligned && i + 4 <= P) {
+      float4 v = summed ? dpk_io<TI>::load4(summed + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+      if (exact_div) {
+        v = make_float4(v.x / denom, v.y / denom, v.z / denom, v.w / denom);
+      } else {
+        v = make_float4((v.x + z.x) * inv, (v.y + z.y) * inv, (v.z + z.z) * inv, (v.w + z.w) * inv);
+      }
+      dpk_io<TO>::store4(grad + i, v);
+    } else {
+      const float zz[4] = {z.x, z.y, z.z, z.w};
+      for (int e = 0; e < 4 && i + e < P; ++e) {
+        const float v = summed ? dpk_io<TI>::load(summed + i + e) : 0.f;
+        dpk_io<TO>::store(grad + i + e, exact_div ? v / denom : (v + zz[e]) * inv);
+      }
     }
   }
 }
 
-template <typename TI, typename TO>
-void launch(const void* summed, void* grad, int64_t P, float std, float denom, uint64_t seed,
-            uint64_t offset, int draws, bool vec, hipStream_t s) {
-  const unsigned blocks = static_cast<unsigned>(dpk_cdiv(dpk_cdiv(P, 4), kThreads));
-  if (vec)
-    hipLaunchKernelGGL((add_noise_kernel<TI, TO, true>), dim3(blocks), dim3(kThreads), 0, s,
-                       static_cast<const TI*>(summed), static_cast<TO*>(grad), P, std, denom, seed,
-                       offset, draws);
-  else
-    hipLaunchKernelGGL((add_noise_kernel<TI, TO, false>), dim3(blocks), dim3(kThreads), 0, s,
-                       static_cast<const TI*>(summed), static_cast<TO*>(grad), P, std, denom, seed,
-                       offset, draws);
+int launch(const char* who, const NoiseArgs& a, unsigned blocks, int in_dtype, int out_dtype, float std,
+           float denom, uint64_t seed, uint64_t offset, int draws, hipStream_t s) {
+  const dim3 grid(blocks), block(kThreads);
+#define DPK_NM(TI, TO) \
+  hipLaunchKernelGGL((add_noise_kernel<TI, TO>), grid, block, 0, s, a, std, denom, seed, offset, draws)
+  if (in_dtype == DPK_F32 && out_dtype == DPK_F32) DPK_NM(float, float);
+  else if (in_dtype == DPK_F32 && out_dtype == DPK_BF16) DPK_NM(float, bf16_t);
+  else if (in_dtype == DPK_BF16 && out_dtype == DPK_F32) DPK_NM(bf16_t, float);
+  else DPK_NM(bf16_t, bf16_t);
+#undef DPK_NM
+  DPK_LAUNCH_CHECK(who);
+  return DPK_OK;
 }
 
-struct NoiseMulti {
-  const void* summed[DPK_MULTI_MAX];
-  void* grad[DPK_MULTI_MAX];
-  int64_t P[DPK_MULTI_MAX];
-  int64_t gprefix[DPK_MULTI_MAX + 1];  // 4-element groups before tensor k: block and counter base
-  int K;
-};
-
-// All parameters of an optimizer in one launch. Tensor k's element i uses Philox
-// group gprefix[k] + i / 4, i.e. the tensors draw from one stream laid end to end.
-// Blocks never straddle tensors (each tensor's groups are padded to whole blocks
-// in the grid, not in the counter space).
-template <typename TI, typename TO>
-__global__ __launch_bounds__(kThreads) void add_noise_multi_kernel(NoiseMulti a, float std, float denom,
-                                                                     uint64_t seed, uint64_t offset,
-                                                                     int draws) {
-  // Which tensor this block belongs to: tensor k owns ceil(groups_k / kThreads) blocks.
-  int k = 0;
-  int64_t b0 = 0;
-  for (;;) {
-    const int64_t nb = ((a.gprefix[k + 1] - a.gprefix[k]) + kThreads - 1) / kThreads;
-    if (static_cast<int64_t>(blockIdx.x) < b0 + nb || k + 1 >= a.K) break;
-    b0 += nb;
-    ++k;
-  }
-  const int64_t g = (static_cast<int64_t>(blockIdx.x) - b0) * kThreads + threadIdx.x;
-  const int64_t i = g * 4, P = a.P[k];
-  if (i >= P) return;
-  const TI* summed = static_cast<const TI*>(a.summed[k]);
-  TO* grad = static_cast<TO*>(a.grad[k]);
-  float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
-  if (std != 0.f) {
-    z = noise4(static_cast<uint64_t>(a.gprefix[k] + g), seed, offset, draws);
-    z.x *= std;
-    z.y *= std;
-    z.z *= std;
-    z.w *= std;
-  }
-  const bool vec = i + 4 <= P && ((reinterpret_cast<uintptr_t>(summed) | reinterpret_cast<uintptr_t>(grad)) & 15) == 0;
-  if (vec) {
-    float4 v = dpk_io<TI>::load4(summed + i);
-    v.x = (v.x + z.x) / denom;
-    v.y = (v.y + z.y) / denom;
-    v.z = (v.z + z.z) / denom;
-    v.w = (v.w + z.w) / denom;
-    dpk_io<TO>::store4(grad + i, v);
-  } else {
-    const float zz[4] = {z.x, z.y, z.z, z.w};
-    for (int e = 0; e < 4 && i + e < P; ++e)
-      dpk_io<TO>::store(grad + i + e, (dpk_io<TI>::load(summed + i + e) + zz[e]) / denom);
-  }
+// Fills slot k; returns false when the block count would overflow the grid.
+bool add_tensor(NoiseArgs& a, int k, const void* summed, void* grad, int64_t P) {
+  a.summed[k] = summed;
+  a.grad[k] = grad;
+  a.P[k] = P;
+  const int64_t groups = dpk_cdiv(P, 4);
+  a.gprefix[k + 1] = a.gprefix[k] + groups;
+  const int64_t nb = static_cast<int64_t>(a.bprefix[k]) + dpk_cdiv(groups, kGroupsPerBlock);
+  if (nb > DPK_MAX_GRID_X) return false;
+  a.bprefix[k + 1] = static_cast<uint32_t>(nb);
+  return true;
 }
 
 }  // namespace
@@ -181,20 +180,13 @@ extern "C" int dpk_add_noise(const void* summed, int in_dtype, void* grad, int o
               (double)denom);
   DPK_REQUIRE(dpk_aligned(summed, dpk_elsize(in_dtype)) && dpk_aligned(grad, dpk_elsize(out_dtype)),
               DPK_E_ALIGN, "%s: misaligned tensor", who);
-  DPK_REQUIRE(dpk_cdiv(dpk_cdiv(P, 4), kThreads) <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: P too large", who);
-  const bool vec = dpk_aligned(summed, in_dtype == DPK_BF16 ? 8 : 16) &&
-                   dpk_aligned(grad, out_dtype == DPK_BF16 ? 8 : 16);
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  if (in_dtype == DPK_F32 && out_dtype == DPK_F32)
-    launch<float, float>(summed, grad, P, std, denom, seed, offset, draws, vec, s);
-  else if (in_dtype == DPK_F32 && out_dtype == DPK_BF16)
-    launch<float, bf16_t>(summed, grad, P, std, denom, seed, offset, draws, vec, s);
-  else if (in_dtype == DPK_BF16 && out_dtype == DPK_F32)
-    launch<bf16_t, float>(summed, grad, P, std, denom, seed, offset, draws, vec, s);
-  else
-    launch<bf16_t, bf16_t>(summed, grad, P, std, denom, seed, offset, draws, vec, s);
-  DPK_LAUNCH_CHECK(who);
-  return DPK_OK;
+  NoiseArgs a;
+  a.K = 1;
+  a.gprefix[0] = 0;
+  a.bprefix[0] = 0;
+  DPK_REQUIRE(add_tensor(a, 0, summed, grad, P), DPK_E_SHAPE, "%s: P too large", who);
+  return launch(who, a, a.bprefix[1], in_dtype, out_dtype, std, denom, seed, offset, draws,
+                static_cast<hipStream_t>(stream));
 }
 
 extern "C" int dpk_fill_normal(float* out, int64_t P, float std, uint64_t seed, uint64_t offset,
@@ -203,12 +195,15 @@ extern "C" int dpk_fill_normal(float* out, int64_t P, float std, uint64_t seed, 
   DPK_REQUIRE(P >= 0, DPK_E_SHAPE, "%s: P=%lld", who, (long long)P);
   if (P == 0) return DPK_OK;
   DPK_REQUIRE(out, DPK_E_ARG, "%s: NULL tensor", who);
+  DPK_REQUIRE(std >= 0.f, DPK_E_ARG, "%s: std=%g", who, (double)std);
   DPK_REQUIRE(dpk_aligned(out, 4), DPK_E_ALIGN, "%s: misaligned tensor", who);
-  DPK_REQUIRE(dpk_cdiv(dpk_cdiv(P, 4), kThreads) <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: P too large", who);
-  launch<float, float>(nullptr, out, P, std, 1.0f, seed, offset, 1, dpk_aligned(out, 16),
-                       static_cast<hipStream_t>(stream));
-  DPK_LAUNCH_CHECK(who);
-  return DPK_OK;
+  NoiseArgs a;
+  a.K = 1;
+  a.gprefix[0] = 0;
+  a.bprefix[0] = 0;
+  DPK_REQUIRE(add_tensor(a, 0, nullptr, out, P), DPK_E_SHAPE, "%s: P too large", who);
+  return launch(who, a, a.bprefix[1], DPK_F32, DPK_F32, std, 1.0f, seed, offset, 1,
+                static_cast<hipStream_t>(stream));
 }
 
 extern "C" int dpk_add_noise_multi(const void* const* summed, void* const* grad, const int64_t* P,
@@ -222,32 +217,17 @@ extern "C" int dpk_add_noise_multi(const void* const* summed, void* const* grad,
               in_dtype, out_dtype);
   DPK_REQUIRE(draws == 1 || draws == 4, DPK_E_ARG, "%s: draws=%d (1 or 4)", who, draws);
   DPK_REQUIRE(std >= 0.f && denom != 0.f, DPK_E_ARG, "%s: std=%g denom=%g", who, (double)std, (double)denom);
-  NoiseMulti a;
+  NoiseArgs a;
   a.K = static_cast<int>(K);
   a.gprefix[0] = 0;
-  int64_t blocks = 0;
+  a.bprefix[0] = 0;
   for (int k = 0; k < K; ++k) {
     DPK_REQUIRE(P[k] >= 1, DPK_E_SHAPE, "%s: P[%d]=%lld", who, k, (long long)P[k]);
     DPK_REQUIRE(summed[k] && grad[k], DPK_E_ARG, "%s: tensor %d is NULL", who, k);
     DPK_REQUIRE(dpk_aligned(summed[k], dpk_elsize(in_dtype)) && dpk_aligned(grad[k], dpk_elsize(out_dtype)),
                 DPK_E_ALIGN, "%s: tensor %d misaligned", who, k);
-    a.summed[k] = summed[k];
-    a.grad[k] = grad[k];
-    a.P[k] = P[k];
-    const int64_t groups = dpk_cdiv(P[k], 4);
-    a.gprefix[k + 1] = a.gprefix[k] + groups;
-    blocks += dpk_cdiv(groups, kThreads);
+    DPK_REQUIRE(add_tensor(a, k, summed[k], grad[k], P[k]), DPK_E_SHAPE, "%s: too many blocks", who);
   }
-  DPK_REQUIRE(blocks <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: too many blocks", who);
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  const dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
-#define DPK_NM(TI, TO) \
-  hipLaunchKernelGGL((add_noise_multi_kernel<TI, TO>), grid, block, 0, s, a, std, denom, seed, offset, draws)
-  if (in_dtype == DPK_F32 && out_dtype == DPK_F32) DPK_NM(float, float);
-  else if (in_dtype == DPK_F32 && out_dtype == DPK_BF16) DPK_NM(float, bf16_t);
-  else if (in_dtype == DPK_BF16 && out_dtype == DPK_F32) DPK_NM(bf16_t, float);
-  else DPK_NM(bf16_t, bf16_t);
-#undef DPK_NM
-  DPK_LAUNCH_CHECK(who);
-  return DPK_OK;
+  return launch(who, a, a.bprefix[K], in_dtype, out_dtype, std, denom, seed, offset, draws,
+                static_cast<hipStream_t>(stream));
 }
