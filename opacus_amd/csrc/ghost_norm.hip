@@ -263,8 +263,10 @@ extern "C" int dpk_linear_ghost_norm(const void* b, const void* a, int dtype, fl
   const int B = tile_edge(T);
   const int64_t nt = dpk_cdiv(T, B);
   // bf16 with 64-aligned feature sizes takes the direct-to-LDS kernel
+  // (and a sample small enough for 32-bit byte offsets inside it)
+  const int64_t widest = out > in ? out : in;
   const bool dlds = dtype == DPK_BF16 && B == 128 && out % 64 == 0 && (in % 64 == 0 || !norm_w) &&
-                    dpk_aligned(b, 16) && dpk_aligned(a, 16);
+                    dpk_aligned(b, 16) && dpk_aligned(a, 16) && T * widest * 2 < (int64_t{1} << 32);
   const int64_t npairs = dlds ? ghost_pairs(T, GhostCfg::BM, GhostCfg::BN) : nt * (nt + 1) / 2;
   const int64_t blocks = n * npairs;
   DPK_REQUIRE(nt < 32768 && blocks <= DPK_MAX_GRID_X, DPK_E_SHAPE,

@@ -81,26 +81,39 @@ __device__ __forceinline__ uint32_t lds_offset(const void* p) {
   return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lptr_t)p));
 }
 
-// issue_one: the r-th global->LDS load of a tile (rows m0.., k offset k0) whose
-// LDS image starts at byte offset `dst`; issue_tile: all NLOADS of them.
+// The same with the address split into a wave-uniform base (scalar registers) and a
+// 32-bit per-lane byte offset: the per-lane part of a tile's addresses never changes
+// along k, so the main loop computes it once and only moves the scalar base.
+__device__ __forceinline__ void load16_to_lds(const void* sbase, uint32_t voff, uint32_t lds_base) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, %2\n\t"
+      :
+      : "s"(lds_base), "v"(voff), "s"(sbase)
+      : "memory", "m0");
+}
+
+// The r-th global->LDS load of a tile covers 1 KB of consecutive tile rows per wave:
+// group r * kWaves + wave. lane_offset: this lane's byte offset from the matrix base
+// for that load (rows >= M read row M - 1 instead); group_lds: where the group lands
+// in the tile's LDS image.
 template <class C>
-__device__ __forceinline__ void issue_one(const bf16_t* base, int64_t ld, int64_t m0, int64_t M,
-                                          int64_t k0, uint32_t dst, int r) {
+__device__ __forceinline__ uint32_t lane_offset(int64_t ld, int64_t m0, int64_t M, int r) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int grp = r * C::kWaves + wave;  // 1 KB of consecutive rows per wave instruction
+  const int grp = r * C::kWaves + wave;
   const int row = grp * C::kRowsPerKB + lane / C::kChunks;
   const int lc = swz<C>(row, lane % C::kChunks);  // which logical chunk lives at this physical slot
   int64_t m = m0 + row;
   m = m < M ? m : M - 1;
-  load16_to_lds(base + m * ld + k0 + lc * 8, dst + grp * 1024);
+  return static_cast<uint32_t>((m * ld + lc * 8) * 2);
 }
 
-template <class C, int NLOADS>
-__device__ __forceinline__ void issue_tile(const bf16_t* base, int64_t ld, int64_t m0, int64_t M,
-                                           int64_t k0, uint32_t dst) {
-#pragma unroll
-  for (int r = 0; r < NLOADS; ++r) issue_one<C>(base, ld, m0, M, k0, dst, r);
+template <class C>
+__device__ __forceinline__ uint32_t group_lds(int r) {
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  return static_cast<uint32_t>((r * C::kWaves + wave) * 1024);
 }
 
 // Waits until at most N of this wave's loads are outstanding, then meets the
@@ -163,7 +176,11 @@ struct Tile {
     __builtin_amdgcn_sched_barrier(0);  // keep the reads ahead of the MFMAs
     // MFMAs execute asynchronously: the global->LDS loads of the tile after next
     // (and their address arithmetic) are issued in their shadow, a few per step.
+#ifdef DPK_DLDS_PER_STEP
+    constexpr int PER_STEP = DPK_DLDS_PER_STEP;
+#else
     constexpr int PER_STEP = (NLOADS + KS - 1) / KS;
+#endif
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
@@ -182,7 +199,8 @@ struct Tile {
 // issues exactly one tile's worth of loads (past the end the last tile is
 // fetched again into a stage nobody reads), so the number of loads that may
 // stay outstanding while tile kt is awaited is the constant
-// kLoadsPerTile * (NS - 2).
+// kLoadsPerTile * (NS - 2). abase / bbase must be wave-uniform and every byte
+// offset inside the matrices must fit 32 bits (M * ld * 2 < 2^32).
 template <class C>
 __device__ __forceinline__ void mainloop(Tile& t, Smem<C>& sm, const bf16_t* abase,
                                          const bf16_t* bbase, int64_t ld, int64_t m0a, int64_t m0b,
@@ -191,14 +209,25 @@ __device__ __forceinline__ void mainloop(Tile& t, Smem<C>& sm, const bf16_t* aba
   constexpr int BK = C::BK, ROW_BYTES = C::ROW_BYTES;
   const int64_t nk = K / BK;
   const uint32_t lds0 = lds_offset(&sm.stage[0][0]);
-  auto issue = [&](int64_t kt, int stage) {
-    const int64_t kc = kt < nk ? kt : nk - 1;
-    const uint32_t st = lds0 + stage * C::kStageBytes;
-    issue_tile<C, C::kLoadsA>(abase, ld, m0a, M, kc * BK, st);
-    issue_tile<C, C::kLoadsB>(bbase, ld, m0b, M, kc * BK, st + C::BM * ROW_BYTES);
+  // Per-lane offsets of the tile's loads, fixed for the whole k loop. The empty asm
+  // makes them opaque values: recomputing them per load (a 64-bit multiply and a
+  // clamp each) would cost more vector instructions than the MFMAs they feed.
+  uint32_t off[C::kLoadsPerTile];
+#pragma unroll
+  for (int q = 0; q < C::kLoadsPerTile; ++q) {
+    off[q] = q < C::kLoadsA ? lane_offset<C>(ld, m0a, M, q) : lane_offset<C>(ld, m0b, M, q - C::kLoadsA);
+    asm volatile("" : "+v"(off[q]));
+  }
+  auto issue_q = [&](int64_t kt, uint32_t st, int q) {
+    if (q < C::kLoadsA) load16_to_lds(abase + kt * BK, off[q], st + group_lds<C>(q));
+    else load16_to_lds(bbase + kt * BK, off[q], st + C::BM * ROW_BYTES + group_lds<C>(q - C::kLoadsA));
   };
 #pragma unroll
-  for (int s = 0; s < NS - 1; ++s) issue(s, s);
+  for (int s = 0; s < NS - 1; ++s) {
+    const int64_t kc = s < nk ? s : nk - 1;
+#pragma unroll
+    for (int q = 0; q < C::kLoadsPerTile; ++q) issue_q(kc, lds0 + s * C::kStageBytes, q);
+  }
   int stage = 0;  // stage of tile kt
   for (int64_t kt = 0; kt < nk; ++kt) {
     // tile kt has landed for every wave, and the stage of tile kt - 1 is free again
@@ -206,10 +235,8 @@ __device__ __forceinline__ void mainloop(Tile& t, Smem<C>& sm, const bf16_t* aba
     const int64_t kn = kt + NS - 1 < nk ? kt + NS - 1 : nk - 1;
     const uint32_t dst = lds0 + (stage == 0 ? NS - 1 : stage - 1) * C::kStageBytes;
     const unsigned char* st = sm.stage[stage];
-    t.template mma<C, C::kLoadsPerTile>(st, st + C::BM * ROW_BYTES, wm0, wn0, [&](int q) {
-      if (q < C::kLoadsA) issue_one<C>(abase, ld, m0a, M, kn * BK, dst, q);
-      else issue_one<C>(bbase, ld, m0b, M, kn * BK, dst + C::BM * ROW_BYTES, q - C::kLoadsA);
-    });
+    t.template mma<C, C::kLoadsPerTile>(st, st + C::BM * ROW_BYTES, wm0, wn0,
+                                        [&](int q) { issue_q(kn, dst, q); });
     stage = stage + 1 == NS ? 0 : stage + 1;
   }
   wait_and_barrier<0>();  // the ring may be reused by the caller's next main loop
