@@ -14,7 +14,8 @@ same workload.
 
 The other four benchmark configurations can be timed with ``--workload c1|c3|c4|c5``
 (same JSON shape, no CPU baseline); they are parity-test shapes first and bench lines
-second.
+second. ``--kernels`` times each kernel of the library on its own at those shapes and
+prints one JSON line per kernel (time, algorithmic work, fraction of its roofline).
 """
 
 from __future__ import annotations
@@ -332,6 +333,112 @@ def cpu_baseline(n_sample: int = 16, steps: int = 3) -> dict:
     }
 
 
+def kernel_table(dev, iters: int = 10, warm: int = 3):
+    """Every kernel of the library on its own at the benchmark configurations' shapes: yields one
+    dict per kernel with its time (HIP events on the launch stream) against the roofline that
+    bounds it. Work figures are algorithmic: bytes that must cross HBM once, or executed MFMA
+    FLOPs (the ghost-norm kernels visit the block-triangle of the T x T Gram)."""
+    from opacus_amd import kernels as K
+
+    def timed(fn):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(iters):
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        return s.elapsed_time(e) / iters
+
+    def row(name, ref_row, shape, ms, bound, work):
+        peak, unit, scale = {
+            "hbm": (HBM_PEAK_GBS, "GB/s", 1e9),
+            "mfma_bf16": (MFMA_BF16_PEAK_TFLOPS, "TFLOP/s", 1e12),
+            "mfma_fp32": (MFMA_FP32_PEAK_TFLOPS, "TFLOP/s", 1e12),
+        }[bound]
+        ach = work / (ms * 1e-3) / scale
+        return {"kernel": name, "row": ref_row, "shape": shape, "ms": ms, "bound": bound, "achieved": ach,
+                "peak": peak, "unit": unit, "frac": ach / peak, "algorithmic_work": work}
+
+    def tri_tiles(T, tile=128):
+        nt = -(-T // tile)
+        return nt * (nt + 1) // 2, nt * nt
+
+    torch.manual_seed(0)
+    # ---- C2: Linear 4096x4096 fp32, batch 128, T = 1
+    n, d = 128, 4096
+    a, b = torch.randn(n, d, device=dev), torch.randn(n, d, device=dev)
+    gs, ss = K.linear_grad_sample(b, a)
+    yield row("linear_gs (T=1 outer product)", "a1", "C2 n=128 4096x4096 f32", timed(lambda: K.linear_grad_sample(b, a)),
+              "hbm", gs.numel() * 4 + 2 * n * d * 4)
+    yield row("sumsq_rows", "a10", "C2 n=128 P=16.8M f32", timed(lambda: K.sumsq_rows([gs])), "hbm", gs.numel() * 4)
+    _, clip = K.clip_factor(ss.reshape(1, -1), 1.0)
+    out = torch.empty(d, d, device=dev)
+    yield row("clip_accumulate", "a10", "C2 n=128 P=16.8M f32", timed(lambda: K.clip_accumulate([gs], clip, [out], False)),
+              "hbm", gs.numel() * 4 + out.numel() * 4)
+    g = torch.empty_like(out)
+    yield row("add_noise", "a11", "C2 P=16.8M f32", timed(lambda: K.add_noise(out, g, 1.0, 128.0, 1, 0)), "hbm", 2 * out.numel() * 4)
+    yield row("linear_bias_gs", "a1", "C2 n=128 out=4096 f32", timed(lambda: K.linear_bias_grad_sample(b)), "hbm", 2 * n * d * 4)
+    del gs, out, g
+    # ---- Linear per-sample gradients with a sequence dimension (fp32 MFMA)
+    n, T, i, o = 16, 256, 1024, 1024
+    a, b = torch.randn(n, T, i, device=dev), torch.randn(n, T, o, device=dev)
+    yield row("linear_gs (T>1, fp32 MFMA)", "a1", "n=16 T=256 1024x1024 f32", timed(lambda: K.linear_grad_sample(b, a)),
+              "mfma_fp32", 2.0 * n * T * i * o)
+    # ---- C3 / C5: ghost norms, bf16
+    for cfg, n, T, layers in (
+        ("C3", 32, 512, [(1024, 4096, "fc1"), (4096, 1024, "fc2")]),
+        ("C5", 16, 1024, [(2048, 2048, "q/o"), (2048, 512, "k/v"), (2048, 5632, "gate/up"), (5632, 2048, "down"),
+                          (2048, 32000, "lm_head")]),
+    ):
+        tri, full = tri_tiles(T)
+        for i, o, name in layers:
+            a = torch.randn(n, T, i, device=dev).bfloat16()
+            b = (torch.randn(n, T, o, device=dev) * 0.02).bfloat16()
+            ms = timed(lambda: K.linear_ghost_norm(b, a, want_weight=True, want_bias=False))
+            yield row("linear_ghost_norm", "a2", f"{cfg} {name} n={n} T={T} {i}->{o} bf16", ms, "mfma_bf16",
+                      2.0 * n * T * T * (i + o) * tri / full)
+            del a, b
+    # ---- C5: embedding ghost norm, RMSNorm, noise over all parameters (bf16)
+    n, T, D, V = 16, 1024, 2048, 32000
+    ids = torch.randint(0, V, (n, T), device=dev)
+    b = (torch.randn(n, T, D, device=dev) * 0.02).bfloat16()
+    x = torch.randn(n, T, D, device=dev).bfloat16()
+    yield row("embedding_ghost_norm", "a5", "C5 n=16 T=1024 D=2048 bf16", timed(lambda: K.embedding_ghost_norm(ids, b)),
+              "hbm", b.numel() * 2 + ids.numel() * 8)
+    yield row("rms_norm_gs", "a6", "C5 n=16 T=1024 D=2048 bf16", timed(lambda: K.rms_norm_grad_sample(x, b, D, 1e-5)),
+              "hbm", 2 * b.numel() * 2)
+    small = 2
+    idsm = torch.randint(0, V, (small, T), device=dev)
+    yield row("embedding_gs", "a4", f"n={small} T=1024 V=32000 D=2048 bf16", timed(lambda: K.embedding_grad_sample(idsm, b[:small], V)),
+              "hbm", small * V * D * 2 + small * T * D * 2)
+    P = 245_900_000
+    sm_, gr_ = torch.randn(P, device=dev).bfloat16(), torch.empty(P, device=dev, dtype=torch.bfloat16)
+    yield row("add_noise", "a11", "C5 P=245.9M bf16", timed(lambda: K.add_noise(sm_, gr_, 0.8, 16.0, 1, 0)), "hbm", 2 * P * 2)
+    del sm_, gr_, x, b
+    # ---- C4: conv 64->64 3x3 on 32x32, GroupNorm(32, 64), fp32, batch 256
+    n = 256
+    x, b = torch.randn(n, 64, 32, 32, device=dev), torch.randn(n, 64, 32, 32, device=dev)
+    yield row("conv2d_gs", "a3", "C4 n=256 64->64 3x3 32x32 f32",
+              timed(lambda: K.conv2d_grad_sample(x, b, (3, 3), (1, 1), (1, 1, 1, 1), (1, 1), 1)), "mfma_fp32",
+              2.0 * n * 64 * 576 * 1024)
+    yield row("group_norm_gs", "a6", "C4 n=256 C=64 G=32 32x32 f32", timed(lambda: K.group_norm_grad_sample(x, b, 32, 1e-5)),
+              "hbm", 2 * x.numel() * 4)
+    yield row("conv_bias_gs", "a3", "C4 n=256 O=64 32x32 f32", timed(lambda: K.conv_bias_grad_sample(b)), "hbm", b.numel() * 4)
+    # ---- C1: the small CNN's layers, fp32, batch 256
+    n = 256
+    x, b = torch.randn(n, 1, 28, 28, device=dev), torch.randn(n, 16, 14, 14, device=dev)
+    yield row("conv2d_gs", "a3", "C1 conv1 n=256 1->16 k8 s2 p3 f32",
+              timed(lambda: K.conv2d_grad_sample(x, b, (8, 8), (2, 2), (3, 3, 3, 3), (1, 1), 1)), "mfma_fp32",
+              2.0 * n * 16 * 64 * 196)
+    x, b = torch.randn(n, 16, 13, 13, device=dev), torch.randn(n, 32, 5, 5, device=dev)
+    yield row("conv2d_gs", "a3", "C1 conv2 n=256 16->32 k4 s2 f32",
+              timed(lambda: K.conv2d_grad_sample(x, b, (4, 4), (2, 2), (0, 0, 0, 0), (1, 1), 1)), "mfma_fp32",
+              2.0 * n * 32 * 256 * 25)
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -345,6 +452,12 @@ def main() -> None:
         help="also run one 1 GiB device-to-device copy before the timed region (a dispatch of known "
         "traffic against which profiler byte counters can be scaled)",
     )
+    ap.add_argument(
+        "--kernels",
+        action="store_true",
+        help="instead of a training step, time every kernel of the library on its own at the five "
+        "configurations' shapes and print one JSON line per kernel",
+    )
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build uses one GPU; run with --gpus 1 (a larger count is not measured)")
@@ -354,6 +467,10 @@ def main() -> None:
     from opacus_amd import kernels
 
     dev = torch.device("cuda:0")
+    if args.kernels:
+        for r in kernel_table(dev):
+            print(json.dumps(r), flush=True)
+        return
     w = WORKLOADS[args.workload](dev)
     step = w["step"]
     for _ in range(args.warmup):

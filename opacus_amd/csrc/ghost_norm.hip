@@ -122,60 +122,114 @@ __device__ __forceinline__ uint32_t xcd_contiguous_id(uint32_t bid, uint32_t nb)
 // the block-triangle J >= R * I is visited. Column blocks inside the row block's
 // own diagonal square (J < R * (I + 1)) count once - together they cover that
 // square completely - the ones beyond it twice.
+//
+// Work units are (sample, tile pair), numbered sample-major. The first nbig units
+// get a block each; when the launch would otherwise end in a thinly filled round
+// of resident blocks, the remaining units are cut into quadrants of 64 x 64 and
+// every quadrant gets a block of its own that splits k over its waves. Unit u
+// writes its partial sums at u * slots (a quadrant at u * slots + quadrant).
+template <class C>
+constexpr bool ghost_cfg_has_quadrants() {
+  return C::BM == 128 && C::BN == 128 && C::BK == 64 && C::kWaves == 4 && C::kStages == 2;
+}
+
 template <class C>
 __global__ __launch_bounds__(C::kThreads) void ghost_norm_bf16_dlds_kernel(
     const bf16_t* __restrict__ b, const bf16_t* __restrict__ a, float* __restrict__ pw,
-    float* __restrict__ pb, int64_t T, int64_t Dout, int64_t Din, int nJ, int npairs) {
+    float* __restrict__ pb, int64_t T, int64_t Dout, int64_t Din, int nJ, int npairs, uint32_t nbig,
+    int slots) {
   constexpr int R = C::BM / C::BN;
+  constexpr bool kQuadrants = ghost_cfg_has_quadrants<C>();
   __shared__ mb16d::Smem<C> sm;
   __shared__ float red[C::kWaves];
-  const uint32_t lid = xcd_contiguous_id(blockIdx.x, gridDim.x);
-  const int64_t sample = lid / static_cast<uint32_t>(npairs);
-  int pair = static_cast<int>(lid % static_cast<uint32_t>(npairs));
+  const bool big = !kQuadrants || blockIdx.x < nbig;
+  uint32_t unit, quad = 0;
+  if (big) {
+    unit = xcd_contiguous_id(blockIdx.x, nbig);
+  } else {
+    // nbig is a multiple of 8, so the low bits still name the XCD
+    const uint32_t sid = xcd_contiguous_id(blockIdx.x - nbig, gridDim.x - nbig);
+    unit = nbig + (sid >> 2);
+    quad = sid & 3u;
+  }
+  const int64_t sample = unit / static_cast<uint32_t>(npairs);
+  int pair = static_cast<int>(unit % static_cast<uint32_t>(npairs));
   int I = 0;
   while (pair >= nJ - R * I) {
     pair -= nJ - R * I;
     ++I;
   }
   const int J = R * I + pair;
-  const int64_t m0a = static_cast<int64_t>(I) * C::BM, m0b = static_cast<int64_t>(J) * C::BN;
+  const float weight = J < R * (I + 1) ? 1.f : 2.f;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int wm0 = (wave / C::kWaveCols) * 64, wn0 = (wave % C::kWaveCols) * 64;
-  mb16d::Tile tg, ta;
-  tg.clear();
-  ta.clear();
-  const bf16_t* bs = b + sample * T * Dout;
-  mb16d::mainloop<C>(tg, sm, bs, bs, Dout, m0a, m0b, T, Dout, wm0, wn0);
-  if (pw) {
-    const bf16_t* as = a + sample * T * Din;
-    mb16d::mainloop<C>(ta, sm, as, as, Din, m0a, m0b, T, Din, wm0, wn0);
-  }
-  // rows past T hold copies of row T - 1: leave them out
-  const int rmax = static_cast<int>(T - m0a < C::BM ? T - m0a : C::BM);
-  const int cmax = static_cast<int>(T - m0b < C::BN ? T - m0b : C::BN);
-  float sw = 0.f, sb = 0.f;
   const int kh = lane >> 5, l32 = lane & 31;
+  const bf16_t* bs = b + sample * T * Dout;
+  const bf16_t* as = a + sample * T * Din;
+  float sw = 0.f, sb = 0.f;
+  size_t slot;
+  if (big) {
+    const int64_t m0a = static_cast<int64_t>(I) * C::BM, m0b = static_cast<int64_t>(J) * C::BN;
+    const int wm0 = (wave / C::kWaveCols) * 64, wn0 = (wave % C::kWaveCols) * 64;
+    mb16d::Tile tg, ta;
+    tg.clear();
+    ta.clear();
+    mb16d::mainloop<C>(tg, sm, bs, bs, Dout, m0a, m0b, T, Dout, wm0, wn0);
+    if (pw) mb16d::mainloop<C>(ta, sm, as, as, Din, m0a, m0b, T, Din, wm0, wn0);
+    // rows past T hold copies of row T - 1: leave them out
+    const int rmax = static_cast<int>(T - m0a < C::BM ? T - m0a : C::BM);
+    const int cmax = static_cast<int>(T - m0b < C::BN ? T - m0b : C::BN);
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int row = wm0 + i * 32 + (v >> 2) * 8 + kh * 4 + (v & 3), col = wn0 + j * 32 + l32;
+          if (row < rmax && col < cmax) {
+            const float g = tg.acc[i][j][v];
+            sb += g;
+            sw = fmaf(g, ta.acc[i][j][v], sw);
+          }
+        }
+    slot = static_cast<size_t>(unit) * slots;
+  } else if constexpr (kQuadrants) {
+    // quadrant (quad >> 1, quad & 1) of the unit's tile; R == 1 on this path
+    const int64_t m0a = static_cast<int64_t>(I) * C::BM + (quad >> 1) * 64;
+    const int64_t m0b = static_cast<int64_t>(J) * C::BN + (quad & 1u) * 64;
+    slot = static_cast<size_t>(unit) * slots + quad;
+    if (m0a < T && m0b < T) {  // block-uniform
+      mb16d::Tile t;
+      t.clear();
+      mb16d::mainloop_splitk<C>(t, sm, bs, bs, Dout, m0a, m0b, T, Dout);
+      const mb16d::floatx16 g = mb16d::splitk_reduce<C>(t, sm);
+      mb16d::floatx16 h;
+      if (pw) {
+        t.clear();
+        mb16d::mainloop_splitk<C>(t, sm, as, as, Din, m0a, m0b, T, Din);
+        h = mb16d::splitk_reduce<C>(t, sm);
+      }
+      const int rmax = static_cast<int>(T - m0a < 64 ? T - m0a : 64);
+      const int cmax = static_cast<int>(T - m0b < 64 ? T - m0b : 64);
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const int row = wm0 + i * 32 + (v >> 2) * 8 + kh * 4 + (v & 3), col = wn0 + j * 32 + l32;
+        const int row = (wave >> 1) * 32 + (v >> 2) * 8 + kh * 4 + (v & 3), col = (wave & 1) * 32 + l32;
         if (row < rmax && col < cmax) {
-          const float g = tg.acc[i][j][v];
-          sb += g;
-          sw = fmaf(g, ta.acc[i][j][v], sw);
+          sb += g[v];
+          if (pw) sw = fmaf(g[v], h[v], sw);
         }
       }
-  const float weight = J < R * (I + 1) ? 1.f : 2.f;
+    }
+  }
   if (pw) {
     const float s = block_sum<C::kWaves>(sw, red);
-    if (threadIdx.x == 0) pw[lid] = s * weight;
+    if (threadIdx.x == 0) pw[slot] = s * weight;
+    // a whole unit leaves the other quadrant slots empty
+    if (big && slots > 1 && threadIdx.x < slots && threadIdx.x > 0) pw[slot + threadIdx.x] = 0.f;
   }
   if (pb) {
     const float s = block_sum<C::kWaves>(sb, red);
-    if (threadIdx.x == 0) pb[lid] = s * weight;
+    if (threadIdx.x == 0) pb[slot] = s * weight;
+    if (big && slots > 1 && threadIdx.x < slots && threadIdx.x > 0) pb[slot + threadIdx.x] = 0.f;
   }
 }
 
@@ -228,9 +282,10 @@ extern "C" size_t dpk_linear_ghost_norm_workspace_bytes(int64_t n, int64_t T, in
   (void)out;
   (void)in;
   if (n <= 0 || T <= 1) return 0;
-  // Sized for the smallest tile edge, which has the most tile pairs.
-  const int64_t nt = dpk_cdiv(T, 64);
-  return dpk_align_up(static_cast<size_t>(2 * n * (nt * (nt + 1) / 2)) * sizeof(float), 256);
+  // Room for any tiling: 64-row tile pairs, or 128-row tile pairs with four
+  // quadrant slots each (2 m^2 + 2 m slots per sample covers both).
+  const int64_t m = dpk_cdiv(T, 128);
+  return dpk_align_up(static_cast<size_t>(2 * n * (2 * m * m + 2 * m)) * sizeof(float), 256);
 }
 
 extern "C" int dpk_linear_ghost_norm(const void* b, const void* a, int dtype, float* norm_w,
@@ -269,14 +324,28 @@ extern "C" int dpk_linear_ghost_norm(const void* b, const void* a, int dtype, fl
                     dpk_aligned(b, 16) && dpk_aligned(a, 16) && T * widest * 2 < (int64_t{1} << 32);
   const int64_t npairs = dlds ? ghost_pairs(T, GhostCfg::BM, GhostCfg::BN) : nt * (nt + 1) / 2;
   const int64_t blocks = n * npairs;
-  DPK_REQUIRE(nt < 32768 && blocks <= DPK_MAX_GRID_X, DPK_E_SHAPE,
-              "%s: %lld blocks exceed the grid limit", who, (long long)blocks);
-  const size_t need = static_cast<size_t>(2 * blocks) * sizeof(float);
+  // A last round of resident blocks (two per CU) that is at most a quarter full is
+  // served by quadrant blocks instead, which then fit one round of their own: a lone
+  // tile block per CU runs latency-bound and takes most of a full round's time, a
+  // round of quadrant blocks about a third of it.
+  int64_t tail = 0;
+  if (dlds && ghost_cfg_has_quadrants<GhostCfg>()) {
+    const int cus = dpk_device_cus();
+    DPK_REQUIRE(cus > 0, DPK_E_LAUNCH, "%s: cannot query the device", who);
+    const int64_t resident = 2 * static_cast<int64_t>(cus);
+    const int64_t r = blocks % resident;
+    if (resident % 8 == 0 && r > 0 && r * 4 <= resident) tail = r;
+  }
+  const int slots = tail ? 4 : 1;
+  const int64_t grid_blocks = blocks - tail + 4 * tail;
+  DPK_REQUIRE(nt < 32768 && grid_blocks <= DPK_MAX_GRID_X && blocks * slots <= DPK_MAX_GRID_X, DPK_E_SHAPE,
+              "%s: %lld blocks exceed the grid limit", who, (long long)grid_blocks);
+  const size_t need = static_cast<size_t>(2 * blocks * slots) * sizeof(float);
   DPK_REQUIRE(ws && ws_bytes >= need, DPK_E_WORKSPACE, "%s: workspace %zu < %zu bytes", who, ws_bytes,
               need);
   DPK_REQUIRE(dpk_aligned(ws, 4), DPK_E_ALIGN, "%s: workspace misaligned", who);
   float* pw = norm_w ? static_cast<float*>(ws) : nullptr;
-  float* pb = norm_b ? static_cast<float*>(ws) + blocks : nullptr;
+  float* pb = norm_b ? static_cast<float*>(ws) + blocks * slots : nullptr;
   const dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
   if (dtype == DPK_F32) {
     const bool vec = out % 4 == 0 && in % 4 == 0 && dpk_aligned(b, 16) && dpk_aligned(a, 16);
@@ -298,9 +367,10 @@ extern "C" int dpk_linear_ghost_norm(const void* b, const void* a, int dtype, fl
     const bf16_t* bp = static_cast<const bf16_t*>(b);
     const bf16_t* ap = static_cast<const bf16_t*>(a);
     if (dlds) {
-      hipLaunchKernelGGL((ghost_norm_bf16_dlds_kernel<GhostCfg>), dim3(static_cast<unsigned>(blocks)),
+      hipLaunchKernelGGL((ghost_norm_bf16_dlds_kernel<GhostCfg>), dim3(static_cast<unsigned>(grid_blocks)),
                          dim3(GhostCfg::kThreads), 0, s, bp, ap, pw, pb, T, out, in,
-                         (int)dpk_cdiv(T, GhostCfg::BN), (int)npairs);
+                         (int)dpk_cdiv(T, GhostCfg::BN), (int)npairs, static_cast<uint32_t>(blocks - tail),
+                         slots);
       DPK_LAUNCH_CHECK(who);
     } else {
 #define DPK_GN_LAUNCH(B_, V_)                                                                  \
@@ -318,11 +388,11 @@ extern "C" int dpk_linear_ghost_norm(const void* b, const void* a, int dtype, fl
   }
   DPK_LAUNCH_CHECK(who);
   if (pw) {
-    dpk_launch_reduce_rows(pw, n, npairs, norm_w, 1, absscale, s);
+    dpk_launch_reduce_rows(pw, n, npairs * slots, norm_w, 1, absscale, s);
     DPK_LAUNCH_CHECK(who);
   }
   if (pb) {
-    dpk_launch_reduce_rows(pb, n, npairs, norm_b, 1, absscale, s);
+    dpk_launch_reduce_rows(pb, n, npairs * slots, norm_b, 1, absscale, s);
     DPK_LAUNCH_CHECK(who);
   }
   return DPK_OK;

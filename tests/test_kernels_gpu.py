@@ -297,7 +297,20 @@ def test_linear_ghost_norm_2d_inputs(K):
     assert_rel(nb, want_b, FP32_REL)
 
 
-@pytest.mark.parametrize("n,T,fin,fout", [(3, 2, 8, 16), (2, 70, 40, 24), (2, 200, 136, 264), (2, 256, 1024, 512), (3, 33, 30, 18)])
+@pytest.mark.parametrize(
+    "n,T,fin,fout",
+    [
+        (3, 2, 8, 16),
+        (2, 70, 40, 24),
+        (2, 200, 136, 264),
+        (2, 256, 1024, 512),  # direct-to-LDS kernel, few units: every unit cut into quadrant blocks
+        (3, 33, 30, 18),
+        (3, 150, 64, 64),  # quadrants that start beyond T
+        (3, 200, 64, 128),  # quadrants with a few valid rows
+        (20, 640, 64, 64),  # 300 units on a 256-CU device: whole-tile blocks only
+        (16, 1000, 64, 128),  # 576 units: 512 whole-tile blocks and a tail of quadrant blocks, ragged T
+    ],
+)
 def test_linear_ghost_norm_bf16(K, n, T, fin, fout):
     torch.manual_seed(T)
     a = torch.randn(n, T, fin).bfloat16()
