@@ -54,7 +54,12 @@ size_t ws_layout(int64_t n, int64_t T, int64_t D, void* ws, EmbWs* out) {
   return off;
 }
 
-// grid = n * ceil(T / 256); thread <-> one position t of one sample.
+// grid = n * ceil(T / 256); thread <-> one position t of one sample. Every thread
+// scans the sample's whole id row, staged through LDS a tile at a time (all lanes
+// read the same address: a broadcast). The scan is branch-free so that the reads of
+// an unrolled stretch are in flight together. Positions left of the block's own
+// stretch [t0, t1) can only be earlier occurrences and positions right of it only
+// later ones, which leaves one compare and one or two selects per id there.
 __global__ __launch_bounds__(kThreads) void emb_link_kernel(const int64_t* __restrict__ ids,
                                                              int64_t T, int64_t V, int blocks_per_sample,
                                                              int32_t* __restrict__ next,
@@ -62,30 +67,40 @@ __global__ __launch_bounds__(kThreads) void emb_link_kernel(const int64_t* __res
                                                              int32_t* __restrict__ flag) {
   __shared__ int64_t tile[kIdTile];
   const int64_t sample = blockIdx.x / blocks_per_sample;
-  const int64_t t = static_cast<int64_t>(blockIdx.x % blocks_per_sample) * kThreads + threadIdx.x;
+  const int32_t Ti = static_cast<int32_t>(T);
+  const int32_t t0 = static_cast<int32_t>(blockIdx.x % blocks_per_sample) * kThreads;
+  const int32_t t1 = t0 + kThreads < Ti ? t0 + kThreads : Ti;
+  const int32_t t = t0 + threadIdx.x;
   const int64_t* row = ids + sample * T;
-  const bool live = t < T;
+  const bool live = t < Ti;
   const int64_t mine = live ? row[t] : 0;
-  bool seen_before = false;
-  int64_t nxt = -1;
-  for (int64_t c0 = 0; c0 < T; c0 += kIdTile) {
-    const int64_t cn = (T - c0 < kIdTile) ? T - c0 : kIdTile;
+  bool before = false;  // an earlier position holds the same id
+  int32_t nxt = Ti;     // first later position with the same id
+  for (int32_t c0 = 0; c0 < Ti; c0 += kIdTile) {
+    const int32_t c1 = c0 + kIdTile < Ti ? c0 + kIdTile : Ti;
     __syncthreads();
-    for (int64_t i = threadIdx.x; i < cn; i += kThreads) tile[i] = row[c0 + i];
+    for (int32_t i = c0 + threadIdx.x; i < c1; i += kThreads) tile[i - c0] = row[i];
     __syncthreads();
-    if (live) {
-      for (int64_t i = 0; i < cn; ++i) {
-        const int64_t u = c0 + i;
-        if (tile[i] == mine) {
-          if (u < t) seen_before = true;
-          else if (u > t && nxt < 0) nxt = u;
-        }
-      }
+    const int32_t lo = t0 < c1 ? (t0 > c0 ? t0 : c0) : c1;  // [c0, lo): left of the block's stretch
+    const int32_t hi = t1 > c0 ? (t1 < c1 ? t1 : c1) : c0;  // [hi, c1): right of it
+#pragma unroll 8
+    for (int32_t u = c0; u < lo; ++u) before |= tile[u - c0] == mine;
+#pragma unroll 8
+    for (int32_t u = lo; u < hi; ++u) {
+      const bool eq = tile[u - c0] == mine;
+      before |= eq && u < t;
+      const int32_t cand = (eq && u > t) ? u : Ti;
+      nxt = cand < nxt ? cand : nxt;
+    }
+#pragma unroll 8
+    for (int32_t u = hi > lo ? hi : lo; u < c1; ++u) {
+      const int32_t cand = tile[u - c0] == mine ? u : Ti;
+      nxt = cand < nxt ? cand : nxt;
     }
   }
   if (live) {
-    next[sample * T + t] = static_cast<int32_t>(nxt);
-    leader[sample * T + t] = seen_before ? 0 : 1;
+    next[sample * T + t] = nxt < Ti ? nxt : -1;
+    leader[sample * T + t] = before ? 0 : 1;
     if (V > 0 && (mine < 0 || mine >= V)) *flag = 1;
   }
 }
