@@ -6,6 +6,8 @@
 // materialises normalize(x) and the product; here the statistics are computed
 // and applied in registers, x is read from HBM once (re-reads hit the cache) and
 // b once. HBM-bound.
+#include <algorithm>
+
 #include "dpk_common.h"
 
 namespace {
@@ -53,6 +55,85 @@ __global__ __launch_bounds__(kThreads) void group_norm_gs_kernel(
       const float bv = dpk_io<TIN>::load(bc + i);
       sw = fmaf((dpk_io<TIN>::load(xc + i) - mean) * rstd, bv, sw);
       sb += bv;
+    }
+    sw = wave_sum(sw);
+    sb = wave_sum(sb);
+    if (lane == 0) {
+      const int64_t o = sample * C + grp * Cg + c;
+      if (gw) dpk_io<TOUT>::store(gw + o, sw * scale);
+      if (gb) dpk_io<TOUT>::store(gb + o, sb * scale);
+    }
+  }
+}
+
+// Groups of at most 1024 * K elements whose channels are whole multiples of four
+// elements: every thread keeps its K four-element chunks of x in registers, so x and
+// b are read from memory exactly once. Per-chunk products go to LDS and one wave per
+// channel adds them up in a fixed order.
+template <typename TIN, typename TOUT, int K>
+__global__ __launch_bounds__(kThreads) void group_norm_gs_reg_kernel(
+    const TIN* __restrict__ x, const TIN* __restrict__ b, TOUT* __restrict__ gw,
+    TOUT* __restrict__ gb, int64_t C, int64_t S, int64_t G, float eps, float scale) {
+  __shared__ float red[kWaves];
+  __shared__ float stat[2];
+  __shared__ float cw[kThreads * K], cb[kThreads * K];
+  const int64_t sample = blockIdx.x / G, grp = blockIdx.x % G;
+  const int Cg = static_cast<int>(C / G);
+  const int len4 = static_cast<int>(Cg * S / 4), S4 = static_cast<int>(S / 4);
+  const int64_t base = (sample * C + grp * Cg) * S;
+  const TIN* xg = x + base;
+  const TIN* bg = b + base;
+  float4 xv[K];
+  float s = 0.f;
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    const int j = k * kThreads + threadIdx.x;
+    xv[k] = j < len4 ? dpk_io<TIN>::load4(xg + j * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+    s += (xv[k].x + xv[k].y) + (xv[k].z + xv[k].w);
+  }
+  s = block_sum<kWaves>(s, red);
+  if (threadIdx.x == 0) stat[0] = s / static_cast<float>(len4 * 4);
+  __syncthreads();
+  const float mean = stat[0];
+  float v = 0.f;
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    const int j = k * kThreads + threadIdx.x;
+    if (j < len4) {
+      xv[k].x -= mean;
+      xv[k].y -= mean;
+      xv[k].z -= mean;
+      xv[k].w -= mean;
+      v = fmaf(xv[k].x, xv[k].x, v);
+      v = fmaf(xv[k].y, xv[k].y, v);
+      v = fmaf(xv[k].z, xv[k].z, v);
+      v = fmaf(xv[k].w, xv[k].w, v);
+    }
+  }
+  v = block_sum<kWaves>(v, red);
+  if (threadIdx.x == 0) stat[1] = 1.0f / sqrtf(v / static_cast<float>(len4 * 4) + eps);
+  __syncthreads();
+  const float rstd = stat[1];
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    const int j = k * kThreads + threadIdx.x;
+    if (j < len4) {
+      const float4 bv = dpk_io<TIN>::load4(bg + j * 4);
+      float pw = xv[k].x * rstd * bv.x;
+      pw = fmaf(xv[k].y * rstd, bv.y, pw);
+      pw = fmaf(xv[k].z * rstd, bv.z, pw);
+      pw = fmaf(xv[k].w * rstd, bv.w, pw);
+      cw[j] = pw;
+      cb[j] = (bv.x + bv.y) + (bv.z + bv.w);
+    }
+  }
+  __syncthreads();
+  const int lane = threadIdx.x & (DPK_WAVE - 1), wave = threadIdx.x / DPK_WAVE;
+  for (int c = wave; c < Cg; c += kWaves) {
+    float sw = 0.f, sb = 0.f;
+    for (int i = lane; i < S4; i += DPK_WAVE) {
+      sw += cw[c * S4 + i];
+      sb += cb[c * S4 + i];
     }
     sw = wave_sum(sw);
     sb = wave_sum(sb);
@@ -126,9 +207,117 @@ __global__ __launch_bounds__(kThreads) void rms_final_kernel(const float* __rest
                                                               TOUT* __restrict__ gw) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (i >= nD) return;
-  float s = 0.f;
-  for (int ts = 0; ts < TS; ++ts) s += part[static_cast<int64_t>(ts) * nD + i];
-  dpk_io<TOUT>::store(gw + i, s * scale);
+  // four independent chains keep several loads in flight; the order is fixed
+  float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+  int ts = 0;
+  for (; ts + 4 <= TS; ts += 4) {
+    s0 += part[static_cast<int64_t>(ts) * nD + i];
+    s1 += part[static_cast<int64_t>(ts + 1) * nD + i];
+    s2 += part[static_cast<int64_t>(ts + 2) * nD + i];
+    s3 += part[static_cast<int64_t>(ts + 3) * nD + i];
+  }
+  for (; ts < TS; ++ts) s0 += part[static_cast<int64_t>(ts) * nD + i];
+  dpk_io<TOUT>::store(gw + i, ((s0 + s1) + (s2 + s3)) * scale);
+}
+
+// One pass: a wave keeps a whole row of x in registers (D = 256 * NCH elements, four
+// per lane and chunk), reduces its square sum across the wave, then streams the
+// matching row of b and accumulates x * rstd * b per feature. Rows t of a block's
+// stretch are dealt to its waves round-robin; the waves' partial sums meet in LDS.
+// part[ts][sample][d] as above. x and b cross HBM exactly once.
+template <typename TIN, int NCH>
+__global__ __launch_bounds__(kThreads) void rms_fused_kernel(const TIN* __restrict__ x,
+                                                              const TIN* __restrict__ b, int64_t n,
+                                                              int64_t T, float eps, int TS,
+                                                              float* __restrict__ part) {
+  constexpr int D = 256 * NCH;
+  __shared__ float red[kWaves][D];
+  const int ts = static_cast<int>(blockIdx.x % TS);
+  const int64_t sample = blockIdx.x / TS;
+  const int lane = threadIdx.x & (DPK_WAVE - 1), wave = threadIdx.x / DPK_WAVE;
+  const int64_t per = (T + TS - 1) / TS;
+  const int64_t t0 = ts * per, t1 = (t0 + per < T) ? t0 + per : T;
+  float4 acc[NCH];
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) acc[c] = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int64_t t = t0 + wave; t < t1; t += kWaves) {
+    const TIN* xr = x + (sample * T + t) * D + lane * 4;
+    const TIN* br = b + (sample * T + t) * D + lane * 4;
+    float4 xv[NCH];
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+      xv[c] = dpk_io<TIN>::load4(xr + c * 256);
+      ss = fmaf(xv[c].x, xv[c].x, ss);
+      ss = fmaf(xv[c].y, xv[c].y, ss);
+      ss = fmaf(xv[c].z, xv[c].z, ss);
+      ss = fmaf(xv[c].w, xv[c].w, ss);
+    }
+    ss = wave_sum(ss);
+    const float r = 1.0f / sqrtf(ss / static_cast<float>(D) + eps);
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+      const float4 bv = dpk_io<TIN>::load4(br + c * 256);
+      acc[c].x = fmaf(xv[c].x * r, bv.x, acc[c].x);
+      acc[c].y = fmaf(xv[c].y * r, bv.y, acc[c].y);
+      acc[c].z = fmaf(xv[c].z * r, bv.z, acc[c].z);
+      acc[c].w = fmaf(xv[c].w * r, bv.w, acc[c].w);
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) *reinterpret_cast<float4*>(&red[wave][c * 256 + lane * 4]) = acc[c];
+  __syncthreads();
+  float* o = part + (static_cast<int64_t>(ts) * n + sample) * D;
+  for (int d = threadIdx.x * 4; d < D; d += kThreads * 4) {
+    float4 s = *reinterpret_cast<const float4*>(&red[0][d]);
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) {
+      const float4 v = *reinterpret_cast<const float4*>(&red[w][d]);
+      s.x += v.x;
+      s.y += v.y;
+      s.z += v.z;
+      s.w += v.w;
+    }
+    *reinterpret_cast<float4*>(o + d) = s;
+  }
+}
+
+// Feature sizes the one-pass kernel is instantiated for (D = 256 * NCH).
+bool rms_fused_ok(int64_t D) {
+  if (D % 256 != 0) return false;
+  const int64_t c = D / 256;
+  return c == 1 || c == 2 || c == 3 || c == 4 || c == 6 || c == 8 || c == 12 || c == 16;
+}
+
+// Stretches of t per sample for the one-pass kernel: enough blocks to fill the
+// device, at least one row per wave.
+int rms_fused_splits(int64_t n, int64_t T) {
+  int64_t ts = dpk_cdiv(1024, n);
+  const int64_t most = dpk_cdiv(T, kWaves);
+  if (ts > most) ts = most;
+  if (ts > 256) ts = 256;
+  return static_cast<int>(ts < 1 ? 1 : ts);
+}
+
+template <typename TIN>
+void launch_rms_fused(const TIN* x, const TIN* b, int64_t n, int64_t T, int64_t D, float eps, int TS,
+                      float* part, hipStream_t s) {
+  const dim3 grid(static_cast<unsigned>(n * TS)), block(kThreads);
+#define DPK_RF(N_) \
+  case N_: hipLaunchKernelGGL((rms_fused_kernel<TIN, N_>), grid, block, 0, s, x, b, n, T, eps, TS, part); break
+  switch (D / 256) {
+    DPK_RF(1);
+    DPK_RF(2);
+    DPK_RF(3);
+    DPK_RF(4);
+    DPK_RF(6);
+    DPK_RF(8);
+    DPK_RF(12);
+    default:
+      hipLaunchKernelGGL((rms_fused_kernel<TIN, 16>), grid, block, 0, s, x, b, n, T, eps, TS, part);
+      break;
+  }
+#undef DPK_RF
 }
 
 int rms_splits(int64_t T) {
@@ -157,23 +346,37 @@ extern "C" int dpk_group_norm_gs(const void* x, const void* b, int in_dtype, voi
   DPK_REQUIRE(n * groups <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: too many blocks", who);
   const dim3 grid(static_cast<unsigned>(n * groups)), block(kThreads);
   hipStream_t s = static_cast<hipStream_t>(stream);
+  // register-resident path: whole chunks of four per channel, group of at most 8192
+  const int64_t len = (C / groups) * S;
+  const size_t va = in_dtype == DPK_BF16 ? 8 : 16;
+  const bool reg = S % 4 == 0 && len <= 1024 * 8 && dpk_aligned(x, va) && dpk_aligned(b, va);
+  const int K = len <= 1024 ? 1 : len <= 2048 ? 2 : len <= 4096 ? 4 : 8;
+#define DPK_GN_ARGS(TI, TO)                                                                    \
+  grid, block, 0, s, static_cast<const TI*>(x), static_cast<const TI*>(b), static_cast<TO*>(gs_w), \
+      static_cast<TO*>(gs_b), C, S, groups, eps, scale
 #define DPK_GN(TI, TO)                                                                           \
-  hipLaunchKernelGGL((group_norm_gs_kernel<TI, TO>), grid, block, 0, s, static_cast<const TI*>(x), \
-                     static_cast<const TI*>(b), static_cast<TO*>(gs_w), static_cast<TO*>(gs_b), C, S, \
-                     groups, eps, scale)
+  do {                                                                                           \
+    if (!reg) hipLaunchKernelGGL((group_norm_gs_kernel<TI, TO>), DPK_GN_ARGS(TI, TO));           \
+    else if (K == 1) hipLaunchKernelGGL((group_norm_gs_reg_kernel<TI, TO, 1>), DPK_GN_ARGS(TI, TO)); \
+    else if (K == 2) hipLaunchKernelGGL((group_norm_gs_reg_kernel<TI, TO, 2>), DPK_GN_ARGS(TI, TO)); \
+    else if (K == 4) hipLaunchKernelGGL((group_norm_gs_reg_kernel<TI, TO, 4>), DPK_GN_ARGS(TI, TO)); \
+    else hipLaunchKernelGGL((group_norm_gs_reg_kernel<TI, TO, 8>), DPK_GN_ARGS(TI, TO));         \
+  } while (0)
   if (in_dtype == DPK_F32 && gs_dtype == DPK_F32) DPK_GN(float, float);
   else if (in_dtype == DPK_BF16 && gs_dtype == DPK_BF16) DPK_GN(bf16_t, bf16_t);
   else if (in_dtype == DPK_BF16 && gs_dtype == DPK_F32) DPK_GN(bf16_t, float);
   else DPK_GN(float, bf16_t);
 #undef DPK_GN
+#undef DPK_GN_ARGS
   DPK_LAUNCH_CHECK(who);
   return DPK_OK;
 }
 
 extern "C" size_t dpk_rms_norm_gs_workspace_bytes(int64_t n, int64_t T, int64_t D) {
   if (n <= 0 || T <= 0 || D <= 0) return 0;
+  const int64_t splits = std::max<int64_t>(rms_splits(T), rms_fused_ok(D) ? rms_fused_splits(n, T) : 0);
   return dpk_align_up(static_cast<size_t>(n * T) * 4, 256) +
-         dpk_align_up(static_cast<size_t>(rms_splits(T)) * n * D * 4, 256);
+         dpk_align_up(static_cast<size_t>(splits) * n * D * 4, 256);
 }
 
 extern "C" int dpk_rms_norm_gs(const void* x, const void* b, int in_dtype, void* gs_w, int gs_dtype,
@@ -196,16 +399,22 @@ extern "C" int dpk_rms_norm_gs(const void* x, const void* b, int in_dtype, void*
   float* rstd = static_cast<float*>(ws);
   float* part = reinterpret_cast<float*>(static_cast<char*>(ws) +
                                          dpk_align_up(static_cast<size_t>(n * T) * 4, 256));
-  const int TS = rms_splits(T);
   const size_t va = in_dtype == DPK_BF16 ? 8 : 16;
   const bool vec = D % 4 == 0 && dpk_aligned(x, va) && dpk_aligned(b, va);
+  const bool fused = vec && rms_fused_ok(D) && n * rms_fused_splits(n, T) <= DPK_MAX_GRID_X;
+  const int TS = fused ? rms_fused_splits(n, T) : rms_splits(T);
   const int dch = static_cast<int>(dpk_cdiv(D, kThreads * (vec ? 4 : 1)));
   DPK_REQUIRE(n * dch * TS <= DPK_MAX_GRID_X && dpk_cdiv(n * T, kWaves) <= DPK_MAX_GRID_X, DPK_E_SHAPE,
               "%s: too many blocks", who);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 block(kThreads);
   const dim3 g1(static_cast<unsigned>(dpk_cdiv(n * T, kWaves))), g2(static_cast<unsigned>(n * dch * TS));
-  if (in_dtype == DPK_F32) {
+  if (fused) {
+    if (in_dtype == DPK_F32)
+      launch_rms_fused<float>(static_cast<const float*>(x), static_cast<const float*>(b), n, T, D, eps, TS, part, s);
+    else
+      launch_rms_fused<bf16_t>(static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(b), n, T, D, eps, TS, part, s);
+  } else if (in_dtype == DPK_F32) {
     const float* xp = static_cast<const float*>(x);
     const float* bp = static_cast<const float*>(b);
     hipLaunchKernelGGL(rms_rstd_kernel<float>, g1, block, 0, s, xp, n * T, D, eps, rstd);

@@ -432,7 +432,20 @@ def test_embedding_out_of_range_id_is_an_error(K):
 
 
 # ---- Normalisation layers ---------------------------------------------------------------
-@pytest.mark.parametrize("n,C,G,spatial", [(4, 6, 2, (3, 5)), (3, 64, 32, (32, 32)), (2, 8, 1, (7,)), (2, 10, 10, (4, 4)), (2, 256, 4, ())])
+@pytest.mark.parametrize(
+    "n,C,G,spatial",
+    [
+        (4, 6, 2, (3, 5)),
+        (3, 64, 32, (32, 32)),  # register-resident kernel, two chunks per thread
+        (2, 8, 1, (7,)),
+        (2, 10, 10, (4, 4)),  # one channel per group, four chunks in all
+        (2, 256, 4, ()),
+        (2, 16, 2, (16, 16)),  # eight channels per group
+        (2, 12, 3, (8, 8)),  # fewer chunks per channel than lanes
+        (1, 32, 1, (16, 16)),  # 8192 elements: the largest register-resident group
+        (1, 4, 1, (48, 48)),  # 9216 elements: streaming kernel
+    ],
+)
 @pytest.mark.parametrize("scale", [1.0, 3.0])
 def test_group_norm_grad_sample_f32(K, n, C, G, spatial, scale):
     torch.manual_seed(C + G)
@@ -444,7 +457,23 @@ def test_group_norm_grad_sample_f32(K, n, C, G, spatial, scale):
     assert_rel(gb, want_b, FP32_REL, "gn bias")
 
 
-@pytest.mark.parametrize("shape,D", [((4, 8), 8), ((3, 5, 8), 8), ((2, 3, 4, 16), 16), ((2, 200, 260), 260), ((2, 130, 33), 33)])
+@pytest.mark.parametrize(
+    "shape,D",
+    [
+        ((4, 8), 8),
+        ((3, 5, 8), 8),
+        ((2, 3, 4, 16), 16),
+        ((2, 200, 260), 260),
+        ((2, 130, 33), 33),
+        # multiples of 256: the one-pass kernel (a row per wave in registers)
+        ((2, 37, 256), 256),
+        ((5, 2, 512), 512),  # fewer rows than waves
+        ((3, 9, 768), 768),
+        ((2, 130, 2048), 2048),
+        ((1, 3, 4096), 4096),
+        ((2, 5, 1280), 1280),  # a multiple of 256 without an instantiation: three-kernel path
+    ],
+)
 def test_rms_norm_grad_sample_f32(K, shape, D):
     torch.manual_seed(D)
     x = torch.randn(*shape) + 0.3
@@ -460,6 +489,9 @@ def test_norm_layers_bf16(K):
     b = torch.randn(2, 70, 64).bfloat16()
     want = O.rms_norm_grad_sample(x.double(), b.double(), (64,), 1e-6)
     assert_rel(K.rms_norm_grad_sample(dev(x), dev(b), 64, 1e-6), want, BF16_REL)
+    x, b = torch.randn(3, 50, 1024).bfloat16(), torch.randn(3, 50, 1024).bfloat16()  # one-pass kernel
+    want = O.rms_norm_grad_sample(x.double(), b.double(), (1024,), 1e-6)
+    assert_rel(K.rms_norm_grad_sample(dev(x), dev(b), 1024, 1e-6), want, BF16_REL)
     x4, b4 = torch.randn(2, 8, 6, 6).bfloat16(), torch.randn(2, 8, 6, 6).bfloat16()
     want_w, want_b = O.group_norm_grad_sample(x4.double(), b4.double(), 4, 1e-5)
     gw, gb = K.group_norm_grad_sample(dev(x4), dev(b4), 4, 1e-5)
