@@ -333,12 +333,15 @@ def cpu_baseline(n_sample: int = 16, steps: int = 3) -> dict:
     }
 
 
-def kernel_table(dev, iters: int = 10, warm: int = 3):
+def kernel_table(dev, iters: int = 10, warm: int = 3, with_cpu: bool = True):
     """Every kernel of the library on its own at the benchmark configurations' shapes: yields one
     dict per kernel with its time (HIP events on the launch stream) against the roofline that
     bounds it. Work figures are algorithmic: bytes that must cross HBM once, or executed MFMA
     FLOPs (the ghost-norm kernels visit the block-triangle of the T x T Gram)."""
     from opacus_amd import kernels as K
+
+    if with_cpu:
+        from oracle import dp_oracle as O
 
     def timed(fn):
         for _ in range(warm):
@@ -352,15 +355,30 @@ def kernel_table(dev, iters: int = 10, warm: int = 3):
         torch.cuda.synchronize()
         return s.elapsed_time(e) / iters
 
-    def row(name, ref_row, shape, ms, bound, work):
+    def cpu(fn, factor, sample):
+        """The CPU oracle's function for the same row on a bounded sample of the batch, scaled
+        linearly (every one of these passes is linear in the number of samples)."""
+        if not with_cpu:
+            return None
+        fn()
+        t0 = time.perf_counter()
+        fn()
+        dt = time.perf_counter() - t0
+        return {"ms": dt * 1e3 * factor, "kind": "port", "cores": torch.get_num_threads(),
+                "sample": f"{sample}, time x {factor:g}"}
+
+    def row(name, ref_row, shape, ms, bound, work, cpu_baseline=None):
         peak, unit, scale = {
             "hbm": (HBM_PEAK_GBS, "GB/s", 1e9),
             "mfma_bf16": (MFMA_BF16_PEAK_TFLOPS, "TFLOP/s", 1e12),
             "mfma_fp32": (MFMA_FP32_PEAK_TFLOPS, "TFLOP/s", 1e12),
         }[bound]
         ach = work / (ms * 1e-3) / scale
-        return {"kernel": name, "row": ref_row, "shape": shape, "ms": ms, "bound": bound, "achieved": ach,
-                "peak": peak, "unit": unit, "frac": ach / peak, "algorithmic_work": work}
+        out = {"kernel": name, "row": ref_row, "shape": shape, "ms": ms, "bound": bound, "achieved": ach,
+               "peak": peak, "unit": unit, "frac": ach / peak, "algorithmic_work": work}
+        if cpu_baseline is not None:
+            out["cpu_baseline"] = cpu_baseline
+        return out
 
     def tri_tiles(T, tile=128):
         nt = -(-T // tile)
@@ -371,22 +389,30 @@ def kernel_table(dev, iters: int = 10, warm: int = 3):
     n, d = 128, 4096
     a, b = torch.randn(n, d, device=dev), torch.randn(n, d, device=dev)
     gs, ss = K.linear_grad_sample(b, a)
+    ca, cb = a[:8].cpu(), b[:8].cpu()
     yield row("linear_gs (T=1 outer product)", "a1", "C2 n=128 4096x4096 f32", timed(lambda: K.linear_grad_sample(b, a)),
-              "hbm", gs.numel() * 4 + 2 * n * d * 4)
-    yield row("sumsq_rows", "a10", "C2 n=128 P=16.8M f32", timed(lambda: K.sumsq_rows([gs])), "hbm", gs.numel() * 4)
+              "hbm", gs.numel() * 4 + 2 * n * d * 4,
+              cpu(lambda: O.store_grad_sample(O.linear_grad_sample(ca, cb)[0], 8), 16, "8 of 128 samples, einsum + zero/copy buffer"))
+    cgs = O.linear_grad_sample(ca, cb)[0] if with_cpu else None
+    yield row("sumsq_rows", "a10", "C2 n=128 P=16.8M f32", timed(lambda: K.sumsq_rows([gs])), "hbm", gs.numel() * 4,
+              cpu(lambda: cgs.reshape(8, -1).norm(2, dim=-1), 16, "8 of 128 samples"))
     _, clip = K.clip_factor(ss.reshape(1, -1), 1.0)
     out = torch.empty(d, d, device=dev)
     yield row("clip_accumulate", "a10", "C2 n=128 P=16.8M f32", timed(lambda: K.clip_accumulate([gs], clip, [out], False)),
-              "hbm", gs.numel() * 4 + out.numel() * 4)
+              "hbm", gs.numel() * 4 + out.numel() * 4,
+              cpu(lambda: O.clip_and_accumulate([cgs], 1.0), 16, "8 of 128 samples, norm + clip + einsum"))
     g = torch.empty_like(out)
-    yield row("add_noise", "a11", "C2 P=16.8M f32", timed(lambda: K.add_noise(out, g, 1.0, 128.0, 1, 0)), "hbm", 2 * out.numel() * 4)
+    csum = torch.zeros(d, d) if with_cpu else None
+    yield row("add_noise", "a11", "C2 P=16.8M f32", timed(lambda: K.add_noise(out, g, 1.0, 128.0, 1, 0)), "hbm", 2 * out.numel() * 4,
+              cpu(lambda: O.add_noise_and_scale([csum], [csum.shape], 1.0, 1.0, 128), 1, "full size"))
     yield row("linear_bias_gs", "a1", "C2 n=128 out=4096 f32", timed(lambda: K.linear_bias_grad_sample(b)), "hbm", 2 * n * d * 4)
-    del gs, out, g
+    del gs, out, g, cgs, csum
     # ---- Linear per-sample gradients with a sequence dimension (fp32 MFMA)
     n, T, i, o = 16, 256, 1024, 1024
     a, b = torch.randn(n, T, i, device=dev), torch.randn(n, T, o, device=dev)
+    ca, cb = a[:4].cpu(), b[:4].cpu()
     yield row("linear_gs (T>1, fp32 MFMA)", "a1", "n=16 T=256 1024x1024 f32", timed(lambda: K.linear_grad_sample(b, a)),
-              "mfma_fp32", 2.0 * n * T * i * o)
+              "mfma_fp32", 2.0 * n * T * i * o, cpu(lambda: O.linear_grad_sample(ca, cb), 4, "4 of 16 samples"))
     # ---- C3 / C5: ghost norms, bf16
     for cfg, n, T, layers in (
         ("C3", 32, 512, [(1024, 4096, "fc1"), (4096, 1024, "fc2")]),
@@ -398,34 +424,45 @@ def kernel_table(dev, iters: int = 10, warm: int = 3):
             a = torch.randn(n, T, i, device=dev).bfloat16()
             b = (torch.randn(n, T, o, device=dev) * 0.02).bfloat16()
             ms = timed(lambda: K.linear_ghost_norm(b, a, want_weight=True, want_bias=False))
+            ca, cb = a[:1].cpu(), b[:1].cpu()
             yield row("linear_ghost_norm", "a2", f"{cfg} {name} n={n} T={T} {i}->{o} bf16", ms, "mfma_bf16",
-                      2.0 * n * T * T * (i + o) * tri / full)
+                      2.0 * n * T * T * (i + o) * tri / full,
+                      cpu(lambda: O.linear_norm_sample(ca, cb), n, f"1 of {n} samples, bf16 bmm Grams"))
             del a, b
     # ---- C5: embedding ghost norm, RMSNorm, noise over all parameters (bf16)
     n, T, D, V = 16, 1024, 2048, 32000
     ids = torch.randint(0, V, (n, T), device=dev)
     b = (torch.randn(n, T, D, device=dev) * 0.02).bfloat16()
     x = torch.randn(n, T, D, device=dev).bfloat16()
+    cids, cb, cx = ids[:4].cpu(), b[:4].cpu(), x[:4].cpu()
     yield row("embedding_ghost_norm", "a5", "C5 n=16 T=1024 D=2048 bf16", timed(lambda: K.embedding_ghost_norm(ids, b)),
-              "hbm", b.numel() * 2 + ids.numel() * 8)
+              "hbm", b.numel() * 2 + ids.numel() * 8,
+              cpu(lambda: O.embedding_norm_sample(cids, cb), 4, "4 of 16 samples"))
     yield row("rms_norm_gs", "a6", "C5 n=16 T=1024 D=2048 bf16", timed(lambda: K.rms_norm_grad_sample(x, b, D, 1e-5)),
-              "hbm", 2 * b.numel() * 2)
+              "hbm", 2 * b.numel() * 2, cpu(lambda: O.rms_norm_grad_sample(cx, cb, (D,), 1e-5), 4, "4 of 16 samples"))
     small = 2
     idsm = torch.randint(0, V, (small, T), device=dev)
+    cidm, cbm = idsm.cpu(), b[:small].cpu()
     yield row("embedding_gs", "a4", f"n={small} T=1024 V=32000 D=2048 bf16", timed(lambda: K.embedding_grad_sample(idsm, b[:small], V)),
-              "hbm", small * V * D * 2 + small * T * D * 2)
+              "hbm", small * V * D * 2 + small * T * D * 2,
+              cpu(lambda: O.embedding_grad_sample(cidm, cbm, V), 1, "full size"))
     P = 245_900_000
     sm_, gr_ = torch.randn(P, device=dev).bfloat16(), torch.empty(P, device=dev, dtype=torch.bfloat16)
-    yield row("add_noise", "a11", "C5 P=245.9M bf16", timed(lambda: K.add_noise(sm_, gr_, 0.8, 16.0, 1, 0)), "hbm", 2 * P * 2)
+    csum = torch.zeros(P // 10, dtype=torch.bfloat16) if with_cpu else None
+    yield row("add_noise", "a11", "C5 P=245.9M bf16", timed(lambda: K.add_noise(sm_, gr_, 0.8, 16.0, 1, 0)), "hbm", 2 * P * 2,
+              cpu(lambda: O.add_noise_and_scale([csum], [csum.shape], 0.8, 1.0, 16), 10, "a tenth of the elements"))
     del sm_, gr_, x, b
     # ---- C4: conv 64->64 3x3 on 32x32, GroupNorm(32, 64), fp32, batch 256
     n = 256
     x, b = torch.randn(n, 64, 32, 32, device=dev), torch.randn(n, 64, 32, 32, device=dev)
+    cx, cb = x[:16].cpu(), b[:16].cpu()
     yield row("conv2d_gs", "a3", "C4 n=256 64->64 3x3 32x32 f32",
               timed(lambda: K.conv2d_grad_sample(x, b, (3, 3), (1, 1), (1, 1, 1, 1), (1, 1), 1)), "mfma_fp32",
-              2.0 * n * 64 * 576 * 1024)
+              2.0 * n * 64 * 576 * 1024,
+              cpu(lambda: O.conv2d_grad_sample(cx, cb, kernel_size=(3, 3), padding=(1, 1), stride=(1, 1), dilation=(1, 1), groups=1),
+                  16, "16 of 256 samples, unfold + einsum"))
     yield row("group_norm_gs", "a6", "C4 n=256 C=64 G=32 32x32 f32", timed(lambda: K.group_norm_grad_sample(x, b, 32, 1e-5)),
-              "hbm", 2 * x.numel() * 4)
+              "hbm", 2 * x.numel() * 4, cpu(lambda: O.group_norm_grad_sample(cx, cb, 32, 1e-5), 16, "16 of 256 samples"))
     yield row("conv_bias_gs", "a3", "C4 n=256 O=64 32x32 f32", timed(lambda: K.conv_bias_grad_sample(b)), "hbm", b.numel() * 4)
     # ---- C1: the small CNN's layers, fp32, batch 256
     n = 256
@@ -468,7 +505,7 @@ def main() -> None:
 
     dev = torch.device("cuda:0")
     if args.kernels:
-        for r in kernel_table(dev):
+        for r in kernel_table(dev, with_cpu=not args.no_cpu_baseline):
             print(json.dumps(r), flush=True)
         return
     w = WORKLOADS[args.workload](dev)
