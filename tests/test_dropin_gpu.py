@@ -333,6 +333,43 @@ def test_virtual_steps_accumulate_summed_grad(A):
     close(gsm._module.bias.grad, total[1] / 10, 1e-4, 1e-6)
 
 
+def test_batch_memory_manager_equals_one_large_batch(A):
+    """Logical batches of 12 run as physical batches of at most 5 give the update of the
+    undivided batch (sigma = 0), and the model only moves at the end of a logical batch
+    (the reference's tests/batch_memory_manager_test.py checks the same two things)."""
+    from opacus_amd.utils.batch_memory_manager import BatchMemoryManager
+
+    torch.manual_seed(11)
+    net = nn.Sequential(nn.Linear(6, 8), nn.ReLU(), nn.Linear(8, 3))
+    x, y = torch.randn(24, 6), torch.randint(0, 3, (24,))
+    dl = DataLoader(TensorDataset(x, y), batch_size=12, shuffle=False)
+
+    def make():
+        gsm = A.GradSampleModule(copy.deepcopy(net).to(DEV), loss_reduction="mean")
+        opt = A.DPOptimizer(torch.optim.SGD(gsm.parameters(), lr=0.5), noise_multiplier=0.0, max_grad_norm=0.3, expected_batch_size=12)
+        return gsm, opt
+
+    whole, opt_w = make()
+    for xb, yb in dl:
+        opt_w.zero_grad()
+        F.cross_entropy(whole(xb.to(DEV)), yb.to(DEV)).backward()
+        opt_w.step()
+
+    pieces, opt_p = make()
+    moved = []
+    with BatchMemoryManager(data_loader=dl, max_physical_batch_size=5, optimizer=opt_p) as dl2:
+        for xb, yb in dl2:
+            assert len(xb) <= 5
+            before = pieces._module[0].weight.detach().clone()
+            opt_p.zero_grad()
+            F.cross_entropy(pieces(xb.to(DEV)), yb.to(DEV), reduction="sum").div(len(xb)).backward()
+            opt_p.step()
+            moved.append(not torch.equal(before, pieces._module[0].weight.detach()))
+    assert moved == [False, False, True, False, False, True]
+    for pw, pp in zip(whole.parameters(), pieces.parameters()):
+        close(pp, pw, 1e-5, 1e-6, "parameters after two logical batches")
+
+
 def test_noise_level(A):
     """privacy_engine_test.py:676-739: with zero gradients, after k steps sum p^2 ~ k P (sigma C lr / B)^2."""
     torch.manual_seed(8)
