@@ -210,6 +210,18 @@ int dpk_clip_accumulate_multi(const void* const* gs /*host*/, void* const* summe
                               const int64_t* P /*host*/, int64_t K, int gs_dtype, int out_dtype,
                               const float* clip, int64_t n, int accumulate, dpk_stream_t stream);
 
+/* Per-layer clipping (opacus/optimizers/perlayeroptimizer.py:58-76): every parameter k
+ * has its own bound. clip[k*n + i] = min(1, C[k] / (sqrt(sumsq[k*n + i]) + 1e-6))
+ * (with `is_norm` != 0 the input holds norms), max_grad_norms: host array of K floats,
+ * K <= DPK_MULTI_MAX. dpk_clip_accumulate_per_layer is dpk_clip_accumulate_multi with
+ * tensor k weighted by row k of that [K,n] factor table. */
+int dpk_clip_factor_per_layer(const float* sumsq, int64_t K, int64_t n, int is_norm,
+                              const float* max_grad_norms /*host*/, float* clip, dpk_stream_t stream);
+int dpk_clip_accumulate_per_layer(const void* const* gs /*host*/, void* const* summed /*host*/,
+                                  const int64_t* P /*host*/, int64_t K, int gs_dtype, int out_dtype,
+                                  const float* clip /*[K,n]*/, int64_t n, int accumulate,
+                                  dpk_stream_t stream);
+
 /* grad[p] = (summed[p] + std * z[p]) / denom,  z ~ N(0,1)   (optimizer.py:485-504)
  * Folds _generate_noise (optimizer.py:104-169), the add (:491) and scale_grad's
  * division (:502-504) into one pass. std == 0 adds exact zeros and draws

@@ -103,12 +103,14 @@ __global__ void clip_factor_kernel(const float* __restrict__ v, int64_t K, int64
 // ceiling. RS > 1 keeps the chip busy when P is small and n large.
 template <typename TG, typename TO, bool VEC, int RS, int NT, int U>
 __global__ __launch_bounds__(NT) void clip_accumulate_kernel(MultiArgs a, int64_t n,
-                                                               const float* __restrict__ clip,
-                                                               int accumulate) {
+                                                               const float* __restrict__ clip_base,
+                                                               int64_t clip_stride, int accumulate) {
   constexpr int W = VEC ? 4 : 1;
   constexpr int CX = NT / RS;
   __shared__ float4 part[RS > 1 ? NT : 1];
   const int k = find_tensor(a, blockIdx.x);
+  // one factor vector for all tensors (stride 0) or one per tensor (per-layer clipping)
+  const float* __restrict__ clip = clip_base + k * clip_stride;
   const int64_t P = a.P[k];
   const int64_t blk = blockIdx.x - a.prefix[k];
   const int cx = threadIdx.x % CX;
@@ -191,16 +193,17 @@ constexpr int kStreamUnroll = 16;
 
 template <typename TG, typename TO, bool VEC, int RS>
 void launch_clip_accumulate(const MultiArgs& a, int64_t blocks, int64_t n, const float* clip,
-                            int accumulate, hipStream_t s) {
+                            int64_t clip_stride, int accumulate, hipStream_t s) {
   constexpr int NT = RS == 1 ? kStreamThreads : kThreads;
   constexpr int U = RS == 1 ? kStreamUnroll : 8;
   hipLaunchKernelGGL((clip_accumulate_kernel<TG, TO, VEC, RS, NT, U>),
-                     dim3(static_cast<unsigned>(blocks)), dim3(NT), 0, s, a, n, clip, accumulate);
+                     dim3(static_cast<unsigned>(blocks)), dim3(NT), 0, s, a, n, clip, clip_stride, accumulate);
 }
 
 template <typename TG, typename TO>
 void dispatch_clip_accumulate(MultiArgs& a, const int64_t* P, int K, int64_t n, const float* clip,
-                              int accumulate, bool vec, int rs, hipStream_t s, int64_t* blocks_out) {
+                              int64_t clip_stride, int accumulate, bool vec, int rs, hipStream_t s,
+                              int64_t* blocks_out) {
   const int W = vec ? 4 : 1;
   const int64_t cols_per_block = static_cast<int64_t>((rs == 1 ? kStreamThreads : kThreads) / rs) * W;
   a.prefix[0] = 0;
@@ -209,11 +212,11 @@ void dispatch_clip_accumulate(MultiArgs& a, const int64_t* P, int K, int64_t n, 
   *blocks_out = blocks;
   if (blocks == 0 || blocks > DPK_MAX_GRID_X) return;
   if (vec) {
-    if (rs == 1) launch_clip_accumulate<TG, TO, true, 1>(a, blocks, n, clip, accumulate, s);
-    else launch_clip_accumulate<TG, TO, true, 16>(a, blocks, n, clip, accumulate, s);
+    if (rs == 1) launch_clip_accumulate<TG, TO, true, 1>(a, blocks, n, clip, clip_stride, accumulate, s);
+    else launch_clip_accumulate<TG, TO, true, 16>(a, blocks, n, clip, clip_stride, accumulate, s);
   } else {
-    if (rs == 1) launch_clip_accumulate<TG, TO, false, 1>(a, blocks, n, clip, accumulate, s);
-    else launch_clip_accumulate<TG, TO, false, 16>(a, blocks, n, clip, accumulate, s);
+    if (rs == 1) launch_clip_accumulate<TG, TO, false, 1>(a, blocks, n, clip, clip_stride, accumulate, s);
+    else launch_clip_accumulate<TG, TO, false, 16>(a, blocks, n, clip, clip_stride, accumulate, s);
   }
 }
 
@@ -307,11 +310,10 @@ extern "C" int dpk_clip_factor(const float* sumsq, int64_t K, int64_t n, int is_
   return DPK_OK;
 }
 
-extern "C" int dpk_clip_accumulate_multi(const void* const* gs, void* const* summed,
-                                         const int64_t* P, int64_t K, int gs_dtype, int out_dtype,
-                                         const float* clip, int64_t n, int accumulate,
-                                         dpk_stream_t stream) {
-  const char* who = "dpk_clip_accumulate_multi";
+namespace {
+int clip_accumulate_impl(const char* who, const void* const* gs, void* const* summed, const int64_t* P,
+                         int64_t K, int gs_dtype, int out_dtype, const float* clip, int64_t clip_stride,
+                         int64_t n, int accumulate, dpk_stream_t stream) {
   DPK_REQUIRE(n >= 0, DPK_E_SHAPE, "%s: n=%lld", who, (long long)n);
   DPK_REQUIRE(gs && summed && P, DPK_E_ARG, "%s: NULL pointer table", who);
   DPK_REQUIRE(K >= 1 && K <= DPK_MULTI_MAX, DPK_E_SHAPE, "%s: K=%lld not in [1,%d]", who,
@@ -343,15 +345,70 @@ extern "C" int dpk_clip_accumulate_multi(const void* const* gs, void* const* sum
   hipStream_t s = static_cast<hipStream_t>(stream);
   int64_t blocks = 0;
   if (gs_dtype == DPK_F32 && out_dtype == DPK_F32)
-    dispatch_clip_accumulate<float, float>(a, P, (int)K, n, clip, accumulate, vec, rs, s, &blocks);
+    dispatch_clip_accumulate<float, float>(a, P, (int)K, n, clip, clip_stride, accumulate, vec, rs, s, &blocks);
   else if (gs_dtype == DPK_BF16 && out_dtype == DPK_F32)
-    dispatch_clip_accumulate<bf16_t, float>(a, P, (int)K, n, clip, accumulate, vec, rs, s, &blocks);
+    dispatch_clip_accumulate<bf16_t, float>(a, P, (int)K, n, clip, clip_stride, accumulate, vec, rs, s, &blocks);
   else if (gs_dtype == DPK_F32 && out_dtype == DPK_BF16)
-    dispatch_clip_accumulate<float, bf16_t>(a, P, (int)K, n, clip, accumulate, vec, rs, s, &blocks);
+    dispatch_clip_accumulate<float, bf16_t>(a, P, (int)K, n, clip, clip_stride, accumulate, vec, rs, s, &blocks);
   else
-    dispatch_clip_accumulate<bf16_t, bf16_t>(a, P, (int)K, n, clip, accumulate, vec, rs, s, &blocks);
+    dispatch_clip_accumulate<bf16_t, bf16_t>(a, P, (int)K, n, clip, clip_stride, accumulate, vec, rs, s, &blocks);
   DPK_REQUIRE(blocks <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: %lld blocks exceed the grid limit", who,
               (long long)blocks);
+  DPK_LAUNCH_CHECK(who);
+  return DPK_OK;
+}
+}  // namespace
+
+extern "C" int dpk_clip_accumulate_multi(const void* const* gs, void* const* summed,
+                                         const int64_t* P, int64_t K, int gs_dtype, int out_dtype,
+                                         const float* clip, int64_t n, int accumulate,
+                                         dpk_stream_t stream) {
+  return clip_accumulate_impl("dpk_clip_accumulate_multi", gs, summed, P, K, gs_dtype, out_dtype, clip, 0,
+                              n, accumulate, stream);
+}
+
+extern "C" int dpk_clip_accumulate_per_layer(const void* const* gs, void* const* summed,
+                                             const int64_t* P, int64_t K, int gs_dtype, int out_dtype,
+                                             const float* clip, int64_t n, int accumulate,
+                                             dpk_stream_t stream) {
+  return clip_accumulate_impl("dpk_clip_accumulate_per_layer", gs, summed, P, K, gs_dtype, out_dtype, clip,
+                              n, n, accumulate, stream);
+}
+
+namespace {
+struct LayerBounds {
+  float C[DPK_MULTI_MAX];
+};
+
+__global__ void clip_factor_per_layer_kernel(const float* __restrict__ v, int64_t n, int is_norm,
+                                             LayerBounds bounds, float* __restrict__ clip) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int k = blockIdx.y;
+  const float x = v[k * n + i];
+  const float nr = is_norm ? fabsf(x) : sqrtf(x);
+  clip[k * n + i] = fminf(bounds.C[k] / (nr + 1e-6f), 1.0f);
+}
+}  // namespace
+
+extern "C" int dpk_clip_factor_per_layer(const float* sumsq, int64_t K, int64_t n, int is_norm,
+                                         const float* max_grad_norms, float* clip,
+                                         dpk_stream_t stream) {
+  const char* who = "dpk_clip_factor_per_layer";
+  DPK_REQUIRE(K >= 1 && K <= DPK_MULTI_MAX && n >= 0, DPK_E_SHAPE, "%s: K=%lld (1..%d) n=%lld", who,
+              (long long)K, DPK_MULTI_MAX, (long long)n);
+  if (n == 0) return DPK_OK;
+  DPK_REQUIRE(sumsq && clip && max_grad_norms, DPK_E_ARG, "%s: NULL argument", who);
+  DPK_REQUIRE(dpk_cdiv(n, 256) <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: n too large", who);
+  LayerBounds bounds;
+  for (int k = 0; k < K; ++k) {
+    DPK_REQUIRE(max_grad_norms[k] >= 0.f, DPK_E_ARG, "%s: max_grad_norms[%d]=%g", who, k,
+                (double)max_grad_norms[k]);
+    bounds.C[k] = max_grad_norms[k];
+  }
+  hipLaunchKernelGGL(clip_factor_per_layer_kernel,
+                     dim3(static_cast<unsigned>(dpk_cdiv(n, 256)), static_cast<unsigned>(K)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), sumsq, n, is_norm, bounds, clip);
   DPK_LAUNCH_CHECK(who);
   return DPK_OK;
 }

@@ -455,18 +455,44 @@ def clip_factor(
     return norm, clip
 
 
+def clip_factor_per_layer(
+    values: torch.Tensor, max_grad_norms: Sequence[float], is_norm: bool = False
+) -> torch.Tensor:
+    """``clip[K, n]`` with ``clip[k] = min(1, C_k / (norm_k + 1e-6))`` from ``values[K, n]``
+    (squared norms, or norms with ``is_norm``)."""
+    dev = _need_gpu(values)
+    v = _dense(values.to(torch.float32)).reshape(-1, values.shape[-1])
+    K, n = v.shape
+    if len(max_grad_norms) != K:
+        raise ValueError(f"{len(max_grad_norms)} bounds for {K} parameters")
+    clip = torch.empty((K, n), dtype=torch.float32, device=dev)
+    if n == 0:
+        return clip
+    L = lib()
+    for lo in range(0, K, DPK_MULTI_MAX):
+        k = min(DPK_MULTI_MAX, K - lo)
+        bounds = (ctypes.c_float * k)(*[float(c) for c in max_grad_norms[lo : lo + k]])
+        check(
+            "dpk_clip_factor_per_layer",
+            L.dpk_clip_factor_per_layer(_ptr(v[lo:]), k, n, int(is_norm), bounds, _ptr(clip[lo:]), _stream(dev)),
+        )
+    return clip
+
+
 def clip_accumulate(
     gs_list: Sequence[torch.Tensor],
     clip: torch.Tensor,
     summed_list: Sequence[torch.Tensor],
     accumulate: bool,
 ) -> None:
-    """``summed_k (+)= sum_n clip[n] * gs_k[n]`` for every k, reading each gs once."""
+    """``summed_k (+)= sum_n clip[n] * gs_k[n]`` for every k, reading each gs once. ``clip`` is
+    one vector ``[n]`` for all tensors, or a table ``[K, n]`` with a row per tensor."""
     dev = _need_gpu(clip, *gs_list, *summed_list)
     K = len(gs_list)
     if K == 0:
         return
     n = gs_list[0].shape[0]
+    per_layer = clip.dim() == 2
     flats = [_flat2d(g) for g in gs_list]
     gdt, odt = flats[0].dtype, summed_list[0].dtype
     for f, s in zip(flats, summed_list):
@@ -474,23 +500,23 @@ def clip_accumulate(
             raise ValueError("tensors of one clip_accumulate call must share batch size and dtypes")
         if not s.is_contiguous() or s.numel() != f.shape[1]:
             raise ValueError("summed tensors must be dense and match the per-sample gradient size")
-    if clip.dtype != torch.float32 or clip.numel() != n:
-        raise ValueError("clip must be a float32 tensor with one entry per sample")
+    if clip.dtype != torch.float32 or clip.shape != ((K, n) if per_layer else (n,)):
+        raise ValueError("clip must be float32 of shape [n], or [K, n] with a row per tensor")
     clip = _dense(clip)
     L = lib()
+    name = "dpk_clip_accumulate_per_layer" if per_layer else "dpk_clip_accumulate_multi"
+    fn = getattr(L, name)
     for lo in range(0, K, DPK_MULTI_MAX):
         fs, ss = flats[lo : lo + DPK_MULTI_MAX], summed_list[lo : lo + DPK_MULTI_MAX]
         k = len(fs)
         gptrs = (ctypes.c_void_p * k)(*[f.data_ptr() for f in fs])
         sptrs = (ctypes.c_void_p * k)(*[s.data_ptr() for s in ss])
         sizes = (ctypes.c_int64 * k)(*[f.shape[1] for f in fs])
+        factors = clip[lo:] if per_layer else clip
         with _timed("clip_accumulate", dev):
             check(
-                "dpk_clip_accumulate_multi",
-                L.dpk_clip_accumulate_multi(
-                    gptrs, sptrs, sizes, k, _code(gdt), _code(odt), _ptr(clip), n, int(accumulate),
-                    _stream(dev),
-                ),
+                name,
+                fn(gptrs, sptrs, sizes, k, _code(gdt), _code(odt), _ptr(factors), n, int(accumulate), _stream(dev)),
             )
 
 

@@ -228,6 +228,16 @@ class DPOptimizer(Optimizer):
                 rows[k] = got[j]
         return torch.stack([r.to(dev) for r in rows], dim=0) if len(rows) > 1 else rows[0].to(dev).reshape(1, n)
 
+    def _clip_factors(self, plist: List[nn.Parameter], flats: List[torch.Tensor]) -> torch.Tensor:
+        """Per-sample clip factors ``min(1, C / (norm + 1e-6))`` of the whole gradient
+        (optimizer.py:444-455): ``float32[n]``. Subclasses with another clipping rule return
+        their own vector, or a ``[K, n]`` table with a row per parameter."""
+        n = len(flats[0])
+        if n == 0:
+            return torch.zeros((0,), device=flats[0].device, dtype=torch.float32)
+        sumsq = self._per_param_sumsq(plist, flats)
+        return kernels.clip_factor(sumsq, float(self.max_grad_norm))[1]
+
     def clip_and_accumulate(self):
         """Clips every sample's gradient to ``max_grad_norm`` and adds the clipped gradients
         into ``p.summed_grad`` (optimizer.py:432-475)."""
@@ -239,12 +249,8 @@ class DPOptimizer(Optimizer):
             if not kernels.supported_dtype(g.dtype):
                 raise TypeError(f"per-sample gradients must be float32 or bfloat16 on this path, got {g.dtype}")
             flats.append(g)
-        n = len(flats[0])
-        if n == 0:
-            clip = torch.zeros((0,), device=flats[0].device, dtype=torch.float32)
-        else:
-            sumsq = self._per_param_sumsq(plist, flats)
-            _, clip = kernels.clip_factor(sumsq, float(self.max_grad_norm))
+        clip = self._clip_factors(plist, flats)
+        per_layer = clip.dim() == 2
         # one launch per (device, per-sample dtype, parameter dtype, fresh/accumulate) group
         groups: Dict[tuple, List[int]] = {}
         for k, (p, g) in enumerate(zip(plist, flats)):
@@ -258,8 +264,9 @@ class DPOptimizer(Optimizer):
                     raise ValueError("summed_grad must be a dense tensor of the parameter's dtype")
             groups.setdefault((g.device, g.dtype, out_dtype, fresh), []).append(k)
         for (dev, _, _, fresh), idxs in groups.items():
+            factors = clip[idxs] if per_layer and len(idxs) != len(plist) else clip
             kernels.clip_accumulate(
-                [flats[k] for k in idxs], clip.to(dev), [plist[k].summed_grad for k in idxs], accumulate=not fresh
+                [flats[k] for k in idxs], factors.to(dev), [plist[k].summed_grad for k in idxs], accumulate=not fresh
             )
         for p in plist:
             if p.summed_grad.dtype != p.dtype:

@@ -21,6 +21,9 @@ What pins each function (see ``tests/test_oracle_pins.py``):
   * clip_and_accumulate / add_noise / scale_grad: closed forms, batch-of-one gives a sum
     of norm C (opacus/tests/privacy_engine_test.py:302-327), C -> inf and sigma = 0
     reproduce plain SGD (:220-273);
+  * per-layer clipping: reduces to flat clipping for one parameter, to the plain sum for
+    huge bounds, and bounds every parameter's norm by its own C_k; AdaClip's count and
+    bound update: hand-checked numbers;
   * Philox4x32-10: the Random123 known-answer vectors.
 No function here is "parity unpinned".
 """
@@ -304,6 +307,33 @@ def clip_and_accumulate(
             grad = summed[k] + grad
         out.append(grad)
     return norms, clip, out
+
+
+def per_layer_clip_and_accumulate(
+    grad_samples: Sequence[torch.Tensor], max_grad_norms: Sequence[float]
+) -> Tuple[List[torch.Tensor], List[torch.Tensor]]:
+    """opacus/optimizers/perlayeroptimizer.py:58-76: every parameter clipped on its own norm with
+    its own bound. Returns (clip factors per parameter, summed grads)."""
+    clips, out = [], []
+    for g, c in zip(grad_samples, max_grad_norms):
+        norms = g.reshape(len(g), -1).norm(2, dim=-1)
+        clip = (c / (norms + 1e-6)).clamp(max=1.0)
+        clips.append(clip)
+        out.append(torch.einsum("i,i...", clip, g))
+    return clips, out
+
+
+def adaclip_update(
+    clip: torch.Tensor, max_grad_norm: float, target_quantile: float, learning_rate: float, min_bound: float,
+    max_bound: float, count_noise: float = 0.0,
+) -> Tuple[float, float]:
+    """opacus/optimizers/adaclipoptimizer.py:119-121, 181-194: the unclipped count
+    ``n - #(clip < 1)`` (plus its noise) and the bound after one geometric update, kept inside
+    ``[min_bound, max_bound]``. Returns (noisy count, new bound)."""
+    n = len(clip)
+    count = float(n - int((clip < 1).sum())) + count_noise
+    new = max_grad_norm * math.exp(-learning_rate * (count / n - target_quantile))
+    return count, min(max(new, min_bound), max_bound)
 
 
 def generate_noise(std: float, reference: torch.Tensor, generator=None, secure_mode: bool = False) -> torch.Tensor:

@@ -36,6 +36,8 @@ def test_header_declares_the_expected_surface():
         "dpk_clip_accumulate_multi",
         "dpk_add_noise",
         "dpk_add_noise_multi",
+        "dpk_clip_factor_per_layer",
+        "dpk_clip_accumulate_per_layer",
     ]:
         assert must in names
 

@@ -370,6 +370,72 @@ def test_batch_memory_manager_equals_one_large_batch(A):
         close(pp, pw, 1e-5, 1e-6, "parameters after two logical batches")
 
 
+def test_per_layer_clipping_matches_oracle(A):
+    """perlayeroptimizer.py:58-76 through ``make_private(clipping="per_layer")``: every parameter
+    clipped on its own norm, all of them in one launch with a [K, n] factor table."""
+    torch.manual_seed(21)
+    net = SmallCNN()
+    x, y = torch.randn(6, 1, 28, 28), torch.randint(0, 10, (6,))
+    bounds = [0.05, 0.5, 0.02, 1e3, 0.3, 0.01, 0.2, 0.4]
+    gs = per_sample_grads_cpu(net, x, y, ce_sum)
+    names = [k for k, _ in net.named_parameters()]
+    _, want = O.per_layer_clip_and_accumulate([gs[k] for k in names], bounds)
+    model = copy.deepcopy(net).to(DEV)
+    engine = A.PrivacyEngine()
+    dl = DataLoader(TensorDataset(x, y), batch_size=6)
+    gsm, opt, _ = engine.make_private(
+        module=model, optimizer=torch.optim.SGD(model.parameters(), lr=0.0), data_loader=dl, noise_multiplier=0.0,
+        max_grad_norm=bounds, poisson_sampling=False, clipping="per_layer",
+    )
+    assert type(opt).__name__ == "DPPerLayerOptimizer"
+    opt.zero_grad()
+    F.cross_entropy(gsm(x.to(DEV)), y.to(DEV)).backward()
+    opt.step()
+    for (k, p), w in zip(gsm._module.named_parameters(), want):
+        close(p.grad, w / 6, 2e-4, 1e-7, f"per-layer clipped mean gradient of {k}")
+    # a second, accumulated step (virtual batch) adds into summed_grad with the same table form
+    opt.signal_skip_step(True)
+    opt.zero_grad()
+    F.cross_entropy(gsm(x.to(DEV)), y.to(DEV)).backward()
+    assert opt.step() is None
+    opt.zero_grad()
+    F.cross_entropy(gsm(x.to(DEV)), y.to(DEV)).backward()
+    opt.step()
+    for (k, p), w in zip(gsm._module.named_parameters(), want):
+        close(p.grad, 2 * w / 6, 2e-4, 1e-7, f"accumulated per-layer gradient of {k}")
+
+
+def test_adaptive_clipping_counts_and_updates_the_bound(A):
+    """adaclipoptimizer.py: unclipped count from the clip factors, bound update after a full step."""
+    torch.manual_seed(22)
+    net = nn.Linear(12, 5)
+    x, y = torch.randn(16, 12), torch.randint(0, 5, (16,))
+    gs = per_sample_grads_cpu(net, x, y, ce_sum)
+    C = float(torch.sqrt(gs["weight"].flatten(1).pow(2).sum(1) + gs["bias"].pow(2).sum(1)).median())
+    _, clip, summed = O.clip_and_accumulate([gs["weight"], gs["bias"]], C)
+    count, new_bound = O.adaclip_update(clip, C, 0.7, 0.2, 0.01, 100.0)
+    assert 0 < count < 16
+    gsm = A.GradSampleModule(copy.deepcopy(net).to(DEV), loss_reduction="mean")
+    opt = A.optimizers.AdaClipDPOptimizer(
+        torch.optim.SGD(gsm.parameters(), lr=0.1), noise_multiplier=0.0, max_grad_norm=C, expected_batch_size=16,
+        target_unclipped_quantile=0.7, clipbound_learning_rate=0.2, max_clipbound=100.0, min_clipbound=0.01,
+        unclipped_num_std=1e-4,
+    )
+    opt.zero_grad()
+    F.cross_entropy(gsm(x.to(DEV)), y.to(DEV)).backward()
+    opt.pre_step()
+    assert opt.sample_size == 16 and abs(opt.unclipped_num - count) < 1e-2
+    assert abs(opt.max_grad_norm - new_bound) < 1e-3 * new_bound
+    close(gsm._module.weight.grad, summed[0] / 16, 2e-4, 1e-7)
+    # with noise the gradient noise uses the adjusted multiplier of Theorem 1
+    opt2 = A.optimizers.AdaClipDPOptimizer(
+        torch.optim.SGD(gsm.parameters(), lr=0.1), noise_multiplier=1.0, max_grad_norm=2.0, expected_batch_size=16,
+        target_unclipped_quantile=0.5, clipbound_learning_rate=0.2, max_clipbound=100.0, min_clipbound=0.01,
+        unclipped_num_std=2.0,
+    )
+    assert abs(opt2._noise_std() - 2.0 * (1 - 1 / 16) ** -0.5) < 1e-9
+
+
 def test_noise_level(A):
     """privacy_engine_test.py:676-739: with zero gradients, after k steps sum p^2 ~ k P (sigma C lr / B)^2."""
     torch.manual_seed(8)

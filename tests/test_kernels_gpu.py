@@ -176,6 +176,36 @@ def test_clip_accumulate_many_tensors(K):
         assert_rel(o, s, FP32_REL)
 
 
+def test_per_layer_clip_factors_and_accumulate(K):
+    """[K, n] factor table: row k from parameter k's own norm and bound; bf16 and fp32 tensors,
+    fresh and accumulating, more tensors than one launch holds."""
+    torch.manual_seed(31)
+    n = 9
+    gs = [torch.randn(n, 5, 7), torch.randn(n, 33) * 3, torch.randn(n, 4, 2, 2) * 0.01]
+    bounds = [0.5, 2.0, 1.0]
+    want_clip, want = O.per_layer_clip_and_accumulate([g.double() for g in gs], bounds)
+    dgs = [dev(g) for g in gs]
+    clip = K.clip_factor_per_layer(K.sumsq_rows(dgs), bounds)
+    assert clip.shape == (3, n)
+    assert_rel(clip, torch.stack(want_clip), FP32_REL, "per-layer factors")
+    outs = [torch.empty(g.shape[1:], device="cuda") for g in gs]
+    K.clip_accumulate(dgs, clip, outs, accumulate=False)
+    K.clip_accumulate(dgs, clip, outs, accumulate=True)
+    for o, w in zip(outs, want):
+        assert_rel(o, 2 * w, FP32_REL, "per-layer clipped sum, accumulated once")
+    norms_in = K.clip_factor_per_layer(K.sumsq_rows(dgs).sqrt(), bounds, is_norm=True)
+    assert torch.equal(norms_in, clip) or (norms_in - clip).abs().max() < 1e-6
+    many = [torch.randn(4, 6) * (k + 1) for k in range(50)]
+    mb = [0.1 * (k + 1) for k in range(50)]
+    _, mwant = O.per_layer_clip_and_accumulate([g.double() for g in many], mb)
+    dm = [dev(g) for g in many]
+    mclip = K.clip_factor_per_layer(K.sumsq_rows(dm), mb)
+    mouts = [torch.empty(6, device="cuda") for _ in many]
+    K.clip_accumulate(dm, mclip, mouts, accumulate=False)
+    for o, w in zip(mouts, mwant):
+        assert_rel(o, w, FP32_REL)
+
+
 # ---- Noise ---------------------------------------------------------------------------
 def test_add_noise_zero_std_is_exact(K):
     torch.manual_seed(5)

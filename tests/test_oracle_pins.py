@@ -269,6 +269,41 @@ def test_clip_empty_batch():
     assert clip.shape == (0,) and summed[0].shape == (3, 2) and summed[0].abs().sum() == 0
 
 
+def test_per_layer_clipping_reduces_to_flat_clipping_and_bounds_every_layer():
+    """What the mathematics fixes for perlayeroptimizer.py:58-76: with a single parameter it is flat
+    clipping; with huge bounds the plain sum; with tiny bounds every parameter's clipped sample
+    has norm C_k exactly, so a batch of one gives sums of norms C_k."""
+    torch.manual_seed(12)
+    g1, g2 = torch.randn(5, 3, 4, dtype=torch.float64), torch.randn(5, 6, dtype=torch.float64)
+    _, _, flat = O.clip_and_accumulate([g1], 0.5)
+    clips, summed = O.per_layer_clip_and_accumulate([g1], [0.5])
+    torch.testing.assert_close(summed[0], flat[0])
+    clips, summed = O.per_layer_clip_and_accumulate([g1, g2], [1e9, 1e9])
+    assert all((c == 1).all() for c in clips)
+    torch.testing.assert_close(summed[0], g1.sum(0))
+    torch.testing.assert_close(summed[1], g2.sum(0))
+    clips, summed = O.per_layer_clip_and_accumulate([g1[:1], g2[:1]], [0.3, 0.02])
+    assert math.isclose(summed[0].norm().item(), 0.3, rel_tol=1e-5)
+    assert math.isclose(summed[1].norm().item(), 0.02, rel_tol=1e-4)
+    # the layers do not see each other: scaling one leaves the other's factors alone
+    c_a, _ = O.per_layer_clip_and_accumulate([g1, g2], [0.5, 0.5])
+    c_b, _ = O.per_layer_clip_and_accumulate([g1 * 100, g2], [0.5, 0.5])
+    torch.testing.assert_close(c_a[1], c_b[1])
+
+
+def test_adaclip_update_moves_towards_the_target_quantile():
+    """adaclipoptimizer.py:119-121, 181-194 on hand-checked numbers."""
+    clip = torch.tensor([1.0, 1.0, 0.5, 0.25])  # two of four unclipped
+    count, new = O.adaclip_update(clip, 2.0, target_quantile=0.5, learning_rate=0.3, min_bound=0.1, max_bound=10.0)
+    assert count == 2.0 and new == 2.0  # at the target: no change
+    count, new = O.adaclip_update(clip, 2.0, 0.75, 0.3, 0.1, 10.0)
+    assert math.isclose(new, 2.0 * math.exp(0.3 * 0.25))  # too few unclipped: the bound grows
+    count, new = O.adaclip_update(torch.ones(4), 2.0, 0.5, 0.3, 0.1, 10.0)
+    assert count == 4.0 and math.isclose(new, 2.0 * math.exp(-0.15))
+    assert O.adaclip_update(torch.zeros(4), 9.0, 0.9, 5.0, 0.1, 10.0)[1] == 10.0
+    assert O.adaclip_update(torch.ones(4), 0.11, 0.0, 5.0, 0.1, 10.0)[1] == 0.1
+
+
 def test_clipping_coef_from_norm_samples():
     ns = [torch.tensor([3.0, 0.0, 0.3]), torch.tensor([4.0, 0.0, 0.4])]
     torch.testing.assert_close(O.per_sample_norm(ns), torch.tensor([5.0, 0.0, 0.5]))
