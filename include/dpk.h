@@ -154,7 +154,8 @@ int dpk_embedding_ghost_norm(const int64_t* ids, const void* b, int dtype, float
 
 /* ------------------------------------------------------------------------- *
  * Normalisation layers with an affine weight
- * replaces opacus/grad_sample/group_norm.py:26-47 and rms_norm.py:27-47
+ * replaces opacus/grad_sample/group_norm.py:26-47, rms_norm.py:27-47,
+ * layer_norm.py:27-52 and instance_norm.py:30-56
  * ------------------------------------------------------------------------- */
 
 /* gs_w[n,c] = scale * sum_s group_norm(x)[n,c,s] * b[n,c,s]   (group_norm.py:43-44)
@@ -171,6 +172,18 @@ size_t dpk_rms_norm_gs_workspace_bytes(int64_t n, int64_t T, int64_t D);
 int dpk_rms_norm_gs(const void* x, const void* b, int in_dtype, void* gs_w, int gs_dtype,
                     int64_t n, int64_t T, int64_t D, float eps, float scale, void* ws,
                     size_t ws_bytes, dpk_stream_t stream);
+
+/* gs_w[n,d] = scale * sum_t layer_norm(x)[n,t,d] * b[n,t,d]   (layer_norm.py:41-47)
+ * gs_b[n,d] = scale * sum_t b[n,t,d]                          (layer_norm.py:49)
+ * x, b: [n,T,D], D = number of normalised elements (the product of
+ * normalized_shape), T = everything between the batch and those dimensions.
+ * Normalisation without affine: (x - mean) * rsqrt(var + eps), biased variance.
+ * Either output may be NULL. (InstanceNorm, instance_norm.py:50-55, is
+ * dpk_group_norm_gs with groups == C.) */
+size_t dpk_layer_norm_gs_workspace_bytes(int64_t n, int64_t T, int64_t D);
+int dpk_layer_norm_gs(const void* x, const void* b, int in_dtype, void* gs_w, void* gs_b,
+                      int gs_dtype, int64_t n, int64_t T, int64_t D, float eps, float scale,
+                      void* ws, size_t ws_bytes, dpk_stream_t stream);
 
 /* ------------------------------------------------------------------------- *
  * DPOptimizer.clip_and_accumulate, add_noise, scale_grad

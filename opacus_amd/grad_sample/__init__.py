@@ -20,6 +20,8 @@ from .utils import (
 from .conv import compute_conv_grad_sample  # noqa: E402
 from .embedding import compute_embedding_grad_sample, compute_embedding_norm_sample  # noqa: E402
 from .group_norm import compute_group_norm_grad_sample  # noqa: E402
+from .instance_norm import compute_instance_norm_grad_sample  # noqa: E402
+from .layer_norm import compute_layer_norm_grad_sample  # noqa: E402
 from .linear import compute_linear_grad_sample, compute_linear_norm_sample  # noqa: E402
 from .rms_norm import compute_rms_norm_grad_sample  # noqa: E402
 

@@ -400,6 +400,40 @@ def rms_norm_grad_sample(
     return gw
 
 
+def layer_norm_grad_sample(
+    x: torch.Tensor,
+    backprops: torch.Tensor,
+    normalized_numel: int,
+    eps: float,
+    scale: float = 1.0,
+    want_weight: bool = True,
+    want_bias: bool = True,
+) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
+    """Per-sample gradients ``[n, D]`` of LayerNorm's weight and bias (``D = normalized_numel``)."""
+    dev = _need_gpu(x, backprops)
+    if x.dtype != backprops.dtype:
+        x = x.to(backprops.dtype)
+    n, D = x.shape[0], normalized_numel
+    gw = torch.empty((n, D), dtype=backprops.dtype, device=dev) if want_weight else None
+    gb = torch.empty((n, D), dtype=backprops.dtype, device=dev) if want_bias else None
+    if n == 0 or not (want_weight or want_bias):
+        return gw, gb
+    xd = _dense(x).reshape(n, -1, D)
+    bd = _dense(backprops).reshape(n, -1, D)
+    T = xd.shape[1]
+    L = lib()
+    ws, wsb = _ws(L.dpk_layer_norm_gs_workspace_bytes(n, T, D), dev)
+    with _timed("layer_norm_gs", dev):
+        check(
+            "dpk_layer_norm_gs",
+            L.dpk_layer_norm_gs(
+                _ptr(xd), _ptr(bd), _code(bd), _ptr(gw), _ptr(gb), _code(bd), n, T, D, float(eps), float(scale),
+                _ptr(ws), wsb, _stream(dev),
+            ),
+        )
+    return gw, gb
+
+
 # ---- optimizer: norms, clip factor, clip-weighted sum, noise ---------------------------
 def _flat2d(gs: torch.Tensor) -> torch.Tensor:
     g = _dense(gs)

@@ -7,7 +7,7 @@ timed as the CPU baseline. Nothing in the ``opacus_amd`` package imports it; onl
 tests, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` do.
 
 What pins each function (see ``tests/test_oracle_pins.py``):
-  * linear/conv/embedding/norm-layer grad samples: batch-of-one autograd (the
+  * linear/conv/embedding/norm-layer (Group, RMS, Layer, Instance) grad samples: batch-of-one autograd (the
     reference's own microbatch method, opacus/utils/per_sample_gradients_utils.py:96-167)
     and the invariant sum_n gs[n] == autograd's .grad for a sum loss;
   * unfold2d: exact equality with torch.nn.functional.unfold
@@ -245,6 +245,25 @@ def group_norm_grad_sample(
     gs_w = torch.einsum("ni...->ni", F.group_norm(x, num_groups, eps=eps) * backprops)
     gs_b = torch.einsum("ni...->ni", backprops)
     return gs_w, gs_b
+
+
+def layer_norm_grad_sample(
+    x: torch.Tensor, backprops: torch.Tensor, normalized_shape: Sequence[int], eps: float
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """opacus/grad_sample/layer_norm.py:41-50: ``layer_norm(x) * b`` and ``b`` summed over all but
+    the batch and the normalised dimensions."""
+    k = len(normalized_shape)
+    prod = F.layer_norm(x, tuple(normalized_shape), eps=eps) * backprops
+    if prod.dim() == k + 1:
+        return prod, backprops
+    dims = list(range(1, prod.dim() - k))
+    return prod.sum(dim=dims), backprops.sum(dim=dims)
+
+
+def instance_norm_grad_sample(x: torch.Tensor, backprops: torch.Tensor, eps: float) -> Tuple[torch.Tensor, torch.Tensor]:
+    """opacus/grad_sample/instance_norm.py:50-55: ``instance_norm(x) * b`` and ``b`` summed over
+    the spatial dimensions."""
+    return torch.einsum("ni...->ni", F.instance_norm(x, eps=eps) * backprops), torch.einsum("ni...->ni", backprops)
 
 
 def rms_norm_grad_sample(

@@ -30,6 +30,7 @@ def test_header_declares_the_expected_surface():
         "dpk_embedding_unique_pairs",
         "dpk_group_norm_gs",
         "dpk_rms_norm_gs",
+        "dpk_layer_norm_gs",
         "dpk_sumsq_rows",
         "dpk_clip_factor",
         "dpk_clip_accumulate",

@@ -168,6 +168,37 @@ def test_res_block_grad_samples(A):
         assert (p.grad_sample.cpu() - want[k]).abs().max() <= 5e-5 * want[k].abs().max(), k
 
 
+def test_layer_norm_and_instance_norm_grad_samples(A):
+    """LayerNorm and InstanceNorm have kernels of their own (no functorch fallback): per-sample
+    gradients against batch-of-one autograd, as tests/grad_samples/layer_norm_test.py and
+    instance_norm2d_test.py do."""
+
+    class Net(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.conv = nn.Conv2d(3, 6, 3, padding=1)
+            self.inorm = nn.InstanceNorm2d(6, affine=True)
+            self.ln = nn.LayerNorm([6, 5, 5])
+            self.fc = nn.Linear(150, 4)
+
+        def forward(self, x):
+            return self.fc(self.ln(F.relu(self.inorm(self.conv(x)))).flatten(1))
+
+    torch.manual_seed(5)
+    net = Net()
+    n = 6
+    x, y = torch.randn(n, 3, 5, 5), torch.randint(0, 4, (n,))
+    want = per_sample_grads_cpu(net, x, y, ce_sum)
+    gsm = A.GradSampleModule(copy.deepcopy(net).to(DEV), loss_reduction="mean")
+    from opacus_amd.grad_sample import GradSampleHooks
+
+    assert nn.LayerNorm in GradSampleHooks.GRAD_SAMPLERS and nn.InstanceNorm2d in GradSampleHooks.GRAD_SAMPLERS
+    F.cross_entropy(gsm(x.to(DEV)), y.to(DEV)).backward()
+    for k, p in gsm._module.named_parameters():
+        assert p.grad_sample.shape == (n, *p.shape), k
+        close(p.grad_sample, want[k], 1e-3, 1e-5, k)
+
+
 @pytest.mark.parametrize("batch_first", [True, False])
 def test_sequence_model_grad_samples(A, batch_first):
     """Embedding -> Linear over [batch, seq]; also with the batch in dimension 1."""

@@ -513,6 +513,43 @@ def test_rms_norm_grad_sample_f32(K, shape, D):
     assert_rel(got, want, FP32_REL, "rms weight")
 
 
+@pytest.mark.parametrize(
+    "shape,D",
+    [
+        ((4, 8), 8),
+        ((3, 5, 12), 12),
+        ((2, 3, 4, 6), 24),  # two normalised dimensions
+        ((2, 130, 33), 33),
+        ((2, 37, 256), 256),  # one-pass kernel
+        ((3, 9, 768), 768),
+        ((2, 70, 1024), 1024),
+        ((5, 2, 512), 512),
+    ],
+)
+@pytest.mark.parametrize("scale", [1.0, 2.0])
+def test_layer_norm_grad_sample_f32(K, shape, D, scale):
+    torch.manual_seed(D + 1)
+    x = torch.randn(*shape) * 1.5 + 0.7
+    b = torch.randn(*shape)
+    nshape = shape[-2:] if D == 24 else shape[-1:]
+    want_w, want_b = O.layer_norm_grad_sample(x.double(), (b * scale).double(), nshape, 1e-5)
+    gw, gb = K.layer_norm_grad_sample(dev(x), dev(b), D, 1e-5, scale=scale)
+    assert_rel(gw, want_w.reshape(shape[0], D), FP32_REL, "ln weight")
+    assert_rel(gb, want_b.reshape(shape[0], D), FP32_REL, "ln bias")
+    only_w, none_b = K.layer_norm_grad_sample(dev(x), dev(b), D, 1e-5, scale=scale, want_bias=False)
+    assert none_b is None
+    assert_rel(only_w, want_w.reshape(shape[0], D), FP32_REL, "ln weight alone")
+
+
+def test_instance_norm_is_group_norm_with_one_channel_per_group(K):
+    torch.manual_seed(41)
+    x, b = torch.randn(3, 5, 6, 8) + 0.3, torch.randn(3, 5, 6, 8)
+    want_w, want_b = O.instance_norm_grad_sample(x.double(), b.double(), 1e-5)
+    gw, gb = K.group_norm_grad_sample(dev(x), dev(b), 5, 1e-5)
+    assert_rel(gw, want_w, FP32_REL)
+    assert_rel(gb, want_b, FP32_REL)
+
+
 def test_norm_layers_bf16(K):
     torch.manual_seed(3)
     x = torch.randn(2, 70, 64).bfloat16()
@@ -522,6 +559,11 @@ def test_norm_layers_bf16(K):
     x, b = torch.randn(3, 50, 1024).bfloat16(), torch.randn(3, 50, 1024).bfloat16()  # one-pass kernel
     want = O.rms_norm_grad_sample(x.double(), b.double(), (1024,), 1e-6)
     assert_rel(K.rms_norm_grad_sample(dev(x), dev(b), 1024, 1e-6), want, BF16_REL)
+    x, b = torch.randn(3, 50, 512).bfloat16(), torch.randn(3, 50, 512).bfloat16()
+    want_w, want_b = O.layer_norm_grad_sample(x.double(), b.double(), (512,), 1e-5)
+    gw, gb = K.layer_norm_grad_sample(dev(x), dev(b), 512, 1e-5)
+    assert_rel(gw, want_w, BF16_REL)
+    assert_rel(gb, want_b, BF16_REL)
     x4, b4 = torch.randn(2, 8, 6, 6).bfloat16(), torch.randn(2, 8, 6, 6).bfloat16()
     want_w, want_b = O.group_norm_grad_sample(x4.double(), b4.double(), 4, 1e-5)
     gw, gb = K.group_norm_grad_sample(dev(x4), dev(b4), 4, 1e-5)

@@ -234,6 +234,39 @@ def test_rms_norm_grad_sample_vs_microbatch(shape):
     torch.testing.assert_close(gs_w, want["weight"], rtol=1e-10, atol=1e-10)
 
 
+@pytest.mark.parametrize("shape,normalized", [((4, 8), (8,)), ((3, 5, 8), (8,)), ((2, 3, 4, 6), (4, 6))])
+def test_layer_norm_grad_sample_vs_microbatch(shape, normalized):
+    torch.manual_seed(13)
+    ln = nn.LayerNorm(normalized, eps=1e-4).double()
+    ln.weight.data.normal_()
+    ln.bias.data.normal_()
+    x = torch.randn(*shape, dtype=torch.float64) * 2 + 1
+    loss = lambda y: y.pow(3).sum()  # noqa: E731
+    b = _backprops(ln, x, loss)
+    gs_w, gs_b = O.layer_norm_grad_sample(x, b, normalized, 1e-4)
+    want = _per_sample_autograd(ln, x, loss)
+    torch.testing.assert_close(gs_w, want["weight"], rtol=1e-10, atol=1e-10)
+    torch.testing.assert_close(gs_b, want["bias"], rtol=1e-10, atol=1e-10)
+
+
+@pytest.mark.parametrize("cls,shape", [(nn.InstanceNorm1d, (3, 4, 7)), (nn.InstanceNorm2d, (2, 3, 4, 5))])
+def test_instance_norm_grad_sample_vs_microbatch(cls, shape):
+    torch.manual_seed(14)
+    inorm = cls(shape[1], eps=1e-3, affine=True).double()
+    inorm.weight.data.normal_()
+    inorm.bias.data.normal_()
+    x = torch.randn(*shape, dtype=torch.float64) + 0.5
+    loss = lambda y: y.pow(2).sum()  # noqa: E731
+    b = _backprops(inorm, x, loss)
+    gs_w, gs_b = O.instance_norm_grad_sample(x, b, 1e-3)
+    want = _per_sample_autograd(inorm, x, loss)
+    torch.testing.assert_close(gs_w, want["weight"], rtol=1e-10, atol=1e-10)
+    torch.testing.assert_close(gs_b, want["bias"], rtol=1e-10, atol=1e-10)
+    # and it is group normalisation with one channel per group
+    gw2, gb2 = O.group_norm_grad_sample(x, b, shape[1], 1e-3)
+    torch.testing.assert_close(gs_w, gw2, rtol=1e-12, atol=1e-12)
+
+
 # ---- Clipping -------------------------------------------------------------------------
 def test_clip_and_accumulate_closed_form():
     torch.manual_seed(10)
