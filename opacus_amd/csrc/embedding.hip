@@ -54,51 +54,54 @@ size_t ws_layout(int64_t n, int64_t T, int64_t D, void* ws, EmbWs* out) {
   return off;
 }
 
-// grid = n * ceil(T / 256); thread <-> one position t of one sample. Every thread
-// scans the sample's whole id row, staged through LDS a tile at a time (all lanes
-// read the same address: a broadcast). The scan is branch-free so that the reads of
-// an unrolled stretch are in flight together. Positions left of the block's own
-// stretch [t0, t1) can only be earlier occurrences and positions right of it only
-// later ones, which leaves one compare and one or two selects per id there.
+// grid = n * ceil(T / 64); a block owns 64 consecutive positions t of one sample, lane
+// <-> position, and its four waves each scan a quarter of every LDS-staged tile of the
+// sample's id row (all lanes of a wave read the same address: a broadcast). The scan is
+// branch-free so that the reads of an unrolled stretch are in flight together; the
+// waves' findings (seen before? nearest later occurrence) meet in LDS.
+constexpr int kLinkPositions = DPK_WAVE;
+
 __global__ __launch_bounds__(kThreads) void emb_link_kernel(const int64_t* __restrict__ ids,
                                                              int64_t T, int64_t V, int blocks_per_sample,
                                                              int32_t* __restrict__ next,
                                                              int32_t* __restrict__ leader,
                                                              int32_t* __restrict__ flag) {
   __shared__ int64_t tile[kIdTile];
+  __shared__ int32_t w_before[kWaves][kLinkPositions], w_next[kWaves][kLinkPositions];
   const int64_t sample = blockIdx.x / blocks_per_sample;
   const int32_t Ti = static_cast<int32_t>(T);
-  const int32_t t0 = static_cast<int32_t>(blockIdx.x % blocks_per_sample) * kThreads;
-  const int32_t t1 = t0 + kThreads < Ti ? t0 + kThreads : Ti;
-  const int32_t t = t0 + threadIdx.x;
+  const int lane = threadIdx.x & (DPK_WAVE - 1), wave = threadIdx.x / DPK_WAVE;
+  const int32_t t = static_cast<int32_t>(blockIdx.x % blocks_per_sample) * kLinkPositions + lane;
   const int64_t* row = ids + sample * T;
   const bool live = t < Ti;
   const int64_t mine = live ? row[t] : 0;
-  bool before = false;  // an earlier position holds the same id
-  int32_t nxt = Ti;     // first later position with the same id
+  int32_t before = 0;  // an earlier position holds the same id
+  int32_t nxt = Ti;    // first later position with the same id
   for (int32_t c0 = 0; c0 < Ti; c0 += kIdTile) {
     const int32_t c1 = c0 + kIdTile < Ti ? c0 + kIdTile : Ti;
     __syncthreads();
     for (int32_t i = c0 + threadIdx.x; i < c1; i += kThreads) tile[i - c0] = row[i];
     __syncthreads();
-    const int32_t lo = t0 < c1 ? (t0 > c0 ? t0 : c0) : c1;  // [c0, lo): left of the block's stretch
-    const int32_t hi = t1 > c0 ? (t1 < c1 ? t1 : c1) : c0;  // [hi, c1): right of it
+    const int32_t quarter = (c1 - c0 + kWaves - 1) / kWaves;
+    const int32_t u0 = c0 + wave * quarter;
+    const int32_t u1 = u0 + quarter < c1 ? u0 + quarter : c1;
 #pragma unroll 8
-    for (int32_t u = c0; u < lo; ++u) before |= tile[u - c0] == mine;
-#pragma unroll 8
-    for (int32_t u = lo; u < hi; ++u) {
+    for (int32_t u = u0; u < u1; ++u) {
       const bool eq = tile[u - c0] == mine;
-      before |= eq && u < t;
+      before |= (eq && u < t) ? 1 : 0;
       const int32_t cand = (eq && u > t) ? u : Ti;
       nxt = cand < nxt ? cand : nxt;
     }
-#pragma unroll 8
-    for (int32_t u = hi > lo ? hi : lo; u < c1; ++u) {
-      const int32_t cand = tile[u - c0] == mine ? u : Ti;
-      nxt = cand < nxt ? cand : nxt;
-    }
   }
-  if (live) {
+  w_before[wave][lane] = before;
+  w_next[wave][lane] = nxt;
+  __syncthreads();
+  if (wave == 0 && live) {
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) {
+      before |= w_before[w][lane];
+      nxt = w_next[w][lane] < nxt ? w_next[w][lane] : nxt;
+    }
     next[sample * T + t] = nxt < Ti ? nxt : -1;
     leader[sample * T + t] = before ? 0 : 1;
     if (V > 0 && (mine < 0 || mine >= V)) *flag = 1;
@@ -251,7 +254,7 @@ int check_common(const char* who, const int64_t* ids, int64_t n, int64_t T, int6
                  size_t ws_bytes, EmbWs* w) {
   DPK_REQUIRE(ids, DPK_E_ARG, "%s: ids is NULL", who);
   DPK_REQUIRE(dpk_aligned(ids, 8), DPK_E_ALIGN, "%s: ids misaligned", who);
-  DPK_REQUIRE(T < (1LL << 31) && n * dpk_cdiv(T, kThreads) <= DPK_MAX_GRID_X, DPK_E_SHAPE,
+  DPK_REQUIRE(T < (1LL << 31) && n * dpk_cdiv(T, kLinkPositions) <= DPK_MAX_GRID_X, DPK_E_SHAPE,
               "%s: n=%lld T=%lld too large", who, (long long)n, (long long)T);
   const size_t need = ws_layout(n, T, D, nullptr, nullptr);
   DPK_REQUIRE(ws && ws_bytes >= need, DPK_E_WORKSPACE, "%s: workspace %zu < %zu bytes", who, ws_bytes,
@@ -262,7 +265,7 @@ int check_common(const char* who, const int64_t* ids, int64_t n, int64_t T, int6
 }
 
 void launch_link(const int64_t* ids, int64_t n, int64_t T, int64_t V, const EmbWs& w, hipStream_t s) {
-  const int bps = static_cast<int>(dpk_cdiv(T, kThreads));
+  const int bps = static_cast<int>(dpk_cdiv(T, kLinkPositions));
   hipLaunchKernelGGL(zero_flag_kernel, dim3(1), dim3(1), 0, s, w.flag);
   hipLaunchKernelGGL(emb_link_kernel, dim3(static_cast<unsigned>(n * bps)), dim3(kThreads), 0, s, ids, T,
                      V, bps, w.next, w.leader, w.flag);
