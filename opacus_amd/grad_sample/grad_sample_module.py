@@ -146,13 +146,32 @@ class GradSampleHooks(AbstractGradSampleHooks):
         for module in self.iterate_submodules(self._module):
             if force_functorch or self._get_module_type(module) not in self.GRAD_SAMPLERS:
                 prepare_layer(module, batch_first=batch_first)
-            self.autograd_grad_sample_hooks.append(module.register_forward_hook(self.capture_activations_hook))
             self.autograd_grad_sample_hooks.append(
-                module.register_full_backward_hook(
-                    partial(self.capture_backprops_hook, loss_reduction=loss_reduction, batch_first=batch_first)
+                module.register_forward_hook(
+                    partial(self._forward_hook, loss_reduction=loss_reduction, batch_first=batch_first)
                 )
             )
         self.enable_hooks()
+
+    def _forward_hook(self, module: nn.Module, forward_input, forward_output, *, loss_reduction: str, batch_first: bool):
+        """Captures the activations and arranges for ``capture_backprops_hook`` to run when the
+        gradient of this call's output is known. The reference installs a full backward hook
+        on the module for that (grad_sample_module.py:215-224); a hook on the output tensor
+        delivers the same ``grad_output`` without wrapping the module's inputs and outputs in
+        an extra autograd node per call, which is what a small launch-bound model pays for
+        in every step, and it tolerates an in-place op on the output."""
+        pending = len(getattr(module, "activations", ()))
+        self.capture_activations_hook(module, forward_input, forward_output)
+        if len(getattr(module, "activations", ())) == pending:
+            return  # nothing captured: eval mode, no grad, hooks disabled, frozen module
+        out = forward_output if isinstance(forward_output, torch.Tensor) else forward_output[0]
+        if not out.requires_grad:
+            return
+
+        def on_grad_output(grad: torch.Tensor) -> None:
+            self.capture_backprops_hook(module, None, (grad,), loss_reduction=loss_reduction, batch_first=batch_first)
+
+        out.register_hook(on_grad_output)
 
     def remove_hooks(self) -> None:
         self.disable_hooks()

@@ -110,7 +110,7 @@ def test_wrapper_surface():
     gsm = GradSampleModule(net)
     assert all(k.startswith("_module.") for k in gsm.state_dict())
     assert gsm._module[0] is net[0]
-    assert len(net.autograd_grad_sample_hooks) == 4  # forward + backward hook for each Linear
+    assert len(net.autograd_grad_sample_hooks) == 2  # one forward hook per Linear; it hooks the output's gradient
     for p in net.parameters():
         assert p.grad_sample is None and p._forward_counter == 0
     with pytest.raises(ValueError, match="twice"):
@@ -152,6 +152,42 @@ def test_wrap_model_false_returns_hooks_object():
     assert isinstance(hooks, GradSampleHooks) and not isinstance(hooks, nn.Module)
     hooks.cleanup()
     assert not hasattr(net.weight, "grad_sample")
+
+
+def test_inplace_op_on_a_hooked_output_is_fine():
+    """The output-gradient hook sees the gradient with respect to the layer's own output even when
+    the next op rewrites that tensor in place (a module-level full backward hook refuses this)."""
+
+    class Net(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.fc = Tmp(3, 4)
+
+        def forward(self, x):
+            return torch.relu_(self.fc(x))
+
+    class Tmp(nn.Linear):
+        pass
+
+    seen = {}
+
+    def sampler(layer, activations, backprops):
+        seen["b"] = backprops.clone()
+        return {layer.weight: torch.einsum("ni,nj->nij", backprops, activations[0]), layer.bias: backprops.clone()}
+
+    register_grad_sampler(Tmp)(sampler)
+    try:
+        torch.manual_seed(0)
+        net = Net()
+        x = torch.randn(5, 3)
+        gsm = GradSampleModule(net, loss_reduction="sum")
+        out = gsm(x)
+        out.sum().backward()
+        want = (net.fc(x) > 0).float()  # d relu(y).sum() / dy
+        assert torch.equal(seen["b"], want)
+        torch.testing.assert_close(net.fc.weight.grad_sample.sum(0), net.fc.weight.grad)
+    finally:
+        GradSampleHooks.GRAD_SAMPLERS.pop(Tmp, None)
 
 
 def test_no_capture_in_eval_or_no_grad_or_disabled():
