@@ -146,6 +146,18 @@ int dpk_embedding_gs(const int64_t* ids, const void* b, int in_dtype, void* gs, 
                      int64_t n, int64_t T, int64_t V, int64_t D, float scale, void* ws,
                      size_t ws_bytes, dpk_stream_t stream);
 
+/* nn.EmbeddingBag (embedding.py:67-94): bag i = index[offsets[i] : offsets[i+1]] (the
+ * last one runs to L); gs[i, index[j], :] = scale * b[i,:] for every j of bag i, divided
+ * by the bag length when `mean` != 0. An index that occurs several times in a bag still
+ * receives b[i,:] once, as the reference's indexed "+=" leaves it. gs: [bags,V,D], fully
+ * written, 16-byte aligned. Indices outside [0,V) or offsets that are not ascending in
+ * [0,L] make the call fail with DPK_E_ARG after a device-side check (this entry point
+ * waits for the stream). Workspace: dpk_embedding_bag_workspace_bytes(). */
+size_t dpk_embedding_bag_workspace_bytes(void);
+int dpk_embedding_bag_gs(const int64_t* index, const int64_t* offsets, const void* b, int in_dtype,
+                         void* gs, int gs_dtype, int64_t bags, int64_t L, int64_t V, int64_t D,
+                         int mean, float scale, void* ws, size_t ws_bytes, dpk_stream_t stream);
+
 /* norm[n] = sqrt(sum_{v} || scale * sum_{t : ids[n,t]==v} b[n,t,:] ||^2)
  * (embedding_norm_sample.py:131-150). fp32 output. */
 int dpk_embedding_ghost_norm(const int64_t* ids, const void* b, int dtype, float* norm, int64_t n,

@@ -250,6 +250,52 @@ __global__ __launch_bounds__(kThreads) void zero_fill_kernel(uint4* __restrict__
 
 __global__ void zero_flag_kernel(int32_t* flag) { *flag = 0; }
 
+// ---- EmbeddingBag ---------------------------------------------------------------
+// flag |= 1 when an index lies outside [0, V), an offset outside [0, L] or the
+// offsets decrease.
+__global__ __launch_bounds__(kThreads) void bag_check_kernel(const int64_t* __restrict__ index,
+                                                              const int64_t* __restrict__ offsets,
+                                                              int64_t L, int64_t nbags, int64_t V,
+                                                              int32_t* __restrict__ flag) {
+  const int64_t j = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  bool bad = false;
+  if (j < L) bad = index[j] < 0 || index[j] >= V;
+  if (j < nbags) {
+    const int64_t o = offsets[j];
+    bad = bad || o < 0 || o > L || (j + 1 < nbags && offsets[j + 1] < o);
+  }
+  if (bad) *flag = 1;
+}
+
+// One block per position j of the flat index list: finds the bag i that holds j
+// (last i with offsets[i] <= j) and writes b[i,:] (divided by the bag length in mean
+// mode) to gs[i, index[j], :]. Positions of one bag that repeat an index write the
+// same values to the same row, so the row holds b[i,:] once however often the index
+// occurs: the result of the reference's indexed "+=" (embedding.py:84-87).
+template <typename TIN, typename TOUT>
+__global__ __launch_bounds__(kThreads) void bag_scatter_kernel(
+    const int64_t* __restrict__ index, const int64_t* __restrict__ offsets, const TIN* __restrict__ b,
+    TOUT* __restrict__ gs, int64_t L, int64_t nbags, int64_t V, int64_t D, int mean, float scale) {
+  const int64_t j = blockIdx.x;
+  int64_t lo = 0, hi = nbags - 1;
+  if (offsets[0] > j) return;  // before the first bag: belongs to none
+  while (lo < hi) {
+    const int64_t mid = (lo + hi + 1) >> 1;
+    if (offsets[mid] <= j) lo = mid;
+    else hi = mid - 1;
+  }
+  const int64_t bag = lo;
+  const int64_t end = bag + 1 < nbags ? offsets[bag + 1] : L;
+  const float len = static_cast<float>(end - offsets[bag]);
+  const TIN* src = b + bag * D;
+  TOUT* dst = gs + (bag * V + index[j]) * D;
+  for (int64_t d = threadIdx.x; d < D; d += kThreads) {
+    float v = dpk_io<TIN>::load(src + d) * scale;
+    if (mean) v = v / len;
+    dpk_io<TOUT>::store(dst + d, v);
+  }
+}
+
 int check_common(const char* who, const int64_t* ids, int64_t n, int64_t T, int64_t D, void* ws,
                  size_t ws_bytes, EmbWs* w) {
   DPK_REQUIRE(ids, DPK_E_ARG, "%s: ids is NULL", who);
@@ -388,5 +434,59 @@ extern "C" int dpk_embedding_gs(const int64_t* ids, const void* b, int in_dtype,
   if (in_dtype == DPK_F32) launch_walk<float, float, 1>(vec, ids, b, w, n, T, D, V, scale, gs, s);
   else launch_walk<bf16_t, bf16_t, 1>(vec, ids, b, w, n, T, D, V, scale, gs, s);
   DPK_LAUNCH_CHECK(who);
+  return DPK_OK;
+}
+
+extern "C" size_t dpk_embedding_bag_workspace_bytes(void) { return 256; }
+
+extern "C" int dpk_embedding_bag_gs(const int64_t* index, const int64_t* offsets, const void* b,
+                                    int in_dtype, void* gs, int gs_dtype, int64_t nbags, int64_t L,
+                                    int64_t V, int64_t D, int mean, float scale, void* ws,
+                                    size_t ws_bytes, dpk_stream_t stream) {
+  const char* who = "dpk_embedding_bag_gs";
+  DPK_REQUIRE(nbags >= 0 && L >= 0 && V >= 1 && D >= 1, DPK_E_SHAPE, "%s: bags=%lld L=%lld V=%lld D=%lld",
+              who, (long long)nbags, (long long)L, (long long)V, (long long)D);
+  if (nbags == 0) return DPK_OK;
+  DPK_REQUIRE(offsets && b && gs && (index || L == 0), DPK_E_ARG, "%s: NULL tensor", who);
+  DPK_REQUIRE(dpk_dtype_ok(in_dtype) && in_dtype == gs_dtype, DPK_E_DTYPE,
+              "%s: dtypes %d,%d (must be equal)", who, in_dtype, gs_dtype);
+  DPK_REQUIRE(dpk_aligned(index, 8) && dpk_aligned(offsets, 8) && dpk_aligned(b, dpk_elsize(in_dtype)) &&
+                  dpk_aligned(gs, 16),
+              DPK_E_ALIGN, "%s: misaligned tensor (gs needs 16 bytes)", who);
+  DPK_REQUIRE(ws && ws_bytes >= 4 && dpk_aligned(ws, 4), DPK_E_WORKSPACE, "%s: workspace of 4 bytes needed", who);
+  DPK_REQUIRE(L <= DPK_MAX_GRID_X && nbags <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: too many positions", who);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  int32_t* dflag = static_cast<int32_t*>(ws);
+  hipLaunchKernelGGL(zero_flag_kernel, dim3(1), dim3(1), 0, s, dflag);
+  const int64_t most = L > nbags ? L : nbags;
+  hipLaunchKernelGGL(bag_check_kernel, dim3(static_cast<unsigned>(dpk_cdiv(most, kThreads))), dim3(kThreads), 0,
+                     s, index, offsets, L, nbags, V, dflag);
+  DPK_LAUNCH_CHECK(who);
+  // Bad indices would address memory outside gs: find out before writing.
+  int32_t flag = 0;
+  hipError_t e = hipMemcpyAsync(&flag, dflag, sizeof(flag), hipMemcpyDeviceToHost, s);
+  if (e == hipSuccess) e = hipStreamSynchronize(s);
+  DPK_REQUIRE(e == hipSuccess, DPK_E_LAUNCH, "%s: %s", who, hipGetErrorString(e));
+  DPK_REQUIRE(flag == 0, DPK_E_ARG, "%s: an index lies outside [0, %lld) or the offsets are not ascending in [0, %lld]",
+              who, (long long)V, (long long)L);
+  const size_t bytes = static_cast<size_t>(nbags) * V * D * dpk_elsize(gs_dtype);
+  const int64_t n16 = static_cast<int64_t>(bytes / 16);
+  const int64_t ntail = static_cast<int64_t>(bytes - static_cast<size_t>(n16) * 16);
+  int64_t blocks = dpk_cdiv(n16 > 0 ? n16 : 1, kThreads * 4);
+  if (blocks > 65536) blocks = 65536;
+  hipLaunchKernelGGL(zero_fill_kernel, dim3(static_cast<unsigned>(blocks)), dim3(kThreads), 0, s,
+                     static_cast<uint4*>(gs), n16, static_cast<unsigned char*>(gs) + static_cast<size_t>(n16) * 16,
+                     ntail);
+  DPK_LAUNCH_CHECK(who);
+  if (L > 0) {
+    const dim3 grid(static_cast<unsigned>(L)), block(kThreads);
+    if (in_dtype == DPK_F32)
+      hipLaunchKernelGGL((bag_scatter_kernel<float, float>), grid, block, 0, s, index, offsets,
+                         static_cast<const float*>(b), static_cast<float*>(gs), L, nbags, V, D, mean, scale);
+    else
+      hipLaunchKernelGGL((bag_scatter_kernel<bf16_t, bf16_t>), grid, block, 0, s, index, offsets,
+                         static_cast<const bf16_t*>(b), static_cast<bf16_t*>(gs), L, nbags, V, D, mean, scale);
+    DPK_LAUNCH_CHECK(who);
+  }
   return DPK_OK;
 }

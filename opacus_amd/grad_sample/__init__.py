@@ -18,7 +18,11 @@ from .utils import (
     wrap_model,
 )
 from .conv import compute_conv_grad_sample  # noqa: E402
-from .embedding import compute_embedding_grad_sample, compute_embedding_norm_sample  # noqa: E402
+from .embedding import (  # noqa: E402
+    compute_embedding_grad_sample,
+    compute_embedding_norm_sample,
+    compute_embeddingbag_gradsampler,
+)
 from .group_norm import compute_group_norm_grad_sample  # noqa: E402
 from .instance_norm import compute_instance_norm_grad_sample  # noqa: E402
 from .layer_norm import compute_layer_norm_grad_sample  # noqa: E402

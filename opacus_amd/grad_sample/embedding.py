@@ -32,6 +32,29 @@ def compute_embedding_grad_sample(
     return ret
 
 
+@register_grad_sampler(nn.EmbeddingBag)
+@owns_output
+@fused_scale
+def compute_embeddingbag_gradsampler(
+    layer: nn.EmbeddingBag, activations: List[torch.Tensor], backprops: torch.Tensor, scale: float = 1.0
+) -> Dict[nn.Parameter, torch.Tensor]:
+    """Per-sample gradient ``[bags, num_embeddings, dim]`` (embedding.py:67-94): every index of
+    bag ``i`` receives ``backprops[i]`` (divided by the bag length for ``mode="mean"``); an index
+    repeated inside a bag receives it once, ``per_sample_weights`` and ``padding_idx`` are not
+    looked at - all as in the reference. A 2-D index tensor without offsets is one bag per row."""
+    if not layer.weight.requires_grad:
+        return {}
+    index = activations[0]
+    if len(activations) > 1 and activations[1] is not None:
+        offsets = activations[1]
+    elif index.dim() == 2:
+        offsets = torch.arange(0, index.numel(), index.shape[1], device=index.device, dtype=torch.int64)
+    else:
+        raise ValueError("EmbeddingBag needs offsets for a 1-D index tensor")
+    gs = kernels.embedding_bag_grad_sample(index, offsets, backprops, layer.num_embeddings, mode=layer.mode, scale=scale)
+    return {layer.weight: gs}
+
+
 @register_norm_sampler(nn.Embedding)
 @fused_scale
 def compute_embedding_norm_sample(

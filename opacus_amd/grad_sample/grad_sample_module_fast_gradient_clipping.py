@@ -114,7 +114,8 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
             return
         if not hasattr(module, "activations"):
             module.activations = []
-        module.activations.append([t.detach() for t in forward_input])
+        # non-tensor inputs (an omitted optional argument passed as None) are not activations
+        module.activations.append([t.detach() for t in forward_input if isinstance(t, torch.Tensor)])
         for _, p in trainable_parameters(module):
             p._forward_counter += 1
             if self.use_ghost_clipping and p._forward_counter > 1 and type(module) in self.NORM_SAMPLERS:

@@ -341,6 +341,41 @@ def embedding_ghost_norm(ids: torch.Tensor, backprops: torch.Tensor, scale: floa
     return norm
 
 
+def embedding_bag_grad_sample(
+    index: torch.Tensor,
+    offsets: torch.Tensor,
+    backprops: torch.Tensor,
+    num_embeddings: int,
+    mode: str = "sum",
+    scale: float = 1.0,
+) -> torch.Tensor:
+    """Per-sample gradient ``[bags, V, D]`` of ``nn.EmbeddingBag``: every index of bag ``i``
+    receives ``backprops[i]`` (``/ len(bag)`` for ``mode="mean"``) once."""
+    dev = _need_gpu(index, offsets, backprops)
+    if mode not in ("sum", "mean"):
+        raise NotImplementedError(f"EmbeddingBag mode {mode!r}: only 'sum' and 'mean' have per-sample gradients")
+    if index.dtype != torch.int64 or offsets.dtype != torch.int64:
+        raise TypeError("EmbeddingBag indices and offsets must be int64")
+    nbags, D = offsets.shape[0], backprops.shape[-1]
+    if backprops.shape[0] != nbags:
+        raise ValueError(f"{nbags} bags but backprops of shape {tuple(backprops.shape)}")
+    idx, off, b = _dense(index).reshape(-1), _dense(offsets), _dense(backprops).reshape(nbags, D)
+    gs = torch.empty((nbags, num_embeddings, D), dtype=b.dtype, device=dev)
+    if nbags == 0:
+        return gs
+    L = lib()
+    ws, wsb = _ws(L.dpk_embedding_bag_workspace_bytes(), dev)
+    with _timed("embedding_bag_gs", dev):
+        check(
+            "dpk_embedding_bag_gs",
+            L.dpk_embedding_bag_gs(
+                _ptr(idx), _ptr(off), _ptr(b), _code(b), _ptr(gs), _code(gs), nbags, idx.numel(), num_embeddings, D,
+                int(mode == "mean"), float(scale), _ptr(ws), wsb, _stream(dev),
+            ),
+        )
+    return gs
+
+
 # ---- normalisation layers -----------------------------------------------------------
 def group_norm_grad_sample(
     x: torch.Tensor,

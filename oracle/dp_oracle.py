@@ -21,6 +21,9 @@ What pins each function (see ``tests/test_oracle_pins.py``):
   * clip_and_accumulate / add_noise / scale_grad: closed forms, batch-of-one gives a sum
     of norm C (opacus/tests/privacy_engine_test.py:302-327), C -> inf and sigma = 0
     reproduce plain SGD (:220-273);
+  * EmbeddingBag grad sample: batch-of-one autograd for bags without repeated indices
+    (with repeats the reference's indexed "+=" writes the row once; that is restated as it
+    is and checked on a hand-computed case);
   * per-layer clipping: reduces to flat clipping for one parameter, to the plain sum for
     huge bounds, and bounds every parameter's norm by its own C_k; AdaClip's count and
     bound update: hand-checked numbers;
@@ -191,6 +194,25 @@ def embedding_grad_sample(ids: torch.Tensor, backprops: torch.Tensor, num_embedd
     index = ids.unsqueeze(-1).expand(*ids.shape, D).reshape(n, -1, D)
     gs = torch.zeros(n, num_embeddings, D, dtype=backprops.dtype)
     gs.scatter_add_(1, index, backprops.reshape(n, -1, D))
+    return gs
+
+
+def embedding_bag_grad_sample(
+    index: torch.Tensor, offsets: torch.Tensor, backprops: torch.Tensor, num_embeddings: int, mode: str
+) -> torch.Tensor:
+    """opacus/grad_sample/embedding.py:67-94, loop and all: bag ``i`` is
+    ``index[offsets[i]:offsets[i+1]]`` (the last one runs to the end); its rows receive
+    ``backprops[i]`` (``/ len`` for "mean") through an indexed ``+=``, which writes a row once
+    even when the index repeats."""
+    nbags = offsets.shape[0]
+    gs = torch.zeros(nbags, num_embeddings, backprops.shape[-1], dtype=backprops.dtype)
+    for i in range(nbags):
+        begin = int(offsets[i])
+        end = int(offsets[i + 1]) if i < nbags - 1 else index.shape[0]
+        if mode == "sum":
+            gs[i][index[begin:end]] += backprops[i]
+        elif mode == "mean":
+            gs[i][index[begin:end]] += backprops[i] / (end - begin)
     return gs
 
 

@@ -199,6 +199,39 @@ def test_layer_norm_and_instance_norm_grad_samples(A):
         close(p.grad_sample, want[k], 1e-3, 1e-5, k)
 
 
+def test_embedding_bag_grad_samples(A):
+    """nn.EmbeddingBag through the wrapper, with offsets and with a 2-D index tensor; bags hold
+    distinct indices so that batch-of-one autograd is the reference."""
+
+    class Net(nn.Module):
+        def __init__(self, mode):
+            super().__init__()
+            self.bag = nn.EmbeddingBag(11, 6, mode=mode)
+            self.fc = nn.Linear(6, 3)
+
+        def forward(self, index, offsets=None):
+            return self.fc(self.bag(index, offsets))
+
+    for mode in ("sum", "mean"):
+        torch.manual_seed(6)
+        net = Net(mode)
+        index2d = torch.stack([torch.randperm(11)[:4] for _ in range(5)])
+        y = torch.randint(0, 3, (5,))
+        gsm = A.GradSampleModule(copy.deepcopy(net).to(DEV), loss_reduction="mean")
+        for flat in (False, True):
+            gsm.zero_grad()
+            if flat:
+                out = gsm(index2d.reshape(-1).to(DEV), torch.arange(0, 20, 4).to(DEV))
+            else:
+                out = gsm(index2d.to(DEV))
+            F.cross_entropy(out, y.to(DEV)).backward()
+            for i in range(5):
+                net.zero_grad()
+                F.cross_entropy(net(index2d[i : i + 1]), y[i : i + 1], reduction="sum").backward()
+                close(gsm._module.bag.weight.grad_sample[i], net.bag.weight.grad, 1e-5, 1e-7, f"{mode} bag {i}")
+                close(gsm._module.fc.weight.grad_sample[i], net.fc.weight.grad, 1e-5, 1e-7)
+
+
 @pytest.mark.parametrize("batch_first", [True, False])
 def test_sequence_model_grad_samples(A, batch_first):
     """Embedding -> Linear over [batch, seq]; also with the batch in dimension 1."""

@@ -453,6 +453,32 @@ def test_embedding_bf16(K):
     assert_rel(norm, want.flatten(1).norm(dim=1), 1e-4)
 
 
+@pytest.mark.parametrize("mode", ["sum", "mean"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embedding_bag_grad_sample_is_bit_exact(K, mode, dtype):
+    torch.manual_seed(17)
+    V, D = 23, 10
+    index = torch.randint(0, V, (40,))
+    offsets = torch.tensor([0, 5, 5, 17, 18, 39])  # an empty bag, bags with repeated indices, a bag of one
+    b = torch.randn(6, D).to(dtype)
+    for scale in (1.0, 8.0):
+        want = O.embedding_bag_grad_sample(index, offsets, (b.float() * scale).to(dtype), V, mode)
+        got = K.embedding_bag_grad_sample(dev(index), dev(offsets), dev(b), V, mode=mode, scale=scale)
+        assert got.dtype == dtype and torch.equal(got.cpu(), want), (mode, dtype, scale)
+
+
+def test_embedding_bag_bad_inputs_are_errors(K):
+    from opacus_amd._lib import DpkError
+
+    b = torch.zeros(2, 4, device="cuda")
+    with pytest.raises(DpkError, match="outside"):
+        K.embedding_bag_grad_sample(dev(torch.tensor([0, 9])), dev(torch.tensor([0, 1])), b, 9)
+    with pytest.raises(DpkError, match="ascending"):
+        K.embedding_bag_grad_sample(dev(torch.tensor([0, 1, 2])), dev(torch.tensor([2, 1])), b, 9)
+    with pytest.raises(NotImplementedError):
+        K.embedding_bag_grad_sample(dev(torch.tensor([0, 1])), dev(torch.tensor([0, 1])), b, 9, mode="max")
+
+
 def test_embedding_out_of_range_id_is_an_error(K):
     from opacus_amd._lib import DpkError
 

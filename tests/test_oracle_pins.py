@@ -206,6 +206,32 @@ def test_embedding_norm_equals_norm_of_grad_sample():
     torch.testing.assert_close(r["result_sqrt"], gs.flatten(1).norm(dim=1), rtol=1e-12, atol=1e-12)
 
 
+@pytest.mark.parametrize("mode", ["sum", "mean"])
+def test_embedding_bag_grad_sample_vs_microbatch_and_repeat_rule(mode):
+    """Bags without repeated indices: equal to batch-of-one autograd of nn.EmbeddingBag. A repeated
+    index receives the backprop once (embedding.py:84-87 uses an indexed "+="): hand-computed."""
+    torch.manual_seed(15)
+    V, D = 9, 4
+    bag = nn.EmbeddingBag(V, D, mode=mode).double()
+    index = torch.tensor([1, 4, 7, 0, 2, 3, 5, 8, 6])
+    offsets = torch.tensor([0, 3, 4, 8])  # bags of 3, 1, 4, 1
+    out = bag(index, offsets)
+    b = torch.autograd.grad((out.pow(2)).sum(), out)[0]
+    gs = O.embedding_bag_grad_sample(index, offsets, b, V, mode)
+    ends = [3, 4, 8, 9]
+    for i in range(4):
+        bag.zero_grad()
+        lo, hi = int(offsets[i]), ends[i]
+        o = bag(index[lo:hi], torch.tensor([0]))
+        (o.pow(2)).sum().backward()
+        torch.testing.assert_close(gs[i], bag.weight.grad, rtol=1e-12, atol=1e-12)
+    # repeated index: the row is written once
+    b2 = torch.tensor([[1.0, 2.0, 3.0, 4.0]], dtype=torch.float64)
+    g2 = O.embedding_bag_grad_sample(torch.tensor([2, 2, 5]), torch.tensor([0]), b2, V, mode)
+    want = b2[0] / (3 if mode == "mean" else 1)
+    assert torch.equal(g2[0, 2], want) and torch.equal(g2[0, 5], want) and g2[0].abs().sum() == 2 * want.abs().sum()
+
+
 # ---- Norm layers ----------------------------------------------------------------------
 def test_group_norm_grad_sample_vs_microbatch():
     torch.manual_seed(8)
