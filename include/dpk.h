@@ -94,7 +94,7 @@ int dpk_linear_ghost_norm(const void* b, const void* a, int dtype, float* norm_w
                           size_t ws_bytes, dpk_stream_t stream);
 
 /* ------------------------------------------------------------------------- *
- * Per-sample gradients of nn.Conv2d
+ * Per-sample gradients of nn.Conv2d (nn.Conv1d as a height-one image) and nn.Conv3d
  * replaces opacus/grad_sample/conv.py:28-119 (compute_conv_grad_sample, the
  * Conv2d branch) together with opacus/utils/tensor_utils.py:116-172 (unfold2d)
  * ------------------------------------------------------------------------- */
@@ -112,6 +112,18 @@ int dpk_conv2d_gs(const void* x, const void* b, int in_dtype, void* gs, int gs_d
                   int64_t n, int64_t C, int64_t H, int64_t W, int64_t O, int64_t KH, int64_t KW,
                   int64_t sh, int64_t sw, int64_t ph_lo, int64_t ph_hi, int64_t pw_lo,
                   int64_t pw_hi, int64_t dh, int64_t dw, int64_t groups, float scale, void* ws,
+                  size_t ws_bytes, dpk_stream_t stream);
+
+/* The same for nn.Conv3d (conv.py:89-96 with unfold3d, tensor_utils.py:175-279):
+ * x: [n,C,D,H,W], b: [n,O,OD,OH,OW], gs: [n,O,C/groups,KD,KH,KW]. kernel, stride,
+ * pad_lo, pad_hi, dilation: host arrays of three values in (depth, height, width) order. */
+size_t dpk_conv3d_gs_workspace_bytes(int64_t n, int64_t C, int64_t O, int64_t KD, int64_t KH,
+                                     int64_t KW, int64_t groups);
+int dpk_conv3d_gs(const void* x, const void* b, int in_dtype, void* gs, int gs_dtype, float* sumsq,
+                  int64_t n, int64_t C, int64_t D, int64_t H, int64_t W, int64_t O,
+                  const int64_t* kernel /*host*/, const int64_t* stride /*host*/,
+                  const int64_t* pad_lo /*host*/, const int64_t* pad_hi /*host*/,
+                  const int64_t* dilation /*host*/, int64_t groups, float scale, void* ws,
                   size_t ws_bytes, dpk_stream_t stream);
 
 /* gs_bias[n,o] = scale * sum_q b[n,o,q]                    (conv.py:117)

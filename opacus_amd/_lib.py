@@ -48,6 +48,11 @@ SIGNATURES = {
         c_int,
         [_P, _P, c_int, _P, c_int, _P] + [_I] * 16 + [c_float, _P, c_size_t, _P],
     ),
+    "dpk_conv3d_gs_workspace_bytes": (c_size_t, [_I, _I, _I, _I, _I, _I, _I]),
+    "dpk_conv3d_gs": (
+        c_int,
+        [_P, _P, c_int, _P, c_int, _P, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, c_float, _P, c_size_t, _P],
+    ),
     "dpk_conv_bias_gs": (c_int, [_P, c_int, _P, c_int, _I, _I, _I, c_float, _P]),
     "dpk_embedding_workspace_bytes": (c_size_t, [_I, _I, _I]),
     "dpk_embedding_unique_pairs": (c_int, [_P, _I, _I, _P, _P, _P, _P, c_size_t, _P]),

@@ -22,17 +22,22 @@ struct ConvGeom {
   int KH, KW, Pg;       // kernel, kernel elements per group (Cg*KH*KW)
   int sh, sw, dh, dw;   // stride, dilation
   int ph, pw;           // top / left padding
+  // Conv3d only (all 1 / 0 for two dimensions): input depth, kernel depth, depth
+  // stride / dilation / front padding, output positions per depth slice (OH*OW).
+  int Dd, KD, sd, dd, pd, OHW;
 };
 
 // Element (k = q, col = p) of the unfolded activation, staged as S[k][p].
-template <int BN, typename T>
+// D3: the input has a depth dimension as well (nn.Conv3d), p = (c, kd, kh, kw) and
+// q = (od, oh, ow).
+template <int BN, typename T, bool D3 = false>
 struct LoaderIm2col {
   static constexpr int R = mf32::BK * BN / mf32::NTHREADS;
   static constexpr int PSTEP = mf32::NTHREADS / mf32::BK;
   const T* x;  // first channel of this sample's group
   ConvGeom g;
   int kq, pl0;
-  int off[R], dy[R], dx[R];
+  int off[R], dy[R], dx[R], dz[D3 ? R : 1];
   float st[R];
   __device__ __forceinline__ LoaderIm2col(const T* x_, const ConvGeom& g_, int p0) : x(x_), g(g_) {
     kq = threadIdx.x % mf32::BK;
@@ -41,27 +46,46 @@ struct LoaderIm2col {
     for (int r = 0; r < R; ++r) {
       const int p = p0 + pl0 + r * PSTEP;
       if (p < g.Pg) {
-        const int c = p / (g.KH * g.KW), rem = p % (g.KH * g.KW);
-        off[r] = c * g.H * g.W;
+        const int kvol = g.KD * g.KH * g.KW;
+        const int c = p / kvol;
+        int rem = p % kvol;
+        off[r] = c * g.Dd * g.H * g.W;
+        if (D3) {
+          dz[r] = (rem / (g.KH * g.KW)) * g.dd - g.pd;
+          rem %= g.KH * g.KW;
+        }
         dy[r] = (rem / g.KW) * g.dh - g.ph;
         dx[r] = (rem % g.KW) * g.dw - g.pw;
       } else {
         off[r] = -1;
         dy[r] = dx[r] = 0;
+        if (D3) dz[r] = 0;
       }
     }
   }
   __device__ __forceinline__ void fetch(int64_t k0) {
     const int q = static_cast<int>(k0) + kq;
-    const int oh = q / g.OW, ow = q - oh * g.OW;
+    int q2 = q, iz0 = 0;
+    if (D3) {
+      const int od = q / g.OHW;
+      q2 = q - od * g.OHW;
+      iz0 = od * g.sd;
+    }
+    const int oh = q2 / g.OW, ow = q2 - oh * g.OW;
     const int iy0 = oh * g.sh, ix0 = ow * g.sw;
     const bool inq = q < g.Q;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const int iy = iy0 + dy[r], ix = ix0 + dx[r];
-      const bool ok = inq && off[r] >= 0 && static_cast<unsigned>(iy) < static_cast<unsigned>(g.H) &&
-                      static_cast<unsigned>(ix) < static_cast<unsigned>(g.W);
-      st[r] = ok ? dpk_io<T>::load(x + off[r] + iy * g.W + ix) : 0.f;
+      bool ok = inq && off[r] >= 0 && static_cast<unsigned>(iy) < static_cast<unsigned>(g.H) &&
+                static_cast<unsigned>(ix) < static_cast<unsigned>(g.W);
+      int plane = 0;
+      if (D3) {
+        const int iz = iz0 + dz[r];
+        ok = ok && static_cast<unsigned>(iz) < static_cast<unsigned>(g.Dd);
+        plane = iz * g.H;
+      }
+      st[r] = ok ? dpk_io<T>::load(x + off[r] + (plane + iy) * g.W + ix) : 0.f;
     }
   }
   __device__ __forceinline__ void commit(float (*S)[BN + mf32::PAD]) {
@@ -70,7 +94,7 @@ struct LoaderIm2col {
   }
 };
 
-template <int BM, int BN, typename TIN, typename TOUT, bool VEC>
+template <int BM, int BN, typename TIN, typename TOUT, bool VEC, bool D3>
 __global__ __launch_bounds__(kThreads) void conv2d_gs_kernel(
     const TIN* __restrict__ x, const TIN* __restrict__ b, TOUT* __restrict__ gs,
     float* __restrict__ partials, ConvGeom g, int C, int O, int groups, float scale, int tiles_m,
@@ -87,9 +111,9 @@ __global__ __launch_bounds__(kThreads) void conv2d_gs_kernel(
   const int64_t sample = bid / groups;
   const int m0 = tm * BM, p0 = tn * BN;
   const TIN* bg = b + (sample * O + static_cast<int64_t>(grp) * Og) * g.Q;
-  const TIN* xg = x + (sample * C + static_cast<int64_t>(grp) * Cg) * g.H * g.W;
+  const TIN* xg = x + (sample * C + static_cast<int64_t>(grp) * Cg) * g.Dd * g.H * g.W;
   mf32::LoaderKContig<BM, TIN, VEC> la(bg, g.Q, m0, Og, g.Q);
-  LoaderIm2col<BN, TIN> lb(xg, g, p0);
+  LoaderIm2col<BN, TIN, D3> lb(xg, g, p0);
   mf32::Tile<BM, BN> tile;
   tile.clear();
   mf32::mainloop<BM, BN>(tile, sm, la, lb, g.Q);
@@ -336,18 +360,34 @@ void launch(const Plan& p, bool vec, const void* x, const void* b, void* gs, flo
                          xp, bp, gp, partials, g, C, O, groups, scale, p.tiles_m, p.tiles_n, Hp, Wp, 0, 0);
     return;
   }
-#define DPK_CONV_LAUNCH(BM, BN, V)                                                              \
-  hipLaunchKernelGGL((conv2d_gs_kernel<BM, BN, TIN, TOUT, V>), grid, block, 0, s, xp, bp, gp,   \
+#define DPK_CONV_LAUNCH(BM, BN, V, D3)                                                            \
+  hipLaunchKernelGGL((conv2d_gs_kernel<BM, BN, TIN, TOUT, V, D3>), grid, block, 0, s, xp, bp, gp, \
                      partials, g, C, O, groups, scale, p.tiles_m, p.tiles_n)
+  const bool d3 = g.Dd > 1 || g.KD > 1 || g.pd > 0;
   if (p.bm == 128) {
-    if (vec) DPK_CONV_LAUNCH(128, 128, true);
-    else DPK_CONV_LAUNCH(128, 128, false);
+    if (vec && d3) DPK_CONV_LAUNCH(128, 128, true, true);
+    else if (vec) DPK_CONV_LAUNCH(128, 128, true, false);
+    else if (d3) DPK_CONV_LAUNCH(128, 128, false, true);
+    else DPK_CONV_LAUNCH(128, 128, false, false);
   } else {
-    if (vec) DPK_CONV_LAUNCH(64, 64, true);
-    else DPK_CONV_LAUNCH(64, 64, false);
+    if (vec && d3) DPK_CONV_LAUNCH(64, 64, true, true);
+    else if (vec) DPK_CONV_LAUNCH(64, 64, true, false);
+    else if (d3) DPK_CONV_LAUNCH(64, 64, false, true);
+    else DPK_CONV_LAUNCH(64, 64, false, false);
   }
 #undef DPK_CONV_LAUNCH
 }
+
+// Depth extents of a Conv3d call; {1, 1, 1, 0, 0, 1} for two dimensions.
+struct Depth {
+  int64_t D, KD, sd, pd_lo, pd_hi, dd;
+};
+
+int conv_gs(const char* who, const void* x, const void* b, int in_dtype, void* gs, int gs_dtype,
+            float* sumsq, int64_t n, int64_t C, const Depth& z, int64_t H, int64_t W, int64_t O,
+            int64_t KH, int64_t KW, int64_t sh, int64_t sw, int64_t ph_lo, int64_t ph_hi, int64_t pw_lo,
+            int64_t pw_hi, int64_t dh, int64_t dw, int64_t groups, float scale, void* ws, size_t ws_bytes,
+            dpk_stream_t stream);
 
 }  // namespace
 
@@ -359,27 +399,27 @@ extern "C" size_t dpk_conv2d_gs_workspace_bytes(int64_t n, int64_t C, int64_t O,
   return dpk_align_up(static_cast<size_t>(n * groups * p.tiles_m * p.tiles_n) * sizeof(float), 256);
 }
 
-extern "C" int dpk_conv2d_gs(const void* x, const void* b, int in_dtype, void* gs, int gs_dtype,
-                             float* sumsq, int64_t n, int64_t C, int64_t H, int64_t W, int64_t O,
-                             int64_t KH, int64_t KW, int64_t sh, int64_t sw, int64_t ph_lo,
-                             int64_t ph_hi, int64_t pw_lo, int64_t pw_hi, int64_t dh, int64_t dw,
-                             int64_t groups, float scale, void* ws, size_t ws_bytes,
-                             dpk_stream_t stream) {
-  const char* who = "dpk_conv2d_gs";
-  DPK_REQUIRE(n >= 0 && C >= 1 && H >= 1 && W >= 1 && O >= 1 && KH >= 1 && KW >= 1, DPK_E_SHAPE,
-              "%s: bad tensor sizes", who);
+namespace {
+int conv_gs(const char* who, const void* x, const void* b, int in_dtype, void* gs, int gs_dtype,
+            float* sumsq, int64_t n, int64_t C, const Depth& z, int64_t H, int64_t W, int64_t O,
+            int64_t KH, int64_t KW, int64_t sh, int64_t sw, int64_t ph_lo, int64_t ph_hi, int64_t pw_lo,
+            int64_t pw_hi, int64_t dh, int64_t dw, int64_t groups, float scale, void* ws, size_t ws_bytes,
+            dpk_stream_t stream) {
+  DPK_REQUIRE(n >= 0 && C >= 1 && H >= 1 && W >= 1 && O >= 1 && KH >= 1 && KW >= 1 && z.D >= 1 && z.KD >= 1,
+              DPK_E_SHAPE, "%s: bad tensor sizes", who);
   DPK_REQUIRE(sh >= 1 && sw >= 1 && dh >= 1 && dw >= 1 && ph_lo >= 0 && ph_hi >= 0 && pw_lo >= 0 &&
-                  pw_hi >= 0 && groups >= 1,
+                  pw_hi >= 0 && groups >= 1 && z.sd >= 1 && z.dd >= 1 && z.pd_lo >= 0 && z.pd_hi >= 0,
               DPK_E_SHAPE, "%s: bad geometry", who);
   DPK_REQUIRE(C % groups == 0 && O % groups == 0, DPK_E_SHAPE,
               "%s: groups=%lld does not divide C=%lld and O=%lld", who, (long long)groups,
               (long long)C, (long long)O);
   if (n == 0) return DPK_OK;
   const int64_t eh = H + ph_lo + ph_hi - (dh * (KH - 1) + 1), ew = W + pw_lo + pw_hi - (dw * (KW - 1) + 1);
-  DPK_REQUIRE(eh >= 0 && ew >= 0, DPK_E_SHAPE, "%s: kernel larger than the padded input", who);
-  const int64_t OH = eh / sh + 1, OW = ew / sw + 1;
-  const int64_t Q = OH * OW, Pg = (C / groups) * KH * KW;
-  DPK_REQUIRE(C * H * W < (1LL << 31) && O * Q < (1LL << 31) && O * Pg < (1LL << 31), DPK_E_SHAPE,
+  const int64_t ed = z.D + z.pd_lo + z.pd_hi - (z.dd * (z.KD - 1) + 1);
+  DPK_REQUIRE(eh >= 0 && ew >= 0 && ed >= 0, DPK_E_SHAPE, "%s: kernel larger than the padded input", who);
+  const int64_t OH = eh / sh + 1, OW = ew / sw + 1, OD = ed / z.sd + 1;
+  const int64_t Q = OD * OH * OW, Pg = (C / groups) * z.KD * KH * KW;
+  DPK_REQUIRE(C * z.D * H * W < (1LL << 31) && O * Q < (1LL << 31) && O * Pg < (1LL << 31), DPK_E_SHAPE,
               "%s: one sample exceeds 2^31 elements", who);
   DPK_REQUIRE(x && b && gs, DPK_E_ARG, "%s: NULL tensor", who);
   DPK_REQUIRE(dpk_dtype_ok(in_dtype) && dpk_dtype_ok(gs_dtype), DPK_E_DTYPE, "%s: dtypes %d,%d", who,
@@ -392,9 +432,12 @@ extern "C" int dpk_conv2d_gs(const void* x, const void* b, int in_dtype, void* g
   g.KH = (int)KH; g.KW = (int)KW; g.Pg = (int)Pg;
   g.sh = (int)sh; g.sw = (int)sw; g.dh = (int)dh; g.dw = (int)dw;
   g.ph = (int)ph_lo; g.pw = (int)pw_lo;
+  g.Dd = (int)z.D; g.KD = (int)z.KD; g.sd = (int)z.sd; g.dd = (int)z.dd; g.pd = (int)z.pd_lo;
+  g.OHW = (int)(OH * OW);
   const int64_t Hp = H + ph_lo + ph_hi, Wp = W + pw_lo + pw_hi;
+  const bool flat = z.D == 1 && z.KD == 1 && z.pd_lo == 0 && z.pd_hi == 0;  // the LDS patch is two-dimensional
   const size_t patch_bytes =
-      Hp * Wp < (1 << 20) ? patch_lds_bytes(g, (int)(C / groups), (int)Hp, (int)Wp) : 0;
+      flat && Hp * Wp < (1 << 20) ? patch_lds_bytes(g, (int)(C / groups), (int)Hp, (int)Wp) : 0;
   const Plan p = make_plan(O / groups, Pg, patch_bytes > 0);
   const int64_t blocks = n * groups * p.tiles_m * p.tiles_n;
   DPK_REQUIRE(blocks <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: %lld blocks exceed the grid limit", who,
@@ -428,4 +471,36 @@ extern "C" int dpk_conv2d_gs(const void* x, const void* b, int in_dtype, void* g
     DPK_LAUNCH_CHECK(who);
   }
   return DPK_OK;
+}
+}  // namespace
+
+extern "C" int dpk_conv2d_gs(const void* x, const void* b, int in_dtype, void* gs, int gs_dtype,
+                             float* sumsq, int64_t n, int64_t C, int64_t H, int64_t W, int64_t O,
+                             int64_t KH, int64_t KW, int64_t sh, int64_t sw, int64_t ph_lo,
+                             int64_t ph_hi, int64_t pw_lo, int64_t pw_hi, int64_t dh, int64_t dw,
+                             int64_t groups, float scale, void* ws, size_t ws_bytes,
+                             dpk_stream_t stream) {
+  const Depth flat = {1, 1, 1, 0, 0, 1};
+  return conv_gs("dpk_conv2d_gs", x, b, in_dtype, gs, gs_dtype, sumsq, n, C, flat, H, W, O, KH, KW, sh, sw,
+                 ph_lo, ph_hi, pw_lo, pw_hi, dh, dw, groups, scale, ws, ws_bytes, stream);
+}
+
+extern "C" size_t dpk_conv3d_gs_workspace_bytes(int64_t n, int64_t C, int64_t O, int64_t KD, int64_t KH,
+                                                int64_t KW, int64_t groups) {
+  if (KD <= 0) return 0;
+  return dpk_conv2d_gs_workspace_bytes(n, C, O, KD * KH, KW, groups);
+}
+
+extern "C" int dpk_conv3d_gs(const void* x, const void* b, int in_dtype, void* gs, int gs_dtype,
+                             float* sumsq, int64_t n, int64_t C, int64_t D, int64_t H, int64_t W,
+                             int64_t O, const int64_t* kernel, const int64_t* stride,
+                             const int64_t* pad_lo, const int64_t* pad_hi, const int64_t* dilation,
+                             int64_t groups, float scale, void* ws, size_t ws_bytes,
+                             dpk_stream_t stream) {
+  const char* who = "dpk_conv3d_gs";
+  DPK_REQUIRE(kernel && stride && pad_lo && pad_hi && dilation, DPK_E_ARG, "%s: NULL geometry array", who);
+  const Depth z = {D, kernel[0], stride[0], pad_lo[0], pad_hi[0], dilation[0]};
+  return conv_gs(who, x, b, in_dtype, gs, gs_dtype, sumsq, n, C, z, H, W, O, kernel[1], kernel[2], stride[1],
+                 stride[2], pad_lo[1], pad_hi[1], pad_lo[2], pad_hi[2], dilation[1], dilation[2], groups, scale,
+                 ws, ws_bytes, stream);
 }

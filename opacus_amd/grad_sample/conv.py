@@ -2,7 +2,7 @@
 
 Conv2d runs the implicit-im2col MFMA kernel; Conv1d is the same kernel on a height-one
 image, as the reference's Conv1d branch does with ``unsqueeze(-2)`` (conv.py:71-88).
-Conv3d has no kernel here and is left to the generic fallback.
+Conv3d runs the same kernel with a depth dimension in the gather (conv.py:89-96).
 """
 
 from __future__ import annotations
@@ -29,11 +29,11 @@ def _pads(padding, kernel: int, dilation: int) -> Tuple[int, int]:
     return int(padding), int(padding)
 
 
-@register_grad_sampler([nn.Conv1d, nn.Conv2d])
+@register_grad_sampler([nn.Conv1d, nn.Conv2d, nn.Conv3d])
 @owns_output
 @fused_scale
 def compute_conv_grad_sample(
-    layer: Union[nn.Conv1d, nn.Conv2d], activations: List[torch.Tensor], backprops: torch.Tensor, scale: float = 1.0
+    layer: Union[nn.Conv1d, nn.Conv2d, nn.Conv3d], activations: List[torch.Tensor], backprops: torch.Tensor, scale: float = 1.0
 ) -> Dict[nn.Parameter, torch.Tensor]:
     """Per-sample gradients ``[n, *weight.shape]`` and ``[n, out_channels]`` (conv.py:28-119).
     An empty batch yields zeros with a batch dimension of one (conv.py:46-53)."""
@@ -47,6 +47,17 @@ def compute_conv_grad_sample(
             ret[layer.bias] = torch.zeros_like(layer.bias).unsqueeze(0)
         return ret
     pad_is_str = isinstance(layer.padding, str)
+    if isinstance(layer, nn.Conv3d):
+        ksize, stride, dilation = tuple(layer.kernel_size), tuple(layer.stride), tuple(layer.dilation)
+        pads3 = tuple(
+            _pads(layer.padding if pad_is_str else layer.padding[d], ksize[d], dilation[d]) for d in range(3)
+        )
+        if layer.weight.requires_grad:
+            gs, sumsq = kernels.conv3d_grad_sample(x, backprops, ksize, stride, pads3, dilation, layer.groups, scale=scale)
+            ret[layer.weight] = tag_sumsq(gs.view(n, *layer.weight.shape), sumsq)
+        if want_b:
+            ret[layer.bias] = kernels.conv_bias_grad_sample(backprops, scale=scale)
+        return ret
     if isinstance(layer, nn.Conv1d):
         x = x.unsqueeze(-2)
         b4 = backprops.unsqueeze(-2)

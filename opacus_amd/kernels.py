@@ -242,6 +242,54 @@ def conv2d_grad_sample(
     return gs, sumsq
 
 
+def conv3d_grad_sample(
+    x: torch.Tensor,
+    backprops: torch.Tensor,
+    kernel_size: Tuple[int, int, int],
+    stride: Tuple[int, int, int],
+    padding: Tuple[Tuple[int, int], Tuple[int, int], Tuple[int, int]],
+    dilation: Tuple[int, int, int],
+    groups: int,
+    scale: float = 1.0,
+    want_sumsq: bool = True,
+) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """Per-sample weight gradients ``[n, O, C/groups, KD, KH, KW]`` of a 3-d convolution.
+
+    ``padding`` is ``((front, back), (top, bottom), (left, right))``; ``backprops`` is
+    ``[n, O, OD, OH, OW]``.
+    """
+    dev = _need_gpu(x, backprops)
+    if x.dtype != backprops.dtype:
+        x = x.to(backprops.dtype)
+    n, C, D, H, W = x.shape
+    O = backprops.shape[1]
+    gs = torch.empty((n, O, C // groups, *kernel_size), dtype=backprops.dtype, device=dev)
+    sumsq = torch.empty((n,), dtype=torch.float32, device=dev) if want_sumsq else None
+    if n == 0:
+        return gs, sumsq
+    x = _dense(x)
+    b = _dense(backprops)
+    out = [
+        (size + lo + hi - (dil * (k - 1) + 1)) // st + 1
+        for size, (lo, hi), dil, k, st in zip((D, H, W), padding, dilation, kernel_size, stride)
+    ]
+    if b.numel() != n * O * out[0] * out[1] * out[2]:
+        raise ValueError(f"backprops {tuple(backprops.shape)} do not match the output geometry [{n},{O},{out}]")
+    arr = lambda v: (ctypes.c_int64 * 3)(*[int(e) for e in v])  # noqa: E731
+    L = lib()
+    ws, wsb = _ws(L.dpk_conv3d_gs_workspace_bytes(n, C, O, *kernel_size, groups) if want_sumsq else 0, dev)
+    with _timed("conv3d_gs", dev):
+        check(
+            "dpk_conv3d_gs",
+            L.dpk_conv3d_gs(
+                _ptr(x), _ptr(b), _code(b), _ptr(gs), _code(gs), _ptr(sumsq), n, C, D, H, W, O, arr(kernel_size),
+                arr(stride), arr([p[0] for p in padding]), arr([p[1] for p in padding]), arr(dilation), groups,
+                float(scale), _ptr(ws), wsb, _stream(dev),
+            ),
+        )
+    return gs, sumsq
+
+
 def conv_bias_grad_sample(backprops: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
     """``gs[n,o] = scale * sum over the spatial dims of b[n,o,...]``."""
     dev = _need_gpu(backprops)

@@ -12,6 +12,8 @@ What pins each function (see ``tests/test_oracle_pins.py``):
     and the invariant sum_n gs[n] == autograd's .grad for a sum loss;
   * unfold2d: exact equality with torch.nn.functional.unfold
     (opacus/tests/grad_samples/conv2d_test.py:121-153);
+  * unfold3d / Conv3d grad sample: batch-of-one autograd of nn.Conv3d over strides,
+    dilations, groups and "same" padding; a depth-one call equals unfold2d exactly;
   * linear ghost norm: equals the Frobenius norm of the materialised grad sample in
     float64, and the closed forms for T == 1;
   * embedding ghost norm: the three input/expected triples of
@@ -174,6 +176,53 @@ def conv2d_grad_sample(
     full = torch.einsum("noq,npq->nop", b, U)
     full = full.view(n, groups, -1, groups, C // groups, kh * kw)
     gs = torch.einsum("ngrg...->ngr...", full).contiguous().view(n, O, C // groups, kh, kw)
+    return gs, (b.sum(dim=2) if bias else None)
+
+
+def unfold3d(x: torch.Tensor, *, kernel_size, padding, stride, dilation) -> torch.Tensor:
+    """im2col of a 5-d input: ``[n, C*kd*kh*kw, OD*OH*OW]``, rows ordered (c, kd, kh, kw)
+    (opacus/utils/tensor_utils.py:175-279), gathered index by index. ``padding`` is a triple,
+    "same" (smaller half first, :224-233) or "valid"."""
+    n, C = x.shape[:2]
+    pads = []
+    for d in range(3):
+        if padding == "same":
+            total = dilation[d] * (kernel_size[d] - 1)
+            pads.append((total // 2, total - total // 2))
+        elif padding == "valid":
+            pads.append((0, 0))
+        else:
+            pads.append((padding[d], padding[d]))
+    xp = F.pad(x, (pads[2][0], pads[2][1], pads[1][0], pads[1][1], pads[0][0], pads[0][1]))
+    idx, outs = [], []
+    for d in range(3):
+        size = x.shape[2 + d] + pads[d][0] + pads[d][1]
+        o = (size - (dilation[d] * (kernel_size[d] - 1) + 1)) // stride[d] + 1
+        outs.append(o)
+        idx.append((torch.arange(o) * stride[d])[None, :] + (torch.arange(kernel_size[d]) * dilation[d])[:, None])
+    zi, yi, xi = idx  # each [k, o]
+    # out[n, c, a, i, j, z, y, x] = xp[n, c, zi[a, z], yi[i, y], xi[j, x]]
+    out = xp[
+        :, :, zi[:, None, None, :, None, None], yi[None, :, None, None, :, None], xi[None, None, :, None, None, :]
+    ]
+    kd, kh, kw = kernel_size
+    return out.reshape(n, C * kd * kh * kw, outs[0] * outs[1] * outs[2])
+
+
+def conv3d_grad_sample(
+    x: torch.Tensor, backprops: torch.Tensor, *, kernel_size, padding, stride, dilation, groups: int, bias: bool = True
+) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """opacus/grad_sample/conv.py:89-117, Conv3d branch: unfold3d, contract over output positions,
+    keep the group-diagonal blocks, reshape to ``[n, O, C/groups, kd, kh, kw]``."""
+    x = x.to(backprops.dtype)
+    n, C = x.shape[0], x.shape[1]
+    O = backprops.shape[1]
+    kd, kh, kw = kernel_size
+    U = unfold3d(x, kernel_size=kernel_size, padding=padding, stride=stride, dilation=dilation)
+    b = backprops.reshape(n, -1, U.shape[-1])
+    full = torch.einsum("noq,npq->nop", b, U)
+    full = full.view(n, groups, -1, groups, C // groups, kd * kh * kw)
+    gs = torch.einsum("ngrg...->ngr...", full).contiguous().view(n, O, C // groups, kd, kh, kw)
     return gs, (b.sum(dim=2) if bias else None)
 
 

@@ -24,6 +24,8 @@ def test_header_declares_the_expected_surface():
         "dpk_linear_bias_gs",
         "dpk_linear_ghost_norm",
         "dpk_conv2d_gs",
+        "dpk_conv3d_gs",
+        "dpk_embedding_bag_gs",
         "dpk_conv_bias_gs",
         "dpk_embedding_gs",
         "dpk_embedding_ghost_norm",

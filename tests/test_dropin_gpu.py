@@ -199,6 +199,31 @@ def test_layer_norm_and_instance_norm_grad_samples(A):
         close(p.grad_sample, want[k], 1e-3, 1e-5, k)
 
 
+def test_conv3d_and_conv1d_grad_samples(A):
+    class Net(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.c3 = nn.Conv3d(2, 4, (2, 3, 3), stride=(1, 2, 1), padding=(0, 1, 1), groups=2)
+            self.c1 = nn.Conv1d(4, 5, 3, padding="same")
+            self.fc = nn.Linear(5, 3)
+
+        def forward(self, x):
+            h = F.relu(self.c3(x))  # [n, 4, 3, 3, 6]
+            h = F.relu(self.c1(h.flatten(2)))  # [n, 5, 54]
+            return self.fc(h.mean(dim=2))
+
+    torch.manual_seed(8)
+    net = Net()
+    n = 4
+    x, y = torch.randn(n, 2, 4, 6, 6), torch.randint(0, 3, (n,))
+    want = per_sample_grads_cpu(net, x, y, ce_sum)
+    gsm = A.GradSampleModule(copy.deepcopy(net).to(DEV), loss_reduction="mean")
+    F.cross_entropy(gsm(x.to(DEV)), y.to(DEV)).backward()
+    for k, p in gsm._module.named_parameters():
+        assert p.grad_sample.shape == (n, *p.shape), k
+        close(p.grad_sample, want[k], 1e-3, 1e-5, k)
+
+
 def test_embedding_bag_grad_samples(A):
     """nn.EmbeddingBag through the wrapper, with offsets and with a 2-D index tensor; bags hold
     distinct indices so that batch-of-one autograd is the reference."""

@@ -396,6 +396,41 @@ def test_conv2d_grad_sample_bf16(K):
     assert_rel(gs, want_w, BF16_REL)
 
 
+CONV3D_GPU_CASES = [
+    dict(n=3, C=2, O=3, k=(2, 3, 2), stride=(1, 1, 1), padding=(0, 1, 0), dilation=(1, 1, 1), groups=1, size=(4, 5, 6)),
+    dict(n=2, C=4, O=4, k=(3, 2, 2), stride=(2, 1, 2), padding=(1, 0, 2), dilation=(1, 2, 1), groups=2, size=(6, 5, 7)),
+    dict(n=2, C=2, O=2, k=(2, 2, 3), stride=(1, 1, 1), padding="same", dilation=(2, 1, 1), groups=1, size=(5, 4, 6)),
+    dict(n=2, C=8, O=80, k=(3, 3, 3), stride=(1, 1, 1), padding=(1, 1, 1), dilation=(1, 1, 1), groups=1, size=(6, 8, 8)),  # 128-tiles
+]
+
+
+@pytest.mark.parametrize("case", CONV3D_GPU_CASES)
+def test_conv3d_grad_sample_f32(K, case):
+    torch.manual_seed(case["C"] * 7 + case["O"])
+    n = case["n"]
+    x = torch.randn(n, case["C"], *case["size"])
+    pads = []
+    for d in range(3):
+        if case["padding"] == "same":
+            total = case["dilation"][d] * (case["k"][d] - 1)
+            pads.append((total // 2, total - total // 2))
+        else:
+            pads.append((case["padding"][d], case["padding"][d]))
+    out = [
+        (case["size"][d] + pads[d][0] + pads[d][1] - (case["dilation"][d] * (case["k"][d] - 1) + 1)) // case["stride"][d] + 1
+        for d in range(3)
+    ]
+    b = torch.randn(n, case["O"], *out)
+    want_w, want_b = O.conv3d_grad_sample(
+        x.double(), (b * 2.0).double(), kernel_size=case["k"], padding=case["padding"], stride=case["stride"],
+        dilation=case["dilation"], groups=case["groups"],
+    )
+    gs, sumsq = K.conv3d_grad_sample(dev(x), dev(b), case["k"], case["stride"], tuple(pads), case["dilation"], case["groups"], scale=2.0)
+    assert_rel(gs, want_w, FP32_REL, "conv3d weight")
+    assert_rel(sumsq, want_w.flatten(1).pow(2).sum(1), 2e-5, "conv3d sumsq")
+    assert_rel(K.conv_bias_grad_sample(dev(b), scale=2.0), want_b, FP32_REL, "conv3d bias")
+
+
 # ---- Embedding ------------------------------------------------------------------------
 def test_embedding_golden_vectors(K, embedding_norm_cases):
     """The reference's own known-answer triples and docstring intermediates, on the GPU."""

@@ -232,6 +232,37 @@ def test_embedding_bag_grad_sample_vs_microbatch_and_repeat_rule(mode):
     assert torch.equal(g2[0, 2], want) and torch.equal(g2[0, 5], want) and g2[0].abs().sum() == 2 * want.abs().sum()
 
 
+CONV3D_CASES = [
+    dict(C=2, O=3, k=(2, 3, 2), stride=(1, 1, 1), padding=(0, 1, 0), dilation=(1, 1, 1), groups=1, size=(4, 5, 6)),
+    dict(C=4, O=4, k=(3, 2, 2), stride=(2, 1, 2), padding=(1, 0, 2), dilation=(1, 2, 1), groups=2, size=(6, 5, 7)),
+    dict(C=2, O=2, k=(2, 2, 3), stride=(1, 1, 1), padding="same", dilation=(2, 1, 1), groups=1, size=(5, 4, 6)),
+    dict(C=3, O=6, k=(1, 1, 1), stride=(1, 2, 1), padding="valid", dilation=(1, 1, 1), groups=3, size=(3, 4, 3)),
+]
+
+
+@pytest.mark.parametrize("case", CONV3D_CASES)
+def test_conv3d_grad_sample_vs_microbatch(case):
+    torch.manual_seed(16)
+    conv = nn.Conv3d(case["C"], case["O"], case["k"], stride=case["stride"], padding=case["padding"],
+                     dilation=case["dilation"], groups=case["groups"]).double()
+    x = torch.randn(3, case["C"], *case["size"], dtype=torch.float64)
+    loss = lambda y: y.pow(2).sum()  # noqa: E731
+    b = _backprops(conv, x, loss)
+    gs_w, gs_b = O.conv3d_grad_sample(x, b, kernel_size=case["k"], padding=case["padding"], stride=case["stride"],
+                                      dilation=case["dilation"], groups=case["groups"])
+    want = _per_sample_autograd(conv, x, loss)
+    torch.testing.assert_close(gs_w, want["weight"], rtol=1e-10, atol=1e-10)
+    torch.testing.assert_close(gs_b, want["bias"], rtol=1e-10, atol=1e-10)
+
+
+def test_unfold3d_of_a_depth_one_volume_is_unfold2d():
+    torch.manual_seed(17)
+    x = torch.randn(2, 3, 6, 7, dtype=torch.float64)
+    u2 = O.unfold2d(x, kernel_size=(3, 2), padding=(1, 2), stride=(2, 1), dilation=(1, 2))
+    u3 = O.unfold3d(x.unsqueeze(2), kernel_size=(1, 3, 2), padding=(0, 1, 2), stride=(1, 2, 1), dilation=(1, 1, 2))
+    assert torch.equal(u2, u3)
+
+
 # ---- Norm layers ----------------------------------------------------------------------
 def test_group_norm_grad_sample_vs_microbatch():
     torch.manual_seed(8)
