@@ -1,0 +1,201 @@
+"""GPU parity at the full sizes of the five benchmark configurations.
+
+The CPU oracle cannot recompute 8.6 GB of per-sample gradients or a 1024 x 1024 x 32000 Gram for
+every sample in test time, so full-size runs are checked through what does not depend on the
+size: closed forms that collapse to a small CPU computation (a clip-weighted sum of rank-one
+gradients is one thin matrix product), the oracle on a few samples of the batch (every sample
+is independent on this path), exact scaling by powers of two, invariance under a permutation of
+the positions t, and additivity in the backprops. Tolerances are the stated bar: fp32 within
+rel 1e-5 of the tensor's scale, bf16 inputs with fp32 accumulation within 2e-2 (in practice
+1e-4, since the inputs are exact in bf16), integer-indexed outputs exact.
+"""
+
+import math
+
+import pytest
+import torch
+
+from oracle import dp_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+FP32_REL = 1e-5
+
+
+@pytest.fixture(scope="module")
+def K():
+    from opacus_amd import kernels
+
+    return kernels
+
+
+def dev(t):
+    return t.to("cuda")
+
+
+def rel_err(got, want):
+    got, want = got.detach().double().cpu(), want.detach().double().cpu()
+    return ((got - want).abs().max() / want.abs().max().clamp_min(1e-300)).item()
+
+
+# ---- C2: Linear 4096 x 4096, batch 128, T = 1, fp32 ----------------------------------------
+def test_c2_linear_grad_sample_clip_accumulate_noise(K):
+    n, d = 128, 4096
+    torch.manual_seed(0)
+    a, b = torch.randn(n, d), torch.randn(n, d)
+    da, db = dev(a), dev(b)
+    gs, sumsq = K.linear_grad_sample(db, da)
+    assert gs.shape == (n, d, d)
+    # rank-one structure: every entry is one fp32 product, so sampled entries are exact
+    g = torch.Generator().manual_seed(1)
+    ii, jj, kk = (torch.randint(0, hi, (4096,), generator=g) for hi in (n, d, d))
+    got = gs[dev(ii), dev(jj), dev(kk)].cpu()
+    assert torch.equal(got, b[ii, jj] * a[ii, kk])
+    # a whole sample against the oracle's einsum
+    want0, _ = O.linear_grad_sample(a[5:6], b[5:6])
+    assert torch.equal(gs[5].cpu(), want0[0])
+    # squared norms: closed form |b|^2 |a|^2 in float64
+    want_ss = a.double().pow(2).sum(1) * b.double().pow(2).sum(1)
+    assert rel_err(sumsq, want_ss) < FP32_REL
+    # and the streaming norm kernel over the 8.6 GB tensor agrees with it
+    assert rel_err(K.sumsq_rows([gs])[0], want_ss) < FP32_REL
+    # clip-weighted sum = (clip * B)^T A, a thin product the CPU does in float64
+    C = math.sqrt(want_ss.median().item())  # about half of the samples are clipped
+    norm, clip = K.clip_factor(sumsq.reshape(1, -1), C)
+    want_clip = (C / (want_ss.sqrt() + 1e-6)).clamp(max=1.0)
+    assert rel_err(clip, want_clip) < FP32_REL and 0 < (want_clip < 1).sum() < n
+    summed = torch.empty(d, d, device="cuda")
+    K.clip_accumulate([gs], clip, [summed], accumulate=False)
+    want_sum = (want_clip[:, None] * b.double()).t() @ a.double()
+    assert rel_err(summed, want_sum) < FP32_REL
+    K.clip_accumulate([gs], clip, [summed], accumulate=True)
+    assert rel_err(summed, 2 * want_sum) < FP32_REL
+    # noise at full size: exact when std = 0, N(0, std^2) / denom otherwise, repeatable
+    grad = torch.empty_like(summed)
+    K.add_noise(summed, grad, 0.0, 128.0, 3, 0)
+    assert torch.equal(grad, summed / 128.0)
+    K.add_noise(summed, grad, 2.0, 4.0, 3, 8)
+    z = (grad.double() * 4.0 - summed.double()) / 2.0
+    P = z.numel()
+    assert abs(z.mean().item()) < 5 / math.sqrt(P) and abs(z.std().item() - 1.0) < 5 / math.sqrt(2 * P)
+    again = torch.empty_like(grad)
+    K.add_noise(summed, again, 2.0, 4.0, 3, 8)
+    assert torch.equal(grad, again)
+
+
+# ---- C3 / C5: ghost norms, bf16 ---------------------------------------------------------------
+@pytest.mark.parametrize(
+    "n,T,fin,fout,check",
+    [
+        (32, 512, 1024, 4096, 3),  # C3 fc1
+        (32, 512, 4096, 1024, 3),  # C3 fc2
+        (16, 1024, 2048, 2048, 2),  # C5 q / o
+        (16, 1024, 2048, 32000, 1),  # C5 LM head
+    ],
+)
+def test_ghost_norm_full_size(K, n, T, fin, fout, check):
+    torch.manual_seed(T + fout)
+    a = torch.randn(n, T, fin, device="cuda").bfloat16()
+    b = (torch.randn(n, T, fout, device="cuda") * 0.02).bfloat16()
+    nw, nb = K.linear_ghost_norm(b, a, want_weight=True, want_bias=True)
+    assert nw.shape == (n,) and nw.dtype == torch.float32
+    # the oracle (float64 Grams) on a few samples: samples are independent
+    want_w, want_b = O.linear_norm_sample(a[:check].cpu().double(), b[:check].cpu().double())
+    assert rel_err(nw[:check], want_w) < 1e-4 and rel_err(nb[:check], want_b) < 1e-4
+    # the same samples alone give the same norms (other tiling of the launch)
+    alone_w, alone_b = K.linear_ghost_norm(b[:check].contiguous(), a[:check].contiguous(), want_weight=True, want_bias=True)
+    assert rel_err(alone_w, nw[:check]) < FP32_REL and rel_err(alone_b, nb[:check]) < FP32_REL
+    # exact scaling: doubling the backprops doubles every accumulator exactly
+    nw2, nb2 = K.linear_ghost_norm((b.float() * 2).bfloat16(), a, want_weight=True, want_bias=True)
+    assert torch.equal(nw2, 2 * nw) and torch.equal(nb2, 2 * nb)
+    # the scale argument is the same factor
+    nw3, _ = K.linear_ghost_norm(b, a, scale=2.0, want_weight=True, want_bias=False)
+    assert rel_err(nw3, 2 * nw) < 1e-6
+    # invariance under a permutation of the positions t
+    perm = torch.randperm(T, device="cuda")
+    nwp, nbp = K.linear_ghost_norm(b[:, perm].contiguous(), a[:, perm].contiguous(), want_weight=True, want_bias=True)
+    assert rel_err(nwp, nw) < FP32_REL and rel_err(nbp, nb) < FP32_REL
+    # the norm of the bias gradient is |sum_t b_t| for every sample
+    assert rel_err(nb, b.double().sum(1).norm(dim=1)) < 1e-4
+
+
+# ---- C4: Conv2d 64 -> 64, 3 x 3, 32 x 32 images, batch 256, fp32 ------------------------------
+def test_c4_conv_and_group_norm_full_size(K):
+    n = 256
+    torch.manual_seed(4)
+    x, b = torch.randn(n, 64, 32, 32), torch.randn(n, 64, 32, 32)
+    dx, db = dev(x), dev(b)
+    geo = dict(kernel_size=(3, 3), stride=(1, 1), padding=(1, 1, 1, 1), dilation=(1, 1), groups=1)
+    gs, sumsq = K.conv2d_grad_sample(dx, db, **geo)
+    pick = [0, 17, 255]
+    want, want_bias = O.conv2d_grad_sample(
+        x[pick].double(), b[pick].double(), kernel_size=(3, 3), padding=(1, 1), stride=(1, 1), dilation=(1, 1), groups=1
+    )
+    assert rel_err(gs[pick], want) < FP32_REL
+    assert rel_err(sumsq, gs.double().flatten(1).pow(2).sum(1)) < FP32_REL
+    assert rel_err(K.conv_bias_grad_sample(db)[pick], want_bias) < FP32_REL
+    # additivity in the backprops over the whole batch
+    b2 = torch.randn(n, 64, 32, 32, device="cuda")
+    gs2, _ = K.conv2d_grad_sample(dx, b2, **geo)
+    gs12, _ = K.conv2d_grad_sample(dx, db + b2, **geo)
+    assert rel_err(gs12, gs.double() + gs2.double()) < FP32_REL
+    # GroupNorm(32, 64) on the same activations
+    gw, gb = K.group_norm_grad_sample(dx, db, 32, 1e-5)
+    want_w, want_b = O.group_norm_grad_sample(x.double(), b.double(), 32, 1e-5)
+    assert rel_err(gw, want_w) < FP32_REL and rel_err(gb, want_b) < FP32_REL
+
+
+# ---- C5: Embedding ghost norm and RMSNorm at batch 16, seq 1024, dim 2048, bf16 ---------------
+def test_c5_embedding_and_rms_norm_full_size(K):
+    n, T, D, V = 16, 1024, 2048, 32000
+    torch.manual_seed(5)
+    ids = torch.randint(0, V, (n, T))
+    ids[3, :500] = ids[3, 0]  # one sample full of repeats
+    b = (torch.randn(n, T, D) * 0.02).bfloat16()
+    x = torch.randn(n, T, D).bfloat16()
+    got = K.embedding_ghost_norm(dev(ids), dev(b))
+    want = O.embedding_norm_sample(ids, b.double())["result_sqrt"]
+    assert rel_err(got, want) < 1e-4
+    # the integer stage is exact at full size too
+    uniq, inverse = O.embedding_unique_pairs(ids)
+    g_uniq, g_inv = K.embedding_unique_pairs(dev(ids))
+    assert torch.equal(g_uniq.cpu(), uniq) and torch.equal(g_inv.cpu(), inverse)
+    gw = K.rms_norm_grad_sample(dev(x), dev(b), D, 1e-5)
+    want_w = O.rms_norm_grad_sample(x.double(), b.double(), (D,), 1e-5)
+    assert rel_err(gw, want_w) < 2e-2  # the output is rounded to bf16
+    gw32 = K.rms_norm_grad_sample(dev(x.float()), dev(b.float()), D, 1e-5)
+    assert rel_err(gw32, want_w) < FP32_REL
+
+
+# ---- C1: the small CNN at batch 256, whole step against the oracle ------------------------------
+def test_c1_small_cnn_full_batch_step():
+    import copy
+
+    import torch.nn.functional as F
+
+    import bench
+    import opacus_amd as A
+
+    torch.manual_seed(0)
+    net = bench.SmallCNN()
+    n = 256
+    x, y = torch.randn(n, 1, 28, 28), torch.randint(0, 10, (n,))
+    names = [k for k, _ in net.named_parameters()]
+    per_sample = {k: [] for k in names}
+    for i in range(n):
+        net.zero_grad()
+        F.cross_entropy(net(x[i : i + 1]), y[i : i + 1], reduction="sum").backward()
+        for k, p in net.named_parameters():
+            per_sample[k].append(p.grad.clone())
+    net.zero_grad()
+    gs = [torch.stack(per_sample[k]) for k in names]
+    norms, clip, summed = O.clip_and_accumulate(gs, 1.0)
+    gsm = A.GradSampleModule(copy.deepcopy(net).cuda(), loss_reduction="mean")
+    opt = A.DPOptimizer(torch.optim.SGD(gsm.parameters(), lr=0.1), noise_multiplier=0.0, max_grad_norm=1.0, expected_batch_size=n)
+    opt.zero_grad()
+    F.cross_entropy(gsm(x.cuda()), y.cuda()).backward()
+    for (k, p), g in zip(gsm._module.named_parameters(), gs):
+        assert rel_err(p.grad_sample, g) < 2e-5, k
+    opt.step()
+    for (k, p), s in zip(gsm._module.named_parameters(), summed):
+        assert rel_err(p.grad, s / n) < 2e-5, k
