@@ -22,6 +22,7 @@ import torch.nn as nn
 
 from .. import kernels
 from ..utils.module_utils import requires_grad, trainable_modules, trainable_parameters
+from ._common import cached_sumsq
 from .grad_sample_module import (
     GradSampleHooks,
     call_sampler,
@@ -34,14 +35,6 @@ logger = logging.getLogger(__name__)
 logger.disabled = True
 
 
-def _cached_sumsq(gs: torch.Tensor):
-    """The per-sample sum of squares a sampler's kernel left on ``gs``, if still valid."""
-    ss = getattr(gs, "_dpk_sumsq", None)
-    if ss is not None and getattr(gs, "_dpk_sumsq_version", None) == gs._version:
-        return ss
-    return None
-
-
 def create_norm_sample(*, param: torch.Tensor, grad_sample: torch.Tensor, max_batch_len: int) -> None:
     """``param._norm_sample`` = per-sample 2-norm of ``grad_sample``; an empty tensor for an
     empty batch (grad_sample_module_fast_gradient_clipping.py:42-70)."""
@@ -50,7 +43,7 @@ def create_norm_sample(*, param: torch.Tensor, grad_sample: torch.Tensor, max_ba
     if max_batch_len == 0:
         param._norm_sample = torch.zeros((0,), device=grad_sample.device, dtype=torch.float32)
         return
-    ss = _cached_sumsq(grad_sample)
+    ss = cached_sumsq(grad_sample)
     if ss is None:
         ss = kernels.sumsq_rows([grad_sample])[0]
     param._norm_sample, _ = kernels.clip_factor(ss.reshape(1, -1), 1.0)

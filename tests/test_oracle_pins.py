@@ -103,9 +103,7 @@ CONV_CASES = [
 def test_unfold2d_equals_F_unfold_exactly(case):
     torch.manual_seed(4)
     x = torch.randn(3, case["C"], case["H"], case["W"])
-    if case["padding"] == "same" and (case["stride"][0] != 1 or case["stride"][1] != 1):
-        # F.unfold has no "same"; pad by hand exactly as unfold2d must
-        pass
+    # F.unfold has no "same": the input is padded by hand with the amounts unfold2d must use
     pt, pb, pl, pr = O.conv2d_padding(case["padding"], case["k"], case["dilation"])
     want = F.unfold(F.pad(x, (pl, pr, pt, pb)), kernel_size=case["k"], stride=case["stride"], dilation=case["dilation"])
     got = O.unfold2d(x, kernel_size=case["k"], padding=case["padding"], stride=case["stride"], dilation=case["dilation"])
