@@ -9,6 +9,7 @@ the GPU: there is no CPU implementation behind these calls.
 from __future__ import annotations
 
 import ctypes
+import math
 from contextlib import contextmanager
 from typing import Dict, List, Optional, Sequence, Tuple
 
@@ -312,7 +313,7 @@ def conv_bias_grad_sample(backprops: torch.Tensor, scale: float = 1.0) -> torch.
 def _ids_2d(ids: torch.Tensor) -> torch.Tensor:
     if ids.dtype != torch.int64:
         ids = ids.to(torch.int64)
-    return _dense(ids).reshape(ids.shape[0], -1)
+    return _dense(ids).reshape(ids.shape[0], math.prod(ids.shape[1:]))  # explicit: -1 is ambiguous for an empty batch
 
 
 def embedding_unique_pairs(ids: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
@@ -520,7 +521,7 @@ def layer_norm_grad_sample(
 # ---- optimizer: norms, clip factor, clip-weighted sum, noise ---------------------------
 def _flat2d(gs: torch.Tensor) -> torch.Tensor:
     g = _dense(gs)
-    return g.reshape(g.shape[0], -1)
+    return g.reshape(g.shape[0], math.prod(g.shape[1:]))  # explicit: -1 is ambiguous for an empty batch
 
 
 def sumsq_rows(gs_list: Sequence[torch.Tensor]) -> torch.Tensor:
@@ -557,7 +558,7 @@ def clip_factor(
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     """``(norm[n], clip[n])`` from ``values[K, n]`` (squared norms, or norms with ``is_norm``)."""
     dev = _need_gpu(values)
-    v = _dense(values.to(torch.float32)).reshape(-1, values.shape[-1])
+    v = _dense(values.to(torch.float32)).reshape(math.prod(values.shape[:-1]), values.shape[-1])
     K, n = v.shape
     norm = torch.empty((n,), dtype=torch.float32, device=dev)
     clip = torch.empty((n,), dtype=torch.float32, device=dev)
@@ -578,7 +579,7 @@ def clip_factor_per_layer(
     """``clip[K, n]`` with ``clip[k] = min(1, C_k / (norm_k + 1e-6))`` from ``values[K, n]``
     (squared norms, or norms with ``is_norm``)."""
     dev = _need_gpu(values)
-    v = _dense(values.to(torch.float32)).reshape(-1, values.shape[-1])
+    v = _dense(values.to(torch.float32)).reshape(math.prod(values.shape[:-1]), values.shape[-1])
     K, n = v.shape
     if len(max_grad_norms) != K:
         raise ValueError(f"{len(max_grad_norms)} bounds for {K} parameters")

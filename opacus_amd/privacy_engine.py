@@ -18,6 +18,7 @@ import torch
 from torch import nn, optim
 from torch.utils.data import DataLoader
 
+from .data_loader import DPDataLoader, switch_generator
 from .grad_sample import AbstractGradSampleModule, GradSampleHooks, get_gsm_class, prepare_module
 from .optimizers import DPOptimizer, get_optimizer_class
 from .utils.fast_gradient_clipping_utils import DPLossFastGradientClipping
@@ -103,7 +104,10 @@ class PrivacyEngine:
             **kwargs,
         )
 
-    def _prepare_data_loader(self, data_loader: DataLoader, *, poisson_sampling: bool, **_unused) -> DataLoader:
+    def _prepare_data_loader(
+        self, data_loader: DataLoader, *, poisson_sampling: bool, batch_first: bool = True, rand_on_empty: bool = False,
+        **_unused,
+    ) -> DataLoader:
         if self.dataset is None:
             self.dataset = data_loader.dataset
         elif self.dataset != data_loader.dataset:
@@ -112,6 +116,14 @@ class PrivacyEngine:
                 "Privacy accounting works per dataset, please initialize new PrivacyEngine if you're using "
                 "different dataset."
             )
+        if poisson_sampling:
+            # privacy_engine.py:165-172: Poisson batches, empty ones included
+            return DPDataLoader.from_data_loader(
+                data_loader, generator=self.secure_rng, distributed=False, batch_first=batch_first,
+                rand_on_empty=rand_on_empty,
+            )
+        if self.secure_mode:
+            return switch_generator(data_loader=data_loader, generator=self.secure_rng)
         return data_loader
 
     def _prepare_model(
@@ -174,11 +186,6 @@ class PrivacyEngine:
         ``(module, optimizer, criterion, data_loader)`` (privacy_engine.py:307-475)."""
         if noise_generator and self.secure_mode:
             raise ValueError("Passing seed is prohibited in secure mode")
-        if poisson_sampling:
-            raise NotImplementedError(
-                "the Poisson-sampling data loader is outside this build (host data pipeline); "
-                "pass poisson_sampling=False, or wrap the loader yourself before make_private"
-            )
         model_parameters = set(module.parameters())
         for p in chain.from_iterable(g["params"] for g in optimizer.param_groups):
             if p not in model_parameters:
@@ -194,6 +201,9 @@ class PrivacyEngine:
             grad_sample_mode=grad_sample_mode,
             wrap_model=wrap_model,
         )
+        if poisson_sampling:
+            # a second backward pass before the step would mix two Poisson draws (privacy_engine.py:429-430)
+            module.forbid_grad_accumulation()
         data_loader = self._prepare_data_loader(
             data_loader, poisson_sampling=poisson_sampling, batch_first=batch_first, rand_on_empty=rand_on_empty
         )

@@ -724,6 +724,35 @@ def test_make_private_trains(A, mode):
     assert all(torch.isfinite(p).all() for p in net.parameters())
 
 
+@pytest.mark.parametrize("mode", ["hooks", "ghost"])
+def test_make_private_with_poisson_batches_including_empty_ones(A, mode):
+    """The default ``poisson_sampling=True``: batch sizes vary and some draws are empty
+    (sample rate 1/8 over 12 items); every step must go through, empty ones adding pure noise."""
+    torch.manual_seed(14)
+    net = nn.Sequential(nn.Linear(6, 8), nn.ReLU(), nn.Linear(8, 3)).to(DEV)
+    ds = TensorDataset(torch.randn(12, 6), torch.randint(0, 3, (12,)))
+    dl = DataLoader(ds, batch_size=1, generator=torch.Generator().manual_seed(3))
+    engine = A.PrivacyEngine()
+    out = engine.make_private(
+        module=net, optimizer=torch.optim.SGD(net.parameters(), lr=0.05), data_loader=DataLoader(ds, batch_size=2),
+        noise_multiplier=0.5, max_grad_norm=1.0, grad_sample_mode=mode,
+        noise_generator=torch.Generator(device=DEV).manual_seed(1),
+    )
+    model, opt, loader = out[0], out[1], out[-1]
+    crit = out[2] if mode == "ghost" else nn.CrossEntropyLoss()
+    loader.batch_sampler.generator = torch.Generator().manual_seed(5)
+    sizes = []
+    for _ in range(6):
+        for x, y in loader:
+            sizes.append(len(y))
+            opt.zero_grad()
+            crit(model(x.to(DEV)), y.to(DEV)).backward()
+            opt.step()
+    assert 0 in sizes and max(sizes) >= 3, sizes
+    assert len(engine.accountant) == len(sizes) == 36
+    assert all(torch.isfinite(p).all() for p in net.parameters())
+
+
 def test_mixed_precision_dtypes(A):
     """mixed_precision_test.py:107-213 checks dtypes only: fp32 parameters under bf16 autocast keep
     fp32 grads; bf16 parameters give bf16 grads."""

@@ -602,9 +602,6 @@ def test_make_private_errors():
     common = dict(data_loader=_loader(), noise_multiplier=1.0, max_grad_norm=1.0)
     with pytest.raises(ValueError, match="Module parameters are different"):
         engine.make_private(module=net, optimizer=torch.optim.SGD(other.parameters(), lr=0.1), poisson_sampling=False, **common)
-    with pytest.raises(NotImplementedError, match="Poisson"):
-        engine.make_private(module=net, optimizer=torch.optim.SGD(net.parameters(), lr=0.1), **common)
-    assert not hasattr(net, "autograd_grad_sample_hooks")  # refused before anything was attached
     wrapped = GradSampleModule(net, loss_reduction="sum")
     with pytest.raises(ValueError, match="Pre-existing GradSampleModule"):
         engine.make_private(module=wrapped, optimizer=torch.optim.SGD(net.parameters(), lr=0.1), poisson_sampling=False, **common)
@@ -613,6 +610,67 @@ def test_make_private_errors():
         module=net, optimizer=torch.optim.SGD(net.parameters(), lr=0.1), poisson_sampling=False, wrap_model=False, **common
     )
     assert isinstance(hooks_obj, GradSampleHooks) and not isinstance(hooks_obj, nn.Module)
+
+
+def test_poisson_sampler_and_empty_batches():
+    """uniform_sampler.py:22-70 and data_loader.py:30-147: independent inclusion with probability
+    ``sample_rate``, ``int(1 / sample_rate)`` batches per epoch, reproducible from the generator; an
+    empty draw is collated into tensors with a batch dimension of zero."""
+    from opacus_amd.data_loader import DPDataLoader, wrap_collate_with_empty
+    from opacus_amd.utils.uniform_sampler import UniformWithReplacementSampler
+
+    g = torch.Generator().manual_seed(0)
+    sampler = UniformWithReplacementSampler(num_samples=1000, sample_rate=0.1, generator=g)
+    batches = list(sampler)
+    assert len(batches) == len(sampler) == 10
+    sizes = torch.tensor([len(b) for b in batches], dtype=torch.float64)
+    assert abs(sizes.mean().item() - 100) < 4 * (90 / 10) ** 0.5  # Binomial(1000, 0.1), ten draws
+    assert all(b == sorted(set(b)) and 0 <= b[0] and b[-1] < 1000 for b in batches)
+    again = list(UniformWithReplacementSampler(num_samples=1000, sample_rate=0.1, generator=torch.Generator().manual_seed(0)))
+    assert again == batches
+    with pytest.raises(ValueError):
+        UniformWithReplacementSampler(num_samples=0, sample_rate=0.5)
+
+    from torch.utils.data._utils.collate import default_collate
+
+    collate = wrap_collate_with_empty(
+        collate_fn=default_collate, sample_empty_shapes=[(0, 4), (0,)], dtypes=[torch.float32, torch.int64]
+    )
+    first_empty = collate([])
+    assert [tuple(t.shape) for t in first_empty] == [(0, 4), (0,)] and first_empty[1].dtype == torch.int64
+    full = collate([(torch.ones(4), torch.tensor(1)), (torch.zeros(4), torch.tensor(0))])
+    assert full[0].shape == (2, 4)
+    empty = collate([])
+    assert type(empty) is type(full) and empty[0].shape == (0, 4) and empty[1].shape == (0,) and empty[1].dtype == torch.int64
+    rnd = wrap_collate_with_empty(collate_fn=default_collate, rand_on_empty=True)
+    rnd([(torch.ones(4), torch.tensor(1))])
+    assert rnd([])[0].shape == (1, 4)
+    nested = wrap_collate_with_empty(collate_fn=None)
+    nested({"x": torch.ones(3, 2), "y": [torch.ones(3)]})
+    e = nested([])
+    assert e["x"].shape == (0, 2) and e["y"][0].shape == (0,)
+    bad = wrap_collate_with_empty(collate_fn=None)
+    bad(["text"])
+    with pytest.raises(TypeError):
+        bad([])
+
+    base = _loader(n=64, bs=8)
+    dp = DPDataLoader.from_data_loader(base, generator=torch.Generator().manual_seed(1))
+    assert dp.sample_rate == 1 / 8 and len(dp) == 8
+    seen = [len(y) for _, y in dp]
+    assert len(seen) == 8 and len(set(seen)) > 1  # sizes vary
+
+
+def test_make_private_with_poisson_sampling_is_the_default():
+    net = nn.Linear(4, 2)
+    model, opt, dl = PrivacyEngine().make_private(
+        module=net, optimizer=torch.optim.SGD(net.parameters(), lr=0.1), data_loader=_loader(n=32, bs=4),
+        noise_multiplier=1.0, max_grad_norm=1.0,
+    )
+    from opacus_amd.data_loader import DPDataLoader
+
+    assert isinstance(dl, DPDataLoader) and dl.sample_rate == 1 / 8 and opt.expected_batch_size == 4
+    assert model.grad_accumulation_allowed is False  # privacy_engine.py:429-430
 
 
 def test_package_surface():

@@ -206,6 +206,36 @@ def test_per_layer_clip_factors_and_accumulate(K):
         assert_rel(o, w, FP32_REL)
 
 
+def test_empty_batch_through_every_wrapper(K):
+    """n == 0 (a Poisson draw can be empty): every wrapper returns tensors of the right shape with a
+    leading zero and launches nothing that could fault."""
+    e = lambda *shape, dtype=torch.float32: torch.empty(*shape, device="cuda", dtype=dtype)  # noqa: E731
+    gs, ss = K.linear_grad_sample(e(0, 5), e(0, 7))
+    assert gs.shape == (0, 5, 7) and ss.shape == (0,)
+    assert K.linear_grad_sample(e(0, 3, 5), e(0, 3, 7))[0].shape == (0, 5, 7)
+    assert K.linear_bias_grad_sample(e(0, 3, 5)).shape == (0, 5)
+    nw, nb = K.linear_ghost_norm(e(0, 3, 5), e(0, 3, 7), want_bias=True)
+    assert nw.shape == (0,) and nb.shape == (0,)
+    assert K.conv2d_grad_sample(e(0, 2, 6, 6), e(0, 4, 4, 4), (3, 3), (1, 1), (0, 0, 0, 0), (1, 1), 1)[0].shape == (0, 4, 2, 3, 3)
+    assert K.conv_bias_grad_sample(e(0, 4, 4, 4)).shape == (0, 4)
+    ids = e(0, 6, dtype=torch.int64)
+    assert K.embedding_grad_sample(ids, e(0, 6, 4), 9).shape == (0, 9, 4)
+    assert K.embedding_ghost_norm(ids, e(0, 6, 4)).shape == (0,)
+    assert K.embedding_bag_grad_sample(e(0, dtype=torch.int64), e(0, dtype=torch.int64), e(0, 4), 9).shape == (0, 9, 4)
+    gw, gb = K.group_norm_grad_sample(e(0, 4, 5), e(0, 4, 5), 2, 1e-5)
+    assert gw.shape == (0, 4) and gb.shape == (0, 4)
+    assert K.rms_norm_grad_sample(e(0, 3, 8), e(0, 3, 8), 8, 1e-5).shape == (0, 8)
+    assert K.layer_norm_grad_sample(e(0, 3, 8), e(0, 3, 8), 8, 1e-5)[0].shape == (0, 8)
+    assert K.sumsq_rows([e(0, 5, 7), e(0, 3)]).shape == (2, 0)
+    norm, clip = K.clip_factor(e(2, 0), 1.0)
+    assert norm.shape == (0,) and clip.shape == (0,)
+    assert K.clip_factor_per_layer(e(2, 0), [1.0, 2.0]).shape == (2, 0)
+    fresh, kept = torch.full((5, 7), 3.0, device="cuda"), torch.full((3,), 3.0, device="cuda")
+    K.clip_accumulate([e(0, 5, 7)], clip, [fresh], accumulate=False)
+    K.clip_accumulate([e(0, 3)], clip, [kept], accumulate=True)
+    assert fresh.abs().sum() == 0 and (kept == 3.0).all()  # an empty sum is zero; accumulating it changes nothing
+
+
 # ---- Noise ---------------------------------------------------------------------------
 def test_add_noise_zero_std_is_exact(K):
     torch.manual_seed(5)
