@@ -173,9 +173,12 @@ def workload_c2(dev):
         step=step, n=N, dtype="f32",
         workload="Linear(4096->4096, bias) fp32, batch 128, T=1, hooks per-sample grad + clip(C=1) + noise(sigma=1) + SGD",
         extra={"per_sample_grad_bytes": N * P * 4},
-        # one launch covers weight and bias: reads n * P * 4 bytes, writes P * 4 bytes
+        # one call covers weight and bias: reads n * P * 4 bytes, writes P * 4 bytes. The timed span
+        # holds two dispatches: the wide kernel on the 512 whole 128 KB spans of the weight and the
+        # one-wave kernel on the 4096 bias columns (a few microseconds).
         roofline=dict(
-            kernel="clip_accumulate_kernel<float,float,vec,RS=1,64 threads,U=16>", timer="clip_accumulate",
+            kernel="clip_accumulate_wide_kernel<float,float> (+ clip_accumulate_kernel on the bias, same call)",
+            timer="clip_accumulate",
             bound="hbm", work_per_launch=float(N * P * 4 + P * 4), unit="GB/s", peak=HBM_PEAK_GBS,
             # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (KiB per
             # dispatch), each scaled by what the counter reads for a 1 GiB device copy

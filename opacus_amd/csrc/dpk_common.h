@@ -74,6 +74,16 @@ template <> struct dpk_io<float> {
   static __device__ __forceinline__ void store4(float* p, float4 v) {
     *reinterpret_cast<float4*>(p) = v;
   }
+  // store4 with a non-temporal hint: for output that nobody re-reads before it has
+  // left the caches anyway
+  static __device__ __forceinline__ void store4_nt(float* p, float4 v) {
+    dpk_vf4 w;
+    w.x = v.x;
+    w.y = v.y;
+    w.z = v.z;
+    w.w = v.w;
+    __builtin_nontemporal_store(w, reinterpret_cast<dpk_vf4*>(p));
+  }
 };
 template <> struct dpk_io<bf16_t> {
   static __device__ __forceinline__ float4 load4_nt(const bf16_t* p) {
@@ -102,6 +112,12 @@ template <> struct dpk_io<bf16_t> {
     r.x = static_cast<uint32_t>(f32_to_bf16(v.x)) | (static_cast<uint32_t>(f32_to_bf16(v.y)) << 16);
     r.y = static_cast<uint32_t>(f32_to_bf16(v.z)) | (static_cast<uint32_t>(f32_to_bf16(v.w)) << 16);
     *reinterpret_cast<uint2*>(p) = r;
+  }
+  static __device__ __forceinline__ void store4_nt(bf16_t* p, float4 v) {
+    dpk_vu2 r;
+    r.x = static_cast<uint32_t>(f32_to_bf16(v.x)) | (static_cast<uint32_t>(f32_to_bf16(v.y)) << 16);
+    r.y = static_cast<uint32_t>(f32_to_bf16(v.z)) | (static_cast<uint32_t>(f32_to_bf16(v.w)) << 16);
+    __builtin_nontemporal_store(r, reinterpret_cast<dpk_vu2*>(p));
   }
 };
 

@@ -176,6 +176,34 @@ def test_clip_accumulate_many_tensors(K):
         assert_rel(o, s, FP32_REL)
 
 
+def test_clip_accumulate_very_large_tensors(K):
+    """The shape for tensors past 8.4 M elements in total: blocks own 32768-element spans, so cover
+    a ragged last span, a tensor shorter than one span, per-layer factors, fp32 and bf16
+    gradients, and accumulation into a previous sum."""
+    torch.manual_seed(41)
+    n = 3
+    sizes = [257 * 32768 + 4 * 1237, 1000, 2 * 32768]
+    gs = [torch.randn(n, p) for p in sizes]
+    dgs = [dev(g) for g in gs]
+    clip = torch.tensor([[0.5, 1.0, 0.25], [1.0, 0.125, 0.75], [0.3, 0.6, 0.9]])
+    want = [(c[:, None].double() * g.double()).sum(0) for c, g in zip(clip, gs)]
+    outs = [torch.full((p,), float("nan"), device="cuda") for p in sizes]
+    K.clip_accumulate(dgs, dev(clip), outs, accumulate=False)
+    for o, w in zip(outs, want):
+        assert_rel(o, w, FP32_REL, "very large, fresh")
+    K.clip_accumulate(dgs, dev(clip), outs, accumulate=True)
+    for o, w in zip(outs, want):
+        assert_rel(o, 2 * w, FP32_REL, "very large, accumulated")
+    shared = dev(clip[0].contiguous())
+    K.clip_accumulate(dgs, shared, outs, accumulate=False)
+    for o, g in zip(outs, gs):
+        assert_rel(o, (clip[0][:, None].double() * g.double()).sum(0), FP32_REL, "very large, one factor row")
+    g16 = [g.bfloat16() for g in gs]
+    K.clip_accumulate([dev(g) for g in g16], shared, outs, accumulate=False)
+    for o, g in zip(outs, g16):
+        assert_rel(o, (clip[0][:, None].double() * g.double()).sum(0), FP32_REL, "very large, bf16 gradients")
+
+
 def test_per_layer_clip_factors_and_accumulate(K):
     """[K, n] factor table: row k from parameter k's own norm and bound; bf16 and fp32 tensors,
     fresh and accumulating, more tensors than one launch holds."""
