@@ -64,7 +64,20 @@ __global__ __launch_bounds__(kThreads) void sumsq_partial_kernel(MultiArgs a, in
   const int64_t lo = chunk * kSumsqChunk;
   const int64_t hi = (lo + kSumsqChunk < P) ? lo + kSumsqChunk : P;
   float acc0 = 0.f, acc1 = 0.f, acc2 = 0.f, acc3 = 0.f;
-  if (VEC) {
+  if (VEC && hi - lo == kSumsqChunk) {
+    // a whole chunk: all of the thread's loads in flight at once, read-once data
+    constexpr int kPer = kSumsqChunk / (kThreads * 4);
+    float4 v[kPer];
+#pragma unroll
+    for (int u = 0; u < kPer; ++u) v[u] = dpk_io<T>::load4_nt(rowp + lo + (u * kThreads + threadIdx.x) * 4);
+#pragma unroll
+    for (int u = 0; u < kPer; ++u) {
+      acc0 += v[u].x * v[u].x;
+      acc1 += v[u].y * v[u].y;
+      acc2 += v[u].z * v[u].z;
+      acc3 += v[u].w * v[u].w;
+    }
+  } else if (VEC) {
     for (int64_t i = lo + threadIdx.x * 4; i < hi; i += kThreads * 4) {
       float4 v = dpk_io<T>::load4(rowp + i);
       acc0 += v.x * v.x;
