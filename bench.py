@@ -182,8 +182,8 @@ def workload_c2(dev):
             bound="hbm", work_per_launch=float(N * P * 4 + P * 4), unit="GB/s", peak=HBM_PEAK_GBS,
             # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (KiB per
             # dispatch), each scaled by what the counter reads for a 1 GiB device copy
-            # (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000): 8,390,223 + 65,552 KiB.
-            traffic=8455775 * 1024,
+            # (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000): 8,390,260 + 65,551 KiB over the two dispatches.
+            traffic=8455811 * 1024,
         ),
     )
 
