@@ -5,6 +5,8 @@ Mirror of opacus/utils/fast_gradient_clipping_utils.py.
 
 from __future__ import annotations
 
+import copy
+
 import torch
 
 
@@ -21,7 +23,10 @@ class DPTensorFastGradientClipping:
         self.loss_reduction = loss_reduction
 
     def _like(self, loss_per_sample: torch.Tensor) -> "DPTensorFastGradientClipping":
-        return DPTensorFastGradientClipping(self.module, self.optimizer, loss_per_sample, self.loss_reduction)
+        # a shallow copy, so that subclasses keep their own settings
+        new = copy.copy(self)
+        new.loss_per_sample = loss_per_sample
+        return new
 
     def _other(self, other):
         if isinstance(other, DPTensorFastGradientClipping):

@@ -28,7 +28,10 @@ What pins each function (see ``tests/test_oracle_pins.py``):
     is and checked on a hand-computed case);
   * per-layer clipping: reduces to flat clipping for one parameter, to the plain sum for
     huge bounds, and bounds every parameter's norm by its own C_k; AdaClip's count and
-    bound update: hand-checked numbers;
+    bound update: hand-checked numbers; the ghost-mode adaptive update: hand-checked
+    numbers, the fixed point at the target quantile, the composition identity
+    sigma'^-2 + (2 n/20)^-2 == sigma^-2, and coefficients that scale every clipped sample
+    to exactly the new bound;
   * Philox4x32-10: the Random123 known-answer vectors.
 No function here is "parity unpinned".
 """
@@ -424,6 +427,34 @@ def adaclip_update(
     count = float(n - int((clip < 1).sum())) + count_noise
     new = max_grad_norm * math.exp(-learning_rate * (count / n - target_quantile))
     return count, min(max(new, min_bound), max_bound)
+
+
+def ghost_adaptive_update(
+    per_sample_norms: torch.Tensor,
+    max_grad_norm: float,
+    target_quantile: float,
+    learning_rate: float,
+    min_bound: float,
+    max_bound: float,
+    noise_multiplier: float,
+    count_noise: float = 0.0,
+) -> Tuple[float, float, torch.Tensor]:
+    """opacus/utils/adaptive_clipping/adaptive_clipping_utils.py:77-175: the ghost-clipping
+    variant of adaptive clipping. Counts ``norm <= C`` (plus ``count_noise``, a draw of
+    N(0, (n/20)^2)), moves C geometrically, raises the noise multiplier to
+    ``(sigma^-2 - (2 n/20)^-2)^-1/2``, and returns the coefficients of the second backward
+    pass from the *new* bound: 1 where ``norm <= C'``, else ``C' / norm`` (no 1e-6 here).
+    Returns (new bound, new noise multiplier, coefficients)."""
+    n = len(per_sample_norms)
+    count = float((per_sample_norms <= max_grad_norm).sum()) + count_noise
+    new = max_grad_norm * math.exp(-learning_rate * (count / n - target_quantile))
+    new = min(max(new, min_bound), max_bound)
+    std = n / 20.0
+    sigma = noise_multiplier
+    if noise_multiplier > 0:
+        sigma = (noise_multiplier ** (-2) - (2.0 * std) ** (-2)) ** (-0.5)
+    coeff = torch.where(per_sample_norms <= new, torch.ones_like(per_sample_norms), new / per_sample_norms)
+    return new, sigma, coeff
 
 
 def generate_noise(std: float, reference: torch.Tensor, generator=None, secure_mode: bool = False) -> torch.Tensor:

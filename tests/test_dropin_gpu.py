@@ -700,6 +700,49 @@ def test_ghost_tied_parameters_raise(A):
         ghost(torch.randn(2, 6, device=DEV))
 
 
+def test_ghost_adaptive_clipping_engine_step_matches_oracle(A, monkeypatch):
+    """adaptive_clipping_utils.py:77-121 end to end: the norms of backward #1 feed the bound
+    update, and the clipped sum of backward #2 equals sum_n coeff[n] * g[n] with the oracle's
+    coefficients of the new bound (sigma = 0, count noise pinned to zero)."""
+    from opacus_amd.utils.adaptive_clipping import DPLossFastGradientAdaptiveClipping, PrivacyEngineAdaptiveClipping
+
+    torch.manual_seed(21)
+    mlp = nn.Sequential(nn.Linear(24, 40), nn.GELU(), nn.Linear(40, 12))
+    n, T, C = 12, 9, 0.3
+    x, y = torch.randn(n, T, 24), torch.randn(n, T, 12)
+    x[: n // 2] *= 0.05  # small inputs, small gradients: some samples end up under the bound
+    ds = TensorDataset(x, y)
+    dl = DataLoader(ds, batch_size=n)
+
+    # per-sample gradients and norms by the materialising path
+    hooks = A.GradSampleModule(copy.deepcopy(mlp).to(DEV), loss_reduction="mean")
+    PerSampleMSE("mean")(hooks(x.to(DEV)), y.to(DEV)).backward()
+    gs = [p.grad_sample.double().cpu() for p in hooks.parameters()]
+    norms = torch.stack([g.flatten(1).norm(dim=1) for g in gs]).norm(dim=0)
+    want_bound, want_sigma, coeff = O.ghost_adaptive_update(norms, C, 0.6, 0.3, 1e-4, 10.0, 0.0)
+    assert 0 < (norms <= C).sum() < n and want_bound != C
+
+    monkeypatch.setattr(torch, "normal", lambda **kw: torch.zeros(kw["size"]))  # the count's noise
+    net = copy.deepcopy(mlp).to(DEV)
+    engine = PrivacyEngineAdaptiveClipping()
+    model, opt, crit, _ = engine.make_private(
+        module=net, optimizer=torch.optim.SGD(net.parameters(), lr=1.0), criterion=PerSampleMSE("mean"), data_loader=dl,
+        noise_multiplier=0.0, max_grad_norm=C, poisson_sampling=False, grad_sample_mode="ghost",
+        target_unclipped_quantile=0.6, min_clipbound=1e-4, max_clipbound=10.0, clipbound_learning_rate=0.3,
+    )
+    assert isinstance(crit, DPLossFastGradientAdaptiveClipping)
+    before = [p.detach().double().cpu().clone() for p in net.parameters()]
+    opt.zero_grad()
+    crit(model(x.to(DEV)), y.to(DEV)).backward()
+    close(model.per_sample_gradient_norms, norms, 1e-4, 1e-8)
+    assert model.max_grad_norm == opt.max_grad_norm == pytest.approx(want_bound, rel=1e-5)
+    assert opt._adjusted_noise_multiplier == 0.0
+    opt.step()
+    for p, b, g in zip(net.parameters(), before, gs):
+        want = b - (coeff.double().view(-1, *[1] * (g.dim() - 1)) * g).sum(0) / n
+        close(p, want, 1e-4, 1e-6)
+
+
 # ---- make_private end to end ----------------------------------------------------------------------
 @pytest.mark.parametrize("mode", ["hooks", "ghost"])
 def test_make_private_trains(A, mode):

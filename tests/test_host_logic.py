@@ -12,6 +12,8 @@ import torch.nn as nn
 import torch.nn.functional as F
 from torch.utils.data import DataLoader, TensorDataset
 
+from oracle import dp_oracle as O
+
 import opacus_amd
 from opacus_amd import (
     DPOptimizer,
@@ -526,6 +528,44 @@ def test_dp_tensor_backward_order():
     assert calls == ["zero_grad", "coef", "off", "on"]
     # first backward left [2, 3]; it was not zeroed by the mock; second adds coef * [2, 3]
     torch.testing.assert_close(w.grad, torch.tensor([2.0 + 1.0, 3.0 + 3.0]))
+
+
+def test_adaptive_dp_tensor_updates_bound_noise_and_uses_new_bound(monkeypatch):
+    """adaptive_clipping_utils.py:77-121: between the two passes the bound and the adjusted
+    noise multiplier are written to module and optimizer, and the second pass is weighted with
+    coefficients of the new bound."""
+    from opacus_amd.utils.adaptive_clipping import DPTensorFastGradientAdaptiveClipping
+
+    module, optimizer = _mock_pair("sum")
+    module.max_grad_norm = optimizer.max_grad_norm = 1.0
+    optimizer.noise_multiplier = 0.0
+    norms = torch.tensor([0.5, 1.0, 2.0, 4.0] * 3)  # half unclipped at C = 1
+    module.get_norm_sample.side_effect = lambda: norms
+    monkeypatch.setattr(torch, "normal", lambda **kw: torch.zeros(kw["size"]))
+    w = torch.ones(12, requires_grad=True)
+    base = torch.arange(1.0, 13.0)
+    loss = DPTensorFastGradientAdaptiveClipping(
+        module, optimizer, w * base, "sum", target_unclipped_quantile=0.75, min_clipbound=0.1, max_clipbound=10.0,
+        clipbound_learning_rate=0.2, initial_noise_multiplier=0.0,
+    )
+    assert isinstance(loss * 2, DPTensorFastGradientAdaptiveClipping) and (loss * 2).target_unclipped_quantile == 0.75
+    loss.backward()
+    want_bound, want_sigma, coeff = O.ghost_adaptive_update(norms, 1.0, 0.75, 0.2, 0.1, 10.0, 0.0)
+    assert module.max_grad_norm == optimizer.max_grad_norm == pytest.approx(want_bound, rel=1e-12)
+    assert optimizer._adjusted_noise_multiplier == want_sigma == 0.0
+    torch.testing.assert_close(w.grad, base + coeff * base)  # pass 1 (not zeroed by the mock) + weighted pass 2
+
+    # noise multiplier: the composition formula, and the batch-size guard
+    module.max_grad_norm = optimizer.max_grad_norm = 1.0
+    loss = DPTensorFastGradientAdaptiveClipping(module, optimizer, (w * base).detach().requires_grad_(), "sum", initial_noise_multiplier=1.0)
+    loss.backward()
+    assert optimizer._adjusted_noise_multiplier == pytest.approx((1.0 - (2 * 12 / 20.0) ** -2) ** -0.5, rel=1e-12)
+    module.max_grad_norm = optimizer.max_grad_norm = 1.0
+    with pytest.raises(AssertionError, match="Batch size is too small"):
+        DPTensorFastGradientAdaptiveClipping(module, optimizer, (w * base).detach().requires_grad_(), "sum", initial_noise_multiplier=1.2).backward()
+    optimizer.max_grad_norm = 2.0
+    with pytest.raises(AssertionError, match="does not match"):
+        DPTensorFastGradientAdaptiveClipping(module, optimizer, (w * base).detach().requires_grad_(), "sum", initial_noise_multiplier=0.0).backward()
 
 
 def test_dp_loss_requires_consistent_reductions_and_restores_reduction():

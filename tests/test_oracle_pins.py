@@ -466,3 +466,30 @@ def test_philox_normal_moments():
     assert abs((z**3).mean()) < 2e-2 and abs((z**4).mean() - 3.0) < 5e-2
     z2 = O.philox_normal(1_000_000, seed=1234, offset=8)
     assert abs(np.corrcoef(z, z2)[0, 1]) < 5e-3
+
+
+def test_ghost_adaptive_update_hand_numbers_and_identities():
+    """adaptive_clipping_utils.py:123-175 by hand. norms (0.5, 1, 2, 4), C = 1: two of four are
+    unclipped (<=), so at target 0.5 the bound is a fixed point; at target 0.75 it grows by
+    exp(0.2 * 0.25)."""
+    norms = torch.tensor([0.5, 1.0, 2.0, 4.0])
+    new, sigma, coeff = O.ghost_adaptive_update(norms, 1.0, 0.5, 0.2, 0.1, 10.0, noise_multiplier=0.0)
+    assert new == 1.0 and sigma == 0.0
+    assert torch.equal(coeff, torch.tensor([1.0, 1.0, 0.5, 0.25]))
+    new, _, coeff = O.ghost_adaptive_update(norms, 1.0, 0.75, 0.2, 0.1, 10.0, 0.0)
+    assert new == pytest.approx(math.exp(0.05), rel=1e-12)
+    # every clipped sample lands exactly on the new bound, unclipped ones are untouched
+    scaled = coeff.double() * norms.double()
+    assert torch.allclose(scaled[2:], torch.full((2,), new, dtype=torch.float64), rtol=1e-6)
+    assert torch.equal(scaled[:2], norms[:2].double())
+    # the count noise enters the fraction additively: +1 sample of noise at n = 4 is +0.25
+    noisy, _, _ = O.ghost_adaptive_update(norms, 1.0, 0.5, 0.2, 0.1, 10.0, 0.0, count_noise=1.0)
+    assert noisy == pytest.approx(math.exp(-0.2 * 0.25), rel=1e-12)
+    # clamps
+    assert O.ghost_adaptive_update(norms, 1.0, 1.0, 50.0, 0.1, 3.0, 0.0)[0] == 3.0
+    assert O.ghost_adaptive_update(norms, 1.0, 0.0, 50.0, 0.4, 3.0, 0.0)[0] == 0.4
+    # privacy composition of the two Gaussian mechanisms: sigma'^-2 + (2 n / 20)^-2 == sigma^-2
+    big = torch.rand(200)
+    _, sigma, _ = O.ghost_adaptive_update(big, 1.0, 0.5, 0.2, 0.1, 10.0, noise_multiplier=1.3)
+    assert sigma > 1.3
+    assert sigma ** -2 + (2 * 200 / 20.0) ** -2 == pytest.approx(1.3 ** -2, rel=1e-12)
