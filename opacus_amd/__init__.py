@@ -6,7 +6,7 @@ and error behaviour; the arithmetic runs in hand-written HIP kernels (``libdpsgd
 C ABI in ``include/dpk.h``) on the GPU that holds the tensors. There is no CPU path.
 """
 
-from . import grad_sample, optimizers
+from . import grad_sample, layers, optimizers
 from .grad_sample import (
     GradSampleHooks,
     GradSampleHooksFastGradientClipping,
@@ -34,5 +34,6 @@ __all__ = [
     "register_grad_sampler",
     "register_norm_sampler",
     "grad_sample",
+    "layers",
     "optimizers",
 ]

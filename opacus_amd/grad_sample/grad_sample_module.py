@@ -130,7 +130,9 @@ class GradSampleHooks(AbstractGradSampleHooks):
         """Modules that get hooks: every one with trainable parameters of its own. Below a
         module that has them but no registered sampler nothing is visited: the generic
         fallback differentiates that whole subtree (grad_sample_module.py:152-165)."""
-        own = has_trainable_params(module)
+        # a module that only lists its children's parameters under other names (DPLSTM and
+        # its kind, grad_sample_module.py:202-204) gets no hook of its own
+        own = has_trainable_params(module) and not getattr(module, "grad_sample_through_children", False)
         if own:
             yield module
             if self._get_module_type(module) not in self.GRAD_SAMPLERS:
@@ -231,6 +233,13 @@ class GradSampleHooks(AbstractGradSampleHooks):
             module=module, backprops=backprops, loss_reduction=loss_reduction, batch_first=batch_first
         )
         sampler = self._sampler_for(module)
+        if getattr(module, "stack_uses", False):
+            stacked = self._stack_uses(module, activations, backprops)
+            if stacked is None:
+                return  # earlier uses of this pass are still to come
+            activations, backprops = stacked
+            for _, p in trainable_parameters(module):
+                p._forward_counter += 1  # taken off again below, as for a module used once
         grad_samples = call_sampler(sampler, module, activations, backprops, scale)
         adopt = getattr(sampler, "owns_output", False)
         for param, gs in grad_samples.items():
@@ -251,6 +260,35 @@ class GradSampleHooks(AbstractGradSampleHooks):
         if len(module.activations) == 0 and hasattr(module, "max_batch_len"):
             del module.max_batch_len
 
+    def _stack_uses(self, module: nn.Module, activations: List[torch.Tensor], backprops: torch.Tensor):
+        """For a module applied many times per forward pass (``stack_uses``, the RNNLinear
+        of the recurrent layers): keeps this use's activations and backprops and takes the use
+        off the parameters' forward counters. Once the counters are back at zero, returns
+        every use of the pass stacked along a new dimension 1, so that the sampler sums over
+        the uses inside one contraction instead of the hooks adding one full per-sample
+        gradient per use in memory (what grad_sample_module.py:43-66 does for such layers).
+        Uses that saw fewer samples than ``max_batch_len`` are padded with zero rows."""
+        pending = module.__dict__.setdefault("_pending_uses", [])
+        pending.append((activations, backprops))
+        done = True
+        for _, p in trainable_parameters(module):
+            p._forward_counter -= 1
+            done = done and p._forward_counter == 0
+        if not done:
+            return None
+        module.__dict__.pop("_pending_uses")
+        if len(pending) == 1:
+            return pending[0]
+        n = module.max_batch_len
+
+        def rows(t: torch.Tensor) -> torch.Tensor:
+            if t.shape[0] == n:
+                return t
+            return torch.cat([t, t.new_zeros((n - t.shape[0],) + tuple(t.shape[1:]))], dim=0)
+
+        acts = [torch.stack([rows(u[0][i]) for u in pending], dim=1) for i in range(len(pending[0][0]))]
+        return acts, torch.stack([rows(u[1]) for u in pending], dim=1)
+
     def _take_activations(
         self, *, module: nn.Module, backprops: torch.Tensor, loss_reduction: str, batch_first: bool
     ) -> Tuple[List[torch.Tensor], torch.Tensor, float]:
@@ -258,7 +296,9 @@ class GradSampleHooks(AbstractGradSampleHooks):
         (not yet scaled) and the factor that turns them into sum-loss backprops."""
         if not hasattr(module, "activations"):
             raise ValueError(f"No activations detected for {type(module)}, run forward after add_hooks(model)")
-        batch_dim = 0 if batch_first else 1
+        # the recurrent layers feed their RNNLinear batch first whatever the model's layout
+        # (grad_sample_module.py:391)
+        batch_dim = 0 if batch_first or getattr(module, "stack_uses", False) else 1
         if not hasattr(module, "max_batch_len"):
             module.max_batch_len = _get_batch_size(module=module, batch_dim=batch_dim)
         activations = module.activations.pop()

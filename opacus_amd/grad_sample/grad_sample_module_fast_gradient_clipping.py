@@ -111,7 +111,12 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
         module.activations.append([t.detach() for t in forward_input if isinstance(t, torch.Tensor)])
         for _, p in trainable_parameters(module):
             p._forward_counter += 1
-            if self.use_ghost_clipping and p._forward_counter > 1 and type(module) in self.NORM_SAMPLERS:
+            if (
+                self.use_ghost_clipping
+                and p._forward_counter > 1
+                and type(module) in self.NORM_SAMPLERS
+                and not getattr(module, "stack_uses", False)  # its uses are contracted together
+            ):
                 # the norm of a sum of two layers' gradients is not a function of their norms
                 raise NotImplementedError("Parameter tying is not supported with Ghost Clipping")
 
@@ -125,6 +130,13 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
         activations, backprops, scale = self._take_activations(
             module=module, backprops=backprops, loss_reduction=loss_reduction, batch_first=batch_first
         )
+        if getattr(module, "stack_uses", False):
+            stacked = self._stack_uses(module, activations, backprops)
+            if stacked is None:
+                return
+            activations, backprops = stacked
+            for _, p in trainable_parameters(module):
+                p._forward_counter += 1  # taken off again below, as for a module used once
         if self.use_ghost_clipping and type(module) in self.NORM_SAMPLERS:
             norm_samples = call_sampler(self.NORM_SAMPLERS[type(module)], module, activations, backprops, scale)
             for param, ns in norm_samples.items():

@@ -294,6 +294,83 @@ def test_sequence_model_grad_samples(A, batch_first):
         close(p.grad_sample, want[k], 1e-4, 1e-5, k)
 
 
+class RecurrentNet(nn.Module):
+    """A recurrent layer and a Linear head on its last output (batch-first tensors), or on the
+    final hidden state for packed input."""
+
+    def __init__(self, rnn):
+        super().__init__()
+        self.rnn = rnn
+        self.head = nn.Linear(rnn.hidden_size * (2 if rnn.bidirectional else 1), 3)
+
+    def forward(self, x):
+        out, state = self.rnn(x)
+        if isinstance(out, torch.nn.utils.rnn.PackedSequence):
+            h = state[0] if isinstance(state, tuple) else state
+            last = torch.cat([h[-2], h[-1]], dim=1) if self.rnn.bidirectional else h[-1]
+        else:
+            last = out.mean(dim=1 if self.rnn.batch_first else 0)  # every step feeds the loss
+        return self.head(last)
+
+
+@pytest.mark.parametrize("kind", ["lstm", "gru", "rnn"])
+@pytest.mark.parametrize("packed", [False, True])
+def test_recurrent_layers_grad_samples_and_ghost_norms(A, kind, packed):
+    """dp_rnn_test.py / grad_samples/dp_rnn_test.py: DPLSTM, DPGRU, DPRNN produce torch.nn's
+    outputs from torch.nn's state dict, and their per-sample gradients (input projection
+    contracted over time in one call, recurrent projection over its stacked uses) equal
+    batch-of-one autograd through the torch.nn module; two layers, bidirectional, packed
+    sequences of unsorted lengths (row i of every gradient is sample i of the caller's batch,
+    also for the recurrent parameters); ghost norms equal the norms of those gradients."""
+    from torch.nn.utils.rnn import pack_padded_sequence
+
+    from opacus_amd.layers import DPGRU, DPLSTM, DPRNN
+
+    torch.manual_seed(31 + packed)
+    DP, NN = {"lstm": (DPLSTM, nn.LSTM), "gru": (DPGRU, nn.GRU), "rnn": (DPRNN, nn.RNN)}[kind]
+    kw = dict(num_layers=2, bidirectional=True, batch_first=True)
+    ref = RecurrentNet(NN(5, 6, **kw))
+    net = RecurrentNet(DP(5, 6, **kw))
+    assert [k for k, _ in net.named_parameters()] == [k for k, _ in ref.named_parameters()]
+    net.load_state_dict(ref.state_dict())
+    n, T = 5, 7
+    x, y = torch.randn(n, T, 5), torch.randn(n, 3)
+    lengths = torch.tensor([4, 7, 2, 7, 5])
+
+    def feed(xx, ll, dev="cpu"):
+        if not packed:
+            return xx.to(dev)
+        return pack_padded_sequence(xx, ll, batch_first=True, enforce_sorted=False).to(dev)
+
+    want = {k: [] for k, _ in ref.named_parameters()}
+    for i in range(n):
+        ref.zero_grad()
+        (ref(feed(x[i : i + 1], lengths[i : i + 1])) - y[i : i + 1]).pow(2).sum().backward()
+        for k, p in ref.named_parameters():
+            want[k].append(p.grad.clone())
+    want = {k: torch.stack(v) for k, v in want.items()}
+    close(net(feed(x, lengths)), ref(feed(x, lengths)), 1e-5, 1e-6, "forward on the CPU")
+
+    gsm = A.GradSampleModule(copy.deepcopy(net).to(DEV), loss_reduction="sum")
+    out = gsm(feed(x, lengths, DEV))
+    close(out, ref(feed(x, lengths)), 1e-4, 1e-5, "forward")
+    (out - y.to(DEV)).pow(2).sum().backward()
+    for k, p in gsm._module.named_parameters():
+        assert p.grad_sample.shape == want[k].shape, k
+        close(p.grad_sample, want[k], 1e-4, 1e-5, k)
+    # a second pass must start clean (pending uses and counters were consumed)
+    gsm.zero_grad()
+    (gsm(feed(x, lengths, DEV)) - y.to(DEV)).pow(2).sum().backward()
+    for k, p in gsm._module.named_parameters():
+        close(p.grad_sample, want[k], 1e-4, 1e-5, f"second pass {k}")
+
+    ghost = A.GradSampleModuleFastGradientClipping(copy.deepcopy(net).to(DEV), loss_reduction="sum", max_grad_norm=1.0)
+    (ghost(feed(x, lengths, DEV)) - y.to(DEV)).pow(2).sum().backward()
+    for k, p in ghost._module.named_parameters():
+        assert p.grad_sample is None
+        close(p._norm_sample, want[k].flatten(1).norm(dim=1), 1e-4, 1e-6, f"ghost {k}")
+
+
 def test_accumulation_tied_parameters_and_functorch_fallback(A):
     torch.manual_seed(3)
 

@@ -713,6 +713,58 @@ def test_make_private_with_poisson_sampling_is_the_default():
     assert model.grad_accumulation_allowed is False  # privacy_engine.py:429-430
 
 
+@pytest.mark.parametrize("kind", ["lstm", "gru", "rnn_tanh", "rnn_relu"])
+def test_recurrent_layers_equal_torch_modules_and_share_their_state_dict(kind):
+    """opacus/tests/dp_layers/dp_rnn_test.py: same parameter names, state dict loadable both ways,
+    same outputs and final states as torch.nn for tensors and packed sequences (unsorted lengths,
+    initial states), over layers x directions x batch_first x bias. Forward only: no kernel runs."""
+    from torch.nn.utils.rnn import pack_padded_sequence
+
+    from opacus_amd.layers import DPGRU, DPLSTM, DPRNN
+
+    DP, NN, kw = {
+        "lstm": (DPLSTM, nn.LSTM, {}),
+        "gru": (DPGRU, nn.GRU, {}),
+        "rnn_tanh": (DPRNN, nn.RNN, {"nonlinearity": "tanh"}),
+        "rnn_relu": (DPRNN, nn.RNN, {"nonlinearity": "relu"}),
+    }[kind]
+    torch.manual_seed(5)
+    for layers, bi, bf, bias in [(1, False, False, True), (2, True, True, True), (2, True, False, False), (1, True, True, False)]:
+        ref = NN(5, 7, num_layers=layers, bidirectional=bi, batch_first=bf, bias=bias, **kw).double()
+        dp = DP(5, 7, num_layers=layers, bidirectional=bi, batch_first=bf, bias=bias, **kw).double()
+        assert [k for k, _ in dp.named_parameters()] == [k for k, _ in ref.named_parameters()]
+        assert list(dp.state_dict()) == list(ref.state_dict())
+        dp.load_state_dict(ref.state_dict())
+        ref.load_state_dict(dp.state_dict())
+        B, T = 4, 6
+        x = torch.randn(B, T, 5).double() if bf else torch.randn(T, B, 5).double()
+        h0 = torch.randn(layers * (2 if bi else 1), B, 7).double()
+        state = (h0, torch.randn_like(h0)) if kind == "lstm" else h0
+        for inp in (x, pack_padded_sequence(x, torch.tensor([3, 6, 1, 4]), batch_first=bf, enforce_sorted=False)):
+            for st in (None, state):
+                o1, s1 = ref(inp, st)
+                o2, s2 = dp(inp, st)
+                if isinstance(o1, torch.nn.utils.rnn.PackedSequence):
+                    assert torch.equal(o1.batch_sizes, o2.batch_sizes) and torch.equal(o1.sorted_indices, o2.sorted_indices)
+                    o1, o2 = o1.data, o2.data
+                torch.testing.assert_close(o2, o1, rtol=1e-10, atol=1e-12)
+                for a, b in zip(s1 if isinstance(s1, tuple) else (s1,), s2 if isinstance(s2, tuple) else (s2,)):
+                    torch.testing.assert_close(b, a, rtol=1e-10, atol=1e-12)
+    with pytest.raises(NotImplementedError):
+        DP(5, 7, proj_size=2, **kw)
+    with pytest.raises(ValueError):
+        DP(5, 7, dropout=1.5, **kw)
+
+
+def test_recurrent_layers_get_hooks_on_their_linear_maps_only():
+    from opacus_amd.layers import DPLSTM, RNNLinear
+
+    gsm = GradSampleModule(nn.Sequential(DPLSTM(4, 3, num_layers=2, bidirectional=True)))
+    hooked = list(gsm.iterate_submodules(gsm._module))
+    assert len(hooked) == 8 and all(type(m) is RNNLinear for m in hooked)
+    assert len(list(gsm.parameters())) == 16  # four cells x (ih, hh) x (weight, bias), each listed once
+
+
 def test_package_surface():
     for name in opacus_amd.__all__:
         assert hasattr(opacus_amd, name)
