@@ -70,10 +70,11 @@ class ResBlock(nn.Module):
 
 
 class Llama(nn.Module):
-    """Decoder stack: RMSNorm, grouped-query attention with rotary embedding, SwiGLU; untied
-    embedding and LM head (ghost clipping does not support tied parameters); bias-free."""
+    """Decoder stack: RMSNorm, grouped-query attention with rotary embedding, SwiGLU;
+    bias-free. ``tied=False`` keeps embedding and LM head apart, which is what the reference
+    can run (it refuses tied parameters under ghost clipping); ``tied=True`` shares the table."""
 
-    def __init__(self, vocab=32000, d=2048, heads=16, kv=4, ffn=5632, layers=4):
+    def __init__(self, vocab=32000, d=2048, heads=16, kv=4, ffn=5632, layers=4, tied=False):
         super().__init__()
         self.emb = nn.Embedding(vocab, d)
         self.heads, self.kv, self.hd = heads, kv, d // heads
@@ -95,6 +96,8 @@ class Llama(nn.Module):
         )
         self.norm = nn.RMSNorm(d, eps=1e-5)
         self.lm_head = nn.Linear(d, vocab, bias=False)
+        if tied:
+            self.lm_head.weight = self.emb.weight
 
     @staticmethod
     def rope(x):
@@ -274,12 +277,12 @@ def workload_c3(dev):
     )
 
 
-def workload_c5(dev):
+def workload_c5(dev, tied=False):
     from opacus_amd import DPLossFastGradientClipping
 
     torch.manual_seed(0)
     n, T, V = 16, 1024, 32000
-    net = Llama()
+    net = Llama(tied=tied)
     crit = {}
 
     def loss_call(model, opt, ids):
@@ -290,11 +293,19 @@ def workload_c5(dev):
 
     return _ghost_workload(
         dev, net, lambda: torch.randint(0, V, (n, T)).to(dev), loss_call, n, T, 0.8,
-        "4-layer Llama-style decoder (d 2048, 16 heads / 4 KV, SwiGLU 5632, vocab 32000, untied), bf16, batch 16, seq 1024, ghost clipping, C=1, sigma=0.8",
+        f"4-layer Llama-style decoder (d 2048, 16 heads / 4 KV, SwiGLU 5632, vocab 32000, {'tied' if tied else 'untied'}), "
+        "bf16, batch 16, seq 1024, ghost clipping, C=1, sigma=0.8",
     )
 
 
-WORKLOADS = {"c1": workload_c1, "c2": workload_c2, "c3": workload_c3, "c4": workload_c4, "c5": workload_c5}
+def workload_c5_tied(dev):
+    return workload_c5(dev, tied=True)
+
+
+WORKLOADS = {
+    "c1": workload_c1, "c2": workload_c2, "c3": workload_c3, "c4": workload_c4, "c5": workload_c5,
+    "c5t": workload_c5_tied,
+}
 
 
 def cpu_baseline(n_sample: int = 16, steps: int = 3) -> dict:
@@ -443,6 +454,13 @@ def kernel_table(dev, iters: int = 10, warm: int = 3, with_cpu: bool = True):
               cpu(lambda: O.embedding_norm_sample(cids, cb), 4, "4 of 16 samples"))
     yield row("rms_norm_gs", "a6", "C5 n=16 T=1024 D=2048 bf16", timed(lambda: K.rms_norm_grad_sample(x, b, D, 1e-5)),
               "hbm", 2 * b.numel() * 2, cpu(lambda: O.rms_norm_grad_sample(cx, cb, (D,), 1e-5), 4, "4 of 16 samples"))
+    ah = torch.randn(n, T, D, device=dev).bfloat16()
+    gh = (torch.randn(n, T, V, device=dev) * 0.01).bfloat16()
+    yield row("tied_embedding_cross", "a5+a2", "C5 tied n=16 T=1024 D=2048 V=32000 bf16",
+              timed(lambda: K.tied_embedding_cross_term(ids, b, ah, gh)), "mfma_fp32", 2.0 * n * T * T * D,
+              cpu(lambda: O.tied_embedding_norm_sample(cids[:1], cb[:1].float(), ah[:1].cpu().float(), gh[:1].cpu().float()),
+                  16, "1 of 16 samples, both gradients materialised"))
+    del ah, gh
     small = 2
     idsm = torch.randint(0, V, (small, T), device=dev)
     cidm, cbm = idsm.cpu(), b[:small].cpu()

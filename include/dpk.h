@@ -176,6 +176,23 @@ int dpk_embedding_ghost_norm(const int64_t* ids, const void* b, int dtype, float
                              int64_t T, int64_t D, float scale, void* ws, size_t ws_bytes,
                              dpk_stream_t stream);
 
+/* An embedding table that is also the weight of the output projection (tied input and
+ * output embeddings). The reference refuses tied parameters under ghost clipping
+ * (opacus/grad_sample/grad_sample_module_fast_gradient_clipping.py:172-179); the materialising
+ * path handles them by adding the two layers' gradients (grad_sample_module.py:58-59), and
+ * this entry point supplies what the norm of that sum needs beyond the two layers' own ghost
+ * norms:  |G_emb + G_head|^2 = |G_emb|^2 + |G_head|^2 + 2 cross,
+ *   cross[n] = scale * sum_t < e[n,t,:] , sum_t2 g[n,t2,ids[n,t]] * a[n,t2,:] >.
+ * ids: int64 [n,T]; e: [n,T,D] backprops of the embedding output (`emb_dtype`); a: [n,T2,D]
+ * inputs and g: [n,T2,V] output backprops of the projection (`head_dtype`); cross: float[n].
+ * An id outside [0,V) contributes nothing. Workspace 256-byte aligned. */
+size_t dpk_tied_embedding_cross_workspace_bytes(int64_t n, int64_t T, int64_t T2, int64_t D,
+                                                int head_dtype);
+int dpk_tied_embedding_cross(const int64_t* ids, const void* e, int emb_dtype, const void* a,
+                             const void* g, int head_dtype, float* cross, int64_t n, int64_t T,
+                             int64_t T2, int64_t D, int64_t V, float scale, void* ws,
+                             size_t ws_bytes, dpk_stream_t stream);
+
 /* ------------------------------------------------------------------------- *
  * Normalisation layers with an affine weight
  * replaces opacus/grad_sample/group_norm.py:26-47, rms_norm.py:27-47,

@@ -63,6 +63,11 @@ SIGNATURES = {
         [_P, _P, _P, c_int, _P, c_int, _I, _I, _I, _I, c_int, c_float, _P, c_size_t, _P],
     ),
     "dpk_embedding_ghost_norm": (c_int, [_P, _P, c_int, _P, _I, _I, _I, c_float, _P, c_size_t, _P]),
+    "dpk_tied_embedding_cross_workspace_bytes": (c_size_t, [_I, _I, _I, _I, c_int]),
+    "dpk_tied_embedding_cross": (
+        c_int,
+        [_P, _P, c_int, _P, _P, c_int, _P, _I, _I, _I, _I, _I, c_float, _P, c_size_t, _P],
+    ),
     "dpk_group_norm_gs": (c_int, [_P, _P, c_int, _P, _P, c_int, _I, _I, _I, _I, c_float, c_float, _P]),
     "dpk_rms_norm_gs_workspace_bytes": (c_size_t, [_I, _I, _I]),
     "dpk_rms_norm_gs": (c_int, [_P, _P, c_int, _P, c_int, _I, _I, _I, c_float, c_float, _P, c_size_t, _P]),

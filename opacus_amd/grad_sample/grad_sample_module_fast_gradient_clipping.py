@@ -7,6 +7,11 @@ Embedding) get it from the ghost-norm kernels without the gradient ever existing
 layers have their per-sample gradient formed by the grad sampler, reduced to a norm and
 dropped at once. ``get_clipping_coef`` then yields ``min(1, C / (norm + 1e-6))``.
 
+One kind of parameter tying is taken under ghost clipping, which the reference refuses
+altogether (:172-179): an ``nn.Embedding`` whose table is also the weight of an ``nn.Linear``
+(tied input and output embeddings). The norm of the sum of the two layers' gradients is
+their two ghost norms plus twice a cross term, ``kernels.tied_embedding_cross_term``.
+
 Norm samples are kept in float32 whatever the dtype of the backprops (the kernels
 accumulate in fp32; rounding a norm to bf16 before it meets the other parameters' norms
 would only lose bits).
@@ -70,9 +75,41 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
             m, batch_first=batch_first, loss_reduction=loss_reduction, strict=strict, force_functorch=force_functorch
         )
         self.trainable_parameters = [p for _, p in trainable_parameters(self._module)]
+        self._tied_embedding_weights = self._find_tied_embedding_weights()
         self.max_grad_norm = max_grad_norm
         self.use_ghost_clipping = use_ghost_clipping
         self._per_sample_gradient_norms = None
+
+    # ---- tied input / output embeddings ------------------------------------------------
+    def _find_tied_embedding_weights(self) -> set:
+        """ids of the weights owned by exactly one ``nn.Embedding`` and one ``nn.Linear``."""
+        owners = {}
+        for _, m in trainable_modules(self._module):
+            for name, p in m.named_parameters(recurse=False):
+                owners.setdefault(id(p), []).append((m, name))
+        tied = set()
+        for pid, uses in owners.items():
+            if (
+                len(uses) == 2
+                and {type(m) for m, _ in uses} == {nn.Embedding, nn.Linear}
+                and all(name == "weight" for _, name in uses)
+            ):
+                tied.add(pid)
+        return tied
+
+    def _tied_embedding_norm(self, param, module, activations, backprops, scale, ns):
+        """Keeps this layer's share of a tied table; once both layers of the pass have
+        reported, returns ``sqrt(|G_emb|^2 + |G_head|^2 + 2 <G_emb, G_head>)``. Until then the
+        layer's own norm stands in."""
+        parts = param.__dict__.setdefault("_tied_parts", {})
+        parts["emb" if isinstance(module, nn.Embedding) else "head"] = (activations[0], backprops, scale, ns)
+        if len(parts) < 2:
+            return ns
+        del param.__dict__["_tied_parts"]
+        ids, e, s_e, ns_e = parts["emb"]
+        a, g, s_h, ns_h = parts["head"]
+        cross = kernels.tied_embedding_cross_term(ids, e, a, g, scale=s_e * s_h)
+        return (ns_e.float().square() + ns_h.float().square() + 2.0 * cross).clamp_(min=0).sqrt_()
 
     # ---- clipping coefficient ----------------------------------------------------------
     def get_norm_sample(self) -> torch.Tensor:
@@ -111,11 +148,14 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
         module.activations.append([t.detach() for t in forward_input if isinstance(t, torch.Tensor)])
         for _, p in trainable_parameters(module):
             p._forward_counter += 1
+            if p._forward_counter == 1:
+                p.__dict__.pop("_tied_parts", None)  # left by a backward pass that did not finish
             if (
                 self.use_ghost_clipping
                 and p._forward_counter > 1
                 and type(module) in self.NORM_SAMPLERS
                 and not getattr(module, "stack_uses", False)  # its uses are contracted together
+                and not (id(p) in self._tied_embedding_weights and p._forward_counter == 2)
             ):
                 # the norm of a sum of two layers' gradients is not a function of their norms
                 raise NotImplementedError("Parameter tying is not supported with Ghost Clipping")
@@ -141,6 +181,8 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
             norm_samples = call_sampler(self.NORM_SAMPLERS[type(module)], module, activations, backprops, scale)
             for param, ns in norm_samples.items():
                 if param.requires_grad:
+                    if id(param) in self._tied_embedding_weights:
+                        ns = self._tied_embedding_norm(param, module, activations, backprops, scale, ns)
                     param._norm_sample = ns
                     param._forward_counter -= 1
         else:

@@ -390,6 +390,48 @@ def embedding_ghost_norm(ids: torch.Tensor, backprops: torch.Tensor, scale: floa
     return norm
 
 
+def tied_embedding_cross_term(
+    ids: torch.Tensor,
+    emb_backprops: torch.Tensor,
+    head_activations: torch.Tensor,
+    head_backprops: torch.Tensor,
+    scale: float = 1.0,
+) -> torch.Tensor:
+    """``<G_emb, G_head>`` per sample (fp32 ``[n]``) for a weight shared by an Embedding
+    (``ids`` ``[n, ...]``, output backprops ``[n, ..., D]``) and a bias-free or biased Linear
+    (inputs ``[n, ..., D]``, output backprops ``[n, ..., V]``), without forming either
+    gradient: ``scale * sum_t <e_t, sum_t' g[t', ids_t] a_t'>``."""
+    dev = _need_gpu(ids, emb_backprops, head_activations, head_backprops)
+    ids2 = _ids_2d(ids)
+    n, T = ids2.shape
+    D, V = emb_backprops.shape[-1], head_backprops.shape[-1]
+    cross = torch.empty((n,), dtype=torch.float32, device=dev)
+    if n == 0:
+        return cross
+    e = _dense(emb_backprops).reshape(n, -1, D)
+    g = _dense(head_backprops).reshape(n, -1, V)
+    a = _dense(head_activations).reshape(n, -1, D)
+    if a.dtype != g.dtype:
+        a = a.to(g.dtype)
+    T2 = g.shape[1]
+    if e.shape[1] != T or a.shape[1] != T2:
+        raise ValueError(
+            f"ids {tuple(ids.shape)}, embedding backprops {tuple(emb_backprops.shape)}, projection inputs "
+            f"{tuple(head_activations.shape)} and backprops {tuple(head_backprops.shape)} disagree"
+        )
+    L = lib()
+    ws, wsb = _ws(L.dpk_tied_embedding_cross_workspace_bytes(n, T, T2, D, _code(g)), dev)
+    with _timed("tied_embedding_cross", dev):
+        check(
+            "dpk_tied_embedding_cross",
+            L.dpk_tied_embedding_cross(
+                _ptr(ids2), _ptr(e), _code(e), _ptr(a), _ptr(g), _code(g), _ptr(cross), n, T, T2, D, V,
+                float(scale), _ptr(ws), wsb, _stream(dev),
+            ),
+        )
+    return cross
+
+
 def embedding_bag_grad_sample(
     index: torch.Tensor,
     offsets: torch.Tensor,

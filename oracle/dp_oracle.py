@@ -32,6 +32,9 @@ What pins each function (see ``tests/test_oracle_pins.py``):
     numbers, the fixed point at the target quantile, the composition identity
     sigma'^-2 + (2 n/20)^-2 == sigma^-2, and coefficients that scale every clipped sample
     to exactly the new bound;
+  * tied embedding / projection norm: it is the materialised definition (sum of the two
+    pinned gradients); checked against autograd's gradient of the shared table with a batch
+    of one, and against |G_emb|^2 + |G_head|^2 + 2 cross from the two pinned ghost norms;
   * Philox4x32-10: the Random123 known-answer vectors.
 No function here is "parity unpinned".
 """
@@ -282,6 +285,26 @@ def embedding_unique_pairs(ids: torch.Tensor) -> Tuple[torch.Tensor, torch.Tenso
         return paired, torch.zeros(0, dtype=torch.int64)
     uniq, inverse = torch.unique(paired, dim=0, return_inverse=True, sorted=True)
     return uniq, inverse
+
+
+def tied_embedding_norm_sample(
+    ids: torch.Tensor,
+    emb_backprops: torch.Tensor,
+    head_activations: torch.Tensor,
+    head_backprops: torch.Tensor,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """A table shared by nn.Embedding and nn.Linear, by the materialising path's rule that the
+    uses of a parameter add up (opacus/grad_sample/grad_sample_module.py:58-59): forms both
+    per-sample gradients ``[n, V, D]`` (embedding.py:40-63, linear.py:41-51), and returns the
+    norm of their sum and the inner product of the two, per sample. This is the brute-force
+    definition; the reference itself raises for tied parameters under ghost clipping
+    (grad_sample_module_fast_gradient_clipping.py:172-179)."""
+    V = head_backprops.shape[-1]
+    g_emb = embedding_grad_sample(ids, emb_backprops, V)
+    g_head, _ = linear_grad_sample(head_activations, head_backprops, bias=False)
+    norm = (g_emb + g_head).flatten(1).norm(dim=1)
+    cross = (g_emb * g_head).flatten(1).sum(dim=1)
+    return norm, cross
 
 
 def embedding_norm_sample(ids: torch.Tensor, backprops: torch.Tensor) -> Dict[str, torch.Tensor]:

@@ -740,6 +740,57 @@ def test_ghost_tiny_llama_norms(A, dtype):
             close(p1, p0 - 0.1 * g, 1e-3, 1e-5, k)
 
 
+def test_ghost_tied_embedding_and_lm_head(A):
+    """Config 5 as written (tied embeddings), down-scaled. The reference raises for tied
+    parameters under ghost clipping; here an Embedding table shared with the LM head takes the
+    two ghost norms plus the cross term. Checked against batch-of-one autograd, whose gradient
+    of the shared table is the sum of both uses, and against the materialising hooks path."""
+    torch.manual_seed(14)
+    net = TinyLlama()
+    net.lm_head.weight = net.emb.weight
+    assert len(list(net.parameters())) == len(list(TinyLlama().parameters())) - 1
+    n, T, V = 4, 16, 50
+    ids = torch.randint(0, V, (n, T))
+    ids[0, :8] = 3
+    tgt = torch.randint(0, V, (n, T))
+
+    def seq_loss(logits, t):
+        return F.cross_entropy(logits.flatten(0, 1).float(), t.flatten(), reduction="none").view(1, -1).mean(1).sum()
+
+    want = per_sample_grads_cpu(net, ids, tgt, seq_loss)
+    want_norm = torch.sqrt(sum(v.double().flatten(1).pow(2).sum(1) for v in want.values()))
+
+    gnet = copy.deepcopy(net).to(DEV)
+    assert gnet.lm_head.weight is gnet.emb.weight
+    ghost = A.GradSampleModuleFastGradientClipping(gnet, loss_reduction="mean", max_grad_norm=1.0)
+    gopt = A.DPOptimizerFastGradientClipping(torch.optim.SGD(ghost.parameters(), lr=0.1), noise_multiplier=0.0, max_grad_norm=1.0, expected_batch_size=n)
+    dpl = A.DPLossFastGradientClipping(ghost, gopt, nn.CrossEntropyLoss(), "mean")
+    for _ in range(2):  # the second pass must find no leftovers of the first
+        gopt.zero_grad()
+        logits = ghost(ids.to(DEV))
+        dpl(logits.flatten(0, 1).float(), tgt.flatten().to(DEV), shape=(n, T, V)).backward()
+        close(gnet.emb.weight._norm_sample, want["emb.weight"].flatten(1).norm(dim=1), 1e-3, 1e-7, "shared table")
+        close(ghost.per_sample_gradient_norms, want_norm, 1e-3, 1e-6)
+    coef = (1.0 / (want_norm + 1e-6)).clamp(max=1.0).float()
+    gopt.step()
+    for (k, p0), p1 in zip(net.named_parameters(), gnet.parameters()):
+        g = (coef.view(-1, *[1] * (want[k].dim() - 1)) * want[k]).sum(0) / n
+        close(p1, p0 - 0.1 * g, 1e-3, 1e-5, k)
+
+    # the same weight used by two Linear layers is still refused
+    class TwoHeads(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.a, self.b = nn.Linear(6, 6, bias=False), nn.Linear(6, 6, bias=False)
+            self.b.weight = self.a.weight
+
+        def forward(self, x):
+            return self.b(self.a(x))
+
+    with pytest.raises(NotImplementedError, match="tying"):
+        A.GradSampleModuleFastGradientClipping(TwoHeads().to(DEV))(torch.randn(2, 6, device=DEV))
+
+
 def test_ghost_bf16_mlp(A):
     """Config 3, down-scaled, bf16 parameters with fp32 accumulation inside the kernels."""
     torch.manual_seed(12)

@@ -167,6 +167,35 @@ def test_c5_embedding_and_rms_norm_full_size(K):
     assert rel_err(gw32, want_w) < FP32_REL
 
 
+# ---- C5 with tied embeddings: the cross term at batch 16, seq 1024, dim 2048, vocab 32000 ----------
+def test_c5_tied_embedding_cross_term_full_size(K):
+    n, T, D, V = 16, 1024, 2048, 32000
+    torch.manual_seed(6)
+    ids = torch.randint(0, V, (n, T), device="cuda")
+    ids[2, :300] = ids[2, 0]
+    e = (torch.randn(n, T, D, device="cuda") * 0.02).bfloat16()
+    a = torch.randn(n, T, D, device="cuda").bfloat16()
+    g = (torch.randn(n, T, V, device="cuda") * 0.01).bfloat16()
+    got = K.tied_embedding_cross_term(ids, e, a, g)
+    # the definition in float64, sample by sample (plain torch: an independent route)
+    want = []
+    for i in range(n):
+        gathered = g[i].double().gather(1, ids[i].unsqueeze(0).expand(T, T))  # [t2, t] = g[t2, ids[t]]
+        want.append((e[i].double() * (gathered.t() @ a[i].double())).sum())
+    want = torch.stack(want)
+    # the sum has ~2 M terms of either sign: compare on the scale of its terms' root sum of squares
+    scale = (e.double().pow(2).sum((1, 2)) * a.double().pow(2).sum((1, 2)) / D).sqrt() * 0.01
+    assert ((got.double() - want).abs() / scale).max().item() < 1e-4
+    # exact scaling by a power of two, and invariance under a permutation of the embedding positions
+    assert torch.equal(K.tied_embedding_cross_term(ids, (e.float() * 2).bfloat16(), a, g), 2 * got)
+    perm = torch.randperm(T, device="cuda")
+    gotp = K.tied_embedding_cross_term(ids[:, perm].contiguous(), e[:, perm].contiguous(), a, g)
+    assert ((gotp - got).abs().double() / scale).max().item() < 1e-4
+    # the oracle (materialised gradients) on one sample of the batch
+    _, want0 = O.tied_embedding_norm_sample(ids[:1].cpu(), e[:1].cpu().float(), a[:1].cpu().float(), g[:1].cpu().float())
+    assert abs(got[0].item() - want0.item()) / scale[0].item() < 1e-3
+
+
 # ---- C1: the small CNN at batch 256, whole step against the oracle ------------------------------
 def test_c1_small_cnn_full_batch_step():
     import copy

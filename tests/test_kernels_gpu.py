@@ -688,3 +688,27 @@ def test_norm_layers_bf16(K):
     gw, gb = K.group_norm_grad_sample(dev(x4), dev(b4), 4, 1e-5)
     assert_rel(gw, want_w, BF16_REL)
     assert_rel(gb, want_b, BF16_REL)
+
+
+# ---- tied input / output embeddings: the cross term --------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n,T,T2,D,V", [(3, 7, 7, 12, 19), (2, 33, 5, 64, 300), (4, 1, 9, 8, 16)])
+def test_tied_embedding_cross_term(K, dtype, n, T, T2, D, V):
+    """<G_emb, G_head> against the materialised definition; embedding and projection may see
+    different numbers of positions; repeated ids; the scale is a plain factor."""
+    torch.manual_seed(n * 100 + T)
+    ids = torch.randint(0, V, (n, T))
+    if T > 2:
+        ids[0, 1:3] = ids[0, 0]
+    e = torch.randn(n, T, D).to(dtype)
+    a = torch.randn(n, T2, D).to(dtype)
+    g = (torch.randn(n, T2, V) * 0.1).to(dtype)
+    _, want = O.tied_embedding_norm_sample(ids, e.double(), a.double(), g.double())
+    got = K.tied_embedding_cross_term(dev(ids), dev(e), dev(a), dev(g))
+    assert got.dtype == torch.float32 and got.shape == (n,)
+    assert_rel(got, want, 1e-5 if dtype == torch.float32 else 1e-4, "cross term")
+    assert_rel(K.tied_embedding_cross_term(dev(ids), dev(e), dev(a), dev(g), scale=4.0), 4 * want, 1e-4, "scale")
+    # mixed dtypes: fp32 embedding backprops with the projection in its own dtype
+    got32 = K.tied_embedding_cross_term(dev(ids), dev(e.float()), dev(a), dev(g))
+    assert_rel(got32, want, 1e-4, "fp32 embedding backprops")
+    assert K.tied_embedding_cross_term(dev(ids[:0]), dev(e[:0]), dev(a[:0]), dev(g[:0])).shape == (0,)

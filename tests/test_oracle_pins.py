@@ -493,3 +493,38 @@ def test_ghost_adaptive_update_hand_numbers_and_identities():
     _, sigma, _ = O.ghost_adaptive_update(big, 1.0, 0.5, 0.2, 0.1, 10.0, noise_multiplier=1.3)
     assert sigma > 1.3
     assert sigma ** -2 + (2 * 200 / 20.0) ** -2 == pytest.approx(1.3 ** -2, rel=1e-12)
+
+
+def test_tied_embedding_norm_is_the_norm_of_autograds_shared_gradient():
+    """A table used as nn.Embedding weight and as nn.Linear weight: with a batch of one,
+    autograd's gradient of the shared parameter is the sample's whole gradient, so its norm
+    pins the oracle; the decomposition into the two ghost norms and the cross term pins the
+    inner product."""
+    torch.manual_seed(12)
+    V, D, n, T = 11, 6, 4, 5
+    emb = nn.Embedding(V, D).double()
+    ids = torch.randint(0, V, (n, T))
+    ids[1, 1:4] = ids[1, 0]  # repeated ids in one sample
+    mix = torch.randn(D, D).double()
+    y = torch.randint(0, V, (n, T))
+    e_rows, a_rows, g_rows, want = [], [], [], []
+    for i in range(n):
+        emb.zero_grad()
+        h = emb(ids[i : i + 1])
+        h.retain_grad()
+        a = torch.tanh(h @ mix)
+        a.retain_grad()
+        logits = F.linear(a, emb.weight)
+        logits.retain_grad()
+        F.cross_entropy(logits.flatten(0, 1), y[i], reduction="sum").backward()
+        want.append(emb.weight.grad.norm())
+        e_rows.append(h.grad[0])
+        a_rows.append(a.detach()[0])
+        g_rows.append(logits.grad[0])
+    e, a, g = torch.stack(e_rows), torch.stack(a_rows), torch.stack(g_rows)
+    norm, cross = O.tied_embedding_norm_sample(ids, e, a, g)
+    torch.testing.assert_close(norm, torch.stack(want), rtol=1e-12, atol=1e-14)
+    n_emb = O.embedding_norm_sample(ids, e)["result_sqrt"]
+    n_head, _ = O.linear_norm_sample(a, g, bias=False)
+    torch.testing.assert_close(norm**2, n_emb**2 + n_head**2 + 2 * cross, rtol=1e-10, atol=1e-14)
+    assert (cross.abs() > 1e-6).all()  # the term is not negligible in this setting
