@@ -427,6 +427,15 @@ def kernel_table(dev, iters: int = 10, warm: int = 3, with_cpu: bool = True):
     ca, cb = a[:4].cpu(), b[:4].cpu()
     yield row("linear_gs (T>1, fp32 MFMA)", "a1", "n=16 T=256 1024x1024 f32", timed(lambda: K.linear_grad_sample(b, a)),
               "mfma_fp32", 2.0 * n * T * i * o, cpu(lambda: O.linear_grad_sample(ca, cb), 4, "4 of 16 samples"))
+    a16, b16 = a.bfloat16(), b.bfloat16()
+    yield row("linear_gs (T>1, bf16 MFMA)", "a1", "n=16 T=256 1024x1024 bf16 in, f32 out",
+              timed(lambda: K.linear_grad_sample(b16, a16, out_dtype=torch.float32)), "mfma_bf16", 2.0 * n * T * i * o)
+    n2, T2 = 16, 1024
+    a2 = torch.randn(n2, T2, 2048, device=dev).bfloat16()
+    b2 = torch.randn(n2, T2, 1024, device=dev).bfloat16()
+    yield row("linear_gs (T>1, bf16 MFMA)", "a1", "n=16 T=1024 2048->1024 bf16 in, f32 out",
+              timed(lambda: K.linear_grad_sample(b2, a2, out_dtype=torch.float32)), "mfma_bf16", 2.0 * n2 * T2 * 2048 * 1024)
+    del a16, b16, a2, b2
     # ---- C3 / C5: ghost norms, bf16
     for cfg, n, T, layers in (
         ("C3", 32, 512, [(1024, 4096, "fc1"), (4096, 1024, "fc2")]),
@@ -457,7 +466,7 @@ def kernel_table(dev, iters: int = 10, warm: int = 3, with_cpu: bool = True):
     ah = torch.randn(n, T, D, device=dev).bfloat16()
     gh = (torch.randn(n, T, V, device=dev) * 0.01).bfloat16()
     yield row("tied_embedding_cross", "a5+a2", "C5 tied n=16 T=1024 D=2048 V=32000 bf16",
-              timed(lambda: K.tied_embedding_cross_term(ids, b, ah, gh)), "mfma_fp32", 2.0 * n * T * T * D,
+              timed(lambda: K.tied_embedding_cross_term(ids, b, ah, gh)), "mfma_bf16", 2.0 * n * T * T * D,
               cpu(lambda: O.tied_embedding_norm_sample(cids[:1], cb[:1].float(), ah[:1].cpu().float(), gh[:1].cpu().float()),
                   16, "1 of 16 samples, both gradients materialised"))
     del ah, gh

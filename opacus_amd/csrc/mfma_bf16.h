@@ -64,6 +64,22 @@ struct Tile {
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[i], bv[j], acc[i][j], 0, 0, 0);
     }
   }
+
+  // f(row, col, value) for every accumulator element this thread owns; row and
+  // col are relative to the block tile.
+  template <typename F>
+  __device__ __forceinline__ void for_each(F f) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
+    const int kk = lane >> 5, l32 = lane & 31;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          f(wm0 + i * 32 + (v >> 2) * 8 + kk * 4 + (v & 3), wn0 + j * 32 + l32, acc[i][j][v]);
+  }
 };
 
 // Rows of the source run along k: element (m, k) at base[m * ld + k].
@@ -110,6 +126,76 @@ struct Loader {
     for (int r = 0; r < R; ++r) {
       const int idx = threadIdx.x + r * NTHREADS;
       *reinterpret_cast<uint4*>(&S[idx / (BK / 8)][(idx % (BK / 8)) * 8]) = st[SLOT][r];
+    }
+  }
+};
+
+// Rows of the source run along m: element (m, k) at base[k * ld + m] (a [T, features]
+// matrix contracted over T). The instruction wants k contiguous, so the tile is transposed
+// on its way into LDS: a thread loads an 8 (m) x 4 (k) patch as four 16-byte rows, regroups
+// it in registers (one v_perm_b32 per output dword) and writes eight 8-byte pieces, one per
+// m. Lanes 0..15 of a wave take consecutive k quads of the same 8 m, so their LDS writes
+// fall into 32 consecutive dwords of a row, and four such groups share a 64-byte stretch
+// of every source row they read.
+// VEC: ld % 8 == 0, m0 % 8 == 0 and base 16-byte aligned.
+__device__ __forceinline__ uint32_t dword(const uint4& v, int i) {
+  return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w;
+}
+
+template <int BMN, bool VEC>
+struct LoaderMContig {
+  static constexpr int PATCHES = (BMN / 8) * (BK / 4);
+  static constexpr int R = (PATCHES + NTHREADS - 1) / NTHREADS;
+  const bf16_t* base;
+  int64_t ld, m0, M, K;
+  uint4 st[2][R][4];
+  __device__ __forceinline__ LoaderMContig(const bf16_t* base_, int64_t ld_, int64_t m0_, int64_t M_,
+                                           int64_t K_)
+      : base(base_), ld(ld_), m0(m0_), M(M_), K(K_) {}
+  template <int SLOT>
+  __device__ __forceinline__ void fetch(int64_t k0) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int idx = threadIdx.x + r * NTHREADS;
+      const int kq = idx % (BK / 4), mg = idx / (BK / 4);
+      const int64_t m = m0 + mg * 8;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int64_t k = k0 + kq * 4 + j;
+        uint4 v = make_uint4(0u, 0u, 0u, 0u);
+        if (idx < PATCHES && k < K && m < M) {
+          const bf16_t* p = base + k * ld + m;
+          if (VEC) {
+            v = *reinterpret_cast<const uint4*>(p);
+          } else {
+            uint32_t w[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              if (m + e < M) w[e >> 1] |= static_cast<uint32_t>(p[e]) << ((e & 1) * 16);
+            v = make_uint4(w[0], w[1], w[2], w[3]);
+          }
+        }
+        st[SLOT][r][j] = v;
+      }
+    }
+  }
+  template <int SLOT>
+  __device__ __forceinline__ void commit(bf16_t (*S)[LDK]) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int idx = threadIdx.x + r * NTHREADS;
+      if (idx >= PATCHES) continue;
+      const int kq = idx % (BK / 4), mg = idx / (BK / 4);
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        // element c of rows k, k+1 | rows k+2, k+3: low halves of the dwords for even c,
+        // high halves for odd c
+        const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
+        uint2 o;
+        o.x = __builtin_amdgcn_perm(dword(st[SLOT][r][1], c >> 1), dword(st[SLOT][r][0], c >> 1), sel);
+        o.y = __builtin_amdgcn_perm(dword(st[SLOT][r][3], c >> 1), dword(st[SLOT][r][2], c >> 1), sel);
+        *reinterpret_cast<uint2*>(&S[mg * 8 + c][kq * 4]) = o;
+      }
     }
   }
 };

@@ -70,7 +70,18 @@ def test_linear_grad_sample_f32(K, n, mid, fin, fout, scale):
     assert_rel(sumsq, want_w.double().flatten(1).pow(2).sum(1), 2e-5, "sumsq")
 
 
-@pytest.mark.parametrize("n,mid,fin,fout", [(4, (), 64, 32), (2, (40,), 136, 200), (3, (5,), 30, 18)])
+@pytest.mark.parametrize(
+    "n,mid,fin,fout",
+    [
+        (4, (), 64, 32),
+        (2, (40,), 136, 200),  # 128 tiles with ragged edges, K under one k tile
+        (3, (5,), 30, 18),  # odd sizes: element-wise loads
+        (2, (200,), 256, 384),  # whole 128 tiles, K = 3 k tiles + 8
+        (3, (65,), 64, 72),  # 64 tiles, K = one k tile + 1
+        (1, (7, 19), 132, 260),  # two middle dimensions, sizes that are multiples of 4 only
+        (2, (128,), 1024, 8),  # a narrow output
+    ],
+)
 def test_linear_grad_sample_bf16(K, n, mid, fin, fout):
     torch.manual_seed(7)
     a = torch.randn(n, *mid, fin).bfloat16()
