@@ -168,7 +168,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
   mb16::LoaderMContig<BN, VEC> lb(a + sample * T * N, N, n0, N, T);
   mb16::Tile<BM, BN> tile;
   tile.clear();
-  mb16::mainloop<BM, BN>(tile, sm, la, lb, T);
+  mb16::mainloop_pairs<BM, BN>(tile, sm, la, lb, T);
   TOUT* out = gs + sample * M * N;
   float ss = 0.f;
   tile.for_each([&](int r, int c, float v) {
@@ -288,7 +288,8 @@ void launch_linear(const Plan& p, bool vec, const void* b, const void* a, void* 
 #undef DPK_OUTER
   } else if constexpr (std::is_same<TIN, bf16_t>::value) {
     // 16-byte rows of 8 elements for the transposing loader
-    const bool vec8 = M % 8 == 0 && N % 8 == 0 && dpk_aligned(b, 16) && dpk_aligned(a, 16);
+    const bool vec8 = M % 8 == 0 && N % 8 == 0 && dpk_aligned(b, 16) && dpk_aligned(a, 16) &&
+                      T * (M > N ? M : N) * 2 < (1LL << 30);
 #define DPK_BF16(BMN, V)                                                                              \
   hipLaunchKernelGGL((linear_mfma_bf16_kernel<BMN, BMN, TOUT, V>), grid, block, 0, s, bp, ap, gp, partials, \
                      T, M, N, scale, p.tiles_m, p.tiles_n)

@@ -137,7 +137,10 @@ struct Loader {
 // m. Lanes 0..15 of a wave take consecutive k quads of the same 8 m, so their LDS writes
 // fall into 32 consecutive dwords of a row, and four such groups share a 64-byte stretch
 // of every source row they read.
-// VEC: ld % 8 == 0, m0 % 8 == 0 and base 16-byte aligned.
+// VEC: ld % 8 == 0, m0 % 8 == 0, base 16-byte aligned and the matrix below 1 GiB. Its loads
+// go through a buffer descriptor over the K x ld matrix: the row offset of the k tile sits
+// in a scalar register, each lane adds one constant byte offset, and rows past K read as
+// zero without a test.
 __device__ __forceinline__ uint32_t dword(const uint4& v, int i) {
   return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w;
 }
@@ -146,32 +149,65 @@ template <int BMN, bool VEC>
 struct LoaderMContig {
   static constexpr int PATCHES = (BMN / 8) * (BK / 4);
   static constexpr int R = (PATCHES + NTHREADS - 1) / NTHREADS;
-  const bf16_t* base;
-  int64_t ld, m0, M, K;
+  // per patch: pointer to its element (k = kq * 4, m) of the k tile at k0 = 0, advanced
+  // by whole k tiles; the bounds are 32-bit and the column test is made once
+  const bf16_t* ptr[R];
+  int64_t ld;
+  int kfirst[R], K, mleft[R];
+  uint32_t voff[R];
+  __amdgpu_buffer_rsrc_t rsrc;
   uint4 st[2][R][4];
-  __device__ __forceinline__ LoaderMContig(const bf16_t* base_, int64_t ld_, int64_t m0_, int64_t M_,
+  __device__ __forceinline__ LoaderMContig(const bf16_t* base, int64_t ld_, int64_t m0, int64_t M,
                                            int64_t K_)
-      : base(base_), ld(ld_), m0(m0_), M(M_), K(K_) {}
-  template <int SLOT>
-  __device__ __forceinline__ void fetch(int64_t k0) {
+      : ld(ld_), K(static_cast<int>(K_)) {
+    if (VEC)
+      rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(base), 0, static_cast<int>(K_ * ld_ * 2), 0x00020000);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const int idx = threadIdx.x + r * NTHREADS;
       const int kq = idx % (BK / 4), mg = idx / (BK / 4);
       const int64_t m = m0 + mg * 8;
+      kfirst[r] = kq * 4;
+      // elements of the patch's 8 columns that exist (0: the patch is outside the matrix)
+      mleft[r] = (idx < PATCHES && m < M) ? static_cast<int>(M - m < 8 ? M - m : 8) : 0;
+      ptr[r] = base + kfirst[r] * ld + m;
+      // a patch outside the matrix points past the descriptor's end and reads zeros
+      voff[r] = mleft[r] > 0 ? static_cast<uint32_t>((kfirst[r] * ld + m) * 2) : 0x7fffffffu;
+    }
+  }
+  // k0 must advance by BK from call to call of the same slot sequence: the loader keeps no
+  // pointer per slot, it recomputes from k0
+  template <int SLOT>
+  __device__ __forceinline__ void fetch(int64_t k0) {
+    const int k0i = static_cast<int>(k0);
+    if (VEC) {
+      typedef int vi4 __attribute__((ext_vector_type(4)));
+      const int row_bytes = static_cast<int>(ld) * 2;
+      const int tile_off = k0i * row_bytes;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const vi4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff[r], tile_off + j * row_bytes, 0);
+          st[SLOT][r][j] = make_uint4(v.x, v.y, v.z, v.w);
+        }
+      }
+      return;
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const bf16_t* p = ptr[r] + k0 * ld;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const int64_t k = k0 + kq * 4 + j;
         uint4 v = make_uint4(0u, 0u, 0u, 0u);
-        if (idx < PATCHES && k < K && m < M) {
-          const bf16_t* p = base + k * ld + m;
+        if (mleft[r] > 0 && k0i + kfirst[r] + j < K) {
           if (VEC) {
-            v = *reinterpret_cast<const uint4*>(p);
+            v = *reinterpret_cast<const uint4*>(p + j * ld);
           } else {
             uint32_t w[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
             for (int e = 0; e < 8; ++e)
-              if (m + e < M) w[e >> 1] |= static_cast<uint32_t>(p[e]) << ((e & 1) * 16);
+              if (e < mleft[r]) w[e >> 1] |= static_cast<uint32_t>(p[j * ld + e]) << ((e & 1) * 16);
             v = make_uint4(w[0], w[1], w[2], w[3]);
           }
         }
@@ -186,6 +222,7 @@ struct LoaderMContig {
       const int idx = threadIdx.x + r * NTHREADS;
       if (idx >= PATCHES) continue;
       const int kq = idx % (BK / 4), mg = idx / (BK / 4);
+      bf16_t* dst = &S[mg * 8][kq * 4];
 #pragma unroll
       for (int c = 0; c < 8; ++c) {
         // element c of rows k, k+1 | rows k+2, k+3: low halves of the dwords for even c,
@@ -194,7 +231,7 @@ struct LoaderMContig {
         uint2 o;
         o.x = __builtin_amdgcn_perm(dword(st[SLOT][r][1], c >> 1), dword(st[SLOT][r][0], c >> 1), sel);
         o.y = __builtin_amdgcn_perm(dword(st[SLOT][r][3], c >> 1), dword(st[SLOT][r][2], c >> 1), sel);
-        *reinterpret_cast<uint2*>(&S[mg * 8 + c][kq * 4]) = o;
+        *reinterpret_cast<uint2*>(dst + c * LDK) = o;
       }
     }
   }
@@ -240,6 +277,41 @@ __device__ __forceinline__ void mainloop(Tile<BM, BN>& t, Smem<BM, BN>& sm, LA& 
       la.template commit<0>(sm.a[0]);
       lb.template commit<0>(sm.b[0]);
     }
+    __syncthreads();
+  }
+}
+
+}  // namespace mb16
+
+namespace mb16 {
+
+// The same pipeline without a way out in the middle of a trip, for loaders that deliver
+// zeros for k tiles past K (both of the above do): tiles are taken in pairs, and for an odd
+// count the last pair's second tile is all zeros. One basic block per trip keeps the
+// accumulators in place.
+template <int BM, int BN, class LA, class LB>
+__device__ __forceinline__ void mainloop_pairs(Tile<BM, BN>& t, Smem<BM, BN>& sm, LA& la, LB& lb,
+                                               int64_t K) {
+  const int64_t nk = (K + BK - 1) / BK;
+  la.template fetch<0>(0);
+  lb.template fetch<0>(0);
+  la.template fetch<1>(BK);
+  lb.template fetch<1>(BK);
+  la.template commit<0>(sm.a[0]);
+  lb.template commit<0>(sm.b[0]);
+  __syncthreads();
+  for (int64_t kt = 0; kt < nk; kt += 2) {
+    la.template fetch<0>((kt + 2) * BK);
+    lb.template fetch<0>((kt + 2) * BK);
+    t.mma(sm.a[0], sm.b[0]);
+    la.template commit<1>(sm.a[1]);
+    lb.template commit<1>(sm.b[1]);
+    __syncthreads();
+    la.template fetch<1>((kt + 3) * BK);
+    lb.template fetch<1>((kt + 3) * BK);
+    t.mma(sm.a[1], sm.b[1]);
+    la.template commit<0>(sm.a[0]);
+    lb.template commit<0>(sm.b[0]);
     __syncthreads();
   }
 }
