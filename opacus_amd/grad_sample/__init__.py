@@ -18,6 +18,7 @@ from .utils import (
     wrap_model,
 )
 from .conv import compute_conv_grad_sample  # noqa: E402
+from .dp_multihead_attention import compute_sequence_bias_grad_sample  # noqa: E402
 from .dp_rnn import compute_rnn_linear_grad_sample, compute_rnn_linear_norm_sample  # noqa: E402
 from .embedding import (  # noqa: E402
     compute_embedding_grad_sample,

@@ -371,6 +371,48 @@ def test_recurrent_layers_grad_samples_and_ghost_norms(A, kind, packed):
         close(p._norm_sample, want[k].flatten(1).norm(dim=1), 1e-4, 1e-6, f"ghost {k}")
 
 
+@pytest.mark.parametrize("batch_first", [False, True])
+def test_multihead_attention_grad_samples(A, batch_first):
+    """grad_samples/dp_multihead_attention_test.py: per-sample gradients of the four projections
+    and of the key/value sequence biases equal batch-of-one autograd through
+    torch.nn.MultiheadAttention holding the same state."""
+    from opacus_amd.layers import DPMultiheadAttention
+
+    torch.manual_seed(41)
+    E, H, N, L, S = 8, 2, 4, 5, 6
+    ref = nn.MultiheadAttention(E, H, add_bias_kv=True, add_zero_attn=True, batch_first=batch_first)
+    dp = DPMultiheadAttention(E, H, add_bias_kv=True, add_zero_attn=True, batch_first=batch_first)
+    dp.load_state_dict(ref.state_dict())
+    bdim = 0 if batch_first else 1
+    q = torch.randn(N, L, E) if batch_first else torch.randn(L, N, E)
+    kv = torch.randn(N, S, E) if batch_first else torch.randn(S, N, E)
+    tgt = torch.randn_like(q)
+    want = {k: [] for k, _ in ref.named_parameters()}
+    for i in range(N):
+        ref.zero_grad()
+        qi, kvi = q.narrow(bdim, i, 1), kv.narrow(bdim, i, 1)
+        (ref(qi, kvi, kvi)[0] - tgt.narrow(bdim, i, 1)).pow(2).sum().backward()
+        for k, p in ref.named_parameters():
+            want[k].append(p.grad.clone())
+    want = {k: torch.stack(v) for k, v in want.items()}
+    wq, wk, wv = want["in_proj_weight"].chunk(3, dim=1)
+    bq, bk, bv = want["in_proj_bias"].chunk(3, dim=1)
+    mapped = {
+        "qlinear.weight": wq, "klinear.weight": wk, "vlinear.weight": wv,
+        "qlinear.bias": bq, "klinear.bias": bk, "vlinear.bias": bv,
+        "out_proj.weight": want["out_proj.weight"], "out_proj.bias": want["out_proj.bias"],
+        "seq_bias_k.bias": want["bias_k"].reshape(N, E), "seq_bias_v.bias": want["bias_v"].reshape(N, E),
+    }
+    gsm = A.GradSampleModule(dp.to(DEV), loss_reduction="sum", batch_first=batch_first)
+    out, _ = gsm(q.to(DEV), kv.to(DEV), kv.to(DEV))
+    close(out, ref(q, kv, kv)[0], 1e-4, 1e-5, "forward")
+    (out - tgt.to(DEV)).pow(2).sum().backward()
+    got = dict(gsm._module.named_parameters())
+    assert set(got) == set(mapped)
+    for k, w in mapped.items():
+        close(got[k].grad_sample, w, 1e-4, 1e-5, k)
+
+
 def test_accumulation_tied_parameters_and_functorch_fallback(A):
     torch.manual_seed(3)
 

@@ -765,6 +765,39 @@ def test_recurrent_layers_get_hooks_on_their_linear_maps_only():
     assert len(list(gsm.parameters())) == 16  # four cells x (ih, hh) x (weight, bias), each listed once
 
 
+@pytest.mark.parametrize("batch_first", [False, True])
+def test_multihead_attention_equals_torch_module_and_shares_its_state_dict(batch_first):
+    """opacus/tests/dp_layers/dp_multihead_attention_test.py: outputs and averaged weights of
+    torch.nn.MultiheadAttention from its own state dict (and back, same keys in the same order),
+    over bias / add_bias_kv / add_zero_attn / kdim, vdim / masks, with and without the weights."""
+    from opacus_amd.layers import DPMultiheadAttention
+
+    torch.manual_seed(8)
+    N, L, S = 3, 5, 7
+    for bias, kv, zero, kdim, vdim in [(True, False, False, None, None), (False, True, True, None, None), (True, True, False, 6, 10)]:
+        ref = nn.MultiheadAttention(8, 2, bias=bias, add_bias_kv=kv, add_zero_attn=zero, kdim=kdim, vdim=vdim, batch_first=batch_first).double()
+        dp = DPMultiheadAttention(8, 2, bias=bias, add_bias_kv=kv, add_zero_attn=zero, kdim=kdim, vdim=vdim, batch_first=batch_first).double()
+        dp.load_state_dict(ref.state_dict())
+        assert list(dp.state_dict()) == list(ref.state_dict())
+        ref.load_state_dict(dp.state_dict())
+        shape = (lambda T, E: (N, T, E)) if batch_first else (lambda T, E: (T, N, E))
+        q, k, v = (torch.randn(*shape(T, E)).double() for T, E in ((L, 8), (S, kdim or 8), (S, vdim or 8)))
+        kpm = torch.zeros(N, S, dtype=torch.bool)
+        kpm[1, -2:] = True
+        am = torch.rand(L, S) > 0.8
+        am[:, 0] = False
+        for kwargs in ({}, {"key_padding_mask": kpm}, {"attn_mask": am}, {"attn_mask": torch.randn(L, S).double()}):
+            o1, w1 = ref(q, k, v, **kwargs)
+            o2, w2 = dp(q, k, v, **kwargs)
+            torch.testing.assert_close(o2, o1, rtol=1e-9, atol=1e-11)
+            torch.testing.assert_close(w2, w1, rtol=1e-9, atol=1e-11)
+            o3, w3 = dp(q, k, v, need_weights=False, **kwargs)
+            assert w3 is None
+            torch.testing.assert_close(o3, o1, rtol=1e-7, atol=1e-9)
+    with pytest.raises(AssertionError):
+        dp(q, k, v, is_causal=True)
+
+
 def test_package_surface():
     for name in opacus_amd.__all__:
         assert hasattr(opacus_amd, name)
