@@ -76,6 +76,7 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
         )
         self.trainable_parameters = [p for _, p in trainable_parameters(self._module)]
         self._tied_embedding_weights = self._find_tied_embedding_weights()
+
         self.max_grad_norm = max_grad_norm
         self.use_ghost_clipping = use_ghost_clipping
         self._per_sample_gradient_norms = None
@@ -110,6 +111,55 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
         a, g, s_h, ns_h = parts["head"]
         cross = kernels.tied_embedding_cross_term(ids, e, a, g, scale=s_e * s_h)
         return (ns_e.float().square() + ns_h.float().square() + 2.0 * cross).clamp_(min=0).sqrt_()
+
+    def add_hooks(self, *, loss_reduction: str = "mean", batch_first: bool = True, force_functorch: bool = False) -> None:
+        super().add_hooks(loss_reduction=loss_reduction, batch_first=batch_first, force_functorch=force_functorch)
+        self._first_pass_leaves = {}
+        self._first_pass_open = False
+        self.autograd_grad_sample_hooks.append(
+            self._module.register_forward_pre_hook(self._note_model_inputs, with_kwargs=True)
+        )
+
+    # ---- what the first backward pass has to reach -----------------------------------------
+    def _note_first_pass_leaves(self, module: nn.Module, forward_input) -> None:
+        """The norm pass needs the gradient of every hooked module's OUTPUT, never a weight
+        gradient (``optimizer.zero_grad()`` discards those right after,
+        fast_gradient_clipping_utils.py:190-191). Autograd computes exactly the output
+        gradients, and skips every other weight-gradient GEMM, when it is asked only for the
+        leaves at the start of the graph: the parameters of modules none of whose inputs
+        requires grad, and inputs that are themselves leaves requiring grad."""
+        tensors = [t for t in forward_input if isinstance(t, torch.Tensor)]
+        if not any(t.requires_grad for t in tensors):
+            for _, p in trainable_parameters(module):
+                self._first_pass_leaves[id(p)] = p
+        for t in tensors:
+            if t.requires_grad and t.is_leaf:
+                self._first_pass_leaves[id(t)] = t
+
+    def _note_model_inputs(self, _module, args, kwargs) -> None:
+        """Inputs of the model that carry a graph of their own: a leaf that requires grad is
+        one more leaf to reach; a computed tensor that requires grad has leaves this object
+        cannot see, and the first pass then stays unrestricted."""
+        stack = list(args) + list(kwargs.values())
+        while stack:
+            t = stack.pop()
+            if isinstance(t, (list, tuple)):
+                stack.extend(t)
+            elif isinstance(t, dict):
+                stack.extend(t.values())
+            elif isinstance(t, torch.Tensor) and t.requires_grad:
+                if t.is_leaf:
+                    self._first_pass_leaves[id(t)] = t
+                else:
+                    self._first_pass_open = True
+
+    def first_backward_inputs(self) -> List[torch.Tensor]:
+        """Leaves to pass as ``inputs=`` to the first backward pass of ghost clipping (empty:
+        do not restrict the pass); the record starts afresh for the next forward pass."""
+        leaves = [] if self._first_pass_open else list(self._first_pass_leaves.values())
+        self._first_pass_leaves = {}
+        self._first_pass_open = False
+        return leaves
 
     # ---- clipping coefficient ----------------------------------------------------------
     def get_norm_sample(self) -> torch.Tensor:
@@ -146,6 +196,7 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
             module.activations = []
         # non-tensor inputs (an omitted optional argument passed as None) are not activations
         module.activations.append([t.detach() for t in forward_input if isinstance(t, torch.Tensor)])
+        self._note_first_pass_leaves(module, forward_input)
         for _, p in trainable_parameters(module):
             p._forward_counter += 1
             if p._forward_counter == 1:

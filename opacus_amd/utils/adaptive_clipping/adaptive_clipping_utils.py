@@ -19,7 +19,11 @@ import torch
 import torch.nn as nn
 
 from ...privacy_engine import PrivacyEngine
-from ..fast_gradient_clipping_utils import DPLossFastGradientClipping, DPTensorFastGradientClipping
+from ..fast_gradient_clipping_utils import (
+    DPLossFastGradientClipping,
+    DPTensorFastGradientClipping,
+    first_pass_backward,
+)
 
 
 class DPTensorFastGradientAdaptiveClipping(DPTensorFastGradientClipping):
@@ -53,7 +57,7 @@ class DPTensorFastGradientAdaptiveClipping(DPTensorFastGradientClipping):
             reduced = torch.sum(self.loss_per_sample, dim=0)
         else:
             raise ValueError(f"loss_reduction = {self.loss_reduction}. Only 'sum' and 'mean' losses are supported")
-        reduced.backward(retain_graph=True)
+        first_pass_backward(self.module, reduced)
         self.optimizer.zero_grad()
 
         per_sample_norms = self.module.get_norm_sample()

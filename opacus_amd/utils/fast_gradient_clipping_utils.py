@@ -10,6 +10,20 @@ import copy
 import torch
 
 
+def first_pass_backward(module, reduced: torch.Tensor) -> None:
+    """Backward pass #1 of ghost clipping (fast_gradient_clipping_utils.py:189): only there
+    to let the hooks see the gradients of the layers' outputs. When the module can name the
+    leaves at the start of the graph, autograd is asked for those alone, which leaves out
+    the weight-gradient GEMMs of all other layers; what they would have written to ``.grad``
+    is zeroed by the caller in the next line anyway."""
+    leaves = getattr(module, "first_backward_inputs", None)
+    inputs = leaves() if callable(leaves) else None
+    if isinstance(inputs, (list, tuple)) and len(inputs) > 0:
+        reduced.backward(retain_graph=True, inputs=list(inputs))
+    else:
+        reduced.backward(retain_graph=True)
+
+
 class DPTensorFastGradientClipping:
     """A per-sample loss bound to its module and optimizer. ``backward()`` runs: backward #1
     (hooks collect per-sample gradient norms), ``optimizer.zero_grad()``, clipping
@@ -84,7 +98,7 @@ class DPTensorFastGradientClipping:
             reduced = torch.sum(self.loss_per_sample, dim=0)
         else:
             raise ValueError(f"loss_reduction = {self.loss_reduction}. Only 'sum' and 'mean' losses are supported")
-        reduced.backward(retain_graph=True)
+        first_pass_backward(self.module, reduced)
         self.optimizer.zero_grad()
         coeff = self.module.get_clipping_coef()
         weighted = coeff.to(self.loss_per_sample.device) * self.loss_per_sample

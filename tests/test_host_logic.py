@@ -568,6 +568,57 @@ def test_adaptive_dp_tensor_updates_bound_noise_and_uses_new_bound(monkeypatch):
         DPTensorFastGradientAdaptiveClipping(module, optimizer, (w * base).detach().requires_grad_(), "sum", initial_noise_multiplier=0.0).backward()
 
 
+def test_first_backward_pass_asks_for_the_entry_leaves_only():
+    """The first pass of ghost clipping exists for the hooks; its weight gradients are thrown
+    away. The hooks name the leaves at the start of the graph, and the pass is restricted to
+    them: parameters of modules fed by tensors without grad, and leaf inputs that require grad."""
+    from opacus_amd.utils.fast_gradient_clipping_utils import first_pass_backward
+
+    def forget_forward(module):  # what the backward hooks would have done, without kernels
+        for m in module.modules():
+            m.__dict__.pop("activations", None)
+        for p in module.parameters():
+            p._forward_counter = 0
+
+    net = nn.Sequential(nn.Linear(4, 5), nn.ReLU(), nn.Linear(5, 3), nn.Tanh(), nn.Linear(3, 2))
+    ghost = GradSampleModuleFastGradientClipping(net)
+    ghost.disable_hooks()
+    ghost(torch.randn(2, 4))
+    assert ghost.first_backward_inputs() == []
+    ghost.enable_hooks()
+    ghost.capture_backprops_hook = lambda *a, **k: None
+    out = ghost(torch.randn(2, 4))
+    leaves = ghost.first_backward_inputs()
+    assert {id(t) for t in leaves} == {id(net[0].weight), id(net[0].bias)}
+    assert ghost.first_backward_inputs() == []  # consumed
+    # restricted pass: the entry layer gets its gradient, the others are skipped
+    ghost._first_pass_leaves = {id(t): t for t in leaves}
+    first_pass_backward(ghost, out.sum())
+    assert net[0].weight.grad is not None and net[2].weight.grad is None and net[4].bias.grad is None
+    # a frozen entry layer moves the entry to the next trainable module; a leaf input that
+    # requires grad is a leaf to reach as well
+    net[0].weight.requires_grad_(False)
+    net[0].bias.requires_grad_(False)
+    forget_forward(net)
+    ghost.remove_hooks()
+    ghost2 = GradSampleModuleFastGradientClipping(nn.Sequential(net[0], net[1], net[2]))
+    ghost2.capture_backprops_hook = lambda *a, **k: None
+    x = torch.randn(2, 4)
+    ghost2(x)
+    assert {id(t) for t in ghost2.first_backward_inputs()} == {id(net[2].weight), id(net[2].bias)}
+    forget_forward(net)
+    x.requires_grad_(True)
+    ghost2(x)
+    assert {id(t) for t in ghost2.first_backward_inputs()} == {id(x)}  # seen at the model's entrance
+    forget_forward(net)
+    ghost2(x * 2.0)  # a computed input has leaves of its own: no restriction
+    assert ghost2.first_backward_inputs() == []
+    # a module object without the method (or a mock) falls back to the plain pass
+    w = torch.ones(3, requires_grad=True)
+    first_pass_backward(object(), (w * 2).sum())
+    torch.testing.assert_close(w.grad, torch.full((3,), 2.0))
+
+
 def test_dp_loss_requires_consistent_reductions_and_restores_reduction():
     module, optimizer = _mock_pair("mean")
     crit = nn.CrossEntropyLoss(reduction="mean")
