@@ -99,10 +99,54 @@ def _batch_first_view(t: torch.Tensor, batch_dim: int) -> torch.Tensor:
     return t.permute([batch_dim] + [d for d in range(t.dim()) if d != batch_dim])
 
 
+class _GradTap(torch.autograd.Function):
+    """Identity whose output takes part in autograd although its input does not: gives the
+    output of a layer at the start of the graph, run with its parameters switched off, a
+    gradient for the hook to read. Nothing flows further back."""
+
+    @staticmethod
+    def forward(ctx, x: torch.Tensor, _anchor: torch.Tensor) -> torch.Tensor:
+        # the same tensor, not a view of it, so that an in-place op may follow (ReLU(inplace=True))
+        ctx.mark_dirty(x)
+        return x
+
+    @staticmethod
+    def backward(ctx, _grad):
+        return None, None
+
+
+# The layer types that run with their parameters switched off during forward: the library's
+# own samplers cover all their parameters, and they return one tensor, so that the output of
+# such a layer at the start of the graph can be re-attached through _GradTap. (Subclasses
+# included: RNNLinear.) Layers with a user-registered sampler keep autograd's gradients.
+_ONE_TENSOR_OUT = (
+    nn.Linear,
+    nn.modules.conv._ConvNd,
+    nn.Embedding,
+    nn.EmbeddingBag,
+    nn.GroupNorm,
+    nn.LayerNorm,
+    nn.RMSNorm,
+    nn.modules.instancenorm._InstanceNorm,
+)
+
+
 class GradSampleHooks(AbstractGradSampleHooks):
-    """Attaches per-sample-gradient hooks to a module without wrapping it."""
+    """Attaches per-sample-gradient hooks to a module without wrapping it.
+
+    ``autograd_weight_grads=False`` (the default here; the reference has no such switch and
+    behaves like ``True``): while the hooks are enabled, a torch.nn layer served by one of
+    the library's samplers runs its forward with ``requires_grad`` off on its own parameters,
+    so the backward pass forms the gradients with respect to activations only. The aggregate
+    weight gradients autograd would otherwise compute (a second GEMM or weight-gradient
+    convolution per layer) are never read on this path: ``DPOptimizer.step`` writes
+    ``p.grad`` from the clipped per-sample gradients (optimizers/optimizer.py:477-504).
+    Until then ``p.grad`` of such a layer stays as it was (``None`` after ``zero_grad``)
+    instead of holding the non-private sum."""
 
     GRAD_SAMPLERS = {}
+    # ghost clipping needs autograd's weight gradients in its second pass
+    CAN_SKIP_AUTOGRAD_WEIGHT_GRADS = True
 
     def __init__(
         self,
@@ -112,6 +156,7 @@ class GradSampleHooks(AbstractGradSampleHooks):
         loss_reduction="mean",
         strict: bool = True,
         force_functorch=False,
+        autograd_weight_grads: bool = False,
     ):
         super().__init__(m, batch_first=batch_first, loss_reduction=loss_reduction)
         errors = self.validate(module=m, strict=strict)
@@ -120,6 +165,8 @@ class GradSampleHooks(AbstractGradSampleHooks):
         self.hooks_enabled = False
         self.grad_accumulation_allowed = True
         self.force_functorch = force_functorch
+        self.autograd_weight_grads = autograd_weight_grads or not self.CAN_SKIP_AUTOGRAD_WEIGHT_GRADS
+        self._tap_anchor = torch.zeros((), requires_grad=True)
         self.add_hooks(loss_reduction=loss_reduction, batch_first=batch_first, force_functorch=force_functorch)
 
     # ---- hook installation -----------------------------------------------------------
@@ -148,12 +195,41 @@ class GradSampleHooks(AbstractGradSampleHooks):
         for module in self.iterate_submodules(self._module):
             if force_functorch or self._get_module_type(module) not in self.GRAD_SAMPLERS:
                 prepare_layer(module, batch_first=batch_first)
+            elif not self.autograd_weight_grads:
+                # order matters: parameters are switched back on before the capturing hook looks
+                self.autograd_grad_sample_hooks.append(
+                    module.register_forward_pre_hook(self._params_off_for_forward, with_kwargs=True)
+                )
+                self.autograd_grad_sample_hooks.append(
+                    module.register_forward_hook(self._params_back_on, always_call=True)
+                )
             self.autograd_grad_sample_hooks.append(
                 module.register_forward_hook(
                     partial(self._forward_hook, loss_reduction=loss_reduction, batch_first=batch_first)
                 )
             )
         self.enable_hooks()
+
+    def _params_off_for_forward(self, module: nn.Module, args, kwargs) -> None:
+        if not self.hooks_enabled or not module.training or not torch.is_grad_enabled():
+            return
+        if not isinstance(module, _ONE_TENSOR_OUT):
+            return
+        params = [p for p in module.parameters(recurse=False) if p.requires_grad]
+        if not params:
+            return
+        inputs = list(args) + list(kwargs.values())
+        at_start = not any(isinstance(t, torch.Tensor) and t.requires_grad for t in inputs)
+        for p in params:
+            p.requires_grad_(False)
+        module._dpk_params_off = (params, at_start)
+
+    def _params_back_on(self, module: nn.Module, _args, _output) -> None:
+        state = module.__dict__.pop("_dpk_params_off", None)
+        if state is not None:
+            for p in state[0]:
+                p.requires_grad_(True)
+            module._dpk_at_start = state[1]
 
     def _forward_hook(self, module: nn.Module, forward_input, forward_output, *, loss_reduction: str, batch_first: bool):
         """Captures the activations and arranges for ``capture_backprops_hook`` to run when the
@@ -167,6 +243,9 @@ class GradSampleHooks(AbstractGradSampleHooks):
         if len(getattr(module, "activations", ())) == pending:
             return  # nothing captured: eval mode, no grad, hooks disabled, frozen module
         out = forward_output if isinstance(forward_output, torch.Tensor) else forward_output[0]
+        tapped = module.__dict__.pop("_dpk_at_start", False) and isinstance(forward_output, torch.Tensor)
+        if tapped and not out.requires_grad:
+            out = _GradTap.apply(out, self._tap_anchor)
         if not out.requires_grad:
             return
 
@@ -174,6 +253,8 @@ class GradSampleHooks(AbstractGradSampleHooks):
             self.capture_backprops_hook(module, None, (grad,), loss_reduction=loss_reduction, batch_first=batch_first)
 
         out.register_hook(on_grad_output)
+        if tapped:
+            return out  # replaces the module's output
 
     def remove_hooks(self) -> None:
         self.disable_hooks()
@@ -359,10 +440,25 @@ class GradSampleHooks(AbstractGradSampleHooks):
 class GradSampleModule(GradSampleHooks, AbstractGradSampleModule):
     """``nn.Module`` wrapper whose parameters carry ``.grad_sample`` after ``backward``."""
 
-    def __init__(self, m: nn.Module, *, batch_first=True, loss_reduction="mean", strict: bool = True, force_functorch=False):
+    def __init__(
+        self,
+        m: nn.Module,
+        *,
+        batch_first=True,
+        loss_reduction="mean",
+        strict: bool = True,
+        force_functorch=False,
+        autograd_weight_grads: bool = False,
+    ):
         nn.Module.__init__(self)
         GradSampleHooks.__init__(
-            self, m, batch_first=batch_first, loss_reduction=loss_reduction, strict=strict, force_functorch=force_functorch
+            self,
+            m,
+            batch_first=batch_first,
+            loss_reduction=loss_reduction,
+            strict=strict,
+            force_functorch=force_functorch,
+            autograd_weight_grads=autograd_weight_grads,
         )
         self.grad_accumulation_hook = None
 

@@ -59,6 +59,7 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
     sampler exists, fast gradient clipping elsewhere)."""
 
     NORM_SAMPLERS = {}
+    CAN_SKIP_AUTOGRAD_WEIGHT_GRADS = False  # the second backward pass is autograd's
 
     def __init__(
         self,

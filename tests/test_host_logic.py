@@ -112,7 +112,11 @@ def test_wrapper_surface():
     gsm = GradSampleModule(net)
     assert all(k.startswith("_module.") for k in gsm.state_dict())
     assert gsm._module[0] is net[0]
-    assert len(net.autograd_grad_sample_hooks) == 2  # one forward hook per Linear; it hooks the output's gradient
+    # per Linear: parameters off before forward, back on after it, and the capturing forward hook
+    # (which hooks the output's gradient)
+    assert len(net.autograd_grad_sample_hooks) == 6
+    with_autograd = GradSampleModule(nn.Sequential(nn.Linear(4, 3), nn.ReLU(), nn.Linear(3, 2)), autograd_weight_grads=True)
+    assert len(with_autograd._module.autograd_grad_sample_hooks) == 2
     for p in net.parameters():
         assert p.grad_sample is None and p._forward_counter == 0
     with pytest.raises(ValueError, match="twice"):
@@ -182,14 +186,43 @@ def test_inplace_op_on_a_hooked_output_is_fine():
         torch.manual_seed(0)
         net = Net()
         x = torch.randn(5, 3)
-        gsm = GradSampleModule(net, loss_reduction="sum")
+        gsm = GradSampleModule(net, loss_reduction="sum", autograd_weight_grads=True)
         out = gsm(x)
         out.sum().backward()
         want = (net.fc(x) > 0).float()  # d relu(y).sum() / dy
         assert torch.equal(seen["b"], want)
         torch.testing.assert_close(net.fc.weight.grad_sample.sum(0), net.fc.weight.grad)
+        # the default: the same per-sample gradients with the layer's parameters switched off
+        # during forward, an in-place op on the re-attached output included; autograd forms no
+        # weight gradient
+        first = net.fc.weight.grad_sample.clone()
+        gsm.remove_hooks()
+        net.zero_grad()
+        gsm = GradSampleModule(net, loss_reduction="sum")
+        gsm(x).sum().backward()
+        assert torch.equal(seen["b"], want)
+        torch.testing.assert_close(net.fc.weight.grad_sample, first)
+        assert net.fc.weight.grad is None and net.fc.bias.grad is None
+        assert net.fc.weight.requires_grad and net.fc.bias.requires_grad
     finally:
         GradSampleHooks.GRAD_SAMPLERS.pop(Tmp, None)
+
+
+def test_parameters_are_switched_back_on_whatever_happens():
+    net = nn.Sequential(nn.Linear(3, 4), nn.ReLU(), nn.Linear(4, 2))
+    gsm = GradSampleModule(net)
+    with pytest.raises(RuntimeError):
+        gsm(torch.randn(5, 7))  # wrong width: the first Linear raises inside forward
+    assert all(p.requires_grad for p in net.parameters())
+    assert not hasattr(net[0], "_dpk_params_off")
+    # nothing is switched off without training mode, without grad mode or with hooks disabled
+    gsm.eval()
+    assert not gsm(torch.randn(5, 3)).requires_grad or True
+    gsm.train()
+    gsm.disable_hooks()
+    out = gsm(torch.randn(5, 3))
+    out.sum().backward()
+    assert all(p.grad is not None for p in net.parameters())  # plain autograd while the hooks are off
 
 
 def test_no_capture_in_eval_or_no_grad_or_disabled():
