@@ -141,7 +141,35 @@ __global__ __launch_bounds__(kThreads) void conv2d_gs_kernel(
 //   qtab[q] = oh * sh * Wp + ow * sw                              (table in LDS)
 // and the MFMA's B operand is read straight from the patch. The gather kernel
 // above spends more VALU cycles on (iy, ix) bounds and addresses than the MFMAs
-// take; here the k loop is MFMAs, LDS reads and the staging of the backprop tile.
+// take; here the k loop is MFMAs, LDS reads of the patch and register loads of the
+// backprops.
+// 4 consecutive elements / one element at a byte offset of a buffer descriptor (zeros past
+// its end)
+template <typename T> __device__ __forceinline__ float4 buffer_load4(__amdgpu_buffer_rsrc_t r, uint32_t off);
+template <> __device__ __forceinline__ float4 buffer_load4<float>(__amdgpu_buffer_rsrc_t r, uint32_t off) {
+  typedef int vi4 __attribute__((ext_vector_type(4)));
+  const vi4 v = __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0);
+  return make_float4(__int_as_float(v.x), __int_as_float(v.y), __int_as_float(v.z), __int_as_float(v.w));
+}
+template <> __device__ __forceinline__ float4 buffer_load4<bf16_t>(__amdgpu_buffer_rsrc_t r, uint32_t off) {
+  typedef int vi2 __attribute__((ext_vector_type(2)));
+  const vi2 v = __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 0);
+  return make_float4(__uint_as_float(static_cast<uint32_t>(v.x) << 16),
+                     __uint_as_float(static_cast<uint32_t>(v.x) & 0xffff0000u),
+                     __uint_as_float(static_cast<uint32_t>(v.y) << 16),
+                     __uint_as_float(static_cast<uint32_t>(v.y) & 0xffff0000u));
+}
+template <typename T> __device__ __forceinline__ float buffer_load1(__amdgpu_buffer_rsrc_t r, uint32_t off);
+template <> __device__ __forceinline__ float buffer_load1<float>(__amdgpu_buffer_rsrc_t r, uint32_t off) {
+  return __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, off, 0, 0));
+}
+template <> __device__ __forceinline__ float buffer_load1<bf16_t>(__amdgpu_buffer_rsrc_t r, uint32_t off) {
+  return __uint_as_float(static_cast<uint32_t>(static_cast<uint16_t>(__builtin_amdgcn_raw_buffer_load_b16(r, off, 0, 0))) << 16);
+}
+
+constexpr int kPatchDepth = 4;                        // backprop k-tiles in flight per lane
+constexpr int kPatchTrip = kPatchDepth * mf32::BK;    // k extent of one trip of the k loop
+
 template <int BM, int BN, typename TIN, typename TOUT, bool VEC>
 __global__ __launch_bounds__(kThreads) void conv2d_gs_patch_kernel(
     const TIN* __restrict__ x, const TIN* __restrict__ b, TOUT* __restrict__ gs,
@@ -149,12 +177,11 @@ __global__ __launch_bounds__(kThreads) void conv2d_gs_patch_kernel(
     int tiles_n, int Hp, int Wp, int pr, int nch_max) {
   using Tile = mf32::Tile<BM, BN>;
   extern __shared__ __align__(16) unsigned char dyn_lds[];
-  // layout: A stages | qtab | patch
-  typedef float (*AStage)[BM + mf32::PAD];
-  float* a_mem = reinterpret_cast<float*>(dyn_lds);
-  constexpr int kAStage = mf32::BK * (BM + mf32::PAD);
-  const int Qpad = (g.Q + mf32::BK - 1) / mf32::BK * mf32::BK;
-  int* qtab = reinterpret_cast<int*>(a_mem + 2 * kAStage);
+  // layout: qtab | patch. The k loop runs in trips of kPatchDepth k-tiles, all of them
+  // unconditional: past the end the backprops read as zeros and the table points at the
+  // patch's first element.
+  const int Qpad = (g.Q + kPatchTrip - 1) / kPatchTrip * kPatchTrip;
+  int* qtab = reinterpret_cast<int*>(dyn_lds);
   float* xs = reinterpret_cast<float*>(qtab + Qpad);
   __shared__ float red[kWaves];
 
@@ -174,27 +201,38 @@ __global__ __launch_bounds__(kThreads) void conv2d_gs_patch_kernel(
   const int nch = c_hi - c_lo + 1;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 
-  // stage the patch (zero outside the image): 8 independent loads per thread are
-  // issued before any of them is stored, so the block pays global latency once per
-  // batch rather than once per element
+  // stage the patch (zero outside the image). A wave takes whole rows of the padded patch,
+  // lane = column, so no index is ever divided: (channel, row) advance by additions. Eight
+  // rows are loaded before any of them is stored, so global latency is paid once per eight.
   const TIN* xg = x + ((sample * C + static_cast<int64_t>(grp) * Cg + c_lo) * g.H) * g.W;
-  const int plane = Hp * Wp, total = nch * plane;
-  for (int i0 = threadIdx.x; i0 < total; i0 += kThreads * 8) {
-    float v[8];
-#pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const int i = i0 + u * kThreads;
-      const int c = i / plane, r = i - c * plane;
-      const int y = r / Wp, xx = r - y * Wp;
-      const int iy = y - g.ph, ix = xx - g.pw;
-      const bool in = i < total && static_cast<unsigned>(iy) < static_cast<unsigned>(g.H) &&
-                      static_cast<unsigned>(ix) < static_cast<unsigned>(g.W);
-      v[u] = in ? dpk_io<TIN>::load(xg + (static_cast<int64_t>(c) * g.H + iy) * g.W + ix) : 0.f;
+  const int rows = nch * Hp;
+  constexpr int kRowsInFlight = 8;
+  for (int x0 = 0; x0 < Wp; x0 += DPK_WAVE) {
+    const int xx = x0 + lane, ix = xx - g.pw;
+    const bool col_ok = xx < Wp && static_cast<unsigned>(ix) < static_cast<unsigned>(g.W);
+    int c = 0, y = wave;  // of the next row this wave stages
+    while (y >= Hp) {
+      y -= Hp;
+      ++c;
     }
+    for (int row = wave; row < rows; row += kWaves * kRowsInFlight) {
+      float v[kRowsInFlight];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const int i = i0 + u * kThreads;
-      if (i < total) xs[i] = v[u];
+      for (int u = 0; u < kRowsInFlight; ++u) {
+        const int iy = y - g.ph;
+        const bool in = col_ok && row + u * kWaves < rows && static_cast<unsigned>(iy) < static_cast<unsigned>(g.H);
+        v[u] = in ? dpk_io<TIN>::load(xg + (static_cast<int64_t>(c) * g.H + iy) * g.W + ix) : 0.f;
+        y += kWaves;
+        while (y >= Hp) {
+          y -= Hp;
+          ++c;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kRowsInFlight; ++u) {
+        const int r = row + u * kWaves;
+        if (r < rows && xx < Wp) xs[r * Wp + xx] = v[u];
+      }
     }
   }
   for (int q = threadIdx.x; q < Qpad; q += kThreads) {
@@ -219,78 +257,92 @@ __global__ __launch_bounds__(kThreads) void conv2d_gs_patch_kernel(
   (void)pr;
   (void)nch_max;
 
-  // Backprop tile pipeline: BM x 16 floats per k-tile is one 16-byte load per
-  // thread, so D tiles are kept in flight in registers (slot = tile % D) and global
-  // latency is covered by D - 1 steps of MFMAs even with few waves per SIMD.
-  static_assert(BM == 64, "one 16-byte load per thread and k-tile");
-  constexpr int D = 4;
+  // The backprop operand goes from global memory straight into registers. The instruction
+  // contracts two k per step, one from each half of the wave; which k of the tile a half
+  // takes is free, so half kk takes k = 8 kk .. 8 kk + 7: eight consecutive backprops of
+  // the lane's output channel, two 16-byte loads. Nothing is staged in LDS and the k loop
+  // has no barrier: every wave runs at its own pace, with kPatchDepth tiles of loads in
+  // flight, while the gathered operand of the next tile (a table read, then a patch read
+  // that depends on it) is asked for during the MFMAs of the current one.
+  constexpr int D = kPatchDepth;
+  constexpr int K2 = mf32::BK / 2;
+  static_assert(K2 == 8, "two 4-element loads per lane and k-tile");
   const TIN* bg = b + (sample * O + static_cast<int64_t>(grp) * Og) * g.Q;
-  const int am = threadIdx.x / (mf32::BK / 4), ak = (threadIdx.x % (mf32::BK / 4)) * 4;
-  const int64_t arow = m0 + am;
-  const TIN* ap = bg + arow * g.Q + ak;
-  float4 slot[D];
-  auto fetch = [&](int64_t kt, float4& dst) {
-    const int64_t k = kt * mf32::BK + ak;
-    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (arow < Og && k < g.Q) {
-      const TIN* p = ap + kt * mf32::BK;
+  // loads through a buffer descriptor over the group's Og x Q backprops: a lane whose row
+  // or k lies outside gets an offset past the descriptor's end and reads zeros
+  const __amdgpu_buffer_rsrc_t brs = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<TIN*>(bg), 0, Og * g.Q * static_cast<int>(sizeof(TIN)), 0x00020000);
+  constexpr uint32_t kOutside = 0x7fffffffu;
+  int row_el[Tile::TM];  // element offset of (row, k = 8 kk), or -1 for a row outside
+#pragma unroll
+  for (int i = 0; i < Tile::TM; ++i) {
+    const int m = m0 + wm0 + i * 32 + l32;
+    row_el[i] = m < Og ? m * g.Q + kk * K2 : -1;
+  }
+  auto fetch = [&](int kt, float (&a)[Tile::TM][K2]) {
+    const int k = kt * mf32::BK + kk * K2;
+#pragma unroll
+    for (int i = 0; i < Tile::TM; ++i) {
       if (VEC) {
-        v = dpk_io<TIN>::load4(p);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const bool in = row_el[i] >= 0 && k + 4 * h < g.Q;
+          const uint32_t off =
+              in ? static_cast<uint32_t>(row_el[i] + kt * mf32::BK + 4 * h) * sizeof(TIN) : kOutside;
+          const float4 v = buffer_load4<TIN>(brs, off);
+          a[i][4 * h + 0] = v.x;
+          a[i][4 * h + 1] = v.y;
+          a[i][4 * h + 2] = v.z;
+          a[i][4 * h + 3] = v.w;
+        }
       } else {
-        v.x = dpk_io<TIN>::load(p);
-        if (k + 1 < g.Q) v.y = dpk_io<TIN>::load(p + 1);
-        if (k + 2 < g.Q) v.z = dpk_io<TIN>::load(p + 2);
-        if (k + 3 < g.Q) v.w = dpk_io<TIN>::load(p + 3);
+#pragma unroll
+        for (int e = 0; e < K2; ++e) {
+          const bool in = row_el[i] >= 0 && k + e < g.Q;
+          const uint32_t off = in ? static_cast<uint32_t>(row_el[i] + kt * mf32::BK + e) * sizeof(TIN) : kOutside;
+          a[i][e] = buffer_load1<TIN>(brs, off);
+        }
       }
     }
-    dst = v;
   };
-  auto commit = [&](const float4& v, AStage S) {
-    S[ak + 0][am] = v.x;
-    S[ak + 1][am] = v.y;
-    S[ak + 2][am] = v.z;
-    S[ak + 3][am] = v.w;
+  float av[D][Tile::TM][K2], bv[2][K2][Tile::TN];
+  int qo[2][K2];
+  const int nk = Qpad / mf32::BK;  // a multiple of D
+  auto read_q = [&](int kt, int (&q)[K2]) {
+    const int* qt = qtab + (kt < nk ? kt : 0) * mf32::BK + kk * K2;  // past the end: any valid entries
+#pragma unroll
+    for (int k2 = 0; k2 < K2; ++k2) q[k2] = qt[k2];
+  };
+  auto read_b = [&](const int (&q)[K2], float (&bb)[K2][Tile::TN]) {
+#pragma unroll
+    for (int k2 = 0; k2 < K2; ++k2)
+#pragma unroll
+      for (int j = 0; j < Tile::TN; ++j) bb[k2][j] = xs[base_p[j] + q[k2]];
   };
   Tile tile;
   tile.clear();
-  const int64_t nk = (g.Q + mf32::BK - 1) / mf32::BK;
 #pragma unroll
-  for (int d = 0; d < D - 1; ++d)
-    if (d < nk) fetch(d, slot[d]);
-  commit(slot[0], reinterpret_cast<AStage>(a_mem));
-  __syncthreads();  // also publishes the patch and qtab
-  for (int64_t kt0 = 0; kt0 < nk; kt0 += D) {
+  for (int d = 0; d < D - 1; ++d) fetch(d, av[d]);
+  __syncthreads();  // publishes the patch and qtab; the only barrier of the kernel body
+  read_q(0, qo[0]);
+  read_b(qo[0], bv[0]);
+  read_q(1, qo[1]);
+  for (int kt0 = 0; kt0 < nk; kt0 += D) {
 #pragma unroll
     for (int d = 0; d < D; ++d) {
-      const int64_t kt = kt0 + d;
-      if (kt < nk) {
-        if (kt + D - 1 < nk) fetch(kt + D - 1, slot[(d + D - 1) % D]);
-        AStage As = reinterpret_cast<AStage>(a_mem + (d & 1) * kAStage);
-        const int* qt = qtab + kt * mf32::BK;
-        int qo[mf32::BK / 2];
+      const int kt = kt0 + d;
+      const int cur = d & 1, nxt = cur ^ 1;
+      fetch(kt + D - 1, av[(d + D - 1) % D]);
+      read_b(qo[nxt], bv[nxt]);
+      read_q(kt + 2, qo[cur]);  // tile kt's offsets were consumed one step ago
 #pragma unroll
-        for (int k2 = 0; k2 < mf32::BK / 2; ++k2) qo[k2] = qt[2 * k2 + kk];
-        // all operand reads of the k-tile first, then its MFMAs: LDS latency is paid once
-        float av[mf32::BK / 2][Tile::TM], bv[mf32::BK / 2][Tile::TN];
+      for (int k2 = 0; k2 < K2; ++k2)
 #pragma unroll
-        for (int k2 = 0; k2 < mf32::BK / 2; ++k2) {
+        for (int i = 0; i < Tile::TM; ++i)
 #pragma unroll
-          for (int i = 0; i < Tile::TM; ++i) av[k2][i] = As[2 * k2 + kk][wm0 + i * 32 + l32];
-#pragma unroll
-          for (int j = 0; j < Tile::TN; ++j) bv[k2][j] = xs[base_p[j] + qo[k2]];
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int k2 = 0; k2 < mf32::BK / 2; ++k2)
-#pragma unroll
-          for (int i = 0; i < Tile::TM; ++i)
-#pragma unroll
-            for (int j = 0; j < Tile::TN; ++j)
-              tile.acc[i][j] =
-                  __builtin_amdgcn_mfma_f32_32x32x2f32(av[k2][i], bv[k2][j], tile.acc[i][j], 0, 0, 0);
-        if (kt + 1 < nk) commit(slot[(d + 1) % D], reinterpret_cast<AStage>(a_mem + ((d + 1) & 1) * kAStage));
-        __syncthreads();
-      }
+          for (int j = 0; j < Tile::TN; ++j)
+            tile.acc[i][j] =
+                __builtin_amdgcn_mfma_f32_32x32x2f32(av[d][i][k2], bv[cur][k2][j], tile.acc[i][j], 0, 0, 0);
     }
   }
   TOUT* out = gs + (sample * O + static_cast<int64_t>(grp) * Og) * g.Pg;
@@ -314,8 +366,8 @@ size_t patch_lds_bytes(const ConvGeom& g, int Cg, int Hp, int Wp) {
   const int KK = g.KH * g.KW;
   int nch = (64 + KK - 2) / KK + 1;  // channels a run of 64 columns can touch
   if (nch > Cg) nch = Cg;
-  const size_t a_bytes = 2 * mf32::BK * (64 + mf32::PAD) * sizeof(float);
-  const size_t q_bytes = static_cast<size_t>((g.Q + mf32::BK - 1) / mf32::BK * mf32::BK) * sizeof(int);
+  const size_t a_bytes = 0;  // the backprop operand is not staged
+  const size_t q_bytes = static_cast<size_t>((g.Q + kPatchTrip - 1) / kPatchTrip * kPatchTrip) * sizeof(int);
   const size_t x_bytes = static_cast<size_t>(nch) * Hp * Wp * sizeof(float);
   const size_t total = a_bytes + q_bytes + x_bytes;
   return total <= 64 * 1024 - 64 ? total : 0;
@@ -437,7 +489,9 @@ int conv_gs(const char* who, const void* x, const void* b, int in_dtype, void* g
   const int64_t Hp = H + ph_lo + ph_hi, Wp = W + pw_lo + pw_hi;
   const bool flat = z.D == 1 && z.KD == 1 && z.pd_lo == 0 && z.pd_hi == 0;  // the LDS patch is two-dimensional
   const size_t patch_bytes =
-      flat && Hp * Wp < (1 << 20) ? patch_lds_bytes(g, (int)(C / groups), (int)Hp, (int)Wp) : 0;
+      flat && Hp * Wp < (1 << 20) && (O / groups) * Q * 4 < (1LL << 30)
+          ? patch_lds_bytes(g, (int)(C / groups), (int)Hp, (int)Wp)
+          : 0;
   const Plan p = make_plan(O / groups, Pg, patch_bytes > 0);
   const int64_t blocks = n * groups * p.tiles_m * p.tiles_n;
   DPK_REQUIRE(blocks <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: %lld blocks exceed the grid limit", who,
@@ -450,6 +504,7 @@ int conv_gs(const char* who, const void* x, const void* b, int in_dtype, void* g
     DPK_REQUIRE(dpk_aligned(ws, 4), DPK_E_ALIGN, "%s: workspace misaligned", who);
     partials = static_cast<float*>(ws);
   }
+  // 16-byte (8-byte for bf16) loads of 4 backprops
   const bool vec = Q % 4 == 0 && dpk_aligned(b, in_dtype == DPK_BF16 ? 8 : 16);
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (in_dtype == DPK_F32 && gs_dtype == DPK_F32)
