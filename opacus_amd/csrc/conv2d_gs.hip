@@ -174,7 +174,7 @@ template <int BM, int BN, typename TIN, typename TOUT, bool VEC>
 __global__ __launch_bounds__(kThreads) void conv2d_gs_patch_kernel(
     const TIN* __restrict__ x, const TIN* __restrict__ b, TOUT* __restrict__ gs,
     float* __restrict__ partials, ConvGeom g, int C, int O, int groups, float scale, int tiles_m,
-    int tiles_n, int Hp, int Wp, int pr, int nch_max) {
+    int tiles_n, int Hp, int Wp, int xvec, int nch_max) {
   using Tile = mf32::Tile<BM, BN>;
   extern __shared__ __align__(16) unsigned char dyn_lds[];
   // layout: qtab | patch. The k loop runs in trips of kPatchDepth k-tiles, all of them
@@ -202,12 +202,45 @@ __global__ __launch_bounds__(kThreads) void conv2d_gs_patch_kernel(
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 
   // stage the patch (zero outside the image). A wave takes whole rows of the padded patch,
-  // lane = column, so no index is ever divided: (channel, row) advance by additions. Eight
-  // rows are loaded before any of them is stored, so global latency is paid once per eight.
+  // lane = column, so no index is ever divided: (channel, row) advance by additions. 32 rows
+  // are loaded before any of them is stored: the staging is bound by global latency.
+  // When image rows are whole 16-byte chunks (xvec) the interior is instead fetched as
+  // 4-element chunks, eight per thread all in flight at once - one round trip per block -
+  // after the patch has been zeroed for its padding.
   const TIN* xg = x + ((sample * C + static_cast<int64_t>(grp) * Cg + c_lo) * g.H) * g.W;
   const int rows = nch * Hp;
-  constexpr int kRowsInFlight = 8;
-  for (int x0 = 0; x0 < Wp; x0 += DPK_WAVE) {
+  constexpr int kRowsInFlight = 32;
+  if (xvec) {
+    const int total4 = rows * Wp / 4;  // the patch starts 16-byte aligned; a ragged tail is zeroed below
+    for (int i = threadIdx.x; i < total4; i += kThreads)
+      reinterpret_cast<float4*>(xs)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int i = total4 * 4 + threadIdx.x; i < rows * Wp; i += kThreads) xs[i] = 0.f;
+    __syncthreads();
+    const int W4 = g.W / 4, chunks = nch * g.H * W4;
+    constexpr int kChunksInFlight = 8;
+    for (int i0 = threadIdx.x; i0 < chunks; i0 += kThreads * kChunksInFlight) {
+      float4 v[kChunksInFlight];
+#pragma unroll
+      for (int u = 0; u < kChunksInFlight; ++u) {
+        const int i = i0 + u * kThreads;
+        v[u] = i < chunks ? dpk_io<TIN>::load4(xg + static_cast<int64_t>(i) * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+#pragma unroll
+      for (int u = 0; u < kChunksInFlight; ++u) {
+        const int i = i0 + u * kThreads;
+        if (i < chunks) {
+          const int r = i / W4, x4 = i - r * W4;     // r = c * H + iy
+          const int c = r / g.H, iy = r - c * g.H;
+          float* dst = xs + (c * Hp + iy + g.ph) * Wp + g.pw + x4 * 4;
+          dst[0] = v[u].x;
+          dst[1] = v[u].y;
+          dst[2] = v[u].z;
+          dst[3] = v[u].w;
+        }
+      }
+    }
+  }
+  for (int x0 = 0; x0 < (xvec ? 0 : Wp); x0 += DPK_WAVE) {
     const int xx = x0 + lane, ix = xx - g.pw;
     const bool col_ok = xx < Wp && static_cast<unsigned>(ix) < static_cast<unsigned>(g.W);
     int c = 0, y = wave;  // of the next row this wave stages
@@ -254,7 +287,6 @@ __global__ __launch_bounds__(kThreads) void conv2d_gs_patch_kernel(
       base_p[j] = 0;  // result discarded below; any address inside the patch will do
     }
   }
-  (void)pr;
   (void)nch_max;
 
   // The backprop operand goes from global memory straight into registers. The instruction
@@ -404,12 +436,14 @@ void launch(const Plan& p, bool vec, const void* x, const void* b, void* gs, flo
   const TIN* bp = static_cast<const TIN*>(b);
   TOUT* gp = static_cast<TOUT*>(gs);
   if (patch_bytes > 0) {
+    // image rows made of whole, aligned 4-element chunks: the patch interior is staged with vector loads
+    const int xvec = (g.W % 4 == 0 && dpk_aligned(x, sizeof(TIN) == 2 ? 8 : 16)) ? 1 : 0;
     if (vec)
       hipLaunchKernelGGL((conv2d_gs_patch_kernel<64, 64, TIN, TOUT, true>), grid, block, patch_bytes, s, xp,
-                         bp, gp, partials, g, C, O, groups, scale, p.tiles_m, p.tiles_n, Hp, Wp, 0, 0);
+                         bp, gp, partials, g, C, O, groups, scale, p.tiles_m, p.tiles_n, Hp, Wp, xvec, 0);
     else
       hipLaunchKernelGGL((conv2d_gs_patch_kernel<64, 64, TIN, TOUT, false>), grid, block, patch_bytes, s,
-                         xp, bp, gp, partials, g, C, O, groups, scale, p.tiles_m, p.tiles_n, Hp, Wp, 0, 0);
+                         xp, bp, gp, partials, g, C, O, groups, scale, p.tiles_m, p.tiles_n, Hp, Wp, xvec, 0);
     return;
   }
 #define DPK_CONV_LAUNCH(BM, BN, V, D3)                                                            \
