@@ -367,6 +367,9 @@ __global__ __launch_bounds__(kThreads) void conv2d_gs_patch_kernel(
       fetch(kt + D - 1, av[(d + D - 1) % D]);
       read_b(qo[nxt], bv[nxt]);
       read_q(kt + 2, qo[cur]);  // tile kt's offsets were consumed one step ago
+      // keep the requests above ahead of the MFMAs below: left to itself the scheduler
+      // sinks each LDS read to just before the MFMA that uses it
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int k2 = 0; k2 < K2; ++k2)
 #pragma unroll
