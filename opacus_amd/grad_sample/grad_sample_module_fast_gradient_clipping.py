@@ -122,20 +122,26 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
         )
 
     # ---- what the first backward pass has to reach -----------------------------------------
-    def _note_first_pass_leaves(self, module: nn.Module, forward_input) -> None:
+    def _note_first_pass_leaves(self, module: nn.Module, forward_input, forward_output) -> None:
         """The norm pass needs the gradient of every hooked module's OUTPUT, never a weight
         gradient (``optimizer.zero_grad()`` discards those right after,
         fast_gradient_clipping_utils.py:190-191). Autograd computes exactly the output
-        gradients, and skips every other weight-gradient GEMM, when it is asked only for the
-        leaves at the start of the graph: the parameters of modules none of whose inputs
-        requires grad, and inputs that are themselves leaves requiring grad."""
+        gradients, and skips every weight-gradient GEMM, when it is asked only for the
+        tensors at the start of the graph: the outputs of modules none of whose inputs
+        requires grad (or, where such an output is not a single tensor, their parameters),
+        and inputs that are leaves requiring grad."""
         tensors = [t for t in forward_input if isinstance(t, torch.Tensor)]
         if not any(t.requires_grad for t in tensors):
-            for _, p in trainable_parameters(module):
-                self._first_pass_leaves[id(p)] = p
+            if isinstance(forward_output, torch.Tensor) and forward_output.requires_grad:
+                # kept with its version: an in-place op on it later moves the tensor to
+                # another node of the graph, and the module's parameters are asked for instead
+                self._first_pass_leaves[id(forward_output)] = (forward_output, forward_output._version, module)
+            else:
+                for _, p in trainable_parameters(module):
+                    self._first_pass_leaves[id(p)] = (p, None, module)
         for t in tensors:
             if t.requires_grad and t.is_leaf:
-                self._first_pass_leaves[id(t)] = t
+                self._first_pass_leaves[id(t)] = (t, None, module)
 
     def _note_model_inputs(self, _module, args, kwargs) -> None:
         """Inputs of the model that carry a graph of their own: a leaf that requires grad is
@@ -150,14 +156,20 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
                 stack.extend(t.values())
             elif isinstance(t, torch.Tensor) and t.requires_grad:
                 if t.is_leaf:
-                    self._first_pass_leaves[id(t)] = t
+                    self._first_pass_leaves[id(t)] = (t, None, None)
                 else:
                     self._first_pass_open = True
 
     def first_backward_inputs(self) -> List[torch.Tensor]:
         """Leaves to pass as ``inputs=`` to the first backward pass of ghost clipping (empty:
         do not restrict the pass); the record starts afresh for the next forward pass."""
-        leaves = [] if self._first_pass_open else list(self._first_pass_leaves.values())
+        leaves = []
+        if not self._first_pass_open:
+            for t, version, module in self._first_pass_leaves.values():
+                if version is None or t._version == version:
+                    leaves.append(t)
+                else:
+                    leaves.extend(p for _, p in trainable_parameters(module))
         self._first_pass_leaves = {}
         self._first_pass_open = False
         return leaves
@@ -197,7 +209,7 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
             module.activations = []
         # non-tensor inputs (an omitted optional argument passed as None) are not activations
         module.activations.append([t.detach() for t in forward_input if isinstance(t, torch.Tensor)])
-        self._note_first_pass_leaves(module, forward_input)
+        self._note_first_pass_leaves(module, forward_input, _forward_output)
         for _, p in trainable_parameters(module):
             p._forward_counter += 1
             if p._forward_counter == 1:

@@ -13,13 +13,16 @@ import torch
 def first_pass_backward(module, reduced: torch.Tensor) -> None:
     """Backward pass #1 of ghost clipping (fast_gradient_clipping_utils.py:189): only there
     to let the hooks see the gradients of the layers' outputs. When the module can name the
-    leaves at the start of the graph, autograd is asked for those alone, which leaves out
-    the weight-gradient GEMMs of all other layers; what they would have written to ``.grad``
-    is zeroed by the caller in the next line anyway."""
+    tensors at the start of the graph, autograd is asked for those alone, which leaves out
+    the weight-gradient GEMMs of the pass; what they would have written to ``.grad`` is
+    zeroed by the caller in the next line anyway."""
     leaves = getattr(module, "first_backward_inputs", None)
     inputs = leaves() if callable(leaves) else None
     if isinstance(inputs, (list, tuple)) and len(inputs) > 0:
         reduced.backward(retain_graph=True, inputs=list(inputs))
+        for t in inputs:
+            if not t.is_leaf:
+                t.grad = None  # an activation's gradient: the hooks have seen it, nobody else needs it
     else:
         reduced.backward(retain_graph=True)
 

@@ -601,10 +601,10 @@ def test_adaptive_dp_tensor_updates_bound_noise_and_uses_new_bound(monkeypatch):
         DPTensorFastGradientAdaptiveClipping(module, optimizer, (w * base).detach().requires_grad_(), "sum", initial_noise_multiplier=0.0).backward()
 
 
-def test_first_backward_pass_asks_for_the_entry_leaves_only():
+def test_first_backward_pass_asks_for_the_entry_tensors_only():
     """The first pass of ghost clipping exists for the hooks; its weight gradients are thrown
-    away. The hooks name the leaves at the start of the graph, and the pass is restricted to
-    them: parameters of modules fed by tensors without grad, and leaf inputs that require grad."""
+    away. The hooks name the tensors at the start of the graph, and the pass is restricted to
+    them: outputs of modules fed by tensors without grad, and leaf inputs that require grad."""
     from opacus_amd.utils.fast_gradient_clipping_utils import first_pass_backward
 
     def forget_forward(module):  # what the backward hooks would have done, without kernels
@@ -613,32 +613,45 @@ def test_first_backward_pass_asks_for_the_entry_leaves_only():
         for p in module.parameters():
             p._forward_counter = 0
 
-    net = nn.Sequential(nn.Linear(4, 5), nn.ReLU(), nn.Linear(5, 3), nn.Tanh(), nn.Linear(3, 2))
+    net = nn.Sequential(nn.Linear(4, 5), nn.Tanh(), nn.Linear(5, 3), nn.Tanh(), nn.Linear(3, 2))
     ghost = GradSampleModuleFastGradientClipping(net)
     ghost.disable_hooks()
     ghost(torch.randn(2, 4))
     assert ghost.first_backward_inputs() == []
     ghost.enable_hooks()
-    ghost.capture_backprops_hook = lambda *a, **k: None
+    fired = []
+    ghost.capture_backprops_hook = lambda module, *a, **k: fired.append(module)
     out = ghost(torch.randn(2, 4))
     leaves = ghost.first_backward_inputs()
-    assert {id(t) for t in leaves} == {id(net[0].weight), id(net[0].bias)}
+    assert len(leaves) == 1 and leaves[0].shape == (2, 5) and not leaves[0].is_leaf  # the first Linear's output
     assert ghost.first_backward_inputs() == []  # consumed
-    # restricted pass: the entry layer gets its gradient, the others are skipped
-    ghost._first_pass_leaves = {id(t): t for t in leaves}
+    # the restricted pass reaches every hooked layer's output, forms no weight gradient and
+    # leaves no gradient behind on the activation it was asked for
+    ghost.first_backward_inputs = lambda: leaves
     first_pass_backward(ghost, out.sum())
-    assert net[0].weight.grad is not None and net[2].weight.grad is None and net[4].bias.grad is None
+    assert fired == [net[4], net[2], net[0]]
+    assert all(p.grad is None for p in net.parameters()) and leaves[0].grad is None
+    del ghost.first_backward_inputs
+    # an in-place op on the entry layer's output: its parameters are asked for instead
+    forget_forward(net)
+    ghost.remove_hooks()
+    inplace = nn.Sequential(net[0], nn.ReLU(inplace=True), net[2])
+    ghost1 = GradSampleModuleFastGradientClipping(inplace)
+    ghost1.capture_backprops_hook = lambda *a, **k: None
+    ghost1(torch.randn(2, 4))
+    assert {id(t) for t in ghost1.first_backward_inputs()} == {id(net[0].weight), id(net[0].bias)}
     # a frozen entry layer moves the entry to the next trainable module; a leaf input that
-    # requires grad is a leaf to reach as well
+    # requires grad is a tensor to reach as well
     net[0].weight.requires_grad_(False)
     net[0].bias.requires_grad_(False)
     forget_forward(net)
-    ghost.remove_hooks()
+    ghost1.remove_hooks()
     ghost2 = GradSampleModuleFastGradientClipping(nn.Sequential(net[0], net[1], net[2]))
     ghost2.capture_backprops_hook = lambda *a, **k: None
     x = torch.randn(2, 4)
     ghost2(x)
-    assert {id(t) for t in ghost2.first_backward_inputs()} == {id(net[2].weight), id(net[2].bias)}
+    (leaf,) = ghost2.first_backward_inputs()
+    assert leaf.shape == (2, 3)  # the second Linear's output
     forget_forward(net)
     x.requires_grad_(True)
     ghost2(x)
