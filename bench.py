@@ -513,6 +513,9 @@ def main() -> None:
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default="c2")
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing")
+    ap.add_argument("--all-kernel-timers", action="store_true",
+                    help="HIP-event timers around every entry point of the library (kernel_ms_per_step lists them all); "
+                         "by default only the roofline kernel's entry point is timed")
     ap.add_argument(
         "--calibrate-copy",
         action="store_true",
@@ -548,7 +551,9 @@ def main() -> None:
         dst.copy_(src)
         del src, dst
     torch.cuda.synchronize()
-    with kernels.record_kernel_times() as times:
+    # HIP events around the dominant kernel's entry point only, unless every entry point is asked for
+    only = None if args.all_kernel_timers else {w["roofline"]["timer"]}
+    with kernels.record_kernel_times(only=only) as times:
         t0 = time.perf_counter()
         for _ in range(args.steps):
             step()

@@ -67,26 +67,30 @@ def _ws(nbytes: int, dev: torch.device) -> Tuple[Optional[torch.Tensor], int]:
 
 # ---- optional per-kernel timing (HIP events on the launch stream) -------------------
 _TIMING: Optional[Dict[str, List[Tuple[torch.cuda.Event, torch.cuda.Event]]]] = None
+_TIMING_ONLY: Optional[frozenset] = None
 
 
 @contextmanager
-def record_kernel_times():
-    """Collects (start, end) event pairs around every wrapper call made inside the block.
+def record_kernel_times(only=None):
+    """Collects (start, end) event pairs around every wrapper call made inside the block, or
+    around the calls of the wrappers named in ``only`` (two event records per call are not
+    free for a launch-bound model).
 
     Yields a dict ``name -> [(start, end), ...]``; after a device synchronize,
     ``start.elapsed_time(end)`` is the duration in ms of that call's kernels.
     """
-    global _TIMING
+    global _TIMING, _TIMING_ONLY
     prev, _TIMING = _TIMING, {}
+    prev_only, _TIMING_ONLY = _TIMING_ONLY, (None if only is None else frozenset(only))
     try:
         yield _TIMING
     finally:
-        _TIMING = prev
+        _TIMING, _TIMING_ONLY = prev, prev_only
 
 
 @contextmanager
 def _timed(name: str, dev: torch.device):
-    if _TIMING is None:
+    if _TIMING is None or (_TIMING_ONLY is not None and name not in _TIMING_ONLY):
         yield
         return
     with torch.cuda.device(dev):
