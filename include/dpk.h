@@ -72,9 +72,11 @@ int dpk_linear_gs(const void* b, const void* a, int in_dtype, void* gs, int gs_d
                   float* sumsq, int64_t n, int64_t T, int64_t out, int64_t in, float scale,
                   void* ws, size_t ws_bytes, dpk_stream_t stream);
 
-/* gs_bias[n,k] = scale * sum_t b[n,t,k]                   (linear.py:50) */
-int dpk_linear_bias_gs(const void* b, int in_dtype, void* gs_bias, int gs_dtype, int64_t n,
-                       int64_t T, int64_t out, float scale, dpk_stream_t stream);
+/* gs_bias[n,k] = scale * sum_t b[n,t,k]                   (linear.py:50)
+ * sumsq (nullable, float[n]) receives sum_k gs_bias[n,k]^2 of the values as stored, for
+ * the optimizer's norm pass (optimizers/optimizer.py:444-446). */
+int dpk_linear_bias_gs(const void* b, int in_dtype, void* gs_bias, int gs_dtype, float* sumsq,
+                       int64_t n, int64_t T, int64_t out, float scale, dpk_stream_t stream);
 
 /* ------------------------------------------------------------------------- *
  * Ghost-clipping per-sample norms of nn.Linear
@@ -127,9 +129,9 @@ int dpk_conv3d_gs(const void* x, const void* b, int in_dtype, void* gs, int gs_d
                   size_t ws_bytes, dpk_stream_t stream);
 
 /* gs_bias[n,o] = scale * sum_q b[n,o,q]                    (conv.py:117)
- * b: [n,O,q]. */
-int dpk_conv_bias_gs(const void* b, int in_dtype, void* gs_bias, int gs_dtype, int64_t n,
-                     int64_t O, int64_t q, float scale, dpk_stream_t stream);
+ * b: [n,O,q]. sumsq as for dpk_linear_bias_gs. */
+int dpk_conv_bias_gs(const void* b, int in_dtype, void* gs_bias, int gs_dtype, float* sumsq,
+                     int64_t n, int64_t O, int64_t q, float scale, dpk_stream_t stream);
 
 /* ------------------------------------------------------------------------- *
  * nn.Embedding

@@ -40,7 +40,7 @@ SIGNATURES = {
     "dpk_device_cus": (c_int, []),
     "dpk_linear_gs_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
     "dpk_linear_gs": (c_int, [_P, _P, c_int, _P, c_int, _P, _I, _I, _I, _I, c_float, _P, c_size_t, _P]),
-    "dpk_linear_bias_gs": (c_int, [_P, c_int, _P, c_int, _I, _I, _I, c_float, _P]),
+    "dpk_linear_bias_gs": (c_int, [_P, c_int, _P, c_int, _P, _I, _I, _I, c_float, _P]),
     "dpk_linear_ghost_norm_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
     "dpk_linear_ghost_norm": (c_int, [_P, _P, c_int, _P, _P, _I, _I, _I, _I, c_float, _P, c_size_t, _P]),
     "dpk_conv2d_gs_workspace_bytes": (c_size_t, [_I, _I, _I, _I, _I, _I]),
@@ -53,7 +53,7 @@ SIGNATURES = {
         c_int,
         [_P, _P, c_int, _P, c_int, _P, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, c_float, _P, c_size_t, _P],
     ),
-    "dpk_conv_bias_gs": (c_int, [_P, c_int, _P, c_int, _I, _I, _I, c_float, _P]),
+    "dpk_conv_bias_gs": (c_int, [_P, c_int, _P, c_int, _P, _I, _I, _I, c_float, _P]),
     "dpk_embedding_workspace_bytes": (c_size_t, [_I, _I, _I]),
     "dpk_embedding_unique_pairs": (c_int, [_P, _I, _I, _P, _P, _P, _P, c_size_t, _P]),
     "dpk_embedding_gs": (c_int, [_P, _P, c_int, _P, c_int, _I, _I, _I, _I, c_float, _P, c_size_t, _P]),

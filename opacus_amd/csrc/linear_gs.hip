@@ -405,6 +405,30 @@ void launch_colsum(const void* b, void* out, int64_t n, int64_t T, int64_t K, fl
                        K, scale, bps);
   }
 }
+// sumsq[r] = sum_k v[r,k]^2 of the values as stored: one wave per row.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void rowsq_kernel(const T* __restrict__ v, float* __restrict__ sumsq,
+                                                          int64_t rows, int64_t K) {
+  const int64_t w = (static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x) / DPK_WAVE;
+  const int lane = threadIdx.x & (DPK_WAVE - 1);
+  if (w >= rows) return;
+  const T* p = v + w * K;
+  float s = 0.f;
+  for (int64_t i = lane; i < K; i += DPK_WAVE) {
+    const float x = dpk_io<T>::load(p + i);
+    s = fmaf(x, x, s);
+  }
+  s = wave_sum(s);
+  if (lane == 0) sumsq[w] = s;
+}
+void launch_rowsq(const void* v, int dtype, float* sumsq, int64_t rows, int64_t K, hipStream_t s) {
+  const dim3 grid(static_cast<unsigned>(dpk_cdiv(rows, kWaves))), block(kThreads);
+  if (dtype == DPK_F32)
+    hipLaunchKernelGGL(rowsq_kernel<float>, grid, block, 0, s, static_cast<const float*>(v), sumsq, rows, K);
+  else
+    hipLaunchKernelGGL(rowsq_kernel<bf16_t>, grid, block, 0, s, static_cast<const bf16_t*>(v), sumsq, rows, K);
+}
+
 template <typename TIN, typename TOUT>
 void launch_rowsum(const void* b, void* out, int64_t rows, int64_t q, float scale, hipStream_t s) {
   hipLaunchKernelGGL((rowsum_kernel<TIN, TOUT>), dim3(static_cast<unsigned>(dpk_cdiv(rows, kWaves))),
@@ -413,7 +437,7 @@ void launch_rowsum(const void* b, void* out, int64_t rows, int64_t q, float scal
 }
 }  // namespace
 
-extern "C" int dpk_linear_bias_gs(const void* b, int in_dtype, void* gs_bias, int gs_dtype,
+extern "C" int dpk_linear_bias_gs(const void* b, int in_dtype, void* gs_bias, int gs_dtype, float* sumsq,
                                   int64_t n, int64_t T, int64_t out, float scale,
                                   dpk_stream_t stream) {
   const char* who = "dpk_linear_bias_gs";
@@ -431,12 +455,13 @@ extern "C" int dpk_linear_bias_gs(const void* b, int in_dtype, void* gs_bias, in
   else if (in_dtype == DPK_BF16 && gs_dtype == DPK_BF16) launch_colsum<bf16_t, bf16_t>(b, gs_bias, n, T, out, scale, s);
   else if (in_dtype == DPK_BF16 && gs_dtype == DPK_F32) launch_colsum<bf16_t, float>(b, gs_bias, n, T, out, scale, s);
   else launch_colsum<float, bf16_t>(b, gs_bias, n, T, out, scale, s);
+  if (sumsq) launch_rowsq(gs_bias, gs_dtype, sumsq, n, out, s);
   DPK_LAUNCH_CHECK(who);
   return DPK_OK;
 }
 
-extern "C" int dpk_conv_bias_gs(const void* b, int in_dtype, void* gs_bias, int gs_dtype, int64_t n,
-                                int64_t O, int64_t q, float scale, dpk_stream_t stream) {
+extern "C" int dpk_conv_bias_gs(const void* b, int in_dtype, void* gs_bias, int gs_dtype, float* sumsq,
+                                int64_t n, int64_t O, int64_t q, float scale, dpk_stream_t stream) {
   const char* who = "dpk_conv_bias_gs";
   DPK_REQUIRE(n >= 0 && O >= 1 && q >= 1, DPK_E_SHAPE, "%s: n=%lld O=%lld q=%lld", who,
               (long long)n, (long long)O, (long long)q);
@@ -452,6 +477,7 @@ extern "C" int dpk_conv_bias_gs(const void* b, int in_dtype, void* gs_bias, int 
   else if (in_dtype == DPK_BF16 && gs_dtype == DPK_BF16) launch_rowsum<bf16_t, bf16_t>(b, gs_bias, n * O, q, scale, s);
   else if (in_dtype == DPK_BF16 && gs_dtype == DPK_F32) launch_rowsum<bf16_t, float>(b, gs_bias, n * O, q, scale, s);
   else launch_rowsum<float, bf16_t>(b, gs_bias, n * O, q, scale, s);
+  if (sumsq) launch_rowsq(gs_bias, gs_dtype, sumsq, n, O, s);
   DPK_LAUNCH_CHECK(who);
   return DPK_OK;
 }

@@ -145,24 +145,34 @@ def linear_grad_sample(
     return gs, sumsq
 
 
+def _with_sumsq(gs: torch.Tensor, sumsq: torch.Tensor) -> torch.Tensor:
+    """Leaves the per-sample sum of squares on the tensor it describes, with the tensor's
+    version, so that the optimizer's norm pass can use it while nobody has written to ``gs``."""
+    gs._dpk_sumsq = sumsq
+    gs._dpk_sumsq_version = gs._version
+    return gs
+
+
 def linear_bias_grad_sample(
     backprops: torch.Tensor, scale: float = 1.0, out_dtype: Optional[torch.dtype] = None
 ) -> torch.Tensor:
-    """``gs[n,k] = scale * sum over middle dims of b[n,*,k]``."""
+    """``gs[n,k] = scale * sum over middle dims of b[n,*,k]``; its per-sample sum of squares
+    rides on the result for the optimizer."""
     dev = _need_gpu(backprops)
     n, out_f = backprops.shape[0], backprops.shape[-1]
     gs = torch.empty((n, out_f), dtype=out_dtype or backprops.dtype, device=dev)
     if n == 0:
         return gs
+    sumsq = torch.empty((n,), dtype=torch.float32, device=dev)
     b = _dense(backprops).reshape(n, -1, out_f)
     with _timed("linear_bias_gs", dev):
         check(
             "dpk_linear_bias_gs",
             lib().dpk_linear_bias_gs(
-                _ptr(b), _code(b), _ptr(gs), _code(gs), n, b.shape[1], out_f, float(scale), _stream(dev)
+                _ptr(b), _code(b), _ptr(gs), _code(gs), _ptr(sumsq), n, b.shape[1], out_f, float(scale), _stream(dev)
             ),
         )
-    return gs
+    return _with_sumsq(gs, sumsq)
 
 
 def linear_ghost_norm(
@@ -296,21 +306,23 @@ def conv3d_grad_sample(
 
 
 def conv_bias_grad_sample(backprops: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
-    """``gs[n,o] = scale * sum over the spatial dims of b[n,o,...]``."""
+    """``gs[n,o] = scale * sum over the spatial dims of b[n,o,...]``; its per-sample sum of
+    squares rides on the result for the optimizer."""
     dev = _need_gpu(backprops)
     n, O = backprops.shape[0], backprops.shape[1]
     gs = torch.empty((n, O), dtype=backprops.dtype, device=dev)
     if n == 0:
         return gs
+    sumsq = torch.empty((n,), dtype=torch.float32, device=dev)
     b = _dense(backprops).reshape(n, O, -1)
     with _timed("conv_bias_gs", dev):
         check(
             "dpk_conv_bias_gs",
             lib().dpk_conv_bias_gs(
-                _ptr(b), _code(b), _ptr(gs), _code(gs), n, O, b.shape[2], float(scale), _stream(dev)
+                _ptr(b), _code(b), _ptr(gs), _code(gs), _ptr(sumsq), n, O, b.shape[2], float(scale), _stream(dev)
             ),
         )
-    return gs
+    return _with_sumsq(gs, sumsq)
 
 
 # ---- nn.Embedding -------------------------------------------------------------------

@@ -723,3 +723,20 @@ def test_tied_embedding_cross_term(K, dtype, n, T, T2, D, V):
     got32 = K.tied_embedding_cross_term(dev(ids), dev(e.float()), dev(a), dev(g))
     assert_rel(got32, want, 1e-4, "fp32 embedding backprops")
     assert K.tied_embedding_cross_term(dev(ids[:0]), dev(e[:0]), dev(a[:0]), dev(g[:0])).shape == (0,)
+
+
+def test_bias_grad_samples_carry_their_sumsq(K):
+    """The bias entry points also return the per-sample sum of squares of what they wrote,
+    so the optimizer's norm pass has nothing left to read for these tensors."""
+    torch.manual_seed(9)
+    b = torch.randn(7, 5, 33)
+    gs = K.linear_bias_grad_sample(dev(b), scale=3.0)
+    assert_rel(gs._dpk_sumsq, gs.double().pow(2).sum(1), 1e-6, "linear bias sumsq")
+    assert gs._dpk_sumsq_version == gs._version
+    g16 = K.linear_bias_grad_sample(dev(b.bfloat16()))
+    assert_rel(g16._dpk_sumsq, g16.double().pow(2).sum(1), 1e-6, "linear bias sumsq, bf16 as stored")
+    c = torch.randn(6, 9, 4, 5)
+    gc = K.conv_bias_grad_sample(dev(c), scale=0.5)
+    assert_rel(gc._dpk_sumsq, gc.double().pow(2).sum(1), 1e-6, "conv bias sumsq")
+    gc.mul_(2.0)
+    assert gc._dpk_sumsq_version != gc._version  # a write invalidates it
