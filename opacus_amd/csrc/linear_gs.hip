@@ -10,6 +10,7 @@
 // tensor disappears.
 #include "dpk_common.h"
 #include "mfma_bf16.h"
+#include "mfma_bf16_tr.h"
 #include "mfma_f32.h"
 
 #include <type_traits>
@@ -185,6 +186,92 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
   }
 }
 
+// The same contraction with the transposition left to the LDS read (mfma_bf16_tr.h): tiles
+// travel global -> LDS as they lie in memory, four k tiles deep. The product is formed
+// transposed, rows = input features, columns = output features, because a lane of the
+// accumulator layout owns four consecutive ROWS: that way they are four consecutive elements
+// of a row of gs. Results are gathered into whole rows of the output tile in
+// the (by then idle) stage memory and leave as 16-byte non-temporal stores.
+// M % 8 == 0, N % 8 == 0, T >= 32, 16-byte aligned b and a, 128 x 128 tiles.
+// Row pitch of the output tile in the stage memory, in bytes. bf16: 66 dwords, so the 32
+// rows a half-wave writes 8 bytes each into cover the banks once. fp32: 132 dwords, the same
+// for 16-byte writes in two passes; half the tile's rows at a time fit the stage memory.
+template <typename TOUT> struct TrOut;
+template <> struct TrOut<bf16_t> { static constexpr int kPitch = 128 * 2 + 8, kRows = 128; };
+template <> struct TrOut<float> { static constexpr int kPitch = 128 * 4 + 16, kRows = 64; };
+
+template <typename TOUT>
+__global__ __launch_bounds__(kThreads) void linear_tr_bf16_kernel(
+    const bf16_t* __restrict__ b, const bf16_t* __restrict__ a, TOUT* __restrict__ gs,
+    float* __restrict__ partials, int64_t T, int64_t M, int64_t N, float scale, int64_t tiles_m,
+    int64_t tiles_n) {
+  __shared__ mb16t::Smem sm;
+  __shared__ float red[kWaves];
+  constexpr int kPitch = TrOut<TOUT>::kPitch, kRows = TrOut<TOUT>::kRows;
+  static_assert(kRows * kPitch <= sizeof(mb16t::Smem), "output rows must fit the stage memory");
+  const int64_t per_sample = tiles_m * tiles_n;
+  const int64_t sample = blockIdx.x / per_sample;
+  const int64_t rem = blockIdx.x % per_sample;
+  const int64_t m0 = (rem / tiles_n) * 128, n0 = (rem % tiles_n) * 128;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wj0 = (wave >> 1) * 64, wi0 = (wave & 1) * 64;  // this wave's corner: input, output features
+  mb16t::Tile tile;
+  tile.clear();
+  mb16t::mainloop(tile, sm, a + sample * T * N, N, n0, b + sample * T * M, M, m0, T, wj0, wi0);
+  TOUT* out = gs + sample * M * N;
+  const int kk = lane >> 5, l32 = lane & 31;
+  float ss = 0.f;
+  unsigned char* stage_out = &sm.stage[0][0];
+  // 128 / kRows passes; in a pass the waves that own rows [pass * kRows, + kRows) of the tile
+  // put them into the stage memory, then all threads send whole rows on their way
+#pragma unroll
+  for (int pass = 0; pass < 128 / kRows; ++pass) {
+    if (pass > 0) __syncthreads();
+    if (kRows == 128 || wi0 == pass * kRows) {
+#pragma unroll
+      for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+        for (int it = 0; it < 2; ++it)
+#pragma unroll
+          for (int vg = 0; vg < 4; ++vg) {
+            const int il = wi0 + it * 32 + l32, jl = wj0 + jt * 32 + vg * 8 + kk * 4;
+            float4 x;
+            x.x = tile.acc[jt][it][vg * 4 + 0] * scale;
+            x.y = tile.acc[jt][it][vg * 4 + 1] * scale;
+            x.z = tile.acc[jt][it][vg * 4 + 2] * scale;
+            x.w = tile.acc[jt][it][vg * 4 + 3] * scale;
+            // N % 4 == 0: the four columns are inside or outside together
+            if (m0 + il < M && n0 + jl < N) ss = fmaf(x.x, x.x, fmaf(x.y, x.y, fmaf(x.z, x.z, fmaf(x.w, x.w, ss))));
+            dpk_io<TOUT>::store4(reinterpret_cast<TOUT*>(stage_out + (il - pass * kRows) * kPitch) + jl, x);
+          }
+    }
+    __syncthreads();
+    constexpr int kChunksPerRow = 128 * sizeof(TOUT) / 16, kPerChunk = 16 / sizeof(TOUT);
+#pragma unroll
+    for (int r = 0; r < kRows * kChunksPerRow / kThreads; ++r) {
+      const int idx = threadIdx.x + r * kThreads;
+      const int il = idx / kChunksPerRow, c = idx % kChunksPerRow;
+      const int64_t i = m0 + pass * kRows + il, j = n0 + c * kPerChunk;
+      if (i < M && j < N) {  // N % 8 == 0: whole chunks
+        const uint2* src = reinterpret_cast<const uint2*>(stage_out + il * kPitch + c * 16);
+        const uint2 lo = src[0], hi = src[1];
+        typedef uint32_t vu4 __attribute__((ext_vector_type(4)));
+        vu4 w;
+        w.x = lo.x;
+        w.y = lo.y;
+        w.z = hi.x;
+        w.w = hi.y;
+        __builtin_nontemporal_store(w, reinterpret_cast<vu4*>(out + i * N + j));
+      }
+    }
+  }
+  if (partials) {
+    const float s = block_sum<kWaves>(ss, red);
+    if (threadIdx.x == 0) partials[blockIdx.x] = s;
+  }
+}
+
 // ---- bias / row sums -----------------------------------------------------------
 // out[n,k] = scale * sum_t b[n,t,k]; threads along k, RS row groups along t.
 template <typename TIN, typename TOUT, int RS>
@@ -293,7 +380,14 @@ void launch_linear(const Plan& p, bool vec, const void* b, const void* a, void* 
 #define DPK_BF16(BMN, V)                                                                              \
   hipLaunchKernelGGL((linear_mfma_bf16_kernel<BMN, BMN, TOUT, V>), grid, block, 0, s, bp, ap, gp, partials, \
                      T, M, N, scale, p.tiles_m, p.tiles_n)
-    if (p.bm == 128) {
+    // the transposing-read kernel: whole 16-byte chunks, at least one whole k tile, and
+    // per-lane byte offsets inside a k tile that fit 32 bits
+    const bool tr = vec8 && p.bm == 128 && T >= mb16t::BK && M < (1LL << 24) && N < (1LL << 24) &&
+                    dpk_aligned(gs, 16);
+    if (tr) {
+      hipLaunchKernelGGL((linear_tr_bf16_kernel<TOUT>), grid, block, 0, s, bp, ap, gp, partials, T, M, N, scale,
+                         p.tiles_m, p.tiles_n);
+    } else if (p.bm == 128) {
       if (vec8) DPK_BF16(128, true);
       else DPK_BF16(128, false);
     } else {

@@ -80,6 +80,11 @@ def test_linear_grad_sample_f32(K, n, mid, fin, fout, scale):
         (3, (65,), 64, 72),  # 64 tiles, K = one k tile + 1
         (1, (7, 19), 132, 260),  # two middle dimensions, sizes that are multiples of 4 only
         (2, (128,), 1024, 8),  # a narrow output
+        (2, (32,), 128, 128),  # exactly one k tile of the transposing-read kernel, one block tile
+        (1, (33,), 72, 136),  # its last k tile repeats 31 rows of the first
+        (2, (96,), 520, 264),  # three whole k tiles, ragged block tiles in both directions
+        (1, (1000,), 128, 256),  # a long contraction: the ring wraps many times
+        (3, (4, 16), 256, 128),  # 64 positions in two middle dimensions
     ],
 )
 def test_linear_grad_sample_bf16(K, n, mid, fin, fout):
