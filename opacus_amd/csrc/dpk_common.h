@@ -47,12 +47,19 @@ typedef uint16_t bf16_t;  // raw bfloat16 bits
 __device__ __forceinline__ float bf16_to_f32(bf16_t v) {
   return __uint_as_float(static_cast<uint32_t>(v) << 16);
 }
-// Round to nearest even, NaN kept quiet: what torch's float -> bfloat16 cast does.
+// Round to nearest even, NaN kept quiet: what torch's float -> bfloat16 cast does. gfx950
+// converts in hardware (v_cvt_pk_bf16_f32, two values per instruction).
 __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<bf16_t>((u >> 16) | 0x40u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return static_cast<bf16_t>(u >> 16);
+  return __builtin_bit_cast(bf16_t, static_cast<__bf16>(f));
+}
+// lo in bits 0..15, hi in bits 16..31
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2(float lo, float hi) {
+  typedef float dpk_f2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 dpk_bf2 __attribute__((ext_vector_type(2)));
+  dpk_f2 v;
+  v.x = lo;
+  v.y = hi;
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, dpk_bf2));
 }
 
 typedef float dpk_vf4 __attribute__((ext_vector_type(4)));
@@ -109,17 +116,26 @@ template <> struct dpk_io<bf16_t> {
   }
   static __device__ __forceinline__ void store4(bf16_t* p, float4 v) {
     uint2 r;
-    r.x = static_cast<uint32_t>(f32_to_bf16(v.x)) | (static_cast<uint32_t>(f32_to_bf16(v.y)) << 16);
-    r.y = static_cast<uint32_t>(f32_to_bf16(v.z)) | (static_cast<uint32_t>(f32_to_bf16(v.w)) << 16);
+    r.x = f32x2_to_bf16x2(v.x, v.y);
+    r.y = f32x2_to_bf16x2(v.z, v.w);
     *reinterpret_cast<uint2*>(p) = r;
   }
   static __device__ __forceinline__ void store4_nt(bf16_t* p, float4 v) {
     dpk_vu2 r;
-    r.x = static_cast<uint32_t>(f32_to_bf16(v.x)) | (static_cast<uint32_t>(f32_to_bf16(v.y)) << 16);
-    r.y = static_cast<uint32_t>(f32_to_bf16(v.z)) | (static_cast<uint32_t>(f32_to_bf16(v.w)) << 16);
+    r.x = f32x2_to_bf16x2(v.x, v.y);
+    r.y = f32x2_to_bf16x2(v.z, v.w);
     __builtin_nontemporal_store(r, reinterpret_cast<dpk_vu2*>(p));
   }
 };
+
+// Workgroups are handed to the 8 XCDs round-robin by hardware id. Renumbering
+// them so that each XCD works through one contiguous range of work units
+// keeps what neighbouring units share (the rows of a sample) in that XCD's L2.
+__device__ __forceinline__ uint32_t xcd_contiguous_id(uint32_t bid, uint32_t nb) {
+  const uint32_t x = bid & 7u, idx = bid >> 3;
+  const uint32_t base = nb >> 3, rem = nb & 7u;
+  return x * base + (x < rem ? x : rem) + idx;
+}
 
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

@@ -107,15 +107,6 @@ __global__ __launch_bounds__(kThreads) void ghost_norm_bf16_kernel(
   contract_and_store(tg, ta, pw != nullptr, ti == tj ? 1.f : 2.f, pw, pb, red);
 }
 
-// Workgroups are handed to the 8 XCDs round-robin by hardware id. Renumbering
-// them so that each XCD works through one contiguous range of (sample, tile pair)
-// keeps the rows of a sample in that XCD's L2 while its tile pairs are computed.
-__device__ __forceinline__ uint32_t xcd_contiguous_id(uint32_t bid, uint32_t nb) {
-  const uint32_t x = bid & 7u, idx = bid >> 3;
-  const uint32_t base = nb >> 3, rem = nb & 7u;
-  return x * base + (x < rem ? x : rem) + idx;
-}
-
 // Fast path: operand tiles go global -> LDS directly through a ring of stages
 // (mfma_bf16_dlds.h). Needs Dout % 64 == Din % 64 == 0 and 16-byte aligned rows.
 // The block tile is BM x BN with BM = R * BN: row blocks I, column blocks J, and

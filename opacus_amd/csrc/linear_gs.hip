@@ -13,6 +13,7 @@
 #include "mfma_bf16_tr.h"
 #include "mfma_f32.h"
 
+#include <cstdlib>
 #include <type_traits>
 
 namespace {
@@ -192,65 +193,71 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
 // accumulator layout owns four consecutive ROWS: that way they are four consecutive elements
 // of a row of gs. Results are gathered into whole rows of the output tile in
 // the (by then idle) stage memory and leave as 16-byte non-temporal stores.
-// M % 8 == 0, N % 8 == 0, T >= 32, 16-byte aligned b and a, 128 x 128 tiles.
-// Row pitch of the output tile in the stage memory, in bytes. bf16: 66 dwords, so the 32
-// rows a half-wave writes 8 bytes each into cover the banks once. fp32: 132 dwords, the same
-// for 16-byte writes in two passes; half the tile's rows at a time fit the stage memory.
+// M % 8 == 0, N % 8 == 0, T >= 32, 16-byte aligned b, a and gs.
+// The output tile passes through the stage memory kRows rows at a time; a row is padded so
+// that the 32 rows a half-wave writes into (8 bytes each for bf16: pitch = 2 mod 64 dwords;
+// 16 bytes in two passes for fp32: pitch = 4 mod 64 dwords) cover the banks once.
 template <typename TOUT> struct TrOut;
-template <> struct TrOut<bf16_t> { static constexpr int kPitch = 128 * 2 + 8, kRows = 128; };
-template <> struct TrOut<float> { static constexpr int kPitch = 128 * 4 + 16, kRows = 64; };
+template <> struct TrOut<bf16_t> { static constexpr int kPad = 8, kRows = 128; };
+template <> struct TrOut<float> { static constexpr int kPad = 16, kRows = 64; };
 
-template <typename TOUT>
-__global__ __launch_bounds__(kThreads) void linear_tr_bf16_kernel(
+template <class C, typename TOUT>
+__global__ __launch_bounds__(C::kThreads) void linear_tr_bf16_kernel(
     const bf16_t* __restrict__ b, const bf16_t* __restrict__ a, TOUT* __restrict__ gs,
     float* __restrict__ partials, int64_t T, int64_t M, int64_t N, float scale, int64_t tiles_m,
     int64_t tiles_n) {
-  __shared__ mb16t::Smem sm;
-  __shared__ float red[kWaves];
-  constexpr int kPitch = TrOut<TOUT>::kPitch, kRows = TrOut<TOUT>::kRows;
-  static_assert(kRows * kPitch <= sizeof(mb16t::Smem), "output rows must fit the stage memory");
+  __shared__ mb16t::Smem<C> sm;
+  __shared__ float red[C::kWaves];
+  // rows of the product = input features (P = a), columns = output features (Q = b)
+  constexpr int BJ = C::BP, BI = C::BQ;
+  constexpr int kPitch = BJ * sizeof(TOUT) + TrOut<TOUT>::kPad, kRows = TrOut<TOUT>::kRows;
+  static_assert(kRows * kPitch <= sizeof(mb16t::Smem<C>), "output rows must fit the stage memory");
+  static_assert(BI % kRows == 0 && kRows % 32 == 0, "passes of whole MFMA tiles");
+  // neighbouring tiles of a sample share operand panels: keep them on one XCD
+  const uint32_t bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
   const int64_t per_sample = tiles_m * tiles_n;
-  const int64_t sample = blockIdx.x / per_sample;
-  const int64_t rem = blockIdx.x % per_sample;
-  const int64_t m0 = (rem / tiles_n) * 128, n0 = (rem % tiles_n) * 128;
+  const int64_t sample = bid / per_sample;
+  const int64_t rem = bid % per_sample;
+  const int64_t m0 = (rem / tiles_n) * BI, n0 = (rem % tiles_n) * BJ;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int wj0 = (wave >> 1) * 64, wi0 = (wave & 1) * 64;  // this wave's corner: input, output features
-  mb16t::Tile tile;
+  const int wj0 = (wave / C::WQ) * (32 * C::TP), wi0 = (wave % C::WQ) * (32 * C::TQ);  // this wave's corner
+  mb16t::Tile<C> tile;
   tile.clear();
-  mb16t::mainloop(tile, sm, a + sample * T * N, N, n0, b + sample * T * M, M, m0, T, wj0, wi0);
+  mb16t::mainloop<C>(tile, sm, a + sample * T * N, N, n0, b + sample * T * M, M, m0, T, wj0, wi0);
   TOUT* out = gs + sample * M * N;
   const int kk = lane >> 5, l32 = lane & 31;
   float ss = 0.f;
   unsigned char* stage_out = &sm.stage[0][0];
-  // 128 / kRows passes; in a pass the waves that own rows [pass * kRows, + kRows) of the tile
-  // put them into the stage memory, then all threads send whole rows on their way
+  // In a pass the waves that own rows [pass * kRows, + kRows) of the tile put them into the
+  // stage memory, then all threads send whole rows on their way.
 #pragma unroll
-  for (int pass = 0; pass < 128 / kRows; ++pass) {
+  for (int pass = 0; pass < BI / kRows; ++pass) {
     if (pass > 0) __syncthreads();
-    if (kRows == 128 || wi0 == pass * kRows) {
 #pragma unroll
-      for (int jt = 0; jt < 2; ++jt)
+    for (int it = 0; it < C::TQ; ++it) {
+      if ((wi0 + it * 32) / kRows != pass) continue;  // wave-uniform
 #pragma unroll
-        for (int it = 0; it < 2; ++it)
+      for (int jt = 0; jt < C::TP; ++jt)
 #pragma unroll
-          for (int vg = 0; vg < 4; ++vg) {
-            const int il = wi0 + it * 32 + l32, jl = wj0 + jt * 32 + vg * 8 + kk * 4;
-            float4 x;
-            x.x = tile.acc[jt][it][vg * 4 + 0] * scale;
-            x.y = tile.acc[jt][it][vg * 4 + 1] * scale;
-            x.z = tile.acc[jt][it][vg * 4 + 2] * scale;
-            x.w = tile.acc[jt][it][vg * 4 + 3] * scale;
-            // N % 4 == 0: the four columns are inside or outside together
-            if (m0 + il < M && n0 + jl < N) ss = fmaf(x.x, x.x, fmaf(x.y, x.y, fmaf(x.z, x.z, fmaf(x.w, x.w, ss))));
-            dpk_io<TOUT>::store4(reinterpret_cast<TOUT*>(stage_out + (il - pass * kRows) * kPitch) + jl, x);
-          }
+        for (int vg = 0; vg < 4; ++vg) {
+          const int il = wi0 + it * 32 + l32, jl = wj0 + jt * 32 + vg * 8 + kk * 4;
+          float4 x;
+          x.x = tile.acc[jt][it][vg * 4 + 0] * scale;
+          x.y = tile.acc[jt][it][vg * 4 + 1] * scale;
+          x.z = tile.acc[jt][it][vg * 4 + 2] * scale;
+          x.w = tile.acc[jt][it][vg * 4 + 3] * scale;
+          // N % 4 == 0: the four columns are inside or outside together
+          if (m0 + il < M && n0 + jl < N) ss = fmaf(x.x, x.x, fmaf(x.y, x.y, fmaf(x.z, x.z, fmaf(x.w, x.w, ss))));
+          dpk_io<TOUT>::store4(reinterpret_cast<TOUT*>(stage_out + (il - pass * kRows) * kPitch) + jl, x);
+        }
     }
     __syncthreads();
-    constexpr int kChunksPerRow = 128 * sizeof(TOUT) / 16, kPerChunk = 16 / sizeof(TOUT);
+    constexpr int kChunksPerRow = BJ * sizeof(TOUT) / 16, kPerChunk = 16 / sizeof(TOUT);
+    static_assert(kRows * kChunksPerRow % C::kThreads == 0, "whole trips of the block over the rows");
 #pragma unroll
-    for (int r = 0; r < kRows * kChunksPerRow / kThreads; ++r) {
-      const int idx = threadIdx.x + r * kThreads;
+    for (int r = 0; r < kRows * kChunksPerRow / C::kThreads; ++r) {
+      const int idx = threadIdx.x + r * C::kThreads;
       const int il = idx / kChunksPerRow, c = idx % kChunksPerRow;
       const int64_t i = m0 + pass * kRows + il, j = n0 + c * kPerChunk;
       if (i < M && j < N) {  // N % 8 == 0: whole chunks
@@ -267,10 +274,15 @@ __global__ __launch_bounds__(kThreads) void linear_tr_bf16_kernel(
     }
   }
   if (partials) {
-    const float s = block_sum<kWaves>(ss, red);
-    if (threadIdx.x == 0) partials[blockIdx.x] = s;
+    const float s = block_sum<C::kWaves>(ss, red);
+    if (threadIdx.x == 0) partials[bid] = s;
   }
 }
+
+using TrSmall = mb16t::Config<2, 2, 2, 2, 4>;  // 128 x 128, 4 waves, 64 KB: two blocks per CU
+using TrLarge = mb16t::Config<4, 2, 2, 4, 4>;  // 256 x 256, 8 waves, 128 KB: one block per CU
+// time of a 256 x 256 block relative to four 128 x 128 blocks run two at a time
+constexpr double kTrLargeGain = 0.9;
 
 // ---- bias / row sums -----------------------------------------------------------
 // out[n,k] = scale * sum_t b[n,t,k]; threads along k, RS row groups along t.
@@ -319,11 +331,13 @@ struct Plan {
   int cx_log2;
   int rows_pb;
   int bm;
+  int tr;  // 0, or the tile edge of the transposing-read bf16 kernel (it replaces bm)
   int64_t tiles_m, tiles_n;
 };
 
 Plan make_plan(int64_t T, int64_t M, int64_t N, bool vec) {
   Plan p;
+  p.tr = 0;
   p.outer = (T == 1);
   if (p.outer) {
     const int64_t cols = dpk_cdiv(N, vec ? 4 : 1);
@@ -342,6 +356,29 @@ Plan make_plan(int64_t T, int64_t M, int64_t N, bool vec) {
     p.tiles_n = dpk_cdiv(N, p.bm);
   }
   return p;
+}
+
+// Whether the transposing-read bf16 kernel takes the shape, and with which tile: whole
+// 16-byte chunks, at least one whole k tile, per-lane byte offsets inside a k tile that fit
+// 32 bits. The 256-tile blocks move half the operand bytes per product and run one to a
+// CU; the 128-tile blocks two to a CU. The cheaper of the two by rounds of resident blocks
+// times work per block wins. DPK_LINEAR_BF16_TILE=128|256 in the environment overrides the
+// choice (for tests that want both kernels on small shapes).
+void plan_tr(Plan& p, const void* b, const void* a, const void* gs, int64_t n, int64_t T, int64_t M, int64_t N,
+             int cus) {
+  if (cus <= 0) cus = 256;
+  if (p.outer || p.bm != 128 || T < mb16t::BK || M % 8 != 0 || N % 8 != 0 || M >= (1LL << 24) || N >= (1LL << 24) ||
+      !dpk_aligned(b, 16) || !dpk_aligned(a, 16) || !dpk_aligned(gs, 16))
+    return;
+  const char* force = getenv("DPK_LINEAR_BF16_TILE");
+  const int64_t small = n * dpk_cdiv(M, 128) * dpk_cdiv(N, 128), large = n * dpk_cdiv(M, 256) * dpk_cdiv(N, 256);
+  const double cost_small = static_cast<double>(dpk_cdiv(small, 2 * cus)) * 2.0;
+  const double cost_large = static_cast<double>(dpk_cdiv(large, cus)) * 4.0 * kTrLargeGain;
+  p.tr = (M >= 256 && N >= 256 && cost_large < cost_small) ? 256 : 128;
+  if (force) p.tr = atoi(force) == 256 ? 256 : 128;
+  p.bm = p.tr;
+  p.tiles_m = dpk_cdiv(M, p.tr);
+  p.tiles_n = dpk_cdiv(N, p.tr);
 }
 
 template <typename TIN, typename TOUT>
@@ -380,13 +417,12 @@ void launch_linear(const Plan& p, bool vec, const void* b, const void* a, void* 
 #define DPK_BF16(BMN, V)                                                                              \
   hipLaunchKernelGGL((linear_mfma_bf16_kernel<BMN, BMN, TOUT, V>), grid, block, 0, s, bp, ap, gp, partials, \
                      T, M, N, scale, p.tiles_m, p.tiles_n)
-    // the transposing-read kernel: whole 16-byte chunks, at least one whole k tile, and
-    // per-lane byte offsets inside a k tile that fit 32 bits
-    const bool tr = vec8 && p.bm == 128 && T >= mb16t::BK && M < (1LL << 24) && N < (1LL << 24) &&
-                    dpk_aligned(gs, 16);
-    if (tr) {
-      hipLaunchKernelGGL((linear_tr_bf16_kernel<TOUT>), grid, block, 0, s, bp, ap, gp, partials, T, M, N, scale,
-                         p.tiles_m, p.tiles_n);
+    if (p.tr == 256) {
+      hipLaunchKernelGGL((linear_tr_bf16_kernel<TrLarge, TOUT>), grid, dim3(TrLarge::kThreads), 0, s, bp, ap, gp,
+                         partials, T, M, N, scale, p.tiles_m, p.tiles_n);
+    } else if (p.tr == 128) {
+      hipLaunchKernelGGL((linear_tr_bf16_kernel<TrSmall, TOUT>), grid, dim3(TrSmall::kThreads), 0, s, bp, ap, gp,
+                         partials, T, M, N, scale, p.tiles_m, p.tiles_n);
     } else if (p.bm == 128) {
       if (vec8) DPK_BF16(128, true);
       else DPK_BF16(128, false);
@@ -442,7 +478,8 @@ extern "C" int dpk_linear_gs(const void* b, const void* a, int in_dtype, void* g
                   dpk_aligned(gs, dpk_elsize(gs_dtype)),
               DPK_E_ALIGN, "%s: misaligned tensor", who);
   const bool vec = linear_vec(b, a, gs, in_dtype, gs_dtype, out, in);
-  const Plan p = make_plan(T, out, in, vec);
+  Plan p = make_plan(T, out, in, vec);
+  if (in_dtype == DPK_BF16) plan_tr(p, b, a, gs, n, T, out, in, dpk_device_cus());
   const int64_t blocks = n * p.tiles_m * p.tiles_n;
   DPK_REQUIRE(blocks <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: %lld blocks exceed the grid limit", who,
               (long long)blocks);

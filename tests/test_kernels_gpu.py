@@ -87,7 +87,12 @@ def test_linear_grad_sample_f32(K, n, mid, fin, fout, scale):
         (3, (4, 16), 256, 128),  # 64 positions in two middle dimensions
     ],
 )
-def test_linear_grad_sample_bf16(K, n, mid, fin, fout):
+@pytest.mark.parametrize("tile", [None, "128", "256"])
+def test_linear_grad_sample_bf16(K, n, mid, fin, fout, tile, monkeypatch):
+    """`tile` forces the 128 x 128 or the 256 x 256 variant of the transposing-read kernel where
+    the shape qualifies for it (None: the library's own choice)."""
+    if tile is not None:
+        monkeypatch.setenv("DPK_LINEAR_BF16_TILE", tile)
     torch.manual_seed(7)
     a = torch.randn(n, *mid, fin).bfloat16()
     b = torch.randn(n, *mid, fout).bfloat16()
