@@ -39,6 +39,8 @@ typedef short shortx4 __attribute__((ext_vector_type(4)));
 typedef short shortx8 __attribute__((ext_vector_type(8)));
 typedef __attribute__((address_space(3))) shortx4* lds_shortx4_ptr;
 
+// s_waitcnt lgkmcnt(0) with the other counters left alone (gfx9 encoding: vmcnt 63, expcnt 7)
+constexpr int kWaitLgkm0 = 0xC07F;
 constexpr int BK = 32;                      // rows (k) of a stage
 constexpr int SUB = 128;                    // columns of a sub-tile
 constexpr int ROW_BYTES = SUB * 2;          // 256
@@ -97,12 +99,31 @@ __device__ __forceinline__ shortx4 read_tr(const unsigned char* p) {
   return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4_ptr)(p));
 }
 
-// Operand of one MFMA: k = 16 s + (lane / 32) * 8 .. + 7 of column (lane % 32) of the piece.
-__device__ __forceinline__ bf16x8 read_operand(const unsigned char* opnd, uint32_t frag, int s) {
-  const shortx4 lo = read_tr(opnd + frag + (16 * s) * ROW_BYTES);
-  const shortx4 hi = read_tr(opnd + frag + (16 * s + 4) * ROW_BYTES);
-  return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-}
+// The operand registers of one k tile for one wave, as the halves that one transposing read
+// delivers: half h of operand (s, i) is k = 16 s + (lane / 32) * 8 + 4 h .. + 3 of column
+// (lane % 32) of the i-th 32-column piece.
+template <class C>
+struct Frags {
+  static constexpr int KS = BK / 16;
+  static constexpr int kPerStep = 2 * (C::TP + C::TQ);  // reads of one k16 step
+  static constexpr int kReads = KS * kPerStep;
+  shortx4 p[KS][C::TP][2], q[KS][C::TQ][2];
+
+  // the r-th read of the tile, r < kReads: k16 steps in order, P's pieces before Q's
+  __device__ __forceinline__ void read(int r, const unsigned char* Ps, const unsigned char* Qs,
+                                       const uint32_t (&fp)[C::TP], const uint32_t (&fq)[C::TQ]) {
+    const int s = r / kPerStep, x = (r % kPerStep) / 2, h = r % 2;
+    const int row_bytes = (16 * s + 4 * h) * ROW_BYTES;
+    if (x < C::TP) p[s][x][h] = read_tr(Ps + fp[x] + row_bytes);
+    else q[s][x - C::TP][h] = read_tr(Qs + fq[x - C::TP] + row_bytes);
+  }
+  __device__ __forceinline__ bf16x8 operand_p(int s, int i) const {
+    return __builtin_bit_cast(bf16x8, __builtin_shufflevector(p[s][i][0], p[s][i][1], 0, 1, 2, 3, 4, 5, 6, 7));
+  }
+  __device__ __forceinline__ bf16x8 operand_q(int s, int j) const {
+    return __builtin_bit_cast(bf16x8, __builtin_shufflevector(q[s][j][0], q[s][j][1], 0, 1, 2, 3, 4, 5, 6, 7));
+  }
+};
 
 // The accumulator piece of one wave: acc[i][j] covers rows (columns of P) wp0 + 32 i ..,
 // columns (columns of Q) wq0 + 32 j ..; element v of lane l is row
@@ -120,38 +141,36 @@ struct Tile {
         for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
   }
 
+  // The MFMAs of the tile in `cur`, with the LDS reads of the next tile (into `nxt`) and
+  // the global -> LDS loads of a later one (issue(q), q < kLoads) dealt out evenly between
+  // them: a wave issues in order, so reads queued in one burst would hold its MFMAs back for
+  // as long as the LDS takes to accept them.
   template <class IssueFn>
-  __device__ __forceinline__ void mma(const unsigned char* Ps, const unsigned char* Qs, const uint32_t (&fp)[C::TP],
+  __device__ __forceinline__ void mma(const Frags<C>& cur, Frags<C>& nxt, const unsigned char* Ps,
+                                      const unsigned char* Qs, const uint32_t (&fp)[C::TP],
                                       const uint32_t (&fq)[C::TQ], IssueFn issue) {
-    constexpr int KS = BK / 16;
-    bf16x8 pv[KS][C::TP], qv[KS][C::TQ];
+    constexpr int KS = Frags<C>::KS, M = KS * C::TP * C::TQ, R = Frags<C>::kReads, L = C::kLoads;
 #pragma unroll
-    for (int s = 0; s < KS; ++s) {
+    for (int m = 0; m < M; ++m) {
+      const int s = m / (C::TP * C::TQ), i = (m / C::TQ) % C::TP, j = m % C::TQ;
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur.operand_p(s, i), cur.operand_q(s, j), acc[i][j], 0, 0, 0);
 #pragma unroll
-      for (int i = 0; i < C::TP; ++i) pv[s][i] = read_operand(Ps, fp[i], s);
+      for (int r = m * R / M; r < (m + 1) * R / M; ++r) nxt.read(r, Ps, Qs, fp, fq);
 #pragma unroll
-      for (int j = 0; j < C::TQ; ++j) qv[s][j] = read_operand(Qs, fq[j], s);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    constexpr int PER_STEP = (C::kLoads + KS - 1) / KS;
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-#pragma unroll
-      for (int i = 0; i < C::TP; ++i)
-#pragma unroll
-        for (int j = 0; j < C::TQ; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pv[s][i], qv[s][j], acc[i][j], 0, 0, 0);
-#pragma unroll
-      for (int q = s * PER_STEP; q < (s + 1) * PER_STEP && q < C::kLoads; ++q) issue(q);
+      for (int q = m * L / M; q < (m + 1) * L / M; ++q) issue(q);
       __builtin_amdgcn_sched_barrier(0);
     }
   }
 };
 
 // acc += P[:, p0 .. p0 + BP - 1]^T . Q[:, q0 .. q0 + BQ - 1] over all K rows. (wp0, wq0):
-// this wave's corner in the block tile. Every trip issues exactly one tile's loads (past
-// the end the last tile again, into a stage nobody reads), so kLoads * (NS - 2) loads may
-// stay in flight while a tile is awaited.
+// this wave's corner in the block tile.
+//
+// Software pipeline: while the MFMAs of tile kt run out of one set of operand registers,
+// the LDS reads of tile kt + 1 fill the other set and NS - 1 further tiles are on their way
+// from memory. Tile kt lives in stage kt % NS, which is refilled as soon as every wave holds
+// tile kt in registers. Every step issues exactly one tile's loads (past the end the last
+// tile again), so kLoads * (NS - 2) loads may stay in flight while a tile is awaited.
 template <class C>
 __device__ __forceinline__ void mainloop(Tile<C>& t, Smem<C>& sm, const bf16_t* P, int64_t ldp, int64_t p0,
                                          const bf16_t* Q, int64_t ldq, int64_t q0, int64_t K, int wp0,
@@ -175,38 +194,58 @@ __device__ __forceinline__ void mainloop(Tile<C>& t, Smem<C>& sm, const bf16_t* 
   for (int i = 0; i < C::TP; ++i) fp[i] = frag_offset(wp0 + 32 * i);
 #pragma unroll
   for (int j = 0; j < C::TQ; ++j) fq[j] = frag_offset(wq0 + 32 * j);
-  auto first_row = [&](int64_t kt) { return kt + 1 < nk ? kt * BK : K - BK; };
-  auto issue_q = [&](int64_t kt, uint32_t st, int q) {
-    const int64_t row = first_row(kt);
-    const uint32_t dst = st + static_cast<uint32_t>((q * C::kWaves + wave) * 1024);
+  // tile kt lives in stage kt % NS; tiles past the end are the last tile again (their
+  // stages are read into registers that no MFMA uses, or not at all)
+  auto issue_q = [&](int64_t kt, int q) {
+    const int64_t kc = kt < nk ? kt : nk - 1;
+    const int64_t row = kc + 1 < nk ? kc * BK : K - BK;
+    const uint32_t dst = lds0 + static_cast<uint32_t>(kt & (NS - 1)) * C::kStageBytes +
+                         static_cast<uint32_t>((q * C::kWaves + wave) * 1024);
     if (sub_of(q) < C::SUBP) load16_to_lds(P + row * ldp, off[q], dst);
     else load16_to_lds(Q + row * ldq, off[q], dst);
   };
-#pragma unroll
-  for (int s = 0; s < NS - 1; ++s) {
-    const int64_t kc = s < nk ? s : nk - 1;
-#pragma unroll
-    for (int q = 0; q < C::kLoads; ++q) issue_q(kc, lds0 + s * C::kStageBytes, q);
-  }
-  // One trip: wait for tile kt, refill the stage read in the trip before with tile
-  // kt + NS - 1, multiply. A last tile that repeats rows of the one before has them zeroed
-  // in P's part of its stage first.
-  int stage = 0;
-  for (int64_t kt = 0; kt < nk; ++kt) {
-    wait_and_barrier<C::kLoads*(NS - 2)>();
-    if (kt + 1 == nk && dup > 0) {
-      for (int idx = threadIdx.x; idx < C::SUBP * dup * (ROW_BYTES / 16); idx += C::kThreads) {
-        const int sub = idx / (dup * (ROW_BYTES / 16)), rest = idx % (dup * (ROW_BYTES / 16));
-        *reinterpret_cast<uint4*>(&sm.stage[stage][sub * SUB_BYTES + rest * 16]) = make_uint4(0u, 0u, 0u, 0u);
-      }
-      __syncthreads();
+  // rows of the last tile that repeat the tile before: zero them in P's part of the stage
+  auto zero_repeated_rows = [&](int64_t kt) {
+    if (kt + 1 != nk || dup == 0) return;
+    unsigned char* st = sm.stage[kt & (NS - 1)];
+    for (int idx = threadIdx.x; idx < C::SUBP * dup * (ROW_BYTES / 16); idx += C::kThreads) {
+      const int sub = idx / (dup * (ROW_BYTES / 16)), rest = idx % (dup * (ROW_BYTES / 16));
+      *reinterpret_cast<uint4*>(st + sub * SUB_BYTES + rest * 16) = make_uint4(0u, 0u, 0u, 0u);
     }
-    const int64_t kn = kt + NS - 1 < nk ? kt + NS - 1 : nk - 1;
-    const uint32_t dst = lds0 + ((stage + NS - 1) & (NS - 1)) * C::kStageBytes;
-    const unsigned char* st = sm.stage[stage];
-    t.mma(st, st + C::SUBP * SUB_BYTES, fp, fq, [&](int q) { issue_q(kn, dst, q); });
-    stage = (stage + 1) & (NS - 1);
+    __syncthreads();
+  };
+#pragma unroll
+  for (int s = 0; s < NS; ++s)
+#pragma unroll
+    for (int q = 0; q < C::kLoads; ++q) issue_q(s, q);
+  Frags<C> f0, f1;
+  wait_and_barrier<C::kLoads*(NS - 1)>();  // tile 0 has landed for every wave
+  zero_repeated_rows(0);
+  {
+    const unsigned char* st = sm.stage[0];
+#pragma unroll
+    for (int r = 0; r < Frags<C>::kReads; ++r) f0.read(r, st, st + C::SUBP * SUB_BYTES, fp, fq);
   }
+  // Step kt: MFMAs of tile kt out of `cur` while the reads of tile kt + 1 fill `nxt`.
+  // Before the barrier every wave has received its reads of tile kt (so stage kt % NS may be
+  // refilled, with tile kt + NS) and its loads of tile kt + 1 have landed.
+  auto step = [&](int64_t kt, const Frags<C>& cur, Frags<C>& nxt) {
+    // as a builtin, not inline assembly: the compiler's own wait insertion then knows that
+    // `cur` is complete and does not wait for the reads of `nxt` before an MFMA
+    __builtin_amdgcn_s_waitcnt(kWaitLgkm0);
+    __builtin_amdgcn_sched_barrier(0);
+    wait_and_barrier<C::kLoads*(NS - 2)>();
+    zero_repeated_rows(kt + 1);
+    const unsigned char* st = sm.stage[(kt + 1) & (NS - 1)];
+    t.mma(cur, nxt, st, st + C::SUBP * SUB_BYTES, fp, fq, [&](int q) { issue_q(kt + NS, q); });
+  };
+  int64_t kt = 0;
+  for (; kt + 1 < nk; kt += 2) {
+    step(kt, f0, f1);
+    step(kt + 1, f1, f0);
+  }
+  if (kt < nk) step(kt, f0, f1);
+  __builtin_amdgcn_s_waitcnt(kWaitLgkm0);
   wait_and_barrier<0>();  // the stage memory is the caller's again
 }
 
