@@ -428,13 +428,14 @@ def kernel_table(dev, iters: int = 10, warm: int = 3, with_cpu: bool = True):
     yield row("linear_gs (T>1, fp32 MFMA)", "a1", "n=16 T=256 1024x1024 f32", timed(lambda: K.linear_grad_sample(b, a)),
               "mfma_fp32", 2.0 * n * T * i * o, cpu(lambda: O.linear_grad_sample(ca, cb), 4, "4 of 16 samples"))
     a16, b16 = a.bfloat16(), b.bfloat16()
-    yield row("linear_gs (T>1, bf16 MFMA)", "a1", "n=16 T=256 1024x1024 bf16 in, f32 out",
-              timed(lambda: K.linear_grad_sample(b16, a16, out_dtype=torch.float32)), "mfma_bf16", 2.0 * n * T * i * o)
+    yield row("linear_gs (T>1, bf16 MFMA)", "a1", "n=16 T=256 1024x1024 bf16",
+              timed(lambda: K.linear_grad_sample(b16, a16)), "mfma_bf16", 2.0 * n * T * i * o)
     n2, T2 = 16, 1024
     a2 = torch.randn(n2, T2, 2048, device=dev).bfloat16()
-    b2 = torch.randn(n2, T2, 1024, device=dev).bfloat16()
-    yield row("linear_gs (T>1, bf16 MFMA)", "a1", "n=16 T=1024 2048->1024 bf16 in, f32 out",
-              timed(lambda: K.linear_grad_sample(b2, a2, out_dtype=torch.float32)), "mfma_bf16", 2.0 * n2 * T2 * 2048 * 1024)
+    for o2 in (1024, 5632):
+        b2 = torch.randn(n2, T2, o2, device=dev).bfloat16()
+        yield row("linear_gs (T>1, bf16 MFMA)", "a1", f"n=16 T=1024 2048->{o2} bf16",
+                  timed(lambda: K.linear_grad_sample(b2, a2)), "mfma_bf16", 2.0 * n2 * T2 * 2048 * o2)
     del a16, b16, a2, b2
     # ---- C3 / C5: ghost norms, bf16
     for cfg, n, T, layers in (
