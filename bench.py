@@ -233,12 +233,12 @@ def workload_c4(dev):
     )
 
 
-def _ghost_workload(dev, net, make_inputs, loss_call, n, T, sigma, desc):
+def _ghost_workload(dev, net, make_inputs, loss_call, n, T, sigma, desc, single=False):
     from opacus_amd import GradSampleModuleFastGradientClipping
     from opacus_amd.optimizers import DPOptimizerFastGradientClipping
 
     net = net.to(dev).bfloat16()
-    model = GradSampleModuleFastGradientClipping(net, loss_reduction="mean", max_grad_norm=1.0)
+    model = GradSampleModuleFastGradientClipping(net, loss_reduction="mean", max_grad_norm=1.0, single_backward=single)
     opt = DPOptimizerFastGradientClipping(
         torch.optim.SGD(model.parameters(), lr=0.01), noise_multiplier=sigma, max_grad_norm=1.0, expected_batch_size=n
     )
@@ -251,14 +251,15 @@ def _ghost_workload(dev, net, make_inputs, loss_call, n, T, sigma, desc):
 
     flops = ghost_executed_flops(net, n, T)
     return dict(
-        step=step, n=n, dtype="bf16", workload=desc, extra={"ghost_norm_executed_flops_per_step": flops},
+        step=step, n=n, dtype="bf16", workload=desc + (", single backward pass" if single else ""),
+        extra={"ghost_norm_executed_flops_per_step": flops},
         roofline=dict(kernel="ghost_norm_bf16_dlds_kernel<128x128, 2 stages> (all Linear layers of a step)",
                       timer="linear_ghost_norm", bound="mfma", work_per_step=flops, unit="TFLOP/s",
                       peak=MFMA_BF16_PEAK_TFLOPS, traffic=None),
     )
 
 
-def workload_c3(dev):
+def workload_c3(dev, single=False):
     from opacus_amd import DPLossFastGradientClipping
 
     torch.manual_seed(0)
@@ -274,10 +275,11 @@ def workload_c3(dev):
     return _ghost_workload(
         dev, net, lambda: torch.randn(n, T, 1024).to(dev).bfloat16(), loss_call, n, T, 1.0,
         "MLP Linear(1024->4096) GELU Linear(4096->1024), bf16, batch 32, T=512, ghost clipping, C=1, sigma=1",
+        single=single,
     )
 
 
-def workload_c5(dev, tied=False):
+def workload_c5(dev, tied=False, single=False):
     from opacus_amd import DPLossFastGradientClipping
 
     torch.manual_seed(0)
@@ -295,6 +297,7 @@ def workload_c5(dev, tied=False):
         dev, net, lambda: torch.randint(0, V, (n, T)).to(dev), loss_call, n, T, 0.8,
         f"4-layer Llama-style decoder (d 2048, 16 heads / 4 KV, SwiGLU 5632, vocab 32000, {'tied' if tied else 'untied'}), "
         "bf16, batch 16, seq 1024, ghost clipping, C=1, sigma=0.8",
+        single=single,
     )
 
 
@@ -305,6 +308,8 @@ def workload_c5_tied(dev):
 WORKLOADS = {
     "c1": workload_c1, "c2": workload_c2, "c3": workload_c3, "c4": workload_c4, "c5": workload_c5,
     "c5t": workload_c5_tied,
+    # the same two with the clipped sum formed from the first backward pass (single_backward=True)
+    "c3s": lambda dev: workload_c3(dev, single=True), "c5s": lambda dev: workload_c5(dev, single=True),
 }
 
 

@@ -12,6 +12,15 @@ altogether (:172-179): an ``nn.Embedding`` whose table is also the weight of an 
 (tied input and output embeddings). The norm of the sum of the two layers' gradients is
 their two ghost norms plus twice a cross term, ``kernels.tied_embedding_cross_term``.
 
+``single_backward=True`` replaces the second backward pass: the hooks keep every layer's
+(activations, backprops) of the first pass, and once the clipping coefficients are known the
+clipped gradient sum of each layer is formed from them directly: one GEMM
+``(coef * b)^T a`` for a Linear layer, the weighted embedding backward for an Embedding, the
+layer's grad sampler and the clip-weighted sum for anything else. The sum is the one the
+second pass would have left in ``p.grad`` (the gradient of ``sum_n coef[n] loss[n]`` is linear
+in the per-sample backprops); what is saved is the pass's walk back through the activations,
+at the price of keeping the backprops alive until the coefficients exist.
+
 Norm samples are kept in float32 whatever the dtype of the backprops (the kernels
 accumulate in fp32; rounding a norm to bf16 before it meets the other parameters' norms
 would only lose bits).
@@ -71,10 +80,13 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
         force_functorch=False,
         max_grad_norm=1,
         use_ghost_clipping=True,
+        single_backward: bool = False,
     ):
         super().__init__(
             m, batch_first=batch_first, loss_reduction=loss_reduction, strict=strict, force_functorch=force_functorch
         )
+        self.single_backward = single_backward
+        self._kept_passes = []
         self.trainable_parameters = [p for _, p in trainable_parameters(self._module)]
         self._tied_embedding_weights = self._find_tied_embedding_weights()
 
@@ -147,6 +159,9 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
         """Inputs of the model that carry a graph of their own: a leaf that requires grad is
         one more leaf to reach; a computed tensor that requires grad has leaves this object
         cannot see, and the first pass then stays unrestricted."""
+        # records are made by backward hooks and consumed at the end of the same backward();
+        # anything still here was left by one that did not get that far
+        self._kept_passes = []
         stack = list(args) + list(kwargs.values())
         while stack:
             t = stack.pop()
@@ -241,6 +256,8 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
             activations, backprops = stacked
             for _, p in trainable_parameters(module):
                 p._forward_counter += 1  # taken off again below, as for a module used once
+        if self.single_backward:
+            self._kept_passes.append((module, activations, backprops, scale))
         if self.use_ghost_clipping and type(module) in self.NORM_SAMPLERS:
             norm_samples = call_sampler(self.NORM_SAMPLERS[type(module)], module, activations, backprops, scale)
             for param, ns in norm_samples.items():
@@ -266,6 +283,70 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
                     p.grad_sample = None
         if len(module.activations) == 0 and hasattr(module, "max_batch_len"):
             del module.max_batch_len
+
+    # ---- the clipped sum without a second backward pass ---------------------------------------
+    def accumulate_clipped_gradients(self, coef: torch.Tensor) -> None:
+        """Adds ``sum_n coef[n] * grad_n`` of every layer seen by the last backward pass to
+        ``p.grad``, from the kept (activations, backprops): what the second backward pass of
+        ``sum_n coef[n] * loss[n]`` leaves there (fast_gradient_clipping_utils.py:193-201)."""
+        kept, self._kept_passes = self._kept_passes, []
+        sums = {}
+
+        def add(param, value):
+            if not param.requires_grad:
+                return
+            value = value.reshape(param.shape)
+            if id(param) in sums:
+                sums[id(param)][1].add_(value.to(sums[id(param)][1].dtype))
+            else:
+                sums[id(param)] = (param, value)
+
+        for module, activations, backprops, scale in kept:
+            n = backprops.shape[0]
+            c = coef.to(device=backprops.device, dtype=torch.float32)
+            if n == 0:
+                continue
+            if isinstance(module, nn.Linear):
+                a = activations[0].to(backprops.dtype)
+                w = (c * scale).to(backprops.dtype).view(n, *([1] * (backprops.dim() - 1)))
+                if module.bias is None and a.shape[-1] < backprops.shape[-1]:
+                    # (coef * b)^T a == b^T (coef * a): weight the narrower of the two
+                    rows, cols = backprops, a * w
+                else:
+                    rows, cols = backprops * w, a
+                rows = rows.reshape(-1, rows.shape[-1])
+                add(module.weight, rows.t().mm(cols.reshape(-1, cols.shape[-1])))
+                if module.bias is not None:
+                    add(module.bias, rows.sum(dim=0))
+            elif type(module) is nn.Embedding and module.max_norm is None:
+                ids = activations[0]
+                weighted = backprops * (c * scale).to(backprops.dtype).view(n, *([1] * (backprops.dim() - 1)))
+                pad = -1 if module.padding_idx is None else module.padding_idx
+                add(
+                    module.weight,
+                    torch.ops.aten.embedding_dense_backward(
+                        weighted.reshape(-1, weighted.shape[-1]),
+                        ids.reshape(-1),
+                        module.num_embeddings,
+                        pad,
+                        module.scale_grad_by_freq,
+                    ),
+                )
+            else:
+                grad_samples = call_sampler(self._sampler_for(module), module, activations, backprops, scale)
+                for param, gs in grad_samples.items():
+                    if not param.requires_grad:
+                        continue
+                    out = torch.empty(gs.shape[1:], device=gs.device, dtype=gs.dtype)
+                    kernels.clip_accumulate([gs], c, [out], accumulate=False)
+                    add(param, out)
+                del grad_samples
+        for param, total in sums.values():
+            total = total.to(param.dtype)
+            if param.grad is None:
+                param.grad = total
+            else:
+                param.grad.add_(total)
 
     def log_module_gradient_sample_mode(self, module: nn.Module, *, force_functorch=False, use_ghost_clipping=True):
         """Logs, per trainable module, which of the three paths it takes (:255-290)."""
@@ -303,6 +384,7 @@ class GradSampleModuleFastGradientClipping(GradSampleHooksFastGradientClipping, 
         force_functorch=False,
         max_grad_norm=1,
         use_ghost_clipping=True,
+        single_backward: bool = False,
     ):
         nn.Module.__init__(self)
         GradSampleHooksFastGradientClipping.__init__(
@@ -314,6 +396,7 @@ class GradSampleModuleFastGradientClipping(GradSampleHooksFastGradientClipping, 
             force_functorch=force_functorch,
             max_grad_norm=max_grad_norm,
             use_ghost_clipping=use_ghost_clipping,
+            single_backward=single_backward,
         )
         self.grad_accumulation_hook = None
 

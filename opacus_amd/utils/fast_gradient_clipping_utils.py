@@ -10,7 +10,7 @@ import copy
 import torch
 
 
-def first_pass_backward(module, reduced: torch.Tensor) -> None:
+def first_pass_backward(module, reduced: torch.Tensor, retain_graph: bool = True) -> None:
     """Backward pass #1 of ghost clipping (fast_gradient_clipping_utils.py:189): only there
     to let the hooks see the gradients of the layers' outputs. When the module can name the
     tensors at the start of the graph, autograd is asked for those alone, which leaves out
@@ -19,19 +19,20 @@ def first_pass_backward(module, reduced: torch.Tensor) -> None:
     leaves = getattr(module, "first_backward_inputs", None)
     inputs = leaves() if callable(leaves) else None
     if isinstance(inputs, (list, tuple)) and len(inputs) > 0:
-        reduced.backward(retain_graph=True, inputs=list(inputs))
+        reduced.backward(retain_graph=retain_graph, inputs=list(inputs))
         for t in inputs:
             if not t.is_leaf:
                 t.grad = None  # an activation's gradient: the hooks have seen it, nobody else needs it
     else:
-        reduced.backward(retain_graph=True)
+        reduced.backward(retain_graph=retain_graph)
 
 
 class DPTensorFastGradientClipping:
     """A per-sample loss bound to its module and optimizer. ``backward()`` runs: backward #1
     (hooks collect per-sample gradient norms), ``optimizer.zero_grad()``, clipping
     coefficients, hooks off, backward #2 of ``sum_n coef[n] * loss[n]`` (which leaves the
-    clipped gradient sum in ``p.grad``), hooks on (fast_gradient_clipping_utils.py:179-201)."""
+    clipped gradient sum in ``p.grad``), hooks on (fast_gradient_clipping_utils.py:179-201).
+    A module built with ``single_backward=True`` forms that sum from the first pass instead."""
 
     def __init__(self, module, optimizer, loss_per_sample: torch.Tensor, loss_reduction: str = "mean"):
         self.module = module
@@ -101,9 +102,14 @@ class DPTensorFastGradientClipping:
             reduced = torch.sum(self.loss_per_sample, dim=0)
         else:
             raise ValueError(f"loss_reduction = {self.loss_reduction}. Only 'sum' and 'mean' losses are supported")
-        first_pass_backward(self.module, reduced)
+        single = getattr(self.module, "single_backward", False) is True
+        first_pass_backward(self.module, reduced, retain_graph=not single)
         self.optimizer.zero_grad()
         coeff = self.module.get_clipping_coef()
+        if single:
+            # the clipped sum straight from what the hooks kept of the first pass
+            self.module.accumulate_clipped_gradients(coeff)
+            return
         weighted = coeff.to(self.loss_per_sample.device) * self.loss_per_sample
         second_loss = torch.sum(weighted)
         self.module.disable_hooks()

@@ -856,6 +856,88 @@ def test_ghost_bf16_mlp(A):
     gopt.step()
 
 
+def _ghost_grads(A, net, batch, loss_call, *, single, steps=2, C=0.05, reduction="mean"):
+    """p.grad after `steps` forward / DP-backward rounds (the last one's), plus the module."""
+    ghost = A.GradSampleModuleFastGradientClipping(
+        copy.deepcopy(net).to(DEV), loss_reduction=reduction, max_grad_norm=C, single_backward=single
+    )
+    n = batch[0].shape[0]
+    opt = A.DPOptimizerFastGradientClipping(
+        torch.optim.SGD(ghost.parameters(), lr=0.1), noise_multiplier=0.0, max_grad_norm=C, expected_batch_size=n, loss_reduction=reduction
+    )
+    for _ in range(steps):  # a second round must find no leftovers of the first
+        opt.zero_grad()
+        loss_call(ghost, opt, [t.to(DEV) for t in batch]).backward()
+    return [p.grad.detach().clone() for p in ghost.parameters()], ghost
+
+
+@pytest.mark.parametrize("case", ["mlp_mean", "mlp_sum", "llama", "llama_tied", "cnn", "lstm"])
+def test_ghost_single_backward_leaves_the_second_pass_gradients(A, case):
+    """single_backward=True forms the clipped gradient sum from what the hooks kept of the first
+    backward pass. It must equal what the reference's second pass of sum_n coef[n] loss[n]
+    (fast_gradient_clipping_utils.py:193-201) leaves in p.grad: Linear with and without a
+    sequence dimension and bias, Embedding with repeated ids, RMSNorm / GroupNorm / Conv2d
+    through their grad samplers, a table tied to the LM head, and a layer whose uses are
+    stacked (the recurrent projection of an LSTM)."""
+    torch.manual_seed(21)
+    reduction = "sum" if case == "mlp_sum" else "mean"
+    if case.startswith("mlp"):
+        net = nn.Sequential(nn.Linear(24, 40), nn.GELU(), nn.Linear(40, 12))
+        batch = (torch.randn(6, 33, 24), torch.randn(6, 33, 12))
+
+        def loss_call(model, opt, b):
+            return A.DPLossFastGradientClipping(model, opt, PerSampleMSE(reduction), reduction)(model(b[0]), b[1])
+
+    elif case.startswith("llama"):
+        net = TinyLlama()
+        if case == "llama_tied":
+            net.lm_head.weight = net.emb.weight
+        n, T, V = 4, 16, 50
+        ids = torch.randint(0, V, (n, T))
+        ids[0, :8] = 3
+        batch = (ids, torch.randint(0, V, (n, T)))
+
+        def loss_call(model, opt, b):
+            crit = A.DPLossFastGradientClipping(model, opt, nn.CrossEntropyLoss(), "mean")
+            return crit(model(b[0]).flatten(0, 1).float(), b[1].flatten(), shape=(n, T, V))
+
+    elif case == "cnn":
+        net = nn.Sequential(
+            nn.Conv2d(3, 8, 3, padding=1), nn.GroupNorm(2, 8), nn.ReLU(), nn.Conv2d(8, 8, 3, stride=2), nn.ReLU(),
+            nn.Flatten(), nn.Linear(8 * 3 * 3, 5),
+        )
+        batch = (torch.randn(7, 3, 8, 8), torch.randint(0, 5, (7,)))
+
+        def loss_call(model, opt, b):
+            return A.DPLossFastGradientClipping(model, opt, nn.CrossEntropyLoss(), "mean")(model(b[0]), b[1])
+
+    else:
+        from opacus_amd.layers import DPLSTM
+
+        class Tagger(nn.Module):
+            def __init__(self):
+                super().__init__()
+                self.rnn = DPLSTM(6, 10, num_layers=1, batch_first=True, bidirectional=True)
+                self.out = nn.Linear(20, 4)
+
+            def forward(self, x):
+                return self.out(self.rnn(x)[0])
+
+        net = Tagger()
+        batch = (torch.randn(5, 9, 6), torch.randn(5, 9, 4))
+
+        def loss_call(model, opt, b):
+            return A.DPLossFastGradientClipping(model, opt, PerSampleMSE("mean"), "mean")(model(b[0]), b[1])
+
+    two, _ = _ghost_grads(A, net, batch, loss_call, single=False, reduction=reduction)
+    one, ghost = _ghost_grads(A, net, batch, loss_call, single=True, reduction=reduction)
+    assert ghost._kept_passes == []
+    assert (ghost.per_sample_gradient_norms > 0.05).any()  # some sample is clipped
+    for (name, _), g1, g2 in zip(ghost.named_parameters(), one, two):
+        scale = g2.abs().max().item() + 1e-12
+        close(g1 / scale, g2 / scale, 1e-4, 2e-6, f"{case} {name}")
+
+
 def test_ghost_tied_parameters_raise(A):
     class Tied(nn.Module):
         def __init__(self):
