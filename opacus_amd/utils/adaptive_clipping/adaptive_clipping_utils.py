@@ -57,7 +57,8 @@ class DPTensorFastGradientAdaptiveClipping(DPTensorFastGradientClipping):
             reduced = torch.sum(self.loss_per_sample, dim=0)
         else:
             raise ValueError(f"loss_reduction = {self.loss_reduction}. Only 'sum' and 'mean' losses are supported")
-        first_pass_backward(self.module, reduced)
+        single = getattr(self.module, "single_backward", False) is True
+        first_pass_backward(self.module, reduced, retain_graph=not single)
         self.optimizer.zero_grad()
 
         per_sample_norms = self.module.get_norm_sample()
@@ -74,6 +75,9 @@ class DPTensorFastGradientAdaptiveClipping(DPTensorFastGradientClipping):
             torch.ones_like(per_sample_norms),
             new_max_grad_norm / per_sample_norms,
         )
+        if single:  # the clipped sum straight from what the hooks kept of the first pass
+            self.module.accumulate_clipped_gradients(coeff)
+            return
         second_loss = torch.sum(coeff.to(self.loss_per_sample.device) * self.loss_per_sample)
         self.module.disable_hooks()
         second_loss.backward()

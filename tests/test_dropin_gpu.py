@@ -952,10 +952,12 @@ def test_ghost_tied_parameters_raise(A):
         ghost(torch.randn(2, 6, device=DEV))
 
 
-def test_ghost_adaptive_clipping_engine_step_matches_oracle(A, monkeypatch):
+@pytest.mark.parametrize("single", [False, True])
+def test_ghost_adaptive_clipping_engine_step_matches_oracle(A, monkeypatch, single):
     """adaptive_clipping_utils.py:77-121 end to end: the norms of backward #1 feed the bound
-    update, and the clipped sum of backward #2 equals sum_n coeff[n] * g[n] with the oracle's
-    coefficients of the new bound (sigma = 0, count noise pinned to zero)."""
+    update, and the clipped sum of backward #2 (or, with single_backward, the sum formed from
+    backward #1) equals sum_n coeff[n] * g[n] with the oracle's coefficients of the new bound
+    (sigma = 0, count noise pinned to zero)."""
     from opacus_amd.utils.adaptive_clipping import DPLossFastGradientAdaptiveClipping, PrivacyEngineAdaptiveClipping
 
     torch.manual_seed(21)
@@ -983,6 +985,7 @@ def test_ghost_adaptive_clipping_engine_step_matches_oracle(A, monkeypatch):
         target_unclipped_quantile=0.6, min_clipbound=1e-4, max_clipbound=10.0, clipbound_learning_rate=0.3,
     )
     assert isinstance(crit, DPLossFastGradientAdaptiveClipping)
+    model.single_backward = single
     before = [p.detach().double().cpu().clone() for p in net.parameters()]
     opt.zero_grad()
     crit(model(x.to(DEV)), y.to(DEV)).backward()
