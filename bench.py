@@ -432,6 +432,10 @@ def kernel_table(dev, iters: int = 10, warm: int = 3, with_cpu: bool = True):
     ca, cb = a[:4].cpu(), b[:4].cpu()
     yield row("linear_gs (T>1, fp32 MFMA)", "a1", "n=16 T=256 1024x1024 f32", timed(lambda: K.linear_grad_sample(b, a)),
               "mfma_fp32", 2.0 * n * T * i * o, cpu(lambda: O.linear_grad_sample(ca, cb), 4, "4 of 16 samples"))
+    a3, b3 = torch.randn(16, 1024, 2048, device=dev), torch.randn(16, 1024, 1024, device=dev)
+    yield row("linear_gs (T>1, fp32 MFMA)", "a1", "n=16 T=1024 2048->1024 f32", timed(lambda: K.linear_grad_sample(b3, a3)),
+              "mfma_fp32", 2.0 * 16 * 1024 * 2048 * 1024)
+    del a3, b3
     a16, b16 = a.bfloat16(), b.bfloat16()
     yield row("linear_gs (T>1, bf16 MFMA)", "a1", "n=16 T=256 1024x1024 bf16",
               timed(lambda: K.linear_grad_sample(b16, a16)), "mfma_bf16", 2.0 * n * T * i * o)

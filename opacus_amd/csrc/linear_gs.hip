@@ -11,6 +11,7 @@
 #include "dpk_common.h"
 #include "mfma_bf16.h"
 #include "mfma_bf16_tr.h"
+#include "mfma_f32_dlds.h"
 #include "mfma_f32.h"
 
 #include <cstdlib>
@@ -201,17 +202,37 @@ template <typename TOUT> struct TrOut;
 template <> struct TrOut<bf16_t> { static constexpr int kPad = 8, kRows = 128; };
 template <> struct TrOut<float> { static constexpr int kPad = 16, kRows = 64; };
 
-template <class C, typename TOUT>
-__global__ __launch_bounds__(C::kThreads) void linear_tr_bf16_kernel(
-    const bf16_t* __restrict__ b, const bf16_t* __restrict__ a, TOUT* __restrict__ gs,
+// The two engines behind the kernel: input element type, stage memory, accumulator tile and
+// main loop of mfma_bf16_tr.h (bf16, transposing LDS reads) or mfma_f32_dlds.h (fp32).
+struct TrBf16 {
+  typedef bf16_t elem;
+  template <class C> using Smem = mb16t::Smem<C>;
+  template <class C> using Tile = mb16t::Tile<C>;
+  template <class C, class... A> static __device__ __forceinline__ void mainloop(A&&... args) {
+    mb16t::mainloop<C>(static_cast<A&&>(args)...);
+  }
+};
+struct DldsF32 {
+  typedef float elem;
+  template <class C> using Smem = mf32d::Smem<C>;
+  template <class C> using Tile = mf32d::Tile<C>;
+  template <class C, class... A> static __device__ __forceinline__ void mainloop(A&&... args) {
+    mf32d::mainloop<C>(static_cast<A&&>(args)...);
+  }
+};
+
+template <class E, class C, typename TOUT>
+__global__ __launch_bounds__(C::kThreads) void linear_dlds_kernel(
+    const typename E::elem* __restrict__ b, const typename E::elem* __restrict__ a, TOUT* __restrict__ gs,
     float* __restrict__ partials, int64_t T, int64_t M, int64_t N, float scale, int64_t tiles_m,
     int64_t tiles_n) {
-  __shared__ mb16t::Smem<C> sm;
+  typedef typename E::template Smem<C> SmemT;
+  __shared__ SmemT sm;
   __shared__ float red[C::kWaves];
   // rows of the product = input features (P = a), columns = output features (Q = b)
   constexpr int BJ = C::BP, BI = C::BQ;
   constexpr int kPitch = BJ * sizeof(TOUT) + TrOut<TOUT>::kPad, kRows = TrOut<TOUT>::kRows;
-  static_assert(kRows * kPitch <= sizeof(mb16t::Smem<C>), "output rows must fit the stage memory");
+  static_assert(kRows * kPitch <= sizeof(SmemT), "output rows must fit the stage memory");
   static_assert(BI % kRows == 0 && kRows % 32 == 0, "passes of whole MFMA tiles");
   // neighbouring tiles of a sample share operand panels: keep them on one XCD
   const uint32_t bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
@@ -222,9 +243,9 @@ __global__ __launch_bounds__(C::kThreads) void linear_tr_bf16_kernel(
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wj0 = (wave / C::WQ) * (32 * C::TP), wi0 = (wave % C::WQ) * (32 * C::TQ);  // this wave's corner
-  mb16t::Tile<C> tile;
+  typename E::template Tile<C> tile;
   tile.clear();
-  mb16t::mainloop<C>(tile, sm, a + sample * T * N, N, n0, b + sample * T * M, M, m0, T, wj0, wi0);
+  E::template mainloop<C>(tile, sm, a + sample * T * N, N, n0, b + sample * T * M, M, m0, T, wj0, wi0);
   TOUT* out = gs + sample * M * N;
   const int kk = lane >> 5, l32 = lane & 31;
   float ss = 0.f;
@@ -260,7 +281,7 @@ __global__ __launch_bounds__(C::kThreads) void linear_tr_bf16_kernel(
       const int idx = threadIdx.x + r * C::kThreads;
       const int il = idx / kChunksPerRow, c = idx % kChunksPerRow;
       const int64_t i = m0 + pass * kRows + il, j = n0 + c * kPerChunk;
-      if (i < M && j < N) {  // N % 8 == 0: whole chunks
+      if (i < M && j < N) {  // N is a multiple of the chunk: whole chunks
         const uint2* src = reinterpret_cast<const uint2*>(stage_out + il * kPitch + c * 16);
         const uint2 lo = src[0], hi = src[1];
         typedef uint32_t vu4 __attribute__((ext_vector_type(4)));
@@ -279,6 +300,7 @@ __global__ __launch_bounds__(C::kThreads) void linear_tr_bf16_kernel(
   }
 }
 
+using DldsF32Cfg = mf32d::Config<2, 2, 2, 2, 4>;  // 128 x 128, 4 waves, 64 KB: two blocks per CU
 using TrSmall = mb16t::Config<2, 2, 2, 2, 4>;  // 128 x 128, 4 waves, 64 KB: two blocks per CU
 using TrLarge = mb16t::Config<4, 2, 2, 4, 4>;  // 256 x 256, 8 waves, 128 KB: one block per CU
 // time of a 256 x 256 block relative to four 128 x 128 blocks run two at a time
@@ -381,6 +403,17 @@ void plan_tr(Plan& p, const void* b, const void* a, const void* gs, int64_t n, i
   p.tiles_n = dpk_cdiv(N, p.tr);
 }
 
+// Whether the direct-load fp32 kernel takes the shape: whole 16-byte chunks, at least one whole
+// k tile, a bf16 result only in whole 16-byte chunks too. Same 128 x 128 tiling as the plan.
+void plan_dlds_f32(Plan& p, const void* b, const void* a, const void* gs, int gs_dtype, int64_t T, int64_t M,
+                   int64_t N) {
+  const int64_t out_chunk = gs_dtype == DPK_BF16 ? 8 : 4;
+  if (p.outer || p.bm != 128 || T < mf32d::BK || M % 4 != 0 || N % out_chunk != 0 || M >= (1LL << 24) || N >= (1LL << 24) ||
+      !dpk_aligned(b, 16) || !dpk_aligned(a, 16) || !dpk_aligned(gs, 16))
+    return;
+  p.tr = 128;
+}
+
 template <typename TIN, typename TOUT>
 void launch_linear(const Plan& p, bool vec, const void* b, const void* a, void* gs, float* partials,
                    int64_t n, int64_t T, int64_t M, int64_t N, float scale, hipStream_t s) {
@@ -418,10 +451,10 @@ void launch_linear(const Plan& p, bool vec, const void* b, const void* a, void* 
   hipLaunchKernelGGL((linear_mfma_bf16_kernel<BMN, BMN, TOUT, V>), grid, block, 0, s, bp, ap, gp, partials, \
                      T, M, N, scale, p.tiles_m, p.tiles_n)
     if (p.tr == 256) {
-      hipLaunchKernelGGL((linear_tr_bf16_kernel<TrLarge, TOUT>), grid, dim3(TrLarge::kThreads), 0, s, bp, ap, gp,
+      hipLaunchKernelGGL((linear_dlds_kernel<TrBf16, TrLarge, TOUT>), grid, dim3(TrLarge::kThreads), 0, s, bp, ap, gp,
                          partials, T, M, N, scale, p.tiles_m, p.tiles_n);
     } else if (p.tr == 128) {
-      hipLaunchKernelGGL((linear_tr_bf16_kernel<TrSmall, TOUT>), grid, dim3(TrSmall::kThreads), 0, s, bp, ap, gp,
+      hipLaunchKernelGGL((linear_dlds_kernel<TrBf16, TrSmall, TOUT>), grid, dim3(TrSmall::kThreads), 0, s, bp, ap, gp,
                          partials, T, M, N, scale, p.tiles_m, p.tiles_n);
     } else if (p.bm == 128) {
       if (vec8) DPK_BF16(128, true);
@@ -431,6 +464,9 @@ void launch_linear(const Plan& p, bool vec, const void* b, const void* a, void* 
       else DPK_BF16(64, false);
     }
 #undef DPK_BF16
+  } else if (p.tr == 128) {
+    hipLaunchKernelGGL((linear_dlds_kernel<DldsF32, DldsF32Cfg, TOUT>), grid, dim3(DldsF32Cfg::kThreads), 0, s, bp, ap,
+                       gp, partials, T, M, N, scale, p.tiles_m, p.tiles_n);
   } else if (p.bm == 128) {
     if (vec)
       hipLaunchKernelGGL((linear_mfma_kernel<128, 128, TIN, TOUT, true>), grid, block, 0, s, bp, ap,
@@ -480,6 +516,7 @@ extern "C" int dpk_linear_gs(const void* b, const void* a, int in_dtype, void* g
   const bool vec = linear_vec(b, a, gs, in_dtype, gs_dtype, out, in);
   Plan p = make_plan(T, out, in, vec);
   if (in_dtype == DPK_BF16) plan_tr(p, b, a, gs, n, T, out, in, dpk_device_cus());
+  else plan_dlds_f32(p, b, a, gs, gs_dtype, T, out, in);
   const int64_t blocks = n * p.tiles_m * p.tiles_n;
   DPK_REQUIRE(blocks <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: %lld blocks exceed the grid limit", who,
               (long long)blocks);

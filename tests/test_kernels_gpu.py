@@ -53,6 +53,9 @@ LINEAR_SHAPES = [
     (2, (33,), 70, 30),  # MFMA small tile, odd sizes -> scalar loads
     (2, (4, 9), 132, 260),  # two middle dims
     (1, (300,), 128, 128),  # long K
+    (2, (16,), 128, 128),  # exactly one k tile of the direct-load fp32 kernel
+    (1, (17,), 68, 132),  # its last k tile repeats 15 rows of the first; sizes that are multiples of 4 only
+    (2, (48,), 516, 260),  # three whole k tiles, ragged block tiles in both directions
 ]
 
 
@@ -68,6 +71,9 @@ def test_linear_grad_sample_f32(K, n, mid, fin, fout, scale):
     assert_rel(gs, want_w, FP32_REL, "weight")
     assert_rel(gb, want_b, FP32_REL, "bias")
     assert_rel(sumsq, want_w.double().flatten(1).pow(2).sum(1), 2e-5, "sumsq")
+    gs16, _ = K.linear_grad_sample(dev(b), dev(a), scale=scale, out_dtype=torch.bfloat16)
+    assert gs16.dtype == torch.bfloat16
+    assert_rel(gs16, want_w, BF16_REL, "weight, fp32 in, bf16 out")
 
 
 @pytest.mark.parametrize(
