@@ -140,14 +140,18 @@ class PerSampleMSE(nn.Module):
 
 
 def ghost_executed_flops(model: nn.Module, n: int, T: int) -> float:
-    """MFMA FLOPs the ghost-norm kernel executes per step: 128 x 128 tiles of the upper
-    block-triangle of both Gram matrices of every Linear layer."""
+    """MFMA FLOPs the ghost-norm entry point executes per step over the (bf16) Linear layers:
+    128 x 128 tiles of the upper block-triangle of both Gram matrices, or, for a layer thin
+    enough that forming its gradient tiles is cheaper (the library's rule, repeated here), the
+    contraction over T itself."""
     nt = (T + 127) // 128
     pairs = nt * (nt + 1) // 2
     total = 0.0
     for m in model.modules():
         if isinstance(m, nn.Linear):
-            total += n * pairs * 2.0 * 128 * 128 * (m.in_features + m.out_features)
+            gram = pairs * 128.0 * 128 * (m.in_features + m.out_features)
+            direct = float(T) * m.in_features * m.out_features
+            total += n * 2.0 * (direct if T > 1 and direct < 0.9 * gram else gram)
     return total
 
 
@@ -253,7 +257,7 @@ def _ghost_workload(dev, net, make_inputs, loss_call, n, T, sigma, desc, single=
     return dict(
         step=step, n=n, dtype="bf16", workload=desc + (", single backward pass" if single else ""),
         extra={"ghost_norm_executed_flops_per_step": flops},
-        roofline=dict(kernel="ghost_norm_bf16_dlds_kernel<128x128, 2 stages> (all Linear layers of a step)",
+        roofline=dict(kernel="ghost_norm_bf16_dlds_kernel<128x128, 2 stages> (all Linear layers of a step; thin layers by linear_dlds_kernel)",
                       timer="linear_ghost_norm", bound="mfma", work_per_step=flops, unit="TFLOP/s",
                       peak=MFMA_BF16_PEAK_TFLOPS, traffic=None),
     )
@@ -458,10 +462,20 @@ def kernel_table(dev, iters: int = 10, warm: int = 3, with_cpu: bool = True):
             b = (torch.randn(n, T, o, device=dev) * 0.02).bfloat16()
             ms = timed(lambda: K.linear_ghost_norm(b, a, want_weight=True, want_bias=False))
             ca, cb = a[:1].cpu(), b[:1].cpu()
-            yield row("linear_ghost_norm", "a2", f"{cfg} {name} n={n} T={T} {i}->{o} bf16", ms, "mfma_bf16",
-                      2.0 * n * T * T * (i + o) * tri / full,
+            gram, direct = T * T * (i + o) * tri / full, float(T) * i * o
+            thin = direct < 0.9 * gram  # the library's rule: form the gradient tiles and square them
+            yield row("linear_ghost_norm", "a2", f"{cfg} {name} n={n} T={T} {i}->{o} bf16" + (" (direct)" if thin else ""),
+                      ms, "mfma_bf16", 2.0 * n * (direct if thin else gram),
                       cpu(lambda: O.linear_norm_sample(ca, cb), n, f"1 of {n} samples, bf16 bmm Grams"))
             del a, b
+    # a low-rank adapter on C5's width: the direct route
+    a = torch.randn(16, 1024, 2048, device=dev).bfloat16()
+    b = (torch.randn(16, 1024, 16, device=dev) * 0.02).bfloat16()
+    ca, cb = a[:1].cpu(), b[:1].cpu()
+    yield row("linear_ghost_norm", "a2", "rank-16 adapter n=16 T=1024 2048->16 bf16 (direct)",
+              timed(lambda: K.linear_ghost_norm(b, a, want_weight=True, want_bias=False)), "mfma_bf16",
+              2.0 * 16 * 1024 * 2048 * 16, cpu(lambda: O.linear_norm_sample(ca, cb), 16, "1 of 16 samples, bf16 bmm Grams"))
+    del a, b
     # ---- C5: embedding ghost norm, RMSNorm, noise over all parameters (bf16)
     n, T, D, V = 16, 1024, 2048, 32000
     ids = torch.randint(0, V, (n, T), device=dev)

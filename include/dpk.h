@@ -66,6 +66,8 @@ int dpk_device_cus(void);
  * written (fp32 accumulators before any down-cast), so that the optimizer's
  * norm pass (optimizers/optimizer.py:444-446) need not re-read gs.
  * T == 1 takes a store-bound outer-product kernel; T > 1 an MFMA kernel.
+ * gs may be NULL when sumsq is given: only the squared norms are formed then
+ * (the gradient tiles never leave the registers).
  * ws is needed only when sumsq != NULL. */
 size_t dpk_linear_gs_workspace_bytes(int64_t n, int64_t T, int64_t out, int64_t in);
 int dpk_linear_gs(const void* b, const void* a, int in_dtype, void* gs, int gs_dtype,

@@ -9,6 +9,9 @@
 // ti <= tj are visited and off-diagonal ones count twice. One float per block
 // goes to the workspace; a fixed-order reduction applies clamp(min=0) and sqrt
 // (linear.py:87-89, :92).
+#include <cstdlib>
+#include <cstring>
+
 #include "dpk_common.h"
 #include "mfma_bf16.h"
 #include "mfma_bf16_dlds.h"
@@ -268,15 +271,46 @@ int tile_edge(int64_t T) { return T > 64 ? 128 : 64; }
 
 }  // namespace
 
+// The Gram route costs 2 T'^2 (in + out) multiply-adds per sample over the tile pairs it
+// visits, forming the gradient and squaring it 2 T in out: for thin layers (a low-rank
+// adapter, a narrow head) the second is far cheaper although the gradient tile exists for a
+// moment in registers. The two routes run at about the same rate for bf16; for fp32 the
+// contraction kernel is the faster of the two by half again.
+// DPK_GHOST_NORM_ROUTE=gram|direct in the environment overrides the choice (for tests that
+// want both routes on the same shapes).
+bool direct_is_cheaper(int dtype, int64_t T, int64_t out, int64_t in) {
+  if (const char* force = getenv("DPK_GHOST_NORM_ROUTE")) {
+    if (strcmp(force, "gram") == 0) return false;
+    if (strcmp(force, "direct") == 0) return true;
+  }
+  const int B = T > 64 ? 128 : 64;
+  const int64_t nt = dpk_cdiv(T, B);
+  const double gram = static_cast<double>(nt * (nt + 1) / 2) * B * B * static_cast<double>(in + out);
+  const double direct = static_cast<double>(T) * static_cast<double>(in) * static_cast<double>(out);
+  return direct < (dtype == DPK_F32 ? 1.5 : 0.9) * gram;
+}
+
+struct DirectLayout {
+  size_t bias, total;  // [0, bias): the Linear kernel's partial sums; then float[n, out]
+};
+
+DirectLayout direct_layout(int64_t n, int64_t T, int64_t out, int64_t in) {
+  DirectLayout l;
+  l.bias = dpk_align_up(dpk_linear_gs_workspace_bytes(n, T, out, in), 256);
+  l.total = l.bias + dpk_align_up(static_cast<size_t>(n) * out * sizeof(float), 256);
+  return l;
+}
+
 extern "C" size_t dpk_linear_ghost_norm_workspace_bytes(int64_t n, int64_t T, int64_t out,
                                                         int64_t in) {
-  (void)out;
-  (void)in;
   if (n <= 0 || T <= 1) return 0;
   // Room for any tiling: 64-row tile pairs, or 128-row tile pairs with four
   // quadrant slots each (2 m^2 + 2 m slots per sample covers both).
   const int64_t m = dpk_cdiv(T, 128);
-  return dpk_align_up(static_cast<size_t>(2 * n * (2 * m * m + 2 * m)) * sizeof(float), 256);
+  const size_t gram = dpk_align_up(static_cast<size_t>(2 * n * (2 * m * m + 2 * m)) * sizeof(float), 256);
+  // whichever dtype: the caller does not say, and the fp32 rule takes every shape the bf16 rule takes
+  const size_t direct = direct_is_cheaper(DPK_F32, T, out, in) ? direct_layout(n, T, out, in).total : 0;
+  return gram > direct ? gram : direct;
 }
 
 extern "C" int dpk_linear_ghost_norm(const void* b, const void* a, int dtype, float* norm_w,
@@ -304,6 +338,25 @@ extern "C" int dpk_linear_ghost_norm(const void* b, const void* a, int dtype, fl
                          static_cast<const bf16_t*>(b), static_cast<const bf16_t*>(a), norm_w, norm_b,
                          out, in, absscale);
     DPK_LAUNCH_CHECK(who);
+    return DPK_OK;
+  }
+  if (norm_w && direct_is_cheaper(dtype, T, out, in)) {
+    // |sum_t b_t a_t^T|_F from the per-sample gradient tiles themselves, never stored;
+    // the bias norm from the column sums of b
+    const DirectLayout l = direct_layout(n, T, out, in);
+    DPK_REQUIRE(ws && ws_bytes >= l.total, DPK_E_WORKSPACE, "%s: workspace %zu < %zu bytes", who, ws_bytes, l.total);
+    DPK_REQUIRE(dpk_aligned(ws, 256), DPK_E_ALIGN, "%s: workspace must be 256-byte aligned", who);
+    char* base = static_cast<char*>(ws);
+    int rc = dpk_linear_gs(b, a, dtype, nullptr, dtype, norm_w, n, T, out, in, 1.0f, base, l.bias, stream);
+    if (rc != DPK_OK) return rc;
+    dpk_launch_reduce_rows(norm_w, n, 1, norm_w, 1, absscale, s);  // in place: sqrt, times |scale|
+    DPK_LAUNCH_CHECK(who);
+    if (norm_b) {
+      rc = dpk_linear_bias_gs(b, dtype, base + l.bias, DPK_F32, norm_b, n, T, out, 1.0f, stream);
+      if (rc != DPK_OK) return rc;
+      dpk_launch_reduce_rows(norm_b, n, 1, norm_b, 1, absscale, s);
+      DPK_LAUNCH_CHECK(who);
+    }
     return DPK_OK;
   }
   const int B = tile_edge(T);

@@ -143,7 +143,7 @@ __global__ __launch_bounds__(kThreads) void linear_mfma_kernel(
     const int64_t i = m0 + r, j = n0 + c;
     if (i < M && j < N) {
       const float x = v * scale;
-      dpk_io<TOUT>::store(out + i * N + j, x);
+      if (gs) dpk_io<TOUT>::store(out + i * N + j, x);
       ss = fmaf(x, x, ss);
     }
   });
@@ -178,7 +178,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     const int64_t i = m0 + r, j = n0 + c;
     if (i < M && j < N) {
       const float x = v * scale;
-      dpk_io<TOUT>::store(out + i * N + j, x);
+      if (gs) dpk_io<TOUT>::store(out + i * N + j, x);
       ss = fmaf(x, x, ss);
     }
   });
@@ -250,10 +250,27 @@ __global__ __launch_bounds__(C::kThreads) void linear_dlds_kernel(
   const int kk = lane >> 5, l32 = lane & 31;
   float ss = 0.f;
   unsigned char* stage_out = &sm.stage[0][0];
+  if (gs == nullptr) {  // only the squared norm is wanted
+#pragma unroll
+    for (int it = 0; it < C::TQ; ++it)
+#pragma unroll
+      for (int jt = 0; jt < C::TP; ++jt)
+#pragma unroll
+        for (int vg = 0; vg < 4; ++vg) {
+          const int il = wi0 + it * 32 + l32, jl = wj0 + jt * 32 + vg * 8 + kk * 4;
+          if (m0 + il < M && n0 + jl < N) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const float x = tile.acc[jt][it][vg * 4 + e] * scale;
+              ss = fmaf(x, x, ss);
+            }
+          }
+        }
+  }
   // In a pass the waves that own rows [pass * kRows, + kRows) of the tile put them into the
   // stage memory, then all threads send whole rows on their way.
 #pragma unroll
-  for (int pass = 0; pass < BI / kRows; ++pass) {
+  for (int pass = 0; gs != nullptr && pass < BI / kRows; ++pass) {
     if (pass > 0) __syncthreads();
 #pragma unroll
     for (int it = 0; it < C::TQ; ++it) {
@@ -507,7 +524,7 @@ extern "C" int dpk_linear_gs(const void* b, const void* a, int in_dtype, void* g
               "%s: n=%lld T=%lld out=%lld in=%lld", who, (long long)n, (long long)T, (long long)out,
               (long long)in);
   if (n == 0) return DPK_OK;
-  DPK_REQUIRE(b && a && gs, DPK_E_ARG, "%s: NULL tensor", who);
+  DPK_REQUIRE(b && a && (gs || sumsq), DPK_E_ARG, "%s: NULL tensor", who);
   DPK_REQUIRE(dpk_dtype_ok(in_dtype) && dpk_dtype_ok(gs_dtype), DPK_E_DTYPE, "%s: dtypes %d,%d", who,
               in_dtype, gs_dtype);
   DPK_REQUIRE(dpk_aligned(b, dpk_elsize(in_dtype)) && dpk_aligned(a, dpk_elsize(in_dtype)) &&
@@ -540,7 +557,9 @@ extern "C" int dpk_linear_gs(const void* b, const void* a, int in_dtype, void* g
                          static_cast<const bf16_t*>(b), static_cast<const bf16_t*>(a), sumsq, out, in, scale);
     DPK_LAUNCH_CHECK(who);
   }
-  if (in_dtype == DPK_F32 && gs_dtype == DPK_F32)
+  if (p.outer && !gs)
+    ;  // norm only, rank one: the closed form above is the whole answer
+  else if (in_dtype == DPK_F32 && gs_dtype == DPK_F32)
     launch_linear<float, float>(p, vec, b, a, gs, partials, n, T, out, in, scale, s);
   else if (in_dtype == DPK_BF16 && gs_dtype == DPK_BF16)
     launch_linear<bf16_t, bf16_t>(p, vec, b, a, gs, partials, n, T, out, in, scale, s);

@@ -384,9 +384,17 @@ GHOST_SHAPES = [
 ]
 
 
-@pytest.mark.parametrize("n,T,fin,fout", GHOST_SHAPES)
+# "gram": sum over the T x T Grams (the reference's formula); "direct": the squared norm of the
+# per-sample gradient tiles as they are formed; None: the library's choice by cost
+GHOST_ROUTES = [None, "gram", "direct"]
+
+
+@pytest.mark.parametrize("n,T,fin,fout", GHOST_SHAPES + [(3, 200, 256, 16), (2, 130, 8, 520)])
 @pytest.mark.parametrize("scale", [1.0, 4.0])
-def test_linear_ghost_norm_f32(K, n, T, fin, fout, scale):
+@pytest.mark.parametrize("route", GHOST_ROUTES)
+def test_linear_ghost_norm_f32(K, n, T, fin, fout, scale, route, monkeypatch):
+    if route is not None:
+        monkeypatch.setenv("DPK_GHOST_NORM_ROUTE", route)
     torch.manual_seed(T * 7 + fin)
     a = torch.randn(n, T, fin)
     b = torch.randn(n, T, fout) * 0.1
@@ -424,9 +432,14 @@ def test_linear_ghost_norm_2d_inputs(K):
         (3, 200, 64, 128),  # quadrants with a few valid rows
         (20, 640, 64, 64),  # 300 units on a 256-CU device: whole-tile blocks only
         (16, 1000, 64, 128),  # 576 units: 512 whole-tile blocks and a tail of quadrant blocks, ragged T
+        (4, 512, 1024, 16),  # a low-rank adapter: thin on one side
+        (4, 512, 16, 1024),
     ],
 )
-def test_linear_ghost_norm_bf16(K, n, T, fin, fout):
+@pytest.mark.parametrize("route", GHOST_ROUTES)
+def test_linear_ghost_norm_bf16(K, n, T, fin, fout, route, monkeypatch):
+    if route is not None:
+        monkeypatch.setenv("DPK_GHOST_NORM_ROUTE", route)
     torch.manual_seed(T)
     a = torch.randn(n, T, fin).bfloat16()
     b = (torch.randn(n, T, fout) * 0.02).bfloat16()
