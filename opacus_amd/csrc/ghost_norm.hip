@@ -127,13 +127,14 @@ constexpr bool ghost_cfg_has_quadrants() {
   return C::BM == 128 && C::BN == 128 && C::BK == 64 && C::kWaves == 4 && C::kStages == 2;
 }
 
-template <class C>
+// TE: bf16_t, or float (whole-tile blocks only; a stage row of 128 bytes is then 32 k values).
+template <class C, typename TE = bf16_t>
 __global__ __launch_bounds__(C::kThreads) void ghost_norm_bf16_dlds_kernel(
-    const bf16_t* __restrict__ b, const bf16_t* __restrict__ a, float* __restrict__ pw,
+    const TE* __restrict__ b, const TE* __restrict__ a, float* __restrict__ pw,
     float* __restrict__ pb, int64_t T, int64_t Dout, int64_t Din, int nJ, int npairs, uint32_t nbig,
     int slots) {
   constexpr int R = C::BM / C::BN;
-  constexpr bool kQuadrants = ghost_cfg_has_quadrants<C>();
+  constexpr bool kQuadrants = ghost_cfg_has_quadrants<C>() && std::is_same<TE, bf16_t>::value;
   __shared__ mb16d::Smem<C> sm;
   __shared__ float red[C::kWaves];
   const bool big = !kQuadrants || blockIdx.x < nbig;
@@ -157,8 +158,8 @@ __global__ __launch_bounds__(C::kThreads) void ghost_norm_bf16_dlds_kernel(
   const float weight = J < R * (I + 1) ? 1.f : 2.f;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int kh = lane >> 5, l32 = lane & 31;
-  const bf16_t* bs = b + sample * T * Dout;
-  const bf16_t* as = a + sample * T * Din;
+  const TE* bs = b + sample * T * Dout;
+  const TE* as = a + sample * T * Din;
   float sw = 0.f, sb = 0.f;
   size_t slot;
   if (big) {
@@ -167,8 +168,8 @@ __global__ __launch_bounds__(C::kThreads) void ghost_norm_bf16_dlds_kernel(
     mb16d::Tile tg, ta;
     tg.clear();
     ta.clear();
-    mb16d::mainloop<C>(tg, sm, bs, bs, Dout, m0a, m0b, T, Dout, wm0, wn0);
-    if (pw) mb16d::mainloop<C>(ta, sm, as, as, Din, m0a, m0b, T, Din, wm0, wn0);
+    mb16d::mainloop<C, TE>(tg, sm, bs, bs, Dout, m0a, m0b, T, Dout, wm0, wn0);
+    if (pw) mb16d::mainloop<C, TE>(ta, sm, as, as, Din, m0a, m0b, T, Din, wm0, wn0);
     // rows past T hold copies of row T - 1: leave them out
     const int rmax = static_cast<int>(T - m0a < C::BM ? T - m0a : C::BM);
     const int cmax = static_cast<int>(T - m0b < C::BN ? T - m0b : C::BN);
@@ -275,7 +276,7 @@ int tile_edge(int64_t T) { return T > 64 ? 128 : 64; }
 // visits, forming the gradient and squaring it 2 T in out: for thin layers (a low-rank
 // adapter, a narrow head) the second is far cheaper although the gradient tile exists for a
 // moment in registers. The two routes run at about the same rate for bf16; for fp32 the
-// contraction kernel is the faster of the two by half again.
+// contraction kernel is the faster of the two by a sixth.
 // DPK_GHOST_NORM_ROUTE=gram|direct in the environment overrides the choice (for tests that
 // want both routes on the same shapes).
 bool direct_is_cheaper(int dtype, int64_t T, int64_t out, int64_t in) {
@@ -287,7 +288,7 @@ bool direct_is_cheaper(int dtype, int64_t T, int64_t out, int64_t in) {
   const int64_t nt = dpk_cdiv(T, B);
   const double gram = static_cast<double>(nt * (nt + 1) / 2) * B * B * static_cast<double>(in + out);
   const double direct = static_cast<double>(T) * static_cast<double>(in) * static_cast<double>(out);
-  return direct < (dtype == DPK_F32 ? 1.5 : 0.9) * gram;
+  return direct < (dtype == DPK_F32 ? 1.1 : 0.9) * gram;
 }
 
 struct DirectLayout {
@@ -364,8 +365,10 @@ extern "C" int dpk_linear_ghost_norm(const void* b, const void* a, int dtype, fl
   // bf16 with 64-aligned feature sizes takes the direct-to-LDS kernel
   // (and a sample small enough for 32-bit byte offsets inside it)
   const int64_t widest = out > in ? out : in;
-  const bool dlds = dtype == DPK_BF16 && B == 128 && out % 64 == 0 && (in % 64 == 0 || !norm_w) &&
-                    dpk_aligned(b, 16) && dpk_aligned(a, 16) && T * widest * 2 < (int64_t{1} << 32);
+  // (fp32 too: 32 k values fill the 128-byte stage row that 64 bf16 do)
+  const int64_t es = dpk_elsize(dtype), kmul = 128 / es;
+  const bool dlds = B == 128 && out % kmul == 0 && (in % kmul == 0 || !norm_w) &&
+                    dpk_aligned(b, 16) && dpk_aligned(a, 16) && T * widest * es < (int64_t{1} << 32);
   const int64_t npairs = dlds ? ghost_pairs(T, GhostCfg::BM, GhostCfg::BN) : nt * (nt + 1) / 2;
   const int64_t blocks = n * npairs;
   // A last round of resident blocks (two per CU) that is at most a quarter full is
@@ -373,7 +376,7 @@ extern "C" int dpk_linear_ghost_norm(const void* b, const void* a, int dtype, fl
   // tile block per CU runs latency-bound and takes most of a full round's time, a
   // round of quadrant blocks about a third of it.
   int64_t tail = 0;
-  if (dlds && ghost_cfg_has_quadrants<GhostCfg>()) {
+  if (dlds && dtype == DPK_BF16 && ghost_cfg_has_quadrants<GhostCfg>()) {
     const int cus = dpk_device_cus();
     DPK_REQUIRE(cus > 0, DPK_E_LAUNCH, "%s: cannot query the device", who);
     const int64_t resident = 2 * static_cast<int64_t>(cus);
@@ -391,7 +394,12 @@ extern "C" int dpk_linear_ghost_norm(const void* b, const void* a, int dtype, fl
   float* pw = norm_w ? static_cast<float*>(ws) : nullptr;
   float* pb = norm_b ? static_cast<float*>(ws) + blocks * slots : nullptr;
   const dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
-  if (dtype == DPK_F32) {
+  if (dtype == DPK_F32 && dlds) {
+    hipLaunchKernelGGL((ghost_norm_bf16_dlds_kernel<GhostCfg, float>), dim3(static_cast<unsigned>(grid_blocks)),
+                       dim3(GhostCfg::kThreads), 0, s, static_cast<const float*>(b), static_cast<const float*>(a),
+                       pw, pb, T, out, in, (int)dpk_cdiv(T, GhostCfg::BN), (int)npairs,
+                       static_cast<uint32_t>(blocks), slots);
+  } else if (dtype == DPK_F32) {
     const bool vec = out % 4 == 0 && in % 4 == 0 && dpk_aligned(b, 16) && dpk_aligned(a, 16);
     const float* bp = static_cast<const float*>(b);
     const float* ap = static_cast<const float*>(a);

@@ -9,6 +9,13 @@
 // Requirements of this path (the caller falls back to mfma_bf16.h otherwise):
 // K % 64 == 0, row stride % 8 == 0, 16-byte aligned base.
 //
+// fp32 operands take the same road (element type float: a stage row of 128 bytes is then 32
+// k values, K % 32 == 0). v_mfma_f32_32x32x2f32 wants lane l to hold k = l / 32 of row
+// l % 32; which two k values meet in one instruction does not matter to a contraction as
+// long as both operands agree, so lanes 0..31 read the 16-byte chunk 2 c of their row and
+// lanes 32..63 chunk 2 c + 1, exactly as for bf16, and the e-th float of the two chunks
+// (k = 8 c + e and 8 c + 4 + e) feeds the e-th of four instructions.
+//
 // LDS stage layout: row-major [rows][64 bf16] = 128 bytes per row, no padding
 // (a wave's 64 lanes must land contiguously), 16-byte chunks XOR-swizzled:
 //   physical chunk = logical chunk ^ ((row >> 1) & 7).
@@ -19,10 +26,14 @@
 // reduction.
 #pragma once
 
+#include <type_traits>
+
 #include "dpk_common.h"
 #include "mfma_bf16.h"
 
 namespace mb16d {
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 using mb16::bf16x8;
 using mb16::floatx16;
@@ -98,7 +109,7 @@ __device__ __forceinline__ void load16_to_lds(const void* sbase, uint32_t voff, 
 // group r * kWaves + wave. lane_offset: this lane's byte offset from the matrix base
 // for that load (rows >= M read row M - 1 instead); group_lds: where the group lands
 // in the tile's LDS image.
-template <class C>
+template <class C, int ES = 2>
 __device__ __forceinline__ uint32_t lane_offset(int64_t ld, int64_t m0, int64_t M, int r) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -107,7 +118,7 @@ __device__ __forceinline__ uint32_t lane_offset(int64_t ld, int64_t m0, int64_t 
   const int lc = swz<C>(row, lane % C::kChunks);  // which logical chunk lives at this physical slot
   int64_t m = m0 + row;
   m = m < M ? m : M - 1;
-  return static_cast<uint32_t>((m * ld + lc * 8) * 2);
+  return static_cast<uint32_t>(m * ld * ES + lc * 16);  // ld in elements of ES bytes
 }
 
 template <class C>
@@ -150,7 +161,7 @@ struct Tile {
 
   // As / Bs: the stage's operand tiles; (wm0, wn0): this wave's corner in the block tile;
   // issue(q), q < NLOADS: issues the q-th load of the tile being prefetched.
-  template <class C, int NLOADS, class IssueFn>
+  template <class C, int NLOADS, typename T = bf16_t, class IssueFn>
   __device__ __forceinline__ void mma(const unsigned char* As, const unsigned char* Bs, int wm0, int wn0,
                                       IssueFn issue) {
     const int lane = threadIdx.x & 63;
@@ -159,18 +170,20 @@ struct Tile {
     // bytes per lane); the MFMAs of step ks then only wait for their own four,
     // so LDS latency is paid once per tile instead of once per step.
     constexpr int KS = C::BK / 16, ROW_BYTES = C::ROW_BYTES;
-    bf16x8 av[KS][2], bv[KS][2];
+    constexpr bool kF32 = std::is_same<T, float>::value;
+    typedef typename std::conditional<kF32, floatx4, bf16x8>::type frag_t;  // 16 bytes either way
+    frag_t av[KS][2], bv[KS][2];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         const int row = wm0 + i * 32 + l32;
-        av[ks][i] = *reinterpret_cast<const bf16x8*>(As + row * ROW_BYTES + swz<C>(row, ks * 2 + kh) * 16);
+        av[ks][i] = *reinterpret_cast<const frag_t*>(As + row * ROW_BYTES + swz<C>(row, ks * 2 + kh) * 16);
       }
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         const int row = wn0 + j * 32 + l32;
-        bv[ks][j] = *reinterpret_cast<const bf16x8*>(Bs + row * ROW_BYTES + swz<C>(row, ks * 2 + kh) * 16);
+        bv[ks][j] = *reinterpret_cast<const frag_t*>(Bs + row * ROW_BYTES + swz<C>(row, ks * 2 + kh) * 16);
       }
     }
     __builtin_amdgcn_sched_barrier(0);  // keep the reads ahead of the MFMAs
@@ -183,11 +196,21 @@ struct Tile {
 #endif
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
+      if constexpr (kF32) {
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+        for (int e = 0; e < 4; ++e)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[ks][i], bv[ks][j], acc[i][j], 0, 0, 0);
+          for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[ks][i][e], bv[ks][j][e], acc[i][j], 0, 0, 0);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[ks][i], bv[ks][j], acc[i][j], 0, 0, 0);
+      }
 #pragma unroll
       for (int q = ks * PER_STEP; q < (ks + 1) * PER_STEP && q < NLOADS; ++q) issue(q);
       __builtin_amdgcn_sched_barrier(0);
@@ -201,12 +224,13 @@ struct Tile {
 // stay outstanding while tile kt is awaited is the constant
 // kLoadsPerTile * (NS - 2). abase / bbase must be wave-uniform and every byte
 // offset inside the matrices must fit 32 bits (M * ld * 2 < 2^32).
-template <class C>
-__device__ __forceinline__ void mainloop(Tile& t, Smem<C>& sm, const bf16_t* abase,
-                                         const bf16_t* bbase, int64_t ld, int64_t m0a, int64_t m0b,
+template <class C, typename T = bf16_t>
+__device__ __forceinline__ void mainloop(Tile& t, Smem<C>& sm, const T* abase,
+                                         const T* bbase, int64_t ld, int64_t m0a, int64_t m0b,
                                          int64_t M, int64_t K, int wm0, int wn0) {
   constexpr int NS = C::kStages;
-  constexpr int BK = C::BK, ROW_BYTES = C::ROW_BYTES;
+  constexpr int ROW_BYTES = C::ROW_BYTES, ES = sizeof(T);
+  constexpr int BK = ROW_BYTES / ES;  // k values of a stage row: 64 bf16 or 32 floats
   const int64_t nk = K / BK;
   const uint32_t lds0 = lds_offset(&sm.stage[0][0]);
   // Per-lane offsets of the tile's loads, fixed for the whole k loop. The empty asm
@@ -215,7 +239,7 @@ __device__ __forceinline__ void mainloop(Tile& t, Smem<C>& sm, const bf16_t* aba
   uint32_t off[C::kLoadsPerTile];
 #pragma unroll
   for (int q = 0; q < C::kLoadsPerTile; ++q) {
-    off[q] = q < C::kLoadsA ? lane_offset<C>(ld, m0a, M, q) : lane_offset<C>(ld, m0b, M, q - C::kLoadsA);
+    off[q] = q < C::kLoadsA ? lane_offset<C, ES>(ld, m0a, M, q) : lane_offset<C, ES>(ld, m0b, M, q - C::kLoadsA);
     asm volatile("" : "+v"(off[q]));
   }
   auto issue_q = [&](int64_t kt, uint32_t st, int q) {
@@ -235,8 +259,8 @@ __device__ __forceinline__ void mainloop(Tile& t, Smem<C>& sm, const bf16_t* aba
     const int64_t kn = kt + NS - 1 < nk ? kt + NS - 1 : nk - 1;
     const uint32_t dst = lds0 + (stage == 0 ? NS - 1 : stage - 1) * C::kStageBytes;
     const unsigned char* st = sm.stage[stage];
-    t.template mma<C, C::kLoadsPerTile>(st, st + C::BM * ROW_BYTES, wm0, wn0,
-                                        [&](int q) { issue_q(kn, dst, q); });
+    t.template mma<C, C::kLoadsPerTile, T>(st, st + C::BM * ROW_BYTES, wm0, wn0,
+                                           [&](int q) { issue_q(kn, dst, q); });
     stage = stage + 1 == NS ? 0 : stage + 1;
   }
   wait_and_barrier<0>();  // the ring may be reused by the caller's next main loop

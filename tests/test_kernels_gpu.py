@@ -389,7 +389,13 @@ GHOST_SHAPES = [
 GHOST_ROUTES = [None, "gram", "direct"]
 
 
-@pytest.mark.parametrize("n,T,fin,fout", GHOST_SHAPES + [(3, 200, 256, 16), (2, 130, 8, 520)])
+@pytest.mark.parametrize(
+    "n,T,fin,fout",
+    GHOST_SHAPES
+    + [(3, 200, 256, 16), (2, 130, 8, 520)]  # thin layers: the direct route by choice
+    # feature sizes that are multiples of 32: the direct-load kernel on fp32 operands (route "gram")
+    + [(3, 200, 64, 96), (2, 300, 160, 288), (5, 1000, 32, 64)],
+)
 @pytest.mark.parametrize("scale", [1.0, 4.0])
 @pytest.mark.parametrize("route", GHOST_ROUTES)
 def test_linear_ghost_norm_f32(K, n, T, fin, fout, scale, route, monkeypatch):
