@@ -127,14 +127,14 @@ constexpr bool ghost_cfg_has_quadrants() {
   return C::BM == 128 && C::BN == 128 && C::BK == 64 && C::kWaves == 4 && C::kStages == 2;
 }
 
-// TE: bf16_t, or float (whole-tile blocks only; a stage row of 128 bytes is then 32 k values).
+// TE: bf16_t, or float (a stage row of 128 bytes is then 32 k values).
 template <class C, typename TE = bf16_t>
 __global__ __launch_bounds__(C::kThreads) void ghost_norm_bf16_dlds_kernel(
     const TE* __restrict__ b, const TE* __restrict__ a, float* __restrict__ pw,
     float* __restrict__ pb, int64_t T, int64_t Dout, int64_t Din, int nJ, int npairs, uint32_t nbig,
     int slots) {
   constexpr int R = C::BM / C::BN;
-  constexpr bool kQuadrants = ghost_cfg_has_quadrants<C>() && std::is_same<TE, bf16_t>::value;
+  constexpr bool kQuadrants = ghost_cfg_has_quadrants<C>();
   __shared__ mb16d::Smem<C> sm;
   __shared__ float red[C::kWaves];
   const bool big = !kQuadrants || blockIdx.x < nbig;
@@ -195,12 +195,12 @@ __global__ __launch_bounds__(C::kThreads) void ghost_norm_bf16_dlds_kernel(
     if (m0a < T && m0b < T) {  // block-uniform
       mb16d::Tile t;
       t.clear();
-      mb16d::mainloop_splitk<C>(t, sm, bs, bs, Dout, m0a, m0b, T, Dout);
+      mb16d::mainloop_splitk<C, TE>(t, sm, bs, bs, Dout, m0a, m0b, T, Dout);
       const mb16d::floatx16 g = mb16d::splitk_reduce<C>(t, sm);
       mb16d::floatx16 h;
       if (pw) {
         t.clear();
-        mb16d::mainloop_splitk<C>(t, sm, as, as, Din, m0a, m0b, T, Din);
+        mb16d::mainloop_splitk<C, TE>(t, sm, as, as, Din, m0a, m0b, T, Din);
         h = mb16d::splitk_reduce<C>(t, sm);
       }
       const int rmax = static_cast<int>(T - m0a < 64 ? T - m0a : 64);
@@ -275,8 +275,7 @@ int tile_edge(int64_t T) { return T > 64 ? 128 : 64; }
 // The Gram route costs 2 T'^2 (in + out) multiply-adds per sample over the tile pairs it
 // visits, forming the gradient and squaring it 2 T in out: for thin layers (a low-rank
 // adapter, a narrow head) the second is far cheaper although the gradient tile exists for a
-// moment in registers. The two routes run at about the same rate for bf16; for fp32 the
-// contraction kernel is the faster of the two by a sixth.
+// moment in registers.
 // DPK_GHOST_NORM_ROUTE=gram|direct in the environment overrides the choice (for tests that
 // want both routes on the same shapes).
 bool direct_is_cheaper(int dtype, int64_t T, int64_t out, int64_t in) {
@@ -288,7 +287,8 @@ bool direct_is_cheaper(int dtype, int64_t T, int64_t out, int64_t in) {
   const int64_t nt = dpk_cdiv(T, B);
   const double gram = static_cast<double>(nt * (nt + 1) / 2) * B * B * static_cast<double>(in + out);
   const double direct = static_cast<double>(T) * static_cast<double>(in) * static_cast<double>(out);
-  return direct < (dtype == DPK_F32 ? 1.1 : 0.9) * gram;
+  (void)dtype;  // the two routes run at about the same rate for either element type
+  return direct < 0.9 * gram;
 }
 
 struct DirectLayout {
@@ -309,7 +309,6 @@ extern "C" size_t dpk_linear_ghost_norm_workspace_bytes(int64_t n, int64_t T, in
   // quadrant slots each (2 m^2 + 2 m slots per sample covers both).
   const int64_t m = dpk_cdiv(T, 128);
   const size_t gram = dpk_align_up(static_cast<size_t>(2 * n * (2 * m * m + 2 * m)) * sizeof(float), 256);
-  // whichever dtype: the caller does not say, and the fp32 rule takes every shape the bf16 rule takes
   const size_t direct = direct_is_cheaper(DPK_F32, T, out, in) ? direct_layout(n, T, out, in).total : 0;
   return gram > direct ? gram : direct;
 }
@@ -376,7 +375,7 @@ extern "C" int dpk_linear_ghost_norm(const void* b, const void* a, int dtype, fl
   // tile block per CU runs latency-bound and takes most of a full round's time, a
   // round of quadrant blocks about a third of it.
   int64_t tail = 0;
-  if (dlds && dtype == DPK_BF16 && ghost_cfg_has_quadrants<GhostCfg>()) {
+  if (dlds && ghost_cfg_has_quadrants<GhostCfg>()) {
     const int cus = dpk_device_cus();
     DPK_REQUIRE(cus > 0, DPK_E_LAUNCH, "%s: cannot query the device", who);
     const int64_t resident = 2 * static_cast<int64_t>(cus);
@@ -398,7 +397,7 @@ extern "C" int dpk_linear_ghost_norm(const void* b, const void* a, int dtype, fl
     hipLaunchKernelGGL((ghost_norm_bf16_dlds_kernel<GhostCfg, float>), dim3(static_cast<unsigned>(grid_blocks)),
                        dim3(GhostCfg::kThreads), 0, s, static_cast<const float*>(b), static_cast<const float*>(a),
                        pw, pb, T, out, in, (int)dpk_cdiv(T, GhostCfg::BN), (int)npairs,
-                       static_cast<uint32_t>(blocks), slots);
+                       static_cast<uint32_t>(blocks - tail), slots);
   } else if (dtype == DPK_F32) {
     const bool vec = out % 4 == 0 && in % 4 == 0 && dpk_aligned(b, 16) && dpk_aligned(a, 16);
     const float* bp = static_cast<const float*>(b);

@@ -272,13 +272,16 @@ __device__ __forceinline__ void mainloop(Tile& t, Smem<C>& sm, const T* abase,
 // 64 x 64 tile, wave w takes the w-th 16-wide k slice of every stage, and the
 // partial tiles are summed through LDS afterwards. Same swizzle; a stage holds 64 A
 // rows then 64 B rows (16 KB).
-template <class C>
-__device__ __forceinline__ void mainloop_splitk(Tile& t, Smem<C>& sm, const bf16_t* abase,
-                                                const bf16_t* bbase, int64_t ld, int64_t m0a,
+template <class C, typename T = bf16_t>
+__device__ __forceinline__ void mainloop_splitk(Tile& t, Smem<C>& sm, const T* abase,
+                                                const T* bbase, int64_t ld, int64_t m0a,
                                                 int64_t m0b, int64_t M, int64_t K) {
   static_assert(C::BK == 64 && C::kWaves == 4 && C::kStages == 2,
-                "split-k small tile: one 16-wide k slice per wave, two stages");
-  constexpr int BK = C::BK, ROW_BYTES = C::ROW_BYTES;
+                "split-k small tile: one 32-byte k slice per wave, two stages");
+  constexpr int ROW_BYTES = C::ROW_BYTES, ES = sizeof(T);
+  constexpr int BK = ROW_BYTES / ES;  // k values of a stage row: 64 bf16 or 32 floats
+  constexpr bool kF32 = std::is_same<T, float>::value;
+  typedef typename std::conditional<kF32, floatx4, bf16x8>::type frag_t;
   constexpr int kLoads = 2 * 64 * ROW_BYTES / 1024 / C::kWaves;  // per wave and stage: 4
   constexpr int kHalf = kLoads / 2;                              // the first half fetch A rows
   const int64_t nk = K / BK;
@@ -289,7 +292,7 @@ __device__ __forceinline__ void mainloop_splitk(Tile& t, Smem<C>& sm, const bf16
 #pragma unroll
   for (int q = 0; q < kLoads; ++q) {
     // group q * kWaves + wave of the stage image; groups 0..7 are A rows, 8..15 B rows
-    off[q] = q < kHalf ? lane_offset<C>(ld, m0a, M, q) : lane_offset<C>(ld, m0b, M, q - kHalf);
+    off[q] = q < kHalf ? lane_offset<C, ES>(ld, m0a, M, q) : lane_offset<C, ES>(ld, m0b, M, q - kHalf);
     asm volatile("" : "+v"(off[q]));
   }
   auto issue = [&](int64_t kt, uint32_t st) {
@@ -315,19 +318,29 @@ __device__ __forceinline__ void mainloop_splitk(Tile& t, Smem<C>& sm, const bf16
     issue(kn, lds0 + ((stage + kRing - 1) & (kRing - 1)) * kSmallStage);
     const unsigned char* As = &sm.stage[0][0] + stage * kSmallStage;
     const unsigned char* Bs = As + 64 * ROW_BYTES;
-    bf16x8 av[2], bv[2];
+    frag_t av[2], bv[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int row = i * 32 + l32;
-      av[i] = *reinterpret_cast<const bf16x8*>(As + row * ROW_BYTES + swz<C>(row, wave * 2 + kh) * 16);
-      bv[i] = *reinterpret_cast<const bf16x8*>(Bs + row * ROW_BYTES + swz<C>(row, wave * 2 + kh) * 16);
+      av[i] = *reinterpret_cast<const frag_t*>(As + row * ROW_BYTES + swz<C>(row, wave * 2 + kh) * 16);
+      bv[i] = *reinterpret_cast<const frag_t*>(Bs + row * ROW_BYTES + swz<C>(row, wave * 2 + kh) * 16);
     }
     __builtin_amdgcn_sched_barrier(0);
+    if constexpr (kF32) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+      for (int e = 0; e < 4; ++e)
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
-        t.acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[i], bv[j], t.acc[i][j], 0, 0, 0);
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+            t.acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i][e], bv[j][e], t.acc[i][j], 0, 0, 0);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          t.acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[i], bv[j], t.acc[i][j], 0, 0, 0);
+    }
     __builtin_amdgcn_sched_barrier(0);
     stage = (stage + 1) & (kRing - 1);
   }

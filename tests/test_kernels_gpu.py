@@ -394,7 +394,9 @@ GHOST_ROUTES = [None, "gram", "direct"]
     GHOST_SHAPES
     + [(3, 200, 256, 16), (2, 130, 8, 520)]  # thin layers: the direct route by choice
     # feature sizes that are multiples of 32: the direct-load kernel on fp32 operands (route "gram")
-    + [(3, 200, 64, 96), (2, 300, 160, 288), (5, 1000, 32, 64)],
+    + [(3, 200, 64, 96), (2, 300, 160, 288), (5, 1000, 32, 64)]
+    # ... with a tail of quadrant blocks: few units (all quadrants), 576 units (512 whole tiles + 256 quadrants)
+    + [(2, 256, 512, 256), (3, 150, 64, 64), (16, 1000, 64, 128)],
 )
 @pytest.mark.parametrize("scale", [1.0, 4.0])
 @pytest.mark.parametrize("route", GHOST_ROUTES)
