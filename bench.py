@@ -468,6 +468,14 @@ def kernel_table(dev, iters: int = 10, warm: int = 3, with_cpu: bool = True):
                       ms, "mfma_bf16", 2.0 * n * (direct if thin else gram),
                       cpu(lambda: O.linear_norm_sample(ca, cb), n, f"1 of {n} samples, bf16 bmm Grams"))
             del a, b
+    # the same kernel on fp32 operands
+    tri, full = tri_tiles(1024)
+    a = torch.randn(16, 1024, 2048, device=dev)
+    b = torch.randn(16, 1024, 2048, device=dev) * 0.02
+    yield row("linear_ghost_norm", "a2", "C5 q/o shape in fp32: n=16 T=1024 2048->2048 f32",
+              timed(lambda: K.linear_ghost_norm(b, a, want_weight=True, want_bias=False)), "mfma_fp32",
+              2.0 * 16 * 1024 * 1024 * 4096 * tri / full)
+    del a, b
     # a low-rank adapter on C5's width: the direct route
     a = torch.randn(16, 1024, 2048, device=dev).bfloat16()
     b = (torch.randn(16, 1024, 16, device=dev) * 0.02).bfloat16()
