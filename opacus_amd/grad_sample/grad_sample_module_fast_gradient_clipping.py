@@ -37,6 +37,7 @@ import torch.nn as nn
 from .. import kernels
 from ..utils.module_utils import requires_grad, trainable_modules, trainable_parameters
 from ._common import cached_sumsq
+from .linear import compute_linear_grad_sample as linear_grad_sampler
 from .grad_sample_module import (
     GradSampleHooks,
     call_sampler,
@@ -306,7 +307,7 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
             c = coef.to(device=backprops.device, dtype=torch.float32)
             if n == 0:
                 continue
-            if isinstance(module, nn.Linear):
+            if self._sampler_for(module) is linear_grad_sampler:  # nn.Linear itself and RNNLinear, not a subclass with a forward of its own
                 a = activations[0].to(backprops.dtype)
                 w = (c * scale).to(backprops.dtype).view(n, *([1] * (backprops.dim() - 1)))
                 if module.bias is None and a.shape[-1] < backprops.shape[-1]:
