@@ -37,7 +37,6 @@ import torch.nn as nn
 from .. import kernels
 from ..utils.module_utils import requires_grad, trainable_modules, trainable_parameters
 from ._common import cached_sumsq
-from .linear import compute_linear_grad_sample as linear_grad_sampler
 from .grad_sample_module import (
     GradSampleHooks,
     call_sampler,
@@ -290,6 +289,8 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
         """Adds ``sum_n coef[n] * grad_n`` of every layer seen by the last backward pass to
         ``p.grad``, from the kept (activations, backprops): what the second backward pass of
         ``sum_n coef[n] * loss[n]`` leaves there (fast_gradient_clipping_utils.py:193-201)."""
+        from .linear import compute_linear_grad_sample as linear_grad_sampler  # imports this module's package
+
         kept, self._kept_passes = self._kept_passes, []
         sums = {}
 
