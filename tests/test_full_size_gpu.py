@@ -119,6 +119,40 @@ def test_ghost_norm_full_size(K, n, T, fin, fout, check):
     assert rel_err(nb, b.double().sum(1).norm(dim=1)) < 1e-4
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("n,T,fin,fout", [(16, 1024, 2048, 1024), (8, 1000, 2048, 5632)])
+def test_linear_grad_sample_with_sequence_full_size(K, dtype, n, T, fin, fout):
+    """The materialising counterpart of the ghost norms at C5's layer shapes (hooks mode on a
+    sequence model): per-sample weight gradients contracted over T by the direct-load kernels."""
+    torch.manual_seed(T + fout)
+    a = torch.randn(n, T, fin, device="cuda").to(dtype)
+    b = (torch.randn(n, T, fout, device="cuda") * 0.02).to(dtype)
+    gs, sumsq = K.linear_grad_sample(b, a)
+    assert gs.shape == (n, fout, fin) and gs.dtype == dtype and sumsq.dtype == torch.float32
+    tol = FP32_REL if dtype == torch.float32 else 2 ** -8  # one rounding to bf16 on the way out
+    # the oracle (float64 einsum) on two samples: samples are independent
+    want, _ = O.linear_grad_sample(a[:2].cpu().double(), b[:2].cpu().double())
+    assert rel_err(gs[:2], want) < tol
+    # the squared norms are those of the fp32 accumulators, before any rounding of gs
+    assert rel_err(sumsq[:2], want.flatten(1).pow(2).sum(1)) < 1e-5
+    # and they are the ghost norms of the same layer
+    nw, _ = K.linear_ghost_norm(b, a, want_weight=True, want_bias=False)
+    assert rel_err(sumsq.sqrt(), nw) < 1e-4
+    # exact scaling: doubling the backprops doubles every accumulator exactly
+    gs2, sumsq2 = K.linear_grad_sample((b.float() * 2).to(dtype), a)
+    assert torch.equal(gs2.float(), 2 * gs.float()) and torch.equal(sumsq2, 4 * sumsq)
+    # invariance under a permutation of the positions t (fp32 sums in another order)
+    perm = torch.randperm(T, device="cuda")
+    gsp, sumsqp = K.linear_grad_sample(b[:, perm].contiguous(), a[:, perm].contiguous())
+    assert rel_err(gsp, gs) < (FP32_REL if dtype == torch.float32 else 2 ** -7) and rel_err(sumsqp, sumsq) < FP32_REL
+    # additivity in the backprops, in fp32 outputs so that no rounding to bf16 interferes
+    h = T // 2
+    g1, _ = K.linear_grad_sample(b[:, :h].contiguous(), a[:, :h].contiguous(), out_dtype=torch.float32)
+    g2, _ = K.linear_grad_sample(b[:, h:].contiguous(), a[:, h:].contiguous(), out_dtype=torch.float32)
+    gf, _ = K.linear_grad_sample(b, a, out_dtype=torch.float32)
+    assert rel_err(g1 + g2, gf) < FP32_REL
+
+
 # ---- C4: Conv2d 64 -> 64, 3 x 3, 32 x 32 images, batch 256, fp32 ------------------------------
 def test_c4_conv_and_group_norm_full_size(K):
     n = 256
