@@ -91,7 +91,10 @@ int dpk_linear_bias_gs(const void* b, int in_dtype, void* gs_bias, int gs_dtype,
  * Either output may be NULL (parameter without requires_grad). Outputs are
  * fp32 whatever `dtype` the inputs have. The T x T Gram matrices are never
  * written to memory: matching tiles of b b^T and a a^T are formed in MFMA
- * accumulators, multiplied and reduced in registers. */
+ * accumulators, multiplied and reduced in registers. A layer thin enough that
+ * T * in * out is below the work of the two Grams has the tiles of
+ * sum_t b_t a_t^T formed and squared instead (never stored either); the
+ * results agree to rounding. ws must be 256-byte aligned. */
 size_t dpk_linear_ghost_norm_workspace_bytes(int64_t n, int64_t T, int64_t out, int64_t in);
 int dpk_linear_ghost_norm(const void* b, const void* a, int dtype, float* norm_w, float* norm_b,
                           int64_t n, int64_t T, int64_t out, int64_t in, float scale, void* ws,
