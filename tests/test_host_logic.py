@@ -898,3 +898,17 @@ def test_multihead_attention_equals_torch_module_and_shares_its_state_dict(batch
 def test_package_surface():
     for name in opacus_amd.__all__:
         assert hasattr(opacus_amd, name)
+
+
+# ---- bench.py command line ------------------------------------------------------------------------
+def test_bench_refuses_more_than_one_gpu():
+    """One GPU is all this build measures: a larger --gpus must end at once with a message
+    that says so, before anything touches a device."""
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    bench = Path(__file__).resolve().parents[1] / "bench.py"
+    done = subprocess.run([sys.executable, str(bench), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert done.returncode != 0
+    assert "one GPU" in (done.stdout + done.stderr)
