@@ -69,6 +69,7 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
 
     NORM_SAMPLERS = {}
     CAN_SKIP_AUTOGRAD_WEIGHT_GRADS = False  # the second backward pass is autograd's
+    KEEP_GRAD_SAMPLES_BELOW = 1 << 22  # elements per layer and pass, single_backward only
 
     def __init__(
         self,
@@ -256,9 +257,10 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
             activations, backprops = stacked
             for _, p in trainable_parameters(module):
                 p._forward_counter += 1  # taken off again below, as for a module used once
-        if self.single_backward:
-            self._kept_passes.append((module, activations, backprops, scale))
-        if self.use_ghost_clipping and type(module) in self.NORM_SAMPLERS:
+        ghost = self.use_ghost_clipping and type(module) in self.NORM_SAMPLERS
+        if self.single_backward and ghost:
+            self._kept_passes.append((module, activations, backprops, scale, None))
+        if ghost:
             norm_samples = call_sampler(self.NORM_SAMPLERS[type(module)], module, activations, backprops, scale)
             for param, ns in norm_samples.items():
                 if param.requires_grad:
@@ -269,6 +271,13 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
         else:
             sampler = self._sampler_for(module)
             grad_samples = call_sampler(sampler, module, activations, backprops, scale)
+            if self.single_backward:
+                # small per-sample gradients (norm layers, biases) are kept as they are; large
+                # ones are formed again when the coefficients exist
+                small = sum(gs.numel() for gs in grad_samples.values()) <= self.KEEP_GRAD_SAMPLES_BELOW
+                # (copies: a tensor adopted as p._current_grad_sample has later uses of the module added into it)
+                kept_gs = {p: gs.clone() for p, gs in grad_samples.items()} if small else None
+                self._kept_passes.append((module, activations, backprops, scale, kept_gs))
             adopt = getattr(sampler, "owns_output", False)
             for param, gs in grad_samples.items():
                 create_or_accumulate_grad_sample(
@@ -303,7 +312,7 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
             else:
                 sums[id(param)] = (param, value)
 
-        for module, activations, backprops, scale in kept:
+        for module, activations, backprops, scale, grad_samples in kept:
             n = backprops.shape[0]
             c = coef.to(device=backprops.device, dtype=torch.float32)
             if n == 0:
@@ -335,7 +344,8 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
                     ),
                 )
             else:
-                grad_samples = call_sampler(self._sampler_for(module), module, activations, backprops, scale)
+                if grad_samples is None:
+                    grad_samples = call_sampler(self._sampler_for(module), module, activations, backprops, scale)
                 for param, gs in grad_samples.items():
                     if not param.requires_grad:
                         continue

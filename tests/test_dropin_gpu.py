@@ -871,14 +871,15 @@ def _ghost_grads(A, net, batch, loss_call, *, single, steps=2, C=0.05, reduction
     return [p.grad.detach().clone() for p in ghost.parameters()], ghost
 
 
-@pytest.mark.parametrize("case", ["mlp_mean", "mlp_sum", "llama", "llama_tied", "cnn", "lstm"])
+@pytest.mark.parametrize("case", ["mlp_mean", "mlp_sum", "llama", "llama_tied", "cnn", "lstm", "norm_twice"])
 def test_ghost_single_backward_leaves_the_second_pass_gradients(A, case):
     """single_backward=True forms the clipped gradient sum from what the hooks kept of the first
     backward pass. It must equal what the reference's second pass of sum_n coef[n] loss[n]
     (fast_gradient_clipping_utils.py:193-201) leaves in p.grad: Linear with and without a
     sequence dimension and bias, Embedding with repeated ids, RMSNorm / GroupNorm / Conv2d
-    through their grad samplers, a table tied to the LM head, and a layer whose uses are
-    stacked (the recurrent projection of an LSTM)."""
+    through their grad samplers, a table tied to the LM head, a layer whose uses are
+    stacked (the recurrent projection of an LSTM), and a LayerNorm applied twice in one pass
+    (its two per-sample gradients are kept apart and both counted once)."""
     torch.manual_seed(21)
     reduction = "sum" if case == "mlp_sum" else "mean"
     if case.startswith("mlp"):
@@ -910,6 +911,23 @@ def test_ghost_single_backward_leaves_the_second_pass_gradients(A, case):
 
         def loss_call(model, opt, b):
             return A.DPLossFastGradientClipping(model, opt, nn.CrossEntropyLoss(), "mean")(model(b[0]), b[1])
+
+    elif case == "norm_twice":
+
+        class TwoUses(nn.Module):
+            def __init__(self):
+                super().__init__()
+                self.ln = nn.LayerNorm(12)
+                self.fc = nn.Linear(12, 12)
+
+            def forward(self, x):
+                return self.ln(self.fc(self.ln(x)))
+
+        net = TwoUses()
+        batch = (torch.randn(6, 5, 12), torch.randn(6, 5, 12))
+
+        def loss_call(model, opt, b):
+            return A.DPLossFastGradientClipping(model, opt, PerSampleMSE("mean"), "mean")(model(b[0]), b[1])
 
     else:
         from opacus_amd.layers import DPLSTM
