@@ -238,21 +238,34 @@ constexpr int64_t kWideSpan = static_cast<int64_t>(kThreads) * kWideChunks * 4; 
 typedef int span_vi4 __attribute__((ext_vector_type(4)));
 typedef int span_vi2 __attribute__((ext_vector_type(2)));
 template <typename T> struct span_io;
+// raw_t: the four elements as loaded.
 template <> struct span_io<float> {
-  static __device__ __forceinline__ float4 load4_nt(__amdgpu_buffer_rsrc_t row, uint32_t lane_bytes, int chunk_bytes) {
-    const span_vi4 r = __builtin_amdgcn_raw_buffer_load_b128(row, lane_bytes, chunk_bytes, 2);
+  typedef span_vi4 raw_t;
+  static __device__ __forceinline__ raw_t load_raw_nt(__amdgpu_buffer_rsrc_t row, uint32_t lane_bytes, int chunk_bytes) {
+    return __builtin_amdgcn_raw_buffer_load_b128(row, lane_bytes, chunk_bytes, 2);
+  }
+  static __device__ __forceinline__ float4 unpack(raw_t r) {
     return make_float4(__int_as_float(r.x), __int_as_float(r.y), __int_as_float(r.z), __int_as_float(r.w));
+  }
+  static __device__ __forceinline__ float4 load4_nt(__amdgpu_buffer_rsrc_t row, uint32_t lane_bytes, int chunk_bytes) {
+    return unpack(load_raw_nt(row, lane_bytes, chunk_bytes));
   }
 };
 template <> struct span_io<bf16_t> {
-  static __device__ __forceinline__ float4 load4_nt(__amdgpu_buffer_rsrc_t row, uint32_t lane_bytes, int chunk_bytes) {
-    const span_vi2 r = __builtin_amdgcn_raw_buffer_load_b64(row, lane_bytes, chunk_bytes, 2);
+  typedef span_vi2 raw_t;
+  static __device__ __forceinline__ raw_t load_raw_nt(__amdgpu_buffer_rsrc_t row, uint32_t lane_bytes, int chunk_bytes) {
+    return __builtin_amdgcn_raw_buffer_load_b64(row, lane_bytes, chunk_bytes, 2);
+  }
+  static __device__ __forceinline__ float4 unpack(raw_t r) {
     float4 v;
     v.x = __uint_as_float(static_cast<uint32_t>(r.x) << 16);
     v.y = __uint_as_float(static_cast<uint32_t>(r.x) & 0xffff0000u);
     v.z = __uint_as_float(static_cast<uint32_t>(r.y) << 16);
     v.w = __uint_as_float(static_cast<uint32_t>(r.y) & 0xffff0000u);
     return v;
+  }
+  static __device__ __forceinline__ float4 load4_nt(__amdgpu_buffer_rsrc_t row, uint32_t lane_bytes, int chunk_bytes) {
+    return unpack(load_raw_nt(row, lane_bytes, chunk_bytes));
   }
 };
 
@@ -270,21 +283,25 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   float4 acc[kWideChunks];
 #pragma unroll
   for (int v = 0; v < kWideChunks; ++v) acc[v] = make_float4(0.f, 0.f, 0.f, 0.f);
+  typedef typename span_io<TG>::raw_t raw_t;
+  // One row at a time; its loads stay as loaded until every one of them is issued (an
+  // unpacking of bf16 pairs placed next to each load would have the wave wait for that
+  // load before it asks for the next).
   for (int64_t r = 0; r < n; ++r, row += stride) {
     const float c = clip[r];
-    float4 x[kWideChunks];
-    // descriptor of this block's span of row r: raw bytes, bounds = the span
+    raw_t x[kWideChunks];
     const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<TG*>(row), 0, kWideChunks * kChunkBytes, 0x00020000);
 #pragma unroll
     for (int v = 0; v < kWideChunks; ++v)
-      x[v] = span_io<TG>::load4_nt(rsrc, lane * static_cast<uint32_t>(sizeof(TG)), v * kChunkBytes);
+      x[v] = span_io<TG>::load_raw_nt(rsrc, lane * static_cast<uint32_t>(sizeof(TG)), v * kChunkBytes);
 #pragma unroll
     for (int v = 0; v < kWideChunks; ++v) {
-      acc[v].x = fmaf(c, x[v].x, acc[v].x);
-      acc[v].y = fmaf(c, x[v].y, acc[v].y);
-      acc[v].z = fmaf(c, x[v].z, acc[v].z);
-      acc[v].w = fmaf(c, x[v].w, acc[v].w);
+      const float4 f = span_io<TG>::unpack(x[v]);
+      acc[v].x = fmaf(c, f.x, acc[v].x);
+      acc[v].y = fmaf(c, f.y, acc[v].y);
+      acc[v].z = fmaf(c, f.z, acc[v].z);
+      acc[v].w = fmaf(c, f.w, acc[v].w);
     }
   }
   TO* out = static_cast<TO*>(a.out[k]) + span0;
