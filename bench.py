@@ -424,6 +424,12 @@ def kernel_table(dev, iters: int = 10, warm: int = 3, with_cpu: bool = True):
     yield row("clip_accumulate", "a10", "C2 n=128 P=16.8M f32", timed(lambda: K.clip_accumulate([gs], clip, [out], False)),
               "hbm", gs.numel() * 4 + out.numel() * 4,
               cpu(lambda: O.clip_and_accumulate([cgs], 1.0), 16, "8 of 128 samples, norm + clip + einsum"))
+    gs16 = gs.bfloat16()  # the same tensor as a bf16 model's hooks would hold it
+    out16 = torch.empty(d, d, device=dev, dtype=torch.bfloat16)
+    yield row("clip_accumulate", "a10", "C2 shape in bf16: n=128 P=16.8M", timed(lambda: K.clip_accumulate([gs16], clip, [out16], False)),
+              "hbm", gs16.numel() * 2 + out16.numel() * 2)
+    yield row("sumsq_rows", "a10", "C2 shape in bf16: n=128 P=16.8M", timed(lambda: K.sumsq_rows([gs16])), "hbm", gs16.numel() * 2)
+    del gs16, out16
     g = torch.empty_like(out)
     csum = torch.zeros(d, d) if with_cpu else None
     yield row("add_noise", "a11", "C2 P=16.8M f32", timed(lambda: K.add_noise(out, g, 1.0, 128.0, 1, 0)), "hbm", 2 * out.numel() * 4,

@@ -72,6 +72,11 @@ template <> struct dpk_io<float> {
     const dpk_vf4 v = __builtin_nontemporal_load(reinterpret_cast<const dpk_vf4*>(p));
     return make_float4(v.x, v.y, v.z, v.w);
   }
+  // The same four elements as loaded, to be unpacked later: a kernel that wants many loads
+  // in flight issues them all as raw4 and unpacks once they are all on their way.
+  typedef dpk_vf4 raw4;
+  static __device__ __forceinline__ raw4 load4_raw(const float* p) { return *reinterpret_cast<const dpk_vf4*>(p); }
+  static __device__ __forceinline__ float4 unpack4(raw4 v) { return make_float4(v.x, v.y, v.z, v.w); }
   static __device__ __forceinline__ float load(const float* p) { return *p; }
   static __device__ __forceinline__ void store(float* p, float v) { *p = v; }
   // 4 consecutive elements, p 16-byte aligned
@@ -95,6 +100,16 @@ template <> struct dpk_io<float> {
 template <> struct dpk_io<bf16_t> {
   static __device__ __forceinline__ float4 load4_nt(const bf16_t* p) {
     const dpk_vu2 r = __builtin_nontemporal_load(reinterpret_cast<const dpk_vu2*>(p));
+    float4 v;
+    v.x = __uint_as_float(r.x << 16);
+    v.y = __uint_as_float(r.x & 0xffff0000u);
+    v.z = __uint_as_float(r.y << 16);
+    v.w = __uint_as_float(r.y & 0xffff0000u);
+    return v;
+  }
+  typedef dpk_vu2 raw4;
+  static __device__ __forceinline__ raw4 load4_raw(const bf16_t* p) { return *reinterpret_cast<const dpk_vu2*>(p); }
+  static __device__ __forceinline__ float4 unpack4(raw4 r) {
     float4 v;
     v.x = __uint_as_float(r.x << 16);
     v.y = __uint_as_float(r.x & 0xffff0000u);

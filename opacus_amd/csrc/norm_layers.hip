@@ -299,11 +299,18 @@ __global__ __launch_bounds__(kThreads) void row_fused_kernel(const TIN* __restri
   for (int64_t t = t0 + wave; t < t1; t += kWaves) {
     const TIN* xr = x + (sample * T + t) * D + lane * 4;
     const TIN* br = b + (sample * T + t) * D + lane * 4;
+    // both rows are asked for before either is used: the row of b does not wait for the
+    // statistics of x
+    typename dpk_io<TIN>::raw4 xraw[NCH], braw[NCH];
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) xraw[c] = dpk_io<TIN>::load4_raw(xr + c * 256);
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) braw[c] = dpk_io<TIN>::load4_raw(br + c * 256);
     float4 xv[NCH];
     float sum = 0.f;
 #pragma unroll
     for (int c = 0; c < NCH; ++c) {
-      xv[c] = dpk_io<TIN>::load4(xr + c * 256);
+      xv[c] = dpk_io<TIN>::unpack4(xraw[c]);
       if (LN) sum += (xv[c].x + xv[c].y) + (xv[c].z + xv[c].w);
     }
     if (LN) {
@@ -328,7 +335,7 @@ __global__ __launch_bounds__(kThreads) void row_fused_kernel(const TIN* __restri
     const float r = 1.0f / sqrtf(ss / static_cast<float>(D) + eps);
 #pragma unroll
     for (int c = 0; c < NCH; ++c) {
-      const float4 bv = dpk_io<TIN>::load4(br + c * 256);
+      const float4 bv = dpk_io<TIN>::unpack4(braw[c]);
       acc[c].x = fmaf(xv[c].x * r, bv.x, acc[c].x);
       acc[c].y = fmaf(xv[c].y * r, bv.y, acc[c].y);
       acc[c].z = fmaf(xv[c].z * r, bv.z, acc[c].z);
