@@ -79,22 +79,36 @@ __global__ __launch_bounds__(kThreads) void linear_outer_kernel(
 // 5.7 TB/s. More chunks per thread or other block sizes measured slower.
 constexpr int kSeqThreads = 256;
 
-template <typename TIN, typename TOUT>
+// E: elements of a chunk, 4, or 8 for bf16 results (16 bytes a store either way: with
+// 8-byte stores the bf16 stream stopped at 5.3 TB/s).
+template <typename TIN, typename TOUT, int E>
 __global__ __launch_bounds__(kSeqThreads) void linear_outer_seq_kernel(
     const TIN* __restrict__ b, const TIN* __restrict__ a, TOUT* __restrict__ gs, uint32_t M,
-    uint32_t cols4, float scale, uint32_t blocks_per_sample) {
+    uint32_t cols, float scale, uint32_t blocks_per_sample) {
+  static_assert(E == 4 || (E == 8 && sizeof(TOUT) == 2), "one or two 4-element pieces; 16-byte stores at most");
   const uint32_t sample = blockIdx.x / blocks_per_sample;
   const uint32_t blk = blockIdx.x - sample * blocks_per_sample;
-  const uint32_t total = M * cols4;  // chunks per sample (< 2^32, checked by the host)
+  const uint32_t total = M * cols;  // chunks per sample (< 2^32, checked by the host)
   const TIN* bs = b + static_cast<int64_t>(sample) * M;
-  const TIN* as = a + static_cast<int64_t>(sample) * cols4 * 4;
-  TOUT* out = gs + static_cast<int64_t>(sample) * total * 4;
+  const TIN* as = a + static_cast<int64_t>(sample) * cols * E;
+  TOUT* out = gs + static_cast<int64_t>(sample) * total * E;
   const uint32_t p = blk * kSeqThreads + threadIdx.x;
   if (p >= total) return;
-  const uint32_t i = p / cols4, j4 = p - i * cols4;
+  const uint32_t i = p / cols, jc = p - i * cols;
   const float bv = scale * dpk_io<TIN>::load(bs + i);
-  const float4 av = dpk_io<TIN>::load4(as + j4 * 4);
-  dpk_io<TOUT>::store4_nt(out + static_cast<int64_t>(p) * 4, make_float4(bv * av.x, bv * av.y, bv * av.z, bv * av.w));
+  const float4 av = dpk_io<TIN>::load4(as + jc * E);
+  if constexpr (E == 4) {
+    dpk_io<TOUT>::store4_nt(out + static_cast<int64_t>(p) * 4, make_float4(bv * av.x, bv * av.y, bv * av.z, bv * av.w));
+  } else {
+    const float4 aw = dpk_io<TIN>::load4(as + jc * E + 4);
+    typedef uint32_t vu4 __attribute__((ext_vector_type(4)));
+    vu4 w;
+    w.x = f32x2_to_bf16x2(bv * av.x, bv * av.y);
+    w.y = f32x2_to_bf16x2(bv * av.z, bv * av.w);
+    w.z = f32x2_to_bf16x2(bv * aw.x, bv * aw.y);
+    w.w = f32x2_to_bf16x2(bv * aw.z, bv * aw.w);
+    __builtin_nontemporal_store(w, reinterpret_cast<vu4*>(out + static_cast<int64_t>(p) * 8));
+  }
 }
 
 // Sum of squares of a rank-one matrix: sum_ij (s b_i a_j)^2 = (sum_i (s b_i)^2)(sum_j a_j^2).
@@ -491,8 +505,16 @@ void launch_linear(const Plan& p, bool vec, const void* b, const void* a, void* 
                      scale, static_cast<uint32_t>(p.tiles_m), static_cast<uint32_t>(p.tiles_n))
     const int64_t cols4 = N / 4, chunks = M * cols4;
     const int64_t bps = dpk_cdiv(chunks, kSeqThreads);
-    if (vec && chunks < (1LL << 32) && n * bps <= DPK_MAX_GRID_X) {
-      hipLaunchKernelGGL((linear_outer_seq_kernel<TIN, TOUT>), dim3(static_cast<unsigned>(n * bps)),
+    const bool wide16 = sizeof(TOUT) == 2 && N % 8 == 0 && dpk_aligned(gs, 16);
+    if (vec && wide16 && n * dpk_cdiv(chunks / 2, kSeqThreads) <= DPK_MAX_GRID_X && chunks / 2 < (1LL << 32)) {
+      if constexpr (sizeof(TOUT) == 2) {
+        const int64_t bps8 = dpk_cdiv(chunks / 2, kSeqThreads);
+        hipLaunchKernelGGL((linear_outer_seq_kernel<TIN, TOUT, 8>), dim3(static_cast<unsigned>(n * bps8)),
+                           dim3(kSeqThreads), 0, s, bp, ap, gp, static_cast<uint32_t>(M), static_cast<uint32_t>(N / 8),
+                           scale, static_cast<uint32_t>(bps8));
+      }
+    } else if (vec && chunks < (1LL << 32) && n * bps <= DPK_MAX_GRID_X) {
+      hipLaunchKernelGGL((linear_outer_seq_kernel<TIN, TOUT, 4>), dim3(static_cast<unsigned>(n * bps)),
                          dim3(kSeqThreads), 0, s, bp, ap, gp, static_cast<uint32_t>(M), static_cast<uint32_t>(cols4), scale,
                          static_cast<uint32_t>(bps));
     } else if (vec) {
