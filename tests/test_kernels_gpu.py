@@ -469,6 +469,8 @@ CONV_CASES = [
     dict(n=2, C=64, O=64, k=(3, 3), stride=(1, 1), padding=(1, 1), dilation=(1, 1), groups=1, H=32, W=32),  # C4
     dict(n=2, C=24, O=160, k=(3, 3), stride=(1, 1), padding=(1, 1), dilation=(1, 1), groups=1, H=10, W=12),  # 128-tiles
     dict(n=2, C=16, O=16, k=(3, 3), stride=(1, 1), padding=(1, 1), dilation=(1, 1), groups=16, H=8, W=8),  # depthwise
+    dict(n=2, C=16, O=24, k=(3, 3), stride=(1, 1), padding=(1, 1), dilation=(1, 1), groups=1, H=56, W=56),  # a patch above 64 KB of LDS
+    dict(n=2, C=16, O=24, k=(3, 3), stride=(2, 2), padding=(1, 1), dilation=(1, 1), groups=1, H=56, W=52),
 ]
 
 
