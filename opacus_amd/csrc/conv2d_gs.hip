@@ -448,14 +448,10 @@ void launch(const Plan& p, bool vec, const void* x, const void* b, void* gs, flo
     // image rows made of whole, aligned 4-element chunks: the patch interior is staged with vector loads
     const int xvec = (g.W % 4 == 0 && dpk_aligned(x, sizeof(TIN) == 2 ? 8 : 16)) ? 1 : 0;
     if (patch_bytes > 64 * 1024 - 64) {
-      static bool told = false;  // per instantiation; setting it twice is harmless
-      if (!told) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&conv2d_gs_patch_kernel<64, 64, TIN, TOUT, true>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kPatchLdsLimit));
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&conv2d_gs_patch_kernel<64, 64, TIN, TOUT, false>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kPatchLdsLimit));
-        told = true;
-      }
+      // per device and cheap: said again at every such launch rather than remembered
+      const void* fn = vec ? reinterpret_cast<const void*>(&conv2d_gs_patch_kernel<64, 64, TIN, TOUT, true>)
+                           : reinterpret_cast<const void*>(&conv2d_gs_patch_kernel<64, 64, TIN, TOUT, false>);
+      (void)hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kPatchLdsLimit));
     }
     if (vec)
       hipLaunchKernelGGL((conv2d_gs_patch_kernel<64, 64, TIN, TOUT, true>), grid, block, patch_bytes, s, xp,
