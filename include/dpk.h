@@ -46,6 +46,12 @@ enum dpk_status {
 
 enum dpk_dtype { DPK_F32 = 0, DPK_BF16 = 1 };
 
+/* Two entry points choose between two kernels by cost. The caller may name the one it wants
+ * instead (tests drive both on one shape); every other caller passes the AUTO value. The
+ * library reads no environment variable and keeps no setting between calls. */
+enum dpk_linear_tile { DPK_TILE_AUTO = 0, DPK_TILE_128 = 128, DPK_TILE_256 = 256 };
+enum dpk_ghost_route { DPK_ROUTE_AUTO = 0, DPK_ROUTE_GRAM = 1, DPK_ROUTE_DIRECT = 2 };
+
 #define DPK_MULTI_MAX 48 /* tensors per call of the *_multi entry points */
 
 /* ABI revision; bumped when a signature changes. */
@@ -68,11 +74,13 @@ int dpk_device_cus(void);
  * T == 1 takes a store-bound outer-product kernel; T > 1 an MFMA kernel.
  * gs may be NULL when sumsq is given: only the squared norms are formed then
  * (the gradient tiles never leave the registers).
+ * tile: DPK_TILE_AUTO, or the block tile of the bf16 T > 1 kernel for shapes that kernel
+ * takes (ignored by the others).
  * ws is needed only when sumsq != NULL. */
 size_t dpk_linear_gs_workspace_bytes(int64_t n, int64_t T, int64_t out, int64_t in);
 int dpk_linear_gs(const void* b, const void* a, int in_dtype, void* gs, int gs_dtype,
                   float* sumsq, int64_t n, int64_t T, int64_t out, int64_t in, float scale,
-                  void* ws, size_t ws_bytes, dpk_stream_t stream);
+                  int tile, void* ws, size_t ws_bytes, dpk_stream_t stream);
 
 /* gs_bias[n,k] = scale * sum_t b[n,t,k]                   (linear.py:50)
  * sumsq (nullable, float[n]) receives sum_k gs_bias[n,k]^2 of the values as stored, for
@@ -94,11 +102,12 @@ int dpk_linear_bias_gs(const void* b, int in_dtype, void* gs_bias, int gs_dtype,
  * accumulators, multiplied and reduced in registers. A layer thin enough that
  * T * in * out is below the work of the two Grams has the tiles of
  * sum_t b_t a_t^T formed and squared instead (never stored either); the
- * results agree to rounding. ws must be 256-byte aligned. */
+ * results agree to rounding. route: DPK_ROUTE_AUTO (by cost), or the route to
+ * take. The workspace query covers either route. ws must be 256-byte aligned. */
 size_t dpk_linear_ghost_norm_workspace_bytes(int64_t n, int64_t T, int64_t out, int64_t in);
 int dpk_linear_ghost_norm(const void* b, const void* a, int dtype, float* norm_w, float* norm_b,
-                          int64_t n, int64_t T, int64_t out, int64_t in, float scale, void* ws,
-                          size_t ws_bytes, dpk_stream_t stream);
+                          int64_t n, int64_t T, int64_t out, int64_t in, float scale, int route,
+                          void* ws, size_t ws_bytes, dpk_stream_t stream);
 
 /* ------------------------------------------------------------------------- *
  * Per-sample gradients of nn.Conv2d (nn.Conv1d as a height-one image) and nn.Conv3d
@@ -159,23 +168,24 @@ int dpk_embedding_unique_pairs(const int64_t* ids, int64_t n, int64_t T, int64_t
 
 /* gs[n,v,:] = scale * sum_{t : ids[n,t]==v} b[n,t,:]        (embedding.py:48-61)
  * gs: [n,V,D] of gs_dtype, fully written (rows no id names are zero).
- * Ids outside [0,V) make the call fail with DPK_E_ARG after a device-side
- * check (the one entry point that waits for the stream). */
+ * An id outside [0,V) contributes nothing and nothing is written for it. status
+ * (nullable, device int32[1], the caller's): set to 1 when such an id is met and
+ * never cleared by the library, so that one flag can collect over many calls and
+ * be read back whenever the caller next waits for the stream anyway. */
 int dpk_embedding_gs(const int64_t* ids, const void* b, int in_dtype, void* gs, int gs_dtype,
-                     int64_t n, int64_t T, int64_t V, int64_t D, float scale, void* ws,
-                     size_t ws_bytes, dpk_stream_t stream);
+                     int64_t n, int64_t T, int64_t V, int64_t D, float scale, int32_t* status,
+                     void* ws, size_t ws_bytes, dpk_stream_t stream);
 
 /* nn.EmbeddingBag (embedding.py:67-94): bag i = index[offsets[i] : offsets[i+1]] (the
  * last one runs to L); gs[i, index[j], :] = scale * b[i,:] for every j of bag i, divided
  * by the bag length when `mean` != 0. An index that occurs several times in a bag still
  * receives b[i,:] once, as the reference's indexed "+=" leaves it. gs: [bags,V,D], fully
- * written, 16-byte aligned. Indices outside [0,V) or offsets that are not ascending in
- * [0,L] make the call fail with DPK_E_ARG after a device-side check (this entry point
- * waits for the stream). Workspace: dpk_embedding_bag_workspace_bytes(). */
-size_t dpk_embedding_bag_workspace_bytes(void);
+ * written, 16-byte aligned. Nothing is written for an index outside [0,V). status as for
+ * dpk_embedding_gs; it is also raised for offsets that are not ascending in [0,L] (the
+ * result is then unspecified but every access stays inside the tensors). */
 int dpk_embedding_bag_gs(const int64_t* index, const int64_t* offsets, const void* b, int in_dtype,
                          void* gs, int gs_dtype, int64_t bags, int64_t L, int64_t V, int64_t D,
-                         int mean, float scale, void* ws, size_t ws_bytes, dpk_stream_t stream);
+                         int mean, float scale, int32_t* status, dpk_stream_t stream);
 
 /* norm[n] = sqrt(sum_{v} || scale * sum_{t : ids[n,t]==v} b[n,t,:] ||^2)
  * (embedding_norm_sample.py:131-150). fp32 output. */

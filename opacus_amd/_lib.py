@@ -13,12 +13,14 @@ from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "lib" / "libdpsgd_hip.so"
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 DPK_OK = 0
 DPK_F32 = 0
 DPK_BF16 = 1
 DPK_MULTI_MAX = 48
+DPK_TILE_AUTO, DPK_TILE_128, DPK_TILE_256 = 0, 128, 256
+DPK_ROUTE_AUTO, DPK_ROUTE_GRAM, DPK_ROUTE_DIRECT = 0, 1, 2
 
 STATUS_NAMES = {
     0: "DPK_OK",
@@ -39,10 +41,10 @@ SIGNATURES = {
     "dpk_last_error": (c_char_p, []),
     "dpk_device_cus": (c_int, []),
     "dpk_linear_gs_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
-    "dpk_linear_gs": (c_int, [_P, _P, c_int, _P, c_int, _P, _I, _I, _I, _I, c_float, _P, c_size_t, _P]),
+    "dpk_linear_gs": (c_int, [_P, _P, c_int, _P, c_int, _P, _I, _I, _I, _I, c_float, c_int, _P, c_size_t, _P]),
     "dpk_linear_bias_gs": (c_int, [_P, c_int, _P, c_int, _P, _I, _I, _I, c_float, _P]),
     "dpk_linear_ghost_norm_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
-    "dpk_linear_ghost_norm": (c_int, [_P, _P, c_int, _P, _P, _I, _I, _I, _I, c_float, _P, c_size_t, _P]),
+    "dpk_linear_ghost_norm": (c_int, [_P, _P, c_int, _P, _P, _I, _I, _I, _I, c_float, c_int, _P, c_size_t, _P]),
     "dpk_conv2d_gs_workspace_bytes": (c_size_t, [_I, _I, _I, _I, _I, _I]),
     "dpk_conv2d_gs": (
         c_int,
@@ -56,11 +58,10 @@ SIGNATURES = {
     "dpk_conv_bias_gs": (c_int, [_P, c_int, _P, c_int, _P, _I, _I, _I, c_float, _P]),
     "dpk_embedding_workspace_bytes": (c_size_t, [_I, _I, _I]),
     "dpk_embedding_unique_pairs": (c_int, [_P, _I, _I, _P, _P, _P, _P, c_size_t, _P]),
-    "dpk_embedding_gs": (c_int, [_P, _P, c_int, _P, c_int, _I, _I, _I, _I, c_float, _P, c_size_t, _P]),
-    "dpk_embedding_bag_workspace_bytes": (c_size_t, []),
+    "dpk_embedding_gs": (c_int, [_P, _P, c_int, _P, c_int, _I, _I, _I, _I, c_float, _P, _P, c_size_t, _P]),
     "dpk_embedding_bag_gs": (
         c_int,
-        [_P, _P, _P, c_int, _P, c_int, _I, _I, _I, _I, c_int, c_float, _P, c_size_t, _P],
+        [_P, _P, _P, c_int, _P, c_int, _I, _I, _I, _I, c_int, c_float, _P, _P],
     ),
     "dpk_embedding_ghost_norm": (c_int, [_P, _P, c_int, _P, _I, _I, _I, c_float, _P, c_size_t, _P]),
     "dpk_tied_embedding_cross_workspace_bytes": (c_size_t, [_I, _I, _I, _I, c_int]),

@@ -444,15 +444,21 @@ void launch(const Plan& p, bool vec, const void* x, const void* b, void* gs, flo
   const TIN* xp = static_cast<const TIN*>(x);
   const TIN* bp = static_cast<const TIN*>(b);
   TOUT* gp = static_cast<TOUT*>(gs);
-  if (patch_bytes > 0) {
+  bool use_patch = patch_bytes > 0;
+  if (patch_bytes > 64 * 1024 - 64) {
+    // per device and cheap: said again at every such launch rather than remembered. A device
+    // or runtime that refuses that much LDS gets the gather kernel on the same 64 x 64 plan.
+    const void* fn = vec ? reinterpret_cast<const void*>(&conv2d_gs_patch_kernel<64, 64, TIN, TOUT, true>)
+                         : reinterpret_cast<const void*>(&conv2d_gs_patch_kernel<64, 64, TIN, TOUT, false>);
+    if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kPatchLdsLimit)) !=
+        hipSuccess) {
+      (void)hipGetLastError();  // the refusal is handled here, not reported by the next launch check
+      use_patch = false;
+    }
+  }
+  if (use_patch) {
     // image rows made of whole, aligned 4-element chunks: the patch interior is staged with vector loads
     const int xvec = (g.W % 4 == 0 && dpk_aligned(x, sizeof(TIN) == 2 ? 8 : 16)) ? 1 : 0;
-    if (patch_bytes > 64 * 1024 - 64) {
-      // per device and cheap: said again at every such launch rather than remembered
-      const void* fn = vec ? reinterpret_cast<const void*>(&conv2d_gs_patch_kernel<64, 64, TIN, TOUT, true>)
-                           : reinterpret_cast<const void*>(&conv2d_gs_patch_kernel<64, 64, TIN, TOUT, false>);
-      (void)hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kPatchLdsLimit));
-    }
     if (vec)
       hipLaunchKernelGGL((conv2d_gs_patch_kernel<64, 64, TIN, TOUT, true>), grid, block, patch_bytes, s, xp,
                          bp, gp, partials, g, C, O, groups, scale, p.tiles_m, p.tiles_n, Hp, Wp, xvec, 0);

@@ -25,7 +25,6 @@ struct EmbWs {
   int32_t* rank;
   int32_t* count;  // [n] distinct ids per sample
   int64_t* base;   // [n + 1] exclusive prefix of count
-  int32_t* flag;   // [1] set when an id is outside [0, V)
   float* partials;
 };
 
@@ -38,7 +37,7 @@ size_t ws_layout(int64_t n, int64_t T, int64_t D, void* ws, EmbWs* out) {
     return o;
   };
   const size_t o_next = take(nt * 4), o_leader = take(nt * 4), o_rank = take(nt * 4);
-  const size_t o_count = take(n * 4), o_base = take((n + 1) * 8), o_flag = take(4);
+  const size_t o_count = take(n * 4), o_base = take((n + 1) * 8);
   const int64_t tch = dpk_cdiv(T, kLeadersPerBlock), dch = dpk_cdiv(D > 0 ? D : 1, kThreads * 4);
   const size_t o_part = take(n * tch * dch * 4);
   if (out && ws) {
@@ -48,7 +47,6 @@ size_t ws_layout(int64_t n, int64_t T, int64_t D, void* ws, EmbWs* out) {
     out->rank = reinterpret_cast<int32_t*>(p + o_rank);
     out->count = reinterpret_cast<int32_t*>(p + o_count);
     out->base = reinterpret_cast<int64_t*>(p + o_base);
-    out->flag = reinterpret_cast<int32_t*>(p + o_flag);
     out->partials = reinterpret_cast<float*>(p + o_part);
   }
   return off;
@@ -104,7 +102,7 @@ __global__ __launch_bounds__(kThreads) void emb_link_kernel(const int64_t* __res
     }
     next[sample * T + t] = nxt < Ti ? nxt : -1;
     leader[sample * T + t] = before ? 0 : 1;
-    if (V > 0 && (mine < 0 || mine >= V)) *flag = 1;
+    if (flag && V > 0 && (mine < 0 || mine >= V)) *flag = 1;
   }
 }
 
@@ -248,11 +246,9 @@ __global__ __launch_bounds__(kThreads) void zero_fill_kernel(uint4* __restrict__
   if (blockIdx.x == 0 && threadIdx.x < ntail) tail[threadIdx.x] = 0;
 }
 
-__global__ void zero_flag_kernel(int32_t* flag) { *flag = 0; }
-
 // ---- EmbeddingBag ---------------------------------------------------------------
-// flag |= 1 when an index lies outside [0, V), an offset outside [0, L] or the
-// offsets decrease.
+// *flag = 1 when an index lies outside [0, V), an offset outside [0, L] or the
+// offsets decrease (never cleared here: the flag is the caller's and sticky).
 __global__ __launch_bounds__(kThreads) void bag_check_kernel(const int64_t* __restrict__ index,
                                                               const int64_t* __restrict__ offsets,
                                                               int64_t L, int64_t nbags, int64_t V,
@@ -287,8 +283,10 @@ __global__ __launch_bounds__(kThreads) void bag_scatter_kernel(
   const int64_t bag = lo;
   const int64_t end = bag + 1 < nbags ? offsets[bag + 1] : L;
   const float len = static_cast<float>(end - offsets[bag]);
+  const int64_t row = index[j];
+  if (row < 0 || row >= V) return;  // reported by bag_check_kernel; nothing is written
   const TIN* src = b + bag * D;
-  TOUT* dst = gs + (bag * V + index[j]) * D;
+  TOUT* dst = gs + (bag * V + row) * D;
   for (int64_t d = threadIdx.x; d < D; d += kThreads) {
     float v = dpk_io<TIN>::load(src + d) * scale;
     if (mean) v = v / len;
@@ -310,11 +308,12 @@ int check_common(const char* who, const int64_t* ids, int64_t n, int64_t T, int6
   return DPK_OK;
 }
 
-void launch_link(const int64_t* ids, int64_t n, int64_t T, int64_t V, const EmbWs& w, hipStream_t s) {
+// status: the caller's sticky flag (NULL: no range check), set when an id lies outside [0, V)
+void launch_link(const int64_t* ids, int64_t n, int64_t T, int64_t V, const EmbWs& w, int32_t* status,
+                 hipStream_t s) {
   const int bps = static_cast<int>(dpk_cdiv(T, kLinkPositions));
-  hipLaunchKernelGGL(zero_flag_kernel, dim3(1), dim3(1), 0, s, w.flag);
   hipLaunchKernelGGL(emb_link_kernel, dim3(static_cast<unsigned>(n * bps)), dim3(kThreads), 0, s, ids, T,
-                     V, bps, w.next, w.leader, w.flag);
+                     V, bps, w.next, w.leader, status);
 }
 
 template <typename TIN, typename TOUT, int MODE>
@@ -352,7 +351,7 @@ extern "C" int dpk_embedding_unique_pairs(const int64_t* ids, int64_t n, int64_t
   int rc = check_common(who, ids, n, T, 0, ws, ws_bytes, &w);
   if (rc != DPK_OK) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  launch_link(ids, n, T, 0, w, s);
+  launch_link(ids, n, T, 0, w, nullptr, s);
   DPK_LAUNCH_CHECK(who);
   const int bps = static_cast<int>(dpk_cdiv(T, kThreads));
   hipLaunchKernelGGL(emb_rank_kernel, dim3(static_cast<unsigned>(n * bps)), dim3(kThreads), 0, s, ids, T,
@@ -380,7 +379,7 @@ extern "C" int dpk_embedding_ghost_norm(const int64_t* ids, const void* b, int d
   const int64_t tch = dpk_cdiv(T, kLeadersPerBlock), dch = dpk_cdiv(D, kThreads * 4);
   DPK_REQUIRE(n * tch * dch <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: too many blocks", who);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  launch_link(ids, n, T, 0, w, s);
+  launch_link(ids, n, T, 0, w, nullptr, s);
   DPK_LAUNCH_CHECK(who);
   const bool vec = D % 4 == 0 && dpk_aligned(b, dtype == DPK_BF16 ? 8 : 16);
   if (dtype == DPK_F32) launch_walk<float, float, 0>(vec, ids, b, w, n, T, D, 0, scale, nullptr, s);
@@ -393,7 +392,8 @@ extern "C" int dpk_embedding_ghost_norm(const int64_t* ids, const void* b, int d
 
 extern "C" int dpk_embedding_gs(const int64_t* ids, const void* b, int in_dtype, void* gs,
                                 int gs_dtype, int64_t n, int64_t T, int64_t V, int64_t D,
-                                float scale, void* ws, size_t ws_bytes, dpk_stream_t stream) {
+                                float scale, int32_t* status, void* ws, size_t ws_bytes,
+                                dpk_stream_t stream) {
   const char* who = "dpk_embedding_gs";
   DPK_REQUIRE(n >= 0 && T >= 1 && V >= 1 && D >= 1, DPK_E_SHAPE, "%s: n=%lld T=%lld V=%lld D=%lld", who,
               (long long)n, (long long)T, (long long)V, (long long)D);
@@ -409,14 +409,11 @@ extern "C" int dpk_embedding_gs(const int64_t* ids, const void* b, int in_dtype,
   const int64_t tch = dpk_cdiv(T, kLeadersPerBlock), dch = dpk_cdiv(D, kThreads * 4);
   DPK_REQUIRE(n * tch * dch <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: too many blocks", who);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  launch_link(ids, n, T, V, w, s);
+  DPK_REQUIRE(dpk_aligned(status, 4), DPK_E_ALIGN, "%s: status misaligned", who);
+  // Ids outside [0, V) would address memory outside gs: the walk below writes nothing for
+  // them, and the link kernel raises the caller's flag.
+  launch_link(ids, n, T, V, w, status, s);
   DPK_LAUNCH_CHECK(who);
-  // Ids outside [0, V) would address memory outside gs: find out before writing.
-  int32_t flag = 0;
-  hipError_t e = hipMemcpyAsync(&flag, w.flag, sizeof(flag), hipMemcpyDeviceToHost, s);
-  if (e == hipSuccess) e = hipStreamSynchronize(s);
-  DPK_REQUIRE(e == hipSuccess, DPK_E_LAUNCH, "%s: %s", who, hipGetErrorString(e));
-  DPK_REQUIRE(flag == 0, DPK_E_ARG, "%s: an id lies outside [0, %lld)", who, (long long)V);
   const size_t bytes = static_cast<size_t>(n) * V * D * dpk_elsize(gs_dtype);
   const int64_t n16 = dpk_aligned(gs, 16) ? static_cast<int64_t>(bytes / 16) : 0;
   const int64_t ntail = static_cast<int64_t>(bytes - static_cast<size_t>(n16) * 16);
@@ -437,12 +434,10 @@ extern "C" int dpk_embedding_gs(const int64_t* ids, const void* b, int in_dtype,
   return DPK_OK;
 }
 
-extern "C" size_t dpk_embedding_bag_workspace_bytes(void) { return 256; }
-
 extern "C" int dpk_embedding_bag_gs(const int64_t* index, const int64_t* offsets, const void* b,
                                     int in_dtype, void* gs, int gs_dtype, int64_t nbags, int64_t L,
-                                    int64_t V, int64_t D, int mean, float scale, void* ws,
-                                    size_t ws_bytes, dpk_stream_t stream) {
+                                    int64_t V, int64_t D, int mean, float scale, int32_t* status,
+                                    dpk_stream_t stream) {
   const char* who = "dpk_embedding_bag_gs";
   DPK_REQUIRE(nbags >= 0 && L >= 0 && V >= 1 && D >= 1, DPK_E_SHAPE, "%s: bags=%lld L=%lld V=%lld D=%lld",
               who, (long long)nbags, (long long)L, (long long)V, (long long)D);
@@ -453,22 +448,17 @@ extern "C" int dpk_embedding_bag_gs(const int64_t* index, const int64_t* offsets
   DPK_REQUIRE(dpk_aligned(index, 8) && dpk_aligned(offsets, 8) && dpk_aligned(b, dpk_elsize(in_dtype)) &&
                   dpk_aligned(gs, 16),
               DPK_E_ALIGN, "%s: misaligned tensor (gs needs 16 bytes)", who);
-  DPK_REQUIRE(ws && ws_bytes >= 4 && dpk_aligned(ws, 4), DPK_E_WORKSPACE, "%s: workspace of 4 bytes needed", who);
+  DPK_REQUIRE(dpk_aligned(status, 4), DPK_E_ALIGN, "%s: status misaligned", who);
   DPK_REQUIRE(L <= DPK_MAX_GRID_X && nbags <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: too many positions", who);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  int32_t* dflag = static_cast<int32_t*>(ws);
-  hipLaunchKernelGGL(zero_flag_kernel, dim3(1), dim3(1), 0, s, dflag);
-  const int64_t most = L > nbags ? L : nbags;
-  hipLaunchKernelGGL(bag_check_kernel, dim3(static_cast<unsigned>(dpk_cdiv(most, kThreads))), dim3(kThreads), 0,
-                     s, index, offsets, L, nbags, V, dflag);
-  DPK_LAUNCH_CHECK(who);
-  // Bad indices would address memory outside gs: find out before writing.
-  int32_t flag = 0;
-  hipError_t e = hipMemcpyAsync(&flag, dflag, sizeof(flag), hipMemcpyDeviceToHost, s);
-  if (e == hipSuccess) e = hipStreamSynchronize(s);
-  DPK_REQUIRE(e == hipSuccess, DPK_E_LAUNCH, "%s: %s", who, hipGetErrorString(e));
-  DPK_REQUIRE(flag == 0, DPK_E_ARG, "%s: an index lies outside [0, %lld) or the offsets are not ascending in [0, %lld]",
-              who, (long long)V, (long long)L);
+  // Bad indices would address memory outside gs: the scatter below writes nothing for them
+  // (and reads b only inside [0, bags)), and the check kernel raises the caller's flag.
+  if (status) {
+    const int64_t most = L > nbags ? L : nbags;
+    hipLaunchKernelGGL(bag_check_kernel, dim3(static_cast<unsigned>(dpk_cdiv(most, kThreads))), dim3(kThreads), 0,
+                       s, index, offsets, L, nbags, V, status);
+    DPK_LAUNCH_CHECK(who);
+  }
   const size_t bytes = static_cast<size_t>(nbags) * V * D * dpk_elsize(gs_dtype);
   const int64_t n16 = static_cast<int64_t>(bytes / 16);
   const int64_t ntail = static_cast<int64_t>(bytes - static_cast<size_t>(n16) * 16);

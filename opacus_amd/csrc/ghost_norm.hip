@@ -9,9 +9,6 @@
 // ti <= tj are visited and off-diagonal ones count twice. One float per block
 // goes to the workspace; a fixed-order reduction applies clamp(min=0) and sqrt
 // (linear.py:87-89, :92).
-#include <cstdlib>
-#include <cstring>
-
 #include "dpk_common.h"
 #include "mfma_bf16.h"
 #include "mfma_bf16_dlds.h"
@@ -276,18 +273,15 @@ int tile_edge(int64_t T) { return T > 64 ? 128 : 64; }
 // visits, forming the gradient and squaring it 2 T in out: for thin layers (a low-rank
 // adapter, a narrow head) the second is far cheaper although the gradient tile exists for a
 // moment in registers.
-// DPK_GHOST_NORM_ROUTE=gram|direct in the environment overrides the choice (for tests that
-// want both routes on the same shapes).
-bool direct_is_cheaper(int dtype, int64_t T, int64_t out, int64_t in) {
-  if (const char* force = getenv("DPK_GHOST_NORM_ROUTE")) {
-    if (strcmp(force, "gram") == 0) return false;
-    if (strcmp(force, "direct") == 0) return true;
-  }
+// The caller's `route` argument overrides the choice (tests drive both routes on one shape).
+bool direct_is_cheaper(int route, int64_t T, int64_t out, int64_t in) {
+  if (route == DPK_ROUTE_GRAM) return false;
+  if (route == DPK_ROUTE_DIRECT) return true;
   const int B = T > 64 ? 128 : 64;
   const int64_t nt = dpk_cdiv(T, B);
   const double gram = static_cast<double>(nt * (nt + 1) / 2) * B * B * static_cast<double>(in + out);
   const double direct = static_cast<double>(T) * static_cast<double>(in) * static_cast<double>(out);
-  (void)dtype;  // the two routes run at about the same rate for either element type
+  // the two routes run at about the same rate for either element type
   return direct < 0.9 * gram;
 }
 
@@ -309,14 +303,18 @@ extern "C" size_t dpk_linear_ghost_norm_workspace_bytes(int64_t n, int64_t T, in
   // quadrant slots each (2 m^2 + 2 m slots per sample covers both).
   const int64_t m = dpk_cdiv(T, 128);
   const size_t gram = dpk_align_up(static_cast<size_t>(2 * n * (2 * m * m + 2 * m)) * sizeof(float), 256);
-  const size_t direct = direct_is_cheaper(DPK_F32, T, out, in) ? direct_layout(n, T, out, in).total : 0;
+  // ... and for the direct route, whichever of the two a call ends up taking
+  const size_t direct = direct_layout(n, T, out, in).total;
   return gram > direct ? gram : direct;
 }
 
 extern "C" int dpk_linear_ghost_norm(const void* b, const void* a, int dtype, float* norm_w,
                                      float* norm_b, int64_t n, int64_t T, int64_t out, int64_t in,
-                                     float scale, void* ws, size_t ws_bytes, dpk_stream_t stream) {
+                                     float scale, int route, void* ws, size_t ws_bytes,
+                                     dpk_stream_t stream) {
   const char* who = "dpk_linear_ghost_norm";
+  DPK_REQUIRE(route == DPK_ROUTE_AUTO || route == DPK_ROUTE_GRAM || route == DPK_ROUTE_DIRECT, DPK_E_ARG,
+              "%s: route %d", who, route);
   DPK_REQUIRE(n >= 0 && T >= 1 && out >= 1 && in >= 1, DPK_E_SHAPE,
               "%s: n=%lld T=%lld out=%lld in=%lld", who, (long long)n, (long long)T, (long long)out,
               (long long)in);
@@ -340,14 +338,15 @@ extern "C" int dpk_linear_ghost_norm(const void* b, const void* a, int dtype, fl
     DPK_LAUNCH_CHECK(who);
     return DPK_OK;
   }
-  if (norm_w && direct_is_cheaper(dtype, T, out, in)) {
+  if (norm_w && direct_is_cheaper(route, T, out, in)) {
     // |sum_t b_t a_t^T|_F from the per-sample gradient tiles themselves, never stored;
     // the bias norm from the column sums of b
     const DirectLayout l = direct_layout(n, T, out, in);
     DPK_REQUIRE(ws && ws_bytes >= l.total, DPK_E_WORKSPACE, "%s: workspace %zu < %zu bytes", who, ws_bytes, l.total);
     DPK_REQUIRE(dpk_aligned(ws, 256), DPK_E_ALIGN, "%s: workspace must be 256-byte aligned", who);
     char* base = static_cast<char*>(ws);
-    int rc = dpk_linear_gs(b, a, dtype, nullptr, dtype, norm_w, n, T, out, in, 1.0f, base, l.bias, stream);
+    int rc = dpk_linear_gs(b, a, dtype, nullptr, dtype, norm_w, n, T, out, in, 1.0f, DPK_TILE_AUTO, base, l.bias,
+                           stream);
     if (rc != DPK_OK) return rc;
     dpk_launch_reduce_rows(norm_w, n, 1, norm_w, 1, absscale, s);  // in place: sqrt, times |scale|
     DPK_LAUNCH_CHECK(who);

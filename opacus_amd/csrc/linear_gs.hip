@@ -14,7 +14,6 @@
 #include "mfma_f32_dlds.h"
 #include "mfma_f32.h"
 
-#include <cstdlib>
 #include <type_traits>
 
 namespace {
@@ -462,20 +461,19 @@ Plan make_plan(int64_t T, int64_t M, int64_t N, bool vec) {
 // 16-byte chunks, at least one whole k tile, per-lane byte offsets inside a k tile that fit
 // 32 bits. The 256-tile blocks move half the operand bytes per product and run one to a
 // CU; the 128-tile blocks two to a CU. The cheaper of the two by rounds of resident blocks
-// times work per block wins. DPK_LINEAR_BF16_TILE=128|256 in the environment overrides the
-// choice (for tests that want both kernels on small shapes).
+// times work per block wins. `tile` (DPK_TILE_128 or DPK_TILE_256) overrides the choice
+// (for tests that want both kernels on small shapes).
 void plan_tr(Plan& p, const void* b, const void* a, const void* gs, int64_t n, int64_t T, int64_t M, int64_t N,
-             int cus) {
+             int cus, int tile) {
   if (cus <= 0) cus = 256;
   if (p.outer || p.bm != 128 || T < mb16t::BK || M % 8 != 0 || N % 8 != 0 || M >= (1LL << 24) || N >= (1LL << 24) ||
       !dpk_aligned(b, 16) || !dpk_aligned(a, 16) || !dpk_aligned(gs, 16))
     return;
-  const char* force = getenv("DPK_LINEAR_BF16_TILE");
   const int64_t small = n * dpk_cdiv(M, 128) * dpk_cdiv(N, 128), large = n * dpk_cdiv(M, 256) * dpk_cdiv(N, 256);
   const double cost_small = static_cast<double>(dpk_cdiv(small, 2 * cus)) * 2.0;
   const double cost_large = static_cast<double>(dpk_cdiv(large, cus)) * 4.0 * kTrLargeGain;
   p.tr = (M >= 256 && N >= 256 && cost_large < cost_small) ? 256 : 128;
-  if (force) p.tr = atoi(force) == 256 ? 256 : 128;
+  if (tile != DPK_TILE_AUTO) p.tr = tile == DPK_TILE_256 ? 256 : 128;
   p.bm = p.tr;
   p.tiles_m = dpk_cdiv(M, p.tr);
   p.tiles_n = dpk_cdiv(N, p.tr);
@@ -587,8 +585,10 @@ extern "C" size_t dpk_linear_gs_workspace_bytes(int64_t n, int64_t T, int64_t ou
 
 extern "C" int dpk_linear_gs(const void* b, const void* a, int in_dtype, void* gs, int gs_dtype,
                              float* sumsq, int64_t n, int64_t T, int64_t out, int64_t in,
-                             float scale, void* ws, size_t ws_bytes, dpk_stream_t stream) {
+                             float scale, int tile, void* ws, size_t ws_bytes, dpk_stream_t stream) {
   const char* who = "dpk_linear_gs";
+  DPK_REQUIRE(tile == DPK_TILE_AUTO || tile == DPK_TILE_128 || tile == DPK_TILE_256, DPK_E_ARG, "%s: tile %d", who,
+              tile);
   DPK_REQUIRE(n >= 0 && T >= 1 && out >= 1 && in >= 1, DPK_E_SHAPE,
               "%s: n=%lld T=%lld out=%lld in=%lld", who, (long long)n, (long long)T, (long long)out,
               (long long)in);
@@ -601,7 +601,7 @@ extern "C" int dpk_linear_gs(const void* b, const void* a, int in_dtype, void* g
               DPK_E_ALIGN, "%s: misaligned tensor", who);
   const bool vec = linear_vec(b, a, gs, in_dtype, gs_dtype, out, in);
   Plan p = make_plan(T, out, in, vec);
-  if (in_dtype == DPK_BF16) plan_tr(p, b, a, gs, n, T, out, in, dpk_device_cus());
+  if (in_dtype == DPK_BF16) plan_tr(p, b, a, gs, n, T, out, in, dpk_device_cus(), tile);
   else plan_dlds_f32(p, b, a, gs, gs_dtype, T, out, in);
   const int64_t blocks = n * p.tiles_m * p.tiles_n;
   DPK_REQUIRE(blocks <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: %lld blocks exceed the grid limit", who,

@@ -189,11 +189,7 @@ struct Tile {
     __builtin_amdgcn_sched_barrier(0);  // keep the reads ahead of the MFMAs
     // MFMAs execute asynchronously: the global->LDS loads of the tile after next
     // (and their address arithmetic) are issued in their shadow, a few per step.
-#ifdef DPK_DLDS_PER_STEP
-    constexpr int PER_STEP = DPK_DLDS_PER_STEP;
-#else
     constexpr int PER_STEP = (NLOADS + KS - 1) / KS;
-#endif
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       if constexpr (kF32) {

@@ -136,7 +136,7 @@ extern "C" int dpk_tied_embedding_cross(const int64_t* ids, const void* e, int e
   // R[s, t, :] = sum_t2 N[s, t2, t] * a[s, t2, :]: the Linear per-sample contraction with
   // "out" = T and the sum over the T2 head positions
   const int rc = dpk_linear_gs(gathered, a, head_dtype, product, DPK_F32, nullptr, n, T2, T, D, 1.0f,
-                               base + l.linear, l.total - l.linear, stream);
+                               DPK_TILE_AUTO, base + l.linear, l.total - l.linear, stream);
   if (rc != DPK_OK) return rc;
 
   const int64_t P = T * D, chunks = dpk_cdiv(P, kDotChunk);

@@ -113,10 +113,13 @@ def linear_grad_sample(
     scale: float = 1.0,
     want_sumsq: bool = True,
     out_dtype: Optional[torch.dtype] = None,
+    tile: int = _lib.DPK_TILE_AUTO,
 ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     """``gs[n,i,j] = scale * sum_t b[n,t,i] a[n,t,j]`` and ``sum_ij gs[n]^2``.
 
     ``backprops`` is ``[n, *, out]``, ``activations`` ``[n, *, in]`` with the same middle dims.
+    ``tile`` (128 or 256) names the block tile of the bf16 contraction kernel instead of
+    leaving the choice to the library; tests use it.
     """
     dev = _need_gpu(backprops, activations)
     if activations.dtype != backprops.dtype:
@@ -139,7 +142,7 @@ def linear_grad_sample(
             "dpk_linear_gs",
             L.dpk_linear_gs(
                 _ptr(b), _ptr(a), _code(b), _ptr(gs), _code(gs), _ptr(sumsq), n, T, out_f, in_f,
-                float(scale), _ptr(ws), wsb, _stream(dev),
+                float(scale), int(tile), _ptr(ws), wsb, _stream(dev),
             ),
         )
     return gs, sumsq
@@ -181,8 +184,11 @@ def linear_ghost_norm(
     scale: float = 1.0,
     want_weight: bool = True,
     want_bias: bool = False,
+    route: int = _lib.DPK_ROUTE_AUTO,
 ) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
-    """Per-sample norms (fp32) of the Linear weight and bias gradients without forming them."""
+    """Per-sample norms (fp32) of the Linear weight and bias gradients without forming them.
+    ``route`` (``DPK_ROUTE_GRAM`` / ``DPK_ROUTE_DIRECT``) names the kernel family instead of
+    leaving the choice to the library; tests use it."""
     dev = _need_gpu(backprops, activations)
     if activations.dtype != backprops.dtype:
         activations = activations.to(backprops.dtype)
@@ -203,7 +209,7 @@ def linear_ghost_norm(
             "dpk_linear_ghost_norm",
             L.dpk_linear_ghost_norm(
                 _ptr(b), _ptr(a), _code(b), _ptr(nw), _ptr(nb), n, T, out_f, in_f, float(scale),
-                _ptr(ws), wsb, _stream(dev),
+                int(route), _ptr(ws), wsb, _stream(dev),
             ),
         )
     return nw, nb
@@ -354,10 +360,43 @@ def embedding_unique_pairs(ids: torch.Tensor) -> Tuple[torch.Tensor, torch.Tenso
     return pairs[: int(count.item())], inverse
 
 
+# ---- index validation of the Embedding samplers --------------------------------------
+# The entry points never wait for the stream. An id outside the table makes them write
+# nothing for that position and raise a sticky int32 flag in device memory, one per device,
+# that is read only when somebody asks. (In a training step nn.Embedding's own forward has
+# already refused such ids before a sampler sees them.)
+VALIDATE_EMBEDDING_INDICES = False  # True: every sampler call reads the flag back (a sync per call)
+_EMB_STATUS: Dict[torch.device, torch.Tensor] = {}
+
+
+def _emb_status(dev: torch.device) -> torch.Tensor:
+    t = _EMB_STATUS.get(dev)
+    if t is None:
+        t = _EMB_STATUS[dev] = torch.zeros(1, dtype=torch.int32, device=dev)
+    return t
+
+
+def check_embedding_indices(device=None) -> None:
+    """Raises ``IndexError`` if an Embedding / EmbeddingBag sampler call on ``device`` since the
+    last check met an index outside its table (or bag offsets that do not ascend inside the
+    index list), and clears the flag. Waits for the device."""
+    devs = [torch.device(device)] if device is not None else list(_EMB_STATUS)
+    for d in devs:
+        d = torch.device("cuda", torch.cuda.current_device()) if d.type == "cuda" and d.index is None else d
+        t = _EMB_STATUS.get(d)
+        if t is not None and int(t.item()) != 0:
+            t.zero_()
+            raise IndexError(
+                "an Embedding sampler met an index outside [0, num_embeddings) or EmbeddingBag offsets that are "
+                "not ascending inside the index list; nothing was written for it"
+            )
+
+
 def embedding_grad_sample(
     ids: torch.Tensor, backprops: torch.Tensor, num_embeddings: int, scale: float = 1.0
 ) -> torch.Tensor:
-    """``gs[n,v,:] = scale * sum_{t: ids[n,t]==v} b[n,t,:]`` as a dense ``[n, V, D]`` tensor."""
+    """``gs[n,v,:] = scale * sum_{t: ids[n,t]==v} b[n,t,:]`` as a dense ``[n, V, D]`` tensor.
+    An id outside ``[0, V)`` contributes nothing; see :func:`check_embedding_indices`."""
     dev = _need_gpu(ids, backprops)
     ids2 = _ids_2d(ids)
     n, T = ids2.shape
@@ -375,9 +414,11 @@ def embedding_grad_sample(
             "dpk_embedding_gs",
             L.dpk_embedding_gs(
                 _ptr(ids2), _ptr(b), _code(b), _ptr(gs), _code(gs), n, T, num_embeddings, D,
-                float(scale), _ptr(ws), wsb, _stream(dev),
+                float(scale), _ptr(_emb_status(dev)), _ptr(ws), wsb, _stream(dev),
             ),
         )
+    if VALIDATE_EMBEDDING_INDICES:
+        check_embedding_indices(dev)
     return gs
 
 
@@ -471,15 +512,16 @@ def embedding_bag_grad_sample(
     if nbags == 0:
         return gs
     L = lib()
-    ws, wsb = _ws(L.dpk_embedding_bag_workspace_bytes(), dev)
     with _timed("embedding_bag_gs", dev):
         check(
             "dpk_embedding_bag_gs",
             L.dpk_embedding_bag_gs(
                 _ptr(idx), _ptr(off), _ptr(b), _code(b), _ptr(gs), _code(gs), nbags, idx.numel(), num_embeddings, D,
-                int(mode == "mean"), float(scale), _ptr(ws), wsb, _stream(dev),
+                int(mode == "mean"), float(scale), _ptr(_emb_status(dev)), _stream(dev),
             ),
         )
+    if VALIDATE_EMBEDDING_INDICES:
+        check_embedding_indices(dev)
     return gs
 
 

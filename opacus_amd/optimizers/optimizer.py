@@ -17,6 +17,7 @@ What changes is how many times the per-sample gradients cross HBM:
 from __future__ import annotations
 
 import logging
+import os
 from collections import defaultdict
 from typing import Callable, Dict, List, Optional, Tuple, Union
 
@@ -61,20 +62,38 @@ def _check_processed_flag(obj: Union[torch.Tensor, List[torch.Tensor]]):
             _check_processed_flag_tensor(x)
 
 
-def philox_stream(generator: Optional[torch.Generator], device: torch.device, calls: int = 1) -> Tuple[int, int]:
+# XORed into the torch generator's seed to make the Philox key of the noise kernels. torch's own
+# kernels (dropout, randn, initialisers) key Philox with the bare seed and lay offset and thread
+# index across the counter differently from the noise kernel, so that with a shared key a
+# noise block could coincide with a block some torch kernel draws; a key of its own keeps
+# the noise independent of every other use of the generator.
+_NOISE_KEY_DOMAIN = 0x44504B5F4E4F4953
+
+
+def philox_stream(
+    generator: Optional[torch.Generator], device: torch.device, calls: int = 1, secure: bool = False
+) -> Tuple[int, int]:
     """``(seed, offset)`` for ``calls`` noise kernel launches (each may use up to four
     consecutive offsets), advancing the generator.
 
-    A generator on the GPU (the default one when ``generator`` is None) is used the way
-    torch's own Philox kernels use it: its seed is the key and its offset moves on, so
+    A generator on the GPU (the default one when ``generator`` is None) supplies the key
+    (its seed, moved into a domain of its own) and the offset, which moves on, so
     ``torch.manual_seed`` / ``generator.manual_seed`` make runs repeat. A CPU generator
-    cannot share an offset with the device; two 63-bit draws from it become the key and
+    cannot share an offset with the device; two 62-bit draws from it become the key and
     the offset, which keeps the same determinism.
+
+    ``secure``: key and offset are 126 fresh bits from ``os.urandom`` for every call and
+    no generator is consulted, so no seed a user or a library sets can reproduce or predict
+    the noise. Philox4x32-10 itself is a counter-based statistical generator, not a
+    cryptographic one (the reference's secure mode draws from torchcsprng).
     """
+    if secure:
+        raw = os.urandom(16)
+        return int.from_bytes(raw[:8], "little"), int.from_bytes(raw[8:], "little") >> 2
     if generator is None:
         generator = torch.cuda.default_generators[device.index if device.index is not None else torch.cuda.current_device()]
     if generator.device.type == "cuda":
-        seed = generator.initial_seed()
+        seed = generator.initial_seed() ^ _NOISE_KEY_DOMAIN
         offset = generator.get_offset()
         generator.set_offset(offset + _OFFSET_PER_CALL * calls)
         return seed, offset
@@ -91,7 +110,7 @@ def _generate_noise(std: float, reference: torch.Tensor, generator=None, secure_
     out = torch.zeros(reference.shape, device=reference.device, dtype=reference.dtype)
     if std == 0:
         return out
-    seed, offset = philox_stream(generator, reference.device)
+    seed, offset = philox_stream(generator, reference.device, secure=secure_mode)
     kernels.add_noise(out, out, std, 1.0, seed, offset, draws=4 if secure_mode else 1)
     return out
 
@@ -303,7 +322,7 @@ class DPOptimizer(Optimizer):
             if std == 0:
                 seed = offset = 0  # nothing is drawn and the generator stays where it is
             else:
-                seed, offset = philox_stream(self.generator, dev, calls=launches)
+                seed, offset = philox_stream(self.generator, dev, calls=launches, secure=self.secure_mode)
             kernels.add_noise_multi(ss, gg, std, denom, seed, offset, draws=draws)
 
     def add_noise(self):

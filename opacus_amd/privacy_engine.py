@@ -10,6 +10,7 @@ reference and are not part of this build: the step hook records what an accounta
 
 from __future__ import annotations
 
+import os
 import warnings
 from itertools import chain
 from typing import List, Optional, Tuple, Union
@@ -67,7 +68,22 @@ class PrivacyEngine:
         self.secure_mode = secure_mode
         self.secure_rng = None
         self.dataset = None
-        if not self.secure_mode:
+        if self.secure_mode:
+            # The reference builds a torchcsprng generator over /dev/urandom here and fails
+            # without that package (privacy_engine.py:86-96). This build keeps what it can
+            # deliver without it and says what it cannot: batch sampling uses a generator of
+            # its own seeded from os.urandom (so no torch.manual_seed reaches it), every noise
+            # launch takes a fresh Philox key and offset from os.urandom, and four draws are
+            # summed and halved as the reference does against floating-point attacks.
+            self.secure_rng = torch.Generator()
+            self.secure_rng.manual_seed(int.from_bytes(os.urandom(8), "little") >> 1)
+            warnings.warn(
+                "secure_mode: noise keys and the sampling generator are seeded from os.urandom and "
+                "cannot be reproduced by any seed, but the generators themselves (Philox4x32-10 on the "
+                "GPU, MT19937 for batch sampling) are statistical, not cryptographically secure as the "
+                "reference's torchcsprng is."
+            )
+        else:
             warnings.warn(
                 "Secure RNG turned off. This is perfectly fine for experimentation as it allows "
                 "for much faster training performance, but remember to turn it on and retrain "

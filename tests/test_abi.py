@@ -85,7 +85,7 @@ def test_workspace_queries_and_argument_errors_without_a_gpu():
     assert lib.dpk_linear_ghost_norm_workspace_bytes(2, 512, 8, 8) >= 2 * 2 * 36 * 4
     assert lib.dpk_embedding_workspace_bytes(2, 100, 64) > 0
     # a bad shape is refused before anything touches a device
-    rc = lib.dpk_linear_gs(None, None, 0, None, 0, None, 4, 0, 8, 8, 1.0, None, 0, None)
+    rc = lib.dpk_linear_gs(None, None, 0, None, 0, None, 4, 0, 8, 8, 1.0, 0, None, 0, None)
     assert rc == -1 and b"dpk_linear_gs" in lib.dpk_last_error()
     rc = lib.dpk_add_noise(None, 0, None, 0, 16, 1.0, 1.0, 0, 0, 1, None)
     assert rc == -6
@@ -93,5 +93,11 @@ def test_workspace_queries_and_argument_errors_without_a_gpu():
     assert rc == -2
     with pytest.raises(_lib.DpkError, match="DPK_E_SHAPE"):
         _lib.check("dpk_conv2d_gs", lib.dpk_conv2d_gs(None, None, 0, None, 0, None, 1, 3, 4, 4, 4, 3, 3, 1, 1, 0, 0, 0, 0, 1, 1, 2, 1.0, None, 0, None))
+    # a kernel choice outside the enum is refused
+    assert lib.dpk_linear_gs(None, None, 0, None, 0, None, 4, 2, 8, 8, 1.0, 64, None, 0, None) == -6
+    assert lib.dpk_linear_ghost_norm(None, None, 0, None, None, 4, 2, 8, 8, 1.0, 3, None, 0, None) == -6
+    # the ghost-norm workspace covers either route whatever the caller later asks for
+    thin = lib.dpk_linear_ghost_norm_workspace_bytes(4, 512, 16, 1024)
+    assert thin >= lib.dpk_linear_gs_workspace_bytes(4, 512, 16, 1024) + 4 * 16 * 4
     # n == 0 is a no-op
-    assert lib.dpk_linear_gs(None, None, 0, None, 0, None, 0, 1, 8, 8, 1.0, None, 0, None) == 0
+    assert lib.dpk_linear_gs(None, None, 0, None, 0, None, 0, 1, 8, 8, 1.0, 0, None, 0, None) == 0

@@ -93,22 +93,20 @@ def test_linear_grad_sample_f32(K, n, mid, fin, fout, scale):
         (3, (4, 16), 256, 128),  # 64 positions in two middle dimensions
     ],
 )
-@pytest.mark.parametrize("tile", [None, "128", "256"])
-def test_linear_grad_sample_bf16(K, n, mid, fin, fout, tile, monkeypatch):
+@pytest.mark.parametrize("tile", [0, 128, 256])
+def test_linear_grad_sample_bf16(K, n, mid, fin, fout, tile):
     """`tile` forces the 128 x 128 or the 256 x 256 variant of the transposing-read kernel where
-    the shape qualifies for it (None: the library's own choice)."""
-    if tile is not None:
-        monkeypatch.setenv("DPK_LINEAR_BF16_TILE", tile)
+    the shape qualifies for it (0: the library's own choice)."""
     torch.manual_seed(7)
     a = torch.randn(n, *mid, fin).bfloat16()
     b = torch.randn(n, *mid, fout).bfloat16()
     want_w, want_b = O.linear_grad_sample(a.float(), b.float())
-    gs, sumsq = K.linear_grad_sample(dev(b), dev(a))
+    gs, sumsq = K.linear_grad_sample(dev(b), dev(a), tile=tile)
     assert gs.dtype == torch.bfloat16
     assert_rel(gs, want_w, BF16_REL, "weight bf16")
     assert_rel(K.linear_bias_grad_sample(dev(b)), want_b, BF16_REL, "bias bf16")
     assert_rel(sumsq, want_w.double().flatten(1).pow(2).sum(1), 1e-4, "sumsq (fp32 accumulators)")
-    gs32, _ = K.linear_grad_sample(dev(b), dev(a), out_dtype=torch.float32)
+    gs32, _ = K.linear_grad_sample(dev(b), dev(a), out_dtype=torch.float32, tile=tile)
     assert_rel(gs32, want_w, FP32_REL, "weight bf16 in, fp32 out")
 
 
@@ -385,8 +383,8 @@ GHOST_SHAPES = [
 
 
 # "gram": sum over the T x T Grams (the reference's formula); "direct": the squared norm of the
-# per-sample gradient tiles as they are formed; None: the library's choice by cost
-GHOST_ROUTES = [None, "gram", "direct"]
+# per-sample gradient tiles as they are formed; "auto": the library's choice by cost
+GHOST_ROUTES = [0, 1, 2]  # DPK_ROUTE_AUTO, DPK_ROUTE_GRAM, DPK_ROUTE_DIRECT
 
 
 @pytest.mark.parametrize(
@@ -400,9 +398,7 @@ GHOST_ROUTES = [None, "gram", "direct"]
 )
 @pytest.mark.parametrize("scale", [1.0, 4.0])
 @pytest.mark.parametrize("route", GHOST_ROUTES)
-def test_linear_ghost_norm_f32(K, n, T, fin, fout, scale, route, monkeypatch):
-    if route is not None:
-        monkeypatch.setenv("DPK_GHOST_NORM_ROUTE", route)
+def test_linear_ghost_norm_f32(K, n, T, fin, fout, scale, route):
     torch.manual_seed(T * 7 + fin)
     a = torch.randn(n, T, fin)
     b = torch.randn(n, T, fout) * 0.1
@@ -410,11 +406,11 @@ def test_linear_ghost_norm_f32(K, n, T, fin, fout, scale, route, monkeypatch):
     want_w, want_b = O.linear_norm_sample(a.double(), (b * scale).double())
     gs_w, gs_b = O.linear_grad_sample(a.double(), (b * scale).double())
     torch.testing.assert_close(want_w, gs_w.flatten(1).norm(dim=1), rtol=1e-9, atol=1e-12)
-    nw, nb = K.linear_ghost_norm(dev(b), dev(a), scale=scale, want_weight=True, want_bias=True)
+    nw, nb = K.linear_ghost_norm(dev(b), dev(a), scale=scale, want_weight=True, want_bias=True, route=route)
     assert nw.dtype == torch.float32
     assert_rel(nw, want_w, FP32_REL, "weight norm")
     assert_rel(nb, want_b, FP32_REL, "bias norm")
-    only_b = K.linear_ghost_norm(dev(b), dev(a), scale=scale, want_weight=False, want_bias=True)
+    only_b = K.linear_ghost_norm(dev(b), dev(a), scale=scale, want_weight=False, want_bias=True, route=route)
     assert only_b[0] is None
     assert_rel(only_b[1], want_b, FP32_REL, "bias norm alone")
 
@@ -445,14 +441,12 @@ def test_linear_ghost_norm_2d_inputs(K):
     ],
 )
 @pytest.mark.parametrize("route", GHOST_ROUTES)
-def test_linear_ghost_norm_bf16(K, n, T, fin, fout, route, monkeypatch):
-    if route is not None:
-        monkeypatch.setenv("DPK_GHOST_NORM_ROUTE", route)
+def test_linear_ghost_norm_bf16(K, n, T, fin, fout, route):
     torch.manual_seed(T)
     a = torch.randn(n, T, fin).bfloat16()
     b = (torch.randn(n, T, fout) * 0.02).bfloat16()
     want_w, want_b = O.linear_norm_sample(a.double(), b.double())
-    nw, nb = K.linear_ghost_norm(dev(b), dev(a), want_weight=True, want_bias=True)
+    nw, nb = K.linear_ghost_norm(dev(b), dev(a), want_weight=True, want_bias=True, route=route)
     # inputs are exact in bf16 and accumulation is fp32: far inside the bf16 bar
     assert_rel(nw, want_w, 1e-4, "weight norm bf16")
     assert_rel(nb, want_b, 1e-4, "bias norm bf16")
@@ -610,24 +604,39 @@ def test_embedding_bag_grad_sample_is_bit_exact(K, mode, dtype):
         assert got.dtype == dtype and torch.equal(got.cpu(), want), (mode, dtype, scale)
 
 
-def test_embedding_bag_bad_inputs_are_errors(K):
-    from opacus_amd._lib import DpkError
-
-    b = torch.zeros(2, 4, device="cuda")
-    with pytest.raises(DpkError, match="outside"):
-        K.embedding_bag_grad_sample(dev(torch.tensor([0, 9])), dev(torch.tensor([0, 1])), b, 9)
-    with pytest.raises(DpkError, match="ascending"):
-        K.embedding_bag_grad_sample(dev(torch.tensor([0, 1, 2])), dev(torch.tensor([2, 1])), b, 9)
+def test_embedding_bag_bad_inputs_raise_the_device_flag(K):
+    """The entry point does not wait for the stream: a bad index writes nothing and raises a
+    sticky device flag that `check_embedding_indices` reads back."""
+    b = torch.ones(2, 4, device="cuda")
+    K.check_embedding_indices("cuda")  # start from a clear flag
+    gs = K.embedding_bag_grad_sample(dev(torch.tensor([0, 9])), dev(torch.tensor([0, 1])), b, 9)
+    assert gs[0, 0].eq(1).all() and gs.sum().item() == 4.0  # bag 0 written, bag 1's index 9 dropped
+    with pytest.raises(IndexError, match="outside"):
+        K.check_embedding_indices("cuda")
+    K.check_embedding_indices("cuda")  # cleared by the failed check
+    K.embedding_bag_grad_sample(dev(torch.tensor([0, 1, 2])), dev(torch.tensor([2, 1])), b, 9)
+    with pytest.raises(IndexError, match="ascending"):
+        K.check_embedding_indices("cuda")
     with pytest.raises(NotImplementedError):
         K.embedding_bag_grad_sample(dev(torch.tensor([0, 1])), dev(torch.tensor([0, 1])), b, 9, mode="max")
+    # a good call leaves the flag alone
+    K.embedding_bag_grad_sample(dev(torch.tensor([0, 1])), dev(torch.tensor([0, 1])), b, 9)
+    K.check_embedding_indices("cuda")
 
 
-def test_embedding_out_of_range_id_is_an_error(K):
-    from opacus_amd._lib import DpkError
-
-    ids = torch.tensor([[0, 3, 9]])
-    with pytest.raises(DpkError, match="outside"):
-        K.embedding_grad_sample(dev(ids), torch.zeros(1, 3, 4, device="cuda"), 9)
+def test_embedding_out_of_range_id_raises_the_device_flag(K, monkeypatch):
+    ids = torch.tensor([[0, 3, 9, -1]])
+    b = torch.ones(1, 4, 4, device="cuda")
+    K.check_embedding_indices("cuda")
+    gs = K.embedding_grad_sample(dev(ids), b, 9)
+    assert gs.sum().item() == 8.0 and gs[0, 0].eq(1).all() and gs[0, 3].eq(1).all()
+    with pytest.raises(IndexError, match="outside"):
+        K.check_embedding_indices("cuda")
+    # the debugging switch checks after every call
+    monkeypatch.setattr(K, "VALIDATE_EMBEDDING_INDICES", True)
+    with pytest.raises(IndexError, match="outside"):
+        K.embedding_grad_sample(dev(ids), b, 9)
+    K.embedding_grad_sample(dev(torch.tensor([[0, 3, 8]])), b[:, :3], 9)
 
 
 # ---- Normalisation layers ---------------------------------------------------------------
