@@ -109,6 +109,21 @@ int dpk_linear_ghost_norm(const void* b, const void* a, int dtype, float* norm_w
                           int64_t n, int64_t T, int64_t out, int64_t in, float scale, int route,
                           void* ws, size_t ws_bytes, dpk_stream_t stream);
 
+/* dpk_linear_ghost_norm for callers that cannot allocate device memory or pass a
+ * workspace: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc. It has no counterpart in the reference. Same arguments, results and kernels;
+ * the partial sums go to a buffer of DPK_STATIC_SCRATCH_BYTES that is part of the library's
+ * device image (every GPU the library runs on holds it until the process ends). The call
+ * allocates and frees nothing; the first call on a device looks up the buffer's address.
+ * Shapes whose dpk_linear_ghost_norm_workspace_bytes() exceeds the buffer are refused with
+ * DPK_E_SHAPE before anything is launched. All calls on one GPU share the one buffer:
+ * calls that may overlap in time on a GPU (different streams, different host threads)
+ * race on it and must be serialised by the caller. */
+#define DPK_STATIC_SCRATCH_BYTES (8u << 20)
+int dpk_linear_ghost_norm_static(const void* b, const void* a, int dtype, float* norm_w,
+                                 float* norm_b, int64_t n, int64_t T, int64_t out, int64_t in,
+                                 float scale, int route, dpk_stream_t stream);
+
 /* ------------------------------------------------------------------------- *
  * Per-sample gradients of nn.Conv2d (nn.Conv1d as a height-one image) and nn.Conv3d
  * replaces opacus/grad_sample/conv.py:28-119 (compute_conv_grad_sample, the

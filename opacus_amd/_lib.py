@@ -21,6 +21,7 @@ DPK_BF16 = 1
 DPK_MULTI_MAX = 48
 DPK_TILE_AUTO, DPK_TILE_128, DPK_TILE_256 = 0, 128, 256
 DPK_ROUTE_AUTO, DPK_ROUTE_GRAM, DPK_ROUTE_DIRECT = 0, 1, 2
+DPK_STATIC_SCRATCH_BYTES = 8 << 20
 
 STATUS_NAMES = {
     0: "DPK_OK",
@@ -45,6 +46,7 @@ SIGNATURES = {
     "dpk_linear_bias_gs": (c_int, [_P, c_int, _P, c_int, _P, _I, _I, _I, c_float, _P]),
     "dpk_linear_ghost_norm_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
     "dpk_linear_ghost_norm": (c_int, [_P, _P, c_int, _P, _P, _I, _I, _I, _I, c_float, c_int, _P, c_size_t, _P]),
+    "dpk_linear_ghost_norm_static": (c_int, [_P, _P, c_int, _P, _P, _I, _I, _I, _I, c_float, c_int, _P]),
     "dpk_conv2d_gs_workspace_bytes": (c_size_t, [_I, _I, _I, _I, _I, _I]),
     "dpk_conv2d_gs": (
         c_int,

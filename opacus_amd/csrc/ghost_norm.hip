@@ -9,6 +9,8 @@
 // ti <= tj are visited and off-diagonal ones count twice. One float per block
 // goes to the workspace; a fixed-order reduction applies clamp(min=0) and sqrt
 // (linear.py:87-89, :92).
+#include <mutex>
+
 #include "dpk_common.h"
 #include "mfma_bf16.h"
 #include "mfma_bf16_dlds.h"
@@ -446,4 +448,58 @@ extern "C" int dpk_linear_ghost_norm(const void* b, const void* a, int dtype, fl
     DPK_LAUNCH_CHECK(who);
   }
   return DPK_OK;
+}
+
+// ---- the same entry point for callers that cannot allocate ---------------------------
+// Partial sums (and, on the direct route, the column sums of b) live in a file-scope
+// device array instead of a caller-provided workspace. Every GPU holds its own copy of the
+// array at its own address; the name below is only the host-side handle by which
+// hipGetSymbolAddress finds the copy of the current device. Host code passes that address,
+// never the name, to the kernels. Each block writes every slot the final reduction reads,
+// so nothing has to start at zero and what an earlier call left behind is never read.
+static __device__ __align__(256) unsigned char scratch[DPK_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// Address of the current device's copy of `scratch`, resolved once per device.
+int scratch_of_current_device(const char* who, void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  DPK_REQUIRE(e == hipSuccess, DPK_E_LAUNCH, "%s: hipGetDevice: %s", who, hipGetErrorString(e));
+  DPK_REQUIRE(dev >= 0 && dev < kMaxDevices, DPK_E_LAUNCH, "%s: device index %d out of range", who, dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    DPK_REQUIRE(e == hipSuccess && ptr, DPK_E_LAUNCH, "%s: hipGetSymbolAddress: %s", who, hipGetErrorString(e));
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return DPK_OK;
+}
+}  // namespace
+
+extern "C" int dpk_linear_ghost_norm_static(const void* b, const void* a, int dtype, float* norm_w,
+                                            float* norm_b, int64_t n, int64_t T, int64_t out, int64_t in,
+                                            float scale, int route, dpk_stream_t stream) {
+  const char* who = "dpk_linear_ghost_norm_static";
+  DPK_REQUIRE(n >= 0 && T >= 1 && out >= 1 && in >= 1, DPK_E_SHAPE, "%s: n=%lld T=%lld out=%lld in=%lld", who,
+              (long long)n, (long long)T, (long long)out, (long long)in);
+  if (n == 0 || (!norm_w && !norm_b)) return DPK_OK;
+  const size_t need = dpk_linear_ghost_norm_workspace_bytes(n, T, out, in);
+  DPK_REQUIRE(need <= DPK_STATIC_SCRATCH_BYTES, DPK_E_SHAPE,
+              "%s: n=%lld T=%lld out=%lld in=%lld needs %zu bytes of scratch, the built-in buffer holds %zu; "
+              "use dpk_linear_ghost_norm with a workspace",
+              who, (long long)n, (long long)T, (long long)out, (long long)in, need,
+              static_cast<size_t>(DPK_STATIC_SCRATCH_BYTES));
+  void* ptr = nullptr;
+  if (need > 0) {
+    const int rc = scratch_of_current_device(who, &ptr);
+    if (rc != DPK_OK) return rc;
+  }
+  return dpk_linear_ghost_norm(b, a, dtype, norm_w, norm_b, n, T, out, in, scale, route, ptr,
+                               need > 0 ? static_cast<size_t>(DPK_STATIC_SCRATCH_BYTES) : 0, stream);
 }
