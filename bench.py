@@ -7,15 +7,18 @@ mode: forward, backward (per-sample gradients, 128 x 4096 x 4096 fp32 = 8.59 GB)
 ``zero_grad``. Inputs are synthetic tensors resident in HBM before the clock starts.
 
 Prints ONE JSON line. ``roofline`` describes the dominant kernel of the step, timed with
-HIP events on the launch stream inside the timed region. ``cpu_baseline`` (default
-workload only) is the CPU oracle - a restatement of the reference's einsum path,
-allocation pattern included - timed on this box's host cores on a bounded sample of the
-same workload.
+HIP events on the launch stream inside the timed region. ``cpu_baseline`` is the CPU
+oracle - a restatement of the reference's einsum path, allocation pattern included -
+timed on this box's host cores on a bounded sample of the same workload.
 
-The other four benchmark configurations can be timed with ``--workload c1|c3|c4|c5``
-(same JSON shape, no CPU baseline); they are parity-test shapes first and bench lines
-second. ``--kernels`` times each kernel of the library on its own at those shapes and
-prints one JSON line per kernel (time, algorithmic work, fraction of its roofline).
+The headline fields are config 2's. The same run then times the other four benchmark
+configurations (c1, c3, c4, c5: full DP-SGD steps through the drop-in API, at most 20
+steps each, 5 for c5) and reports them under ``"configs"``, each with its own
+``ms_per_step``, ``samples_per_s``, ``roofline`` and bounded-sample ``cpu_baseline``.
+``--workload cN`` times one configuration alone (same JSON shape, no ``configs``);
+``--headline-only`` skips the other four. ``--kernels`` times each kernel of the library on
+its own at those shapes and prints one JSON line per kernel (time, algorithmic work,
+fraction of its roofline).
 """
 
 from __future__ import annotations
@@ -25,6 +28,7 @@ import json
 import os
 import sys
 import time
+import warnings
 from pathlib import Path
 
 import torch
@@ -191,6 +195,8 @@ def workload_c2(dev):
             # dispatch), each scaled by what the counter reads for a 1 GiB device copy
             # (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000): 8,390,260 + 65,551 KiB over the two dispatches.
             traffic=8455811 * 1024,
+            traffic_source="recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, "
+                           "profiles/clip_accumulate_linear4096_b128_hbm_traffic.txt (not re-measured by this run)",
         ),
     )
 
@@ -317,31 +323,92 @@ WORKLOADS = {
 }
 
 
-def cpu_baseline(n_sample: int = 16, steps: int = 3) -> dict:
-    """The oracle's DP-SGD step for the default workload on the host cores, on ``n_sample`` of
-    the 128 samples (every pass over per-sample data is linear in the batch size)."""
-    from oracle import dp_oracle as O
+# ---- CPU baselines: the oracle's restatement of the reference's step on the host cores ----------
+warnings.filterwarnings("ignore", message="Full backward hook is firing")  # layers at the graph's start
 
-    N, D_IN, D_OUT = 128, 4096, 4096
-    torch.manual_seed(0)
-    lin = nn.Linear(D_IN, D_OUT, bias=True)
-    x = torch.randn(n_sample, D_IN)
-    b = torch.randn(n_sample, D_OUT)
-    sgd = torch.optim.SGD(lin.parameters(), lr=0.05)
 
-    def step():
-        sgd.zero_grad(set_to_none=True)
-        y = lin(x)
-        y.backward(b)
-        bp = O.scale_backprops(b, n_sample, "sum")
-        gs_w, gs_b = O.linear_grad_sample(x, bp)
-        gs = [O.store_grad_sample(gs_w, n_sample), O.store_grad_sample(gs_b, n_sample)]
-        _, _, summed = O.clip_and_accumulate(gs, 1.0)
-        grads = O.add_noise_and_scale(summed, [lin.weight.shape, lin.bias.shape], 1.0, 1.0, n_sample, "sum")
-        lin.weight.grad, lin.bias.grad = grads
-        sgd.step()
+def _cpu_capture(net):
+    """Forward / backward hooks of plain torch that keep each sampled layer's input and output
+    gradient, as the reference's hooks do (grad_sample_module.py:291-365)."""
+    store, handles = {}, []
+    kinds = (nn.Linear, nn.Conv2d, nn.GroupNorm, nn.RMSNorm, nn.Embedding)
+    for m in net.modules():
+        if isinstance(m, kinds):
+            handles.append(m.register_forward_hook(lambda mod, inp, out: store.setdefault(mod, [None, None]).__setitem__(0, inp[0].detach())))
+            handles.append(m.register_full_backward_hook(lambda mod, gi, go: store[mod].__setitem__(1, go[0].detach())))
+    return store, handles
 
-    step()
+
+def _cpu_grad_samples(O, m, a, b):
+    """Per-sample gradients of one layer's own parameters, in ``m.parameters()`` order."""
+    if isinstance(m, nn.Linear):
+        gw, gb = O.linear_grad_sample(a, b, bias=m.bias is not None)
+    elif isinstance(m, nn.Conv2d):
+        gw, gb = O.conv2d_grad_sample(a, b, kernel_size=m.kernel_size, padding=m.padding, stride=m.stride,
+                                      dilation=m.dilation, groups=m.groups, bias=m.bias is not None)
+    elif isinstance(m, nn.GroupNorm):
+        gw, gb = O.group_norm_grad_sample(a, b, m.num_groups, m.eps)
+    elif isinstance(m, nn.RMSNorm):
+        gw, gb = O.rms_norm_grad_sample(a, b, m.normalized_shape, m.eps), None
+    else:
+        gw, gb = O.embedding_grad_sample(a, b, m.num_embeddings), None
+    return [g for g in (gw, gb) if g is not None]
+
+
+def _cpu_hooks_step(O, net, sgd, x, y, n, sigma, C=1.0):
+    """One step in hooks mode: autograd's backward, every layer's einsum sampler, the zero +
+    copy buffer, norms, clip, sum, noise, scale, SGD (the reference's passes, one by one)."""
+    store, handles = _cpu_capture(net)
+    sgd.zero_grad(set_to_none=True)
+    F.cross_entropy(net(x), y).backward()
+    for h in handles:
+        h.remove()
+    gs, params = [], []
+    for m, (a, b) in store.items():
+        b = O.scale_backprops(b, n, "mean")
+        for g in _cpu_grad_samples(O, m, a, b):
+            gs.append(O.store_grad_sample(g, n))
+        params += list(m.parameters(recurse=False))
+    _, _, summed = O.clip_and_accumulate(gs, C)
+    grads = O.add_noise_and_scale(summed, [p.shape for p in params], sigma, C, n, "mean")
+    for p, g in zip(params, grads):
+        p.grad = g
+    sgd.step()
+
+
+def _cpu_ghost_step(O, net, sgd, inputs, per_sample_loss, n, sigma, C=1.0):
+    """One ghost-clipping step: first backward with the norm samplers (Gram products for Linear,
+    index sums for Embedding, materialised gradients for RMSNorm), clipping coefficients, second
+    backward of the reweighted loss, noise, scale, SGD (fast_gradient_clipping_utils.py:179-203)."""
+    store, handles = _cpu_capture(net)
+    sgd.zero_grad(set_to_none=True)
+    losses = per_sample_loss(net(inputs))
+    losses.mean().backward(retain_graph=True)
+    for h in handles:
+        h.remove()
+    norms = []
+    for m, (a, b) in store.items():
+        b = O.scale_backprops(b, n, "mean")
+        if isinstance(m, nn.Linear):
+            nw, nb = O.linear_norm_sample(a, b, bias=m.bias is not None)
+            norms += [v.float() for v in (nw, nb) if v is not None]
+        elif isinstance(m, nn.Embedding):
+            norms.append(O.embedding_norm_sample(a, b)["result_sqrt"].float())
+        else:
+            norms += [g.flatten(1).norm(2, dim=1).float() for g in _cpu_grad_samples(O, m, a, b)]
+    coef = O.clipping_coef(norms, C)
+    sgd.zero_grad(set_to_none=True)
+    (coef * losses).sum().backward()
+    params = [p for p in net.parameters() if p.grad is not None]
+    grads = O.add_noise_and_scale([p.grad for p in params], [p.shape for p in params], sigma, C, n, "mean")
+    for p, g in zip(params, grads):
+        p.grad = g.to(p.dtype)
+    sgd.step()
+
+
+def _cpu_time(step, n_sample, n_full, steps, what, warm=True):
+    if warm:
+        step()
     t0 = time.perf_counter()
     for _ in range(steps):
         step()
@@ -351,9 +418,67 @@ def cpu_baseline(n_sample: int = 16, steps: int = 3) -> dict:
         "unit": "samples/s",
         "cores": torch.get_num_threads(),
         "kind": "port",
-        "sample": f"{steps} steps at batch {n_sample} of {N} (per-sample passes are linear in the batch); "
-        f"{os.cpu_count()} logical CPUs visible",
+        "sample": f"{steps} step(s) at batch {n_sample} of {n_full}{' after one warm-up step' if warm else ', no warm-up'} ({what}; every per-sample "
+                  f"pass is linear in the batch); {os.cpu_count()} logical CPUs visible",
     }
+
+
+def cpu_baseline(workload: str = "c2") -> dict:
+    """The oracle's DP-SGD step for ``workload`` on the host cores, on a bounded sample of its batch."""
+    from oracle import dp_oracle as O
+
+    torch.manual_seed(0)
+    if workload == "c2":
+        N, D_IN, D_OUT, n_sample = 128, 4096, 4096, 16
+        lin = nn.Linear(D_IN, D_OUT, bias=True)
+        x, b = torch.randn(n_sample, D_IN), torch.randn(n_sample, D_OUT)
+        sgd = torch.optim.SGD(lin.parameters(), lr=0.05)
+
+        def step():
+            sgd.zero_grad(set_to_none=True)
+            lin(x).backward(b)
+            bp = O.scale_backprops(b, n_sample, "sum")
+            gs_w, gs_b = O.linear_grad_sample(x, bp)
+            gs = [O.store_grad_sample(gs_w, n_sample), O.store_grad_sample(gs_b, n_sample)]
+            _, _, summed = O.clip_and_accumulate(gs, 1.0)
+            grads = O.add_noise_and_scale(summed, [lin.weight.shape, lin.bias.shape], 1.0, 1.0, n_sample, "sum")
+            lin.weight.grad, lin.bias.grad = grads
+            sgd.step()
+
+        return _cpu_time(step, n_sample, N, 3, "einsum sampler, zero + copy buffer, norms, clip, sum, noise")
+    if workload in ("c1", "c4"):
+        if workload == "c1":
+            net, N, n_sample, steps = SmallCNN(), 256, 256, 10
+            x, sigma = torch.randn(n_sample, 1, 28, 28), 1.1
+        else:
+            net, N, n_sample, steps = ResBlock(), 256, 64, 3
+            x, sigma = torch.randn(n_sample, 64, 32, 32), 1.0
+        y = torch.randint(0, 10, (n_sample,))
+        sgd = torch.optim.SGD(net.parameters(), lr=0.1)
+        return _cpu_time(lambda: _cpu_hooks_step(O, net, sgd, x, y, n_sample, sigma), n_sample, N, steps,
+                         "hooks mode: unfold + einsum samplers, zero + copy buffers, norms, clip, sum, noise")
+    if workload == "c3":
+        N, n_sample, T = 32, 8, 512
+        net = nn.Sequential(nn.Linear(1024, 4096), nn.GELU(), nn.Linear(4096, 1024)).bfloat16()
+        x = torch.randn(n_sample, T, 1024).bfloat16()
+        sgd = torch.optim.SGD(net.parameters(), lr=0.01)
+        loss = lambda out: out.float().pow(2).flatten(1).mean(1)  # noqa: E731
+        return _cpu_time(lambda: _cpu_ghost_step(O, net, sgd, x, loss, n_sample, 1.0), n_sample, N, 3,
+                         "ghost clipping in bf16: T x T Gram norm samplers, two backward passes, noise")
+    if workload == "c5":
+        N, n_sample, T, V = 16, 1, 1024, 32000
+        net = Llama().bfloat16()
+        ids = torch.randint(0, V, (n_sample, T))
+        sgd = torch.optim.SGD(net.parameters(), lr=0.01)
+
+        def loss(logits):
+            tok = F.cross_entropy(logits[:, :-1].reshape(-1, V).float(), ids[:, 1:].reshape(-1), reduction="none")
+            return tok.view(n_sample, T - 1).mean(1)
+
+        return _cpu_time(lambda: _cpu_ghost_step(O, net, sgd, ids, loss, n_sample, 0.8), n_sample, N, 1,
+                         "ghost clipping in bf16: Gram, embedding and RMSNorm norm samplers, two backward passes, noise",
+                         warm=False)
+    raise ValueError(workload)
 
 
 def kernel_table(dev, iters: int = 10, warm: int = 3, with_cpu: bool = True):
@@ -544,13 +669,68 @@ def kernel_table(dev, iters: int = 10, warm: int = 3, with_cpu: bool = True):
               2.0 * n * 32 * 256 * 25)
 
 
+def run_workload(name: str, dev, steps: int, warmup: int, all_timers: bool = False, calibrate_copy: bool = False) -> dict:
+    """``warmup`` untimed steps, then ``steps`` timed steps of one configuration between device
+    synchronisations; HIP events on the launch stream around the roofline kernel's entry point."""
+    from opacus_amd import kernels
+
+    w = WORKLOADS[name](dev)
+    step = w["step"]
+    for _ in range(warmup):
+        step()
+    if calibrate_copy:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev)  # 1 GiB read + 1 GiB written
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        del src, dst
+    torch.cuda.synchronize()
+    # HIP events around the dominant kernel's entry point only, unless every entry point is asked for
+    only = None if all_timers else {w["roofline"]["timer"]}
+    with kernels.record_kernel_times(only=only) as times:
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+
+    kernel_ms = {k: sum(s.elapsed_time(e) for s, e in v) / steps for k, v in times.items()}
+    r = dict(w["roofline"])
+    spans = [s.elapsed_time(e) for s, e in times.get(r.pop("timer"), [])]
+    if "work_per_step" in r:  # several launches per step share the work figure
+        work, ms = r.pop("work_per_step"), sum(spans) / steps
+        r["launches_per_step"] = len(spans) // steps
+    else:
+        work, ms = r.pop("work_per_launch"), sum(spans) / max(len(spans), 1)
+    scale = 1e9 if r["unit"] == "GB/s" else 1e12
+    achieved = work / (ms * 1e-3) / scale if ms > 0 else 0.0
+    roofline = {
+        "kernel": r["kernel"], "bound": r["bound"], "achieved": achieved, "peak": r["peak"], "unit": r["unit"],
+        "frac": achieved / r["peak"], "traffic": r["traffic"], "algorithmic_work": work, "kernel_ms": ms,
+    }
+    for key in ("traffic_source", "launches_per_step"):
+        if key in r:
+            roofline[key] = r[key]
+    return {
+        "workload": w["workload"], "dtype": w["dtype"], "global_batch": w["n"], "steps": steps, "warmup": warmup,
+        "ms_per_step": elapsed / steps * 1e3, "samples_per_s": w["n"] * steps / elapsed,
+        "kernel_ms_per_step": kernel_ms, "extra": w["extra"], "roofline": roofline,
+    }
+
+
+# Steps of the other configurations inside the default run: enough for a stable mean, few
+# enough that the whole run stays within minutes (a c5 step takes ~60 ms, the others 1-2 ms).
+OTHER_CONFIGS = {"c1": (20, 5), "c3": (20, 5), "c4": (20, 5), "c5": (5, 2)}
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="c2")
-    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS), default=None,
+                    help="time this configuration alone (default: c2 as the headline, then c1, c3, c4, c5 under 'configs')")
+    ap.add_argument("--headline-only", action="store_true", help="config 2 only, without the 'configs' object")
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timings")
     ap.add_argument("--all-kernel-timers", action="store_true",
                     help="HIP-event timers around every entry point of the library (kernel_ms_per_step lists them all); "
                          "by default only the roofline kernel's entry point is timed")
@@ -572,70 +752,46 @@ def main() -> None:
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible; the HIP kernels have no CPU path")
 
-    from opacus_amd import kernels
-
     dev = torch.device("cuda:0")
     if args.kernels:
         for r in kernel_table(dev, with_cpu=not args.no_cpu_baseline):
             print(json.dumps(r), flush=True)
         return
-    w = WORKLOADS[args.workload](dev)
-    step = w["step"]
-    for _ in range(args.warmup):
-        step()
-    if args.calibrate_copy:
-        src = torch.empty(1 << 28, dtype=torch.float32, device=dev)  # 1 GiB read + 1 GiB written
-        dst = torch.empty_like(src)
-        dst.copy_(src)
-        del src, dst
-    torch.cuda.synchronize()
-    # HIP events around the dominant kernel's entry point only, unless every entry point is asked for
-    only = None if args.all_kernel_timers else {w["roofline"]["timer"]}
-    with kernels.record_kernel_times(only=only) as times:
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            step()
-        torch.cuda.synchronize()
-        elapsed = time.perf_counter() - t0
-
-    ms_per_step = elapsed / args.steps * 1e3
-    value = w["n"] * args.steps / elapsed
-    kernel_ms = {k: sum(s.elapsed_time(e) for s, e in v) / args.steps for k, v in times.items()}
-
-    r = dict(w["roofline"])
-    spans = [s.elapsed_time(e) for s, e in times.get(r.pop("timer"), [])]
-    if "work_per_step" in r:  # several launches per step share the work figure
-        work, ms = r.pop("work_per_step"), sum(spans) / args.steps
-        r["launches_per_step"] = len(spans) // args.steps
-    else:
-        work, ms = r.pop("work_per_launch"), sum(spans) / max(len(spans), 1)
-    scale = 1e9 if r["unit"] == "GB/s" else 1e12
-    achieved = work / (ms * 1e-3) / scale if ms > 0 else 0.0
-    roofline = {
-        "kernel": r["kernel"], "bound": r["bound"], "achieved": achieved, "peak": r["peak"], "unit": r["unit"],
-        "frac": achieved / r["peak"], "traffic": r["traffic"], "algorithmic_work": work, "kernel_ms": ms,
-    }
-    if "launches_per_step" in r:
-        roofline["launches_per_step"] = r["launches_per_step"]
-
+    head_name = args.workload or "c2"
+    head = run_workload(head_name, dev, args.steps, args.warmup, args.all_kernel_timers, args.calibrate_copy)
     out = {
         "metric": "dp_sgd_step_samples_per_sec",
-        "value": value,
+        "value": head["samples_per_s"],
         "unit": "samples/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": ms_per_step,
+        "ms_per_step": head["ms_per_step"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": w["dtype"],
+        "dtype": head["dtype"],
         "data": "synthetic",
-        "config": {"workload": w["workload"], "global_batch": w["n"], "kernel_ms_per_step": kernel_ms, **w["extra"]},
-        "roofline": roofline,
+        "config": {"workload": head["workload"], "global_batch": head["global_batch"],
+                   "kernel_ms_per_step": head["kernel_ms_per_step"], **head["extra"]},
+        "roofline": head["roofline"],
     }
-    if args.workload == "c2" and not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline()
+    cpu_ok = not args.no_cpu_baseline and head_name.rstrip("st") in ("c1", "c2", "c3", "c4", "c5")
+    if cpu_ok:
+        out["cpu_baseline"] = cpu_baseline(head_name.rstrip("st"))
+    if args.workload is None and not args.headline_only:
+        configs = {}
+        for name, (k, wu) in OTHER_CONFIGS.items():
+            torch.cuda.empty_cache()
+            k, wu = min(k, args.steps), min(wu, max(args.warmup, 1))
+            r = run_workload(name, dev, k, wu, args.all_kernel_timers)
+            entry = {key: r[key] for key in ("workload", "dtype", "global_batch", "steps", "warmup", "ms_per_step",
+                                             "samples_per_s", "roofline")}
+            entry.update(r["extra"])
+            if not args.no_cpu_baseline:
+                entry["cpu_baseline"] = cpu_baseline(name)
+            configs[name] = entry
+        out["configs"] = configs
     print(json.dumps(out))
 
 
