@@ -1,7 +1,8 @@
 """GPU parity: every HIP kernel, called through the C ABI, against the CPU oracle.
 
-Tolerances follow the stated bar: fp32 within rel 1e-5 (of the tensor's scale), bf16
-within rel 2e-2 with fp32 accumulation, integer outputs bit-exact.
+Tolerances follow the stated bar: fp32 within rel 1e-5, bf16 within rel 2e-2 with fp32
+accumulation - each applied at tensor, sample and element scale (see _compare.py) - and
+integer outputs bit-exact.
 """
 
 import math
@@ -10,6 +11,7 @@ import numpy as np
 import pytest
 import torch
 
+from _compare import assert_rel
 from oracle import dp_oracle as O
 
 pytestmark = pytest.mark.gpu
@@ -27,18 +29,6 @@ def K():
 
 def dev(t):
     return t.to("cuda")
-
-
-def assert_rel(got, want, rel, what=""):
-    """max |got - want| <= rel * max |want| (tensor-scale relative error), plus exact shape."""
-    got = got.detach().float().cpu()
-    want = want.detach().float().cpu()
-    assert got.shape == want.shape, f"{what}: shape {tuple(got.shape)} != {tuple(want.shape)}"
-    if want.numel() == 0:
-        return
-    scale = want.abs().max().item()
-    err = (got - want).abs().max().item()
-    assert err <= rel * max(scale, 1e-30), f"{what}: max err {err:.3e} vs scale {scale:.3e} (rel {err / max(scale, 1e-30):.2e})"
 
 
 # ---- Linear per-sample gradients ---------------------------------------------------------
