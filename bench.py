@@ -201,11 +201,15 @@ def workload_c2(dev):
     )
 
 
-def _hooks_workload(dev, net, x, y, n, sigma, desc, roofline, dtype="f32"):
+def _hooks_workload(dev, net, x, y, n, sigma, desc, roofline, dtype="f32", autograd_weight_grads=False):
+    """``autograd_weight_grads=False``: the library's option under which backward() forms no
+    aggregate (non-private) weight gradients, which the DP step never reads; the default of the
+    library keeps them as the reference does (workloads c1d / c4d)."""
     from opacus_amd import GradSampleModule
     from opacus_amd.optimizers import DPOptimizer
 
-    model = GradSampleModule(net.to(dev), loss_reduction="mean")
+    model = GradSampleModule(net.to(dev), loss_reduction="mean", autograd_weight_grads=autograd_weight_grads)
+    desc += "" if autograd_weight_grads else ", autograd_weight_grads=False"
     opt = DPOptimizer(
         torch.optim.SGD(model.parameters(), lr=0.1), noise_multiplier=sigma, max_grad_norm=1.0, expected_batch_size=n
     )
@@ -216,10 +220,11 @@ def _hooks_workload(dev, net, x, y, n, sigma, desc, roofline, dtype="f32"):
         F.cross_entropy(model(x), y).backward()
         opt.step()
 
-    return dict(step=step, n=n, dtype=dtype, workload=desc, extra={}, roofline=roofline)
+    return dict(step=step, n=n, dtype=dtype, workload=desc, extra={"autograd_weight_grads": autograd_weight_grads},
+                roofline=roofline)
 
 
-def workload_c1(dev):
+def workload_c1(dev, autograd_weight_grads=False):
     torch.manual_seed(0)
     n = 256
     P = 26010
@@ -228,10 +233,11 @@ def workload_c1(dev):
         "Small CNN (conv 1->16 k8 s2 p3, conv 16->32 k4 s2, fc 512->32, fc 32->10) fp32, batch 256, hooks, C=1, sigma=1.1",
         dict(kernel="clip_accumulate_kernel<float,float,*,RS=16> (8 tensors, one launch)", timer="clip_accumulate",
              bound="hbm", work_per_launch=float(n * P * 4 + P * 4), unit="GB/s", peak=HBM_PEAK_GBS, traffic=None),
+        autograd_weight_grads=autograd_weight_grads,
     )
 
 
-def workload_c4(dev):
+def workload_c4(dev, autograd_weight_grads=False):
     torch.manual_seed(0)
     n = 256
     flops = 2.0 * n * 64 * 576 * 1024  # per conv launch
@@ -240,6 +246,7 @@ def workload_c4(dev):
         "ResNet basic block: 2 x Conv2d(64->64, 3x3, p1) + GroupNorm(32), 32x32 images, fp32, batch 256, hooks, C=1, sigma=1",
         dict(kernel="conv2d_gs_patch_kernel<64,64,float,float>", timer="conv2d_gs", bound="mfma",
              work_per_launch=flops, unit="TFLOP/s", peak=MFMA_FP32_PEAK_TFLOPS, traffic=None),
+        autograd_weight_grads=autograd_weight_grads,
     )
 
 
@@ -320,6 +327,9 @@ WORKLOADS = {
     "c5t": workload_c5_tied,
     # the same two with the clipped sum formed from the first backward pass (single_backward=True)
     "c3s": lambda dev: workload_c3(dev, single=True), "c5s": lambda dev: workload_c5(dev, single=True),
+    # c1 and c4 with the library's default hooks (autograd's own weight gradients kept, as in the reference)
+    "c1d": lambda dev: workload_c1(dev, autograd_weight_grads=True),
+    "c4d": lambda dev: workload_c4(dev, autograd_weight_grads=True),
 }
 
 
@@ -776,9 +786,9 @@ def main() -> None:
                    "kernel_ms_per_step": head["kernel_ms_per_step"], **head["extra"]},
         "roofline": head["roofline"],
     }
-    cpu_ok = not args.no_cpu_baseline and head_name.rstrip("st") in ("c1", "c2", "c3", "c4", "c5")
+    cpu_ok = not args.no_cpu_baseline and head_name.rstrip("std") in ("c1", "c2", "c3", "c4", "c5")
     if cpu_ok:
-        out["cpu_baseline"] = cpu_baseline(head_name.rstrip("st"))
+        out["cpu_baseline"] = cpu_baseline(head_name.rstrip("std"))
     if args.workload is None and not args.headline_only:
         configs = {}
         for name, (k, wu) in OTHER_CONFIGS.items():
@@ -788,6 +798,10 @@ def main() -> None:
             entry = {key: r[key] for key in ("workload", "dtype", "global_batch", "steps", "warmup", "ms_per_step",
                                              "samples_per_s", "roofline")}
             entry.update(r["extra"])
+            if name + "d" in WORKLOADS:  # the same configuration with the library's default hooks
+                d = run_workload(name + "d", dev, k, wu, args.all_kernel_timers)
+                entry["default_hooks"] = {"ms_per_step": d["ms_per_step"], "samples_per_s": d["samples_per_s"],
+                                          "autograd_weight_grads": True}
             if not args.no_cpu_baseline:
                 entry["cpu_baseline"] = cpu_baseline(name)
             configs[name] = entry

@@ -19,7 +19,7 @@ from __future__ import annotations
 import logging
 import warnings
 from functools import partial
-from typing import Callable, Iterable, List, Tuple
+from typing import Callable, Iterable, List, Optional, Tuple
 
 import torch
 import torch.nn as nn
@@ -134,19 +134,25 @@ _ONE_TENSOR_OUT = (
 class GradSampleHooks(AbstractGradSampleHooks):
     """Attaches per-sample-gradient hooks to a module without wrapping it.
 
-    ``autograd_weight_grads=False`` (the default here; the reference has no such switch and
-    behaves like ``True``): while the hooks are enabled, a torch.nn layer served by one of
-    the library's samplers runs its forward with ``requires_grad`` off on its own parameters,
-    so the backward pass forms the gradients with respect to activations only. The aggregate
-    weight gradients autograd would otherwise compute (a second GEMM or weight-gradient
-    convolution per layer) are never read on this path: ``DPOptimizer.step`` writes
-    ``p.grad`` from the clipped per-sample gradients (optimizers/optimizer.py:477-504).
-    Until then ``p.grad`` of such a layer stays as it was (``None`` after ``zero_grad``)
-    instead of holding the non-private sum."""
+    ``autograd_weight_grads=True`` (the default) is the reference's behaviour: ``backward()``
+    leaves the non-private summed gradient in ``p.grad`` until ``DPOptimizer.step``
+    overwrites it. With ``autograd_weight_grads=False`` (an option the reference does not
+    have), while the hooks are enabled a torch.nn layer served by one of the library's
+    samplers runs its forward with ``requires_grad`` off on its own parameters, so the
+    backward pass forms the gradients with respect to activations only. The aggregate weight
+    gradients autograd would otherwise compute (a second GEMM or weight-gradient convolution
+    per layer) are never read on this path: ``DPOptimizer.step`` writes ``p.grad`` from the
+    clipped per-sample gradients (optimizers/optimizer.py:477-504). Until then ``p.grad`` of
+    such a layer stays as it was (``None`` after ``zero_grad``), which a caller that reads
+    ``p.grad`` between ``backward()`` and ``step()`` must know; the switch also changes
+    ``requires_grad`` inside forward, so it is not for models whose forward runs concurrently
+    from several threads."""
 
     GRAD_SAMPLERS = {}
     # ghost clipping needs autograd's weight gradients in its second pass
     CAN_SKIP_AUTOGRAD_WEIGHT_GRADS = True
+    # what ``autograd_weight_grads=None`` means
+    DEFAULT_AUTOGRAD_WEIGHT_GRADS = True
 
     def __init__(
         self,
@@ -156,7 +162,7 @@ class GradSampleHooks(AbstractGradSampleHooks):
         loss_reduction="mean",
         strict: bool = True,
         force_functorch=False,
-        autograd_weight_grads: bool = False,
+        autograd_weight_grads: Optional[bool] = None,
     ):
         super().__init__(m, batch_first=batch_first, loss_reduction=loss_reduction)
         errors = self.validate(module=m, strict=strict)
@@ -165,7 +171,9 @@ class GradSampleHooks(AbstractGradSampleHooks):
         self.hooks_enabled = False
         self.grad_accumulation_allowed = True
         self.force_functorch = force_functorch
-        self.autograd_weight_grads = autograd_weight_grads or not self.CAN_SKIP_AUTOGRAD_WEIGHT_GRADS
+        if autograd_weight_grads is None:
+            autograd_weight_grads = self.DEFAULT_AUTOGRAD_WEIGHT_GRADS
+        self.autograd_weight_grads = bool(autograd_weight_grads) or not self.CAN_SKIP_AUTOGRAD_WEIGHT_GRADS
         self._tap_anchor = torch.zeros((), requires_grad=True)
         self.add_hooks(loss_reduction=loss_reduction, batch_first=batch_first, force_functorch=force_functorch)
 
@@ -448,7 +456,7 @@ class GradSampleModule(GradSampleHooks, AbstractGradSampleModule):
         loss_reduction="mean",
         strict: bool = True,
         force_functorch=False,
-        autograd_weight_grads: bool = False,
+        autograd_weight_grads: Optional[bool] = None,
     ):
         nn.Module.__init__(self)
         GradSampleHooks.__init__(

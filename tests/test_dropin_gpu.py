@@ -27,6 +27,17 @@ def A():
     return opacus_amd
 
 
+@pytest.fixture(autouse=True, params=[True, False], ids=["autograd_wgrads", "params_off"])
+def weight_grad_mode(request, monkeypatch):
+    """Every test of this file runs in both modes of the hooks: autograd's own (non-private) weight
+    gradients kept, as in the reference and by default, and switched off during forward
+    (``autograd_weight_grads=False``)."""
+    from opacus_amd.grad_sample.grad_sample_module import GradSampleHooks
+
+    monkeypatch.setattr(GradSampleHooks, "DEFAULT_AUTOGRAD_WEIGHT_GRADS", request.param)
+    return request.param
+
+
 def per_sample_grads_cpu(model, x, y, loss_fn, batch_dim=0):
     """Batch-of-one autograd on the CPU: the reference's microbatch oracle."""
     names = [k for k, p in model.named_parameters() if p.requires_grad]
@@ -1089,3 +1100,67 @@ def test_mixed_precision_dtypes(A):
     ol.step()
     for p in low.parameters():
         assert p.grad.dtype == torch.bfloat16 and p.grad_sample.dtype == torch.bfloat16
+
+
+# ---- what backward() leaves behind, and activation checkpointing --------------------------------
+def test_p_grad_after_backward_is_the_non_private_sum_by_default(A, weight_grad_mode):
+    """grad_sample_module.py:291-365 adds hooks and leaves autograd alone: after ``backward()`` a
+    caller finds the plain summed gradient in ``p.grad`` until ``DPOptimizer.step`` replaces it.
+    That is the default here as well; ``autograd_weight_grads=False`` leaves ``None`` there."""
+    torch.manual_seed(3)
+    net = SmallCNN()
+    x, y = torch.randn(6, 1, 28, 28), torch.randint(0, 10, (6,))
+    plain = copy.deepcopy(net).to(DEV)
+    F.cross_entropy(plain(x.to(DEV)), y.to(DEV)).backward()
+    gsm = A.GradSampleModule(net.to(DEV))
+    opt = A.DPOptimizer(torch.optim.SGD(gsm.parameters(), lr=0.1), noise_multiplier=0.0, max_grad_norm=1e9, expected_batch_size=6)
+    F.cross_entropy(gsm(x.to(DEV)), y.to(DEV)).backward()
+    for (k, p), q in zip(gsm._module.named_parameters(), plain.parameters()):
+        assert p.grad_sample is not None and p.grad_sample.shape[0] == 6
+        if weight_grad_mode:
+            close(p.grad, q.grad, 1e-4, 1e-6, k)
+        else:
+            assert p.grad is None, k
+    opt.step()  # either way the step writes the (here unclipped) mean of the per-sample gradients
+    for (k, p), q in zip(gsm._module.named_parameters(), plain.parameters()):
+        close(p.grad, q.grad, 1e-4, 1e-6, k)
+
+
+def test_hooked_layers_under_activation_checkpointing(A):
+    """A block run through ``torch.utils.checkpoint`` (the re-entrant form, whose first forward runs
+    without grad so that the hooks see the block once, in the recomputation): per-sample gradients
+    and the step's gradient equal those of the same model without checkpointing."""
+    from torch.utils.checkpoint import checkpoint
+
+    class Net(nn.Module):
+        def __init__(self, ckpt):
+            super().__init__()
+            self.inp = nn.Linear(12, 16)
+            self.block = nn.Sequential(nn.Linear(16, 32), nn.GELU(), nn.LayerNorm(32), nn.Linear(32, 16))
+            self.out = nn.Linear(16, 5)
+            self.ckpt = ckpt
+
+        def forward(self, x):
+            h = torch.tanh(self.inp(x))
+            h = checkpoint(self.block, h, use_reentrant=True) if self.ckpt else self.block(h)
+            return self.out(h)
+
+    torch.manual_seed(11)
+    base = Net(False)
+    x, y = torch.randn(7, 9, 12), torch.randint(0, 5, (7,))
+    results = []
+    for ckpt in (False, True):
+        net = copy.deepcopy(base)
+        net.ckpt = ckpt
+        gsm = A.GradSampleModule(net.to(DEV))
+        opt = A.DPOptimizer(torch.optim.SGD(gsm.parameters(), lr=0.1), noise_multiplier=0.0, max_grad_norm=0.5, expected_batch_size=7)
+        F.cross_entropy(gsm(x.to(DEV)).mean(1), y.to(DEV)).backward()
+        gs = [p.grad_sample.detach().clone() for p in net.parameters()]
+        opt.step()
+        results.append((gs, [p.grad.detach().clone() for p in net.parameters()]))
+        assert all(p.requires_grad for p in net.parameters())
+    want = per_sample_grads_cpu(base, x, y, lambda out, t: F.cross_entropy(out.mean(1), t, reduction="sum"))
+    for (k, w), g0, g1, s0, s1 in zip(want.items(), results[0][0], results[1][0], results[0][1], results[1][1]):
+        close(g0, w, 1e-4, 1e-5, f"{k} without checkpointing")
+        close(g1, w, 1e-4, 1e-5, f"{k} with checkpointing")
+        close(s1, s0, 1e-4, 1e-6, f"{k} step gradient")

@@ -109,14 +109,15 @@ def test_mode_tables():
 # ---- wrapper behaviour --------------------------------------------------------------------
 def test_wrapper_surface():
     net = nn.Sequential(nn.Linear(4, 3), nn.ReLU(), nn.Linear(3, 2))
-    gsm = GradSampleModule(net)
+    gsm = GradSampleModule(net, autograd_weight_grads=False)
     assert all(k.startswith("_module.") for k in gsm.state_dict())
     assert gsm._module[0] is net[0]
     # per Linear: parameters off before forward, back on after it, and the capturing forward hook
     # (which hooks the output's gradient)
     assert len(net.autograd_grad_sample_hooks) == 6
-    with_autograd = GradSampleModule(nn.Sequential(nn.Linear(4, 3), nn.ReLU(), nn.Linear(3, 2)), autograd_weight_grads=True)
-    assert len(with_autograd._module.autograd_grad_sample_hooks) == 2
+    # the default keeps autograd's own weight gradients, as the reference does: one hook per layer
+    with_autograd = GradSampleModule(nn.Sequential(nn.Linear(4, 3), nn.ReLU(), nn.Linear(3, 2)))
+    assert with_autograd.autograd_weight_grads and len(with_autograd._module.autograd_grad_sample_hooks) == 2
     for p in net.parameters():
         assert p.grad_sample is None and p._forward_counter == 0
     with pytest.raises(ValueError, match="twice"):
@@ -192,13 +193,13 @@ def test_inplace_op_on_a_hooked_output_is_fine():
         want = (net.fc(x) > 0).float()  # d relu(y).sum() / dy
         assert torch.equal(seen["b"], want)
         torch.testing.assert_close(net.fc.weight.grad_sample.sum(0), net.fc.weight.grad)
-        # the default: the same per-sample gradients with the layer's parameters switched off
-        # during forward, an in-place op on the re-attached output included; autograd forms no
-        # weight gradient
+        # autograd_weight_grads=False: the same per-sample gradients with the layer's parameters
+        # switched off during forward, an in-place op on the re-attached output included; autograd
+        # forms no weight gradient
         first = net.fc.weight.grad_sample.clone()
         gsm.remove_hooks()
         net.zero_grad()
-        gsm = GradSampleModule(net, loss_reduction="sum")
+        gsm = GradSampleModule(net, loss_reduction="sum", autograd_weight_grads=False)
         gsm(x).sum().backward()
         assert torch.equal(seen["b"], want)
         torch.testing.assert_close(net.fc.weight.grad_sample, first)
@@ -210,7 +211,7 @@ def test_inplace_op_on_a_hooked_output_is_fine():
 
 def test_parameters_are_switched_back_on_whatever_happens():
     net = nn.Sequential(nn.Linear(3, 4), nn.ReLU(), nn.Linear(4, 2))
-    gsm = GradSampleModule(net)
+    gsm = GradSampleModule(net, autograd_weight_grads=False)
     with pytest.raises(RuntimeError):
         gsm(torch.randn(5, 7))  # wrong width: the first Linear raises inside forward
     assert all(p.requires_grad for p in net.parameters())
