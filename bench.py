@@ -250,7 +250,7 @@ def workload_c4(dev, autograd_weight_grads=False):
     )
 
 
-def _ghost_workload(dev, net, make_inputs, loss_call, n, T, sigma, desc, single=False):
+def _ghost_workload(dev, net, make_inputs, loss_call, n, T, sigma, desc, single=True):
     from opacus_amd import GradSampleModuleFastGradientClipping
     from opacus_amd.optimizers import DPOptimizerFastGradientClipping
 
@@ -268,15 +268,15 @@ def _ghost_workload(dev, net, make_inputs, loss_call, n, T, sigma, desc, single=
 
     flops = ghost_executed_flops(net, n, T)
     return dict(
-        step=step, n=n, dtype="bf16", workload=desc + (", single backward pass" if single else ""),
-        extra={"ghost_norm_executed_flops_per_step": flops},
+        step=step, n=n, dtype="bf16", workload=desc + (", one backward pass (library default)" if single else ", two backward passes (single_backward=False)"),
+        extra={"ghost_norm_executed_flops_per_step": flops, "single_backward": single},
         roofline=dict(kernel="ghost_norm_bf16_dlds_kernel<128x128, 2 stages> (all Linear layers of a step; thin layers by linear_dlds_kernel)",
                       timer="linear_ghost_norm", bound="mfma", work_per_step=flops, unit="TFLOP/s",
                       peak=MFMA_BF16_PEAK_TFLOPS, traffic=None),
     )
 
 
-def workload_c3(dev, single=False):
+def workload_c3(dev, single=True):
     from opacus_amd import DPLossFastGradientClipping
 
     torch.manual_seed(0)
@@ -296,7 +296,7 @@ def workload_c3(dev, single=False):
     )
 
 
-def workload_c5(dev, tied=False, single=False):
+def workload_c5(dev, tied=False, single=True):
     from opacus_amd import DPLossFastGradientClipping
 
     torch.manual_seed(0)
@@ -325,8 +325,8 @@ def workload_c5_tied(dev):
 WORKLOADS = {
     "c1": workload_c1, "c2": workload_c2, "c3": workload_c3, "c4": workload_c4, "c5": workload_c5,
     "c5t": workload_c5_tied,
-    # the same two with the clipped sum formed from the first backward pass (single_backward=True)
-    "c3s": lambda dev: workload_c3(dev, single=True), "c5s": lambda dev: workload_c5(dev, single=True),
+    # the same two with the reference's two backward passes (single_backward=False)
+    "c3p": lambda dev: workload_c3(dev, single=False), "c5p": lambda dev: workload_c5(dev, single=False),
     # c1 and c4 with the library's default hooks (autograd's own weight gradients kept, as in the reference)
     "c1d": lambda dev: workload_c1(dev, autograd_weight_grads=True),
     "c4d": lambda dev: workload_c4(dev, autograd_weight_grads=True),
@@ -786,9 +786,9 @@ def main() -> None:
                    "kernel_ms_per_step": head["kernel_ms_per_step"], **head["extra"]},
         "roofline": head["roofline"],
     }
-    cpu_ok = not args.no_cpu_baseline and head_name.rstrip("std") in ("c1", "c2", "c3", "c4", "c5")
+    cpu_ok = not args.no_cpu_baseline and head_name.rstrip("stdp") in ("c1", "c2", "c3", "c4", "c5")
     if cpu_ok:
-        out["cpu_baseline"] = cpu_baseline(head_name.rstrip("std"))
+        out["cpu_baseline"] = cpu_baseline(head_name.rstrip("stdp"))
     if args.workload is None and not args.headline_only:
         configs = {}
         for name, (k, wu) in OTHER_CONFIGS.items():
@@ -798,6 +798,10 @@ def main() -> None:
             entry = {key: r[key] for key in ("workload", "dtype", "global_batch", "steps", "warmup", "ms_per_step",
                                              "samples_per_s", "roofline")}
             entry.update(r["extra"])
+            if name + "p" in WORKLOADS:  # the same configuration with the reference's two backward passes
+                d = run_workload(name + "p", dev, k, wu, args.all_kernel_timers)
+                entry["two_backward_passes"] = {"ms_per_step": d["ms_per_step"], "samples_per_s": d["samples_per_s"],
+                                                "single_backward": False}
             if name + "d" in WORKLOADS:  # the same configuration with the library's default hooks
                 d = run_workload(name + "d", dev, k, wu, args.all_kernel_timers)
                 entry["default_hooks"] = {"ms_per_step": d["ms_per_step"], "samples_per_s": d["samples_per_s"],

@@ -12,14 +12,18 @@ altogether (:172-179): an ``nn.Embedding`` whose table is also the weight of an 
 (tied input and output embeddings). The norm of the sum of the two layers' gradients is
 their two ghost norms plus twice a cross term, ``kernels.tied_embedding_cross_term``.
 
-``single_backward=True`` replaces the second backward pass: the hooks keep every layer's
-(activations, backprops) of the first pass, and once the clipping coefficients are known the
+``single_backward=True`` (the default) replaces the second backward pass: the hooks keep every
+layer's (activations, backprops) of the first pass, and once the clipping coefficients are known the
 clipped gradient sum of each layer is formed from them directly: one GEMM
 ``(coef * b)^T a`` for a Linear layer, the weighted embedding backward for an Embedding, the
 layer's grad sampler and the clip-weighted sum for anything else. The sum is the one the
 second pass would have left in ``p.grad`` (the gradient of ``sum_n coef[n] loss[n]`` is linear
 in the per-sample backprops); what is saved is the pass's walk back through the activations,
-at the price of keeping the backprops alive until the coefficients exist.
+at the price of keeping the backprops alive until the coefficients exist (the first pass no
+longer retains the graph, so the peak is about that of the reference's retained graph).
+``single_backward=False`` runs the reference's two passes (fast_gradient_clipping_utils.py:179-201);
+it is the one to use when the loss depends on trainable parameters other than through the
+hooked layers, since only autograd's second pass sees such a dependence.
 
 Norm samples are kept in float32 whatever the dtype of the backprops (the kernels
 accumulate in fp32; rounding a norm to bf16 before it meets the other parameters' norms
@@ -81,7 +85,7 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
         force_functorch=False,
         max_grad_norm=1,
         use_ghost_clipping=True,
-        single_backward: bool = False,
+        single_backward: bool = True,
     ):
         super().__init__(
             m, batch_first=batch_first, loss_reduction=loss_reduction, strict=strict, force_functorch=force_functorch
@@ -396,7 +400,7 @@ class GradSampleModuleFastGradientClipping(GradSampleHooksFastGradientClipping, 
         force_functorch=False,
         max_grad_norm=1,
         use_ghost_clipping=True,
-        single_backward: bool = False,
+        single_backward: bool = True,
     ):
         nn.Module.__init__(self)
         GradSampleHooksFastGradientClipping.__init__(
