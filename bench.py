@@ -270,7 +270,8 @@ def _ghost_workload(dev, net, make_inputs, loss_call, n, T, sigma, desc, single=
     return dict(
         step=step, n=n, dtype="bf16", workload=desc + (", one backward pass (library default)" if single else ", two backward passes (single_backward=False)"),
         extra={"ghost_norm_executed_flops_per_step": flops, "single_backward": single},
-        roofline=dict(kernel="ghost_norm_bf16_dlds_kernel<128x128, 2 stages> (all Linear layers of a step; thin layers by linear_dlds_kernel)",
+        roofline=dict(kernel="ghost_norm_multi_kernel<128x128, 2 stages> (all Linear layers of a step pooled into one launch; thin layers by linear_dlds_kernel; "
+                             "ghost_norm_bf16_dlds_kernel layer by layer with two backward passes)",
                       timer="linear_ghost_norm", bound="mfma", work_per_step=flops, unit="TFLOP/s",
                       peak=MFMA_BF16_PEAK_TFLOPS, traffic=None),
     )
@@ -609,6 +610,23 @@ def kernel_table(dev, iters: int = 10, warm: int = 3, with_cpu: bool = True):
                       ms, "mfma_bf16", 2.0 * n * (direct if thin else gram),
                       cpu(lambda: O.linear_norm_sample(ca, cb), n, f"1 of {n} samples, bf16 bmm Grams"))
             del a, b
+    # ... and pooled: all Linear layers of a backward pass in one launch (what a ghost-clipping step runs)
+    for cfg, n, T, layers in (
+        ("C3 fc1 + fc2", 32, 512, [(1024, 4096), (4096, 1024)]),
+        ("C5 all 29 Linear layers (k/v by the direct route)", 16, 1024,
+         [(2048, 2048), (2048, 512), (2048, 512), (2048, 2048), (2048, 5632), (2048, 5632), (5632, 2048)] * 4 + [(2048, 32000)]),
+    ):
+        tri, full = tri_tiles(T)
+        items, work = [], 0.0
+        for i, o in layers:
+            a = torch.randn(n, T, i, device=dev).bfloat16()
+            b = (torch.randn(n, T, o, device=dev) * 0.02).bfloat16()
+            items.append((b, a, 1.0, torch.empty(n, device=dev), None))
+            gram, direct = T * T * (i + o) * tri / full, float(T) * i * o
+            work += 2.0 * n * (direct if direct < 0.9 * gram else gram)
+        yield row("linear_ghost_norm_multi", "a2", f"{cfg} pooled, n={n} T={T} bf16",
+                  timed(lambda: K.linear_ghost_norm_multi(items)), "mfma_bf16", work)
+        del items
     # the same kernel on fp32 operands
     tri, full = tri_tiles(1024)
     a = torch.randn(16, 1024, 2048, device=dev)

@@ -109,6 +109,27 @@ int dpk_linear_ghost_norm(const void* b, const void* a, int dtype, float* norm_w
                           int64_t n, int64_t T, int64_t out, int64_t in, float scale, int route,
                           void* ws, size_t ws_bytes, dpk_stream_t stream);
 
+/* The ghost norms of several Linear layers in one call: all layers of a backward pass, say,
+ * once their backprops exist (linear.py:54-93 for each of them). One layer's launch is a few
+ * hundred tile pairs, which leaves the device's last round of blocks mostly empty; pooled, the
+ * tile pairs of all layers fill the rounds, longest first. Layers share the batch size n and
+ * the dtype; each has its own T, sizes, outputs (either may be NULL) and scale. A layer the
+ * pooled kernel does not take (T == 1, a thin layer, odd feature sizes) is served as by
+ * dpk_linear_ghost_norm inside the same call. Results equal dpk_linear_ghost_norm's to
+ * rounding. `layers` is a host array of at most DPK_GHOST_MULTI_MAX entries; ws 256-byte aligned. */
+#define DPK_GHOST_MULTI_MAX 256
+typedef struct dpk_ghost_layer {
+  const void* b;  /* [n,T,out] */
+  const void* a;  /* [n,T,in] */
+  float* norm_w;  /* [n] or NULL */
+  float* norm_b;  /* [n] or NULL */
+  int64_t T, out, in;
+  float scale;
+} dpk_ghost_layer;
+size_t dpk_linear_ghost_norm_multi_workspace_bytes(const dpk_ghost_layer* layers /*host*/, int count, int64_t n);
+int dpk_linear_ghost_norm_multi(const dpk_ghost_layer* layers /*host*/, int count, int dtype, int64_t n,
+                                void* ws, size_t ws_bytes, dpk_stream_t stream);
+
 /* dpk_linear_ghost_norm for callers that cannot allocate device memory or pass a
  * workspace: code under HIP graph capture, tight serving loops, harnesses that forbid
  * hipMalloc. It has no counterpart in the reference. Same arguments, results and kernels;

@@ -22,6 +22,16 @@ DPK_MULTI_MAX = 48
 DPK_TILE_AUTO, DPK_TILE_128, DPK_TILE_256 = 0, 128, 256
 DPK_ROUTE_AUTO, DPK_ROUTE_GRAM, DPK_ROUTE_DIRECT = 0, 1, 2
 DPK_STATIC_SCRATCH_BYTES = 8 << 20
+DPK_GHOST_MULTI_MAX = 256
+
+
+class GhostLayer(ctypes.Structure):
+    """``dpk_ghost_layer`` of include/dpk.h."""
+
+    _fields_ = [
+        ("b", c_void_p), ("a", c_void_p), ("norm_w", c_void_p), ("norm_b", c_void_p),
+        ("T", c_int64), ("out", c_int64), ("inp", c_int64), ("scale", c_float),
+    ]
 
 STATUS_NAMES = {
     0: "DPK_OK",
@@ -46,6 +56,8 @@ SIGNATURES = {
     "dpk_linear_bias_gs": (c_int, [_P, c_int, _P, c_int, _P, _I, _I, _I, c_float, _P]),
     "dpk_linear_ghost_norm_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
     "dpk_linear_ghost_norm": (c_int, [_P, _P, c_int, _P, _P, _I, _I, _I, _I, c_float, c_int, _P, c_size_t, _P]),
+    "dpk_linear_ghost_norm_multi_workspace_bytes": (c_size_t, [_P, c_int, _I]),
+    "dpk_linear_ghost_norm_multi": (c_int, [_P, c_int, c_int, _I, _P, c_size_t, _P]),
     "dpk_linear_ghost_norm_static": (c_int, [_P, _P, c_int, _P, _P, _I, _I, _I, _I, c_float, c_int, _P]),
     "dpk_conv2d_gs_workspace_bytes": (c_size_t, [_I, _I, _I, _I, _I, _I]),
     "dpk_conv2d_gs": (

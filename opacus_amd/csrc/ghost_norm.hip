@@ -9,6 +9,7 @@
 // ti <= tj are visited and off-diagonal ones count twice. One float per block
 // goes to the workspace; a fixed-order reduction applies clamp(min=0) and sqrt
 // (linear.py:87-89, :92).
+#include <cstring>
 #include <mutex>
 
 #include "dpk_common.h"
@@ -126,28 +127,17 @@ constexpr bool ghost_cfg_has_quadrants() {
   return C::BM == 128 && C::BN == 128 && C::BK == 64 && C::kWaves == 4 && C::kStages == 2;
 }
 
+// One work unit: tile pair `pair` of one sample of one layer, as a whole 128 x 128 tile (big) or
+// as quadrant `quad` of it. The partial sums of unit `unit_index` (sample * npairs + pair) go
+// to pw / pb at unit_index * slots (+ quad).
 // TE: bf16_t, or float (a stage row of 128 bytes is then 32 k values).
-template <class C, typename TE = bf16_t>
-__global__ __launch_bounds__(C::kThreads) void ghost_norm_bf16_dlds_kernel(
-    const TE* __restrict__ b, const TE* __restrict__ a, float* __restrict__ pw,
-    float* __restrict__ pb, int64_t T, int64_t Dout, int64_t Din, int nJ, int npairs, uint32_t nbig,
-    int slots) {
+template <class C, typename TE>
+__device__ __forceinline__ void ghost_unit(mb16d::Smem<C>& sm, float* red, const TE* __restrict__ bs,
+                                           const TE* __restrict__ as, float* __restrict__ pw,
+                                           float* __restrict__ pb, int64_t T, int64_t Dout, int64_t Din, int nJ,
+                                           int pair, bool big, uint32_t quad, size_t unit_index, int slots) {
   constexpr int R = C::BM / C::BN;
   constexpr bool kQuadrants = ghost_cfg_has_quadrants<C>();
-  __shared__ mb16d::Smem<C> sm;
-  __shared__ float red[C::kWaves];
-  const bool big = !kQuadrants || blockIdx.x < nbig;
-  uint32_t unit, quad = 0;
-  if (big) {
-    unit = xcd_contiguous_id(blockIdx.x, nbig);
-  } else {
-    // nbig is a multiple of 8, so the low bits still name the XCD
-    const uint32_t sid = xcd_contiguous_id(blockIdx.x - nbig, gridDim.x - nbig);
-    unit = nbig + (sid >> 2);
-    quad = sid & 3u;
-  }
-  const int64_t sample = unit / static_cast<uint32_t>(npairs);
-  int pair = static_cast<int>(unit % static_cast<uint32_t>(npairs));
   int I = 0;
   while (pair >= nJ - R * I) {
     pair -= nJ - R * I;
@@ -157,10 +147,8 @@ __global__ __launch_bounds__(C::kThreads) void ghost_norm_bf16_dlds_kernel(
   const float weight = J < R * (I + 1) ? 1.f : 2.f;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int kh = lane >> 5, l32 = lane & 31;
-  const TE* bs = b + sample * T * Dout;
-  const TE* as = a + sample * T * Din;
   float sw = 0.f, sb = 0.f;
-  size_t slot;
+  size_t slot = unit_index * slots;
   if (big) {
     const int64_t m0a = static_cast<int64_t>(I) * C::BM, m0b = static_cast<int64_t>(J) * C::BN;
     const int wm0 = (wave / C::kWaveCols) * 64, wn0 = (wave % C::kWaveCols) * 64;
@@ -185,12 +173,11 @@ __global__ __launch_bounds__(C::kThreads) void ghost_norm_bf16_dlds_kernel(
             sw = fmaf(g, ta.acc[i][j][v], sw);
           }
         }
-    slot = static_cast<size_t>(unit) * slots;
   } else if constexpr (kQuadrants) {
     // quadrant (quad >> 1, quad & 1) of the unit's tile; R == 1 on this path
     const int64_t m0a = static_cast<int64_t>(I) * C::BM + (quad >> 1) * 64;
     const int64_t m0b = static_cast<int64_t>(J) * C::BN + (quad & 1u) * 64;
-    slot = static_cast<size_t>(unit) * slots + quad;
+    slot += quad;
     if (m0a < T && m0b < T) {  // block-uniform
       mb16d::Tile t;
       t.clear();
@@ -225,6 +212,104 @@ __global__ __launch_bounds__(C::kThreads) void ghost_norm_bf16_dlds_kernel(
     if (threadIdx.x == 0) pb[slot] = s * weight;
     if (big && slots > 1 && threadIdx.x < slots && threadIdx.x > 0) pb[slot + threadIdx.x] = 0.f;
   }
+}
+
+template <class C, typename TE = bf16_t>
+__global__ __launch_bounds__(C::kThreads) void ghost_norm_bf16_dlds_kernel(
+    const TE* __restrict__ b, const TE* __restrict__ a, float* __restrict__ pw,
+    float* __restrict__ pb, int64_t T, int64_t Dout, int64_t Din, int nJ, int npairs, uint32_t nbig,
+    int slots) {
+  constexpr bool kQuadrants = ghost_cfg_has_quadrants<C>();
+  __shared__ mb16d::Smem<C> sm;
+  __shared__ float red[C::kWaves];
+  const bool big = !kQuadrants || blockIdx.x < nbig;
+  uint32_t unit, quad = 0;
+  if (big) {
+    unit = xcd_contiguous_id(blockIdx.x, nbig);
+  } else {
+    // nbig is a multiple of 8, so the low bits still name the XCD
+    const uint32_t sid = xcd_contiguous_id(blockIdx.x - nbig, gridDim.x - nbig);
+    unit = nbig + (sid >> 2);
+    quad = sid & 3u;
+  }
+  const int64_t sample = unit / static_cast<uint32_t>(npairs);
+  const int pair = static_cast<int>(unit % static_cast<uint32_t>(npairs));
+  ghost_unit<C, TE>(sm, red, b + sample * T * Dout, a + sample * T * Din, pw, pb, T, Dout, Din, nJ, pair, big, quad,
+                    unit, slots);
+}
+
+// ---- several layers in one launch ------------------------------------------------------
+// The ghost norms of one layer at a benchmark shape are a launch of a few hundred units on
+// 512 resident blocks: its last round of blocks is mostly empty, and every layer pays that
+// again. Pooled, the units of all layers of a backward pass fill the rounds, and the one
+// tail is cut into quadrant blocks. Layers are given in descending order of feature count,
+// so that every XCD starts with its longest units.
+//
+// Hardware block id i runs on XCD i % 8, and an XCD takes its blocks in id order. XCD x is
+// given the samples [s0[x], s0[x] + cnt[x]) of every layer (units that share a sample's
+// rows share that XCD's L2), layer after layer: `len[x]` units, of which the last `tail[x]`
+// are run as four quadrant blocks each.
+constexpr int kGhostMultiMax = 32;               // layers per launch
+constexpr int kGhostMultiLayers = DPK_GHOST_MULTI_MAX;  // layers per call (several launches)
+
+struct GhostMultiArgs {
+  const void* b[kGhostMultiMax];
+  const void* a[kGhostMultiMax];  // NULL: no weight norm for this layer
+  float* pw[kGhostMultiMax];
+  float* pb[kGhostMultiMax];
+  int32_t T[kGhostMultiMax], Dout[kGhostMultiMax], Din[kGhostMultiMax], nJ[kGhostMultiMax], npairs[kGhostMultiMax];
+  uint32_t pair_prefix[kGhostMultiMax + 1];  // tile pairs per sample of the layers before this one
+  int32_t nlayers, slots;
+  uint32_t s0[8], cnt[8], len[8], tail[8];
+};
+
+template <class C, typename TE>
+__global__ __launch_bounds__(C::kThreads) void ghost_norm_multi_kernel(const GhostMultiArgs A) {
+  __shared__ mb16d::Smem<C> sm;
+  __shared__ float red[C::kWaves];
+  const uint32_t x = blockIdx.x & 7u, idx = blockIdx.x >> 3;
+  const uint32_t tail = A.tail[x], nbig = A.len[x] - tail;
+  if (idx >= nbig + 4u * tail) return;
+  const bool big = idx < nbig;
+  const uint32_t u = big ? idx : nbig + ((idx - nbig) >> 2);
+  const uint32_t quad = big ? 0u : ((idx - nbig) & 3u);
+  const uint32_t cnt = A.cnt[x];
+  int l = 0;
+  while (l + 1 < A.nlayers && u >= cnt * A.pair_prefix[l + 1]) ++l;
+  const uint32_t local = u - cnt * A.pair_prefix[l];
+  const uint32_t npairs = static_cast<uint32_t>(A.npairs[l]);
+  const int64_t sample = static_cast<int64_t>(A.s0[x]) + local / npairs;
+  const int pair = static_cast<int>(local % npairs);
+  const int64_t T = A.T[l], Dout = A.Dout[l], Din = A.Din[l];
+  const TE* a = static_cast<const TE*>(A.a[l]);
+  ghost_unit<C, TE>(sm, red, static_cast<const TE*>(A.b[l]) + sample * T * Dout, a ? a + sample * T * Din : nullptr,
+                    a ? A.pw[l] : nullptr, A.pb[l], T, Dout, Din, A.nJ[l], pair, big, quad,
+                    static_cast<size_t>(sample) * npairs + pair, A.slots);
+}
+
+// out = sqrt(max(0, sum of a row of partials)) * factor, for every layer's weight and bias
+// rows: one wave per (layer, which, sample), fixed order.
+struct GhostReduceArgs {
+  const float* part[2 * kGhostMultiMax];  // layer l: pw at 2 l, pb at 2 l + 1 (NULL: skip)
+  float* out[2 * kGhostMultiMax];
+  int32_t cols[kGhostMultiMax];
+  float factor[kGhostMultiMax];
+  int32_t nlayers, n;
+};
+
+__global__ __launch_bounds__(kThreads) void ghost_reduce_multi_kernel(const GhostReduceArgs A) {
+  const int64_t w = (static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x) / DPK_WAVE;
+  const int lane = threadIdx.x & (DPK_WAVE - 1);
+  if (w >= static_cast<int64_t>(A.nlayers) * 2 * A.n) return;
+  const int which = static_cast<int>(w / A.n), row = static_cast<int>(w % A.n), l = which >> 1;
+  const float* p = A.part[which];
+  if (!p) return;
+  const int cols = A.cols[l];
+  p += static_cast<int64_t>(row) * cols;
+  float s = 0.f;
+  for (int i = lane; i < cols; i += DPK_WAVE) s += p[i];
+  s = wave_sum(s);
+  if (lane == 0) A.out[which][row] = sqrtf(fmaxf(s, 0.f)) * A.factor[l];
 }
 
 // 128 x 128 tile, 4 waves, two 32 KB stages: two blocks fit a CU, which measured
@@ -285,6 +370,16 @@ bool direct_is_cheaper(int route, int64_t T, int64_t out, int64_t in) {
   const double direct = static_cast<double>(T) * static_cast<double>(in) * static_cast<double>(out);
   // the two routes run at about the same rate for either element type
   return direct < 0.9 * gram;
+}
+
+// Whether the direct-to-LDS tile kernel takes the layer: 128-row tiles, feature sizes that
+// fill whole 128-byte stage rows (64 bf16 or 32 fp32 values), 16-byte aligned operands, a
+// sample small enough for 32-bit byte offsets inside it.
+bool dlds_takes(const void* b, const void* a, int dtype, bool want_w, int64_t T, int64_t out, int64_t in) {
+  const int64_t widest = out > in ? out : in;
+  const int64_t es = dpk_elsize(dtype), kmul = 128 / es;
+  return T > 64 && out % kmul == 0 && (in % kmul == 0 || !want_w) && dpk_aligned(b, 16) && dpk_aligned(a, 16) &&
+         T * widest * es < (int64_t{1} << 32);
 }
 
 struct DirectLayout {
@@ -364,11 +459,8 @@ extern "C" int dpk_linear_ghost_norm(const void* b, const void* a, int dtype, fl
   const int64_t nt = dpk_cdiv(T, B);
   // bf16 with 64-aligned feature sizes takes the direct-to-LDS kernel
   // (and a sample small enough for 32-bit byte offsets inside it)
-  const int64_t widest = out > in ? out : in;
   // (fp32 too: 32 k values fill the 128-byte stage row that 64 bf16 do)
-  const int64_t es = dpk_elsize(dtype), kmul = 128 / es;
-  const bool dlds = B == 128 && out % kmul == 0 && (in % kmul == 0 || !norm_w) &&
-                    dpk_aligned(b, 16) && dpk_aligned(a, 16) && T * widest * es < (int64_t{1} << 32);
+  const bool dlds = dlds_takes(b, a, dtype, norm_w != nullptr, T, out, in);
   const int64_t npairs = dlds ? ghost_pairs(T, GhostCfg::BM, GhostCfg::BN) : nt * (nt + 1) / 2;
   const int64_t blocks = n * npairs;
   // A last round of resident blocks (two per CU) that is at most a quarter full is
@@ -445,6 +537,159 @@ extern "C" int dpk_linear_ghost_norm(const void* b, const void* a, int dtype, fl
   }
   if (pb) {
     dpk_launch_reduce_rows(pb, n, npairs * slots, norm_b, 1, absscale, s);
+    DPK_LAUNCH_CHECK(who);
+  }
+  return DPK_OK;
+}
+
+// ---- all Linear layers of a backward pass in one call ----------------------------------
+namespace {
+size_t multi_single_region(const dpk_ghost_layer* layers, int count, int64_t n) {
+  size_t m = 0;
+  for (int k = 0; k < count; ++k) {
+    const size_t need = dpk_linear_ghost_norm_workspace_bytes(n, layers[k].T, layers[k].out, layers[k].in);
+    m = need > m ? need : m;
+  }
+  return dpk_align_up(m, 256);
+}
+size_t multi_partials_bytes(int64_t n, int64_t T) {  // pw and pb of one pooled layer, four slots a unit
+  return dpk_align_up(static_cast<size_t>(2 * n * ghost_pairs(T, GhostCfg::BM, GhostCfg::BN) * 4) * sizeof(float), 256);
+}
+}  // namespace
+
+extern "C" size_t dpk_linear_ghost_norm_multi_workspace_bytes(const dpk_ghost_layer* layers, int count, int64_t n) {
+  if (!layers || count <= 0 || n <= 0) return 0;
+  size_t total = multi_single_region(layers, count, n);
+  for (int k = 0; k < count; ++k)
+    if (layers[k].T > 1) total += multi_partials_bytes(n, layers[k].T);
+  return total;
+}
+
+extern "C" int dpk_linear_ghost_norm_multi(const dpk_ghost_layer* layers, int count, int dtype, int64_t n,
+                                           void* ws, size_t ws_bytes, dpk_stream_t stream) {
+  const char* who = "dpk_linear_ghost_norm_multi";
+  DPK_REQUIRE(count >= 0 && count <= kGhostMultiLayers && n >= 0, DPK_E_SHAPE, "%s: count=%d (at most %d) n=%lld", who,
+              count, kGhostMultiLayers, (long long)n);
+  if (count == 0 || n == 0) return DPK_OK;
+  DPK_REQUIRE(layers, DPK_E_ARG, "%s: NULL layer table", who);
+  DPK_REQUIRE(dpk_dtype_ok(dtype), DPK_E_DTYPE, "%s: dtype %d", who, dtype);
+  const size_t need = dpk_linear_ghost_norm_multi_workspace_bytes(layers, count, n);
+  DPK_REQUIRE(need == 0 || (ws && ws_bytes >= need), DPK_E_WORKSPACE, "%s: workspace %zu < %zu bytes", who, ws_bytes,
+              need);
+  DPK_REQUIRE(dpk_aligned(ws, 256), DPK_E_ALIGN, "%s: workspace must be 256-byte aligned", who);
+  char* base = static_cast<char*>(ws);
+  const size_t single_region = multi_single_region(layers, count, n);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int cus = dpk_device_cus();
+  DPK_REQUIRE(cus > 0, DPK_E_LAUNCH, "%s: cannot query the device", who);
+
+  // Layers the tile kernel takes by the Gram route are pooled; every other layer (T == 1, thin
+  // layers on the direct route, feature sizes the tile kernel does not take) goes through the
+  // single-layer entry point, one after the other on the same stream and scratch.
+  int pooled[kGhostMultiLayers];
+  int npooled = 0;
+  for (int k = 0; k < count; ++k) {
+    const dpk_ghost_layer& L = layers[k];
+    DPK_REQUIRE(L.T >= 1 && L.out >= 1 && L.in >= 1, DPK_E_SHAPE, "%s: layer %d: T=%lld out=%lld in=%lld", who, k,
+                (long long)L.T, (long long)L.out, (long long)L.in);
+    if (!L.norm_w && !L.norm_b) continue;
+    DPK_REQUIRE(L.b && (L.a || !L.norm_w), DPK_E_ARG, "%s: layer %d: NULL tensor", who, k);
+    const bool pool = L.T > 1 && !(L.norm_w && direct_is_cheaper(DPK_ROUTE_AUTO, L.T, L.out, L.in)) &&
+                      dlds_takes(L.b, L.a, dtype, L.norm_w != nullptr, L.T, L.out, L.in) &&
+                      dpk_cdiv(L.T, 128) < 32768;
+    if (pool) {
+      pooled[npooled++] = k;
+    } else {
+      const int rc = dpk_linear_ghost_norm(L.b, L.a, dtype, L.norm_w, L.norm_b, n, L.T, L.out, L.in, L.scale,
+                                           DPK_ROUTE_AUTO, base, single_region, stream);
+      if (rc != DPK_OK) return rc;
+    }
+  }
+  if (npooled == 1) {  // nothing to pool with: the single-layer launch has the same kernel and its own tail
+    const dpk_ghost_layer& L = layers[pooled[0]];
+    return dpk_linear_ghost_norm(L.b, L.a, dtype, L.norm_w, L.norm_b, n, L.T, L.out, L.in, L.scale, DPK_ROUTE_GRAM,
+                                 base, single_region, stream);
+  }
+  // longest units first (insertion sort: a few dozen layers)
+  for (int i = 1; i < npooled; ++i) {
+    const int k = pooled[i];
+    const int64_t cost = layers[k].out + (layers[k].norm_w ? layers[k].in : 0);
+    int j = i;
+    for (; j > 0; --j) {
+      const dpk_ghost_layer& P = layers[pooled[j - 1]];
+      if (P.out + (P.norm_w ? P.in : 0) >= cost) break;
+      pooled[j] = pooled[j - 1];
+    }
+    pooled[j] = k;
+  }
+  // every layer with T > 1 has its partial-sum region at a fixed place in table order (the
+  // workspace query sums over exactly these), whichever of them end up pooled
+  size_t lay_off[kGhostMultiLayers];
+  {
+    size_t o = single_region;
+    for (int k = 0; k < count; ++k) {
+      lay_off[k] = o;
+      if (layers[k].T > 1) o += multi_partials_bytes(n, layers[k].T);
+    }
+  }
+  const uint32_t resident = static_cast<uint32_t>(2 * cus / 8);  // blocks an XCD holds at once
+  for (int c0 = 0; c0 < npooled; c0 += kGhostMultiMax) {
+    const int nl = npooled - c0 < kGhostMultiMax ? npooled - c0 : kGhostMultiMax;
+    GhostMultiArgs A;
+    GhostReduceArgs R;
+    memset(&A, 0, sizeof(A));
+    memset(&R, 0, sizeof(R));
+    A.nlayers = nl;
+    R.nlayers = nl;
+    R.n = static_cast<int32_t>(n);
+    uint32_t P = 0;
+    for (int i = 0; i < nl; ++i) {
+      const dpk_ghost_layer& L = layers[pooled[c0 + i]];
+      A.b[i] = L.b;
+      A.a[i] = L.norm_w ? L.a : nullptr;
+      A.T[i] = static_cast<int32_t>(L.T);
+      A.Dout[i] = static_cast<int32_t>(L.out);
+      A.Din[i] = static_cast<int32_t>(L.in);
+      A.nJ[i] = static_cast<int32_t>(dpk_cdiv(L.T, GhostCfg::BN));
+      A.npairs[i] = static_cast<int32_t>(ghost_pairs(L.T, GhostCfg::BM, GhostCfg::BN));
+      A.pair_prefix[i] = P;
+      P += static_cast<uint32_t>(A.npairs[i]);
+    }
+    A.pair_prefix[nl] = P;
+    DPK_REQUIRE(static_cast<uint64_t>(n) * P < (1ull << 28), DPK_E_SHAPE, "%s: too many tile pairs", who);
+    uint32_t longest = 0;
+    bool any_tail = false;
+    for (uint32_t x = 0; x < 8; ++x) {
+      A.s0[x] = static_cast<uint32_t>(x * n / 8);
+      A.cnt[x] = static_cast<uint32_t>((x + 1) * n / 8) - A.s0[x];
+      A.len[x] = A.cnt[x] * P;
+      const uint32_t r = resident > 0 ? A.len[x] % resident : 0;
+      A.tail[x] = (cus % 8 == 0 && r > 0 && r * 4 <= resident) ? r : 0;
+      any_tail = any_tail || A.tail[x] > 0;
+      const uint32_t blocks = A.len[x] - A.tail[x] + 4 * A.tail[x];
+      longest = blocks > longest ? blocks : longest;
+    }
+    A.slots = any_tail ? 4 : 1;
+    for (int i = 0; i < nl; ++i) {
+      const dpk_ghost_layer& L = layers[pooled[c0 + i]];
+      float* part = reinterpret_cast<float*>(base + lay_off[pooled[c0 + i]]);
+      const int64_t per = n * A.npairs[i] * A.slots;
+      A.pw[i] = L.norm_w ? part : nullptr;
+      A.pb[i] = L.norm_b ? part + per : nullptr;
+      R.part[2 * i] = A.pw[i];
+      R.part[2 * i + 1] = A.pb[i];
+      R.out[2 * i] = L.norm_w;
+      R.out[2 * i + 1] = L.norm_b;
+      R.cols[i] = A.npairs[i] * A.slots;
+      R.factor[i] = fabsf(L.scale);
+    }
+    const dim3 grid(8u * longest), block(GhostCfg::kThreads);
+    if (dtype == DPK_F32) hipLaunchKernelGGL((ghost_norm_multi_kernel<GhostCfg, float>), grid, block, 0, s, A);
+    else hipLaunchKernelGGL((ghost_norm_multi_kernel<GhostCfg, bf16_t>), grid, block, 0, s, A);
+    DPK_LAUNCH_CHECK(who);
+    const int64_t waves = static_cast<int64_t>(nl) * 2 * n;
+    hipLaunchKernelGGL(ghost_reduce_multi_kernel, dim3(static_cast<unsigned>(dpk_cdiv(waves, kWaves))), dim3(kThreads), 0,
+                       s, R);
     DPK_LAUNCH_CHECK(who);
   }
   return DPK_OK;

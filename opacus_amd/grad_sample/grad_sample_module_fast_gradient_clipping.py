@@ -92,6 +92,7 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
         )
         self.single_backward = single_backward
         self._kept_passes = []
+        self._pending_ghost = []
         self.trainable_parameters = [p for _, p in trainable_parameters(self._module)]
         self._tied_embedding_weights = self._find_tied_embedding_weights()
 
@@ -167,6 +168,7 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
         # records are made by backward hooks and consumed at the end of the same backward();
         # anything still here was left by one that did not get that far
         self._kept_passes = []
+        self._pending_ghost = []
         stack = list(args) + list(kwargs.values())
         while stack:
             t = stack.pop()
@@ -194,6 +196,52 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
         self._first_pass_open = False
         return leaves
 
+    # ---- Linear ghost norms of a whole pass in one launch ----------------------------------
+    def _defer_linear_ghost_norm(self, module: nn.Module, activations, backprops: torch.Tensor, scale: float):
+        """With ``single_backward`` the (activations, backprops) of every layer stay alive until
+        the coefficients exist anyway, so the Linear layers' norms need not be formed hook by
+        hook: the hook hands out the tensors that will hold them and queues the layer;
+        ``flush_ghost_norms`` forms them all in one pooled launch (the tile pairs of all layers
+        fill the device together, kernels.linear_ghost_norm_multi). Returns None when the layer
+        is not queued (another sampler is registered for it, an empty batch, dtypes the kernels
+        do not take)."""
+        from .linear import compute_linear_norm_sample
+
+        if (
+            not self.single_backward
+            or self.NORM_SAMPLERS.get(type(module)) is not compute_linear_norm_sample
+            or backprops.shape[0] == 0
+            or not backprops.is_cuda
+            or not kernels.supported_dtype(backprops.dtype)
+        ):
+            return None
+        n, dev = backprops.shape[0], backprops.device
+        want_w = module.weight.requires_grad
+        want_b = module.bias is not None and module.bias.requires_grad
+        nw = torch.empty((n,), dtype=torch.float32, device=dev) if want_w else None
+        nb = torch.empty((n,), dtype=torch.float32, device=dev) if want_b else None
+        if not self._pending_ghost:
+            # runs when the backward pass in flight has finished: the norms are in place by the
+            # time backward() returns, whoever reads p._norm_sample next
+            torch.autograd.Variable._execution_engine.queue_callback(self.flush_ghost_norms)
+        self._pending_ghost.append((backprops, activations[0], scale, nw, nb))
+        ret = {}
+        if want_w:
+            ret[module.weight] = nw
+        if want_b:
+            ret[module.bias] = nb
+        return ret
+
+    def flush_ghost_norms(self) -> None:
+        """Forms the queued Linear ghost norms (in place, in the tensors already handed out)."""
+        pending, self._pending_ghost = self._pending_ghost, []
+        groups = {}
+        for item in pending:
+            bp = item[0]
+            groups.setdefault((bp.shape[0], bp.dtype, bp.device), []).append(item)
+        for items in groups.values():
+            kernels.linear_ghost_norm_multi(items)
+
     # ---- clipping coefficient ----------------------------------------------------------
     def get_norm_sample(self) -> torch.Tensor:
         """Per-sample norm over all parameters: 2-norm of the stacked per-parameter norms
@@ -207,6 +255,7 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
         return coef
 
     def _norm_and_coef(self):
+        self.flush_ghost_norms()
         norm_samples = [p._norm_sample for p in self.trainable_parameters]
         if not norm_samples:
             raise ValueError("no trainable parameter carries a norm sample")
@@ -265,10 +314,13 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
         if self.single_backward and ghost:
             self._kept_passes.append((module, activations, backprops, scale, None))
         if ghost:
-            norm_samples = call_sampler(self.NORM_SAMPLERS[type(module)], module, activations, backprops, scale)
+            norm_samples = self._defer_linear_ghost_norm(module, activations, backprops, scale)
+            if norm_samples is None:
+                norm_samples = call_sampler(self.NORM_SAMPLERS[type(module)], module, activations, backprops, scale)
             for param, ns in norm_samples.items():
                 if param.requires_grad:
                     if id(param) in self._tied_embedding_weights:
+                        self.flush_ghost_norms()  # the cross term is combined with finished norms
                         ns = self._tied_embedding_norm(param, module, activations, backprops, scale, ns)
                     param._norm_sample = ns
                     param._forward_counter -= 1

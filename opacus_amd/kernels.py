@@ -215,6 +215,52 @@ def linear_ghost_norm(
     return nw, nb
 
 
+def linear_ghost_norm_multi(
+    items: Sequence[Tuple[torch.Tensor, torch.Tensor, float, Optional[torch.Tensor], Optional[torch.Tensor]]],
+) -> None:
+    """Ghost norms of several Linear layers in one call. Each item is ``(backprops, activations,
+    scale, norm_w, norm_b)`` with ``norm_w`` / ``norm_b`` preallocated float32 ``[n]`` tensors (or
+    None) that receive the results. All items share the batch size, dtype and device; the tile
+    pairs of all layers fill the device together instead of layer by layer."""
+    items = [it for it in items if it[3] is not None or it[4] is not None]
+    if not items:
+        return
+    dev = _need_gpu(*[t for it in items for t in (it[0], it[1])])
+    n, dt = items[0][0].shape[0], items[0][0].dtype
+    L = lib()
+    for lo in range(0, len(items), _lib.DPK_GHOST_MULTI_MAX):
+        chunk = items[lo : lo + _lib.DPK_GHOST_MULTI_MAX]
+        table = (_lib.GhostLayer * len(chunk))()
+        keep = []
+        for row, (bp, act, scale, nw, nb) in zip(table, chunk):
+            if bp.shape[0] != n or bp.dtype != dt:
+                raise ValueError("layers of one linear_ghost_norm_multi call must share batch size and dtype")
+            if act.dtype != dt:
+                act = act.to(dt)
+            out_f, in_f = bp.shape[-1], act.shape[-1]
+            b = _dense(bp).reshape(n, -1, out_f)
+            a = _dense(act).reshape(n, -1, in_f)
+            if a.shape[1] != b.shape[1]:
+                raise ValueError(f"activations {tuple(act.shape)} and backprops {tuple(bp.shape)} disagree")
+            for o in (nw, nb):
+                if o is not None and (o.dtype != torch.float32 or o.numel() != n or not o.is_contiguous()):
+                    raise ValueError("norm outputs must be dense float32 [n] tensors")
+            keep.append((a, b))
+            row.b, row.a = b.data_ptr(), a.data_ptr()
+            row.norm_w = None if nw is None else nw.data_ptr()
+            row.norm_b = None if nb is None else nb.data_ptr()
+            row.T, row.out, row.inp, row.scale = b.shape[1], out_f, in_f, float(scale)
+        if n == 0:
+            continue
+        ws, wsb = _ws(L.dpk_linear_ghost_norm_multi_workspace_bytes(table, len(chunk), n), dev)
+        with _timed("linear_ghost_norm", dev):
+            check(
+                "dpk_linear_ghost_norm_multi",
+                L.dpk_linear_ghost_norm_multi(table, len(chunk), _code(dt), n, _ptr(ws), wsb, _stream(dev)),
+            )
+        del keep
+
+
 # ---- nn.Conv2d ----------------------------------------------------------------------
 def conv2d_grad_sample(
     x: torch.Tensor,

@@ -405,6 +405,48 @@ def test_linear_ghost_norm_f32(K, n, T, fin, fout, scale, route):
     assert_rel(only_b[1], want_b, FP32_REL, "bias norm alone")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize(
+    "n,layers",
+    [
+        # (T, in, out, want_w, want_b): pooled tile layers of two lengths, a thin layer (direct route),
+        # odd feature sizes (register-staged kernel), T = 1, a bias-only layer
+        (3, [(200, 64, 128, True, True), (200, 128, 64, True, False), (130, 1024, 16, True, True),
+             (70, 40, 24, True, True), (1, 96, 64, True, True), (300, 64, 192, False, True)]),
+        # 16 samples: two per XCD; units of three layer shapes in one launch, ragged T
+        (16, [(1000, 64, 128, True, True), (1000, 128, 64, True, True), (520, 192, 64, True, False)]),
+        # 5 samples: XCDs with one sample and XCDs with none
+        (5, [(256, 128, 128, True, True), (256, 64, 256, True, True)]),
+        # 32 samples, 10 + 10 tile pairs each: 80 units per XCD = one round of 64 and a tail of 16 cut into quadrants
+        (32, [(512, 64, 128, True, True), (512, 128, 64, True, True)]),
+    ],
+)
+def test_linear_ghost_norm_multi_matches_layer_by_layer(K, dtype, n, layers):
+    """All layers of a pass in one call (the tile pairs of every layer share the launch, longest
+    first, the tail in quadrant blocks) against the float64 oracle and against one call per layer."""
+    torch.manual_seed(n * 31 + len(layers))
+    items, wants, singles = [], [], []
+    for T, fin, fout, want_w, want_b in layers:
+        a = torch.randn(n, T, fin).to(dtype)
+        b = (torch.randn(n, T, fout) * 0.1).to(dtype)
+        scale = 2.0 if fin == 64 else 1.0
+        ow, ob = O.linear_norm_sample(a.double(), (b.double() * scale))
+        nw = torch.full((n,), float("nan"), device="cuda") if want_w else None
+        nb = torch.full((n,), float("nan"), device="cuda") if want_b else None
+        items.append((dev(b), dev(a), scale, nw, nb))
+        wants.append((ow if want_w else None, ob if want_b else None))
+        singles.append(K.linear_ghost_norm(dev(b), dev(a), scale=scale, want_weight=want_w, want_bias=want_b))
+    K.linear_ghost_norm_multi(items)
+    bar = FP32_REL if dtype == torch.float32 else 1e-4  # bf16 inputs are exact, accumulation is fp32
+    for (_, _, _, nw, nb), (ow, ob), (sw, sb), lay in zip(items, wants, singles, layers):
+        for got, want, single, what in ((nw, ow, sw, "weight"), (nb, ob, sb, "bias")):
+            if want is None:
+                assert got is None
+                continue
+            assert_rel(got, want, bar, f"{what} norm of layer {lay}")
+            assert_rel(got, single, FP32_REL, f"{what} norm of layer {lay} against its own launch")
+
+
 def test_linear_ghost_norm_2d_inputs(K):
     torch.manual_seed(21)
     a, b = torch.randn(6, 50), torch.randn(6, 30)
