@@ -446,7 +446,10 @@ extern "C" int dpk_sumsq_rows_multi(const void* const* gs, const int64_t* P, int
   DPK_REQUIRE(blocks <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: %lld blocks exceed the grid limit", who,
               (long long)blocks);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  float* wsf = static_cast<float*>(ws);
+  // Rows of one chunk each (small parameters: norm layers, biases): the block's sum is the row's
+  // sum of squares and lands in sumsq directly, ws[n k + row] being sumsq[k n + row]; no second kernel.
+  const bool one_chunk = a.prefix[K] == K;
+  float* wsf = one_chunk ? sumsq : static_cast<float*>(ws);
   dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
   if (dtype == DPK_F32) {
     if (vec) hipLaunchKernelGGL((sumsq_partial_kernel<float, true>), grid, block, 0, s, a, n, wsf);
@@ -456,6 +459,7 @@ extern "C" int dpk_sumsq_rows_multi(const void* const* gs, const int64_t* P, int
     else hipLaunchKernelGGL((sumsq_partial_kernel<bf16_t, false>), grid, block, 0, s, a, n, wsf);
   }
   DPK_LAUNCH_CHECK(who);
+  if (one_chunk) return DPK_OK;
   const int64_t waves = K * n;
   hipLaunchKernelGGL(sumsq_final_kernel, dim3(static_cast<unsigned>(dpk_cdiv(waves, kWaves))), block,
                      0, s, a, n, wsf, sumsq);

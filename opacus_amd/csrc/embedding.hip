@@ -10,6 +10,18 @@
 // registers - a fixed order, no atomics, each row of b read exactly once. The
 // sorted-unique view the reference exposes (unique pairs + inverse index) is
 // derived from the same flags: rank[t] = number of distinct ids below ids[t].
+//
+// For samples of up to kSortMax positions the lists come from a sort: one block per sample
+// sorts its (id, position) pairs in LDS (bitonic network, ties broken by position), after
+// which equal ids are neighbours in increasing position. Longer samples take the pairwise
+// scan (quadratic in T, no LDS limit).
+//
+// The ghost norm does not walk the lists for every position: sum_v |sum_{t: id = v} b_t|^2
+// = sum_t |b_t|^2 + sum over ids that occur more than once of (|sum b_t|^2 - sum |b_t|^2).
+// The first term is one streaming pass over b at memory speed; the second touches only the
+// rows of repeated ids, which the leader of each list adds in the same kernel.
+#include <climits>
+
 #include "dpk_common.h"
 
 namespace {
@@ -104,6 +116,281 @@ __global__ __launch_bounds__(kThreads) void emb_link_kernel(const int64_t* __res
     leader[sample * T + t] = before ? 0 : 1;
     if (flag && V > 0 && (mine < 0 || mine >= V)) *flag = 1;
   }
+}
+
+// ---- lists by sorting: one block per sample, T <= kSortMax -------------------------------
+constexpr int kSortMax = 4096;  // (id, position) pairs of 12 bytes: 48 KB of LDS
+
+// next / leader as above; rank[t] = index of ids[t] among the sample's distinct ids in
+// ascending order and count[sample] = number of distinct ids (both only when rank != NULL).
+// flag (nullable): raised when an id lies outside [0, V) and V > 0.
+//
+// The sorting network runs on registers: thread t holds the E = np / 256 pairs with indices
+// t E .. t E + E - 1. A compare-exchange at distance j stays inside the thread for j < E,
+// meets the partner thread t ^ (j / E) of the same wave through a lane exchange for
+// j < 64 E, and goes through LDS (two barriers) only for the few stages beyond that.
+// Two element types: ids that all lie in [0, 2^51) - every vocabulary - are sorted as one
+// 64-bit word, id << 12 | position (T <= 4096), a third of the instructions per comparison;
+// any other ids as (id, position) pairs.
+struct IdPos {
+  int64_t key;
+  int32_t pos;
+  __device__ __forceinline__ bool less(const IdPos& y) const { return key < y.key || (key == y.key && pos < y.pos); }
+  __device__ __forceinline__ IdPos from_lane(int src) const {
+    IdPos o;
+    const uint32_t lo = __builtin_amdgcn_ds_bpermute(src, static_cast<int>(static_cast<uint32_t>(key)));
+    const uint32_t hi = __builtin_amdgcn_ds_bpermute(src, static_cast<int>(static_cast<uint32_t>(key >> 32)));
+    o.key = static_cast<int64_t>((static_cast<uint64_t>(hi) << 32) | lo);
+    o.pos = __builtin_amdgcn_ds_bpermute(src, pos);
+    return o;
+  }
+  __device__ __forceinline__ void put(int64_t* k, int32_t* p, int at) const {
+    k[at] = key;
+    p[at] = pos;
+  }
+  static __device__ __forceinline__ IdPos get(const int64_t* k, const int32_t* p, int at) {
+    IdPos o;
+    o.key = k[at];
+    o.pos = p[at];
+    return o;
+  }
+};
+struct Packed {
+  uint64_t w;  // id << 12 | position
+  __device__ __forceinline__ bool less(const Packed& y) const { return w < y.w; }
+  __device__ __forceinline__ Packed from_lane(int src) const {
+    Packed o;
+    const uint32_t lo = __builtin_amdgcn_ds_bpermute(src, static_cast<int>(static_cast<uint32_t>(w)));
+    const uint32_t hi = __builtin_amdgcn_ds_bpermute(src, static_cast<int>(static_cast<uint32_t>(w >> 32)));
+    o.w = (static_cast<uint64_t>(hi) << 32) | lo;
+    return o;
+  }
+  __device__ __forceinline__ void put(int64_t* k, int32_t*, int at) const { k[at] = static_cast<int64_t>(w); }
+  static __device__ __forceinline__ Packed get(const int64_t* k, const int32_t*, int at) {
+    Packed o;
+    o.w = static_cast<uint64_t>(k[at]);
+    return o;
+  }
+};
+
+// Bitonic network over np = E * kThreads elements, thread t holding elements t E .. t E + E - 1.
+// key / pos: exchange arrays of np entries for the stages whose partner is in another wave.
+template <int E, class Elem>
+__device__ __forceinline__ void bitonic_sort(Elem (&v)[E], int64_t* key, int32_t* pos) {
+  constexpr int np = E * kThreads;
+  const int tid = threadIdx.x;
+#pragma unroll 1
+  for (int k = 2; k <= np; k <<= 1) {
+    // distances that reach another thread, largest first
+#pragma unroll 1
+    for (int j = k >> 1; j >= E && j > 0; j >>= 1) {
+      const int d = j / E;  // partner thread = tid ^ d, same slot
+      const bool lower = (tid & d) == 0;
+      Elem o[E];
+      if (d < DPK_WAVE) {
+        // all lane exchanges of the stage in flight before the first comparison
+        const int src = ((tid & (DPK_WAVE - 1)) ^ d) << 2;
+#pragma unroll
+        for (int e = 0; e < E; ++e) o[e] = v[e].from_lane(src);
+      } else {
+        __syncthreads();  // earlier readers of the exchange arrays are done
+#pragma unroll
+        for (int e = 0; e < E; ++e) v[e].put(key, pos, e * kThreads + tid);
+        __syncthreads();
+#pragma unroll
+        for (int e = 0; e < E; ++e) o[e] = Elem::get(key, pos, e * kThreads + (tid ^ d));
+      }
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        const bool up = ((tid * E + e) & k) == 0;
+        // the lower index keeps the smaller element of an ascending pair
+        if (o[e].less(v[e]) == (lower == up)) v[e] = o[e];
+      }
+    }
+    // distances inside the thread's own E elements (compile-time, so that v stays in registers)
+#pragma unroll
+    for (int j = E >> 1; j > 0; j >>= 1) {
+      if (j >= k) continue;
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        if ((e & j) != 0) continue;  // the pair (e, e + j) once
+        const bool up = ((tid * E + e) & k) == 0;
+        const Elem lo = v[e], hi = v[e | j];
+        const bool swap = hi.less(lo) == up;
+        v[e] = swap ? hi : lo;
+        v[e | j] = swap ? lo : hi;
+      }
+    }
+  }
+}
+
+template <int E>
+__global__ __launch_bounds__(kThreads) void emb_sort_link_kernel(const int64_t* __restrict__ ids, int T, int64_t V,
+                                                                  int32_t* __restrict__ next,
+                                                                  int32_t* __restrict__ leader,
+                                                                  int32_t* __restrict__ rank,
+                                                                  int32_t* __restrict__ count,
+                                                                  int32_t* __restrict__ flag) {
+  constexpr int np = E * kThreads;
+  constexpr int64_t kPackLimit = int64_t{1} << 51;
+  __shared__ int64_t key[np];
+  __shared__ int32_t pos[np];
+  __shared__ int32_t runs[kThreads];
+  __shared__ int32_t wide;  // some id of the sample does not fit the packed form
+  const int64_t sample = blockIdx.x;
+  const int64_t* row = ids + sample * T;
+  const int tid = threadIdx.x;
+  if (tid == 0) wide = 0;
+  __syncthreads();
+  IdPos v[E];
+  bool bad = false, big = false;
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    const int i = tid * E + e;
+    const bool live = i < T;
+    v[e].key = live ? row[i] : INT64_MAX;
+    v[e].pos = live ? i : T + i;  // padding sorts behind every real pair, whatever its id
+    bad = bad || (live && V > 0 && (v[e].key < 0 || v[e].key >= V));
+    big = big || (live && (v[e].key < 0 || v[e].key >= kPackLimit));
+  }
+  if (bad && flag) *flag = 1;
+  if (big) wide = 1;
+  __syncthreads();
+  if (wide) {
+    bitonic_sort<E, IdPos>(v, key, pos);
+  } else {
+    Packed w[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e)  // real words stay below 2^63; padding lies above, behind every real id
+      w[e].w = v[e].pos < T ? (static_cast<uint64_t>(v[e].key) << 12) | static_cast<uint32_t>(v[e].pos)
+                            : (uint64_t{1} << 63) + static_cast<uint32_t>(v[e].pos);
+    bitonic_sort<E, Packed>(w, key, pos);
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      v[e].key = static_cast<int64_t>(w[e].w >> 12);
+      v[e].pos = static_cast<int32_t>(w[e].w & 0xfffu);
+    }
+  }
+  // sorted: equal ids are neighbours, positions ascending inside a run
+  __syncthreads();
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    key[tid * E + e] = v[e].key;
+    pos[tid * E + e] = v[e].pos;
+  }
+  __syncthreads();
+  const int lo = tid * E, hi = lo + E < T ? lo + E : T;
+  int32_t mine = 0;
+  for (int i = lo; i < hi; ++i) {
+    const bool lead = i == 0 || key[i - 1] != key[i];
+    mine += lead ? 1 : 0;
+    const int p = pos[i];
+    next[sample * T + p] = (i + 1 < T && key[i + 1] == key[i]) ? pos[i + 1] : -1;
+    leader[sample * T + p] = lead ? 1 : 0;
+  }
+  if (!rank) return;  // uniform
+  runs[tid] = mine;
+  __syncthreads();
+  int32_t before = 0;
+  for (int t = 0; t < tid; ++t) before += runs[t];
+  for (int i = lo; i < hi; ++i) {
+    if (i == 0 || key[i - 1] != key[i]) ++before;
+    rank[sample * T + pos[i]] = before - 1;
+  }
+  if (tid == kThreads - 1) count[sample] = before;
+}
+
+// ---- ghost norm as one streaming pass ---------------------------------------------------
+// grid = n * ceil(T / kStreamRows). A block owns kStreamRows consecutive positions of one
+// sample and all D columns: thread <-> one 16-byte chunk of a row per step of kThreads
+// chunks, all the block's rows of a step in flight at once. Leaders of a list with more than
+// one member add |sum b|^2 - sum |b|^2 over their list. The block's sum goes to
+// partials[block]; a row reduction in fixed order follows.
+constexpr int kStreamRows = 16;
+
+template <typename TIN> struct Chunk16;
+template <> struct Chunk16<float> {
+  static constexpr int kElems = 4;
+  static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
+    const dpk_vf4 r = __builtin_nontemporal_load(reinterpret_cast<const dpk_vf4*>(p));
+    v[0] = r.x; v[1] = r.y; v[2] = r.z; v[3] = r.w;
+  }
+};
+template <> struct Chunk16<bf16_t> {
+  static constexpr int kElems = 8;
+  typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+  static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[8]) {
+    const u4 r = __builtin_nontemporal_load(reinterpret_cast<const u4*>(p));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[2 * i] = __uint_as_float(r[i] << 16);
+      v[2 * i + 1] = __uint_as_float(r[i] & 0xffff0000u);
+    }
+  }
+};
+
+template <typename TIN>
+__global__ __launch_bounds__(kThreads) void emb_norm_stream_kernel(
+    const TIN* __restrict__ b, const int32_t* __restrict__ next, const int32_t* __restrict__ leader, int T, int64_t D,
+    int tch, float* __restrict__ partials) {
+  constexpr int E = Chunk16<TIN>::kElems;
+  __shared__ float red[kWaves];
+  __shared__ int32_t s_next[kStreamRows], s_lead[kStreamRows];
+  const int64_t sample = blockIdx.x / tch;
+  const int t0 = static_cast<int>(blockIdx.x % tch) * kStreamRows;
+  const int rows = T - t0 < kStreamRows ? T - t0 : kStreamRows;
+  const TIN* bs = b + sample * T * D;
+  if (threadIdx.x < kStreamRows) {
+    const bool live = static_cast<int>(threadIdx.x) < rows;
+    s_next[threadIdx.x] = live ? next[sample * T + t0 + threadIdx.x] : -1;
+    s_lead[threadIdx.x] = live ? leader[sample * T + t0 + threadIdx.x] : 0;
+  }
+  float ss = 0.f;
+  const int64_t chunks = D / E;  // D % E == 0 on this path
+  for (int64_t c = threadIdx.x; c < chunks; c += kThreads) {
+    const TIN* p = bs + static_cast<int64_t>(t0) * D + c * E;
+    if (rows == kStreamRows) {
+      float v[kStreamRows][E];
+#pragma unroll
+      for (int r = 0; r < kStreamRows; ++r) Chunk16<TIN>::load(p + r * D, v[r]);
+#pragma unroll
+      for (int r = 0; r < kStreamRows; ++r)
+#pragma unroll
+        for (int e = 0; e < E; ++e) ss = fmaf(v[r][e], v[r][e], ss);
+    } else {
+      for (int r = 0; r < rows; ++r) {
+        float v[E];
+        Chunk16<TIN>::load(p + r * D, v);
+#pragma unroll
+        for (int e = 0; e < E; ++e) ss = fmaf(v[e], v[e], ss);
+      }
+    }
+  }
+  __syncthreads();
+  // repeated ids: the list's leader replaces the members' sum of squares by the square of their sum
+  for (int r = 0; r < rows; ++r) {
+    if (!s_lead[r] || s_next[r] < 0) continue;  // uniform over the block
+    for (int64_t c = threadIdx.x; c < chunks; c += kThreads) {
+      float acc[E], sq = 0.f;
+#pragma unroll
+      for (int e = 0; e < E; ++e) acc[e] = 0.f;
+      for (int u = t0 + r; u >= 0; u = next[sample * T + u]) {
+        float v[E];
+        Chunk16<TIN>::load(bs + static_cast<int64_t>(u) * D + c * E, v);
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          acc[e] += v[e];
+          sq = fmaf(v[e], v[e], sq);
+        }
+      }
+      float whole = 0.f;
+#pragma unroll
+      for (int e = 0; e < E; ++e) whole = fmaf(acc[e], acc[e], whole);
+      ss += whole - sq;
+    }
+  }
+  const float s = block_sum<kWaves>(ss, red);
+  if (threadIdx.x == 0) partials[blockIdx.x] = s;
 }
 
 // rank[t] = #{leaders t' of the sample with ids[t'] < ids[t]}; count[sample] = #leaders.
@@ -308,12 +595,31 @@ int check_common(const char* who, const int64_t* ids, int64_t n, int64_t T, int6
   return DPK_OK;
 }
 
-// status: the caller's sticky flag (NULL: no range check), set when an id lies outside [0, V)
-void launch_link(const int64_t* ids, int64_t n, int64_t T, int64_t V, const EmbWs& w, int32_t* status,
-                 hipStream_t s) {
+bool sorts_in_lds(int64_t n, int64_t T) { return T <= kSortMax && n <= DPK_MAX_GRID_X; }
+
+// status: the caller's sticky flag (NULL: no range check), set when an id lies outside [0, V).
+// with_rank: also fill w.rank and w.count (the sorting kernel does it in passing; after the
+// pairwise scan the caller runs emb_rank_kernel). Returns whether the sorting kernel ran.
+bool launch_link(const int64_t* ids, int64_t n, int64_t T, int64_t V, const EmbWs& w, int32_t* status,
+                 bool with_rank, hipStream_t s) {
+  if (sorts_in_lds(n, T)) {
+    const dim3 grid(static_cast<unsigned>(n)), block(kThreads);
+    int32_t* rk = with_rank ? w.rank : nullptr;
+    int32_t* ct = with_rank ? w.count : nullptr;
+    const int Ti = static_cast<int>(T);
+#define DPK_SORT(E_) hipLaunchKernelGGL(emb_sort_link_kernel<E_>, grid, block, 0, s, ids, Ti, V, w.next, w.leader, rk, ct, status)
+    if (T <= 256) DPK_SORT(1);
+    else if (T <= 512) DPK_SORT(2);
+    else if (T <= 1024) DPK_SORT(4);
+    else if (T <= 2048) DPK_SORT(8);
+    else DPK_SORT(16);
+#undef DPK_SORT
+    return true;
+  }
   const int bps = static_cast<int>(dpk_cdiv(T, kLinkPositions));
   hipLaunchKernelGGL(emb_link_kernel, dim3(static_cast<unsigned>(n * bps)), dim3(kThreads), 0, s, ids, T,
                      V, bps, w.next, w.leader, status);
+  return false;
 }
 
 template <typename TIN, typename TOUT, int MODE>
@@ -351,11 +657,13 @@ extern "C" int dpk_embedding_unique_pairs(const int64_t* ids, int64_t n, int64_t
   int rc = check_common(who, ids, n, T, 0, ws, ws_bytes, &w);
   if (rc != DPK_OK) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  launch_link(ids, n, T, 0, w, nullptr, s);
+  const bool ranked = launch_link(ids, n, T, 0, w, nullptr, true, s);
   DPK_LAUNCH_CHECK(who);
-  const int bps = static_cast<int>(dpk_cdiv(T, kThreads));
-  hipLaunchKernelGGL(emb_rank_kernel, dim3(static_cast<unsigned>(n * bps)), dim3(kThreads), 0, s, ids, T,
-                     bps, w.leader, w.rank, w.count);
+  if (!ranked) {
+    const int bps = static_cast<int>(dpk_cdiv(T, kThreads));
+    hipLaunchKernelGGL(emb_rank_kernel, dim3(static_cast<unsigned>(n * bps)), dim3(kThreads), 0, s, ids, T,
+                       bps, w.leader, w.rank, w.count);
+  }
   hipLaunchKernelGGL(emb_prefix_kernel, dim3(1), dim3(64), 0, s, w.count, n, w.base, n_unique);
   hipLaunchKernelGGL(emb_emit_pairs_kernel, dim3(static_cast<unsigned>(dpk_cdiv(n * T, kThreads))),
                      dim3(kThreads), 0, s, ids, n, T, w.leader, w.rank, w.base, inverse, unique_pairs);
@@ -379,8 +687,23 @@ extern "C" int dpk_embedding_ghost_norm(const int64_t* ids, const void* b, int d
   const int64_t tch = dpk_cdiv(T, kLeadersPerBlock), dch = dpk_cdiv(D, kThreads * 4);
   DPK_REQUIRE(n * tch * dch <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: too many blocks", who);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  launch_link(ids, n, T, 0, w, nullptr, s);
+  const bool sorted = launch_link(ids, n, T, 0, w, nullptr, false, s);
   DPK_LAUNCH_CHECK(who);
+  const int64_t chunk = dtype == DPK_BF16 ? 8 : 4;
+  if (sorted && D % chunk == 0 && dpk_aligned(b, 16)) {
+    // one streaming pass over b, then the fixed-order sum of the blocks' partial sums
+    const dim3 grid(static_cast<unsigned>(n * tch)), block(kThreads);
+    if (dtype == DPK_F32)
+      hipLaunchKernelGGL(emb_norm_stream_kernel<float>, grid, block, 0, s, static_cast<const float*>(b), w.next,
+                         w.leader, static_cast<int>(T), D, static_cast<int>(tch), w.partials);
+    else
+      hipLaunchKernelGGL(emb_norm_stream_kernel<bf16_t>, grid, block, 0, s, static_cast<const bf16_t*>(b), w.next,
+                         w.leader, static_cast<int>(T), D, static_cast<int>(tch), w.partials);
+    DPK_LAUNCH_CHECK(who);
+    dpk_launch_reduce_rows(w.partials, n, tch, norm, 1, fabsf(scale), s);
+    DPK_LAUNCH_CHECK(who);
+    return DPK_OK;
+  }
   const bool vec = D % 4 == 0 && dpk_aligned(b, dtype == DPK_BF16 ? 8 : 16);
   if (dtype == DPK_F32) launch_walk<float, float, 0>(vec, ids, b, w, n, T, D, 0, scale, nullptr, s);
   else launch_walk<bf16_t, float, 0>(vec, ids, b, w, n, T, D, 0, scale, nullptr, s);
@@ -412,7 +735,7 @@ extern "C" int dpk_embedding_gs(const int64_t* ids, const void* b, int in_dtype,
   DPK_REQUIRE(dpk_aligned(status, 4), DPK_E_ALIGN, "%s: status misaligned", who);
   // Ids outside [0, V) would address memory outside gs: the walk below writes nothing for
   // them, and the link kernel raises the caller's flag.
-  launch_link(ids, n, T, V, w, status, s);
+  launch_link(ids, n, T, V, w, status, false, s);
   DPK_LAUNCH_CHECK(who);
   const size_t bytes = static_cast<size_t>(n) * V * D * dpk_elsize(gs_dtype);
   const int64_t n16 = dpk_aligned(gs, 16) ? static_cast<int64_t>(bytes / 16) : 0;

@@ -410,8 +410,9 @@ __global__ __launch_bounds__(kThreads) void colsum4_kernel(const TIN* __restrict
   }
 }
 
-// out[r] = scale * sum_q b[r,q]: one wave per row (conv bias, conv.py:117).
-template <typename TIN, typename TOUT>
+// out[r] = scale * sum_q b[r,q]: one wave per row (conv bias, conv.py:117). VEC: rows of whole,
+// aligned 4-element chunks, read four chunks a lane at a time with all of them in flight.
+template <typename TIN, typename TOUT, bool VEC>
 __global__ __launch_bounds__(kThreads) void rowsum_kernel(const TIN* __restrict__ b,
                                                             TOUT* __restrict__ out, int64_t rows,
                                                             int64_t q, float scale) {
@@ -420,7 +421,26 @@ __global__ __launch_bounds__(kThreads) void rowsum_kernel(const TIN* __restrict_
   if (w >= rows) return;
   const TIN* p = b + w * q;
   float s = 0.f;
-  for (int64_t i = lane; i < q; i += DPK_WAVE) s += dpk_io<TIN>::load(p + i);
+  if (VEC) {
+    constexpr int U = 4, kStep = DPK_WAVE * 4;
+    int64_t i = lane * 4;
+    for (; i + (U - 1) * kStep < q; i += U * kStep) {
+      typename dpk_io<TIN>::raw4 x[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) x[u] = dpk_io<TIN>::load4_raw(p + i + u * kStep);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const float4 v = dpk_io<TIN>::unpack4(x[u]);
+        s += (v.x + v.y) + (v.z + v.w);
+      }
+    }
+    for (; i < q; i += kStep) {
+      const float4 v = dpk_io<TIN>::unpack4(dpk_io<TIN>::load4_raw(p + i));
+      s += (v.x + v.y) + (v.z + v.w);
+    }
+  } else {
+    for (int64_t i = lane; i < q; i += DPK_WAVE) s += dpk_io<TIN>::load(p + i);
+  }
   s = wave_sum(s);
   if (lane == 0) dpk_io<TOUT>::store(out + w, s * scale);
 }
@@ -692,7 +712,30 @@ __global__ __launch_bounds__(kThreads) void rowsq_kernel(const T* __restrict__ v
   s = wave_sum(s);
   if (lane == 0) sumsq[w] = s;
 }
+// The same with a block per row and 4-element loads, for rows long enough to keep a block busy:
+// a lone wave walks a row of 4096 values in 64 dependent steps.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void rowsq_block_kernel(const T* __restrict__ v, float* __restrict__ sumsq,
+                                                                int64_t K) {
+  __shared__ float red[kWaves];
+  const T* p = v + static_cast<int64_t>(blockIdx.x) * K;
+  float s = 0.f;
+  for (int64_t i = threadIdx.x * 4; i < K; i += kThreads * 4) {
+    const float4 x = dpk_io<T>::load4(p + i);
+    s += (x.x * x.x + x.y * x.y) + (x.z * x.z + x.w * x.w);
+  }
+  const float t = block_sum<kWaves>(s, red);
+  if (threadIdx.x == 0) sumsq[blockIdx.x] = t;
+}
 void launch_rowsq(const void* v, int dtype, float* sumsq, int64_t rows, int64_t K, hipStream_t s) {
+  if (K >= 1024 && K % 4 == 0 && dpk_aligned(v, dtype == DPK_BF16 ? 8 : 16) && rows <= DPK_MAX_GRID_X) {
+    const dim3 grid(static_cast<unsigned>(rows)), block(kThreads);
+    if (dtype == DPK_F32)
+      hipLaunchKernelGGL(rowsq_block_kernel<float>, grid, block, 0, s, static_cast<const float*>(v), sumsq, K);
+    else
+      hipLaunchKernelGGL(rowsq_block_kernel<bf16_t>, grid, block, 0, s, static_cast<const bf16_t*>(v), sumsq, K);
+    return;
+  }
   const dim3 grid(static_cast<unsigned>(dpk_cdiv(rows, kWaves))), block(kThreads);
   if (dtype == DPK_F32)
     hipLaunchKernelGGL(rowsq_kernel<float>, grid, block, 0, s, static_cast<const float*>(v), sumsq, rows, K);
@@ -702,9 +745,13 @@ void launch_rowsq(const void* v, int dtype, float* sumsq, int64_t rows, int64_t 
 
 template <typename TIN, typename TOUT>
 void launch_rowsum(const void* b, void* out, int64_t rows, int64_t q, float scale, hipStream_t s) {
-  hipLaunchKernelGGL((rowsum_kernel<TIN, TOUT>), dim3(static_cast<unsigned>(dpk_cdiv(rows, kWaves))),
-                     dim3(kThreads), 0, s, static_cast<const TIN*>(b), static_cast<TOUT*>(out), rows,
-                     q, scale);
+  const dim3 grid(static_cast<unsigned>(dpk_cdiv(rows, kWaves))), block(kThreads);
+  if (q % 4 == 0 && dpk_aligned(b, 4 * sizeof(TIN)))
+    hipLaunchKernelGGL((rowsum_kernel<TIN, TOUT, true>), grid, block, 0, s, static_cast<const TIN*>(b),
+                       static_cast<TOUT*>(out), rows, q, scale);
+  else
+    hipLaunchKernelGGL((rowsum_kernel<TIN, TOUT, false>), grid, block, 0, s, static_cast<const TIN*>(b),
+                       static_cast<TOUT*>(out), rows, q, scale);
 }
 }  // namespace
 

@@ -577,7 +577,11 @@ def test_embedding_golden_vectors(K, embedding_norm_cases):
             assert inverse.cpu().tolist() == c["intermediates"]["new_index_positions"]
 
 
-@pytest.mark.parametrize("n,T,V", [(1, 1, 1), (7, 10, 6), (3, 300, 50), (2, 2500, 4000), (4, 513, 3)])
+# T up to 4096: lists by sorting in LDS (powers of two and their neighbours); beyond: the pairwise scan
+@pytest.mark.parametrize(
+    "n,T,V",
+    [(1, 1, 1), (7, 10, 6), (3, 300, 50), (2, 2500, 4000), (4, 513, 3), (2, 4096, 100), (3, 2, 5), (2, 4097, 3000), (1, 9000, 7)],
+)
 def test_embedding_unique_pairs_bit_exact(K, n, T, V):
     torch.manual_seed(n * T)
     ids = torch.randint(0, V, (n, T))
@@ -594,7 +598,13 @@ def test_embedding_unique_pairs_any_integer_ids(K):
     assert torch.equal(pairs.cpu(), want_pairs) and torch.equal(inverse.cpu(), want_inv)
 
 
-@pytest.mark.parametrize("n,Tshape,V,D", [(5, (3, 2), 9, 4), (3, (40,), 7, 17), (2, (300,), 5000, 64), (2, (64,), 10, 1030)])
+# D = 17, 1030: scalar walk; multiples of 4: the streaming norm kernel (ragged last block of rows with
+# T = 40, 300); T = 4500: lists by the pairwise scan and the walking norm kernel
+@pytest.mark.parametrize(
+    "n,Tshape,V,D",
+    [(5, (3, 2), 9, 4), (3, (40,), 7, 17), (2, (300,), 5000, 64), (2, (64,), 10, 1030), (3, (40,), 7, 1024),
+     (2, (4500,), 300, 8), (2, (33, 64), 50, 260)],
+)
 @pytest.mark.parametrize("scale", [1.0, 5.0])
 def test_embedding_grad_sample_and_norm_f32(K, n, Tshape, V, D, scale):
     torch.manual_seed(V + D)
