@@ -157,9 +157,15 @@ int dpk_linear_ghost_norm_static(const void* b, const void* a, int dtype, float*
  * unfold2d computes H_effective/W_effective), gs: [n,O,C/groups,KH,KW].
  * The unfolded activation matrix is never materialised. Padding is given per
  * side so that padding="same" (asymmetric, tensor_utils.py:128-134) is
- * expressible. sumsq as for dpk_linear_gs. */
+ * expressible. sumsq as for dpk_linear_gs; gs may be NULL when sumsq is given (norms only:
+ * the gradient tiles are formed and squared, never stored).
+ * Workspace: block sums for sumsq and, for a layer with few and long blocks (few kernel
+ * elements, many output positions: a network's first convolution), room for the pieces
+ * into which the contraction over the output positions is then cut. Q = OH * OW (times OD)
+ * tells the query how long that contraction is; Q = 0 asks for the block sums only, and a
+ * call that finds no room for the pieces runs unsplit. */
 size_t dpk_conv2d_gs_workspace_bytes(int64_t n, int64_t C, int64_t O, int64_t KH, int64_t KW,
-                                     int64_t groups);
+                                     int64_t groups, int64_t Q);
 int dpk_conv2d_gs(const void* x, const void* b, int in_dtype, void* gs, int gs_dtype, float* sumsq,
                   int64_t n, int64_t C, int64_t H, int64_t W, int64_t O, int64_t KH, int64_t KW,
                   int64_t sh, int64_t sw, int64_t ph_lo, int64_t ph_hi, int64_t pw_lo,
@@ -170,7 +176,7 @@ int dpk_conv2d_gs(const void* x, const void* b, int in_dtype, void* gs, int gs_d
  * x: [n,C,D,H,W], b: [n,O,OD,OH,OW], gs: [n,O,C/groups,KD,KH,KW]. kernel, stride,
  * pad_lo, pad_hi, dilation: host arrays of three values in (depth, height, width) order. */
 size_t dpk_conv3d_gs_workspace_bytes(int64_t n, int64_t C, int64_t O, int64_t KD, int64_t KH,
-                                     int64_t KW, int64_t groups);
+                                     int64_t KW, int64_t groups, int64_t Q);
 int dpk_conv3d_gs(const void* x, const void* b, int in_dtype, void* gs, int gs_dtype, float* sumsq,
                   int64_t n, int64_t C, int64_t D, int64_t H, int64_t W, int64_t O,
                   const int64_t* kernel /*host*/, const int64_t* stride /*host*/,

@@ -59,12 +59,12 @@ SIGNATURES = {
     "dpk_linear_ghost_norm_multi_workspace_bytes": (c_size_t, [_P, c_int, _I]),
     "dpk_linear_ghost_norm_multi": (c_int, [_P, c_int, c_int, _I, _P, c_size_t, _P]),
     "dpk_linear_ghost_norm_static": (c_int, [_P, _P, c_int, _P, _P, _I, _I, _I, _I, c_float, c_int, _P]),
-    "dpk_conv2d_gs_workspace_bytes": (c_size_t, [_I, _I, _I, _I, _I, _I]),
+    "dpk_conv2d_gs_workspace_bytes": (c_size_t, [_I, _I, _I, _I, _I, _I, _I]),
     "dpk_conv2d_gs": (
         c_int,
         [_P, _P, c_int, _P, c_int, _P] + [_I] * 16 + [c_float, _P, c_size_t, _P],
     ),
-    "dpk_conv3d_gs_workspace_bytes": (c_size_t, [_I, _I, _I, _I, _I, _I, _I]),
+    "dpk_conv3d_gs_workspace_bytes": (c_size_t, [_I, _I, _I, _I, _I, _I, _I, _I]),
     "dpk_conv3d_gs": (
         c_int,
         [_P, _P, c_int, _P, c_int, _P, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, c_float, _P, c_size_t, _P],

@@ -36,10 +36,11 @@ struct LoaderIm2col {
   static constexpr int PSTEP = mf32::NTHREADS / mf32::BK;
   const T* x;  // first channel of this sample's group
   ConvGeom g;
+  int qend;  // positions from here on read as zeros (the end of this block's share of the contraction)
   int kq, pl0;
   int off[R], dy[R], dx[R], dz[D3 ? R : 1];
   float st[R];
-  __device__ __forceinline__ LoaderIm2col(const T* x_, const ConvGeom& g_, int p0) : x(x_), g(g_) {
+  __device__ __forceinline__ LoaderIm2col(const T* x_, const ConvGeom& g_, int p0, int qend_) : x(x_), g(g_), qend(qend_) {
     kq = threadIdx.x % mf32::BK;
     pl0 = threadIdx.x / mf32::BK;
 #pragma unroll
@@ -73,7 +74,7 @@ struct LoaderIm2col {
     }
     const int oh = q2 / g.OW, ow = q2 - oh * g.OW;
     const int iy0 = oh * g.sh, ix0 = ow * g.sw;
-    const bool inq = q < g.Q;
+    const bool inq = q < qend;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const int iy = iy0 + dy[r], ix = ix0 + dx[r];
@@ -94,15 +95,22 @@ struct LoaderIm2col {
   }
 };
 
+// ksplit > 1: the contraction over the output positions is cut into ksplit pieces of kchunk
+// positions (a multiple of the k tile), one block each; the raw tiles go to
+// split_out[piece, n, O, Pg] and conv_split_reduce_kernel adds them. A layer with few, long
+// blocks (a network's first convolution: three column tiles and 12,544 positions) fills the
+// device that way. gs == NULL (norm only): nothing is stored, the squares are still summed.
 template <int BM, int BN, typename TIN, typename TOUT, bool VEC, bool D3>
 __global__ __launch_bounds__(kThreads) void conv2d_gs_kernel(
     const TIN* __restrict__ x, const TIN* __restrict__ b, TOUT* __restrict__ gs,
     float* __restrict__ partials, ConvGeom g, int C, int O, int groups, float scale, int tiles_m,
-    int tiles_n) {
+    int tiles_n, int ksplit, int kchunk, float* __restrict__ split_out, int64_t n) {
   __shared__ mf32::Smem<BM, BN> sm;
   __shared__ float red[kWaves];
   const int Og = O / groups, Cg = C / groups;
   int64_t bid = blockIdx.x;
+  const int piece = static_cast<int>(bid % ksplit);
+  bid /= ksplit;
   const int tn = static_cast<int>(bid % tiles_n);
   bid /= tiles_n;
   const int tm = static_cast<int>(bid % tiles_m);
@@ -110,26 +118,61 @@ __global__ __launch_bounds__(kThreads) void conv2d_gs_kernel(
   const int grp = static_cast<int>(bid % groups);
   const int64_t sample = bid / groups;
   const int m0 = tm * BM, p0 = tn * BN;
+  const int kb = piece * kchunk;
+  const int ke = kb + kchunk < g.Q ? kb + kchunk : g.Q;
   const TIN* bg = b + (sample * O + static_cast<int64_t>(grp) * Og) * g.Q;
   const TIN* xg = x + (sample * C + static_cast<int64_t>(grp) * Cg) * g.Dd * g.H * g.W;
-  mf32::LoaderKContig<BM, TIN, VEC> la(bg, g.Q, m0, Og, g.Q);
-  LoaderIm2col<BN, TIN, D3> lb(xg, g, p0);
+  mf32::LoaderKContig<BM, TIN, VEC> la(bg, g.Q, m0, Og, ke);
+  LoaderIm2col<BN, TIN, D3> lb(xg, g, p0, ke);
   mf32::Tile<BM, BN> tile;
   tile.clear();
-  mf32::mainloop<BM, BN>(tile, sm, la, lb, g.Q);
+  mf32::mainloop<BM, BN>(tile, sm, la, lb, kb, ke);
+  if (split_out) {
+    float* out = split_out + ((static_cast<int64_t>(piece) * n + sample) * O + static_cast<int64_t>(grp) * Og) * g.Pg;
+    tile.for_each([&](int r, int c, float v) {
+      const int m = m0 + r, p = p0 + c;
+      if (m < Og && p < g.Pg) out[static_cast<int64_t>(m) * g.Pg + p] = v;
+    });
+    return;
+  }
   TOUT* out = gs + (sample * O + static_cast<int64_t>(grp) * Og) * g.Pg;
   float ss = 0.f;
   tile.for_each([&](int r, int c, float v) {
     const int m = m0 + r, p = p0 + c;
     if (m < Og && p < g.Pg) {
       const float val = v * scale;
-      dpk_io<TOUT>::store(out + static_cast<int64_t>(m) * g.Pg + p, val);
+      if (gs) dpk_io<TOUT>::store(out + static_cast<int64_t>(m) * g.Pg + p, val);
       ss = fmaf(val, val, ss);
     }
   });
   if (partials) {
     const float s = block_sum<kWaves>(ss, red);
     if (threadIdx.x == 0) partials[blockIdx.x] = s;
+  }
+}
+
+// gs[sample, i] = scale * sum over the pieces of split[piece, sample, i], i < O * Pg, and the
+// block's sum of squares of what it wrote. grid = n * chunks, kSplitChunk elements a block.
+constexpr int kSplitChunk = 4096;
+template <typename TOUT>
+__global__ __launch_bounds__(kThreads) void conv_split_reduce_kernel(const float* __restrict__ split,
+                                                                      TOUT* __restrict__ gs,
+                                                                      float* __restrict__ partials, int64_t n,
+                                                                      int64_t OP, int ksplit, int chunks, float scale) {
+  __shared__ float red[kWaves];
+  const int64_t sample = blockIdx.x / chunks;
+  const int64_t i0 = static_cast<int64_t>(blockIdx.x % chunks) * kSplitChunk;
+  float ss = 0.f;
+  for (int64_t i = i0 + threadIdx.x; i < i0 + kSplitChunk && i < OP; i += kThreads) {
+    float v = 0.f;
+    for (int s = 0; s < ksplit; ++s) v += split[(static_cast<int64_t>(s) * n + sample) * OP + i];
+    v *= scale;
+    if (gs) dpk_io<TOUT>::store(gs + sample * OP + i, v);
+    ss = fmaf(v, v, ss);
+  }
+  if (partials) {
+    const float t = block_sum<kWaves>(ss, red);
+    if (threadIdx.x == 0) partials[blockIdx.x] = t;
   }
 }
 
@@ -386,7 +429,7 @@ __global__ __launch_bounds__(kThreads) void conv2d_gs_patch_kernel(
     const int m = m0 + r, p = p0 + c;
     if (m < Og && p < g.Pg) {
       const float val = v * scale;
-      dpk_io<TOUT>::store(out + static_cast<int64_t>(m) * g.Pg + p, val);
+      if (gs) dpk_io<TOUT>::store(out + static_cast<int64_t>(m) * g.Pg + p, val);
       ss = fmaf(val, val, ss);
     }
   });
@@ -439,8 +482,8 @@ Plan make_plan(int64_t Og, int64_t Pg, bool small = false) {
 template <typename TIN, typename TOUT>
 void launch(const Plan& p, bool vec, const void* x, const void* b, void* gs, float* partials,
             const ConvGeom& g, int64_t n, int C, int O, int groups, float scale, hipStream_t s,
-            size_t patch_bytes, int Hp, int Wp) {
-  const dim3 grid(static_cast<unsigned>(n * groups * p.tiles_m * p.tiles_n)), block(kThreads);
+            size_t patch_bytes, int Hp, int Wp, int ksplit, int kchunk, float* split_out) {
+  const dim3 grid(static_cast<unsigned>(n * groups * p.tiles_m * p.tiles_n * ksplit)), block(kThreads);
   const TIN* xp = static_cast<const TIN*>(x);
   const TIN* bp = static_cast<const TIN*>(b);
   TOUT* gp = static_cast<TOUT*>(gs);
@@ -469,7 +512,7 @@ void launch(const Plan& p, bool vec, const void* x, const void* b, void* gs, flo
   }
 #define DPK_CONV_LAUNCH(BM, BN, V, D3)                                                            \
   hipLaunchKernelGGL((conv2d_gs_kernel<BM, BN, TIN, TOUT, V, D3>), grid, block, 0, s, xp, bp, gp, \
-                     partials, g, C, O, groups, scale, p.tiles_m, p.tiles_n)
+                     partials, g, C, O, groups, scale, p.tiles_m, p.tiles_n, ksplit, kchunk, split_out, n)
   const bool d3 = g.Dd > 1 || g.KD > 1 || g.pd > 0;
   if (p.bm == 128) {
     if (vec && d3) DPK_CONV_LAUNCH(128, 128, true, true);
@@ -498,12 +541,44 @@ int conv_gs(const char* who, const void* x, const void* b, int in_dtype, void* g
 
 }  // namespace
 
+namespace {
+// Pieces the contraction over Q output positions is cut into: only for the gather kernel's
+// plan, when its blocks would leave most of the device idle and every piece keeps at least
+// kSplitMinK positions.
+constexpr int kSplitMax = 8, kSplitMinK = 512;
+int split_pieces(int64_t blocks, int64_t Q, int cus) {
+  if (cus <= 0 || blocks >= 2 * cus || Q < 2 * kSplitMinK) return 1;
+  int64_t s = dpk_cdiv(4 * static_cast<int64_t>(cus), blocks);
+  if (s > kSplitMax) s = kSplitMax;
+  if (s > Q / kSplitMinK) s = Q / kSplitMinK;
+  return s < 2 ? 1 : static_cast<int>(s);
+}
+struct ConvWs {
+  size_t partials_bytes, total;  // block sums of squares first, then the pieces' raw tiles
+};
+ConvWs conv_ws(int64_t n, int64_t Og, int64_t Pg, int64_t groups, int64_t O, int pieces_max) {
+  const Plan p = make_plan(Og, Pg, true);
+  int64_t slots = n * groups * p.tiles_m * p.tiles_n;
+  const int64_t chunks = n * dpk_cdiv(O * Pg, kSplitChunk);
+  if (pieces_max > 1 && chunks > slots) slots = chunks;
+  ConvWs w;
+  w.partials_bytes = dpk_align_up(static_cast<size_t>(slots) * sizeof(float), 256);
+  w.total = w.partials_bytes;
+  if (pieces_max > 1) w.total += dpk_align_up(static_cast<size_t>(pieces_max) * n * O * Pg * sizeof(float), 256);
+  return w;
+}
+}  // namespace
+
 extern "C" size_t dpk_conv2d_gs_workspace_bytes(int64_t n, int64_t C, int64_t O, int64_t KH,
-                                                int64_t KW, int64_t groups) {
+                                                int64_t KW, int64_t groups, int64_t Q) {
   if (n <= 0 || C <= 0 || O <= 0 || KH <= 0 || KW <= 0 || groups <= 0) return 0;
   if (C % groups != 0 || O % groups != 0) return 0;
-  const Plan p = make_plan(O / groups, (C / groups) * KH * KW, true);
-  return dpk_align_up(static_cast<size_t>(n * groups * p.tiles_m * p.tiles_n) * sizeof(float), 256);
+  const int64_t Og = O / groups, Pg = (C / groups) * KH * KW;
+  // the pieces of a split contraction (decided at call time from the device's size) need room
+  // for their raw tiles; Q <= 0: the caller does not want the split
+  const Plan p = make_plan(Og, Pg, false);
+  const int pieces = Q > 0 ? split_pieces(n * groups * p.tiles_m * p.tiles_n, Q, 256) : 1;
+  return conv_ws(n, Og, Pg, groups, O, pieces > 1 ? kSplitMax : 1).total;
 }
 
 namespace {
@@ -528,7 +603,7 @@ int conv_gs(const char* who, const void* x, const void* b, int in_dtype, void* g
   const int64_t Q = OD * OH * OW, Pg = (C / groups) * z.KD * KH * KW;
   DPK_REQUIRE(C * z.D * H * W < (1LL << 31) && O * Q < (1LL << 31) && O * Pg < (1LL << 31), DPK_E_SHAPE,
               "%s: one sample exceeds 2^31 elements", who);
-  DPK_REQUIRE(x && b && gs, DPK_E_ARG, "%s: NULL tensor", who);
+  DPK_REQUIRE(x && b && (gs || sumsq), DPK_E_ARG, "%s: NULL tensor", who);
   DPK_REQUIRE(dpk_dtype_ok(in_dtype) && dpk_dtype_ok(gs_dtype), DPK_E_DTYPE, "%s: dtypes %d,%d", who,
               in_dtype, gs_dtype);
   DPK_REQUIRE(dpk_aligned(x, dpk_elsize(in_dtype)) && dpk_aligned(b, dpk_elsize(in_dtype)) &&
@@ -549,35 +624,57 @@ int conv_gs(const char* who, const void* x, const void* b, int in_dtype, void* g
           : 0;
   const Plan p = make_plan(O / groups, Pg, patch_bytes > 0);
   const int64_t blocks = n * groups * p.tiles_m * p.tiles_n;
-  DPK_REQUIRE(blocks <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: %lld blocks exceed the grid limit", who,
-              (long long)blocks);
+  // few long blocks on the gather kernel: cut the contraction over the positions into pieces,
+  // if the caller's workspace has room for their raw tiles
+  int ksplit = patch_bytes > 0 ? 1 : split_pieces(blocks, Q, dpk_device_cus());
+  const ConvWs wl = conv_ws(n, O / groups, Pg, groups, O, ksplit);
+  if (ksplit > 1 && !(ws && ws_bytes >= wl.total && dpk_aligned(ws, 256))) ksplit = 1;
+  const int kchunk = ksplit > 1 ? static_cast<int>(dpk_cdiv(dpk_cdiv(Q, ksplit), mf32::BK) * mf32::BK) : static_cast<int>(Q);
+  DPK_REQUIRE(blocks * ksplit <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: %lld blocks exceed the grid limit", who,
+              (long long)(blocks * ksplit));
   float* partials = nullptr;
+  float* split_out = nullptr;
   if (sumsq) {
-    const size_t need = static_cast<size_t>(blocks) * sizeof(float);
+    const size_t need = ksplit > 1 ? wl.total : static_cast<size_t>(blocks) * sizeof(float);
     DPK_REQUIRE(ws && ws_bytes >= need, DPK_E_WORKSPACE, "%s: workspace %zu < %zu bytes", who,
                 ws_bytes, need);
     DPK_REQUIRE(dpk_aligned(ws, 4), DPK_E_ALIGN, "%s: workspace misaligned", who);
     partials = static_cast<float*>(ws);
   }
+  if (ksplit > 1) split_out = reinterpret_cast<float*>(static_cast<char*>(ws) + wl.partials_bytes);
   // 16-byte (8-byte for bf16) loads of 4 backprops
   const bool vec = Q % 4 == 0 && dpk_aligned(b, in_dtype == DPK_BF16 ? 8 : 16);
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (in_dtype == DPK_F32 && gs_dtype == DPK_F32)
     launch<float, float>(p, vec, x, b, gs, partials, g, n, (int)C, (int)O, (int)groups, scale, s, patch_bytes,
-                       (int)Hp, (int)Wp);
+                       (int)Hp, (int)Wp, ksplit, kchunk, split_out);
   else if (in_dtype == DPK_BF16 && gs_dtype == DPK_BF16)
     launch<bf16_t, bf16_t>(p, vec, x, b, gs, partials, g, n, (int)C, (int)O, (int)groups, scale, s, patch_bytes,
-                         (int)Hp, (int)Wp);
+                         (int)Hp, (int)Wp, ksplit, kchunk, split_out);
   else if (in_dtype == DPK_BF16 && gs_dtype == DPK_F32)
     launch<bf16_t, float>(p, vec, x, b, gs, partials, g, n, (int)C, (int)O, (int)groups, scale, s, patch_bytes,
-                        (int)Hp, (int)Wp);
+                        (int)Hp, (int)Wp, ksplit, kchunk, split_out);
   else
     launch<float, bf16_t>(p, vec, x, b, gs, partials, g, n, (int)C, (int)O, (int)groups, scale, s, patch_bytes,
-                        (int)Hp, (int)Wp);
+                        (int)Hp, (int)Wp, ksplit, kchunk, split_out);
   DPK_LAUNCH_CHECK(who);
+  int64_t cols = static_cast<int64_t>(groups) * p.tiles_m * p.tiles_n;
+  if (ksplit > 1) {
+    // add the pieces, scale, store (unless only the norms are wanted) and square
+    const int64_t OP = O * Pg;
+    const int chunks = static_cast<int>(dpk_cdiv(OP, kSplitChunk));
+    const dim3 grid(static_cast<unsigned>(n * chunks)), block(kThreads);
+    if (gs_dtype == DPK_F32)
+      hipLaunchKernelGGL(conv_split_reduce_kernel<float>, grid, block, 0, s, split_out, static_cast<float*>(gs), partials,
+                         n, OP, ksplit, chunks, scale);
+    else
+      hipLaunchKernelGGL(conv_split_reduce_kernel<bf16_t>, grid, block, 0, s, split_out, static_cast<bf16_t*>(gs),
+                         partials, n, OP, ksplit, chunks, scale);
+    DPK_LAUNCH_CHECK(who);
+    cols = chunks;
+  }
   if (sumsq) {
-    dpk_launch_reduce_rows(partials, n, static_cast<int64_t>(groups) * p.tiles_m * p.tiles_n, sumsq, 0,
-                           1.f, s);
+    dpk_launch_reduce_rows(partials, n, cols, sumsq, 0, 1.f, s);
     DPK_LAUNCH_CHECK(who);
   }
   return DPK_OK;
@@ -596,9 +693,9 @@ extern "C" int dpk_conv2d_gs(const void* x, const void* b, int in_dtype, void* g
 }
 
 extern "C" size_t dpk_conv3d_gs_workspace_bytes(int64_t n, int64_t C, int64_t O, int64_t KD, int64_t KH,
-                                                int64_t KW, int64_t groups) {
+                                                int64_t KW, int64_t groups, int64_t Q) {
   if (KD <= 0) return 0;
-  return dpk_conv2d_gs_workspace_bytes(n, C, O, KD * KH, KW, groups);
+  return dpk_conv2d_gs_workspace_bytes(n, C, O, KD * KH, KW, groups, Q);
 }
 
 extern "C" int dpk_conv3d_gs(const void* x, const void* b, int in_dtype, void* gs, int gs_dtype,

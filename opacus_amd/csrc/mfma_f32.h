@@ -175,12 +175,13 @@ struct LoaderKContig {
 // Software-pipelined k loop: while the MFMAs consume LDS buffer `cur`, the next
 // tile is already in flight from global memory into registers; it is committed
 // to the other buffer afterwards. One barrier per k tile.
+// The k range is [k_begin, k_end), k_begin a multiple of BK; the loaders bound k themselves.
 template <int BM, int BN, class LA, class LB>
 __device__ __forceinline__ void mainloop(Tile<BM, BN>& t, Smem<BM, BN>& sm, LA& la, LB& lb,
-                                         int64_t K) {
-  const int64_t nk = (K + BK - 1) / BK;
-  la.fetch(0);
-  lb.fetch(0);
+                                         int64_t k_begin, int64_t k_end) {
+  const int64_t nk = (k_end - k_begin + BK - 1) / BK;
+  la.fetch(k_begin);
+  lb.fetch(k_begin);
   la.commit(sm.a[0]);
   lb.commit(sm.b[0]);
   __syncthreads();
@@ -188,8 +189,8 @@ __device__ __forceinline__ void mainloop(Tile<BM, BN>& t, Smem<BM, BN>& sm, LA& 
     const int cur = static_cast<int>(kt & 1);
     const bool more = kt + 1 < nk;
     if (more) {
-      la.fetch((kt + 1) * BK);
-      lb.fetch((kt + 1) * BK);
+      la.fetch(k_begin + (kt + 1) * BK);
+      lb.fetch(k_begin + (kt + 1) * BK);
     }
     t.mma(sm.a[cur], sm.b[cur]);
     if (more) {
@@ -198,6 +199,11 @@ __device__ __forceinline__ void mainloop(Tile<BM, BN>& t, Smem<BM, BN>& sm, LA& 
     }
     __syncthreads();
   }
+}
+
+template <int BM, int BN, class LA, class LB>
+__device__ __forceinline__ void mainloop(Tile<BM, BN>& t, Smem<BM, BN>& sm, LA& la, LB& lb, int64_t K) {
+  mainloop<BM, BN>(t, sm, la, lb, 0, K);
 }
 
 }  // namespace mf32

@@ -283,6 +283,7 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
             p._forward_counter += 1
             if p._forward_counter == 1:
                 p.__dict__.pop("_tied_parts", None)  # left by a backward pass that did not finish
+                module.__dict__.pop("_dpk_materialise", None)
             if (
                 self.use_ghost_clipping
                 and p._forward_counter > 1
@@ -290,8 +291,13 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
                 and not getattr(module, "stack_uses", False)  # its uses are contracted together
                 and not (id(p) in self._tied_embedding_weights and p._forward_counter == 2)
             ):
-                # the norm of a sum of two layers' gradients is not a function of their norms
-                raise NotImplementedError("Parameter tying is not supported with Ghost Clipping")
+                if getattr(self.NORM_SAMPLERS[type(module)], "reference_materialises", False):
+                    # a layer type the reference serves by forming the per-sample gradients anyway
+                    # (no norm sampler there): used more than once in a pass, it is served that way here too
+                    module._dpk_materialise = True
+                else:
+                    # the norm of a sum of two layers' gradients is not a function of their norms
+                    raise NotImplementedError("Parameter tying is not supported with Ghost Clipping")
 
     def capture_backprops_hook(
         self, module: nn.Module, _forward_input, forward_output, loss_reduction: str, batch_first: bool
@@ -310,7 +316,11 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
             activations, backprops = stacked
             for _, p in trainable_parameters(module):
                 p._forward_counter += 1  # taken off again below, as for a module used once
-        ghost = self.use_ghost_clipping and type(module) in self.NORM_SAMPLERS
+        ghost = (
+            self.use_ghost_clipping
+            and type(module) in self.NORM_SAMPLERS
+            and not getattr(module, "_dpk_materialise", False)
+        )
         if self.single_backward and ghost:
             self._kept_passes.append((module, activations, backprops, scale, None))
         if ghost:
@@ -399,6 +409,25 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
                         module.scale_grad_by_freq,
                     ),
                 )
+            elif (
+                type(module) in (nn.Conv1d, nn.Conv2d)
+                and grad_samples is None
+                and not isinstance(module.padding, str)
+                and module.padding_mode == "zeros"
+            ):
+                # the clip-weighted sum of a convolution's per-sample gradients is the ordinary
+                # weight gradient for backprops weighted per sample: one weight-gradient convolution
+                weighted = backprops * (c * scale).to(backprops.dtype).view(n, *([1] * (backprops.dim() - 1)))
+                x = activations[0].to(backprops.dtype)
+                wgrad = torch.nn.grad.conv1d_weight if type(module) is nn.Conv1d else torch.nn.grad.conv2d_weight
+                if module.weight.requires_grad:
+                    add(
+                        module.weight,
+                        wgrad(x, module.weight.shape, weighted, stride=module.stride, padding=module.padding,
+                              dilation=module.dilation, groups=module.groups),
+                    )
+                if module.bias is not None:
+                    add(module.bias, weighted.sum(dim=[0] + list(range(2, weighted.dim()))))
             else:
                 if grad_samples is None:
                     grad_samples = call_sampler(self._sampler_for(module), module, activations, backprops, scale)

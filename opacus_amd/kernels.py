@@ -54,7 +54,14 @@ def _ptr(t: Optional[torch.Tensor]):
     return None if t is None else ctypes.c_void_p(t.data_ptr())
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(dev: torch.device):
+    """torch's current stream on ``dev`` as a raw handle (the direct binding where torch has it:
+    building a ``torch.cuda.Stream`` object per kernel launch is a visible cost for small models)."""
+    if _raw_stream is not None:
+        return ctypes.c_void_p(_raw_stream(dev.index if dev.index is not None else torch.cuda.current_device()))
     return ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
 
 
@@ -272,10 +279,13 @@ def conv2d_grad_sample(
     groups: int,
     scale: float = 1.0,
     want_sumsq: bool = True,
-) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    norm_only: bool = False,
+) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
     """Per-sample weight gradients ``[n, O, C/groups, KH, KW]`` of a 2-d convolution.
 
     ``padding`` is ``(top, bottom, left, right)``; ``backprops`` is ``[n, O, OH, OW]``.
+    ``norm_only``: the gradient tiles are formed and squared but never stored; returns
+    ``(None, sumsq)``.
     """
     dev = _need_gpu(x, backprops)
     if x.dtype != backprops.dtype:
@@ -283,25 +293,26 @@ def conv2d_grad_sample(
     n, C, H, W = x.shape
     O = backprops.shape[1]
     KH, KW = kernel_size
-    gs = torch.empty((n, O, C // groups, KH, KW), dtype=backprops.dtype, device=dev)
+    want_sumsq = want_sumsq or norm_only
+    gs = None if norm_only else torch.empty((n, O, C // groups, KH, KW), dtype=backprops.dtype, device=dev)
     sumsq = torch.empty((n,), dtype=torch.float32, device=dev) if want_sumsq else None
     if n == 0:
         return gs, sumsq
     x = _dense(x)
     b = _dense(backprops)
     L = lib()
-    ws, wsb = _ws(L.dpk_conv2d_gs_workspace_bytes(n, C, O, KH, KW, groups) if want_sumsq else 0, dev)
     oh = (H + padding[0] + padding[1] - (dilation[0] * (KH - 1) + 1)) // stride[0] + 1
     ow = (W + padding[2] + padding[3] - (dilation[1] * (KW - 1) + 1)) // stride[1] + 1
     if b.numel() != n * O * oh * ow:
         raise ValueError(
             f"backprops {tuple(backprops.shape)} do not match the output geometry [{n},{O},{oh},{ow}]"
         )
+    ws, wsb = _ws(L.dpk_conv2d_gs_workspace_bytes(n, C, O, KH, KW, groups, oh * ow), dev)
     with _timed("conv2d_gs", dev):
         check(
             "dpk_conv2d_gs",
             L.dpk_conv2d_gs(
-                _ptr(x), _ptr(b), _code(b), _ptr(gs), _code(gs), _ptr(sumsq), n, C, H, W, O, KH, KW,
+                _ptr(x), _ptr(b), _code(b), _ptr(gs), _code(b), _ptr(sumsq), n, C, H, W, O, KH, KW,
                 stride[0], stride[1], padding[0], padding[1], padding[2], padding[3], dilation[0],
                 dilation[1], groups, float(scale), _ptr(ws), wsb, _stream(dev),
             ),
@@ -344,7 +355,7 @@ def conv3d_grad_sample(
         raise ValueError(f"backprops {tuple(backprops.shape)} do not match the output geometry [{n},{O},{out}]")
     arr = lambda v: (ctypes.c_int64 * 3)(*[int(e) for e in v])  # noqa: E731
     L = lib()
-    ws, wsb = _ws(L.dpk_conv3d_gs_workspace_bytes(n, C, O, *kernel_size, groups) if want_sumsq else 0, dev)
+    ws, wsb = _ws(L.dpk_conv3d_gs_workspace_bytes(n, C, O, *kernel_size, groups, out[0] * out[1] * out[2]), dev)
     with _timed("conv3d_gs", dev):
         check(
             "dpk_conv3d_gs",

@@ -1164,3 +1164,55 @@ def test_hooked_layers_under_activation_checkpointing(A):
         close(g0, w, 1e-4, 1e-5, f"{k} without checkpointing")
         close(g1, w, 1e-4, 1e-5, f"{k} with checkpointing")
         close(s1, s0, 1e-4, 1e-6, f"{k} step gradient")
+
+
+# ---- convolutions under ghost clipping: norms without stored per-sample gradients ---------------
+@pytest.mark.parametrize("single", [False, True])
+def test_ghost_cnn_norms_and_clipped_sum_against_batch_of_one_autograd(A, single):
+    """The reference forms and drops every conv per-sample gradient under fast gradient clipping
+    (grad_sample_module_fast_gradient_clipping.py:226-250). Here a convolution's norm comes from
+    the conv kernel's norm-only mode (early layers: many positions) or from the Gram route on
+    the unfolded input (late layers: few positions, many channels); a conv layer used twice in
+    one pass falls back to materialising; Conv1d and asymmetric "same" padding included. Norms and
+    the clipped mean gradient against CPU autograd on one sample at a time."""
+
+    class Net(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.c1 = nn.Conv2d(3, 8, 3, padding=1)  # 12 x 12 positions, 27 kernel elements: direct route
+            self.c2 = nn.Conv2d(8, 32, 4, stride=3, padding="valid")  # 3 x 3 positions, 128 elements, 32 channels: Gram route
+            self.c3 = nn.Conv2d(32, 32, 2, padding="same")  # asymmetric padding, 3 x 3 positions: Gram route
+            self.twice = nn.Conv2d(32, 32, 1)  # used twice: materialised
+            self.c1d = nn.Conv1d(32, 16, 3, padding=1)  # 9 positions
+            self.fc = nn.Linear(16 * 9, 5)
+
+        def forward(self, x):
+            h = F.relu(self.c1(x))
+            h = F.relu(self.c2(h))
+            h = F.relu(self.c3(h))
+            h = self.twice(F.relu(self.twice(h)))
+            h = F.relu(self.c1d(h.flatten(2)))
+            return self.fc(h.flatten(1))
+
+    torch.manual_seed(31)
+    net, n, C = Net(), 6, 0.3
+    x, y = torch.randn(n, 3, 12, 12), torch.randint(0, 5, (n,))
+    want = per_sample_grads_cpu(net, x, y, lambda out, t: F.cross_entropy(out, t, reduction="sum"))
+    flat = torch.cat([g.flatten(1) for g in want.values()], dim=1)
+    norms = flat.norm(dim=1)
+    coef = (C / (norms + 1e-6)).clamp(max=1.0)
+    assert (coef < 1).any() and (norms > 0).all()
+    ghost = A.GradSampleModuleFastGradientClipping(copy.deepcopy(net).to(DEV), max_grad_norm=C, single_backward=single)
+    opt = A.DPOptimizerFastGradientClipping(
+        torch.optim.SGD(ghost.parameters(), lr=0.1), noise_multiplier=0.0, max_grad_norm=C, expected_batch_size=n
+    )
+    crit = A.DPLossFastGradientClipping(ghost, opt, nn.CrossEntropyLoss(), "mean")
+    opt.zero_grad()
+    crit(ghost(x.to(DEV)), y.to(DEV)).backward()
+    close(ghost.per_sample_gradient_norms, norms, 1e-4, 1e-6, "per-sample norms")
+    for (k, p), g in zip(ghost._module.named_parameters(), want.values()):
+        assert not hasattr(p, "grad_sample") or p.grad_sample is None, k  # nothing materialised is kept
+        close(p._norm_sample, g.flatten(1).norm(dim=1), 1e-4, 1e-6, f"norm of {k}")
+    opt.pre_step()
+    for (k, p), g in zip(ghost._module.named_parameters(), want.values()):
+        close(p.grad, torch.einsum("n,n...->...", coef, g) / n, 1e-4, 1e-6, f"clipped mean gradient of {k}")

@@ -565,6 +565,46 @@ def test_conv3d_grad_sample_f32(K, case):
     assert_rel(K.conv_bias_grad_sample(dev(b), scale=2.0), want_b, FP32_REL, "conv3d bias")
 
 
+@pytest.mark.parametrize(
+    "n,C,H,W,O,k,stride,pad,groups",
+    [
+        # few kernel elements, many output positions: blocks < 2 x CUs, so the contraction over the
+        # positions is cut into pieces whose raw tiles a second kernel adds (ragged last piece)
+        (4, 3, 96, 96, 64, 7, 2, 3, 1),
+        (3, 2, 70, 66, 24, 3, 1, 1, 1),
+        (2, 4, 64, 64, 8, 3, 1, 1, 2),
+        # the same machinery is not taken for a layer with enough blocks or a short contraction
+        (8, 16, 12, 12, 16, 3, 1, 1, 1),
+    ],
+)
+def test_conv2d_split_contraction_and_norm_only(K, n, C, H, W, O, k, stride, pad, groups):
+    torch.manual_seed(C * 100 + H)
+    x = torch.randn(n, C, H, W)
+    oh, ow = (H + 2 * pad - k) // stride + 1, (W + 2 * pad - k) // stride + 1
+    b = torch.randn(n, O, oh, ow)
+    want_w, _ = O_conv(x, b, k, stride, pad, groups)
+    geo = dict(kernel_size=(k, k), stride=(stride, stride), padding=(pad, pad, pad, pad), dilation=(1, 1), groups=groups)
+    gs, sumsq = K.conv2d_grad_sample(dev(x), dev(b), scale=2.0, **geo)
+    assert_rel(gs, 2.0 * want_w, FP32_REL, "conv gs")
+    want_ss = (2.0 * want_w).double().flatten(1).pow(2).sum(1)
+    assert_rel(sumsq, want_ss, FP32_REL, "conv sumsq")
+    none, ss_only = K.conv2d_grad_sample(dev(x), dev(b), scale=2.0, norm_only=True, **geo)
+    assert none is None
+    assert_rel(ss_only, want_ss, FP32_REL, "conv sumsq, norm only")
+    # bf16 inputs through the same kernels
+    gs16, ss16 = K.conv2d_grad_sample(dev(x.bfloat16()), dev(b.bfloat16()), **geo)
+    want16, _ = O_conv(x.bfloat16().float(), b.bfloat16().float(), k, stride, pad, groups)
+    assert_rel(gs16, want16, BF16_REL, "conv gs bf16")
+    assert_rel(ss16, want16.double().flatten(1).pow(2).sum(1), 1e-4, "conv sumsq bf16 (fp32 accumulators)")
+
+
+def O_conv(x, b, k, stride, pad, groups):
+    return O.conv2d_grad_sample(
+        x.double(), b.double(), kernel_size=(k, k), padding=(pad, pad), stride=(stride, stride), dilation=(1, 1), groups=groups
+    )
+
+
+
 # ---- Embedding ------------------------------------------------------------------------
 def test_embedding_golden_vectors(K, embedding_norm_cases):
     """The reference's own known-answer triples and docstring intermediates, on the GPU."""
