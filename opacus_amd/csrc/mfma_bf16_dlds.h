@@ -220,10 +220,11 @@ struct Tile {
 // stay outstanding while tile kt is awaited is the constant
 // kLoadsPerTile * (NS - 2). abase / bbase must be wave-uniform and every byte
 // offset inside the matrices must fit 32 bits (M * ld * 2 < 2^32).
+// Ma / Mb: rows of the two operand matrices (the same matrix for a Gram).
 template <class C, typename T = bf16_t>
 __device__ __forceinline__ void mainloop(Tile& t, Smem<C>& sm, const T* abase,
                                          const T* bbase, int64_t ld, int64_t m0a, int64_t m0b,
-                                         int64_t M, int64_t K, int wm0, int wn0) {
+                                         int64_t Ma, int64_t Mb, int64_t K, int wm0, int wn0) {
   constexpr int NS = C::kStages;
   constexpr int ROW_BYTES = C::ROW_BYTES, ES = sizeof(T);
   constexpr int BK = ROW_BYTES / ES;  // k values of a stage row: 64 bf16 or 32 floats
@@ -235,7 +236,7 @@ __device__ __forceinline__ void mainloop(Tile& t, Smem<C>& sm, const T* abase,
   uint32_t off[C::kLoadsPerTile];
 #pragma unroll
   for (int q = 0; q < C::kLoadsPerTile; ++q) {
-    off[q] = q < C::kLoadsA ? lane_offset<C, ES>(ld, m0a, M, q) : lane_offset<C, ES>(ld, m0b, M, q - C::kLoadsA);
+    off[q] = q < C::kLoadsA ? lane_offset<C, ES>(ld, m0a, Ma, q) : lane_offset<C, ES>(ld, m0b, Mb, q - C::kLoadsA);
     asm volatile("" : "+v"(off[q]));
   }
   auto issue_q = [&](int64_t kt, uint32_t st, int q) {
@@ -260,6 +261,13 @@ __device__ __forceinline__ void mainloop(Tile& t, Smem<C>& sm, const T* abase,
     stage = stage + 1 == NS ? 0 : stage + 1;
   }
   wait_and_barrier<0>();  // the ring may be reused by the caller's next main loop
+}
+
+template <class C, typename T = bf16_t>
+__device__ __forceinline__ void mainloop(Tile& t, Smem<C>& sm, const T* abase,
+                                         const T* bbase, int64_t ld, int64_t m0a, int64_t m0b,
+                                         int64_t M, int64_t K, int wm0, int wn0) {
+  mainloop<C, T>(t, sm, abase, bbase, ld, m0a, m0b, M, M, K, wm0, wn0);
 }
 
 // ---- 64 x 64 tile with the k extent of a stage split over the block's waves -----

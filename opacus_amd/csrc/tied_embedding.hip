@@ -10,11 +10,16 @@
 //                   = sum_t < e_t , sum_t' g[t', ids_t] a_t' >
 // with e_t the backprops of the embedding output, a_t' the inputs of the head and g the
 // backprops of its output: only the <= T rows of G_head that the sample's ids name are
-// needed. Three steps:
+// needed. Regrouped, cross = sum_{t', t} g[t', ids_t] (a_t' . e_t): a tile of the T' x T product
+// a e^T (both operands contiguous along D, the layout of the ghost norm's Gram kernel) is
+// formed in MFMA accumulators and multiplied, element by element, by the entries of g the
+// ids name, read straight from g; neither the gathered matrix nor the product is stored.
+// Shapes that kernel does not take go through three steps instead:
 //   1. N[t', t] = g[t', ids_t]                       (gather, this file)
 //   2. R[t, :]  = sum_t' N[t', t] a_t'               (the per-sample Linear contraction)
 //   3. cross    = sum_{t,d} e[t,d] R[t,d]            (row dot product, this file)
 #include "dpk_common.h"
+#include "mfma_bf16_dlds.h"
 
 namespace {
 
@@ -75,6 +80,63 @@ __global__ __launch_bounds__(kThreads) void dot_final_kernel(const float* __rest
   if (lane == 0) cross[s] = scale * v;
 }
 
+// One 128 x 128 tile (rows: head positions t', columns: embedding positions t) of one sample.
+// partial[unit] = sum over the tile of g[t', ids_t] * (a_t' . e_t).
+using CrossCfg = mb16d::Config<2, 2, 2, 64>;
+
+template <typename TE>
+__global__ __launch_bounds__(CrossCfg::kThreads) void tied_cross_tile_kernel(
+    const int64_t* __restrict__ ids, const TE* __restrict__ e, const TE* __restrict__ a, const TE* __restrict__ g,
+    float* __restrict__ partial, int64_t T, int64_t T2, int64_t D, int64_t V, int tiles_t, int tiles_t2,
+    uint32_t nunits) {
+  using C = CrossCfg;
+  __shared__ mb16d::Smem<C> sm;
+  __shared__ float red[C::kWaves];
+  __shared__ int64_t s_ids[C::BN];
+  const uint32_t unit = xcd_contiguous_id(blockIdx.x, nunits);
+  const uint32_t per_sample = static_cast<uint32_t>(tiles_t) * tiles_t2;
+  const int64_t sample = unit / per_sample;
+  const uint32_t rest = unit % per_sample;
+  const int64_t r0 = static_cast<int64_t>(rest / tiles_t) * C::BM;  // first head position t'
+  const int64_t c0 = static_cast<int64_t>(rest % tiles_t) * C::BN;  // first embedding position t
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int kh = lane >> 5, l32 = lane & 31;
+  const int wm0 = (wave / C::kWaveCols) * 64, wn0 = (wave % C::kWaveCols) * 64;
+  if (threadIdx.x < C::BN) {
+    const int64_t t = c0 + threadIdx.x;
+    const int64_t id = t < T ? ids[sample * T + t] : -1;
+    s_ids[threadIdx.x] = (id >= 0 && id < V) ? id : -1;  // outside the table: contributes nothing
+  }
+  __syncthreads();
+  // The 64 entries of g this lane's part of the tile meets are requested before the main loop
+  // and used after it: scattered two-byte reads, whose latency the contraction covers.
+  const TE* gs = g + sample * T2 * V;
+  TE gv[2][2][16];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int64_t id = s_ids[wn0 + j * 32 + l32];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int64_t row = r0 + wm0 + i * 32 + (v >> 2) * 8 + kh * 4 + (v & 3);
+        gv[i][j][v] = (id >= 0 && row < T2) ? gs[row * V + id] : static_cast<TE>(0);
+      }
+  }
+  mb16d::Tile tile;
+  tile.clear();
+  mb16d::mainloop<C, TE>(tile, sm, a + sample * T2 * D, e + sample * T * D, D, r0, c0, T2, T, D, wm0, wn0);
+  float sum = 0.f;
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) sum = fmaf(dpk_io<TE>::load(&gv[i][j][v]), tile.acc[i][j][v], sum);
+  const float t = block_sum<C::kWaves>(sum, red);
+  if (threadIdx.x == 0) partial[unit] = t;
+}
+
 struct CrossLayout {
   size_t gathered, product, partial, linear, total;
 };
@@ -119,6 +181,31 @@ extern "C" int dpk_tied_embedding_cross(const int64_t* ids, const void* e, int e
   DPK_REQUIRE(ws && ws_bytes >= l.total, DPK_E_WORKSPACE, "%s: workspace %zu < %zu bytes", who, ws_bytes, l.total);
   DPK_REQUIRE(dpk_aligned(ws, 256), DPK_E_ALIGN, "%s: workspace must be 256-byte aligned", who);
   char* base = static_cast<char*>(ws);
+  {
+    // the tile kernel: one element type, whole 128-byte stage rows, 32-bit offsets inside a sample
+    const int64_t es = dpk_elsize(head_dtype), widest = T > T2 ? T : T2;
+    const int64_t tiles_t = dpk_cdiv(T, CrossCfg::BN), tiles_t2 = dpk_cdiv(T2, CrossCfg::BM);
+    const int64_t units = n * tiles_t * tiles_t2;
+    if (emb_dtype == head_dtype && D % (128 / es) == 0 && dpk_aligned(e, 16) && dpk_aligned(a, 16) &&
+        widest * D * es < (int64_t{1} << 32) && units <= DPK_MAX_GRID_X && units * 4 <= (int64_t)(l.total - l.partial)) {
+      hipStream_t s = static_cast<hipStream_t>(stream);
+      float* part = reinterpret_cast<float*>(base + l.partial);
+      const dim3 grid(static_cast<unsigned>(units)), block(CrossCfg::kThreads);
+      if (head_dtype == DPK_F32)
+        hipLaunchKernelGGL(tied_cross_tile_kernel<float>, grid, block, 0, s, ids, static_cast<const float*>(e),
+                           static_cast<const float*>(a), static_cast<const float*>(g), part, T, T2, D, V, (int)tiles_t,
+                           (int)tiles_t2, static_cast<uint32_t>(units));
+      else
+        hipLaunchKernelGGL(tied_cross_tile_kernel<bf16_t>, grid, block, 0, s, ids, static_cast<const bf16_t*>(e),
+                           static_cast<const bf16_t*>(a), static_cast<const bf16_t*>(g), part, T, T2, D, V, (int)tiles_t,
+                           (int)tiles_t2, static_cast<uint32_t>(units));
+      DPK_LAUNCH_CHECK(who);
+      hipLaunchKernelGGL(dot_final_kernel, dim3(static_cast<unsigned>(dpk_cdiv(n * DPK_WAVE, kThreads))), dim3(kThreads),
+                         0, s, part, n, tiles_t * tiles_t2, scale, cross);
+      DPK_LAUNCH_CHECK(who);
+      return DPK_OK;
+    }
+  }
   void* gathered = base + l.gathered;
   float* product = reinterpret_cast<float*>(base + l.product);
   float* partial = reinterpret_cast<float*>(base + l.partial);

@@ -833,7 +833,12 @@ def test_norm_layers_bf16(K):
 
 # ---- tied input / output embeddings: the cross term --------------------------------------------
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("n,T,T2,D,V", [(3, 7, 7, 12, 19), (2, 33, 5, 64, 300), (4, 1, 9, 8, 16)])
+# D a multiple of 64: the tile kernel (product tile times gathered entries), ragged tiles in both
+# directions, several tiles per sample, few distinct ids; other D: gather, contraction, dot product
+@pytest.mark.parametrize(
+    "n,T,T2,D,V",
+    [(3, 7, 7, 12, 19), (2, 33, 5, 64, 300), (4, 1, 9, 8, 16), (3, 200, 150, 128, 500), (2, 300, 130, 192, 40), (9, 128, 256, 64, 1000)],
+)
 def test_tied_embedding_cross_term(K, dtype, n, T, T2, D, V):
     """<G_emb, G_head> against the materialised definition; embedding and projection may see
     different numbers of positions; repeated ids; the scale is a plain factor."""
@@ -853,6 +858,13 @@ def test_tied_embedding_cross_term(K, dtype, n, T, T2, D, V):
     got32 = K.tied_embedding_cross_term(dev(ids), dev(e.float()), dev(a), dev(g))
     assert_rel(got32, want, 1e-4, "fp32 embedding backprops")
     assert K.tied_embedding_cross_term(dev(ids[:0]), dev(e[:0]), dev(a[:0]), dev(g[:0])).shape == (0,)
+    # an id outside the table contributes nothing
+    bad = ids.clone()
+    bad[0, 0] = V + 3
+    e0 = e.clone()
+    e0[0, 0] = 0
+    _, want_bad = O.tied_embedding_norm_sample(ids, e0.double(), a.double(), g.double())
+    assert_rel(K.tied_embedding_cross_term(dev(bad), dev(e), dev(a), dev(g)), want_bad, 1e-5 if dtype == torch.float32 else 1e-4, "bad id")
 
 
 def test_bias_grad_samples_carry_their_sumsq(K):
