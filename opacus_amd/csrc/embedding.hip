@@ -16,10 +16,10 @@
 // which equal ids are neighbours in increasing position. Longer samples take the pairwise
 // scan (quadratic in T, no LDS limit).
 //
-// The ghost norm does not walk the lists for every position: sum_v |sum_{t: id = v} b_t|^2
-// = sum_t |b_t|^2 + sum over ids that occur more than once of (|sum b_t|^2 - sum |b_t|^2).
-// The first term is one streaming pass over b at memory speed; the second touches only the
-// rows of repeated ids, which the leader of each list adds in the same kernel.
+// (Tried and dropped for the ghost norm: one streaming pass for sum_t |b_t|^2 plus corrections
+// |sum b_t|^2 - sum |b_t|^2 for the ids that occur more than once. It reads the rows of repeated
+// ids twice and handles them list by list: 1.5 us per repeated id and sample, where text has
+// hundreds per sequence. Walking the lists reads every row once whatever the ids are.)
 #include <climits>
 
 #include "dpk_common.h"
@@ -225,19 +225,23 @@ __device__ __forceinline__ void bitonic_sort(Elem (&v)[E], int64_t* key, int32_t
 }
 
 template <int E>
-__global__ __launch_bounds__(kThreads) void emb_sort_link_kernel(const int64_t* __restrict__ ids, int T, int64_t V,
-                                                                  int32_t* __restrict__ next,
-                                                                  int32_t* __restrict__ leader,
-                                                                  int32_t* __restrict__ rank,
-                                                                  int32_t* __restrict__ count,
-                                                                  int32_t* __restrict__ flag) {
-  constexpr int np = E * kThreads;
+struct SortMem {
+  int64_t key[E * kThreads];
+  int32_t pos[E * kThreads];
+  int32_t runs[kThreads];
+  int32_t wide;  // some id of the sample does not fit the packed form
+};
+
+template <int E>
+__device__ __forceinline__ void sort_link_sample(SortMem<E>& m, int64_t sample, const int64_t* __restrict__ ids, int T,
+                                                 int64_t V, int32_t* __restrict__ next, int32_t* __restrict__ leader,
+                                                 int32_t* __restrict__ rank, int32_t* __restrict__ count,
+                                                 int32_t* __restrict__ flag) {
   constexpr int64_t kPackLimit = int64_t{1} << 51;
-  __shared__ int64_t key[np];
-  __shared__ int32_t pos[np];
-  __shared__ int32_t runs[kThreads];
-  __shared__ int32_t wide;  // some id of the sample does not fit the packed form
-  const int64_t sample = blockIdx.x;
+  int64_t* key = m.key;
+  int32_t* pos = m.pos;
+  int32_t* runs = m.runs;
+  int32_t& wide = m.wide;
   const int64_t* row = ids + sample * T;
   const int tid = threadIdx.x;
   if (tid == 0) wide = 0;
@@ -300,97 +304,15 @@ __global__ __launch_bounds__(kThreads) void emb_sort_link_kernel(const int64_t* 
   if (tid == kThreads - 1) count[sample] = before;
 }
 
-// ---- ghost norm as one streaming pass ---------------------------------------------------
-// grid = n * ceil(T / kStreamRows). A block owns kStreamRows consecutive positions of one
-// sample and all D columns: thread <-> one 16-byte chunk of a row per step of kThreads
-// chunks, all the block's rows of a step in flight at once. Leaders of a list with more than
-// one member add |sum b|^2 - sum |b|^2 over their list. The block's sum goes to
-// partials[block]; a row reduction in fixed order follows.
-constexpr int kStreamRows = 16;
-
-template <typename TIN> struct Chunk16;
-template <> struct Chunk16<float> {
-  static constexpr int kElems = 4;
-  static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
-    const dpk_vf4 r = __builtin_nontemporal_load(reinterpret_cast<const dpk_vf4*>(p));
-    v[0] = r.x; v[1] = r.y; v[2] = r.z; v[3] = r.w;
-  }
-};
-template <> struct Chunk16<bf16_t> {
-  static constexpr int kElems = 8;
-  typedef uint32_t u4 __attribute__((ext_vector_type(4)));
-  static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[8]) {
-    const u4 r = __builtin_nontemporal_load(reinterpret_cast<const u4*>(p));
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      v[2 * i] = __uint_as_float(r[i] << 16);
-      v[2 * i + 1] = __uint_as_float(r[i] & 0xffff0000u);
-    }
-  }
-};
-
-template <typename TIN>
-__global__ __launch_bounds__(kThreads) void emb_norm_stream_kernel(
-    const TIN* __restrict__ b, const int32_t* __restrict__ next, const int32_t* __restrict__ leader, int T, int64_t D,
-    int tch, float* __restrict__ partials) {
-  constexpr int E = Chunk16<TIN>::kElems;
-  __shared__ float red[kWaves];
-  __shared__ int32_t s_next[kStreamRows], s_lead[kStreamRows];
-  const int64_t sample = blockIdx.x / tch;
-  const int t0 = static_cast<int>(blockIdx.x % tch) * kStreamRows;
-  const int rows = T - t0 < kStreamRows ? T - t0 : kStreamRows;
-  const TIN* bs = b + sample * T * D;
-  if (threadIdx.x < kStreamRows) {
-    const bool live = static_cast<int>(threadIdx.x) < rows;
-    s_next[threadIdx.x] = live ? next[sample * T + t0 + threadIdx.x] : -1;
-    s_lead[threadIdx.x] = live ? leader[sample * T + t0 + threadIdx.x] : 0;
-  }
-  float ss = 0.f;
-  const int64_t chunks = D / E;  // D % E == 0 on this path
-  for (int64_t c = threadIdx.x; c < chunks; c += kThreads) {
-    const TIN* p = bs + static_cast<int64_t>(t0) * D + c * E;
-    if (rows == kStreamRows) {
-      float v[kStreamRows][E];
-#pragma unroll
-      for (int r = 0; r < kStreamRows; ++r) Chunk16<TIN>::load(p + r * D, v[r]);
-#pragma unroll
-      for (int r = 0; r < kStreamRows; ++r)
-#pragma unroll
-        for (int e = 0; e < E; ++e) ss = fmaf(v[r][e], v[r][e], ss);
-    } else {
-      for (int r = 0; r < rows; ++r) {
-        float v[E];
-        Chunk16<TIN>::load(p + r * D, v);
-#pragma unroll
-        for (int e = 0; e < E; ++e) ss = fmaf(v[e], v[e], ss);
-      }
-    }
-  }
-  __syncthreads();
-  // repeated ids: the list's leader replaces the members' sum of squares by the square of their sum
-  for (int r = 0; r < rows; ++r) {
-    if (!s_lead[r] || s_next[r] < 0) continue;  // uniform over the block
-    for (int64_t c = threadIdx.x; c < chunks; c += kThreads) {
-      float acc[E], sq = 0.f;
-#pragma unroll
-      for (int e = 0; e < E; ++e) acc[e] = 0.f;
-      for (int u = t0 + r; u >= 0; u = next[sample * T + u]) {
-        float v[E];
-        Chunk16<TIN>::load(bs + static_cast<int64_t>(u) * D + c * E, v);
-#pragma unroll
-        for (int e = 0; e < E; ++e) {
-          acc[e] += v[e];
-          sq = fmaf(v[e], v[e], sq);
-        }
-      }
-      float whole = 0.f;
-#pragma unroll
-      for (int e = 0; e < E; ++e) whole = fmaf(acc[e], acc[e], whole);
-      ss += whole - sq;
-    }
-  }
-  const float s = block_sum<kWaves>(ss, red);
-  if (threadIdx.x == 0) partials[blockIdx.x] = s;
+template <int E>
+__global__ __launch_bounds__(kThreads) void emb_sort_link_kernel(const int64_t* __restrict__ ids, int T, int64_t V,
+                                                                  int32_t* __restrict__ next,
+                                                                  int32_t* __restrict__ leader,
+                                                                  int32_t* __restrict__ rank,
+                                                                  int32_t* __restrict__ count,
+                                                                  int32_t* __restrict__ flag) {
+  __shared__ SortMem<E> m;
+  sort_link_sample<E>(m, blockIdx.x, ids, T, V, next, leader, rank, count, flag);
 }
 
 // rank[t] = #{leaders t' of the sample with ids[t'] < ids[t]}; count[sample] = #leaders.
@@ -475,11 +397,37 @@ __global__ __launch_bounds__(kThreads) void emb_walk_kernel(
   const int32_t* nx = next + sample * T;
   const int32_t* ld = leader + sample * T;
   float ss = 0.f;
-  for (int64_t t = t0; t < t1; ++t) {
-    if (!ld[t]) continue;  // uniform over the block
+  // the first row of every list that starts in this block is requested before any is used
+  // (kLeadersPerBlock independent loads in flight); further members follow list by list
+  // Everything a block needs first is requested without a branch in between, so that the
+  // requests overlap: the list flags and second members of its positions (clamped reads, the
+  // values past the end unused), then the first row of every list that starts here (other
+  // positions re-read the block's first row, a cache hit). Further members follow list by list.
+  typename dpk_io<TIN>::raw4 first[kLeadersPerBlock];
+  int32_t head[kLeadersPerBlock], follow[kLeadersPerBlock];
+#pragma unroll
+  for (int r = 0; r < kLeadersPerBlock; ++r) {
+    const int64_t t = (t0 + r < T) ? t0 + r : T - 1;
+    head[r] = ld[t];
+    follow[r] = nx[t];
+  }
+#pragma unroll
+  for (int r = 0; r < kLeadersPerBlock; ++r)
+    if (t0 + r >= t1 || !head[r]) follow[r] = -2;  // < -1: no list starts here
+  if (VEC) {
+    const int64_t dd = (d < D) ? d : 0;
+#pragma unroll
+    for (int r = 0; r < kLeadersPerBlock; ++r)
+      first[r] = dpk_io<TIN>::load4_raw(bs + (follow[r] >= -1 ? t0 + r : t0) * D + dd);
+  }
+#pragma unroll
+  for (int r = 0; r < kLeadersPerBlock; ++r) {
+    const int64_t t = t0 + r;
+    if (follow[r] < -1) continue;  // uniform over the block
     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (VEC && d < D) acc = dpk_io<TIN>::unpack4(first[r]);
     if (d < D) {
-      for (int64_t u = t; u >= 0; u = nx[u]) {
+      for (int64_t u = VEC ? static_cast<int64_t>(follow[r]) : t; u >= 0; u = nx[u]) {
         const TIN* p = bs + u * D + d;
         if (VEC) {
           const float4 v = dpk_io<TIN>::load4(p);
@@ -687,23 +635,8 @@ extern "C" int dpk_embedding_ghost_norm(const int64_t* ids, const void* b, int d
   const int64_t tch = dpk_cdiv(T, kLeadersPerBlock), dch = dpk_cdiv(D, kThreads * 4);
   DPK_REQUIRE(n * tch * dch <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: too many blocks", who);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const bool sorted = launch_link(ids, n, T, 0, w, nullptr, false, s);
+  launch_link(ids, n, T, 0, w, nullptr, false, s);
   DPK_LAUNCH_CHECK(who);
-  const int64_t chunk = dtype == DPK_BF16 ? 8 : 4;
-  if (sorted && D % chunk == 0 && dpk_aligned(b, 16)) {
-    // one streaming pass over b, then the fixed-order sum of the blocks' partial sums
-    const dim3 grid(static_cast<unsigned>(n * tch)), block(kThreads);
-    if (dtype == DPK_F32)
-      hipLaunchKernelGGL(emb_norm_stream_kernel<float>, grid, block, 0, s, static_cast<const float*>(b), w.next,
-                         w.leader, static_cast<int>(T), D, static_cast<int>(tch), w.partials);
-    else
-      hipLaunchKernelGGL(emb_norm_stream_kernel<bf16_t>, grid, block, 0, s, static_cast<const bf16_t*>(b), w.next,
-                         w.leader, static_cast<int>(T), D, static_cast<int>(tch), w.partials);
-    DPK_LAUNCH_CHECK(who);
-    dpk_launch_reduce_rows(w.partials, n, tch, norm, 1, fabsf(scale), s);
-    DPK_LAUNCH_CHECK(who);
-    return DPK_OK;
-  }
   const bool vec = D % 4 == 0 && dpk_aligned(b, dtype == DPK_BF16 ? 8 : 16);
   if (dtype == DPK_F32) launch_walk<float, float, 0>(vec, ids, b, w, n, T, D, 0, scale, nullptr, s);
   else launch_walk<bf16_t, float, 0>(vec, ids, b, w, n, T, D, 0, scale, nullptr, s);
