@@ -24,7 +24,13 @@ from typing import Callable, Iterable, List, Optional, Tuple
 import torch
 import torch.nn as nn
 
-from ..utils.module_utils import has_trainable_params, requires_grad, trainable_modules, trainable_parameters
+from ..utils.module_utils import (
+    has_trainable_params,
+    requires_grad,
+    trainable_modules,
+    trainable_parameter_list,
+    trainable_parameters,
+)
 from .functorch import ft_compute_per_sample_gradient, prepare_layer
 from .gsm_base import AbstractGradSampleHooks, AbstractGradSampleModule
 
@@ -223,21 +229,24 @@ class GradSampleHooks(AbstractGradSampleHooks):
             return
         if not isinstance(module, _ONE_TENSOR_OUT):
             return
-        params = [p for p in module.parameters(recurse=False) if p.requires_grad]
+        params = [p for p in module._parameters.values() if p is not None and p.requires_grad]
         if not params:
             return
-        inputs = list(args) + list(kwargs.values())
-        at_start = not any(isinstance(t, torch.Tensor) and t.requires_grad for t in inputs)
+        at_start = not any(isinstance(t, torch.Tensor) and t.requires_grad for t in args) and not any(
+            isinstance(t, torch.Tensor) and t.requires_grad for t in kwargs.values()
+        )
         for p in params:
             p.requires_grad_(False)
-        module._dpk_params_off = (params, at_start)
+        # plain attributes go through the instance dict: nn.Module.__setattr__ is a visible
+        # cost per layer and step for a small model
+        module.__dict__["_dpk_params_off"] = (params, at_start)
 
     def _params_back_on(self, module: nn.Module, _args, _output) -> None:
         state = module.__dict__.pop("_dpk_params_off", None)
         if state is not None:
             for p in state[0]:
                 p.requires_grad_(True)
-            module._dpk_at_start = state[1]
+            module.__dict__["_dpk_at_start"] = state[1]
 
     def _forward_hook(self, module: nn.Module, forward_input, forward_output, *, loss_reduction: str, batch_first: bool):
         """Captures the activations and arranges for ``capture_backprops_hook`` to run when the
@@ -246,12 +255,13 @@ class GradSampleHooks(AbstractGradSampleHooks):
         delivers the same ``grad_output`` without wrapping the module's inputs and outputs in
         an extra autograd node per call, which is what a small launch-bound model pays for
         in every step, and it tolerates an in-place op on the output."""
-        pending = len(getattr(module, "activations", ()))
+        d = module.__dict__
+        pending = len(d.get("activations", ()))
         self.capture_activations_hook(module, forward_input, forward_output)
-        if len(getattr(module, "activations", ())) == pending:
+        if len(d.get("activations", ())) == pending:
             return  # nothing captured: eval mode, no grad, hooks disabled, frozen module
         out = forward_output if isinstance(forward_output, torch.Tensor) else forward_output[0]
-        tapped = module.__dict__.pop("_dpk_at_start", False) and isinstance(forward_output, torch.Tensor)
+        tapped = d.pop("_dpk_at_start", False) and isinstance(forward_output, torch.Tensor)
         if tapped and not out.requires_grad:
             out = _GradTap.apply(out, self._tap_anchor)
         if not out.requires_grad:
@@ -290,15 +300,17 @@ class GradSampleHooks(AbstractGradSampleHooks):
 
     # ---- the hooks ----------------------------------------------------------------------
     def capture_activations_hook(self, module: nn.Module, forward_input: List[torch.Tensor], _forward_output):
-        if not requires_grad(module) or not module.training or not torch.is_grad_enabled():
+        if not self.hooks_enabled or not module.training or not torch.is_grad_enabled():
             return
-        if not self.hooks_enabled:
+        if not requires_grad(module):
             return
-        if not hasattr(module, "activations"):
-            module.activations = []
+        params = trainable_parameter_list(module)
+        acts = module.__dict__.get("activations")
+        if acts is None:
+            acts = module.__dict__["activations"] = []
         # non-tensor inputs (an omitted optional argument passed as None) are not activations
-        module.activations.append([t.detach() for t in forward_input if isinstance(t, torch.Tensor)])
-        for _, p in trainable_parameters(module):
+        acts.append([t.detach() for t in forward_input if isinstance(t, torch.Tensor)])
+        for p in params:
             p._forward_counter += 1
 
     def _sampler_for(self, module: nn.Module) -> Callable:
@@ -327,7 +339,7 @@ class GradSampleHooks(AbstractGradSampleHooks):
             if stacked is None:
                 return  # earlier uses of this pass are still to come
             activations, backprops = stacked
-            for _, p in trainable_parameters(module):
+            for p in trainable_parameter_list(module):
                 p._forward_counter += 1  # taken off again below, as for a module used once
         grad_samples = call_sampler(sampler, module, activations, backprops, scale)
         adopt = getattr(sampler, "owns_output", False)
@@ -335,7 +347,7 @@ class GradSampleHooks(AbstractGradSampleHooks):
             create_or_accumulate_grad_sample(
                 param=param, grad_sample=gs, max_batch_len=module.max_batch_len, adopt=adopt
             )
-        for _, p in trainable_parameters(module):
+        for p in trainable_parameter_list(module):
             p._forward_counter -= 1
             if p._forward_counter == 0:
                 promote_current_grad_sample(p)
@@ -346,8 +358,8 @@ class GradSampleHooks(AbstractGradSampleHooks):
                         "You need to call optimizer.step() after every forward/backward pass "
                         "or consider using BatchMemoryManager"
                     )
-        if len(module.activations) == 0 and hasattr(module, "max_batch_len"):
-            del module.max_batch_len
+        if len(module.activations) == 0:
+            module.__dict__.pop("max_batch_len", None)
 
     def _stack_uses(self, module: nn.Module, activations: List[torch.Tensor], backprops: torch.Tensor):
         """For a module applied many times per forward pass (``stack_uses``, the RNNLinear
@@ -388,8 +400,8 @@ class GradSampleHooks(AbstractGradSampleHooks):
         # the recurrent layers feed their RNNLinear batch first whatever the model's layout
         # (grad_sample_module.py:391)
         batch_dim = 0 if batch_first or getattr(module, "stack_uses", False) else 1
-        if not hasattr(module, "max_batch_len"):
-            module.max_batch_len = _get_batch_size(module=module, batch_dim=batch_dim)
+        if "max_batch_len" not in module.__dict__:
+            module.__dict__["max_batch_len"] = _get_batch_size(module=module, batch_dim=batch_dim)
         activations = module.activations.pop()
         if loss_reduction == "mean":
             scale = float(module.max_batch_len)
