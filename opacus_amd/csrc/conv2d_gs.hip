@@ -9,6 +9,10 @@
 // is): the n x C*KH*KW x OH*OW matrix the reference writes and re-reads never
 // exists. Only the group-diagonal blocks are computed, where the reference forms
 // the full O x p product and discards the rest (conv.py:102-112).
+#include <cstring>
+#include <mutex>
+#include <type_traits>
+
 #include "dpk_common.h"
 #include "mfma_f32.h"
 
@@ -30,6 +34,13 @@ struct ConvGeom {
 // Element (k = q, col = p) of the unfolded activation, staged as S[k][p].
 // D3: the input has a depth dimension as well (nn.Conv3d), p = (c, kd, kh, kw) and
 // q = (od, oh, ow).
+// The padded patch in LDS: Hp x Wp cells per channel, laid out with a row stride rs >= Wp and
+// a channel stride cs >= Hp * rs chosen so that the cells one wave reads at a time fall into
+// different LDS banks.
+struct PatchDims {
+  int Hp, Wp, rs, cs;
+};
+
 template <int BN, typename T, bool D3 = false>
 struct LoaderIm2col {
   static constexpr int R = mf32::BK * BN / mf32::NTHREADS;
@@ -217,7 +228,8 @@ template <int BM, int BN, typename TIN, typename TOUT, bool VEC>
 __global__ __launch_bounds__(kThreads) void conv2d_gs_patch_kernel(
     const TIN* __restrict__ x, const TIN* __restrict__ b, TOUT* __restrict__ gs,
     float* __restrict__ partials, ConvGeom g, int C, int O, int groups, float scale, int tiles_m,
-    int tiles_n, int Hp, int Wp, int xvec, int nch_max) {
+    int tiles_n, PatchDims pd, int xvec, int nch_max) {
+  const int Hp = pd.Hp, Wp = pd.Wp, RS = pd.rs, CS = pd.cs;
   using Tile = mf32::Tile<BM, BN>;
   extern __shared__ __align__(16) unsigned char dyn_lds[];
   // layout: qtab | patch. The k loop runs in trips of kPatchDepth k-tiles, all of them
@@ -254,10 +266,10 @@ __global__ __launch_bounds__(kThreads) void conv2d_gs_patch_kernel(
   const int rows = nch * Hp;
   constexpr int kRowsInFlight = 32;
   if (xvec) {
-    const int total4 = rows * Wp / 4;  // the patch starts 16-byte aligned; a ragged tail is zeroed below
+    const int total4 = nch * CS / 4;  // the patch starts 16-byte aligned; a ragged tail is zeroed below
     for (int i = threadIdx.x; i < total4; i += kThreads)
       reinterpret_cast<float4*>(xs)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int i = total4 * 4 + threadIdx.x; i < rows * Wp; i += kThreads) xs[i] = 0.f;
+    for (int i = total4 * 4 + threadIdx.x; i < nch * CS; i += kThreads) xs[i] = 0.f;
     __syncthreads();
     const int W4 = g.W / 4, chunks = nch * g.H * W4;
     constexpr int kChunksInFlight = 8;
@@ -274,7 +286,7 @@ __global__ __launch_bounds__(kThreads) void conv2d_gs_patch_kernel(
         if (i < chunks) {
           const int r = i / W4, x4 = i - r * W4;     // r = c * H + iy
           const int c = r / g.H, iy = r - c * g.H;
-          float* dst = xs + (c * Hp + iy + g.ph) * Wp + g.pw + x4 * 4;
+          float* dst = xs + c * CS + (iy + g.ph) * RS + g.pw + x4 * 4;
           dst[0] = v[u].x;
           dst[1] = v[u].y;
           dst[2] = v[u].z;
@@ -293,11 +305,13 @@ __global__ __launch_bounds__(kThreads) void conv2d_gs_patch_kernel(
     }
     for (int row = wave; row < rows; row += kWaves * kRowsInFlight) {
       float v[kRowsInFlight];
+      int cell[kRowsInFlight];
 #pragma unroll
       for (int u = 0; u < kRowsInFlight; ++u) {
         const int iy = y - g.ph;
         const bool in = col_ok && row + u * kWaves < rows && static_cast<unsigned>(iy) < static_cast<unsigned>(g.H);
         v[u] = in ? dpk_io<TIN>::load(xg + (static_cast<int64_t>(c) * g.H + iy) * g.W + ix) : 0.f;
+        cell[u] = c * CS + y * RS + xx;
         y += kWaves;
         while (y >= Hp) {
           y -= Hp;
@@ -307,13 +321,13 @@ __global__ __launch_bounds__(kThreads) void conv2d_gs_patch_kernel(
 #pragma unroll
       for (int u = 0; u < kRowsInFlight; ++u) {
         const int r = row + u * kWaves;
-        if (r < rows && xx < Wp) xs[r * Wp + xx] = v[u];
+        if (r < rows && xx < Wp) xs[cell[u]] = v[u];
       }
     }
   }
   for (int q = threadIdx.x; q < Qpad; q += kThreads) {
     const int oh = q / g.OW, ow = q - oh * g.OW;
-    qtab[q] = q < g.Q ? oh * g.sh * Wp + ow * g.sw : 0;
+    qtab[q] = q < g.Q ? oh * g.sh * RS + ow * g.sw : 0;
   }
   // this lane's columns of the tile
   const int wm0 = (wave >> 1) * Tile::WM, wn0 = (wave & 1) * Tile::WN;
@@ -325,7 +339,7 @@ __global__ __launch_bounds__(kThreads) void conv2d_gs_patch_kernel(
     if (p < g.Pg) {
       const int c = p / KK, rem = p - c * KK;
       const int kh = rem / g.KW, kw = rem - kh * g.KW;
-      base_p[j] = (c - c_lo) * Hp * Wp + kh * g.dh * Wp + kw * g.dw;
+      base_p[j] = (c - c_lo) * CS + kh * g.dh * RS + kw * g.dw;
     } else {
       base_p[j] = 0;  // result discarded below; any address inside the patch will do
     }
@@ -439,22 +453,375 @@ __global__ __launch_bounds__(kThreads) void conv2d_gs_patch_kernel(
   }
 }
 
+// ---- the patch kernel for bf16 input: v_mfma_f32_32x32x16_bf16 ---------------------------
+// Same plan as above (padded patch in LDS, backprops from global memory into registers, a
+// table of patch offsets per output position), with the operands left in bf16. The
+// instruction wants, per lane, 8 consecutive k of one row: half kk of the wave holds
+// k = 8 kk .. 8 kk + 7, which for the backprops is 16 contiguous bytes of global memory and
+// for the gathered operand eight 2-byte LDS reads at table offsets. One MFMA now does the work
+// of eight fp32 ones, so a k-tile's loads no longer hide behind its own arithmetic: the loop
+// runs in trips of kP16Tiles k-tiles and asks for everything of the next trip (offsets two
+// trips ahead) before the MFMAs of the current one.
+constexpr int kP16Tiles = 4;
+constexpr int kP16BK = 16;
+constexpr int kP16TripK = kP16Tiles * kP16BK;
+static_assert(kP16TripK == kPatchTrip, "both patch kernels pad the offset table alike");
+// a row of a trip's backprops in LDS: 64 k and 16 bytes of padding (rows 36 words apart: the
+// 16-byte fragment reads of 8 consecutive rows cover all 32 banks)
+constexpr int kP16RowBytes = kP16TripK * 2 + 16;
+constexpr size_t p16_stage_bytes(int bm) { return static_cast<size_t>(2) * bm * kP16RowBytes; }
+
+template <int BM, int BN, typename TOUT, bool VEC>
+__global__ __launch_bounds__(kThreads) void conv2d_gs_patch16_kernel(
+    const bf16_t* __restrict__ x, const bf16_t* __restrict__ b, TOUT* __restrict__ gs,
+    float* __restrict__ partials, ConvGeom g, int C, int O, int groups, float scale, int tiles_m,
+    int tiles_n, PatchDims pd, int xvec, int a_off) {
+  const int Hp = pd.Hp, Wp = pd.Wp, RS = pd.rs, CS = pd.cs;
+  using Tile = mf32::Tile<BM, BN>;  // accumulator layout of a 32 x 32 MFMA tile: the same
+  typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  extern __shared__ __align__(16) unsigned char dyn_lds[];
+  const int Qpad = (g.Q + kP16TripK - 1) / kP16TripK * kP16TripK;
+  int* qtab = reinterpret_cast<int*>(dyn_lds);  // byte offsets into the patch
+  uint16_t* xs = reinterpret_cast<uint16_t*>(qtab + Qpad);
+  __shared__ float red[kWaves];
+
+  const int Og = O / groups, Cg = C / groups;
+  int64_t bid = blockIdx.x;
+  const int tn = static_cast<int>(bid % tiles_n);
+  bid /= tiles_n;
+  const int tm = static_cast<int>(bid % tiles_m);
+  bid /= tiles_m;
+  const int grp = static_cast<int>(bid % groups);
+  const int64_t sample = bid / groups;
+  const int m0 = tm * BM, p0 = tn * BN;
+  const int KK = g.KH * g.KW;
+  const int c_lo = p0 / KK;
+  int c_hi = (p0 + BN - 1) / KK;
+  c_hi = c_hi < Cg ? c_hi : Cg - 1;
+  const int nch = c_hi - c_lo + 1;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+
+  // stage the patch as above, in bf16
+  const bf16_t* xg = x + ((sample * C + static_cast<int64_t>(grp) * Cg + c_lo) * g.H) * g.W;
+  const int rows = nch * Hp;
+  if (xvec) {
+    const int total8 = nch * CS / 8;  // 16-byte chunks; the patch starts 16-byte aligned
+    for (int i = threadIdx.x; i < total8; i += kThreads)
+      reinterpret_cast<uint4*>(xs)[i] = make_uint4(0u, 0u, 0u, 0u);
+    for (int i = total8 * 8 + threadIdx.x; i < nch * CS; i += kThreads) xs[i] = 0;
+    __syncthreads();
+    const int W4 = g.W / 4, chunks = nch * g.H * W4;
+    constexpr int kChunksInFlight = 8;
+    for (int i0 = threadIdx.x; i0 < chunks; i0 += kThreads * kChunksInFlight) {
+      dpk_vu2 v[kChunksInFlight];
+#pragma unroll
+      for (int u = 0; u < kChunksInFlight; ++u) {
+        const int i = i0 + u * kThreads;
+        v[u] = dpk_io<bf16_t>::load4_raw(xg + static_cast<int64_t>(i < chunks ? i : 0) * 4);
+      }
+#pragma unroll
+      for (int u = 0; u < kChunksInFlight; ++u) {
+        const int i = i0 + u * kThreads;
+        if (i < chunks) {
+          const int r = i / W4, x4 = i - r * W4;  // r = c * H + iy
+          const int c = r / g.H, iy = r - c * g.H;
+          uint16_t* dst = xs + c * CS + (iy + g.ph) * RS + g.pw + x4 * 4;
+          dst[0] = static_cast<uint16_t>(v[u].x);
+          dst[1] = static_cast<uint16_t>(v[u].x >> 16);
+          dst[2] = static_cast<uint16_t>(v[u].y);
+          dst[3] = static_cast<uint16_t>(v[u].y >> 16);
+        }
+      }
+    }
+  }
+  constexpr int kRowsInFlight = 32;
+  for (int x0 = 0; x0 < (xvec ? 0 : Wp); x0 += DPK_WAVE) {
+    const int xx = x0 + lane, ix = xx - g.pw;
+    const bool col_ok = xx < Wp && static_cast<unsigned>(ix) < static_cast<unsigned>(g.W);
+    int c = 0, y = wave;  // of the next row this wave stages
+    while (y >= Hp) {
+      y -= Hp;
+      ++c;
+    }
+    for (int row = wave; row < rows; row += kWaves * kRowsInFlight) {
+      uint16_t v[kRowsInFlight];
+      int cell[kRowsInFlight];
+#pragma unroll
+      for (int u = 0; u < kRowsInFlight; ++u) {
+        const int iy = y - g.ph;
+        const bool in = col_ok && row + u * kWaves < rows && static_cast<unsigned>(iy) < static_cast<unsigned>(g.H);
+        v[u] = in ? xg[(static_cast<int64_t>(c) * g.H + iy) * g.W + ix] : static_cast<uint16_t>(0);
+        cell[u] = c * CS + y * RS + xx;
+        y += kWaves;
+        while (y >= Hp) {
+          y -= Hp;
+          ++c;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kRowsInFlight; ++u) {
+        const int r = row + u * kWaves;
+        if (r < rows && xx < Wp) xs[cell[u]] = v[u];
+      }
+    }
+  }
+  for (int q = threadIdx.x; q < Qpad; q += kThreads) {
+    const int oh = q / g.OW, ow = q - oh * g.OW;
+    qtab[q] = q < g.Q ? (oh * g.sh * RS + ow * g.sw) * 2 : 0;
+  }
+  const int wm0 = (wave >> 1) * Tile::WM, wn0 = (wave & 1) * Tile::WN;
+  const int kk = lane >> 5, l32 = lane & 31;
+  // byte address inside the patch of this lane's patch element (its columns of the tile)
+  const unsigned char* xsb = reinterpret_cast<const unsigned char*>(xs);
+  int base_p[Tile::TN];
+#pragma unroll
+  for (int j = 0; j < Tile::TN; ++j) {
+    const int p = p0 + wn0 + j * 32 + l32;
+    if (p < g.Pg) {
+      const int c = p / KK, rem = p - c * KK;
+      const int kh = rem / g.KW, kw = rem - kh * g.KW;
+      base_p[j] = ((c - c_lo) * CS + kh * g.dh * RS + kw * g.dw) * 2;
+    } else {
+      base_p[j] = 0;  // result discarded below; any address inside the patch will do
+    }
+  }
+  // The backprop operand goes through LDS. Read straight into MFMA layout every lane would
+  // fetch 8 bytes of a different row, 64 cache lines per load instruction, and the address
+  // path of the CU (a line per cycle), not the MFMAs, would set the kernel's time. Here four
+  // threads share a row: a trip's 64 k of one row are one 128-byte line, requested two trips
+  // before they are used, written to LDS one trip before, and read back as 16-byte fragments.
+  const bf16_t* bg = b + (sample * O + static_cast<int64_t>(grp) * Og) * g.Q;
+  const __amdgpu_buffer_rsrc_t brs = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<bf16_t*>(bg), 0, Og * g.Q * static_cast<int>(sizeof(bf16_t)), 0x00020000);
+  constexpr uint32_t kOutside = 0x7fffffffu;
+  constexpr int kRowPasses = BM / 64;  // 256 threads cover 64 rows at a time
+  const int srow = threadIdx.x >> 2, sseg = threadIdx.x & 3;  // staging: row of the pass, 16 k of the trip
+  uint32_t stage_b[kRowPasses];  // byte offset of (row, k = 16 sseg), or past the end for a row outside
+#pragma unroll
+  for (int r = 0; r < kRowPasses; ++r) {
+    const int m = m0 + r * 64 + srow;
+    stage_b[r] = m < Og ? static_cast<uint32_t>(m * g.Q + sseg * 16) * 2u : kOutside;
+  }
+  const int ntrips = Qpad / kP16TripK;
+  const int nfull = g.Q / kP16TripK;  // trips whose every k is a real position
+  unsigned char* As = dyn_lds + a_off;  // [2][BM][kP16RowBytes]
+
+  uint32_t ga[2][kRowPasses][8];  // a trip's share of this thread, as loaded
+  uint32_t bv[2][kP16Tiles][Tile::TN][4];
+  int qo[kP16Tiles][8];
+  auto load_q = [&](int trip) {
+    trip = trip < ntrips ? trip : ntrips - 1;
+#pragma unroll
+    for (int t = 0; t < kP16Tiles; ++t) {
+      const int4* qt = reinterpret_cast<const int4*>(qtab + (trip * kP16Tiles + t) * kP16BK + kk * 8);
+      const int4 lo = qt[0], hi = qt[1];
+      qo[t][0] = lo.x; qo[t][1] = lo.y; qo[t][2] = lo.z; qo[t][3] = lo.w;
+      qo[t][4] = hi.x; qo[t][5] = hi.y; qo[t][6] = hi.z; qo[t][7] = hi.w;
+    }
+  };
+  auto load_b = [&](uint32_t (&bb)[kP16Tiles][Tile::TN][4]) {
+#pragma unroll
+    for (int t = 0; t < kP16Tiles; ++t)
+#pragma unroll
+      for (int j = 0; j < Tile::TN; ++j)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const uint32_t lo = *reinterpret_cast<const uint16_t*>(xsb + base_p[j] + qo[t][2 * e]);
+          const uint32_t hi = *reinterpret_cast<const uint16_t*>(xsb + base_p[j] + qo[t][2 * e + 1]);
+          bb[t][j][e] = lo | (hi << 16);
+        }
+  };
+  // global -> registers: 16 k (32 bytes) of each of this thread's rows
+  auto load_a = [&](int trip, uint32_t (&aa)[kRowPasses][8]) {
+    trip = trip < ntrips ? trip : ntrips - 1;
+    const bool tail = trip >= nfull;  // uniform
+    const int k0 = trip * kP16TripK + sseg * 16;  // this thread's first k
+#pragma unroll
+    for (int r = 0; r < kRowPasses; ++r) {
+      if (VEC) {
+#pragma unroll
+        for (int h = 0; h < 4; ++h) {
+          uint32_t off = stage_b[r] + static_cast<uint32_t>(trip * kP16TripK + 4 * h) * 2u;
+          if (tail && k0 + 4 * h >= g.Q) off = kOutside;
+          typedef int vi2 __attribute__((ext_vector_type(2)));
+          const vi2 v = __builtin_amdgcn_raw_buffer_load_b64(brs, off, 0, 0);
+          aa[r][2 * h + 0] = static_cast<uint32_t>(v.x);
+          aa[r][2 * h + 1] = static_cast<uint32_t>(v.y);
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          uint32_t o0 = stage_b[r] + static_cast<uint32_t>(trip * kP16TripK + 2 * e) * 2u, o1 = o0 + 2u;
+          if (k0 + 2 * e >= g.Q) o0 = kOutside;
+          if (k0 + 2 * e + 1 >= g.Q) o1 = kOutside;
+          const uint32_t lo = static_cast<uint16_t>(__builtin_amdgcn_raw_buffer_load_b16(brs, o0, 0, 0));
+          const uint32_t hi = static_cast<uint16_t>(__builtin_amdgcn_raw_buffer_load_b16(brs, o1, 0, 0));
+          aa[r][e] = lo | (hi << 16);
+        }
+      }
+    }
+  };
+  // registers -> LDS buffer buf
+  auto store_a = [&](int buf, const uint32_t (&aa)[kRowPasses][8]) {
+#pragma unroll
+    for (int r = 0; r < kRowPasses; ++r) {
+      uint4* dst = reinterpret_cast<uint4*>(As + (static_cast<size_t>(buf) * BM + r * 64 + srow) * kP16RowBytes + sseg * 32);
+      dst[0] = make_uint4(aa[r][0], aa[r][1], aa[r][2], aa[r][3]);
+      dst[1] = make_uint4(aa[r][4], aa[r][5], aa[r][6], aa[r][7]);
+    }
+  };
+  Tile tile;
+  tile.clear();
+  load_a(0, ga[0]);
+  load_a(1, ga[1]);
+  store_a(0, ga[0]);
+  load_a(2, ga[0]);
+  __syncthreads();  // publishes the patch, the table and the first trip's backprops
+  load_q(0);
+  load_b(bv[0]);
+  load_q(1);
+  auto trip_body = [&](auto cur_c, int trip) {
+    constexpr int cur = decltype(cur_c)::value, nxt = cur ^ 1;
+    load_b(bv[nxt]);   // uses the offsets of trip + 1
+    load_q(trip + 2);  // and frees them for trip + 2
+    uint4 av[kP16Tiles][Tile::TM];
+#pragma unroll
+    for (int t = 0; t < kP16Tiles; ++t)
+#pragma unroll
+      for (int i = 0; i < Tile::TM; ++i)
+        av[t][i] = *reinterpret_cast<const uint4*>(
+            As + (static_cast<size_t>(cur) * BM + wm0 + i * 32 + l32) * kP16RowBytes + t * 32 + kk * 16);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int t = 0; t < kP16Tiles; ++t)
+#pragma unroll
+      for (int i = 0; i < Tile::TM; ++i)
+#pragma unroll
+        for (int j = 0; j < Tile::TN; ++j) {
+          const u32x4 ar = {av[t][i].x, av[t][i].y, av[t][i].z, av[t][i].w};
+          const u32x4 br = {bv[cur][t][j][0], bv[cur][t][j][1], bv[cur][t][j][2], bv[cur][t][j][3]};
+          tile.acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+              __builtin_bit_cast(bf16x8, ar), __builtin_bit_cast(bf16x8, br), tile.acc[i][j], 0, 0, 0);
+        }
+    // trip + 1's backprops (asked for two trips ago) move to the other buffer, whose last
+    // readers passed the barrier that ended the previous trip; trip + 3 takes their registers
+    store_a(nxt, ga[nxt]);
+    load_a(trip + 3, ga[nxt]);
+    __syncthreads();
+  };
+  for (int trip = 0; trip < ntrips; trip += 2) {
+    trip_body(std::integral_constant<int, 0>(), trip);
+    if (trip + 1 < ntrips) trip_body(std::integral_constant<int, 1>(), trip + 1);
+  }
+  TOUT* out = gs + (sample * O + static_cast<int64_t>(grp) * Og) * g.Pg;
+  float ss = 0.f;
+  tile.for_each([&](int r, int c, float v) {
+    const int m = m0 + r, p = p0 + c;
+    if (m < Og && p < g.Pg) {
+      const float val = v * scale;
+      if (gs) dpk_io<TOUT>::store(out + static_cast<int64_t>(m) * g.Pg + p, val);
+      ss = fmaf(val, val, ss);
+    }
+  });
+  if (partials) {
+    const float s = block_sum<kWaves>(ss, red);
+    if (threadIdx.x == 0) partials[blockIdx.x] = s;
+  }
+}
+
+
 // Most LDS the patch kernel asks for. Above 64 KB a kernel must be told so once
 // (hipFuncSetAttribute); one block then has a CU's LDS nearly to itself, which still beats
 // gathering the operand from global memory (64 -> 64 channels, 3 x 3 on 56 x 56 images, whose
 // patch is 107 KB: 228 us against 371 us).
 constexpr size_t kPatchLdsLimit = 150 * 1024;  // of the CU's 160 KB
 
-// LDS bytes of the patch kernel for a 64 x 64 tile, or 0 if the geometry does not fit.
-size_t patch_lds_bytes(const ConvGeom& g, int Cg, int Hp, int Wp) {
+// Layout and LDS bytes of the patch kernels for a 64 x 64 tile; bytes == 0 if the geometry does
+// not fit. At one position of the k loop the 32 lanes of a half-wave read the patch cells of
+// 32 consecutive columns p = (c, kh, kw), at c * cs + kh * dh * rs + kw * dw: with rs = Wp and
+// cs = Hp * Wp those land in a handful of the 32 banks (3 x 3 on a 34-wide patch: three and
+// four to a bank). A few cells of padding per row and channel, searched here, spread them out.
+struct PatchLayout {
+  PatchDims d;
+  size_t bytes;
+  int a_off;  // bf16 kernel: where the staged backprops start
+};
+PatchLayout search_patch_layout(const ConvGeom& g, int Cg, int Hp, int Wp, size_t elsize);
+
+// The search costs tens of microseconds, a model calls with the same few geometries step
+// after step: the last results are kept.
+PatchLayout patch_layout(const ConvGeom& g, int Cg, int Hp, int Wp, size_t elsize) {
+  struct Entry {
+    int key[10];
+    PatchLayout value;
+  };
+  static std::mutex mu;
+  static Entry cache[32];
+  static int used = 0, next = 0;
+  const int key[10] = {g.KH, g.KW, g.dh, g.dw, g.Q, Cg, Hp, Wp, static_cast<int>(elsize), 0};
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    for (int i = 0; i < used; ++i)
+      if (std::memcmp(cache[i].key, key, sizeof(key)) == 0) return cache[i].value;
+  }
+  const PatchLayout v = search_patch_layout(g, Cg, Hp, Wp, elsize);
+  std::lock_guard<std::mutex> lock(mu);
+  Entry& e = cache[next];
+  std::memcpy(e.key, key, sizeof(key));
+  e.value = v;
+  next = (next + 1) % 32;
+  if (used < 32) ++used;
+  return v;
+}
+
+PatchLayout search_patch_layout(const ConvGeom& g, int Cg, int Hp, int Wp, size_t elsize) {
   const int KK = g.KH * g.KW;
   int nch = (64 + KK - 2) / KK + 1;  // channels a run of 64 columns can touch
   if (nch > Cg) nch = Cg;
-  const size_t a_bytes = 0;  // the backprop operand is not staged
   const size_t q_bytes = static_cast<size_t>((g.Q + kPatchTrip - 1) / kPatchTrip * kPatchTrip) * sizeof(int);
-  const size_t x_bytes = static_cast<size_t>(nch) * Hp * Wp * sizeof(float);
-  const size_t total = a_bytes + q_bytes + x_bytes;
-  return total <= kPatchLdsLimit ? total : 0;
+  const size_t a_bytes = elsize == 2 ? p16_stage_bytes(64) : 0;
+  PatchLayout best;
+  best.d = PatchDims{Hp, Wp, Wp, Hp * Wp};
+  best.bytes = 0;
+  best.a_off = 0;
+  long best_cost = -1;
+  for (int padr = 0; padr < 8; ++padr) {
+    for (int padc = 0; padc < 32; ++padc) {
+      const int rs = Wp + padr, cs = Hp * rs + padc;
+      const size_t bytes = q_bytes + dpk_align_up(static_cast<size_t>(nch) * cs * elsize, 16) + a_bytes;
+      if (bytes > kPatchLdsLimit) continue;
+      // most distinct 4-byte words any bank serves, summed over the two half-tiles of columns
+      long cost = 0;
+      for (int p0 = 0; p0 < 64; p0 += 32) {
+        long word_of[32][8];
+        int served[32] = {0};
+        for (int l = 0; l < 32; ++l) {
+          const int p = p0 + l, c = p / KK, rem = p - c * KK, kh = rem / g.KW, kw = rem - kh * g.KW;
+          if (c >= nch) continue;
+          const long word = (static_cast<long>(c) * cs + kh * g.dh * rs + kw * g.dw) * static_cast<long>(elsize) / 4;
+          const int bank = static_cast<int>(word % 32);
+          bool seen = false;
+          for (int k = 0; k < served[bank] && k < 8; ++k) seen = seen || word_of[bank][k] == word;
+          if (!seen) {
+            if (served[bank] < 8) word_of[bank][served[bank]] = word;
+            ++served[bank];
+          }
+        }
+        int worst = 0;
+        for (int k = 0; k < 32; ++k) worst = served[k] > worst ? served[k] : worst;
+        cost += worst;
+      }
+      // fewer conflicts first, then the smaller patch (more blocks per CU)
+      if (best_cost < 0 || cost < best_cost || (cost == best_cost && bytes < best.bytes)) {
+        best_cost = cost;
+        best.d = PatchDims{Hp, Wp, rs, cs};
+        best.bytes = bytes;
+        best.a_off = static_cast<int>(bytes - a_bytes);
+      }
+    }
+  }
+  return best;
 }
 
 struct Plan {
@@ -482,17 +849,23 @@ Plan make_plan(int64_t Og, int64_t Pg, bool small = false) {
 template <typename TIN, typename TOUT>
 void launch(const Plan& p, bool vec, const void* x, const void* b, void* gs, float* partials,
             const ConvGeom& g, int64_t n, int C, int O, int groups, float scale, hipStream_t s,
-            size_t patch_bytes, int Hp, int Wp, int ksplit, int kchunk, float* split_out) {
+            size_t patch_bytes, PatchDims pd, int a_off, int ksplit, int kchunk, float* split_out) {
   const dim3 grid(static_cast<unsigned>(n * groups * p.tiles_m * p.tiles_n * ksplit)), block(kThreads);
   const TIN* xp = static_cast<const TIN*>(x);
   const TIN* bp = static_cast<const TIN*>(b);
   TOUT* gp = static_cast<TOUT*>(gs);
   bool use_patch = patch_bytes > 0;
+  constexpr bool kIn16 = std::is_same<TIN, bf16_t>::value;
   if (patch_bytes > 64 * 1024 - 64) {
     // per device and cheap: said again at every such launch rather than remembered. A device
     // or runtime that refuses that much LDS gets the gather kernel on the same 64 x 64 plan.
-    const void* fn = vec ? reinterpret_cast<const void*>(&conv2d_gs_patch_kernel<64, 64, TIN, TOUT, true>)
-                         : reinterpret_cast<const void*>(&conv2d_gs_patch_kernel<64, 64, TIN, TOUT, false>);
+    const void* fn;
+    if constexpr (kIn16)
+      fn = vec ? reinterpret_cast<const void*>(&conv2d_gs_patch16_kernel<64, 64, TOUT, true>)
+               : reinterpret_cast<const void*>(&conv2d_gs_patch16_kernel<64, 64, TOUT, false>);
+    else
+      fn = vec ? reinterpret_cast<const void*>(&conv2d_gs_patch_kernel<64, 64, TIN, TOUT, true>)
+               : reinterpret_cast<const void*>(&conv2d_gs_patch_kernel<64, 64, TIN, TOUT, false>);
     if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kPatchLdsLimit)) !=
         hipSuccess) {
       (void)hipGetLastError();  // the refusal is handled here, not reported by the next launch check
@@ -502,12 +875,21 @@ void launch(const Plan& p, bool vec, const void* x, const void* b, void* gs, flo
   if (use_patch) {
     // image rows made of whole, aligned 4-element chunks: the patch interior is staged with vector loads
     const int xvec = (g.W % 4 == 0 && dpk_aligned(x, sizeof(TIN) == 2 ? 8 : 16)) ? 1 : 0;
-    if (vec)
-      hipLaunchKernelGGL((conv2d_gs_patch_kernel<64, 64, TIN, TOUT, true>), grid, block, patch_bytes, s, xp,
-                         bp, gp, partials, g, C, O, groups, scale, p.tiles_m, p.tiles_n, Hp, Wp, xvec, 0);
-    else
-      hipLaunchKernelGGL((conv2d_gs_patch_kernel<64, 64, TIN, TOUT, false>), grid, block, patch_bytes, s,
-                         xp, bp, gp, partials, g, C, O, groups, scale, p.tiles_m, p.tiles_n, Hp, Wp, xvec, 0);
+    if constexpr (kIn16) {
+      if (vec)
+        hipLaunchKernelGGL((conv2d_gs_patch16_kernel<64, 64, TOUT, true>), grid, block, patch_bytes, s, xp, bp,
+                           gp, partials, g, C, O, groups, scale, p.tiles_m, p.tiles_n, pd, xvec, a_off);
+      else
+        hipLaunchKernelGGL((conv2d_gs_patch16_kernel<64, 64, TOUT, false>), grid, block, patch_bytes, s, xp, bp,
+                           gp, partials, g, C, O, groups, scale, p.tiles_m, p.tiles_n, pd, xvec, a_off);
+    } else {
+      if (vec)
+        hipLaunchKernelGGL((conv2d_gs_patch_kernel<64, 64, TIN, TOUT, true>), grid, block, patch_bytes, s, xp,
+                           bp, gp, partials, g, C, O, groups, scale, p.tiles_m, p.tiles_n, pd, xvec, 0);
+      else
+        hipLaunchKernelGGL((conv2d_gs_patch_kernel<64, 64, TIN, TOUT, false>), grid, block, patch_bytes, s,
+                           xp, bp, gp, partials, g, C, O, groups, scale, p.tiles_m, p.tiles_n, pd, xvec, 0);
+    }
     return;
   }
 #define DPK_CONV_LAUNCH(BM, BN, V, D3)                                                            \
@@ -618,10 +1000,13 @@ int conv_gs(const char* who, const void* x, const void* b, int in_dtype, void* g
   g.OHW = (int)(OH * OW);
   const int64_t Hp = H + ph_lo + ph_hi, Wp = W + pw_lo + pw_hi;
   const bool flat = z.D == 1 && z.KD == 1 && z.pd_lo == 0 && z.pd_hi == 0;  // the LDS patch is two-dimensional
-  const size_t patch_bytes =
-      flat && Hp * Wp < (1 << 20) && (O / groups) * Q * 4 < (1LL << 30)
-          ? patch_lds_bytes(g, (int)(C / groups), (int)Hp, (int)Wp)
-          : 0;
+  PatchLayout pl;
+  pl.d = PatchDims{(int)Hp, (int)Wp, (int)Wp, (int)(Hp * Wp)};
+  pl.bytes = 0;
+  pl.a_off = 0;
+  if (flat && Hp * Wp < (1 << 20) && (O / groups) * Q * 4 < (1LL << 30))
+    pl = patch_layout(g, (int)(C / groups), (int)Hp, (int)Wp, in_dtype == DPK_BF16 ? 2 : 4);
+  const size_t patch_bytes = pl.bytes;
   const Plan p = make_plan(O / groups, Pg, patch_bytes > 0);
   const int64_t blocks = n * groups * p.tiles_m * p.tiles_n;
   // few long blocks on the gather kernel: cut the contraction over the positions into pieces,
@@ -647,16 +1032,16 @@ int conv_gs(const char* who, const void* x, const void* b, int in_dtype, void* g
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (in_dtype == DPK_F32 && gs_dtype == DPK_F32)
     launch<float, float>(p, vec, x, b, gs, partials, g, n, (int)C, (int)O, (int)groups, scale, s, patch_bytes,
-                       (int)Hp, (int)Wp, ksplit, kchunk, split_out);
+                       pl.d, pl.a_off, ksplit, kchunk, split_out);
   else if (in_dtype == DPK_BF16 && gs_dtype == DPK_BF16)
     launch<bf16_t, bf16_t>(p, vec, x, b, gs, partials, g, n, (int)C, (int)O, (int)groups, scale, s, patch_bytes,
-                         (int)Hp, (int)Wp, ksplit, kchunk, split_out);
+                         pl.d, pl.a_off, ksplit, kchunk, split_out);
   else if (in_dtype == DPK_BF16 && gs_dtype == DPK_F32)
     launch<bf16_t, float>(p, vec, x, b, gs, partials, g, n, (int)C, (int)O, (int)groups, scale, s, patch_bytes,
-                        (int)Hp, (int)Wp, ksplit, kchunk, split_out);
+                        pl.d, pl.a_off, ksplit, kchunk, split_out);
   else
     launch<float, bf16_t>(p, vec, x, b, gs, partials, g, n, (int)C, (int)O, (int)groups, scale, s, patch_bytes,
-                        (int)Hp, (int)Wp, ksplit, kchunk, split_out);
+                        pl.d, pl.a_off, ksplit, kchunk, split_out);
   DPK_LAUNCH_CHECK(who);
   int64_t cols = static_cast<int64_t>(groups) * p.tiles_m * p.tiles_n;
   if (ksplit > 1) {
