@@ -747,11 +747,11 @@ struct PatchLayout {
   size_t bytes;
   int a_off;  // bf16 kernel: where the staged backprops start
 };
-PatchLayout search_patch_layout(const ConvGeom& g, int Cg, int Hp, int Wp, size_t elsize);
+PatchLayout search_patch_layout(const ConvGeom& g, int Cg, int Hp, int Wp, size_t elsize, size_t a_bytes);
 
 // The search costs tens of microseconds, a model calls with the same few geometries step
 // after step: the last results are kept.
-PatchLayout patch_layout(const ConvGeom& g, int Cg, int Hp, int Wp, size_t elsize) {
+PatchLayout patch_layout(const ConvGeom& g, int Cg, int Hp, int Wp, size_t elsize, size_t a_bytes) {
   struct Entry {
     int key[10];
     PatchLayout value;
@@ -759,13 +759,13 @@ PatchLayout patch_layout(const ConvGeom& g, int Cg, int Hp, int Wp, size_t elsiz
   static std::mutex mu;
   static Entry cache[32];
   static int used = 0, next = 0;
-  const int key[10] = {g.KH, g.KW, g.dh, g.dw, g.Q, Cg, Hp, Wp, static_cast<int>(elsize), 0};
+  const int key[10] = {g.KH, g.KW, g.dh, g.dw, g.Q, Cg, Hp, Wp, static_cast<int>(elsize), static_cast<int>(a_bytes)};
   {
     std::lock_guard<std::mutex> lock(mu);
     for (int i = 0; i < used; ++i)
       if (std::memcmp(cache[i].key, key, sizeof(key)) == 0) return cache[i].value;
   }
-  const PatchLayout v = search_patch_layout(g, Cg, Hp, Wp, elsize);
+  const PatchLayout v = search_patch_layout(g, Cg, Hp, Wp, elsize, a_bytes);
   std::lock_guard<std::mutex> lock(mu);
   Entry& e = cache[next];
   std::memcpy(e.key, key, sizeof(key));
@@ -775,12 +775,11 @@ PatchLayout patch_layout(const ConvGeom& g, int Cg, int Hp, int Wp, size_t elsiz
   return v;
 }
 
-PatchLayout search_patch_layout(const ConvGeom& g, int Cg, int Hp, int Wp, size_t elsize) {
+PatchLayout search_patch_layout(const ConvGeom& g, int Cg, int Hp, int Wp, size_t elsize, size_t a_bytes) {
   const int KK = g.KH * g.KW;
   int nch = (64 + KK - 2) / KK + 1;  // channels a run of 64 columns can touch
   if (nch > Cg) nch = Cg;
   const size_t q_bytes = static_cast<size_t>((g.Q + kPatchTrip - 1) / kPatchTrip * kPatchTrip) * sizeof(int);
-  const size_t a_bytes = elsize == 2 ? p16_stage_bytes(64) : 0;
   PatchLayout best;
   best.d = PatchDims{Hp, Wp, Wp, Hp * Wp};
   best.bytes = 0;
@@ -860,9 +859,14 @@ void launch(const Plan& p, bool vec, const void* x, const void* b, void* gs, flo
     // per device and cheap: said again at every such launch rather than remembered. A device
     // or runtime that refuses that much LDS gets the gather kernel on the same 64 x 64 plan.
     const void* fn;
-    if constexpr (kIn16)
-      fn = vec ? reinterpret_cast<const void*>(&conv2d_gs_patch16_kernel<64, 64, TOUT, true>)
-               : reinterpret_cast<const void*>(&conv2d_gs_patch16_kernel<64, 64, TOUT, false>);
+    if constexpr (kIn16) {
+      if (p.bm == 128)
+        fn = vec ? reinterpret_cast<const void*>(&conv2d_gs_patch16_kernel<128, 64, TOUT, true>)
+                 : reinterpret_cast<const void*>(&conv2d_gs_patch16_kernel<128, 64, TOUT, false>);
+      else
+        fn = vec ? reinterpret_cast<const void*>(&conv2d_gs_patch16_kernel<64, 64, TOUT, true>)
+                 : reinterpret_cast<const void*>(&conv2d_gs_patch16_kernel<64, 64, TOUT, false>);
+    }
     else
       fn = vec ? reinterpret_cast<const void*>(&conv2d_gs_patch_kernel<64, 64, TIN, TOUT, true>)
                : reinterpret_cast<const void*>(&conv2d_gs_patch_kernel<64, 64, TIN, TOUT, false>);
@@ -876,12 +880,17 @@ void launch(const Plan& p, bool vec, const void* x, const void* b, void* gs, flo
     // image rows made of whole, aligned 4-element chunks: the patch interior is staged with vector loads
     const int xvec = (g.W % 4 == 0 && dpk_aligned(x, sizeof(TIN) == 2 ? 8 : 16)) ? 1 : 0;
     if constexpr (kIn16) {
-      if (vec)
-        hipLaunchKernelGGL((conv2d_gs_patch16_kernel<64, 64, TOUT, true>), grid, block, patch_bytes, s, xp, bp,
-                           gp, partials, g, C, O, groups, scale, p.tiles_m, p.tiles_n, pd, xvec, a_off);
-      else
-        hipLaunchKernelGGL((conv2d_gs_patch16_kernel<64, 64, TOUT, false>), grid, block, patch_bytes, s, xp, bp,
-                           gp, partials, g, C, O, groups, scale, p.tiles_m, p.tiles_n, pd, xvec, a_off);
+#define DPK_P16_LAUNCH(BM_, V)                                                                          \
+  hipLaunchKernelGGL((conv2d_gs_patch16_kernel<BM_, 64, TOUT, V>), grid, block, patch_bytes, s, xp, bp, \
+                     gp, partials, g, C, O, groups, scale, p.tiles_m, p.tiles_n, pd, xvec, a_off)
+      if (p.bm == 128) {
+        if (vec) DPK_P16_LAUNCH(128, true);
+        else DPK_P16_LAUNCH(128, false);
+      } else {
+        if (vec) DPK_P16_LAUNCH(64, true);
+        else DPK_P16_LAUNCH(64, false);
+      }
+#undef DPK_P16_LAUNCH
     } else {
       if (vec)
         hipLaunchKernelGGL((conv2d_gs_patch_kernel<64, 64, TIN, TOUT, true>), grid, block, patch_bytes, s, xp,
@@ -1004,10 +1013,24 @@ int conv_gs(const char* who, const void* x, const void* b, int in_dtype, void* g
   pl.d = PatchDims{(int)Hp, (int)Wp, (int)Wp, (int)(Hp * Wp)};
   pl.bytes = 0;
   pl.a_off = 0;
-  if (flat && Hp * Wp < (1 << 20) && (O / groups) * Q * 4 < (1LL << 30))
-    pl = patch_layout(g, (int)(C / groups), (int)Hp, (int)Wp, in_dtype == DPK_BF16 ? 2 : 4);
+  int bm16 = 64;
+  if (flat && Hp * Wp < (1 << 20) && (O / groups) * Q * 4 < (1LL << 30)) {
+    // bf16 input: 128 output channels per block where the layer has them (each gathered
+    // fragment then feeds two MFMAs), if the staged backprops of 128 rows still fit
+    if (in_dtype == DPK_BF16 && O / groups >= 128) {
+      pl = patch_layout(g, (int)(C / groups), (int)Hp, (int)Wp, 2, p16_stage_bytes(128));
+      bm16 = pl.bytes > 0 ? 128 : 64;
+    }
+    if (pl.bytes == 0)
+      pl = patch_layout(g, (int)(C / groups), (int)Hp, (int)Wp, in_dtype == DPK_BF16 ? 2 : 4,
+                        in_dtype == DPK_BF16 ? p16_stage_bytes(64) : 0);
+  }
   const size_t patch_bytes = pl.bytes;
-  const Plan p = make_plan(O / groups, Pg, patch_bytes > 0);
+  Plan p = make_plan(O / groups, Pg, patch_bytes > 0);
+  if (patch_bytes > 0 && bm16 == 128) {
+    p.bm = 128;
+    p.tiles_m = static_cast<int>(dpk_cdiv(O / groups, 128));
+  }
   const int64_t blocks = n * groups * p.tiles_m * p.tiles_n;
   // few long blocks on the gather kernel: cut the contraction over the positions into pieces,
   // if the caller's workspace has room for their raw tiles

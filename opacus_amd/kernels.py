@@ -280,8 +280,10 @@ def conv2d_grad_sample(
     scale: float = 1.0,
     want_sumsq: bool = True,
     norm_only: bool = False,
+    out_dtype: Optional[torch.dtype] = None,
 ) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
-    """Per-sample weight gradients ``[n, O, C/groups, KH, KW]`` of a 2-d convolution.
+    """Per-sample weight gradients ``[n, O, C/groups, KH, KW]`` of a 2-d convolution
+    (in ``out_dtype``, by default the backprops' dtype).
 
     ``padding`` is ``(top, bottom, left, right)``; ``backprops`` is ``[n, O, OH, OW]``.
     ``norm_only``: the gradient tiles are formed and squared but never stored; returns
@@ -294,7 +296,7 @@ def conv2d_grad_sample(
     O = backprops.shape[1]
     KH, KW = kernel_size
     want_sumsq = want_sumsq or norm_only
-    gs = None if norm_only else torch.empty((n, O, C // groups, KH, KW), dtype=backprops.dtype, device=dev)
+    gs = None if norm_only else torch.empty((n, O, C // groups, KH, KW), dtype=out_dtype or backprops.dtype, device=dev)
     sumsq = torch.empty((n,), dtype=torch.float32, device=dev) if want_sumsq else None
     if n == 0:
         return gs, sumsq
@@ -312,7 +314,7 @@ def conv2d_grad_sample(
         check(
             "dpk_conv2d_gs",
             L.dpk_conv2d_gs(
-                _ptr(x), _ptr(b), _code(b), _ptr(gs), _code(b), _ptr(sumsq), n, C, H, W, O, KH, KW,
+                _ptr(x), _ptr(b), _code(b), _ptr(gs), _code(out_dtype or b.dtype), _ptr(sumsq), n, C, H, W, O, KH, KW,
                 stride[0], stride[1], padding[0], padding[1], padding[2], padding[3], dilation[0],
                 dilation[1], groups, float(scale), _ptr(ws), wsb, _stream(dev),
             ),

@@ -520,14 +520,46 @@ def test_conv2d_grad_sample_f32(K, case, scale):
     assert_rel(K.conv_bias_grad_sample(dev(b), scale=scale), want_b, FP32_REL, "conv bias")
 
 
-def test_conv2d_grad_sample_bf16(K):
-    torch.manual_seed(77)
-    x = torch.randn(2, 8, 9, 9).bfloat16()
-    b = torch.randn(2, 12, 9, 9).bfloat16()
-    want_w, _ = O.conv2d_grad_sample(x.double(), b.double(), kernel_size=(3, 3), padding=(1, 1), stride=(1, 1), dilation=(1, 1), groups=1)
-    gs, _ = K.conv2d_grad_sample(dev(x), dev(b), (3, 3), (1, 1), (1, 1, 1, 1), (1, 1), 1)
-    assert gs.dtype == torch.bfloat16
-    assert_rel(gs, want_w, BF16_REL)
+# bf16 input runs its own kernel (bf16 MFMA; the gathered operand read in groups of 8, 4, 2 or 1
+# positions according to the output width and stride): every group size, row-wise and chunked
+# staging of the patch, ragged last trips of the k loop, misaligned backprops
+CONV_BF16_EXTRA = [
+    dict(n=2, C=8, O=12, k=(3, 3), stride=(1, 1), padding=(1, 1), dilation=(1, 1), groups=1, H=9, W=9),     # groups of 1
+    dict(n=2, C=8, O=70, k=(3, 3), stride=(1, 1), padding=(1, 1), dilation=(1, 1), groups=1, H=5, W=6),     # groups of 2, Q % 4 != 0
+    dict(n=2, C=12, O=20, k=(3, 3), stride=(1, 1), padding=(1, 1), dilation=(1, 1), groups=1, H=7, W=12),   # groups of 4
+    dict(n=2, C=12, O=20, k=(3, 3), stride=(1, 1), padding=(1, 1), dilation=(1, 1), groups=2, H=10, W=24),  # groups of 8
+    dict(n=2, C=5, O=9, k=(3, 5), stride=(1, 1), padding=(0, 3), dilation=(2, 2), groups=1, H=12, W=18),    # dilated, groups of 8
+    dict(n=2, C=4, O=8, k=(1, 3), stride=(1, 1), padding=(0, 1), dilation=(1, 1), groups=1, H=1, W=200),    # a Conv1d's shape
+]
+
+
+@pytest.mark.parametrize("case", CONV_CASES + CONV_BF16_EXTRA)
+@pytest.mark.parametrize("out_f32", [False, True])
+def test_conv2d_grad_sample_bf16(K, case, out_f32):
+    torch.manual_seed(case["C"] * 31 + case["O"] + 5)
+    n = case["n"]
+    x = torch.randn(n, case["C"], case["H"], case["W"]).bfloat16()
+    pad = O.conv2d_padding(case["padding"], case["k"], case["dilation"])
+    oh = (case["H"] + pad[0] + pad[1] - (case["dilation"][0] * (case["k"][0] - 1) + 1)) // case["stride"][0] + 1
+    ow = (case["W"] + pad[2] + pad[3] - (case["dilation"][1] * (case["k"][1] - 1) + 1)) // case["stride"][1] + 1
+    b = torch.randn(n, case["O"], oh, ow).bfloat16()
+    want_w, _ = O.conv2d_grad_sample(
+        x.double(), (b.double() * 0.5), kernel_size=case["k"], padding=case["padding"], stride=case["stride"],
+        dilation=case["dilation"], groups=case["groups"],
+    )
+    gs, sumsq = K.conv2d_grad_sample(
+        dev(x), dev(b), case["k"], case["stride"], pad, case["dilation"], case["groups"], scale=0.5,
+        out_dtype=torch.float32 if out_f32 else None,
+    )
+    assert gs.dtype == (torch.float32 if out_f32 else torch.bfloat16)
+    # exact products of bf16 inputs, fp32 accumulation: only a bf16 output rounds
+    assert_rel(gs, want_w, FP32_REL if out_f32 else BF16_REL, "conv weight bf16")
+    assert_rel(sumsq, want_w.flatten(1).pow(2).sum(1), 2e-5, "conv sumsq bf16")
+    # backprops that start 2 bytes off a 16-byte boundary take the element-wise loads
+    odd = torch.empty(b.numel() + 1, dtype=torch.bfloat16, device="cuda")[1:].view(b.shape).copy_(b)
+    gs2, _ = K.conv2d_grad_sample(dev(x), odd, case["k"], case["stride"], pad, case["dilation"], case["groups"], scale=0.5,
+                                  out_dtype=torch.float32 if out_f32 else None)
+    assert torch.equal(gs2, gs)
 
 
 CONV3D_GPU_CASES = [
