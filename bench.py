@@ -682,6 +682,18 @@ def kernel_table(dev, iters: int = 10, warm: int = 3, with_cpu: bool = True):
               2.0 * n * 64 * 576 * 1024,
               cpu(lambda: O.conv2d_grad_sample(cx, cb, kernel_size=(3, 3), padding=(1, 1), stride=(1, 1), dilation=(1, 1), groups=1),
                   16, "16 of 256 samples, unfold + einsum"))
+    yield row("conv2d_gs (norm only)", "a3", "C4 n=256 64->64 3x3 32x32 f32, gradient not stored",
+              timed(lambda: K.conv2d_grad_sample(x, b, (3, 3), (1, 1), (1, 1, 1, 1), (1, 1), 1, norm_only=True)), "mfma_fp32",
+              2.0 * n * 64 * 576 * 1024)
+    x16, b16 = x.bfloat16(), b.bfloat16()
+    yield row("conv2d_gs (bf16 MFMA)", "a3", "C4 shape in bf16: n=256 64->64 3x3 32x32",
+              timed(lambda: K.conv2d_grad_sample(x16, b16, (3, 3), (1, 1), (1, 1, 1, 1), (1, 1), 1)), "mfma_bf16",
+              2.0 * n * 64 * 576 * 1024)
+    x16, b16 = torch.randn(64, 128, 28, 28, device=dev).bfloat16(), torch.randn(64, 128, 28, 28, device=dev).bfloat16()
+    yield row("conv2d_gs (bf16 MFMA)", "a3", "n=64 128->128 3x3 28x28 bf16",
+              timed(lambda: K.conv2d_grad_sample(x16, b16, (3, 3), (1, 1), (1, 1, 1, 1), (1, 1), 1)), "mfma_bf16",
+              2.0 * 64 * 128 * 1152 * 784)
+    del x16, b16
     yield row("group_norm_gs", "a6", "C4 n=256 C=64 G=32 32x32 f32", timed(lambda: K.group_norm_grad_sample(x, b, 32, 1e-5)),
               "hbm", 2 * x.numel() * 4, cpu(lambda: O.group_norm_grad_sample(cx, cb, 32, 1e-5), 16, "16 of 256 samples"))
     yield row("conv_bias_gs", "a3", "C4 n=256 O=64 32x32 f32", timed(lambda: K.conv_bias_grad_sample(b)), "hbm", b.numel() * 4)
