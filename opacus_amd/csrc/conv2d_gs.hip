@@ -229,7 +229,13 @@ template <> __device__ __forceinline__ float buffer_load1<bf16_t>(__amdgpu_buffe
 constexpr int kPatchDepth = 4;                        // backprop k-tiles in flight per lane
 constexpr int kPatchTrip = kPatchDepth * mf32::BK;    // k extent of one trip of the k loop
 
-template <int BM, int BN, typename TIN, typename TOUT, bool VEC>
+// ROWK: the eight positions a half-wave takes of a k-tile lie in one output row at unit stride
+// (stride 1 along the row, output width a multiple of 8), so their patch cells are consecutive:
+// one table read and one address per half and k-tile, the eight LDS reads at immediate offsets.
+// Every vector instruction issued between the MFMAs of a wave costs MFMA time on this device
+// (measured: 4 independent VALU instructions per 64-cycle fp32 MFMA stretch a loop by 23 % with
+// three waves per SIMD), so the k loop keeps its address arithmetic to a minimum.
+template <int BM, int BN, typename TIN, typename TOUT, bool VEC, bool ROWK>
 __global__ __launch_bounds__(kThreads) void conv2d_gs_patch_kernel(
     const TIN* __restrict__ x, const TIN* __restrict__ b, TOUT* __restrict__ gs,
     float* __restrict__ partials, ConvGeom g, int C, int O, int groups, float scale, int tiles_m,
@@ -375,22 +381,25 @@ __global__ __launch_bounds__(kThreads) void conv2d_gs_patch_kernel(
   const __amdgpu_buffer_rsrc_t brs = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<TIN*>(bg), 0, Og * g.Q * static_cast<int>(sizeof(TIN)), 0x00020000);
   constexpr uint32_t kOutside = 0x7fffffffu;
-  int row_el[Tile::TM];  // element offset of (row, k = 8 kk), or -1 for a row outside
+  uint32_t row_off[Tile::TM];  // byte offset of (row, k = 8 kk), or past the end for a row outside
 #pragma unroll
   for (int i = 0; i < Tile::TM; ++i) {
     const int m = m0 + wm0 + i * 32 + l32;
-    row_el[i] = m < Og ? m * g.Q + kk * K2 : -1;
+    row_off[i] = m < Og ? static_cast<uint32_t>(m * g.Q + kk * K2) * static_cast<uint32_t>(sizeof(TIN)) : kOutside;
   }
   auto fetch = [&](int kt, float (&a)[Tile::TM][K2]) {
     const int k = kt * mf32::BK + kk * K2;
+    const bool tail = (kt + 1) * mf32::BK > g.Q;  // uniform: only the last tiles compare positions
 #pragma unroll
     for (int i = 0; i < Tile::TM; ++i) {
       if (VEC) {
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-          const bool in = row_el[i] >= 0 && k + 4 * h < g.Q;
-          const uint32_t off =
-              in ? static_cast<uint32_t>(row_el[i] + kt * mf32::BK + 4 * h) * sizeof(TIN) : kOutside;
+          uint32_t off = row_off[i] + static_cast<uint32_t>(kt * mf32::BK + 4 * h) * static_cast<uint32_t>(sizeof(TIN));
+          if (tail) {
+            asm volatile("" ::: "memory");  // a branch, not a select: the steady loop skips the compare
+            if (k + 4 * h >= g.Q) off = kOutside;
+          }
           const float4 v = buffer_load4<TIN>(brs, off);
           a[i][4 * h + 0] = v.x;
           a[i][4 * h + 1] = v.y;
@@ -400,26 +409,39 @@ __global__ __launch_bounds__(kThreads) void conv2d_gs_patch_kernel(
       } else {
 #pragma unroll
         for (int e = 0; e < K2; ++e) {
-          const bool in = row_el[i] >= 0 && k + e < g.Q;
-          const uint32_t off = in ? static_cast<uint32_t>(row_el[i] + kt * mf32::BK + e) * sizeof(TIN) : kOutside;
+          uint32_t off = row_off[i] + static_cast<uint32_t>(kt * mf32::BK + e) * static_cast<uint32_t>(sizeof(TIN));
+          if (tail) {
+            asm volatile("" ::: "memory");
+            if (k + e >= g.Q) off = kOutside;
+          }
           a[i][e] = buffer_load1<TIN>(brs, off);
         }
       }
     }
   };
+  constexpr int NQ = ROWK ? 1 : K2;  // table entries a half-wave needs per k-tile
   float av[D][Tile::TM][K2], bv[2][K2][Tile::TN];
-  int qo[2][K2];
+  int qo[2][NQ];
   const int nk = Qpad / mf32::BK;  // a multiple of D
-  auto read_q = [&](int kt, int (&q)[K2]) {
+  auto read_q = [&](int kt, int (&q)[NQ]) {
     const int* qt = qtab + (kt < nk ? kt : 0) * mf32::BK + kk * K2;  // past the end: any valid entries
 #pragma unroll
-    for (int k2 = 0; k2 < K2; ++k2) q[k2] = qt[k2];
+    for (int k2 = 0; k2 < NQ; ++k2) q[k2] = qt[k2];
   };
-  auto read_b = [&](const int (&q)[K2], float (&bb)[K2][Tile::TN]) {
+  auto read_b = [&](const int (&q)[NQ], float (&bb)[K2][Tile::TN]) {
+    if constexpr (ROWK) {
 #pragma unroll
-    for (int k2 = 0; k2 < K2; ++k2)
+      for (int j = 0; j < Tile::TN; ++j) {
+        const float* cells = xs + (base_p[j] + q[0]);
 #pragma unroll
-      for (int j = 0; j < Tile::TN; ++j) bb[k2][j] = xs[base_p[j] + q[k2]];
+        for (int k2 = 0; k2 < K2; ++k2) bb[k2][j] = cells[k2];
+      }
+    } else {
+#pragma unroll
+      for (int k2 = 0; k2 < K2; ++k2)
+#pragma unroll
+        for (int j = 0; j < Tile::TN; ++j) bb[k2][j] = xs[base_p[j] + q[k2]];
+    }
   };
   Tile tile;
   tile.clear();
@@ -876,6 +898,8 @@ void launch(const Plan& p, bool vec, const void* x, const void* b, void* gs, flo
   TOUT* gp = static_cast<TOUT*>(gs);
   bool use_patch = patch_bytes > 0;
   constexpr bool kIn16 = std::is_same<TIN, bf16_t>::value;
+  // eight consecutive positions of a k-tile half lie in one output row at unit stride
+  const bool rowk = g.sw == 1 && g.OW % 8 == 0;
   if (patch_bytes > 64 * 1024 - 64) {
     // per device and cheap: said again at every such launch rather than remembered. A device
     // or runtime that refuses that much LDS gets the gather kernel on the same 64 x 64 plan.
@@ -889,8 +913,9 @@ void launch(const Plan& p, bool vec, const void* x, const void* b, void* gs, flo
                  : reinterpret_cast<const void*>(&conv2d_gs_patch16_kernel<64, 64, TOUT, false>);
     }
     else
-      fn = vec ? reinterpret_cast<const void*>(&conv2d_gs_patch_kernel<64, 64, TIN, TOUT, true>)
-               : reinterpret_cast<const void*>(&conv2d_gs_patch_kernel<64, 64, TIN, TOUT, false>);
+      fn = vec ? (rowk ? reinterpret_cast<const void*>(&conv2d_gs_patch_kernel<64, 64, TIN, TOUT, true, true>)
+                       : reinterpret_cast<const void*>(&conv2d_gs_patch_kernel<64, 64, TIN, TOUT, true, false>))
+               : reinterpret_cast<const void*>(&conv2d_gs_patch_kernel<64, 64, TIN, TOUT, false, false>);
     if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kPatchLdsLimit)) !=
         hipSuccess) {
       (void)hipGetLastError();  // the refusal is handled here, not reported by the next launch check
@@ -913,12 +938,13 @@ void launch(const Plan& p, bool vec, const void* x, const void* b, void* gs, flo
       }
 #undef DPK_P16_LAUNCH
     } else {
-      if (vec)
-        hipLaunchKernelGGL((conv2d_gs_patch_kernel<64, 64, TIN, TOUT, true>), grid, block, patch_bytes, s, xp,
-                           bp, gp, partials, g, C, O, groups, scale, p.tiles_m, p.tiles_n, pd, xvec, 0);
-      else
-        hipLaunchKernelGGL((conv2d_gs_patch_kernel<64, 64, TIN, TOUT, false>), grid, block, patch_bytes, s,
-                           xp, bp, gp, partials, g, C, O, groups, scale, p.tiles_m, p.tiles_n, pd, xvec, 0);
+#define DPK_P32_LAUNCH(V, RK)                                                                              \
+  hipLaunchKernelGGL((conv2d_gs_patch_kernel<64, 64, TIN, TOUT, V, RK>), grid, block, patch_bytes, s, xp, bp, \
+                     gp, partials, g, C, O, groups, scale, p.tiles_m, p.tiles_n, pd, xvec, 0)
+      if (vec && rowk) DPK_P32_LAUNCH(true, true);
+      else if (vec) DPK_P32_LAUNCH(true, false);
+      else DPK_P32_LAUNCH(false, false);
+#undef DPK_P32_LAUNCH
     }
     return;
   }
