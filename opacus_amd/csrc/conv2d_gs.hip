@@ -229,13 +229,14 @@ template <> __device__ __forceinline__ float buffer_load1<bf16_t>(__amdgpu_buffe
 constexpr int kPatchDepth = 4;                        // backprop k-tiles in flight per lane
 constexpr int kPatchTrip = kPatchDepth * mf32::BK;    // k extent of one trip of the k loop
 
-// ROWK: the eight positions a half-wave takes of a k-tile lie in one output row at unit stride
-// (stride 1 along the row, output width a multiple of 8), so their patch cells are consecutive:
-// one table read and one address per half and k-tile, the eight LDS reads at immediate offsets.
+// RK (8, 4 or 0): the eight positions a half-wave takes of a k-tile fall into aligned runs of RK
+// positions that lie in one output row at unit stride (stride 1 along the row, output width a
+// multiple of RK), so a run's patch cells are consecutive: one table read and one address per
+// run, the LDS reads at immediate offsets. 0: every position has its own table entry.
 // Every vector instruction issued between the MFMAs of a wave costs MFMA time on this device
 // (measured: 4 independent VALU instructions per 64-cycle fp32 MFMA stretch a loop by 23 % with
 // three waves per SIMD), so the k loop keeps its address arithmetic to a minimum.
-template <int BM, int BN, typename TIN, typename TOUT, bool VEC, bool ROWK>
+template <int BM, int BN, typename TIN, typename TOUT, bool VEC, int RK>
 __global__ __launch_bounds__(kThreads) void conv2d_gs_patch_kernel(
     const TIN* __restrict__ x, const TIN* __restrict__ b, TOUT* __restrict__ gs,
     float* __restrict__ partials, ConvGeom g, int C, int O, int groups, float scale, int tiles_m,
@@ -419,23 +420,26 @@ __global__ __launch_bounds__(kThreads) void conv2d_gs_patch_kernel(
       }
     }
   };
-  constexpr int NQ = ROWK ? 1 : K2;  // table entries a half-wave needs per k-tile
+  constexpr int RUN = RK ? RK : 1;   // positions per table entry
+  constexpr int NQ = K2 / RUN;       // table entries a half-wave needs per k-tile
   float av[D][Tile::TM][K2], bv[2][K2][Tile::TN];
   int qo[2][NQ];
   const int nk = Qpad / mf32::BK;  // a multiple of D
   auto read_q = [&](int kt, int (&q)[NQ]) {
     const int* qt = qtab + (kt < nk ? kt : 0) * mf32::BK + kk * K2;  // past the end: any valid entries
 #pragma unroll
-    for (int k2 = 0; k2 < NQ; ++k2) q[k2] = qt[k2];
+    for (int k2 = 0; k2 < NQ; ++k2) q[k2] = qt[k2 * RUN];
   };
   auto read_b = [&](const int (&q)[NQ], float (&bb)[K2][Tile::TN]) {
-    if constexpr (ROWK) {
+    if constexpr (RK != 0) {
 #pragma unroll
-      for (int j = 0; j < Tile::TN; ++j) {
-        const float* cells = xs + (base_p[j] + q[0]);
+      for (int j = 0; j < Tile::TN; ++j)
 #pragma unroll
-        for (int k2 = 0; k2 < K2; ++k2) bb[k2][j] = cells[k2];
-      }
+        for (int r = 0; r < NQ; ++r) {
+          const float* cells = xs + (base_p[j] + q[r]);
+#pragma unroll
+          for (int e = 0; e < RUN; ++e) bb[r * RUN + e][j] = cells[e];
+        }
     } else {
 #pragma unroll
       for (int k2 = 0; k2 < K2; ++k2)
@@ -506,7 +510,9 @@ static_assert(kP16TripK == kPatchTrip, "both patch kernels pad the offset table 
 constexpr int kP16RowBytes = kP16TripK * 2 + 16;
 constexpr size_t p16_stage_bytes(int bm) { return static_cast<size_t>(2) * bm * kP16RowBytes; }
 
-template <int BM, int BN, typename TOUT, bool VEC>
+// RK as in the fp32 patch kernel: a half-wave's eight positions of a k-tile come as aligned runs
+// of RK consecutive cells of the patch (8, 4, or 0 for no such structure).
+template <int BM, int BN, typename TOUT, bool VEC, int RK>
 __global__ __launch_bounds__(kThreads) void conv2d_gs_patch16_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ b, TOUT* __restrict__ gs,
     float* __restrict__ partials, ConvGeom g, int C, int O, int groups, float scale, int tiles_m,
@@ -652,28 +658,56 @@ __global__ __launch_bounds__(kThreads) void conv2d_gs_patch16_kernel(
 
   uint32_t ga[2][kRowPasses][8];  // a trip's share of this thread, as loaded
   uint32_t bv[2][kP16Tiles][Tile::TN][4];
-  int qo[kP16Tiles][8];
+  constexpr int RUN = RK ? RK : 1;  // positions per table entry
+  constexpr int NQ = 8 / RUN;       // table entries a half-wave needs per k-tile
+  int qo[kP16Tiles][NQ];
   auto load_q = [&](int trip) {
     trip = trip < ntrips ? trip : ntrips - 1;
 #pragma unroll
     for (int t = 0; t < kP16Tiles; ++t) {
-      const int4* qt = reinterpret_cast<const int4*>(qtab + (trip * kP16Tiles + t) * kP16BK + kk * 8);
-      const int4 lo = qt[0], hi = qt[1];
-      qo[t][0] = lo.x; qo[t][1] = lo.y; qo[t][2] = lo.z; qo[t][3] = lo.w;
-      qo[t][4] = hi.x; qo[t][5] = hi.y; qo[t][6] = hi.z; qo[t][7] = hi.w;
+      const int* q8 = qtab + (trip * kP16Tiles + t) * kP16BK + kk * 8;
+      if constexpr (RK != 0) {
+#pragma unroll
+        for (int r = 0; r < NQ; ++r) qo[t][r] = q8[r * RUN];
+      } else {
+        const int4 lo = reinterpret_cast<const int4*>(q8)[0], hi = reinterpret_cast<const int4*>(q8)[1];
+        qo[t][0] = lo.x; qo[t][1] = lo.y; qo[t][2] = lo.z; qo[t][3] = lo.w;
+        qo[t][4] = hi.x; qo[t][5] = hi.y; qo[t][6] = hi.z; qo[t][7] = hi.w;
+      }
     }
   };
+  typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
   auto load_b = [&](uint32_t (&bb)[kP16Tiles][Tile::TN][4]) {
 #pragma unroll
     for (int t = 0; t < kP16Tiles; ++t)
 #pragma unroll
-      for (int j = 0; j < Tile::TN; ++j)
+      for (int j = 0; j < Tile::TN; ++j) {
+        if constexpr (RK != 0) {
+          // RK consecutive 2-byte cells from a 2-byte aligned address: the aligned words around
+          // them, shifted into place per lane (a wide read at 2-byte alignment, which the
+          // compiler would make of the 2-byte reads, is several times slower on this device)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const uint32_t lo = *reinterpret_cast<const uint16_t*>(xsb + base_p[j] + qo[t][2 * e]);
-          const uint32_t hi = *reinterpret_cast<const uint16_t*>(xsb + base_p[j] + qo[t][2 * e + 1]);
-          bb[t][j][e] = lo | (hi << 16);
+          for (int r = 0; r < NQ; ++r) {
+            const uint32_t at = static_cast<uint32_t>(base_p[j] + qo[t][r]);
+            const uint32_t* w = reinterpret_cast<const uint32_t*>(xsb + (at & ~3u));
+            const uint32_t shift = at & 2u;  // bytes
+            uint32_t word[RUN / 2 + 1];
+#pragma unroll
+            for (int e = 0; e <= RUN / 2; ++e) word[e] = w[e];
+#pragma unroll
+            for (int e = 0; e < RUN / 2; ++e)
+              bb[t][j][r * (RUN / 2) + e] = __builtin_amdgcn_alignbyte(word[e + 1], word[e], shift);
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            u16x2 pr;
+            pr.x = *reinterpret_cast<const uint16_t*>(xsb + base_p[j] + qo[t][2 * e]);
+            pr.y = *reinterpret_cast<const uint16_t*>(xsb + base_p[j] + qo[t][2 * e + 1]);
+            bb[t][j][e] = __builtin_bit_cast(uint32_t, pr);
+          }
         }
+      }
   };
   // global -> registers: 16 k (32 bytes) of each of this thread's rows
   auto load_a = [&](int trip, uint32_t (&aa)[kRowPasses][8]) {
@@ -888,65 +922,68 @@ Plan make_plan(int64_t Og, int64_t Pg, bool small = false) {
   return p;
 }
 
+// One variant of the patch kernels (vector loads of the backprops or not, run length of
+// consecutive cells). Above 64 KB of LDS the kernel must be told so: per device and cheap, so it is
+// said again at every such launch rather than remembered; false if that is refused.
+template <typename TIN, typename TOUT, bool V, int RK>
+bool launch_patch(const Plan& p, dim3 grid, dim3 block, size_t patch_bytes, hipStream_t s, const TIN* xp,
+                  const TIN* bp, TOUT* gp, float* partials, const ConvGeom& g, int C, int O, int groups,
+                  float scale, PatchDims pd, int xvec, int a_off) {
+  auto prepare = [&](const void* fn) {
+    if (patch_bytes <= 64 * 1024 - 64) return true;
+    if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kPatchLdsLimit)) ==
+        hipSuccess)
+      return true;
+    (void)hipGetLastError();  // the refusal is handled here, not reported by the next launch check
+    return false;
+  };
+  if constexpr (std::is_same<TIN, bf16_t>::value) {
+    if (p.bm == 128) {
+      if (!prepare(reinterpret_cast<const void*>(&conv2d_gs_patch16_kernel<128, 64, TOUT, V, RK>))) return false;
+      hipLaunchKernelGGL((conv2d_gs_patch16_kernel<128, 64, TOUT, V, RK>), grid, block, patch_bytes, s, xp, bp, gp,
+                         partials, g, C, O, groups, scale, p.tiles_m, p.tiles_n, pd, xvec, a_off);
+    } else {
+      if (!prepare(reinterpret_cast<const void*>(&conv2d_gs_patch16_kernel<64, 64, TOUT, V, RK>))) return false;
+      hipLaunchKernelGGL((conv2d_gs_patch16_kernel<64, 64, TOUT, V, RK>), grid, block, patch_bytes, s, xp, bp, gp,
+                         partials, g, C, O, groups, scale, p.tiles_m, p.tiles_n, pd, xvec, a_off);
+    }
+  } else {
+    if (!prepare(reinterpret_cast<const void*>(&conv2d_gs_patch_kernel<64, 64, TIN, TOUT, V, RK>))) return false;
+    hipLaunchKernelGGL((conv2d_gs_patch_kernel<64, 64, TIN, TOUT, V, RK>), grid, block, patch_bytes, s, xp, bp, gp,
+                       partials, g, C, O, groups, scale, p.tiles_m, p.tiles_n, pd, xvec, 0);
+  }
+  return true;
+}
+
+// (the plan comes back as the kernel that ran used it: a refused patch launch falls back to 64 x 64 tiles)
 template <typename TIN, typename TOUT>
-void launch(const Plan& p, bool vec, const void* x, const void* b, void* gs, float* partials,
+void launch(Plan& p, bool vec, const void* x, const void* b, void* gs, float* partials,
             const ConvGeom& g, int64_t n, int C, int O, int groups, float scale, hipStream_t s,
             size_t patch_bytes, PatchDims pd, int a_off, int ksplit, int kchunk, float* split_out) {
-  const dim3 grid(static_cast<unsigned>(n * groups * p.tiles_m * p.tiles_n * ksplit)), block(kThreads);
+  dim3 grid(static_cast<unsigned>(n * groups * p.tiles_m * p.tiles_n * ksplit)), block(kThreads);
   const TIN* xp = static_cast<const TIN*>(x);
   const TIN* bp = static_cast<const TIN*>(b);
   TOUT* gp = static_cast<TOUT*>(gs);
-  bool use_patch = patch_bytes > 0;
-  constexpr bool kIn16 = std::is_same<TIN, bf16_t>::value;
-  // eight consecutive positions of a k-tile half lie in one output row at unit stride
-  const bool rowk = g.sw == 1 && g.OW % 8 == 0;
-  if (patch_bytes > 64 * 1024 - 64) {
-    // per device and cheap: said again at every such launch rather than remembered. A device
-    // or runtime that refuses that much LDS gets the gather kernel on the same 64 x 64 plan.
-    const void* fn;
-    if constexpr (kIn16) {
-      if (p.bm == 128)
-        fn = vec ? reinterpret_cast<const void*>(&conv2d_gs_patch16_kernel<128, 64, TOUT, true>)
-                 : reinterpret_cast<const void*>(&conv2d_gs_patch16_kernel<128, 64, TOUT, false>);
-      else
-        fn = vec ? reinterpret_cast<const void*>(&conv2d_gs_patch16_kernel<64, 64, TOUT, true>)
-                 : reinterpret_cast<const void*>(&conv2d_gs_patch16_kernel<64, 64, TOUT, false>);
-    }
-    else
-      fn = vec ? (rowk ? reinterpret_cast<const void*>(&conv2d_gs_patch_kernel<64, 64, TIN, TOUT, true, true>)
-                       : reinterpret_cast<const void*>(&conv2d_gs_patch_kernel<64, 64, TIN, TOUT, true, false>))
-               : reinterpret_cast<const void*>(&conv2d_gs_patch_kernel<64, 64, TIN, TOUT, false, false>);
-    if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kPatchLdsLimit)) !=
-        hipSuccess) {
-      (void)hipGetLastError();  // the refusal is handled here, not reported by the next launch check
-      use_patch = false;
-    }
-  }
-  if (use_patch) {
+  if (patch_bytes > 0) {
+    // aligned runs of this many positions lie in one output row at unit stride
+    const int run = g.sw != 1 ? 0 : g.OW % 8 == 0 ? 8 : g.OW % 4 == 0 ? 4 : 0;
     // image rows made of whole, aligned 4-element chunks: the patch interior is staged with vector loads
     const int xvec = (g.W % 4 == 0 && dpk_aligned(x, sizeof(TIN) == 2 ? 8 : 16)) ? 1 : 0;
-    if constexpr (kIn16) {
-#define DPK_P16_LAUNCH(BM_, V)                                                                          \
-  hipLaunchKernelGGL((conv2d_gs_patch16_kernel<BM_, 64, TOUT, V>), grid, block, patch_bytes, s, xp, bp, \
-                     gp, partials, g, C, O, groups, scale, p.tiles_m, p.tiles_n, pd, xvec, a_off)
-      if (p.bm == 128) {
-        if (vec) DPK_P16_LAUNCH(128, true);
-        else DPK_P16_LAUNCH(128, false);
-      } else {
-        if (vec) DPK_P16_LAUNCH(64, true);
-        else DPK_P16_LAUNCH(64, false);
-      }
-#undef DPK_P16_LAUNCH
-    } else {
-#define DPK_P32_LAUNCH(V, RK)                                                                              \
-  hipLaunchKernelGGL((conv2d_gs_patch_kernel<64, 64, TIN, TOUT, V, RK>), grid, block, patch_bytes, s, xp, bp, \
-                     gp, partials, g, C, O, groups, scale, p.tiles_m, p.tiles_n, pd, xvec, 0)
-      if (vec && rowk) DPK_P32_LAUNCH(true, true);
-      else if (vec) DPK_P32_LAUNCH(true, false);
-      else DPK_P32_LAUNCH(false, false);
-#undef DPK_P32_LAUNCH
-    }
-    return;
+    bool done;
+#define DPK_PATCH(V, RK)                                                                                  \
+  done = launch_patch<TIN, TOUT, V, RK>(p, grid, block, patch_bytes, s, xp, bp, gp, partials, g, C, O, groups, \
+                                        scale, pd, xvec, a_off)
+    if (vec && run == 8) DPK_PATCH(true, 8);
+    else if (vec && run == 4) DPK_PATCH(true, 4);
+    else if (vec) DPK_PATCH(true, 0);
+    else DPK_PATCH(false, 0);
+#undef DPK_PATCH
+    if (done) return;
+    // refused (more LDS than the device or runtime grants): the gather kernel on 64 x 64 tiles
+    p.bm = p.bn = 64;
+    p.tiles_m = static_cast<int>(dpk_cdiv(O / groups, 64));
+    p.tiles_n = static_cast<int>(dpk_cdiv(g.Pg, 64));
+    grid = dim3(static_cast<unsigned>(n * groups * p.tiles_m * p.tiles_n * ksplit));
   }
 #define DPK_CONV_LAUNCH(BM, BN, V, D3)                                                            \
   hipLaunchKernelGGL((conv2d_gs_kernel<BM, BN, TIN, TOUT, V, D3>), grid, block, 0, s, xp, bp, gp, \
@@ -1094,7 +1131,8 @@ int conv_gs(const char* who, const void* x, const void* b, int in_dtype, void* g
   float* partials = nullptr;
   float* split_out = nullptr;
   if (sumsq) {
-    const size_t need = ksplit > 1 ? wl.total : static_cast<size_t>(blocks) * sizeof(float);
+    // room for the plan with the most blocks: a refused patch launch falls back to it
+    const size_t need = ksplit > 1 ? wl.total : wl.partials_bytes;
     DPK_REQUIRE(ws && ws_bytes >= need, DPK_E_WORKSPACE, "%s: workspace %zu < %zu bytes", who,
                 ws_bytes, need);
     DPK_REQUIRE(dpk_aligned(ws, 4), DPK_E_ALIGN, "%s: workspace misaligned", who);
