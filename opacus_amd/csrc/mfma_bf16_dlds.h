@@ -173,6 +173,16 @@ struct Tile {
     constexpr bool kF32 = std::is_same<T, float>::value;
     typedef typename std::conditional<kF32, floatx4, bf16x8>::type frag_t;  // 16 bytes either way
     frag_t av[KS][2], bv[KS][2];
+    // bf16: the next tile's loads go out before anything else of this tile. A tile's MFMAs are
+    // 512 cycles of the pipe; loads issued in their shadow, a few per k step, left the last of
+    // them a stage's wait at the next barrier (waves stalled half their cycles; 2048 -> 32000:
+    // 835 -> 728 us with the loads first). fp32 tiles take four times as long to multiply and
+    // run 6 % faster with the loads dealt out between the steps.
+    constexpr bool kLoadsFirst = !kF32;
+    if constexpr (kLoadsFirst) {
+#pragma unroll
+      for (int q = 0; q < NLOADS; ++q) issue(q);
+    }
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
@@ -207,8 +217,10 @@ struct Tile {
           for (int j = 0; j < 2; ++j)
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[ks][i], bv[ks][j], acc[i][j], 0, 0, 0);
       }
+      if constexpr (!kLoadsFirst) {
 #pragma unroll
-      for (int q = ks * PER_STEP; q < (ks + 1) * PER_STEP && q < NLOADS; ++q) issue(q);
+        for (int q = ks * PER_STEP; q < (ks + 1) * PER_STEP && q < NLOADS; ++q) issue(q);
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
   }
