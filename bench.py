@@ -232,7 +232,11 @@ def workload_c1(dev, autograd_weight_grads=False):
         dev, SmallCNN(), torch.randn(n, 1, 28, 28), torch.randint(0, 10, (n,)), n, 1.1,
         "Small CNN (conv 1->16 k8 s2 p3, conv 16->32 k4 s2, fc 512->32, fc 32->10) fp32, batch 256, hooks, C=1, sigma=1.1",
         dict(kernel="clip_accumulate_kernel<float,float,*,RS=16> (8 tensors, one launch)", timer="clip_accumulate",
-             bound="hbm", work_per_launch=float(n * P * 4 + P * 4), unit="GB/s", peak=HBM_PEAK_GBS, traffic=None),
+             bound="hbm", work_per_launch=float(n * P * 4 + P * 4), unit="GB/s", peak=HBM_PEAK_GBS,
+             # scaled with the copy kernel's factor (FETCH_SIZE x 2.000); this kernel's short row pieces may be
+             # fetched in requests the counter sizes correctly, in which case the true figure is half
+             traffic=53396279,
+             traffic_source="recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of bench.py --workload c1, profiles/clip_accumulate_small_cnn_b256_hbm_traffic.txt (not re-measured by this run)"),
         autograd_weight_grads=autograd_weight_grads,
     )
 
@@ -245,12 +249,15 @@ def workload_c4(dev, autograd_weight_grads=False):
         dev, ResBlock(), torch.randn(n, 64, 32, 32), torch.randint(0, 10, (n,)), n, 1.0,
         "ResNet basic block: 2 x Conv2d(64->64, 3x3, p1) + GroupNorm(32), 32x32 images, fp32, batch 256, hooks, C=1, sigma=1",
         dict(kernel="conv2d_gs_patch_kernel<64,64,float,float>", timer="conv2d_gs", bound="mfma",
-             work_per_launch=flops, unit="TFLOP/s", peak=MFMA_FP32_PEAK_TFLOPS, traffic=None),
+             work_per_launch=flops, unit="TFLOP/s", peak=MFMA_FP32_PEAK_TFLOPS,
+             # inputs 134.2 MB + per-sample gradients 37.7 MB = 172.0 MB must move once
+             traffic=174255653,
+             traffic_source="recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of bench.py --workload c4, profiles/conv2d_gs_resblock_b256_hbm_traffic.txt (not re-measured by this run)"),
         autograd_weight_grads=autograd_weight_grads,
     )
 
 
-def _ghost_workload(dev, net, make_inputs, loss_call, n, T, sigma, desc, single=True):
+def _ghost_workload(dev, net, make_inputs, loss_call, n, T, sigma, desc, single=True, traffic=None, traffic_source=None):
     from opacus_amd import GradSampleModuleFastGradientClipping
     from opacus_amd.optimizers import DPOptimizerFastGradientClipping
 
@@ -273,7 +280,7 @@ def _ghost_workload(dev, net, make_inputs, loss_call, n, T, sigma, desc, single=
         roofline=dict(kernel="ghost_norm_multi_kernel<128x128, 2 stages> (all Linear layers of a step pooled into one launch; thin layers by linear_dlds_kernel; "
                              "ghost_norm_bf16_dlds_kernel layer by layer with two backward passes)",
                       timer="linear_ghost_norm", bound="mfma", work_per_step=flops, unit="TFLOP/s",
-                      peak=MFMA_BF16_PEAK_TFLOPS, traffic=None),
+                      peak=MFMA_BF16_PEAK_TFLOPS, traffic=traffic, **({"traffic_source": traffic_source} if traffic else {})),
     )
 
 
@@ -294,6 +301,9 @@ def workload_c3(dev, single=True):
         dev, net, lambda: torch.randn(n, T, 1024).to(dev).bfloat16(), loss_call, n, T, 1.0,
         "MLP Linear(1024->4096) GELU Linear(4096->1024), bf16, batch 32, T=512, ghost clipping, C=1, sigma=1",
         single=single,
+        # HBM bytes of the pooled launch (operands of both layers: 335.5 MB must be read once)
+        traffic=368253058 if single else None,
+        traffic_source="recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of bench.py --workload c3, profiles/ghost_norm_multi_mlp_b32_t512_hbm_traffic.txt (not re-measured by this run)",
     )
 
 
@@ -316,6 +326,12 @@ def workload_c5(dev, tied=False, single=True):
         f"4-layer Llama-style decoder (d 2048, 16 heads / 4 KV, SwiGLU 5632, vocab 32000, {'tied' if tied else 'untied'}), "
         "bf16, batch 16, seq 1024, ghost clipping, C=1, sigma=0.8",
         single=single,
+        # HBM bytes of the pooled launch (21 layers by the Gram route; their operands, 5.21 GB, must be
+        # read once; a unit streams two 128-row blocks of both operands and the 4 MB L2 of an XCD does not
+        # hold a sample's rows of the wide layers, so the units re-fetch from the last-level cache)
+        traffic=12053288261 if single and not tied else None,
+        traffic_source="recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of bench.py --workload c5, "
+                       "profiles/ghost_norm_multi_llama_b16_t1024_hbm_traffic.txt (not re-measured by this run)",
     )
 
 
