@@ -555,6 +555,11 @@ def test_conv2d_grad_sample_bf16(K, case, out_f32):
     # exact products of bf16 inputs, fp32 accumulation: only a bf16 output rounds
     assert_rel(gs, want_w, FP32_REL if out_f32 else BF16_REL, "conv weight bf16")
     assert_rel(sumsq, want_w.flatten(1).pow(2).sum(1), 2e-5, "conv sumsq bf16")
+    # the same launch without storing the gradient
+    none, sumsq_only = K.conv2d_grad_sample(dev(x), dev(b), case["k"], case["stride"], pad, case["dilation"], case["groups"],
+                                            scale=0.5, norm_only=True)
+    assert none is None
+    assert_rel(sumsq_only, want_w.flatten(1).pow(2).sum(1), 2e-5, "conv sumsq bf16, norm only")
     # backprops that start 2 bytes off a 16-byte boundary take the element-wise loads
     odd = torch.empty(b.numel() + 1, dtype=torch.bfloat16, device="cuda")[1:].view(b.shape).copy_(b)
     gs2, _ = K.conv2d_grad_sample(dev(x), odd, case["k"], case["stride"], pad, case["dilation"], case["groups"], scale=0.5,
