@@ -447,6 +447,28 @@ def test_linear_ghost_norm_multi_matches_layer_by_layer(K, dtype, n, layers):
             assert_rel(got, single, FP32_REL, f"{what} norm of layer {lay} against its own launch")
 
 
+@pytest.mark.parametrize("count", [40, 300])
+def test_linear_ghost_norm_multi_many_layers(K, count):
+    """More layers than one pooled launch takes (32) and more than one call's table (256)."""
+    torch.manual_seed(count)
+    n, T = 2, 128
+    items, wants = [], []
+    for k in range(count):
+        fin, fout = (64, 128) if k % 3 else (128, 64)
+        a = torch.randn(n, T, fin).bfloat16()
+        b = (torch.randn(n, T, fout) * 0.1).bfloat16()
+        ow, ob = O.linear_norm_sample(a.double(), b.double())
+        nw = torch.full((n,), float("nan"), device="cuda")
+        nb = torch.full((n,), float("nan"), device="cuda") if k % 2 else None
+        items.append((dev(b), dev(a), 1.0, nw, nb))
+        wants.append((ow, ob if k % 2 else None))
+    K.linear_ghost_norm_multi(items)
+    for k, ((_, _, _, nw, nb), (ow, ob)) in enumerate(zip(items, wants)):
+        assert_rel(nw, ow, 1e-4, f"weight norm of layer {k}")
+        if ob is not None:
+            assert_rel(nb, ob, 1e-4, f"bias norm of layer {k}")
+
+
 def test_linear_ghost_norm_2d_inputs(K):
     torch.manual_seed(21)
     a, b = torch.randn(6, 50), torch.randn(6, 30)
