@@ -203,31 +203,138 @@ __global__ __launch_bounds__(kThreads) void conv_split_reduce_kernel(const float
 // take; here the k loop is MFMAs, LDS reads of the patch and register loads of the
 // backprops.
 // 4 consecutive elements / one element at a byte offset of a buffer descriptor (zeros past
-// its end)
+// its end); the fp32 patch kernel serves fp32 input only (bf16 input has its own kernel)
 template <typename T> __device__ __forceinline__ float4 buffer_load4(__amdgpu_buffer_rsrc_t r, uint32_t off);
 template <> __device__ __forceinline__ float4 buffer_load4<float>(__amdgpu_buffer_rsrc_t r, uint32_t off) {
   typedef int vi4 __attribute__((ext_vector_type(4)));
   const vi4 v = __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0);
   return make_float4(__int_as_float(v.x), __int_as_float(v.y), __int_as_float(v.z), __int_as_float(v.w));
 }
-template <> __device__ __forceinline__ float4 buffer_load4<bf16_t>(__amdgpu_buffer_rsrc_t r, uint32_t off) {
-  typedef int vi2 __attribute__((ext_vector_type(2)));
-  const vi2 v = __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 0);
-  return make_float4(__uint_as_float(static_cast<uint32_t>(v.x) << 16),
-                     __uint_as_float(static_cast<uint32_t>(v.x) & 0xffff0000u),
-                     __uint_as_float(static_cast<uint32_t>(v.y) << 16),
-                     __uint_as_float(static_cast<uint32_t>(v.y) & 0xffff0000u));
-}
 template <typename T> __device__ __forceinline__ float buffer_load1(__amdgpu_buffer_rsrc_t r, uint32_t off);
 template <> __device__ __forceinline__ float buffer_load1<float>(__amdgpu_buffer_rsrc_t r, uint32_t off) {
   return __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, off, 0, 0));
 }
-template <> __device__ __forceinline__ float buffer_load1<bf16_t>(__amdgpu_buffer_rsrc_t r, uint32_t off) {
-  return __uint_as_float(static_cast<uint32_t>(static_cast<uint16_t>(__builtin_amdgcn_raw_buffer_load_b16(r, off, 0, 0))) << 16);
-}
 
 constexpr int kPatchDepth = 4;                        // backprop k-tiles in flight per lane
 constexpr int kPatchTrip = kPatchDepth * mf32::BK;    // k extent of one trip of the k loop
+
+// ---- staging of the padded patch, shared by the two patch kernels ----------------------------
+// CELL is what the patch holds: float (the fp32 kernel widens its input) or uint16_t (the bf16
+// kernel keeps bf16 as it is). The table entry of an output position is the cell offset of its
+// first patch cell times qmul (the bf16 kernel addresses bytes).
+template <typename TIN, typename CELL>
+struct PatchCell;
+template <typename TIN>
+struct PatchCell<TIN, float> {
+  typedef typename dpk_io<TIN>::raw4 raw4;
+  static __device__ __forceinline__ raw4 load4(const TIN* p) { return dpk_io<TIN>::load4_raw(p); }
+  static __device__ __forceinline__ void put4(float* dst, raw4 r) {
+    const float4 v = dpk_io<TIN>::unpack4(r);
+    dst[0] = v.x;
+    dst[1] = v.y;
+    dst[2] = v.z;
+    dst[3] = v.w;
+  }
+  static __device__ __forceinline__ float load1(const TIN* p) { return dpk_io<TIN>::load(p); }
+};
+template <>
+struct PatchCell<bf16_t, uint16_t> {
+  typedef dpk_vu2 raw4;
+  static __device__ __forceinline__ raw4 load4(const bf16_t* p) { return dpk_io<bf16_t>::load4_raw(p); }
+  static __device__ __forceinline__ void put4(uint16_t* dst, raw4 r) {
+    dst[0] = static_cast<uint16_t>(r.x);
+    dst[1] = static_cast<uint16_t>(r.x >> 16);
+    dst[2] = static_cast<uint16_t>(r.y);
+    dst[3] = static_cast<uint16_t>(r.y >> 16);
+  }
+  static __device__ __forceinline__ uint16_t load1(const bf16_t* p) { return *p; }
+};
+
+// Stages nch channels of the image at xg into xs (zero outside the image) and fills the table.
+// A wave takes whole rows of the padded patch, lane = column, so no index is ever divided:
+// (channel, row) advance by additions; 32 rows are loaded before any of them is stored (the
+// staging is bound by global latency). When image rows are whole, aligned 4-element chunks
+// (xvec) the interior is instead fetched as such chunks, eight per thread all in flight at once
+// - one round trip per block - after the patch has been zeroed for its padding. The caller's
+// barrier publishes both.
+template <typename TIN, typename CELL>
+__device__ __forceinline__ void stage_patch(CELL* __restrict__ xs, int* __restrict__ qtab,
+                                            const TIN* __restrict__ xg, const ConvGeom& g, PatchDims pd,
+                                            int nch, int xvec, int Qpad, int qmul) {
+  typedef PatchCell<TIN, CELL> PC;
+  const int Hp = pd.Hp, Wp = pd.Wp, RS = pd.rs, CS = pd.cs;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int rows = nch * Hp;
+  if (xvec) {
+    constexpr int kPer16 = 16 / static_cast<int>(sizeof(CELL));
+    const int total16 = nch * CS / kPer16;  // the patch starts 16-byte aligned; a ragged tail is zeroed below
+    for (int i = threadIdx.x; i < total16; i += kThreads)
+      reinterpret_cast<uint4*>(xs)[i] = make_uint4(0u, 0u, 0u, 0u);
+    for (int i = total16 * kPer16 + threadIdx.x; i < nch * CS; i += kThreads) xs[i] = static_cast<CELL>(0);
+    __syncthreads();
+    const int W4 = g.W / 4, chunks = nch * g.H * W4;
+    constexpr int kChunksInFlight = 8;
+    for (int i0 = threadIdx.x; i0 < chunks; i0 += kThreads * kChunksInFlight) {
+      typename PC::raw4 v[kChunksInFlight];
+#pragma unroll
+      for (int u = 0; u < kChunksInFlight; ++u) {
+        const int i = i0 + u * kThreads;
+        v[u] = PC::load4(xg + static_cast<int64_t>(i < chunks ? i : 0) * 4);
+      }
+#pragma unroll
+      for (int u = 0; u < kChunksInFlight; ++u) {
+        const int i = i0 + u * kThreads;
+        if (i < chunks) {
+          const int r = i / W4, x4 = i - r * W4;  // r = c * H + iy
+          const int c = r / g.H, iy = r - c * g.H;
+          PC::put4(xs + c * CS + (iy + g.ph) * RS + g.pw + x4 * 4, v[u]);
+        }
+      }
+    }
+  } else {
+    constexpr int kRowsInFlight = 32;
+    for (int x0 = 0; x0 < Wp; x0 += DPK_WAVE) {
+      const int xx = x0 + lane, ix = xx - g.pw;
+      const bool col_ok = xx < Wp && static_cast<unsigned>(ix) < static_cast<unsigned>(g.W);
+      int c = 0, y = wave;  // of the next row this wave stages
+      while (y >= Hp) {
+        y -= Hp;
+        ++c;
+      }
+      for (int row = wave; row < rows; row += kWaves * kRowsInFlight) {
+        CELL v[kRowsInFlight];
+        const int c_first = c, y_first = y;
+#pragma unroll
+        for (int u = 0; u < kRowsInFlight; ++u) {
+          const int iy = y - g.ph;
+          const bool in = col_ok && row + u * kWaves < rows && static_cast<unsigned>(iy) < static_cast<unsigned>(g.H);
+          v[u] = in ? PC::load1(xg + (static_cast<int64_t>(c) * g.H + iy) * g.W + ix) : static_cast<CELL>(0);
+          y += kWaves;
+          while (y >= Hp) {
+            y -= Hp;
+            ++c;
+          }
+        }
+        // the same walk again for the cells (wave-uniform, a few scalar additions per row)
+        int cs_ = c_first, ys_ = y_first;
+#pragma unroll
+        for (int u = 0; u < kRowsInFlight; ++u) {
+          const int r = row + u * kWaves;
+          if (r < rows && xx < Wp) xs[cs_ * CS + ys_ * RS + xx] = v[u];
+          ys_ += kWaves;
+          while (ys_ >= Hp) {
+            ys_ -= Hp;
+            ++cs_;
+          }
+        }
+      }
+    }
+  }
+  for (int q = threadIdx.x; q < Qpad; q += kThreads) {
+    const int oh = q / g.OW, ow = q - oh * g.OW;
+    qtab[q] = q < g.Q ? (oh * g.sh * RS + ow * g.sw) * qmul : 0;
+  }
+}
 
 // RK (8, 4 or 0): the eight positions a half-wave takes of a k-tile fall into aligned runs of RK
 // positions that lie in one output row at unit stride (stride 1 along the row, output width a
@@ -241,7 +348,7 @@ __global__ __launch_bounds__(kThreads) void conv2d_gs_patch_kernel(
     const TIN* __restrict__ x, const TIN* __restrict__ b, TOUT* __restrict__ gs,
     float* __restrict__ partials, ConvGeom g, int C, int O, int groups, float scale, int tiles_m,
     int tiles_n, PatchDims pd, int xvec, int nch_max) {
-  const int Hp = pd.Hp, Wp = pd.Wp, RS = pd.rs, CS = pd.cs;
+  const int RS = pd.rs, CS = pd.cs;
   using Tile = mf32::Tile<BM, BN>;
   extern __shared__ __align__(16) unsigned char dyn_lds[];
   // layout: qtab | patch. The k loop runs in trips of kPatchDepth k-tiles, all of them
@@ -270,85 +377,8 @@ __global__ __launch_bounds__(kThreads) void conv2d_gs_patch_kernel(
   const int nch = c_hi - c_lo + 1;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 
-  // stage the patch (zero outside the image). A wave takes whole rows of the padded patch,
-  // lane = column, so no index is ever divided: (channel, row) advance by additions. 32 rows
-  // are loaded before any of them is stored: the staging is bound by global latency.
-  // When image rows are whole 16-byte chunks (xvec) the interior is instead fetched as
-  // 4-element chunks, eight per thread all in flight at once - one round trip per block -
-  // after the patch has been zeroed for its padding.
   const TIN* xg = x + ((sample * C + static_cast<int64_t>(grp) * Cg + c_lo) * g.H) * g.W;
-  const int rows = nch * Hp;
-  constexpr int kRowsInFlight = 32;
-  if (xvec) {
-    const int total4 = nch * CS / 4;  // the patch starts 16-byte aligned; a ragged tail is zeroed below
-    for (int i = threadIdx.x; i < total4; i += kThreads)
-      reinterpret_cast<float4*>(xs)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int i = total4 * 4 + threadIdx.x; i < nch * CS; i += kThreads) xs[i] = 0.f;
-    __syncthreads();
-    const int W4 = g.W / 4, chunks = nch * g.H * W4;
-    constexpr int kChunksInFlight = 8;
-    for (int i0 = threadIdx.x; i0 < chunks; i0 += kThreads * kChunksInFlight) {
-      float4 v[kChunksInFlight];
-#pragma unroll
-      for (int u = 0; u < kChunksInFlight; ++u) {
-        const int i = i0 + u * kThreads;
-        v[u] = i < chunks ? dpk_io<TIN>::load4(xg + static_cast<int64_t>(i) * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
-      }
-#pragma unroll
-      for (int u = 0; u < kChunksInFlight; ++u) {
-        const int i = i0 + u * kThreads;
-        if (i < chunks) {
-          const int r = i / W4, x4 = i - r * W4;     // r = c * H + iy
-          const int c = r / g.H, iy = r - c * g.H;
-          float* dst = xs + c * CS + (iy + g.ph) * RS + g.pw + x4 * 4;
-          dst[0] = v[u].x;
-          dst[1] = v[u].y;
-          dst[2] = v[u].z;
-          dst[3] = v[u].w;
-        }
-      }
-    }
-  }
-  for (int x0 = 0; x0 < (xvec ? 0 : Wp); x0 += DPK_WAVE) {
-    const int xx = x0 + lane, ix = xx - g.pw;
-    const bool col_ok = xx < Wp && static_cast<unsigned>(ix) < static_cast<unsigned>(g.W);
-    int c = 0, y = wave;  // of the next row this wave stages
-    while (y >= Hp) {
-      y -= Hp;
-      ++c;
-    }
-    for (int row = wave; row < rows; row += kWaves * kRowsInFlight) {
-      float v[kRowsInFlight];
-      const int c_first = c, y_first = y;
-#pragma unroll
-      for (int u = 0; u < kRowsInFlight; ++u) {
-        const int iy = y - g.ph;
-        const bool in = col_ok && row + u * kWaves < rows && static_cast<unsigned>(iy) < static_cast<unsigned>(g.H);
-        v[u] = in ? dpk_io<TIN>::load(xg + (static_cast<int64_t>(c) * g.H + iy) * g.W + ix) : 0.f;
-        y += kWaves;
-        while (y >= Hp) {
-          y -= Hp;
-          ++c;
-        }
-      }
-      // the same walk again for the cells (wave-uniform, a few scalar additions per row)
-      int cs_ = c_first, ys_ = y_first;
-#pragma unroll
-      for (int u = 0; u < kRowsInFlight; ++u) {
-        const int r = row + u * kWaves;
-        if (r < rows && xx < Wp) xs[cs_ * CS + ys_ * RS + xx] = v[u];
-        ys_ += kWaves;
-        while (ys_ >= Hp) {
-          ys_ -= Hp;
-          ++cs_;
-        }
-      }
-    }
-  }
-  for (int q = threadIdx.x; q < Qpad; q += kThreads) {
-    const int oh = q / g.OW, ow = q - oh * g.OW;
-    qtab[q] = q < g.Q ? oh * g.sh * RS + ow * g.sw : 0;
-  }
+  stage_patch<TIN, float>(xs, qtab, xg, g, pd, nch, xvec, Qpad, 1);
   // this lane's columns of the tile
   const int wm0 = (wave >> 1) * Tile::WM, wn0 = (wave & 1) * Tile::WN;
   const int kk = lane >> 5, l32 = lane & 31;
@@ -517,7 +547,7 @@ __global__ __launch_bounds__(kThreads) void conv2d_gs_patch16_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ b, TOUT* __restrict__ gs,
     float* __restrict__ partials, ConvGeom g, int C, int O, int groups, float scale, int tiles_m,
     int tiles_n, PatchDims pd, int xvec, int a_off) {
-  const int Hp = pd.Hp, Wp = pd.Wp, RS = pd.rs, CS = pd.cs;
+  const int RS = pd.rs, CS = pd.cs;
   using Tile = mf32::Tile<BM, BN>;  // accumulator layout of a 32 x 32 MFMA tile: the same
   typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
   typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -545,80 +575,8 @@ __global__ __launch_bounds__(kThreads) void conv2d_gs_patch16_kernel(
   const int nch = c_hi - c_lo + 1;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 
-  // stage the patch as above, in bf16
   const bf16_t* xg = x + ((sample * C + static_cast<int64_t>(grp) * Cg + c_lo) * g.H) * g.W;
-  const int rows = nch * Hp;
-  if (xvec) {
-    const int total8 = nch * CS / 8;  // 16-byte chunks; the patch starts 16-byte aligned
-    for (int i = threadIdx.x; i < total8; i += kThreads)
-      reinterpret_cast<uint4*>(xs)[i] = make_uint4(0u, 0u, 0u, 0u);
-    for (int i = total8 * 8 + threadIdx.x; i < nch * CS; i += kThreads) xs[i] = 0;
-    __syncthreads();
-    const int W4 = g.W / 4, chunks = nch * g.H * W4;
-    constexpr int kChunksInFlight = 8;
-    for (int i0 = threadIdx.x; i0 < chunks; i0 += kThreads * kChunksInFlight) {
-      dpk_vu2 v[kChunksInFlight];
-#pragma unroll
-      for (int u = 0; u < kChunksInFlight; ++u) {
-        const int i = i0 + u * kThreads;
-        v[u] = dpk_io<bf16_t>::load4_raw(xg + static_cast<int64_t>(i < chunks ? i : 0) * 4);
-      }
-#pragma unroll
-      for (int u = 0; u < kChunksInFlight; ++u) {
-        const int i = i0 + u * kThreads;
-        if (i < chunks) {
-          const int r = i / W4, x4 = i - r * W4;  // r = c * H + iy
-          const int c = r / g.H, iy = r - c * g.H;
-          uint16_t* dst = xs + c * CS + (iy + g.ph) * RS + g.pw + x4 * 4;
-          dst[0] = static_cast<uint16_t>(v[u].x);
-          dst[1] = static_cast<uint16_t>(v[u].x >> 16);
-          dst[2] = static_cast<uint16_t>(v[u].y);
-          dst[3] = static_cast<uint16_t>(v[u].y >> 16);
-        }
-      }
-    }
-  }
-  constexpr int kRowsInFlight = 32;
-  for (int x0 = 0; x0 < (xvec ? 0 : Wp); x0 += DPK_WAVE) {
-    const int xx = x0 + lane, ix = xx - g.pw;
-    const bool col_ok = xx < Wp && static_cast<unsigned>(ix) < static_cast<unsigned>(g.W);
-    int c = 0, y = wave;  // of the next row this wave stages
-    while (y >= Hp) {
-      y -= Hp;
-      ++c;
-    }
-    for (int row = wave; row < rows; row += kWaves * kRowsInFlight) {
-      uint16_t v[kRowsInFlight];
-      const int c_first = c, y_first = y;
-#pragma unroll
-      for (int u = 0; u < kRowsInFlight; ++u) {
-        const int iy = y - g.ph;
-        const bool in = col_ok && row + u * kWaves < rows && static_cast<unsigned>(iy) < static_cast<unsigned>(g.H);
-        v[u] = in ? xg[(static_cast<int64_t>(c) * g.H + iy) * g.W + ix] : static_cast<uint16_t>(0);
-        y += kWaves;
-        while (y >= Hp) {
-          y -= Hp;
-          ++c;
-        }
-      }
-      // the same walk again for the cells (wave-uniform, a few scalar additions per row)
-      int cs_ = c_first, ys_ = y_first;
-#pragma unroll
-      for (int u = 0; u < kRowsInFlight; ++u) {
-        const int r = row + u * kWaves;
-        if (r < rows && xx < Wp) xs[cs_ * CS + ys_ * RS + xx] = v[u];
-        ys_ += kWaves;
-        while (ys_ >= Hp) {
-          ys_ -= Hp;
-          ++cs_;
-        }
-      }
-    }
-  }
-  for (int q = threadIdx.x; q < Qpad; q += kThreads) {
-    const int oh = q / g.OW, ow = q - oh * g.OW;
-    qtab[q] = q < g.Q ? (oh * g.sh * RS + ow * g.sw) * 2 : 0;
-  }
+  stage_patch<bf16_t, uint16_t>(xs, qtab, xg, g, pd, nch, xvec, Qpad, 2);
   const int wm0 = (wave >> 1) * Tile::WM, wn0 = (wave & 1) * Tile::WN;
   const int kk = lane >> 5, l32 = lane & 31;
   // byte address inside the patch of this lane's patch element (its columns of the tile)
