@@ -178,6 +178,28 @@ def test_c4_conv_and_group_norm_full_size(K):
     assert rel_err(gw, want_w) < FP32_REL and rel_err(gb, want_b) < FP32_REL
 
 
+@pytest.mark.parametrize(
+    "n,C,Oc,H",
+    [(256, 64, 64, 32), (64, 128, 128, 28), (32, 64, 64, 56)],  # C4's shape; 128-row blocks, runs of 4; a patch above 64 KB
+)
+def test_conv_bf16_kernel_against_the_fp32_kernel_full_size(K, n, C, Oc, H):
+    """bf16 input runs its own kernel (bf16 MFMA). On the same bf16-exact data the fp32 kernel forms
+    the same exact products and also accumulates in fp32, so the two must agree to fp32 rounding."""
+    torch.manual_seed(n + H)
+    x = torch.randn(n, C, H, H, device="cuda").bfloat16()
+    b = torch.randn(n, Oc, H, H, device="cuda").bfloat16()
+    geo = dict(kernel_size=(3, 3), stride=(1, 1), padding=(1, 1, 1, 1), dilation=(1, 1), groups=1)
+    g16, s16 = K.conv2d_grad_sample(x, b, out_dtype=torch.float32, **geo)
+    g32, s32 = K.conv2d_grad_sample(x.float(), b.float(), **geo)
+    assert rel_err(g16, g32) < FP32_REL
+    assert rel_err(s16, s32) < FP32_REL
+    pick = [0, n - 1]
+    want, _ = O.conv2d_grad_sample(
+        x[pick].cpu().double(), b[pick].cpu().double(), kernel_size=(3, 3), padding=(1, 1), stride=(1, 1), dilation=(1, 1), groups=1
+    )
+    assert rel_err(g16[pick], want) < FP32_REL
+
+
 # ---- C5: Embedding ghost norm and RMSNorm at batch 16, seq 1024, dim 2048, bf16 ---------------
 def test_c5_embedding_and_rms_norm_full_size(K):
     n, T, D, V = 16, 1024, 2048, 32000
