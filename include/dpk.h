@@ -261,29 +261,33 @@ int dpk_tied_embedding_cross(const int64_t* ids, const void* e, int emb_dtype, c
 /* gs_w[n,c] = scale * sum_s group_norm(x)[n,c,s] * b[n,c,s]   (group_norm.py:43-44)
  * gs_b[n,c] = scale * sum_s b[n,c,s]                          (group_norm.py:46)
  * x, b: [n,C,S]; normalisation without affine over each (n, group). Either
- * output may be NULL. */
+ * output may be NULL. sumsq_w[n] / sumsq_b[n] (float, may be NULL): the per-sample
+ * sums of squares of gs_w / gs_b. */
 int dpk_group_norm_gs(const void* x, const void* b, int in_dtype, void* gs_w, void* gs_b,
-                      int gs_dtype, int64_t n, int64_t C, int64_t S, int64_t groups, float eps,
-                      float scale, dpk_stream_t stream);
+                      int gs_dtype, float* sumsq_w, float* sumsq_b, int64_t n, int64_t C,
+                      int64_t S, int64_t groups, float eps, float scale, dpk_stream_t stream);
 
 /* gs_w[n,d] = scale * sum_t x[n,t,d] * rsqrt(mean_d x[n,t,:]^2 + eps) * b[n,t,d]
- * (rms_norm.py:44-47). x, b: [n,T,D], D = number of normalised elements. */
+ * (rms_norm.py:44-47). x, b: [n,T,D], D = number of normalised elements.
+ * sumsq[n] (float, may be NULL) = sum_d gs_w[n,d]^2, for the optimizer's norm pass. */
 size_t dpk_rms_norm_gs_workspace_bytes(int64_t n, int64_t T, int64_t D);
 int dpk_rms_norm_gs(const void* x, const void* b, int in_dtype, void* gs_w, int gs_dtype,
-                    int64_t n, int64_t T, int64_t D, float eps, float scale, void* ws,
-                    size_t ws_bytes, dpk_stream_t stream);
+                    float* sumsq, int64_t n, int64_t T, int64_t D, float eps, float scale,
+                    void* ws, size_t ws_bytes, dpk_stream_t stream);
 
 /* gs_w[n,d] = scale * sum_t layer_norm(x)[n,t,d] * b[n,t,d]   (layer_norm.py:41-47)
  * gs_b[n,d] = scale * sum_t b[n,t,d]                          (layer_norm.py:49)
  * x, b: [n,T,D], D = number of normalised elements (the product of
  * normalized_shape), T = everything between the batch and those dimensions.
  * Normalisation without affine: (x - mean) * rsqrt(var + eps), biased variance.
- * Either output may be NULL. (InstanceNorm, instance_norm.py:50-55, is
- * dpk_group_norm_gs with groups == C.) */
+ * Either output may be NULL. sumsq_w[n] / sumsq_b[n] (float, may be NULL): the
+ * per-sample sums of squares of gs_w / gs_b. (InstanceNorm, instance_norm.py:50-55,
+ * is dpk_group_norm_gs with groups == C.) */
 size_t dpk_layer_norm_gs_workspace_bytes(int64_t n, int64_t T, int64_t D);
 int dpk_layer_norm_gs(const void* x, const void* b, int in_dtype, void* gs_w, void* gs_b,
-                      int gs_dtype, int64_t n, int64_t T, int64_t D, float eps, float scale,
-                      void* ws, size_t ws_bytes, dpk_stream_t stream);
+                      int gs_dtype, float* sumsq_w, float* sumsq_b, int64_t n, int64_t T,
+                      int64_t D, float eps, float scale, void* ws, size_t ws_bytes,
+                      dpk_stream_t stream);
 
 /* ------------------------------------------------------------------------- *
  * DPOptimizer.clip_and_accumulate, add_noise, scale_grad

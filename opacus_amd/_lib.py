@@ -83,13 +83,13 @@ SIGNATURES = {
         c_int,
         [_P, _P, c_int, _P, _P, c_int, _P, _I, _I, _I, _I, _I, c_float, _P, c_size_t, _P],
     ),
-    "dpk_group_norm_gs": (c_int, [_P, _P, c_int, _P, _P, c_int, _I, _I, _I, _I, c_float, c_float, _P]),
+    "dpk_group_norm_gs": (c_int, [_P, _P, c_int, _P, _P, c_int, _P, _P, _I, _I, _I, _I, c_float, c_float, _P]),
     "dpk_rms_norm_gs_workspace_bytes": (c_size_t, [_I, _I, _I]),
-    "dpk_rms_norm_gs": (c_int, [_P, _P, c_int, _P, c_int, _I, _I, _I, c_float, c_float, _P, c_size_t, _P]),
+    "dpk_rms_norm_gs": (c_int, [_P, _P, c_int, _P, c_int, _P, _I, _I, _I, c_float, c_float, _P, c_size_t, _P]),
     "dpk_layer_norm_gs_workspace_bytes": (c_size_t, [_I, _I, _I]),
     "dpk_layer_norm_gs": (
         c_int,
-        [_P, _P, c_int, _P, _P, c_int, _I, _I, _I, c_float, c_float, _P, c_size_t, _P],
+        [_P, _P, c_int, _P, _P, c_int, _P, _P, _I, _I, _I, c_float, c_float, _P, c_size_t, _P],
     ),
     "dpk_sumsq_rows_workspace_bytes": (c_size_t, [_I, _I]),
     "dpk_sumsq_rows": (c_int, [_P, c_int, _I, _I, _P, _P, c_size_t, _P]),

@@ -248,6 +248,24 @@ __global__ __launch_bounds__(kThreads) void row_final_kernel(const float* __rest
   dpk_io<TOUT>::store(gw + i, ((s0 + s1) + (s2 + s3)) * scale);
 }
 
+// Per-sample sum of squares of the [n, D] result (as stored), a block per sample: the optimizer's
+// norm pass then has nothing to read. The result is a few KB per sample and still in cache; a
+// final sum with a block per sample that squared on the way was tried and is slower (16 blocks
+// read 8 MB of partial sums).
+template <typename TOUT>
+__global__ __launch_bounds__(kThreads) void row_sumsq_kernel(const TOUT* __restrict__ gw, int64_t D,
+                                                              float* __restrict__ sumsq) {
+  __shared__ float red[kWaves];
+  const TOUT* row = gw + static_cast<int64_t>(blockIdx.x) * D;
+  float ss = 0.f;
+  for (int64_t d = threadIdx.x; d < D; d += kThreads) {
+    const float v = dpk_io<TOUT>::load(row + d);
+    ss = fmaf(v, v, ss);
+  }
+  const float total = block_sum<kWaves>(ss, red);
+  if (threadIdx.x == 0) sumsq[blockIdx.x] = total;
+}
+
 // Cross-wave sum of per-lane float4 chunks through LDS, written to o[0..D).
 template <int NCH>
 __device__ __forceinline__ void rows_meet(const float4 (&acc)[NCH], float (&red)[kWaves][256 * NCH],
@@ -443,8 +461,8 @@ void launch_rows(const TIN* x, const TIN* b, int64_t n, int64_t T, int64_t D, fl
 
 // Shared body of the two entry points. gs_b is only meaningful with layer_norm.
 int row_norm_gs(const char* who, bool layer_norm, const void* x, const void* b, int in_dtype, void* gs_w,
-                void* gs_b, int gs_dtype, int64_t n, int64_t T, int64_t D, float eps, float scale, void* ws,
-                size_t ws_bytes, dpk_stream_t stream) {
+                void* gs_b, int gs_dtype, float* sumsq_w, float* sumsq_b, int64_t n, int64_t T, int64_t D, float eps,
+                float scale, void* ws, size_t ws_bytes, dpk_stream_t stream) {
   DPK_REQUIRE(n >= 0 && T >= 1 && D >= 1, DPK_E_SHAPE, "%s: n=%lld T=%lld D=%lld", who, (long long)n,
               (long long)T, (long long)D);
   if (n == 0 || (!gs_w && !gs_b)) return DPK_OK;
@@ -486,6 +504,7 @@ int row_norm_gs(const char* who, bool layer_norm, const void* x, const void* b, 
   const dim3 block(kThreads), g3(static_cast<unsigned>(dpk_cdiv(n * D, kThreads)));
   for (int pass = 0; pass < 2; ++pass) {
     void* out = pass == 0 ? gs_w : gs_b;
+    float* ssq = pass == 0 ? sumsq_w : sumsq_b;
     const float* src = pass == 0 ? w.part(ws) : w.partb(ws);
     if (!out) continue;
     if (gs_dtype == DPK_F32)
@@ -493,6 +512,13 @@ int row_norm_gs(const char* who, bool layer_norm, const void* x, const void* b, 
     else
       hipLaunchKernelGGL(row_final_kernel<bf16_t>, g3, block, 0, s, src, n * D, TS, scale,
                          static_cast<bf16_t*>(out));
+    if (ssq) {
+      const dim3 gn(static_cast<unsigned>(n));
+      if (gs_dtype == DPK_F32)
+        hipLaunchKernelGGL(row_sumsq_kernel<float>, gn, block, 0, s, static_cast<const float*>(out), D, ssq);
+      else
+        hipLaunchKernelGGL(row_sumsq_kernel<bf16_t>, gn, block, 0, s, static_cast<const bf16_t*>(out), D, ssq);
+    }
   }
   DPK_LAUNCH_CHECK(who);
   return DPK_OK;
@@ -501,8 +527,8 @@ int row_norm_gs(const char* who, bool layer_norm, const void* x, const void* b, 
 }  // namespace
 
 extern "C" int dpk_group_norm_gs(const void* x, const void* b, int in_dtype, void* gs_w, void* gs_b,
-                                 int gs_dtype, int64_t n, int64_t C, int64_t S, int64_t groups,
-                                 float eps, float scale, dpk_stream_t stream) {
+                                 int gs_dtype, float* sumsq_w, float* sumsq_b, int64_t n, int64_t C,
+                                 int64_t S, int64_t groups, float eps, float scale, dpk_stream_t stream) {
   const char* who = "dpk_group_norm_gs";
   DPK_REQUIRE(n >= 0 && C >= 1 && S >= 1 && groups >= 1, DPK_E_SHAPE,
               "%s: n=%lld C=%lld S=%lld groups=%lld", who, (long long)n, (long long)C, (long long)S,
@@ -542,6 +568,18 @@ extern "C" int dpk_group_norm_gs(const void* x, const void* b, int in_dtype, voi
 #undef DPK_GN
 #undef DPK_GN_ARGS
   DPK_LAUNCH_CHECK(who);
+  // per-sample sums of squares of the [n, C] results, for the optimizer's norm pass
+  for (int pass = 0; pass < 2; ++pass) {
+    const void* out = pass == 0 ? gs_w : gs_b;
+    float* ssq = pass == 0 ? sumsq_w : sumsq_b;
+    if (!out || !ssq) continue;
+    const dim3 gn(static_cast<unsigned>(n));
+    if (gs_dtype == DPK_F32)
+      hipLaunchKernelGGL(row_sumsq_kernel<float>, gn, block, 0, s, static_cast<const float*>(out), C, ssq);
+    else
+      hipLaunchKernelGGL(row_sumsq_kernel<bf16_t>, gn, block, 0, s, static_cast<const bf16_t*>(out), C, ssq);
+    DPK_LAUNCH_CHECK(who);
+  }
   return DPK_OK;
 }
 
@@ -551,11 +589,11 @@ extern "C" size_t dpk_rms_norm_gs_workspace_bytes(int64_t n, int64_t T, int64_t 
 }
 
 extern "C" int dpk_rms_norm_gs(const void* x, const void* b, int in_dtype, void* gs_w, int gs_dtype,
-                               int64_t n, int64_t T, int64_t D, float eps, float scale, void* ws,
-                               size_t ws_bytes, dpk_stream_t stream) {
+                               float* sumsq, int64_t n, int64_t T, int64_t D, float eps, float scale,
+                               void* ws, size_t ws_bytes, dpk_stream_t stream) {
   DPK_REQUIRE(gs_w || n == 0, DPK_E_ARG, "dpk_rms_norm_gs: NULL tensor");
-  return row_norm_gs("dpk_rms_norm_gs", false, x, b, in_dtype, gs_w, nullptr, gs_dtype, n, T, D, eps, scale,
-                     ws, ws_bytes, stream);
+  return row_norm_gs("dpk_rms_norm_gs", false, x, b, in_dtype, gs_w, nullptr, gs_dtype, sumsq, nullptr, n, T, D,
+                     eps, scale, ws, ws_bytes, stream);
 }
 
 extern "C" size_t dpk_layer_norm_gs_workspace_bytes(int64_t n, int64_t T, int64_t D) {
@@ -563,8 +601,8 @@ extern "C" size_t dpk_layer_norm_gs_workspace_bytes(int64_t n, int64_t T, int64_
 }
 
 extern "C" int dpk_layer_norm_gs(const void* x, const void* b, int in_dtype, void* gs_w, void* gs_b,
-                                 int gs_dtype, int64_t n, int64_t T, int64_t D, float eps, float scale,
-                                 void* ws, size_t ws_bytes, dpk_stream_t stream) {
-  return row_norm_gs("dpk_layer_norm_gs", true, x, b, in_dtype, gs_w, gs_b, gs_dtype, n, T, D, eps, scale, ws,
-                     ws_bytes, stream);
+                                 int gs_dtype, float* sumsq_w, float* sumsq_b, int64_t n, int64_t T, int64_t D,
+                                 float eps, float scale, void* ws, size_t ws_bytes, dpk_stream_t stream) {
+  return row_norm_gs("dpk_layer_norm_gs", true, x, b, in_dtype, gs_w, gs_b, gs_dtype, sumsq_w, sumsq_b, n, T, D,
+                     eps, scale, ws, ws_bytes, stream);
 }

@@ -9,6 +9,7 @@ import torch
 import torch.nn as nn
 
 from .. import kernels
+from ._common import tag_sumsq
 from .grad_sample_module import fused_scale, owns_output
 from .utils import register_grad_sampler
 
@@ -33,7 +34,7 @@ def compute_layer_norm_grad_sample(
         x, backprops, numel, layer.eps, scale=scale, want_weight=want_w, want_bias=want_b
     )
     if want_w:
-        ret[layer.weight] = gw.view(x.shape[0], *layer.normalized_shape)
+        ret[layer.weight] = tag_sumsq(gw.view(x.shape[0], *layer.normalized_shape), getattr(gw, "_dpk_sumsq", None))
     if want_b:
-        ret[layer.bias] = gb.view(x.shape[0], *layer.normalized_shape)
+        ret[layer.bias] = tag_sumsq(gb.view(x.shape[0], *layer.normalized_shape), getattr(gb, "_dpk_sumsq", None))
     return ret

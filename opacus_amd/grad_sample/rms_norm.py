@@ -9,6 +9,7 @@ import torch
 import torch.nn as nn
 
 from .. import kernels
+from ._common import tag_sumsq
 from .grad_sample_module import fused_scale, owns_output
 from .utils import register_grad_sampler
 
@@ -28,4 +29,4 @@ def compute_rms_norm_grad_sample(
     eps = layer.eps if layer.eps is not None else torch.finfo(x.dtype).eps
     numel = math.prod(layer.normalized_shape)
     gw = kernels.rms_norm_grad_sample(x, backprops, numel, eps, scale=scale)
-    return {layer.weight: gw.view(x.shape[0], *layer.normalized_shape)}
+    return {layer.weight: tag_sumsq(gw.view(x.shape[0], *layer.normalized_shape), gw._dpk_sumsq if x.shape[0] else None)}

@@ -594,7 +594,8 @@ def group_norm_grad_sample(
     want_weight: bool = True,
     want_bias: bool = True,
 ) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
-    """Per-sample gradients ``[n, C]`` of GroupNorm's weight and bias."""
+    """Per-sample gradients ``[n, C]`` of GroupNorm's weight and bias, each with its per-sample sum
+    of squares riding on it for the optimizer."""
     dev = _need_gpu(x, backprops)
     if x.dtype != backprops.dtype:
         x = x.to(backprops.dtype)
@@ -605,21 +606,24 @@ def group_norm_grad_sample(
         return gw, gb
     xd = _dense(x).reshape(n, C, -1)
     bd = _dense(backprops).reshape(n, C, -1)
+    ssw = torch.empty((n,), dtype=torch.float32, device=dev) if want_weight else None
+    ssb = torch.empty((n,), dtype=torch.float32, device=dev) if want_bias else None
     with _timed("group_norm_gs", dev):
         check(
             "dpk_group_norm_gs",
             lib().dpk_group_norm_gs(
-                _ptr(xd), _ptr(bd), _code(bd), _ptr(gw), _ptr(gb), _code(backprops.dtype), n, C,
-                xd.shape[2], num_groups, float(eps), float(scale), _stream(dev),
+                _ptr(xd), _ptr(bd), _code(bd), _ptr(gw), _ptr(gb), _code(backprops.dtype), _ptr(ssw), _ptr(ssb),
+                n, C, xd.shape[2], num_groups, float(eps), float(scale), _stream(dev),
             ),
         )
-    return gw, gb
+    return (_with_sumsq(gw, ssw) if want_weight else None), (_with_sumsq(gb, ssb) if want_bias else None)
 
 
 def rms_norm_grad_sample(
     x: torch.Tensor, backprops: torch.Tensor, normalized_numel: int, eps: float, scale: float = 1.0
 ) -> torch.Tensor:
-    """Per-sample gradient ``[n, D]`` of RMSNorm's weight (``D = normalized_numel``)."""
+    """Per-sample gradient ``[n, D]`` of RMSNorm's weight (``D = normalized_numel``); its
+    per-sample sum of squares rides on the result for the optimizer."""
     dev = _need_gpu(x, backprops)
     if x.dtype != backprops.dtype:
         x = x.to(backprops.dtype)
@@ -627,6 +631,7 @@ def rms_norm_grad_sample(
     gw = torch.empty((n, D), dtype=backprops.dtype, device=dev)
     if n == 0:
         return gw
+    sumsq = torch.empty((n,), dtype=torch.float32, device=dev)
     xd = _dense(x).reshape(n, -1, D)
     bd = _dense(backprops).reshape(n, -1, D)
     T = xd.shape[1]
@@ -636,11 +641,11 @@ def rms_norm_grad_sample(
         check(
             "dpk_rms_norm_gs",
             L.dpk_rms_norm_gs(
-                _ptr(xd), _ptr(bd), _code(bd), _ptr(gw), _code(gw), n, T, D, float(eps), float(scale),
+                _ptr(xd), _ptr(bd), _code(bd), _ptr(gw), _code(gw), _ptr(sumsq), n, T, D, float(eps), float(scale),
                 _ptr(ws), wsb, _stream(dev),
             ),
         )
-    return gw
+    return _with_sumsq(gw, sumsq)
 
 
 def layer_norm_grad_sample(
@@ -652,7 +657,8 @@ def layer_norm_grad_sample(
     want_weight: bool = True,
     want_bias: bool = True,
 ) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
-    """Per-sample gradients ``[n, D]`` of LayerNorm's weight and bias (``D = normalized_numel``)."""
+    """Per-sample gradients ``[n, D]`` of LayerNorm's weight and bias (``D = normalized_numel``),
+    each with its per-sample sum of squares riding on it for the optimizer."""
     dev = _need_gpu(x, backprops)
     if x.dtype != backprops.dtype:
         x = x.to(backprops.dtype)
@@ -665,16 +671,18 @@ def layer_norm_grad_sample(
     bd = _dense(backprops).reshape(n, -1, D)
     T = xd.shape[1]
     L = lib()
+    ssw = torch.empty((n,), dtype=torch.float32, device=dev) if want_weight else None
+    ssb = torch.empty((n,), dtype=torch.float32, device=dev) if want_bias else None
     ws, wsb = _ws(L.dpk_layer_norm_gs_workspace_bytes(n, T, D), dev)
     with _timed("layer_norm_gs", dev):
         check(
             "dpk_layer_norm_gs",
             L.dpk_layer_norm_gs(
-                _ptr(xd), _ptr(bd), _code(bd), _ptr(gw), _ptr(gb), _code(bd), n, T, D, float(eps), float(scale),
-                _ptr(ws), wsb, _stream(dev),
+                _ptr(xd), _ptr(bd), _code(bd), _ptr(gw), _ptr(gb), _code(bd), _ptr(ssw), _ptr(ssb), n, T, D,
+                float(eps), float(scale), _ptr(ws), wsb, _stream(dev),
             ),
         )
-    return gw, gb
+    return (_with_sumsq(gw, ssw) if want_weight else None), (_with_sumsq(gb, ssb) if want_bias else None)
 
 
 # ---- optimizer: norms, clip factor, clip-weighted sum, noise ---------------------------

@@ -804,6 +804,8 @@ def test_group_norm_grad_sample_f32(K, n, C, G, spatial, scale):
     gw, gb = K.group_norm_grad_sample(dev(x), dev(b), G, 1e-5, scale=scale)
     assert_rel(gw, want_w, FP32_REL, "gn weight")
     assert_rel(gb, want_b, FP32_REL, "gn bias")
+    assert_rel(gw._dpk_sumsq, want_w.pow(2).sum(1), 2e-5, "gn weight sumsq")
+    assert_rel(gb._dpk_sumsq, want_b.pow(2).sum(1), 2e-5, "gn bias sumsq")
 
 
 @pytest.mark.parametrize(
@@ -830,6 +832,8 @@ def test_rms_norm_grad_sample_f32(K, shape, D):
     want = O.rms_norm_grad_sample(x.double(), b.double(), (D,), 1e-6)
     got = K.rms_norm_grad_sample(dev(x), dev(b), D, 1e-6)
     assert_rel(got, want, FP32_REL, "rms weight")
+    # the per-sample sum of squares the kernel leaves for the optimizer's norm pass
+    assert_rel(got._dpk_sumsq, want.flatten(1).pow(2).sum(1), 2e-5, "rms weight sumsq")
 
 
 @pytest.mark.parametrize(
@@ -853,6 +857,8 @@ def test_layer_norm_grad_sample_f32(K, shape, D, scale):
     nshape = shape[-2:] if D == 24 else shape[-1:]
     want_w, want_b = O.layer_norm_grad_sample(x.double(), (b * scale).double(), nshape, 1e-5)
     gw, gb = K.layer_norm_grad_sample(dev(x), dev(b), D, 1e-5, scale=scale)
+    assert_rel(gw._dpk_sumsq, want_w.flatten(1).pow(2).sum(1), 2e-5, "layer norm weight sumsq")
+    assert_rel(gb._dpk_sumsq, want_b.flatten(1).pow(2).sum(1), 2e-5, "layer norm bias sumsq")
     assert_rel(gw, want_w.reshape(shape[0], D), FP32_REL, "ln weight")
     assert_rel(gb, want_b.reshape(shape[0], D), FP32_REL, "ln bias")
     only_w, none_b = K.layer_norm_grad_sample(dev(x), dev(b), D, 1e-5, scale=scale, want_bias=False)
