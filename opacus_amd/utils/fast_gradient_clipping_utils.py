@@ -19,10 +19,10 @@ def first_pass_backward(module, reduced: torch.Tensor, retain_graph: bool = True
     leaves = getattr(module, "first_backward_inputs", None)
     inputs = leaves() if callable(leaves) else None
     if isinstance(inputs, (list, tuple)) and len(inputs) > 0:
-        reduced.backward(retain_graph=retain_graph, inputs=list(inputs))
-        for t in inputs:
-            if not t.is_leaf:
-                t.grad = None  # an activation's gradient: the hooks have seen it, nobody else needs it
+        # autograd.grad rather than backward(inputs=...): the gradients of these tensors are only
+        # wanted by the hooks on the way, and backward() would clone each of them into ``.grad``
+        # (for an activation at the start of a large model that is a copy of hundreds of MB)
+        torch.autograd.grad(reduced, list(inputs), retain_graph=retain_graph, allow_unused=True)
     else:
         reduced.backward(retain_graph=retain_graph)
 
