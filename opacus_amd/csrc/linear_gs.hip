@@ -224,6 +224,9 @@ struct TrBf16 {
   template <class C, class... A> static __device__ __forceinline__ void mainloop(A&&... args) {
     mb16t::mainloop<C>(static_cast<A&&>(args)...);
   }
+  template <class C, class... A> static __device__ __forceinline__ void mainloop_weighted(A&&... args) {
+    mb16t::mainloop<C, true>(static_cast<A&&>(args)...);
+  }
 };
 struct DldsF32 {
   typedef float elem;
@@ -234,11 +237,17 @@ struct DldsF32 {
   }
 };
 
-template <class E, class C, typename TOUT>
-__global__ __launch_bounds__(C::kThreads) void linear_dlds_kernel(
+//
+// W (bf16 engine only): a "sample" of the launch is a run of T / unit_rows units of unit_rows
+// rows each (unit_rows a multiple of the k tile), and unit u of sample s counts
+// coef[s * (T / unit_rows) + u] times: gs[s] = scale * sum_u coef[..] * b_u^T a_u.
+// (Two waves per SIMD asked for, which these kernels reach anyway, caps W at 256 registers: the
+// accumulators then live in ordinary registers, where they can be multiplied in place.)
+template <class E, class C, typename TOUT, bool W = false>
+__global__ __launch_bounds__(C::kThreads, W ? 2 : 1) void linear_dlds_kernel(
     const typename E::elem* __restrict__ b, const typename E::elem* __restrict__ a, TOUT* __restrict__ gs,
     float* __restrict__ partials, int64_t T, int64_t M, int64_t N, float scale, int64_t tiles_m,
-    int64_t tiles_n) {
+    int64_t tiles_n, const float* __restrict__ coef = nullptr, int64_t unit_rows = 0) {
   typedef typename E::template Smem<C> SmemT;
   __shared__ SmemT sm;
   __shared__ float red[C::kWaves];
@@ -258,7 +267,11 @@ __global__ __launch_bounds__(C::kThreads) void linear_dlds_kernel(
   const int wj0 = (wave / C::WQ) * (32 * C::TP), wi0 = (wave % C::WQ) * (32 * C::TQ);  // this wave's corner
   typename E::template Tile<C> tile;
   tile.clear();
-  E::template mainloop<C>(tile, sm, a + sample * T * N, N, n0, b + sample * T * M, M, m0, T, wj0, wi0);
+  if constexpr (W)
+    E::template mainloop_weighted<C>(tile, sm, a + sample * T * N, N, n0, b + sample * T * M, M, m0, T, wj0, wi0,
+                                     coef + sample * (T / unit_rows), unit_rows / mb16t::BK);
+  else
+    E::template mainloop<C>(tile, sm, a + sample * T * N, N, n0, b + sample * T * M, M, m0, T, wj0, wi0);
   TOUT* out = gs + sample * M * N;
   const int kk = lane >> 5, l32 = lane & 31;
   float ss = 0.f;
@@ -661,6 +674,48 @@ extern "C" int dpk_linear_gs(const void* b, const void* a, int in_dtype, void* g
     dpk_launch_reduce_rows(partials, n, p.tiles_m * p.tiles_n, sumsq, 0, 1.f, s);
     DPK_LAUNCH_CHECK(who);
   }
+  return DPK_OK;
+}
+
+// out[p] = scale * sum over the samples s of piece p of coef[s] * b[s]^T a[s]: the clip-weighted
+// sum of a Linear layer's per-sample gradients, contracted over samples and positions at once
+// (piece p holds samples p * n / pieces .. + n / pieces - 1; the caller adds the pieces).
+extern "C" int dpk_linear_weighted_sum(const void* b, const void* a, int in_dtype, const float* coef, void* out_sum,
+                                       int out_dtype, int64_t n, int64_t T, int64_t out, int64_t in, float scale,
+                                       int pieces, dpk_stream_t stream) {
+  const char* who = "dpk_linear_weighted_sum";
+  DPK_REQUIRE(n >= 1 && T >= 1 && out >= 1 && in >= 1 && pieces >= 1, DPK_E_SHAPE,
+              "%s: n=%lld T=%lld out=%lld in=%lld pieces=%d", who, (long long)n, (long long)T, (long long)out,
+              (long long)in, pieces);
+  DPK_REQUIRE(b && a && coef && out_sum, DPK_E_ARG, "%s: NULL tensor", who);
+  DPK_REQUIRE(in_dtype == DPK_BF16 && dpk_dtype_ok(out_dtype), DPK_E_DTYPE, "%s: dtypes %d,%d (bf16 input only)", who,
+              in_dtype, out_dtype);
+  DPK_REQUIRE(T % mb16t::BK == 0 && n % pieces == 0, DPK_E_SHAPE,
+              "%s: T=%lld must be a multiple of %d and n=%lld of pieces=%d", who, (long long)T, mb16t::BK,
+              (long long)n, pieces);
+  DPK_REQUIRE(dpk_aligned(coef, 4), DPK_E_ALIGN, "%s: misaligned coefficients", who);
+  const int64_t rows = (n / pieces) * T;
+  Plan p = make_plan(rows, out, in, true);
+  plan_tr(p, b, a, out_sum, pieces, rows, out, in, dpk_device_cus(), DPK_TILE_AUTO);
+  DPK_REQUIRE(p.tr != 0, DPK_E_SHAPE,
+              "%s: out=%lld and in=%lld must be multiples of 8 above 64 and the tensors 16-byte aligned", who, (long long)out,
+              (long long)in);
+  const int64_t blocks = pieces * p.tiles_m * p.tiles_n;
+  DPK_REQUIRE(blocks <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: %lld blocks exceed the grid limit", who, (long long)blocks);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid(static_cast<unsigned>(blocks));
+  const bf16_t* bp = static_cast<const bf16_t*>(b);
+  const bf16_t* ap = static_cast<const bf16_t*>(a);
+  float* none = nullptr;
+#define DPK_WSUM(CFG, TOUT)                                                                                    \
+  hipLaunchKernelGGL((linear_dlds_kernel<TrBf16, CFG, TOUT, true>), grid, dim3(CFG::kThreads), 0, s, bp, ap, \
+                     static_cast<TOUT*>(out_sum), none, rows, out, in, scale, p.tiles_m, p.tiles_n, coef, T)
+  if (p.tr == 256 && out_dtype == DPK_BF16) DPK_WSUM(TrLarge, bf16_t);
+  else if (p.tr == 256) DPK_WSUM(TrLarge, float);
+  else if (out_dtype == DPK_BF16) DPK_WSUM(TrSmall, bf16_t);
+  else DPK_WSUM(TrSmall, float);
+#undef DPK_WSUM
+  DPK_LAUNCH_CHECK(who);
   return DPK_OK;
 }
 

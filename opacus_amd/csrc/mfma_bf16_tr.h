@@ -141,18 +141,37 @@ struct Tile {
         for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
   }
 
+  __device__ __forceinline__ void scale(float f) {
+#pragma unroll
+    for (int i = 0; i < C::TP; ++i)
+#pragma unroll
+      for (int j = 0; j < C::TQ; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] *= f;
+  }
+
   // The MFMAs of the tile in `cur`, with the LDS reads of the next tile (into `nxt`) and
   // the global -> LDS loads of a later one (issue(q), q < kLoads) dealt out evenly between
   // them: a wave issues in order, so reads queued in one burst would hold its MFMAs back for
   // as long as the LDS takes to accept them.
-  template <class IssueFn>
+  //
+  // kRescale: every 32 x 32 piece of the accumulator is multiplied by f just before the first
+  // MFMA that adds to it, so that the multiplications of one piece run under the MFMA of the
+  // piece before.
+  template <bool kRescale = false, class IssueFn>
   __device__ __forceinline__ void mma(const Frags<C>& cur, Frags<C>& nxt, const unsigned char* Ps,
                                       const unsigned char* Qs, const uint32_t (&fp)[C::TP],
-                                      const uint32_t (&fq)[C::TQ], IssueFn issue) {
+                                      const uint32_t (&fq)[C::TQ], IssueFn issue, float f = 1.f) {
     constexpr int KS = Frags<C>::KS, M = KS * C::TP * C::TQ, R = Frags<C>::kReads, L = C::kLoads;
 #pragma unroll
     for (int m = 0; m < M; ++m) {
       const int s = m / (C::TP * C::TQ), i = (m / C::TQ) % C::TP, j = m % C::TQ;
+      if constexpr (kRescale) {
+        if (s == 0) {
+#pragma unroll
+          for (int v = 0; v < 16; ++v) acc[i][j][v] *= f;
+        }
+      }
       acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur.operand_p(s, i), cur.operand_q(s, j), acc[i][j], 0, 0, 0);
 #pragma unroll
       for (int r = m * R / M; r < (m + 1) * R / M; ++r) nxt.read(r, Ps, Qs, fp, fq);
@@ -171,12 +190,32 @@ struct Tile {
 // from memory. Tile kt lives in stage kt % NS, which is refilled as soon as every wave holds
 // tile kt in registers. Every step issues exactly one tile's loads (past the end the last
 // tile again), so kLoads * (NS - 2) loads may stay in flight while a tile is awaited.
-template <class C>
+//
+// kWeighted: the K rows are units of tiles_per_unit k tiles each (K a whole number of them)
+// and unit u counts coef[u] times: acc = sum_u coef[u] * (P_u^T Q_u). The accumulator is kept
+// in units of the current unit's coefficient: at a unit's first tile it is rescaled by
+// coef[u - 1] / coef[u], and by the last coefficient at the end. What it holds is then at most
+// (sum of the weighted terms so far) / coef[u], so it overflows only where the unit's own
+// unweighted product nearly does. A coefficient below kMinCoef counts as kMinCoef (an exact
+// zero would turn the rescaling into a division by zero); a NaN stays a NaN.
+constexpr float kMinCoef = 1e-30f;
+__device__ __forceinline__ float at_least_min_coef(float c) { return c < kMinCoef ? kMinCoef : c; }
+
+template <class C, bool kWeighted = false>
 __device__ __forceinline__ void mainloop(Tile<C>& t, Smem<C>& sm, const bf16_t* P, int64_t ldp, int64_t p0,
                                          const bf16_t* Q, int64_t ldq, int64_t q0, int64_t K, int wp0,
-                                         int wq0) {
+                                         int wq0, const float* coef = nullptr, int64_t tiles_per_unit = 0) {
   constexpr int NS = C::NS;
   const int64_t nk = (K + BK - 1) / BK;
+  int64_t boundary = 0, unit = 0, units = 0;
+  float c_cur = 1.f, c_nxt = 1.f;
+  if constexpr (kWeighted) {
+    units = nk / tiles_per_unit;
+    boundary = tiles_per_unit;
+    // (read one unit ahead and not looked at before its unit begins: nothing waits for the load)
+    c_cur = at_least_min_coef(coef[0]);
+    c_nxt = coef[units > 1 ? 1 : 0];
+  }
   const int dup = static_cast<int>(nk * BK - K);  // rows the last tile repeats
   const uint32_t lds0 = lds_offset(&sm.stage[0][0]);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -237,6 +276,25 @@ __device__ __forceinline__ void mainloop(Tile<C>& t, Smem<C>& sm, const bf16_t* 
     wait_and_barrier<C::kLoads*(NS - 2)>();
     zero_repeated_rows(kt + 1);
     const unsigned char* st = sm.stage[(kt + 1) & (NS - 1)];
+    if constexpr (kWeighted) {
+      if (kt == boundary) {  // first tile of the next unit (uniform over the block)
+        const float c_new = at_least_min_coef(c_nxt);
+        const float ratio = c_cur / c_new;
+        c_cur = c_new;
+        ++unit;
+        boundary += tiles_per_unit;
+        c_nxt = coef[unit + 1 < units ? unit + 1 : units - 1];
+        // a wave with a small accumulator has the registers to spare for a second copy of the
+        // step with the multiplications dealt out between its MFMAs; a large one (a long step:
+        // the multiplications are a small part of a unit) rescales first
+        if constexpr (C::TP * C::TQ <= 4) {
+          t.template mma<true>(cur, nxt, st, st + C::SUBP * SUB_BYTES, fp, fq, [&](int q) { issue_q(kt + NS, q); }, ratio);
+          return;
+        } else {
+          t.scale(ratio);
+        }
+      }
+    }
     t.mma(cur, nxt, st, st + C::SUBP * SUB_BYTES, fp, fq, [&](int q) { issue_q(kt + NS, q); });
   };
   int64_t kt = 0;
@@ -247,6 +305,7 @@ __device__ __forceinline__ void mainloop(Tile<C>& t, Smem<C>& sm, const bf16_t* 
   if (kt < nk) step(kt, f0, f1);
   __builtin_amdgcn_s_waitcnt(kWaitLgkm0);
   wait_and_barrier<0>();  // the stage memory is the caller's again
+  if constexpr (kWeighted) t.scale(c_cur);
 }
 
 }  // namespace mb16t

@@ -385,6 +385,14 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
                 continue
             if self._sampler_for(module) is linear_grad_sampler:  # nn.Linear itself and RNNLinear, not a subclass with a forward of its own
                 a = activations[0].to(backprops.dtype)
+                if kernels.linear_weighted_sum_takes(backprops, a):
+                    # the coefficients go onto the accumulators of one contraction over all samples
+                    # and positions: neither operand is weighted (or even copied) beforehand
+                    add(module.weight, kernels.linear_weighted_sum(backprops, a, c, scale=scale))
+                    if module.bias is not None:
+                        per_sample = backprops.sum(dim=tuple(range(1, backprops.dim() - 1)), dtype=torch.float32)
+                        add(module.bias, ((c * scale) @ per_sample).to(backprops.dtype))
+                    continue
                 w = (c * scale).to(backprops.dtype).view(n, *([1] * (backprops.dim() - 1)))
                 if module.bias is None and a.shape[-1] < backprops.shape[-1]:
                     # (coef * b)^T a == b^T (coef * a): weight the narrower of the two

@@ -155,6 +155,59 @@ def linear_grad_sample(
     return gs, sumsq
 
 
+def linear_weighted_sum_takes(backprops: torch.Tensor, activations: torch.Tensor) -> bool:
+    """Whether :func:`linear_weighted_sum` takes the pair (the shapes ``dpk_linear_weighted_sum``
+    accepts): bf16 on the GPU, whole k tiles of 32 positions per sample, feature counts that are
+    multiples of 8 above 64."""
+    if not (backprops.is_cuda and backprops.dtype == torch.bfloat16 and activations.dtype == torch.bfloat16):
+        return False
+    if backprops.dim() < 3 or backprops.shape[0] == 0 or backprops.shape[:-1] != activations.shape[:-1]:
+        return False
+    n, out_f, in_f = backprops.shape[0], backprops.shape[-1], activations.shape[-1]
+    T = backprops.numel() // (n * out_f)
+    return T % 32 == 0 and T >= 32 and out_f % 8 == 0 and in_f % 8 == 0 and out_f > 64 and in_f > 64
+
+
+def linear_weighted_sum(
+    backprops: torch.Tensor,
+    activations: torch.Tensor,
+    coef: torch.Tensor,
+    scale: float = 1.0,
+    pieces: Optional[int] = None,
+    out_dtype: Optional[torch.dtype] = None,
+) -> torch.Tensor:
+    """``sum_n coef[n] * scale * b[n]^T a[n]`` as ``[out, in]``: the clip-weighted sum of a Linear
+    layer's per-sample gradients in one contraction over samples and positions, the weights
+    applied to the accumulators where a sample begins. ``pieces`` cuts the samples into that
+    many runs whose fp32 partial sums are added afterwards (default: 4 for a layer with at most
+    256 output tiles of 128 x 128, which alone would not fill the GPU twice over, when n allows;
+    else 1)."""
+    dev = _need_gpu(backprops, activations, coef)
+    n, out_f, in_f = backprops.shape[0], backprops.shape[-1], activations.shape[-1]
+    b = _dense(backprops).reshape(n, -1, out_f)
+    a = _dense(activations).reshape(n, -1, in_f)
+    T = b.shape[1]
+    if a.shape[1] != T:
+        raise ValueError(f"activations {tuple(activations.shape)} and backprops {tuple(backprops.shape)} disagree")
+    c = _dense(coef.to(torch.float32)).reshape(-1)
+    if c.numel() != n:
+        raise ValueError(f"{c.numel()} coefficients for {n} samples")
+    if pieces is None:
+        few_tiles = -(-out_f // 128) * -(-in_f // 128) <= 256
+        pieces = 4 if few_tiles and n % 4 == 0 else 1
+    out_dtype = out_dtype or backprops.dtype
+    part = torch.empty((pieces, out_f, in_f), dtype=out_dtype if pieces == 1 else torch.float32, device=dev)
+    with _timed("linear_weighted_sum", dev):
+        check(
+            "dpk_linear_weighted_sum",
+            lib().dpk_linear_weighted_sum(
+                _ptr(b), _ptr(a), _code(b), _ptr(c), _ptr(part), _code(part), n, T, out_f, in_f, float(scale),
+                int(pieces), _stream(dev),
+            ),
+        )
+    return part[0] if pieces == 1 else part.sum(0).to(out_dtype)
+
+
 def _with_sumsq(gs: torch.Tensor, sumsq: torch.Tensor) -> torch.Tensor:
     """Leaves the per-sample sum of squares on the tensor it describes, with the tensor's
     version, so that the optimizer's norm pass can use it while nobody has written to ``gs``."""

@@ -469,6 +469,57 @@ def test_linear_ghost_norm_multi_many_layers(K, count):
             assert_rel(nb, ob, 1e-4, f"bias norm of layer {k}")
 
 
+WEIGHTED_SUM_CASES = [
+    # (n, T, in, out, pieces)
+    (8, 32, 128, 128, 1),  # one k tile per sample: a rescaling before every tile
+    (8, 64, 512, 256, 4),
+    (16, 128, 256, 512, None),  # the wrapper's own choice of pieces
+    (6, 96, 72, 136, 2),  # ragged block tiles, three k tiles per sample
+    (4, 256, 1024, 1024, 1),
+    (3, 32, 2048, 2048, 1),  # enough output tiles for the 256-wide block tile
+]
+
+
+@pytest.mark.parametrize("n,T,fin,fout,pieces", WEIGHTED_SUM_CASES)
+@pytest.mark.parametrize("coefs", ["spread", "equal", "tiny_and_zero"])
+@pytest.mark.parametrize("out_f32", [False, True])
+def test_linear_weighted_sum(K, n, T, fin, fout, pieces, coefs, out_f32):
+    """sum_n coef[n] * b[n]^T a[n] with the coefficients applied to the accumulators, against the
+    oracle's per-sample gradients weighted and added in fp64."""
+    torch.manual_seed(n * 100 + T + fin)
+    a = torch.randn(n, T, fin).bfloat16()
+    b = (torch.randn(n, T, fout) * 0.1).bfloat16()
+    if coefs == "spread":
+        c = torch.rand(n) * 0.99 + 0.01
+    elif coefs == "equal":
+        c = torch.full((n,), 0.37)
+    else:  # coefficients twelve orders of magnitude apart and an exact zero, at either end too
+        c = torch.rand(n) * 0.9 + 0.1
+        c[0], c[n // 2], c[-1] = 1e-12, 0.0, 3e-9
+    gs, _ = O.linear_grad_sample(a.double(), b.double())
+    want = (c.double().view(n, 1, 1) * gs.double()).sum(0) * 2.0
+    got = K.linear_weighted_sum(
+        dev(b), dev(a), dev(c), scale=2.0, pieces=pieces, out_dtype=torch.float32 if out_f32 else None
+    )
+    assert got.shape == (fout, fin) and got.dtype == (torch.float32 if out_f32 else torch.bfloat16)
+    # bf16 inputs are exact and accumulation is fp32; a bf16 result is rounded once
+    assert_rel(got[None], want[None], 1e-4 if out_f32 else BF16_REL, "weighted sum")
+
+
+def test_linear_weighted_sum_keeps_a_nan_and_refuses_other_shapes(K):
+    torch.manual_seed(5)
+    a, b = dev(torch.randn(4, 32, 128).bfloat16()), dev(torch.randn(4, 32, 128).bfloat16())
+    c = torch.tensor([0.5, float("nan"), 0.25, 1.0])
+    assert torch.isnan(K.linear_weighted_sum(b, a, dev(c))).all()
+    assert not K.linear_weighted_sum_takes(b[:, :16], a[:, :16])  # half a k tile per sample
+    assert not K.linear_weighted_sum_takes(b.float(), a.float())
+    assert not K.linear_weighted_sum_takes(b[..., :64], a)
+    with pytest.raises(RuntimeError, match="dpk_linear_weighted_sum"):
+        K.linear_weighted_sum(b[:, :16].contiguous(), a[:, :16].contiguous(), dev(c))
+    with pytest.raises(RuntimeError, match="dpk_linear_weighted_sum"):
+        K.linear_weighted_sum(b, a, dev(c), pieces=3)
+
+
 def test_linear_ghost_norm_2d_inputs(K):
     torch.manual_seed(21)
     a, b = torch.randn(6, 50), torch.randn(6, 30)
