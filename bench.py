@@ -14,7 +14,9 @@ timed on this box's host cores on a bounded sample of the same workload.
 The headline fields are config 2's. The same run then times the other four benchmark
 configurations (c1, c3, c4, c5: full DP-SGD steps through the drop-in API, at most 20
 steps each, 5 for c5) and reports them under ``"configs"``, each with its own
-``ms_per_step``, ``samples_per_s``, ``roofline`` and bounded-sample ``cpu_baseline``.
+``ms_per_step``, ``samples_per_s``, ``roofline`` and bounded-sample ``cpu_baseline``
+(c5 also with embedding table and LM head tied, which the reference refuses under ghost
+clipping, as ``tied_embeddings``).
 ``--workload cN`` times one configuration alone (same JSON shape, no ``configs``);
 ``--headline-only`` skips the other four. ``--kernels`` times each kernel of the library on
 its own at those shapes and prints one JSON line per kernel (time, algorithmic work,
@@ -848,6 +850,10 @@ def main() -> None:
                 d = run_workload(name + "p", dev, k, wu, args.all_kernel_timers)
                 entry["two_backward_passes"] = {"ms_per_step": d["ms_per_step"], "samples_per_s": d["samples_per_s"],
                                                 "single_backward": False}
+            if name + "t" in WORKLOADS:  # the same decoder with embedding table and LM head sharing one parameter
+                d = run_workload(name + "t", dev, k, wu, args.all_kernel_timers)
+                entry["tied_embeddings"] = {"ms_per_step": d["ms_per_step"], "samples_per_s": d["samples_per_s"],
+                                            "workload": d["workload"]}
             if name + "d" in WORKLOADS:  # the same configuration with the library's default hooks
                 d = run_workload(name + "d", dev, k, wu, args.all_kernel_timers)
                 entry["default_hooks"] = {"ms_per_step": d["ms_per_step"], "samples_per_s": d["samples_per_s"],

@@ -82,22 +82,25 @@ int dpk_linear_gs(const void* b, const void* a, int in_dtype, void* gs, int gs_d
                   float* sumsq, int64_t n, int64_t T, int64_t out, int64_t in, float scale,
                   int tile, void* ws, size_t ws_bytes, dpk_stream_t stream);
 
-/* out[p,i,j] = scale * sum_{s in piece p} coef[s] * sum_t b[s,t,i] * a[s,t,j]
+/* out[i,j] = scale * sum_s coef[s] * sum_t b[s,t,i] * a[s,t,j]
  * The clip-weighted sum of a Linear layer's per-sample gradients from the activations and
  * backprops of one backward pass: what the reference's second backward pass of
  * sum_s coef[s] * loss[s] leaves in weight.grad (utils/fast_gradient_clipping_utils.py:193-201,
  * DPTensorFastGradientClipping.backward), without that pass and without a weighted copy of
- * either operand. b: [n,T,out], a: [n,T,in], bf16; coef: float[n]; out: [pieces,out,in] of
- * `out_dtype`. Piece p covers samples p*n/pieces .. (p+1)*n/pieces-1 and the caller adds the
- * pieces (more pieces fill the GPU for a layer with few output tiles). One contraction over
- * samples and positions at once: the accumulators are rescaled by coef[s-1]/coef[s] where
- * sample s begins, so no per-sample product is stored anywhere. A coefficient below 1e-30
- * counts as 1e-30. Requires T % 32 == 0, n % pieces == 0, out and in multiples of 8 above 64,
- * 16-byte aligned tensors; anything else is refused with DPK_E_SHAPE (the caller then weights
- * an operand itself and calls dpk_linear_gs on one "sample" of n*T rows). */
+ * either operand. b: [n,T,out], a: [n,T,in], bf16; coef: float[n]; out: [out,in] of `out_dtype`.
+ * One contraction over samples and positions at once: the accumulators are rescaled by
+ * coef[s-1]/coef[s] where sample s begins, so no per-sample product is stored anywhere. A
+ * coefficient below 1e-30 counts as 1e-30. pieces > 1 cuts the samples into that many runs
+ * (more blocks for a layer with few output tiles) whose fp32 sums go through the workspace
+ * (dpk_linear_weighted_sum_workspace_bytes) and are added by a second kernel.
+ * Requires T % 32 == 0, n % pieces == 0, out and in multiples of 8 above 64, 16-byte aligned
+ * tensors; anything else is refused with DPK_E_SHAPE (the caller then weights an operand itself
+ * and calls dpk_linear_gs on one "sample" of n*T rows). */
+size_t dpk_linear_weighted_sum_workspace_bytes(int64_t out_features, int64_t in_features, int pieces);
 int dpk_linear_weighted_sum(const void* b, const void* a, int in_dtype, const float* coef, void* out,
                             int out_dtype, int64_t n, int64_t T, int64_t out_features,
-                            int64_t in_features, float scale, int pieces, dpk_stream_t stream);
+                            int64_t in_features, float scale, int pieces, void* ws, size_t ws_bytes,
+                            dpk_stream_t stream);
 
 /* gs_bias[n,k] = scale * sum_t b[n,t,k]                   (linear.py:50)
  * sumsq (nullable, float[n]) receives sum_k gs_bias[n,k]^2 of the values as stored, for

@@ -53,7 +53,10 @@ SIGNATURES = {
     "dpk_device_cus": (c_int, []),
     "dpk_linear_gs_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
     "dpk_linear_gs": (c_int, [_P, _P, c_int, _P, c_int, _P, _I, _I, _I, _I, c_float, c_int, _P, c_size_t, _P]),
-    "dpk_linear_weighted_sum": (c_int, [_P, _P, c_int, _P, _P, c_int, _I, _I, _I, _I, c_float, c_int, _P]),
+    "dpk_linear_weighted_sum_workspace_bytes": (c_size_t, [_I, _I, c_int]),
+    "dpk_linear_weighted_sum": (
+        c_int, [_P, _P, c_int, _P, _P, c_int, _I, _I, _I, _I, c_float, c_int, _P, c_size_t, _P]
+    ),
     "dpk_linear_bias_gs": (c_int, [_P, c_int, _P, c_int, _P, _I, _I, _I, c_float, _P]),
     "dpk_linear_ghost_norm_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
     "dpk_linear_ghost_norm": (c_int, [_P, _P, c_int, _P, _P, _I, _I, _I, _I, c_float, c_int, _P, c_size_t, _P]),

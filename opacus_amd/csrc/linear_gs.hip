@@ -601,6 +601,20 @@ void launch_linear(const Plan& p, bool vec, const void* b, const void* a, void* 
   }
 }
 
+// out[e] = sum_p part[p * count + e], four elements per thread (count % 4 == 0).
+template <typename TOUT>
+__global__ __launch_bounds__(kThreads) void add_pieces_kernel(const float* __restrict__ part, TOUT* __restrict__ out,
+                                                            int64_t count4, int pieces) {
+  const int64_t e = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (e >= count4) return;
+  typedef float vf4 __attribute__((ext_vector_type(4)));
+  const vf4* src = reinterpret_cast<const vf4*>(part) + e;
+  vf4 sum = __builtin_nontemporal_load(src);
+  for (int p = 1; p < pieces; ++p) sum += __builtin_nontemporal_load(src + p * count4);
+  const float4 acc = make_float4(sum.x, sum.y, sum.z, sum.w);
+  dpk_io<TOUT>::store4(out + 4 * e, acc);
+}
+
 bool linear_vec(const void* b, const void* a, const void* gs, int in_dtype, int gs_dtype, int64_t M,
                 int64_t N) {
   const size_t ia = in_dtype == DPK_BF16 ? 8 : 16, oa = gs_dtype == DPK_BF16 ? 8 : 16;
@@ -677,12 +691,18 @@ extern "C" int dpk_linear_gs(const void* b, const void* a, int in_dtype, void* g
   return DPK_OK;
 }
 
-// out[p] = scale * sum over the samples s of piece p of coef[s] * b[s]^T a[s]: the clip-weighted
-// sum of a Linear layer's per-sample gradients, contracted over samples and positions at once
-// (piece p holds samples p * n / pieces .. + n / pieces - 1; the caller adds the pieces).
+extern "C" size_t dpk_linear_weighted_sum_workspace_bytes(int64_t out, int64_t in, int pieces) {
+  if (out <= 0 || in <= 0 || pieces <= 1) return 0;
+  return dpk_align_up(static_cast<size_t>(pieces) * out * in * sizeof(float), 256);
+}
+
+// out_sum = scale * sum_s coef[s] * b[s]^T a[s]: the clip-weighted sum of a Linear layer's
+// per-sample gradients, contracted over samples and positions at once. With pieces > 1 piece p
+// (samples p * n / pieces .. + n / pieces - 1) leaves its fp32 sum in the workspace and a
+// second kernel adds the pieces into out_sum.
 extern "C" int dpk_linear_weighted_sum(const void* b, const void* a, int in_dtype, const float* coef, void* out_sum,
                                        int out_dtype, int64_t n, int64_t T, int64_t out, int64_t in, float scale,
-                                       int pieces, dpk_stream_t stream) {
+                                       int pieces, void* ws, size_t ws_bytes, dpk_stream_t stream) {
   const char* who = "dpk_linear_weighted_sum";
   DPK_REQUIRE(n >= 1 && T >= 1 && out >= 1 && in >= 1 && pieces >= 1, DPK_E_SHAPE,
               "%s: n=%lld T=%lld out=%lld in=%lld pieces=%d", who, (long long)n, (long long)T, (long long)out,
@@ -694,14 +714,24 @@ extern "C" int dpk_linear_weighted_sum(const void* b, const void* a, int in_dtyp
               "%s: T=%lld must be a multiple of %d and n=%lld of pieces=%d", who, (long long)T, mb16t::BK,
               (long long)n, pieces);
   DPK_REQUIRE(dpk_aligned(coef, 4), DPK_E_ALIGN, "%s: misaligned coefficients", who);
+  const bool split = pieces > 1;
+  if (split) {
+    const size_t need = static_cast<size_t>(pieces) * out * in * sizeof(float);
+    DPK_REQUIRE(ws && ws_bytes >= need, DPK_E_WORKSPACE, "%s: workspace %zu < %zu bytes", who, ws_bytes, need);
+    DPK_REQUIRE(dpk_aligned(ws, 16), DPK_E_ALIGN, "%s: workspace misaligned", who);
+  }
+  void* dst = split ? ws : out_sum;
+  const int dst_dtype = split ? DPK_F32 : out_dtype;
   const int64_t rows = (n / pieces) * T;
   Plan p = make_plan(rows, out, in, true);
   plan_tr(p, b, a, out_sum, pieces, rows, out, in, dpk_device_cus(), DPK_TILE_AUTO);
   DPK_REQUIRE(p.tr != 0, DPK_E_SHAPE,
-              "%s: out=%lld and in=%lld must be multiples of 8 above 64 and the tensors 16-byte aligned", who, (long long)out,
-              (long long)in);
+              "%s: out=%lld and in=%lld must be multiples of 8 above 64 and the tensors 16-byte aligned", who,
+              (long long)out, (long long)in);
   const int64_t blocks = pieces * p.tiles_m * p.tiles_n;
-  DPK_REQUIRE(blocks <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: %lld blocks exceed the grid limit", who, (long long)blocks);
+  const int64_t count4 = out * in / 4;  // out, in multiples of 8
+  DPK_REQUIRE(blocks <= DPK_MAX_GRID_X && dpk_cdiv(count4, kThreads) <= DPK_MAX_GRID_X, DPK_E_SHAPE,
+              "%s: %lld blocks exceed the grid limit", who, (long long)blocks);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 grid(static_cast<unsigned>(blocks));
   const bf16_t* bp = static_cast<const bf16_t*>(b);
@@ -709,13 +739,23 @@ extern "C" int dpk_linear_weighted_sum(const void* b, const void* a, int in_dtyp
   float* none = nullptr;
 #define DPK_WSUM(CFG, TOUT)                                                                                    \
   hipLaunchKernelGGL((linear_dlds_kernel<TrBf16, CFG, TOUT, true>), grid, dim3(CFG::kThreads), 0, s, bp, ap, \
-                     static_cast<TOUT*>(out_sum), none, rows, out, in, scale, p.tiles_m, p.tiles_n, coef, T)
-  if (p.tr == 256 && out_dtype == DPK_BF16) DPK_WSUM(TrLarge, bf16_t);
+                     static_cast<TOUT*>(dst), none, rows, out, in, scale, p.tiles_m, p.tiles_n, coef, T)
+  if (p.tr == 256 && dst_dtype == DPK_BF16) DPK_WSUM(TrLarge, bf16_t);
   else if (p.tr == 256) DPK_WSUM(TrLarge, float);
-  else if (out_dtype == DPK_BF16) DPK_WSUM(TrSmall, bf16_t);
+  else if (dst_dtype == DPK_BF16) DPK_WSUM(TrSmall, bf16_t);
   else DPK_WSUM(TrSmall, float);
 #undef DPK_WSUM
   DPK_LAUNCH_CHECK(who);
+  if (split) {
+    const dim3 g2(static_cast<unsigned>(dpk_cdiv(count4, kThreads)));
+    if (out_dtype == DPK_BF16)
+      hipLaunchKernelGGL(add_pieces_kernel<bf16_t>, g2, dim3(kThreads), 0, s, static_cast<const float*>(ws),
+                         static_cast<bf16_t*>(out_sum), count4, pieces);
+    else
+      hipLaunchKernelGGL(add_pieces_kernel<float>, g2, dim3(kThreads), 0, s, static_cast<const float*>(ws),
+                         static_cast<float*>(out_sum), count4, pieces);
+    DPK_LAUNCH_CHECK(who);
+  }
   return DPK_OK;
 }
 

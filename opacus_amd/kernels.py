@@ -179,7 +179,7 @@ def linear_weighted_sum(
     """``sum_n coef[n] * scale * b[n]^T a[n]`` as ``[out, in]``: the clip-weighted sum of a Linear
     layer's per-sample gradients in one contraction over samples and positions, the weights
     applied to the accumulators where a sample begins. ``pieces`` cuts the samples into that
-    many runs whose fp32 partial sums are added afterwards (default: 4 for a layer with at most
+    many runs whose fp32 sums a second kernel adds (default: 4 for a layer with at most
     256 output tiles of 128 x 128, which alone would not fill the GPU twice over, when n allows;
     else 1)."""
     dev = _need_gpu(backprops, activations, coef)
@@ -195,17 +195,18 @@ def linear_weighted_sum(
     if pieces is None:
         few_tiles = -(-out_f // 128) * -(-in_f // 128) <= 256
         pieces = 4 if few_tiles and n % 4 == 0 else 1
-    out_dtype = out_dtype or backprops.dtype
-    part = torch.empty((pieces, out_f, in_f), dtype=out_dtype if pieces == 1 else torch.float32, device=dev)
+    out = torch.empty((out_f, in_f), dtype=out_dtype or backprops.dtype, device=dev)
+    L = lib()
+    ws, wsb = _ws(L.dpk_linear_weighted_sum_workspace_bytes(out_f, in_f, int(pieces)), dev)
     with _timed("linear_weighted_sum", dev):
         check(
             "dpk_linear_weighted_sum",
-            lib().dpk_linear_weighted_sum(
-                _ptr(b), _ptr(a), _code(b), _ptr(c), _ptr(part), _code(part), n, T, out_f, in_f, float(scale),
-                int(pieces), _stream(dev),
+            L.dpk_linear_weighted_sum(
+                _ptr(b), _ptr(a), _code(b), _ptr(c), _ptr(out), _code(out), n, T, out_f, in_f, float(scale),
+                int(pieces), _ptr(ws), wsb, _stream(dev),
             ),
         )
-    return part[0] if pieces == 1 else part.sum(0).to(out_dtype)
+    return out
 
 
 def _with_sumsq(gs: torch.Tensor, sumsq: torch.Tensor) -> torch.Tensor:
