@@ -31,6 +31,8 @@ from ..utils.module_utils import (
     trainable_parameter_list,
     trainable_parameters,
 )
+from .. import kernels
+from ._common import tag_sumsq
 from .functorch import ft_compute_per_sample_gradient, prepare_layer
 from .gsm_base import AbstractGradSampleHooks, AbstractGradSampleModule
 
@@ -50,8 +52,29 @@ def owns_output(fn: Callable) -> Callable:
     return fn
 
 
+def _runs_on_kernels(fn: Callable) -> bool:
+    """This package's own samplers, which work from activations and backprops alone; not the
+    functorch fallback (it runs the layer, whose parameters keep their dtype) or a sampler a
+    user registered (plain torch takes float16 as it is)."""
+    mod = getattr(getattr(fn, "func", fn), "__module__", None) or ""
+    return mod.startswith(__package__ + ".") and not mod.endswith(".functorch")
+
+
 def call_sampler(fn: Callable, module: nn.Module, activations, backprops: torch.Tensor, scale: float):
-    """Calls a grad or norm sampler, folding ``scale`` into it if it can take it."""
+    """Calls a grad or norm sampler, folding ``scale`` into it if it can take it.
+
+    float16 backprops (the reference's low-precision tests cover them beside bfloat16,
+    tests/mixed_precision_test.py:240-242) have no kernels of their own: they and the activations
+    are widened to float32, which is exact, the sampler runs on the float32 kernels, and
+    per-sample gradients come back as float16 with their float32 sums of squares still attached
+    (per-sample norms stay float32, as for bfloat16)."""
+    if backprops.dtype is torch.float16 and backprops.is_cuda and _runs_on_kernels(fn):
+        wide = [kernels.widen(a) for a in activations]
+        out = call_sampler(fn, module, wide, backprops.float(), scale)
+        return {
+            p: tag_sumsq(v.half(), getattr(v, "_dpk_sumsq", None)) if v.dtype is torch.float32 and v.dim() > 1 else v
+            for p, v in out.items()
+        }
     if getattr(fn, "accepts_scale", False):
         return fn(module, activations, backprops, scale=scale)
     if scale != 1.0:

@@ -212,7 +212,7 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
             or self.NORM_SAMPLERS.get(type(module)) is not compute_linear_norm_sample
             or backprops.shape[0] == 0
             or not backprops.is_cuda
-            or not kernels.supported_dtype(backprops.dtype)
+            or not kernels.native_dtype(backprops.dtype)  # float16 goes through call_sampler, widened
         ):
             return None
         n, dev = backprops.shape[0], backprops.device

@@ -22,7 +22,30 @@ _DTYPES = {torch.float32: DPK_F32, torch.bfloat16: DPK_BF16}
 
 
 def supported_dtype(dtype: torch.dtype) -> bool:
+    """float32 and bfloat16 have kernels of their own; float16 tensors are widened to float32 on
+    the way in (exact) and results narrowed on the way out (:func:`widen`, the optimizer wrappers
+    below, ``grad_sample_module.call_sampler``)."""
+    return dtype in _DTYPES or dtype is torch.float16
+
+
+def native_dtype(dtype: torch.dtype) -> bool:
+    """Whether the kernels read and write the dtype directly (float32, bfloat16)."""
     return dtype in _DTYPES
+
+
+def widen(t):
+    """float16 -> float32 (every float16 value is a float32 value); anything else as it is."""
+    return t.float() if isinstance(t, torch.Tensor) and t.dtype is torch.float16 else t
+
+
+def _any_half(*lists) -> bool:
+    return any(t is not None and t.dtype is torch.float16 for ts in lists for t in ts)
+
+
+def _narrow_back(targets, wide) -> None:
+    for t, w in zip(targets, wide):
+        if t is not w:
+            t.copy_(w)
 
 
 def _code(t_or_dtype) -> int:
@@ -30,7 +53,7 @@ def _code(t_or_dtype) -> int:
     try:
         return _DTYPES[dt]
     except KeyError:
-        raise TypeError(f"dpk kernels take float32 or bfloat16 tensors, got {dt}") from None
+        raise TypeError(f"dpk kernels take float32 or bfloat16 tensors (float16 through kernels.widen), got {dt}") from None
 
 
 def _need_gpu(*tensors: torch.Tensor) -> torch.device:
@@ -571,6 +594,7 @@ def tied_embedding_cross_term(
     (``ids`` ``[n, ...]``, output backprops ``[n, ..., D]``) and a bias-free or biased Linear
     (inputs ``[n, ..., D]``, output backprops ``[n, ..., V]``), without forming either
     gradient: ``scale * sum_t <e_t, sum_t' g[t', ids_t] a_t'>``."""
+    emb_backprops, head_backprops, head_activations = widen(emb_backprops), widen(head_backprops), widen(head_activations)
     dev = _need_gpu(ids, emb_backprops, head_activations, head_backprops)
     ids2 = _ids_2d(ids)
     n, T = ids2.shape
@@ -747,6 +771,8 @@ def _flat2d(gs: torch.Tensor) -> torch.Tensor:
 
 def sumsq_rows(gs_list: Sequence[torch.Tensor]) -> torch.Tensor:
     """``out[k, i] = sum of squares of sample i of tensor k`` (fp32), one pass over each tensor."""
+    if _any_half(gs_list):
+        gs_list = [widen(g) for g in gs_list]
     dev = _need_gpu(*gs_list)
     K = len(gs_list)
     n = gs_list[0].shape[0]
@@ -826,6 +852,11 @@ def clip_accumulate(
 ) -> None:
     """``summed_k (+)= sum_n clip[n] * gs_k[n]`` for every k, reading each gs once. ``clip`` is
     one vector ``[n]`` for all tensors, or a table ``[K, n]`` with a row per tensor."""
+    if _any_half(gs_list, summed_list):
+        wide = [widen(s_) for s_ in summed_list]
+        clip_accumulate([widen(g) for g in gs_list], clip, wide, accumulate)
+        _narrow_back(summed_list, wide)
+        return
     dev = _need_gpu(clip, *gs_list, *summed_list)
     K = len(gs_list)
     if K == 0:
@@ -869,6 +900,11 @@ def add_noise(
     draws: int = 1,
 ) -> None:
     """``grad = (summed + std * z) / denom`` with ``z ~ N(0,1)`` from Philox(seed, offset)."""
+    if _any_half((summed, grad)):
+        wide = widen(grad)
+        add_noise(widen(summed), wide, std, denom, seed, offset, draws)
+        _narrow_back((grad,), (wide,))
+        return
     dev = _need_gpu(summed, grad)
     if not summed.is_contiguous() or not grad.is_contiguous() or summed.numel() != grad.numel():
         raise ValueError("summed and grad must be dense and of equal size")
@@ -897,6 +933,11 @@ def add_noise_multi(
     K = len(summed_list)
     if K == 0:
         return 0
+    if _any_half(summed_list, grad_list):
+        wide = [widen(g) for g in grad_list]
+        used = add_noise_multi([widen(s_) for s_ in summed_list], wide, std, denom, seed, offset, draws)
+        _narrow_back(grad_list, wide)
+        return used
     dev = _need_gpu(*summed_list, *grad_list)
     idt, odt = summed_list[0].dtype, grad_list[0].dtype
     for s, g in zip(summed_list, grad_list):

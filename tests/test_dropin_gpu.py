@@ -1102,6 +1102,86 @@ def test_mixed_precision_dtypes(A):
         assert p.grad.dtype == torch.bfloat16 and p.grad_sample.dtype == torch.bfloat16
 
 
+class _HalfNet(nn.Module):
+    """Embedding, Linear on sequences, LayerNorm, a convolution with GroupNorm: one layer of each
+    kind of sampler."""
+
+    def __init__(self):
+        super().__init__()
+        self.emb = nn.Embedding(20, 16)
+        self.fc = nn.Linear(16, 24)
+        self.ln = nn.LayerNorm(24)
+        self.conv = nn.Conv1d(24, 8, 3, padding=1)
+        self.gn = nn.GroupNorm(2, 8)
+        self.head = nn.Linear(8, 5)
+
+    def forward(self, ids):
+        h = self.ln(F.relu(self.fc(self.emb(ids))))  # [n, T, 24]
+        h = F.relu(self.gn(self.conv(h.transpose(1, 2))))  # [n, 8, T]
+        return self.head(h.mean(2))
+
+
+@pytest.mark.parametrize("mode", ["hooks", "ghost"])
+def test_float16_low_precision(A, mode):
+    """mixed_precision_test.py:164-213 with dtype=float16: a float16 model gives float16 gradients
+    and per-sample gradients. Values: against batch-of-one autograd of the same float16 model
+    taken in float64 (the samplers run on the float32 kernels from widened operands)."""
+    torch.manual_seed(7)
+    net = _HalfNet()
+    n, T = 6, 12
+    ids, y = torch.randint(0, 20, (n, T)), torch.randint(0, 5, (n,))
+    half = copy.deepcopy(net).half()
+    ref = copy.deepcopy(half).double()  # the float16 weights, exactly
+    want = per_sample_grads_cpu(ref, ids, y, lambda out, t: F.cross_entropy(out, t, reduction="sum"))
+    norms = torch.sqrt(sum(v.flatten(1).pow(2).sum(1) for v in want.values()))
+    C = float(norms.median())
+    coef = (C / (norms + 1e-6)).clamp(max=1.0)
+    gnet = half.to(DEV)
+    if mode == "hooks":
+        gsm = A.GradSampleModule(gnet, loss_reduction="mean")
+        opt = A.DPOptimizer(torch.optim.SGD(gsm.parameters(), lr=0.0), noise_multiplier=0.0, max_grad_norm=C, expected_batch_size=n)
+        F.cross_entropy(gsm(ids.to(DEV)).float(), y.to(DEV)).backward()
+        for k, p in gnet.named_parameters():
+            assert p.grad_sample.dtype == torch.float16
+            close(p.grad_sample.double().cpu(), want[k], 2e-2, 2e-3, k)  # float16 forward and backward
+    else:
+        gsm = A.GradSampleModuleFastGradientClipping(gnet, loss_reduction="mean", max_grad_norm=C)
+        opt = A.DPOptimizerFastGradientClipping(torch.optim.SGD(gsm.parameters(), lr=0.0), noise_multiplier=0.0, max_grad_norm=C, expected_batch_size=n)
+        dpl = A.DPLossFastGradientClipping(gsm, opt, nn.CrossEntropyLoss(), "mean")
+        dpl(gsm(ids.to(DEV)).float(), y.to(DEV)).backward()
+        close(gsm.per_sample_gradient_norms.double().cpu(), norms, 1e-2, 1e-4)
+    opt.step()
+    for k, p in gnet.named_parameters():
+        assert p.grad.dtype == torch.float16, k
+        g = (coef.view(-1, *[1] * (want[k].dim() - 1)) * want[k]).sum(0) / n
+        close(p.grad.double().cpu(), g, 2e-2, 1e-3, k)
+
+
+def test_float16_autocast_and_noise(A):
+    """mixed_precision_test.py:107-162 with dtype=float16: float32 parameters under float16
+    autocast keep float32 gradients; a float16 model takes a noisy step."""
+    torch.manual_seed(8)
+    net = nn.Sequential(nn.Linear(16, 32), nn.ReLU(), nn.Linear(32, 4)).to(DEV)
+    gsm = A.GradSampleModule(net, loss_reduction="mean")
+    opt = A.DPOptimizer(torch.optim.SGD(gsm.parameters(), lr=0.1), noise_multiplier=1.0, max_grad_norm=1.0, expected_batch_size=4)
+    with torch.autocast("cuda", dtype=torch.float16):
+        out = gsm(torch.randn(4, 16, device=DEV))
+        assert out.dtype == torch.float16
+        out.float().sum().backward()
+    for p in net.parameters():
+        assert p.grad_sample.dtype in (torch.float16, torch.float32)
+    opt.step()
+    for p in net.parameters():
+        assert p.grad.dtype == torch.float32 and p.summed_grad.dtype == torch.float32
+    low = nn.Linear(16, 4).to(DEV).half()
+    gl = A.GradSampleModule(low, loss_reduction="mean")
+    ol = A.DPOptimizer(torch.optim.SGD(gl.parameters(), lr=0.1), noise_multiplier=1.0, max_grad_norm=1.0, expected_batch_size=4)
+    gl(torch.randn(4, 16, device=DEV).half()).sum().backward()
+    ol.step()
+    for p in low.parameters():
+        assert p.grad.dtype == torch.float16 and p.grad_sample.dtype == torch.float16 and torch.isfinite(p).all()
+
+
 # ---- what backward() leaves behind, and activation checkpointing --------------------------------
 def test_p_grad_after_backward_is_the_non_private_sum_by_default(A, weight_grad_mode):
     """grad_sample_module.py:291-365 adds hooks and leaves autograd alone: after ``backward()`` a

@@ -469,6 +469,32 @@ def test_linear_ghost_norm_multi_many_layers(K, count):
             assert_rel(nb, ob, 1e-4, f"bias norm of layer {k}")
 
 
+def test_float16_tensors_go_through_the_float32_kernels(K):
+    """float16 has no kernels of its own: the optimizer wrappers widen (exactly) and narrow the
+    result, so they agree to the bit with the float32 call on the widened tensors, rounded once."""
+    torch.manual_seed(9)
+    n, P = 5, 300
+    gs = dev(torch.randn(n, P).half())
+    clip = dev(torch.rand(n))
+    assert torch.equal(K.sumsq_rows([gs]), K.sumsq_rows([gs.float()]))
+    out16, out32 = torch.empty(P, device="cuda", dtype=torch.float16), torch.empty(P, device="cuda")
+    K.clip_accumulate([gs], clip, [out16], False)
+    K.clip_accumulate([gs.float()], clip, [out32], False)
+    assert torch.equal(out16, out32.half())
+    base = out32.half().float()
+    K.clip_accumulate([gs], clip, [out16], True)  # accumulates onto the float16 value
+    K.clip_accumulate([gs.float()], clip, [base], True)
+    assert torch.equal(out16, base.half())
+    g16, g32 = torch.empty_like(out16), torch.empty_like(out32)
+    K.add_noise(out16, g16, 0.5, 4.0, 123, 8)
+    K.add_noise(out16.float(), g32, 0.5, 4.0, 123, 8)
+    assert torch.equal(g16, g32.half())
+    assert K.add_noise_multi([out16], [g16], 0.5, 4.0, 123, 8) == 1 and torch.equal(g16, g32.half())
+    assert K.supported_dtype(torch.float16) and not K.native_dtype(torch.float16)
+    with pytest.raises(TypeError):
+        K.linear_grad_sample(dev(torch.randn(2, 4).half()), dev(torch.randn(2, 4).half()))
+
+
 WEIGHTED_SUM_CASES = [
     # (n, T, in, out, pieces)
     (8, 32, 128, 128, 1),  # one k tile per sample: a rescaling before every tile
