@@ -967,6 +967,42 @@ def test_ghost_single_backward_leaves_the_second_pass_gradients(A, case):
         close(g1 / scale, g2 / scale, 1e-4, 2e-6, f"{case} {name}")
 
 
+@pytest.mark.parametrize("bias", [True, False])
+def test_ghost_single_backward_bf16_weighted_contraction(A, bias):
+    """A bf16 MLP on sequences whose Linear layers the weighted contraction takes (whole k tiles of
+    32 positions, widths above 64): the single-pass clipped sum, with the coefficients applied
+    inside the kernel, against the two-pass gradients of the same model (bf16 autograd, whose
+    weighted backprops are rounded to bf16 on the way) and against fp64 on the CPU."""
+    from opacus_amd import kernels
+
+    torch.manual_seed(31)
+    n, T = 8, 64
+    net = nn.Sequential(nn.Linear(128, 256, bias=bias), nn.GELU(), nn.Linear(256, 128, bias=bias))
+    x, y = torch.randn(n, T, 128), torch.randn(n, T, 128) * torch.logspace(-0.7, 0.7, n).view(n, 1, 1)  # norms a decade apart
+    half = copy.deepcopy(net).bfloat16()
+    assert kernels.linear_weighted_sum_takes(torch.empty(n, T, 256, device=DEV, dtype=torch.bfloat16), torch.empty(n, T, 128, device=DEV, dtype=torch.bfloat16))
+
+    def loss_call(model, opt, b):
+        return A.DPLossFastGradientClipping(model, opt, PerSampleMSE("mean"), "mean")(model(b[0]), b[1])
+
+    batch = (x.bfloat16(), y.bfloat16())
+    C = 0.2
+    two, _ = _ghost_grads(A, half, batch, loss_call, single=False, steps=1, C=C)
+    one, ghost = _ghost_grads(A, half, batch, loss_call, single=True, steps=1, C=C)
+    norms = ghost.per_sample_gradient_norms.double().cpu()
+    assert (norms > C).any() and (norms < C).any(), norms  # clipped and unclipped samples
+    # fp64 on the CPU from the same bf16 weights and inputs; the coefficients as the GPU run found them
+    ref = copy.deepcopy(half).double()
+    want = per_sample_grads_cpu(ref, batch[0].double(), batch[1].double(), lambda out, t: PerSampleMSE("sum")(out, t))
+    coef = (C / (norms + 1e-6)).clamp(max=1.0)
+    for (name, _), g1, g2 in zip(ghost.named_parameters(), one, two):
+        scale = g2.float().abs().max().item() + 1e-12
+        close(g1.float() / scale, g2.float() / scale, 2e-2, 2e-2, f"{name} against two passes")
+        w = want[name[len('_module.'):]]
+        g = (coef.view(-1, *[1] * (w.dim() - 1)) * w).sum(0)  # before the optimizer divides by n
+        close(g1.double().cpu() / scale, g / scale, 2e-2, 2e-2, f"{name} against fp64")
+
+
 def test_ghost_tied_parameters_raise(A):
     class Tied(nn.Module):
         def __init__(self):
