@@ -660,6 +660,15 @@ def kernel_table(dev, iters: int = 10, warm: int = 3, with_cpu: bool = True):
                       cpu(lambda: torch.einsum("n,nij->ij", cc, O.linear_grad_sample(ca, cb)[0]), n,
                           f"1 of {n} samples, fp32 einsum + weighted sum"))
             del a, b
+    # ... and pooled: the clipped sums of all of C5's Linear layers in one launch
+    n, T = 16, 1024
+    layers = [(2048, 2048), (2048, 512), (2048, 512), (2048, 2048), (2048, 5632), (2048, 5632), (5632, 2048)] * 4 + [(2048, 32000)]
+    c = torch.rand(n, device=dev) * 0.9 + 0.1
+    items = [((torch.randn(n, T, o, device=dev) * 0.02).bfloat16(), torch.randn(n, T, i, device=dev).bfloat16(), c, 1.0)
+             for i, o in layers]
+    yield row("linear_weighted_sum_multi", "a9", "C5 all 29 Linear layers pooled, n=16 T=1024 bf16",
+              timed(lambda: K.linear_weighted_sum_multi(items)), "mfma_bf16", sum(2.0 * n * T * i * o for i, o in layers))
+    del items
     # the same kernel on fp32 operands
     tri, full = tri_tiles(1024)
     a = torch.randn(16, 1024, 2048, device=dev)

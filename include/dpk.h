@@ -102,6 +102,22 @@ int dpk_linear_weighted_sum(const void* b, const void* a, int in_dtype, const fl
                             int64_t in_features, float scale, int pieces, void* ws, size_t ws_bytes,
                             dpk_stream_t stream);
 
+/* dpk_linear_weighted_sum for several layers in one call: the block tiles of all layers are
+ * one pool of work, so the GPU stays full across layers whose own tile count is not a
+ * multiple of what it holds at once (C5: 29 layers, 37 launches -> one). Every layer is
+ * contracted in one piece (no workspace); per-layer requirements as above, all results of
+ * `out_dtype`. `layers` is a host array of any length (32 layers per launch). */
+typedef struct dpk_wsum_layer {
+  const void* b;     /* [n,T,out] bf16 */
+  const void* a;     /* [n,T,in] bf16 */
+  const float* coef; /* [n] */
+  void* out_sum;     /* [out,in] */
+  int64_t n, T, out, in;
+  float scale;
+} dpk_wsum_layer;
+int dpk_linear_weighted_sum_multi(const dpk_wsum_layer* layers /*host*/, int count, int in_dtype, int out_dtype,
+                                  dpk_stream_t stream);
+
 /* gs_bias[n,k] = scale * sum_t b[n,t,k]                   (linear.py:50)
  * sumsq (nullable, float[n]) receives sum_k gs_bias[n,k]^2 of the values as stored, for
  * the optimizer's norm pass (optimizers/optimizer.py:444-446). */

@@ -33,6 +33,15 @@ class GhostLayer(ctypes.Structure):
         ("T", c_int64), ("out", c_int64), ("inp", c_int64), ("scale", c_float),
     ]
 
+class WsumLayer(ctypes.Structure):
+    """``dpk_wsum_layer`` of include/dpk.h."""
+
+    _fields_ = [
+        ("b", c_void_p), ("a", c_void_p), ("coef", c_void_p), ("out_sum", c_void_p),
+        ("n", c_int64), ("T", c_int64), ("out", c_int64), ("inp", c_int64), ("scale", c_float),
+    ]
+
+
 STATUS_NAMES = {
     0: "DPK_OK",
     -1: "DPK_E_SHAPE",
@@ -57,6 +66,7 @@ SIGNATURES = {
     "dpk_linear_weighted_sum": (
         c_int, [_P, _P, c_int, _P, _P, c_int, _I, _I, _I, _I, c_float, c_int, _P, c_size_t, _P]
     ),
+    "dpk_linear_weighted_sum_multi": (c_int, [_P, c_int, c_int, c_int, _P]),
     "dpk_linear_bias_gs": (c_int, [_P, c_int, _P, c_int, _P, _I, _I, _I, c_float, _P]),
     "dpk_linear_ghost_norm_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
     "dpk_linear_ghost_norm": (c_int, [_P, _P, c_int, _P, _P, _I, _I, _I, _I, c_float, c_int, _P, c_size_t, _P]),

@@ -243,36 +243,30 @@ struct DldsF32 {
 // coef[s * (T / unit_rows) + u] times: gs[s] = scale * sum_u coef[..] * b_u^T a_u.
 // (Two waves per SIMD asked for, which these kernels reach anyway, caps W at 256 registers: the
 // accumulators then live in ordinary registers, where they can be multiplied in place.)
-template <class E, class C, typename TOUT, bool W = false>
-__global__ __launch_bounds__(C::kThreads, W ? 2 : 1) void linear_dlds_kernel(
-    const typename E::elem* __restrict__ b, const typename E::elem* __restrict__ a, TOUT* __restrict__ gs,
-    float* __restrict__ partials, int64_t T, int64_t M, int64_t N, float scale, int64_t tiles_m,
-    int64_t tiles_n, const float* __restrict__ coef = nullptr, int64_t unit_rows = 0) {
+// One block tile of the product of one "sample": the tile at (m0, n0) of out = scale * b^T a
+// over T rows (b, a and out already at the sample), its sum of squares into partials[slot].
+template <class E, class C, typename TOUT, bool W>
+__device__ __forceinline__ void linear_dlds_tile(
+    typename E::template Smem<C>& sm, float* red, const typename E::elem* __restrict__ b,
+    const typename E::elem* __restrict__ a, TOUT* __restrict__ out, float* __restrict__ partials, uint32_t slot,
+    int64_t T, int64_t M, int64_t N, float scale, int64_t m0, int64_t n0, const float* __restrict__ coef,
+    int64_t unit_rows) {
   typedef typename E::template Smem<C> SmemT;
-  __shared__ SmemT sm;
-  __shared__ float red[C::kWaves];
   // rows of the product = input features (P = a), columns = output features (Q = b)
   constexpr int BJ = C::BP, BI = C::BQ;
   constexpr int kPitch = BJ * sizeof(TOUT) + TrOut<TOUT>::kPad, kRows = TrOut<TOUT>::kRows;
   static_assert(kRows * kPitch <= sizeof(SmemT), "output rows must fit the stage memory");
   static_assert(BI % kRows == 0 && kRows % 32 == 0, "passes of whole MFMA tiles");
-  // neighbouring tiles of a sample share operand panels: keep them on one XCD
-  const uint32_t bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
-  const int64_t per_sample = tiles_m * tiles_n;
-  const int64_t sample = bid / per_sample;
-  const int64_t rem = bid % per_sample;
-  const int64_t m0 = (rem / tiles_n) * BI, n0 = (rem % tiles_n) * BJ;
+  TOUT* const gs = out;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wj0 = (wave / C::WQ) * (32 * C::TP), wi0 = (wave % C::WQ) * (32 * C::TQ);  // this wave's corner
   typename E::template Tile<C> tile;
   tile.clear();
   if constexpr (W)
-    E::template mainloop_weighted<C>(tile, sm, a + sample * T * N, N, n0, b + sample * T * M, M, m0, T, wj0, wi0,
-                                     coef + sample * (T / unit_rows), unit_rows / mb16t::BK);
+    E::template mainloop_weighted<C>(tile, sm, a, N, n0, b, M, m0, T, wj0, wi0, coef, unit_rows / mb16t::BK);
   else
-    E::template mainloop<C>(tile, sm, a + sample * T * N, N, n0, b + sample * T * M, M, m0, T, wj0, wi0);
-  TOUT* out = gs + sample * M * N;
+    E::template mainloop<C>(tile, sm, a, N, n0, b, M, m0, T, wj0, wi0);
   const int kk = lane >> 5, l32 = lane & 31;
   float ss = 0.f;
   unsigned char* stage_out = &sm.stage[0][0];
@@ -339,8 +333,58 @@ __global__ __launch_bounds__(C::kThreads, W ? 2 : 1) void linear_dlds_kernel(
   }
   if (partials) {
     const float s = block_sum<C::kWaves>(ss, red);
-    if (threadIdx.x == 0) partials[bid] = s;
+    if (threadIdx.x == 0) partials[slot] = s;
   }
+}
+
+template <class E, class C, typename TOUT, bool W = false>
+__global__ __launch_bounds__(C::kThreads, W ? 2 : 1) void linear_dlds_kernel(
+    const typename E::elem* __restrict__ b, const typename E::elem* __restrict__ a, TOUT* __restrict__ gs,
+    float* __restrict__ partials, int64_t T, int64_t M, int64_t N, float scale, int64_t tiles_m,
+    int64_t tiles_n, const float* __restrict__ coef = nullptr, int64_t unit_rows = 0) {
+  __shared__ typename E::template Smem<C> sm;
+  __shared__ float red[C::kWaves];
+  // neighbouring tiles of a sample share operand panels: keep them on one XCD
+  const uint32_t bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  const int64_t per_sample = tiles_m * tiles_n;
+  const int64_t sample = bid / per_sample;
+  const int64_t rem = bid % per_sample;
+  const float* c = coef;
+  if constexpr (W) c = coef + sample * (T / unit_rows);  // this run of samples' coefficients
+  linear_dlds_tile<E, C, TOUT, W>(sm, red, b + sample * T * M, a + sample * T * N, gs ? gs + sample * M * N : gs, partials,
+                                  bid, T, M, N, scale, (rem / tiles_n) * C::BQ, (rem % tiles_n) * C::BP, c, unit_rows);
+}
+
+// The clip-weighted sums of up to kWsumMax Linear layers in one launch: block -> (layer, tile)
+// through the prefix sums of the layers' tile counts. A layer on its own fills the GPU in
+// whole rounds of blocks only by luck (22 x 8 tiles of 256 x 256 on 256 CUs leave 80 idle for
+// the whole contraction); pooled, the layers' tiles follow one another without a gap.
+constexpr int kWsumMax = 32;
+struct WsumMultiArgs {
+  const bf16_t* b[kWsumMax];
+  const bf16_t* a[kWsumMax];
+  const float* coef[kWsumMax];
+  void* out[kWsumMax];
+  int64_t rows[kWsumMax];       // n * T
+  int32_t unit_rows[kWsumMax];  // T
+  int32_t M[kWsumMax], N[kWsumMax], tiles_n[kWsumMax];
+  uint32_t tile_prefix[kWsumMax + 1];
+  float scale[kWsumMax];
+  int32_t nlayers;
+};
+
+template <class C, typename TOUT>
+__global__ __launch_bounds__(C::kThreads, 2) void linear_wsum_multi_kernel(const WsumMultiArgs A) {
+  __shared__ typename TrBf16::template Smem<C> sm;
+  __shared__ float red[C::kWaves];
+  // consecutive tiles (one layer, neighbouring operand panels) on one XCD
+  const uint32_t bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  int l = 0;
+  while (l + 1 < A.nlayers && bid >= A.tile_prefix[l + 1]) ++l;
+  const uint32_t rem = bid - A.tile_prefix[l], tn = static_cast<uint32_t>(A.tiles_n[l]);
+  linear_dlds_tile<TrBf16, C, TOUT, true>(sm, red, A.b[l], A.a[l], static_cast<TOUT*>(A.out[l]), nullptr, 0u, A.rows[l],
+                                          A.M[l], A.N[l], A.scale[l], static_cast<int64_t>(rem / tn) * C::BQ,
+                                          static_cast<int64_t>(rem % tn) * C::BP, A.coef[l], A.unit_rows[l]);
 }
 
 using DldsF32Cfg = mf32d::Config<2, 2, 2, 2, 4>;  // 128 x 128, 4 waves, 64 KB: two blocks per CU
@@ -754,6 +798,75 @@ extern "C" int dpk_linear_weighted_sum(const void* b, const void* a, int in_dtyp
     else
       hipLaunchKernelGGL(add_pieces_kernel<float>, g2, dim3(kThreads), 0, s, static_cast<const float*>(ws),
                          static_cast<float*>(out_sum), count4, pieces);
+    DPK_LAUNCH_CHECK(who);
+  }
+  return DPK_OK;
+}
+
+// The same sums for several layers at once (dpk_wsum_layer records, host array): one launch per
+// group of up to 32 layers whose results share a dtype, every layer in one piece.
+extern "C" int dpk_linear_weighted_sum_multi(const dpk_wsum_layer* layers, int count, int in_dtype, int out_dtype,
+                                             dpk_stream_t stream) {
+  const char* who = "dpk_linear_weighted_sum_multi";
+  DPK_REQUIRE(count >= 0 && (layers || count == 0), DPK_E_ARG, "%s: count=%d, layers=%p", who, count, (const void*)layers);
+  DPK_REQUIRE(in_dtype == DPK_BF16 && dpk_dtype_ok(out_dtype), DPK_E_DTYPE, "%s: dtypes %d,%d (bf16 input only)", who,
+              in_dtype, out_dtype);
+  int64_t tiles256 = 0, tiles128 = 0;
+  for (int i = 0; i < count; ++i) {
+    const dpk_wsum_layer& L = layers[i];
+    DPK_REQUIRE(L.n >= 1 && L.T >= 1 && L.out >= 1 && L.in >= 1, DPK_E_SHAPE, "%s: layer %d: n=%lld T=%lld out=%lld in=%lld",
+                who, i, (long long)L.n, (long long)L.T, (long long)L.out, (long long)L.in);
+    DPK_REQUIRE(L.b && L.a && L.coef && L.out_sum, DPK_E_ARG, "%s: layer %d: NULL tensor", who, i);
+    DPK_REQUIRE(L.T % mb16t::BK == 0 && L.T < (int64_t{1} << 31), DPK_E_SHAPE, "%s: layer %d: T=%lld must be a multiple of %d",
+                who, i, (long long)L.T, mb16t::BK);
+    DPK_REQUIRE(L.out % 8 == 0 && L.in % 8 == 0 && L.out > 64 && L.in > 64 && L.out < (1LL << 24) && L.in < (1LL << 24) &&
+                    dpk_aligned(L.b, 16) && dpk_aligned(L.a, 16) && dpk_aligned(L.out_sum, 16) && dpk_aligned(L.coef, 4),
+                DPK_E_SHAPE, "%s: layer %d: out=%lld and in=%lld must be multiples of 8 above 64 and the tensors 16-byte aligned",
+                who, i, (long long)L.out, (long long)L.in);
+    tiles256 += dpk_cdiv(L.out, 256) * dpk_cdiv(L.in, 256);
+    tiles128 += dpk_cdiv(L.out, 128) * dpk_cdiv(L.in, 128);
+  }
+  if (count == 0) return DPK_OK;
+  // the same cost rule as for one layer, on the pool: rounds of resident blocks times work per block
+  int cus = dpk_device_cus();
+  if (cus <= 0) cus = 256;
+  const double cost_small = static_cast<double>(dpk_cdiv(tiles128, 2 * cus)) * 2.0;
+  const double cost_large = static_cast<double>(dpk_cdiv(tiles256, cus)) * 4.0 * kTrLargeGain;
+  bool all_wide = true;
+  for (int i = 0; i < count; ++i) all_wide = all_wide && layers[i].out >= 256 && layers[i].in >= 256;
+  const int tile = (all_wide && cost_large < cost_small) ? 256 : 128;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  for (int lo = 0; lo < count; lo += kWsumMax) {
+    const int nl = count - lo < kWsumMax ? count - lo : kWsumMax;
+    WsumMultiArgs A;
+    A.nlayers = nl;
+    A.tile_prefix[0] = 0;
+    int64_t total = 0;
+    for (int i = 0; i < nl; ++i) {
+      const dpk_wsum_layer& L = layers[lo + i];
+      A.b[i] = static_cast<const bf16_t*>(L.b);
+      A.a[i] = static_cast<const bf16_t*>(L.a);
+      A.coef[i] = L.coef;
+      A.out[i] = L.out_sum;
+      A.rows[i] = L.n * L.T;
+      A.unit_rows[i] = static_cast<int32_t>(L.T);
+      A.M[i] = static_cast<int32_t>(L.out);
+      A.N[i] = static_cast<int32_t>(L.in);
+      A.tiles_n[i] = static_cast<int32_t>(dpk_cdiv(L.in, tile));
+      A.scale[i] = L.scale;
+      total += dpk_cdiv(L.out, tile) * dpk_cdiv(L.in, tile);
+      DPK_REQUIRE(total <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: %lld blocks exceed the grid limit", who, (long long)total);
+      A.tile_prefix[i + 1] = static_cast<uint32_t>(total);
+    }
+    const dim3 grid(static_cast<unsigned>(total));
+    if (tile == 256 && out_dtype == DPK_BF16)
+      hipLaunchKernelGGL((linear_wsum_multi_kernel<TrLarge, bf16_t>), grid, dim3(TrLarge::kThreads), 0, s, A);
+    else if (tile == 256)
+      hipLaunchKernelGGL((linear_wsum_multi_kernel<TrLarge, float>), grid, dim3(TrLarge::kThreads), 0, s, A);
+    else if (out_dtype == DPK_BF16)
+      hipLaunchKernelGGL((linear_wsum_multi_kernel<TrSmall, bf16_t>), grid, dim3(TrSmall::kThreads), 0, s, A);
+    else
+      hipLaunchKernelGGL((linear_wsum_multi_kernel<TrSmall, float>), grid, dim3(TrSmall::kThreads), 0, s, A);
     DPK_LAUNCH_CHECK(who);
   }
   return DPK_OK;

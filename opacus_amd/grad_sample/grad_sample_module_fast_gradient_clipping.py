@@ -378,21 +378,37 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
             else:
                 sums[id(param)] = (param, value)
 
-        for module, activations, backprops, scale, grad_samples in kept:
+        # bf16 Linear layers on sequences: the coefficients go onto the accumulators of one
+        # contraction over all samples and positions (neither operand is weighted or copied
+        # beforehand), and the tiles of all such layers are one pooled launch
+        pooled, rest = [], []
+        for entry in kept:
+            module, activations, backprops = entry[0], entry[1], entry[2]
+            if backprops.shape[0] and self._sampler_for(module) is linear_grad_sampler:
+                a = activations[0].to(backprops.dtype)
+                if module.weight.requires_grad and kernels.linear_weighted_sum_takes(backprops, a):
+                    pooled.append((module, a, backprops, entry[3]))
+                    continue
+            rest.append(entry)
+        by_device = {}
+        for item in pooled:
+            by_device.setdefault(item[2].device, []).append(item)
+        for dev, items in by_device.items():
+            c = coef.to(device=dev, dtype=torch.float32)
+            sums_w = kernels.linear_weighted_sum_multi([(b, a, c, scale) for _, a, b, scale in items])
+            for (module, a, backprops, scale), total in zip(items, sums_w):
+                add(module.weight, total)
+                if module.bias is not None:
+                    per_sample = backprops.sum(dim=tuple(range(1, backprops.dim() - 1)), dtype=torch.float32)
+                    add(module.bias, ((c * scale) @ per_sample).to(backprops.dtype))
+        del pooled, by_device
+        for module, activations, backprops, scale, grad_samples in rest:
             n = backprops.shape[0]
             c = coef.to(device=backprops.device, dtype=torch.float32)
             if n == 0:
                 continue
             if self._sampler_for(module) is linear_grad_sampler:  # nn.Linear itself and RNNLinear, not a subclass with a forward of its own
                 a = activations[0].to(backprops.dtype)
-                if kernels.linear_weighted_sum_takes(backprops, a):
-                    # the coefficients go onto the accumulators of one contraction over all samples
-                    # and positions: neither operand is weighted (or even copied) beforehand
-                    add(module.weight, kernels.linear_weighted_sum(backprops, a, c, scale=scale))
-                    if module.bias is not None:
-                        per_sample = backprops.sum(dim=tuple(range(1, backprops.dim() - 1)), dtype=torch.float32)
-                        add(module.bias, ((c * scale) @ per_sample).to(backprops.dtype))
-                    continue
                 w = (c * scale).to(backprops.dtype).view(n, *([1] * (backprops.dim() - 1)))
                 if module.bias is None and a.shape[-1] < backprops.shape[-1]:
                     # (coef * b)^T a == b^T (coef * a): weight the narrower of the two

@@ -232,6 +232,53 @@ def linear_weighted_sum(
     return out
 
 
+def linear_weighted_sum_multi(
+    items: Sequence[Tuple[torch.Tensor, torch.Tensor, torch.Tensor, float]],
+    out_dtype: Optional[torch.dtype] = None,
+    pooled: Optional[bool] = None,
+) -> List[torch.Tensor]:
+    """:func:`linear_weighted_sum` for several layers in one call: each item is ``(backprops,
+    activations, coef, scale)`` (every pair one that :func:`linear_weighted_sum_takes`); returns
+    the ``[out, in]`` sums in order. The block tiles of all layers are one pool of work, so the
+    GPU stays full across layers whose own tile count does not fill it in whole rounds
+    (``pooled=False``/``True`` overrides the choice between that and layer-by-layer calls)."""
+    if not items:
+        return []
+    dev = _need_gpu(*[t for it in items for t in it[:3]])
+    out_dtype = out_dtype or items[0][0].dtype
+    # a small pool (a two-layer MLP) is better off layer by layer, each cut into pieces along the
+    # samples: the pooled launch contracts every layer in one piece and needs several rounds of
+    # 256 x 256 tiles to keep the GPU busy
+    tiles = sum(-(-it[0].shape[-1] // 256) * -(-it[1].shape[-1] // 256) for it in items)
+    if pooled is None:
+        pooled = tiles >= 4 * device_cus()
+    if not pooled:
+        return [linear_weighted_sum(b, a, c, scale=scale, out_dtype=out_dtype) for b, a, c, scale in items]
+    table = (_lib.WsumLayer * len(items))()
+    keep, outs = [], []
+    for row, (bp, act, coef, scale) in zip(table, items):
+        n, out_f, in_f = bp.shape[0], bp.shape[-1], act.shape[-1]
+        b = _dense(bp).reshape(n, -1, out_f)
+        a = _dense(act).reshape(n, -1, in_f)
+        if a.shape[1] != b.shape[1] or b.dtype != torch.bfloat16 or a.dtype != torch.bfloat16:
+            raise ValueError(f"activations {tuple(act.shape)} {act.dtype} and backprops {tuple(bp.shape)} {bp.dtype} disagree or are not bfloat16")
+        c = _dense(coef.to(torch.float32)).reshape(-1)
+        if c.numel() != n:
+            raise ValueError(f"{c.numel()} coefficients for {n} samples")
+        out = torch.empty((out_f, in_f), dtype=out_dtype, device=dev)
+        keep.append((b, a, c))
+        outs.append(out)
+        row.b, row.a, row.coef, row.out_sum = b.data_ptr(), a.data_ptr(), c.data_ptr(), out.data_ptr()
+        row.n, row.T, row.out, row.inp, row.scale = n, b.shape[1], out_f, in_f, float(scale)
+    with _timed("linear_weighted_sum", dev):
+        check(
+            "dpk_linear_weighted_sum_multi",
+            lib().dpk_linear_weighted_sum_multi(table, len(items), DPK_BF16, _code(out_dtype), _stream(dev)),
+        )
+    del keep
+    return outs
+
+
 def _with_sumsq(gs: torch.Tensor, sumsq: torch.Tensor) -> torch.Tensor:
     """Leaves the per-sample sum of squares on the tensor it describes, with the tensor's
     version, so that the optimizer's norm pass can use it while nobody has written to ``gs``."""

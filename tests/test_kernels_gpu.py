@@ -532,6 +532,37 @@ def test_linear_weighted_sum(K, n, T, fin, fout, pieces, coefs, out_f32):
     assert_rel(got[None], want[None], 1e-4 if out_f32 else BF16_REL, "weighted sum")
 
 
+@pytest.mark.parametrize("count", [3, 40])
+def test_linear_weighted_sum_multi(K, count):
+    """Several layers pooled into one launch (more than one launch's table for 40), with
+    different shapes, batch sizes and sequence lengths: each sum as the single-layer call
+    gives it (one piece), and against the oracle for the first."""
+    torch.manual_seed(count)
+    shapes = [(8, 64, 128, 256), (4, 32, 512, 136), (6, 96, 72, 264), (16, 32, 256, 2048)]
+    items = []
+    for k in range(count):
+        n, T, fin, fout = shapes[k % len(shapes)]
+        a = dev(torch.randn(n, T, fin).bfloat16())
+        b = dev((torch.randn(n, T, fout) * 0.1).bfloat16())
+        c = dev(torch.rand(n) * 0.9 + 0.1)
+        items.append((b, a, c, 1.0 + k % 3))
+    for out_dtype in (None, torch.float32):
+        sums = K.linear_weighted_sum_multi(items, out_dtype=out_dtype, pooled=True)
+        assert len(sums) == count
+        for (b, a, c, scale), got in zip(items, sums):
+            want = K.linear_weighted_sum(b, a, c, scale=scale, pieces=1, out_dtype=out_dtype)
+            assert got.dtype == want.dtype and got.shape == want.shape
+            # the pool may choose the other block tile: same products, another order of addition
+            assert_rel(got[None], want[None], 1e-5 if out_dtype else BF16_REL, "pooled against single")
+    b, a, c, scale = items[0]
+    gs, _ = O.linear_grad_sample(a.cpu().double(), b.cpu().double())
+    want = (c.cpu().double().view(-1, 1, 1) * gs).sum(0) * scale
+    assert_rel(K.linear_weighted_sum_multi(items[:1], out_dtype=torch.float32, pooled=True)[0][None], want[None], 1e-4, "pooled against the oracle")
+    assert K.linear_weighted_sum_multi([]) == []
+    with pytest.raises(RuntimeError, match="dpk_linear_weighted_sum_multi"):
+        K.linear_weighted_sum_multi([(b[:, :16].contiguous(), a[:, :16].contiguous(), c, 1.0)], pooled=True)
+
+
 def test_linear_weighted_sum_keeps_a_nan_and_refuses_other_shapes(K):
     torch.manual_seed(5)
     a, b = dev(torch.randn(4, 32, 128).bfloat16()), dev(torch.randn(4, 32, 128).bfloat16())
