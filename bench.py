@@ -13,7 +13,7 @@ timed on this box's host cores on a bounded sample of the same workload.
 
 The headline fields are config 2's. The same run then times the other four benchmark
 configurations (c1, c3, c4, c5: full DP-SGD steps through the drop-in API, at most 20
-steps each, 5 for c5) and reports them under ``"configs"``, each with its own
+steps each, 10 for c5) and reports them under ``"configs"``, each with its own
 ``ms_per_step``, ``samples_per_s``, ``roofline`` and bounded-sample ``cpu_baseline``
 (c5 also with embedding table and LM head tied, which the reference refuses under ghost
 clipping, as ``tied_embeddings``).
@@ -768,12 +768,16 @@ def run_workload(name: str, dev, steps: int, warmup: int, all_timers: bool = Fal
     torch.cuda.synchronize()
     # HIP events around the dominant kernel's entry point only, unless every entry point is asked for
     only = None if all_timers else {w["roofline"]["timer"]}
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]  # step boundaries on the launch stream
     with kernels.record_kernel_times(only=only) as times:
         t0 = time.perf_counter()
-        for _ in range(steps):
+        marks[0].record()
+        for i in range(steps):
             step()
+            marks[i + 1].record()
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - t0
+    per_step = sorted(a.elapsed_time(b) for a, b in zip(marks, marks[1:]))
 
     kernel_ms = {k: sum(s.elapsed_time(e) for s, e in v) / steps for k, v in times.items()}
     r = dict(w["roofline"])
@@ -795,13 +799,15 @@ def run_workload(name: str, dev, steps: int, warmup: int, all_timers: bool = Fal
     return {
         "workload": w["workload"], "dtype": w["dtype"], "global_batch": w["n"], "steps": steps, "warmup": warmup,
         "ms_per_step": elapsed / steps * 1e3, "samples_per_s": w["n"] * steps / elapsed,
+        # the middle step's span on the device: a single stalled step moves the mean of a short run, not this
+        "ms_per_step_median": per_step[len(per_step) // 2] if per_step else None,
         "kernel_ms_per_step": kernel_ms, "extra": w["extra"], "roofline": roofline,
     }
 
 
 # Steps of the other configurations inside the default run: enough for a stable mean, few
-# enough that the whole run stays within minutes (a c5 step takes ~60 ms, the others 1-2 ms).
-OTHER_CONFIGS = {"c1": (20, 5), "c3": (20, 5), "c4": (20, 5), "c5": (5, 2)}
+# enough that the whole run stays within minutes (a c5 step takes 43-65 ms, the others 1-2 ms).
+OTHER_CONFIGS = {"c1": (20, 5), "c3": (20, 5), "c4": (20, 5), "c5": (10, 3)}
 
 
 def main() -> None:
@@ -855,7 +861,8 @@ def main() -> None:
         "dtype": head["dtype"],
         "data": "synthetic",
         "config": {"workload": head["workload"], "global_batch": head["global_batch"],
-                   "kernel_ms_per_step": head["kernel_ms_per_step"], **head["extra"]},
+                   "kernel_ms_per_step": head["kernel_ms_per_step"], "ms_per_step_median": head["ms_per_step_median"],
+                   **head["extra"]},
         "roofline": head["roofline"],
     }
     cpu_ok = not args.no_cpu_baseline and head_name.rstrip("stdp") in ("c1", "c2", "c3", "c4", "c5")
@@ -868,19 +875,22 @@ def main() -> None:
             k, wu = min(k, args.steps), min(wu, max(args.warmup, 1))
             r = run_workload(name, dev, k, wu, args.all_kernel_timers)
             entry = {key: r[key] for key in ("workload", "dtype", "global_batch", "steps", "warmup", "ms_per_step",
-                                             "samples_per_s", "roofline")}
+                                             "ms_per_step_median", "samples_per_s", "roofline")}
             entry.update(r["extra"])
             if name + "p" in WORKLOADS:  # the same configuration with the reference's two backward passes
                 d = run_workload(name + "p", dev, k, wu, args.all_kernel_timers)
-                entry["two_backward_passes"] = {"ms_per_step": d["ms_per_step"], "samples_per_s": d["samples_per_s"],
+                entry["two_backward_passes"] = {"ms_per_step": d["ms_per_step"], "ms_per_step_median": d["ms_per_step_median"],
+                    "samples_per_s": d["samples_per_s"],
                                                 "single_backward": False}
             if name + "t" in WORKLOADS:  # the same decoder with embedding table and LM head sharing one parameter
                 d = run_workload(name + "t", dev, k, wu, args.all_kernel_timers)
-                entry["tied_embeddings"] = {"ms_per_step": d["ms_per_step"], "samples_per_s": d["samples_per_s"],
+                entry["tied_embeddings"] = {"ms_per_step": d["ms_per_step"], "ms_per_step_median": d["ms_per_step_median"],
+                    "samples_per_s": d["samples_per_s"],
                                             "workload": d["workload"]}
             if name + "d" in WORKLOADS:  # the same configuration with the library's default hooks
                 d = run_workload(name + "d", dev, k, wu, args.all_kernel_timers)
-                entry["default_hooks"] = {"ms_per_step": d["ms_per_step"], "samples_per_s": d["samples_per_s"],
+                entry["default_hooks"] = {"ms_per_step": d["ms_per_step"], "ms_per_step_median": d["ms_per_step_median"],
+                    "samples_per_s": d["samples_per_s"],
                                           "autograd_weight_grads": True}
             if not args.no_cpu_baseline:
                 entry["cpu_baseline"] = cpu_baseline(name)
