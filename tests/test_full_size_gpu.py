@@ -153,6 +153,33 @@ def test_linear_grad_sample_with_sequence_full_size(K, dtype, n, T, fin, fout):
 
 
 # ---- C4: Conv2d 64 -> 64, 3 x 3, 32 x 32 images, batch 256, fp32 ------------------------------
+@pytest.mark.parametrize("pooled", [False, True])
+def test_weighted_sum_past_32_bit_offsets(K, pooled):
+    """n*T*out = 2.7e9 elements (5.4 GB of backprops): element and byte offsets inside the operand
+    pass 2^31 and 2^32. Slices of the result against torch on the weighted operand in fp32, and
+    linearity in the coefficients (scaling them by 4 scales the sum by 4, exactly)."""
+    torch.manual_seed(13)
+    n, T, fin, fout = 16, 4096, 256, 40960
+    a = torch.randn(n, T, fin, device="cuda").bfloat16()
+    b = torch.empty(n, T, fout, device="cuda", dtype=torch.bfloat16)
+    for s in range(n):  # filled sample by sample: no fp32 copy of the whole tensor
+        b[s] = (torch.randn(T, fout, device="cuda") * 0.05).bfloat16()
+    c = torch.rand(n, device="cuda") * 0.9 + 0.1
+
+    def run(coef):
+        if pooled:
+            return K.linear_weighted_sum_multi([(b, a, coef, 1.0)], out_dtype=torch.float32, pooled=True)[0]
+        return K.linear_weighted_sum(b, a, coef, out_dtype=torch.float32)
+
+    got = run(c)
+    assert got.shape == (fout, fin)
+    wa = (a.float() * c.view(n, 1, 1)).reshape(n * T, fin)
+    for lo in (0, 20000, fout - 512):  # first, middle and last rows of the result
+        want = b[:, :, lo : lo + 512].reshape(n * T, 512).float().t() @ wa
+        assert rel_err(got[lo : lo + 512], want) < 1e-4, lo
+    assert torch.equal(run(c * 4), got * 4)
+
+
 def test_c4_conv_and_group_norm_full_size(K):
     n = 256
     torch.manual_seed(4)
