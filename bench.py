@@ -259,7 +259,8 @@ def workload_c4(dev, autograd_weight_grads=False):
     )
 
 
-def _ghost_workload(dev, net, make_inputs, loss_call, n, T, sigma, desc, single=True, traffic=None, traffic_source=None):
+def _ghost_workload(dev, net, make_inputs, loss_call, n, T, sigma, desc, single=True, traffic=None, traffic_source=None,
+                    wsum_traffic=None, wsum_traffic_source=None):
     from opacus_amd import GradSampleModuleFastGradientClipping
     from opacus_amd.optimizers import DPOptimizerFastGradientClipping
 
@@ -276,14 +277,26 @@ def _ghost_workload(dev, net, make_inputs, loss_call, n, T, sigma, desc, single=
         opt.step()
 
     flops = ghost_executed_flops(net, n, T)
-    return dict(
+    ghost = dict(kernel="ghost_norm_multi_kernel<128x128, 2 stages> (all Linear layers of a step pooled into one launch; thin layers by linear_dlds_kernel; "
+                        "ghost_norm_bf16_dlds_kernel layer by layer with two backward passes)",
+                 timer="linear_ghost_norm", bound="mfma", work_per_step=flops, unit="TFLOP/s",
+                 peak=MFMA_BF16_PEAK_TFLOPS, traffic=traffic, **({"traffic_source": traffic_source} if traffic else {}))
+    out = dict(
         step=step, n=n, dtype="bf16", workload=desc + (", one backward pass (library default)" if single else ", two backward passes (single_backward=False)"),
         extra={"ghost_norm_executed_flops_per_step": flops, "single_backward": single},
-        roofline=dict(kernel="ghost_norm_multi_kernel<128x128, 2 stages> (all Linear layers of a step pooled into one launch; thin layers by linear_dlds_kernel; "
-                             "ghost_norm_bf16_dlds_kernel layer by layer with two backward passes)",
-                      timer="linear_ghost_norm", bound="mfma", work_per_step=flops, unit="TFLOP/s",
-                      peak=MFMA_BF16_PEAK_TFLOPS, traffic=traffic, **({"traffic_source": traffic_source} if traffic else {})),
+        roofline=ghost,
     )
+    if single:
+        # with one backward pass the clipped sums are this library's kernel too, and the longer of the two
+        wsum_flops = sum(2.0 * n * T * m.in_features * m.out_features for m in net.modules() if isinstance(m, nn.Linear))
+        out["roofline"] = dict(
+            kernel="linear_wsum_multi_kernel<256x256> (clip-weighted sums of all Linear layers in one pooled launch; "
+                   "linear_dlds_kernel<.., weighted> layer by layer, cut into pieces, for a small pool)",
+            timer="linear_weighted_sum", bound="mfma", work_per_step=wsum_flops, unit="TFLOP/s", peak=MFMA_BF16_PEAK_TFLOPS,
+            traffic=wsum_traffic, **({"traffic_source": wsum_traffic_source} if wsum_traffic else {}))
+        out["roofline_also"] = {"roofline_ghost_norm": ghost}
+        out["extra"]["weighted_sum_flops_per_step"] = wsum_flops
+    return out
 
 
 def workload_c3(dev, single=True):
@@ -306,6 +319,9 @@ def workload_c3(dev, single=True):
         # HBM bytes of the pooled launch (operands of both layers: 335.5 MB must be read once)
         traffic=367497514 if single else None,
         traffic_source="recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of bench.py --workload c3, profiles/ghost_norm_multi_mlp_b32_t512_hbm_traffic.txt (not re-measured by this run)",
+        # per launch (one layer: 167.8 MB of operands read once, 67.1 MB of fp32 piece sums written)
+        wsum_traffic=319112972,
+        wsum_traffic_source="recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of bench.py --workload c3, profiles/weighted_sum_mlp_b32_t512_hbm_traffic.txt (not re-measured by this run)",
     )
 
 
@@ -334,6 +350,12 @@ def workload_c5(dev, tied=False, single=True):
         traffic=12127785930 if single and not tied else None,
         traffic_source="recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of bench.py --workload c5, "
                        "profiles/ghost_norm_multi_llama_b16_t1024_hbm_traffic.txt (not re-measured by this run)",
+        # the pooled launch: 5.88 GB of operands and 0.49 GB of results must move once; a tile streams 256
+        # columns of both operands over all 16384 rows, and the narrow operand of a layer (67 MB, which
+        # stays in the 256 MB last-level cache) is fetched again by every row of tiles
+        wsum_traffic=16254303153 if not tied else None,
+        wsum_traffic_source="recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of bench.py --workload c5, "
+                            "profiles/weighted_sum_multi_llama_b16_t1024_hbm_traffic.txt (not re-measured by this run)",
     )
 
 
@@ -767,7 +789,7 @@ def run_workload(name: str, dev, steps: int, warmup: int, all_timers: bool = Fal
         del src, dst
     torch.cuda.synchronize()
     # HIP events around the dominant kernel's entry point only, unless every entry point is asked for
-    only = None if all_timers else {w["roofline"]["timer"]}
+    only = None if all_timers else {w["roofline"]["timer"]} | {r["timer"] for r in w.get("roofline_also", {}).values()}
     marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]  # step boundaries on the launch stream
     with kernels.record_kernel_times(only=only) as times:
         t0 = time.perf_counter()
@@ -780,28 +802,36 @@ def run_workload(name: str, dev, steps: int, warmup: int, all_timers: bool = Fal
     per_step = sorted(a.elapsed_time(b) for a, b in zip(marks, marks[1:]))
 
     kernel_ms = {k: sum(s.elapsed_time(e) for s, e in v) / steps for k, v in times.items()}
-    r = dict(w["roofline"])
-    spans = [s.elapsed_time(e) for s, e in times.get(r.pop("timer"), [])]
-    if "work_per_step" in r:  # several launches per step share the work figure
-        work, ms = r.pop("work_per_step"), sum(spans) / steps
-        r["launches_per_step"] = len(spans) // steps
-    else:
-        work, ms = r.pop("work_per_launch"), sum(spans) / max(len(spans), 1)
-    scale = 1e9 if r["unit"] == "GB/s" else 1e12
-    achieved = work / (ms * 1e-3) / scale if ms > 0 else 0.0
-    roofline = {
-        "kernel": r["kernel"], "bound": r["bound"], "achieved": achieved, "peak": r["peak"], "unit": r["unit"],
-        "frac": achieved / r["peak"], "traffic": r["traffic"], "algorithmic_work": work, "kernel_ms": ms,
-    }
-    for key in ("traffic_source", "launches_per_step"):
-        if key in r:
-            roofline[key] = r[key]
+
+    def roof(spec: dict) -> dict:
+        r = dict(spec)
+        spans = [s.elapsed_time(e) for s, e in times.get(r.pop("timer"), [])]
+        if "work_per_step" in r:  # several launches per step share the work figure
+            work, ms = r.pop("work_per_step"), sum(spans) / steps
+            r["launches_per_step"] = len(spans) // steps
+        else:
+            work, ms = r.pop("work_per_launch"), sum(spans) / max(len(spans), 1)
+        scale = 1e9 if r["unit"] == "GB/s" else 1e12
+        achieved = work / (ms * 1e-3) / scale if ms > 0 else 0.0
+        out = {
+            "kernel": r["kernel"], "bound": r["bound"], "achieved": achieved, "peak": r["peak"], "unit": r["unit"],
+            "frac": achieved / r["peak"], "traffic": r["traffic"], "algorithmic_work": work, "kernel_ms": ms,
+        }
+        for key in ("traffic_source", "launches_per_step"):
+            if key in r:
+                out[key] = r[key]
+        return out
+
+    roofline = roof(w["roofline"])
+    extra = dict(w["extra"])
+    for key, spec in w.get("roofline_also", {}).items():  # the configuration's other contraction kernel
+        extra[key] = roof(spec)
     return {
         "workload": w["workload"], "dtype": w["dtype"], "global_batch": w["n"], "steps": steps, "warmup": warmup,
         "ms_per_step": elapsed / steps * 1e3, "samples_per_s": w["n"] * steps / elapsed,
         # the middle step's span on the device: a single stalled step moves the mean of a short run, not this
         "ms_per_step_median": per_step[len(per_step) // 2] if per_step else None,
-        "kernel_ms_per_step": kernel_ms, "extra": w["extra"], "roofline": roofline,
+        "kernel_ms_per_step": kernel_ms, "extra": extra, "roofline": roofline,
     }
 
 
