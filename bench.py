@@ -347,13 +347,13 @@ def workload_c5(dev, tied=False, single=True):
         # HBM bytes of the pooled launch (21 layers by the Gram route; their operands, 5.21 GB, must be
         # read once; a unit streams two 128-row blocks of both operands and the 4 MB L2 of an XCD does not
         # hold a sample's rows of the wide layers, so the units re-fetch from the last-level cache)
-        traffic=12127785930 if single and not tied else None,
+        traffic=11668405623 if single and not tied else None,
         traffic_source="recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of bench.py --workload c5, "
                        "profiles/ghost_norm_multi_llama_b16_t1024_hbm_traffic.txt (not re-measured by this run)",
         # the pooled launch: 5.88 GB of operands and 0.49 GB of results must move once; a tile streams 256
         # columns of both operands over all 16384 rows, and the narrow operand of a layer (67 MB, which
         # stays in the 256 MB last-level cache) is fetched again by every row of tiles
-        wsum_traffic=16254303153 if not tied else None,
+        wsum_traffic=14198920205 if not tied else None,
         wsum_traffic_source="recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of bench.py --workload c5, "
                             "profiles/weighted_sum_multi_llama_b16_t1024_hbm_traffic.txt (not re-measured by this run)",
     )

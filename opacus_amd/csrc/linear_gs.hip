@@ -367,7 +367,8 @@ struct WsumMultiArgs {
   void* out[kWsumMax];
   int64_t rows[kWsumMax];       // n * T
   int32_t unit_rows[kWsumMax];  // T
-  int32_t M[kWsumMax], N[kWsumMax], tiles_n[kWsumMax];
+  int32_t M[kWsumMax], N[kWsumMax];
+  int32_t tiles_n[kWsumMax];  // tiles along N, columns of tiles varying fastest; or minus the tiles along M, rows fastest
   uint32_t tile_prefix[kWsumMax + 1];
   float scale[kWsumMax];
   int32_t nlayers;
@@ -381,10 +382,16 @@ __global__ __launch_bounds__(C::kThreads, 2) void linear_wsum_multi_kernel(const
   const uint32_t bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
   int l = 0;
   while (l + 1 < A.nlayers && bid >= A.tile_prefix[l + 1]) ++l;
-  const uint32_t rem = bid - A.tile_prefix[l], tn = static_cast<uint32_t>(A.tiles_n[l]);
+  // Tiles that run at the same time on an XCD should need few operand panels between them: with
+  // the shorter tile dimension varying fastest, a CU-count's worth of consecutive tiles is a
+  // block of a few rows by a few columns rather than a strip across the wide dimension.
+  const uint32_t rem = bid - A.tile_prefix[l];
+  const int32_t tn = A.tiles_n[l];  // negative: rows of tiles vary fastest, -tn rows
+  const uint32_t tm_i = tn > 0 ? rem / static_cast<uint32_t>(tn) : rem % static_cast<uint32_t>(-tn);
+  const uint32_t tn_i = tn > 0 ? rem % static_cast<uint32_t>(tn) : rem / static_cast<uint32_t>(-tn);
   linear_dlds_tile<TrBf16, C, TOUT, true>(sm, red, A.b[l], A.a[l], static_cast<TOUT*>(A.out[l]), nullptr, 0u, A.rows[l],
-                                          A.M[l], A.N[l], A.scale[l], static_cast<int64_t>(rem / tn) * C::BQ,
-                                          static_cast<int64_t>(rem % tn) * C::BP, A.coef[l], A.unit_rows[l]);
+                                          A.M[l], A.N[l], A.scale[l], static_cast<int64_t>(tm_i) * C::BQ,
+                                          static_cast<int64_t>(tn_i) * C::BP, A.coef[l], A.unit_rows[l]);
 }
 
 using DldsF32Cfg = mf32d::Config<2, 2, 2, 2, 4>;  // 128 x 128, 4 waves, 64 KB: two blocks per CU
@@ -852,7 +859,8 @@ extern "C" int dpk_linear_weighted_sum_multi(const dpk_wsum_layer* layers, int c
       A.unit_rows[i] = static_cast<int32_t>(L.T);
       A.M[i] = static_cast<int32_t>(L.out);
       A.N[i] = static_cast<int32_t>(L.in);
-      A.tiles_n[i] = static_cast<int32_t>(dpk_cdiv(L.in, tile));
+      const int32_t tm = static_cast<int32_t>(dpk_cdiv(L.out, tile)), tn = static_cast<int32_t>(dpk_cdiv(L.in, tile));
+      A.tiles_n[i] = tm < tn ? -tm : tn;  // the shorter dimension varies fastest
       A.scale[i] = L.scale;
       total += dpk_cdiv(L.out, tile) * dpk_cdiv(L.in, tile);
       DPK_REQUIRE(total <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: %lld blocks exceed the grid limit", who, (long long)total);
