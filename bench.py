@@ -195,8 +195,8 @@ def workload_c2(dev):
             bound="hbm", work_per_launch=float(N * P * 4 + P * 4), unit="GB/s", peak=HBM_PEAK_GBS,
             # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (KiB per
             # dispatch), each scaled by what the counter reads for a 1 GiB device copy
-            # (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000): 8,390,260 + 65,551 KiB over the two dispatches.
-            traffic=8455811 * 1024,
+            # (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000): 8,390,265 + 65,551 KiB over the two dispatches.
+            traffic=8455816 * 1024,
             traffic_source="recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, "
                            "profiles/clip_accumulate_linear4096_b128_hbm_traffic.txt (not re-measured by this run)",
         ),
@@ -237,7 +237,7 @@ def workload_c1(dev, autograd_weight_grads=False):
              bound="hbm", work_per_launch=float(n * P * 4 + P * 4), unit="GB/s", peak=HBM_PEAK_GBS,
              # scaled with the copy kernel's factor (FETCH_SIZE x 2.000); this kernel's short row pieces may be
              # fetched in requests the counter sizes correctly, in which case the true figure is half
-             traffic=53396703,
+             traffic=53396593,
              traffic_source="recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of bench.py --workload c1, profiles/clip_accumulate_small_cnn_b256_hbm_traffic.txt (not re-measured by this run)"),
         autograd_weight_grads=autograd_weight_grads,
     )
@@ -253,7 +253,7 @@ def workload_c4(dev, autograd_weight_grads=False):
         dict(kernel="conv2d_gs_patch_kernel<64,64,float,float>", timer="conv2d_gs", bound="mfma",
              work_per_launch=flops, unit="TFLOP/s", peak=MFMA_FP32_PEAK_TFLOPS,
              # inputs 134.2 MB + per-sample gradients 37.7 MB = 172.0 MB must move once
-             traffic=174316050,
+             traffic=174364893,
              traffic_source="recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of bench.py --workload c4, profiles/conv2d_gs_resblock_b256_hbm_traffic.txt (not re-measured by this run)"),
         autograd_weight_grads=autograd_weight_grads,
     )
@@ -317,10 +317,10 @@ def workload_c3(dev, single=True):
         "MLP Linear(1024->4096) GELU Linear(4096->1024), bf16, batch 32, T=512, ghost clipping, C=1, sigma=1",
         single=single,
         # HBM bytes of the pooled launch (operands of both layers: 335.5 MB must be read once)
-        traffic=367497514 if single else None,
+        traffic=367683253 if single else None,
         traffic_source="recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of bench.py --workload c3, profiles/ghost_norm_multi_mlp_b32_t512_hbm_traffic.txt (not re-measured by this run)",
         # per launch (one layer: 167.8 MB of operands read once, 67.1 MB of fp32 piece sums written)
-        wsum_traffic=319112972,
+        wsum_traffic=319111020,
         wsum_traffic_source="recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of bench.py --workload c3, profiles/weighted_sum_mlp_b32_t512_hbm_traffic.txt (not re-measured by this run)",
     )
 
@@ -347,13 +347,13 @@ def workload_c5(dev, tied=False, single=True):
         # HBM bytes of the pooled launch (21 layers by the Gram route; their operands, 5.21 GB, must be
         # read once; a unit streams two 128-row blocks of both operands and the 4 MB L2 of an XCD does not
         # hold a sample's rows of the wide layers, so the units re-fetch from the last-level cache)
-        traffic=11668405623 if single and not tied else None,
+        traffic=11823073150 if single and not tied else None,
         traffic_source="recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of bench.py --workload c5, "
                        "profiles/ghost_norm_multi_llama_b16_t1024_hbm_traffic.txt (not re-measured by this run)",
         # the pooled launch: 5.88 GB of operands and 0.49 GB of results must move once; a tile streams 256
         # columns of both operands over all 16384 rows, and the narrow operand of a layer (67 MB, which
         # stays in the 256 MB last-level cache) is fetched again by every row of tiles
-        wsum_traffic=14198920205 if not tied else None,
+        wsum_traffic=14198920269 if not tied else None,
         wsum_traffic_source="recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of bench.py --workload c5, "
                             "profiles/weighted_sum_multi_llama_b16_t1024_hbm_traffic.txt (not re-measured by this run)",
     )
