@@ -14,7 +14,10 @@ timed on this box's host cores on a bounded sample of the same workload.
 The headline fields are config 2's. The same run then times the other four benchmark
 configurations (c1, c3, c4, c5: full DP-SGD steps through the drop-in API, at most 20
 steps each, 10 for c5) and reports them under ``"configs"``, each with its own
-``ms_per_step``, ``samples_per_s``, ``roofline`` and bounded-sample ``cpu_baseline``
+``ms_per_step``, ``samples_per_s``, ``roofline`` and bounded-sample ``cpu_baseline``.
+Beside every configuration (the headline included) ``plain_step`` is the same model, batch and
+loss without any DP wrapper (forward + backward + SGD), timed in the same process with the same
+loop, and ``dp_over_plain`` the ratio of the two step times
 (c5 also with embedding table and LM head tied, which the reference refuses under ghost
 clipping, as ``tied_embeddings``).
 ``--workload cN`` times one configuration alone (same JSON shape, no ``configs``);
@@ -26,6 +29,7 @@ fraction of its roofline).
 from __future__ import annotations
 
 import argparse
+import copy
 import json
 import os
 import sys
@@ -181,9 +185,21 @@ def workload_c2(dev):
         model(x).backward(b)  # backprops ~ N(0,1) injected at the layer output
         opt.step()
 
+    def plain():
+        torch.manual_seed(0)
+        ref = nn.Linear(D_IN, D_OUT, bias=True).to(dev)
+        sgd = torch.optim.SGD(ref.parameters(), lr=0.05)
+
+        def plain_step():
+            sgd.zero_grad(set_to_none=True)
+            ref(x).backward(b)
+            sgd.step()
+
+        return plain_step
+
     P = D_OUT * D_IN + D_OUT
     return dict(
-        step=step, n=N, dtype="f32",
+        step=step, plain=plain, n=N, dtype="f32",
         workload="Linear(4096->4096, bias) fp32, batch 128, T=1, hooks per-sample grad + clip(C=1) + noise(sigma=1) + SGD",
         extra={"per_sample_grad_bytes": N * P * 4},
         # one call covers weight and bias: reads n * P * 4 bytes, writes P * 4 bytes. The timed span
@@ -210,6 +226,7 @@ def _hooks_workload(dev, net, x, y, n, sigma, desc, roofline, dtype="f32", autog
     from opacus_amd import GradSampleModule
     from opacus_amd.optimizers import DPOptimizer
 
+    plain_net = copy.deepcopy(net)
     model = GradSampleModule(net.to(dev), loss_reduction="mean", autograd_weight_grads=autograd_weight_grads)
     desc += "" if autograd_weight_grads else ", autograd_weight_grads=False"
     opt = DPOptimizer(
@@ -222,7 +239,18 @@ def _hooks_workload(dev, net, x, y, n, sigma, desc, roofline, dtype="f32", autog
         F.cross_entropy(model(x), y).backward()
         opt.step()
 
-    return dict(step=step, n=n, dtype=dtype, workload=desc, extra={"autograd_weight_grads": autograd_weight_grads},
+    def plain():
+        ref = plain_net.to(dev)
+        sgd = torch.optim.SGD(ref.parameters(), lr=0.1)
+
+        def plain_step():
+            sgd.zero_grad(set_to_none=True)
+            F.cross_entropy(ref(x), y).backward()
+            sgd.step()
+
+        return plain_step
+
+    return dict(step=step, plain=plain, n=n, dtype=dtype, workload=desc, extra={"autograd_weight_grads": autograd_weight_grads},
                 roofline=roofline)
 
 
@@ -260,10 +288,11 @@ def workload_c4(dev, autograd_weight_grads=False):
 
 
 def _ghost_workload(dev, net, make_inputs, loss_call, n, T, sigma, desc, single=True, traffic=None, traffic_source=None,
-                    wsum_traffic=None, wsum_traffic_source=None):
+                    wsum_traffic=None, wsum_traffic_source=None, plain_loss=None):
     from opacus_amd import GradSampleModuleFastGradientClipping
     from opacus_amd.optimizers import DPOptimizerFastGradientClipping
 
+    plain_net = copy.deepcopy(net)
     net = net.to(dev).bfloat16()
     model = GradSampleModuleFastGradientClipping(net, loss_reduction="mean", max_grad_norm=1.0, single_backward=single)
     opt = DPOptimizerFastGradientClipping(
@@ -276,13 +305,24 @@ def _ghost_workload(dev, net, make_inputs, loss_call, n, T, sigma, desc, single=
         loss_call(model, opt, inputs).backward()
         opt.step()
 
+    def plain():
+        ref = plain_net.to(dev).bfloat16()
+        sgd = torch.optim.SGD(ref.parameters(), lr=0.01)
+
+        def plain_step():
+            sgd.zero_grad(set_to_none=True)
+            plain_loss(ref, inputs).backward()
+            sgd.step()
+
+        return plain_step
+
     flops = ghost_executed_flops(net, n, T)
     ghost = dict(kernel="ghost_norm_multi_kernel<128x128, 2 stages> (all Linear layers of a step pooled into one launch; thin layers by linear_dlds_kernel; "
                         "ghost_norm_bf16_dlds_kernel layer by layer with two backward passes)",
                  timer="linear_ghost_norm", bound="mfma", work_per_step=flops, unit="TFLOP/s",
                  peak=MFMA_BF16_PEAK_TFLOPS, traffic=traffic, **({"traffic_source": traffic_source} if traffic else {}))
     out = dict(
-        step=step, n=n, dtype="bf16", workload=desc + (", one backward pass (library default)" if single else ", two backward passes (single_backward=False)"),
+        step=step, plain=plain, n=n, dtype="bf16", workload=desc + (", one backward pass (library default)" if single else ", two backward passes (single_backward=False)"),
         extra={"ghost_norm_executed_flops_per_step": flops, "single_backward": single},
         roofline=ghost,
     )
@@ -315,7 +355,7 @@ def workload_c3(dev, single=True):
     return _ghost_workload(
         dev, net, lambda: torch.randn(n, T, 1024).to(dev).bfloat16(), loss_call, n, T, 1.0,
         "MLP Linear(1024->4096) GELU Linear(4096->1024), bf16, batch 32, T=512, ghost clipping, C=1, sigma=1",
-        single=single,
+        single=single, plain_loss=lambda ref, x: PerSampleMSE("mean")(ref(x)),
         # HBM bytes of the pooled launch (operands of both layers: 335.5 MB must be read once)
         traffic=367683253 if single else None,
         traffic_source="recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of bench.py --workload c3, profiles/ghost_norm_multi_mlp_b32_t512_hbm_traffic.txt (not re-measured by this run)",
@@ -344,6 +384,7 @@ def workload_c5(dev, tied=False, single=True):
         f"4-layer Llama-style decoder (d 2048, 16 heads / 4 KV, SwiGLU 5632, vocab 32000, {'tied' if tied else 'untied'}), "
         "bf16, batch 16, seq 1024, ghost clipping, C=1, sigma=0.8",
         single=single,
+        plain_loss=lambda ref, ids: F.cross_entropy(ref(ids)[:, :-1].reshape(-1, V).float(), ids[:, 1:].reshape(-1)),
         # HBM bytes of the pooled launch (21 layers by the Gram route; their operands, 5.21 GB, must be
         # read once; a unit streams two 128-row blocks of both operands and the 4 MB L2 of an XCD does not
         # hold a sample's rows of the wide layers, so the units re-fetch from the last-level cache)
@@ -773,7 +814,8 @@ def kernel_table(dev, iters: int = 10, warm: int = 3, with_cpu: bool = True):
               2.0 * n * 32 * 256 * 25)
 
 
-def run_workload(name: str, dev, steps: int, warmup: int, all_timers: bool = False, calibrate_copy: bool = False) -> dict:
+def run_workload(name: str, dev, steps: int, warmup: int, all_timers: bool = False, calibrate_copy: bool = False,
+                 with_plain: bool = False) -> dict:
     """``warmup`` untimed steps, then ``steps`` timed steps of one configuration between device
     synchronisations; HIP events on the launch stream around the roofline kernel's entry point."""
     from opacus_amd import kernels
@@ -824,6 +866,9 @@ def run_workload(name: str, dev, steps: int, warmup: int, all_timers: bool = Fal
 
     roofline = roof(w["roofline"])
     extra = dict(w["extra"])
+    plain = None
+    if with_plain and "plain" in w:
+        plain = time_plain_step(w, steps, warmup)
     for key, spec in w.get("roofline_also", {}).items():  # the configuration's other contraction kernel
         extra[key] = roof(spec)
     return {
@@ -831,8 +876,31 @@ def run_workload(name: str, dev, steps: int, warmup: int, all_timers: bool = Fal
         "ms_per_step": elapsed / steps * 1e3, "samples_per_s": w["n"] * steps / elapsed,
         # the middle step's span on the device: a single stalled step moves the mean of a short run, not this
         "ms_per_step_median": per_step[len(per_step) // 2] if per_step else None,
-        "kernel_ms_per_step": kernel_ms, "extra": extra, "roofline": roofline,
+        "kernel_ms_per_step": kernel_ms, "extra": extra, "roofline": roofline, "plain_step": plain,
     }
+
+
+def time_plain_step(w: dict, steps: int, warmup: int) -> dict:
+    """The same network, batch and loss without any wrapper: forward, backward, SGD (the switch
+    --disable-dp of the reference's examples/vision_benchmark.py:65, 259), timed in this process by
+    the loop that times the DP step: ``warmup`` untimed steps, ``steps`` timed ones between device
+    synchronisations."""
+    step = w["plain"]()
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    t0 = time.perf_counter()
+    marks[0].record()
+    for i in range(steps):
+        step()
+        marks[i + 1].record()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    per_step = sorted(a.elapsed_time(b) for a, b in zip(marks, marks[1:]))
+    return {"ms_per_step": elapsed / steps * 1e3, "ms_per_step_median": per_step[len(per_step) // 2],
+            "samples_per_s": w["n"] * steps / elapsed, "steps": steps, "warmup": warmup,
+            "what": "same model, batch and loss, no DP wrapper: forward + backward + SGD"}
 
 
 # Steps of the other configurations inside the default run: enough for a stable mean, few
@@ -849,6 +917,8 @@ def main() -> None:
                     help="time this configuration alone (default: c2 as the headline, then c1, c3, c4, c5 under 'configs')")
     ap.add_argument("--headline-only", action="store_true", help="config 2 only, without the 'configs' object")
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timings")
+    ap.add_argument("--no-plain-step", action="store_true",
+                    help="skip timing the same model without DP (plain_step) beside each configuration")
     ap.add_argument("--all-kernel-timers", action="store_true",
                     help="HIP-event timers around every entry point of the library (kernel_ms_per_step lists them all); "
                          "by default only the roofline kernel's entry point is timed")
@@ -876,7 +946,8 @@ def main() -> None:
             print(json.dumps(r), flush=True)
         return
     head_name = args.workload or "c2"
-    head = run_workload(head_name, dev, args.steps, args.warmup, args.all_kernel_timers, args.calibrate_copy)
+    head = run_workload(head_name, dev, args.steps, args.warmup, args.all_kernel_timers, args.calibrate_copy,
+                        with_plain=not args.no_plain_step)
     out = {
         "metric": "dp_sgd_step_samples_per_sec",
         "value": head["samples_per_s"],
@@ -895,6 +966,9 @@ def main() -> None:
                    **head["extra"]},
         "roofline": head["roofline"],
     }
+    if head["plain_step"]:
+        out["plain_step"] = head["plain_step"]
+        out["dp_over_plain"] = head["ms_per_step"] / head["plain_step"]["ms_per_step"]
     cpu_ok = not args.no_cpu_baseline and head_name.rstrip("stdp") in ("c1", "c2", "c3", "c4", "c5")
     if cpu_ok:
         out["cpu_baseline"] = cpu_baseline(head_name.rstrip("stdp"))
@@ -903,10 +977,13 @@ def main() -> None:
         for name, (k, wu) in OTHER_CONFIGS.items():
             torch.cuda.empty_cache()
             k, wu = min(k, args.steps), min(wu, max(args.warmup, 1))
-            r = run_workload(name, dev, k, wu, args.all_kernel_timers)
+            r = run_workload(name, dev, k, wu, args.all_kernel_timers, with_plain=not args.no_plain_step)
             entry = {key: r[key] for key in ("workload", "dtype", "global_batch", "steps", "warmup", "ms_per_step",
                                              "ms_per_step_median", "samples_per_s", "roofline")}
             entry.update(r["extra"])
+            if r["plain_step"]:
+                entry["plain_step"] = r["plain_step"]
+                entry["dp_over_plain"] = r["ms_per_step"] / r["plain_step"]["ms_per_step"]
             if name + "p" in WORKLOADS:  # the same configuration with the reference's two backward passes
                 d = run_workload(name + "p", dev, k, wu, args.all_kernel_timers)
                 entry["two_backward_passes"] = {"ms_per_step": d["ms_per_step"], "ms_per_step_median": d["ms_per_step_median"],

@@ -21,9 +21,13 @@ second pass would have left in ``p.grad`` (the gradient of ``sum_n coef[n] loss[
 in the per-sample backprops); what is saved is the pass's walk back through the activations,
 at the price of keeping the backprops alive until the coefficients exist (the first pass no
 longer retains the graph, so the peak is about that of the reference's retained graph).
-``single_backward=False`` runs the reference's two passes (fast_gradient_clipping_utils.py:179-201);
-it is the one to use when the loss depends on trainable parameters other than through the
-hooked layers, since only autograd's second pass sees such a dependence.
+``single_backward=False`` runs the reference's two passes (fast_gradient_clipping_utils.py:179-201).
+Only autograd's second pass sees a dependence of the loss on trainable parameters other than
+through the hooked layers (a regulariser on the weights, ``F.linear(x, layer.weight)`` beside the
+layer's own call). ``single_pass_is_exact`` therefore walks the loss's graph before every first
+pass and compares, parameter by parameter, the uses autograd has recorded with the uses the
+forward hooks have seen; a step whose graph holds any other use runs the reference's two passes
+(with one warning), so the default never drops a gradient term.
 
 Norm samples are kept in float32 whatever the dtype of the backprops (the kernels
 accumulate in fp32; rounding a norm to bf16 before it meets the other parameters' norms
@@ -195,6 +199,47 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
         self._first_pass_leaves = {}
         self._first_pass_open = False
         return leaves
+
+    # ---- is the clipped sum of the hooked layers the whole gradient? ------------------------
+    def single_pass_is_exact(self, root: torch.Tensor) -> bool:
+        """True when every use of a trainable parameter in the graph of ``root`` (the reduced
+        loss) is one that a forward hook has seen, i.e. when the clipped sums formed from the
+        hooked layers' (activations, backprops) are all that the reference's second pass would
+        leave in ``p.grad`` (fast_gradient_clipping_utils.py:193-201).
+
+        Autograd keeps one accumulation node per leaf, with one incoming edge per use of the leaf.
+        A hooked layer's call uses each of its own parameters once, and the forward hooks count
+        the calls in ``p._forward_counter``. More edges than calls (a regulariser on the weights,
+        a functional use beside the layer's own), or a trainable leaf that no hooked layer owns,
+        means a term that only a second pass would differentiate. A layer that uses a parameter
+        several times per call is reported as inexact too, which costs that model the second pass
+        and nothing else."""
+        fn = root.grad_fn
+        if fn is None:
+            return True
+        own = {id(p): p for p in self.trainable_parameters}
+        uses = {}
+        seen = {fn}
+        stack = [fn]
+        while stack:
+            node = stack.pop()
+            for nxt, _ in node.next_functions:
+                if nxt is None:
+                    continue
+                var = getattr(nxt, "variable", None)
+                if var is not None:  # an accumulation node: one edge = one use of the leaf
+                    if var.requires_grad:
+                        uses[id(var)] = uses.get(id(var), 0) + 1
+                        if id(var) not in own and isinstance(var, nn.Parameter):
+                            return False  # a trainable parameter outside the wrapped module's hooked layers
+                elif nxt not in seen:
+                    seen.add(nxt)
+                    stack.append(nxt)
+        for pid, count in uses.items():
+            p = own.get(pid)
+            if p is not None and count > getattr(p, "_forward_counter", 0):
+                return False
+        return True
 
     # ---- Linear ghost norms of a whole pass in one launch ----------------------------------
     def _defer_linear_ghost_norm(self, module: nn.Module, activations, backprops: torch.Tensor, scale: float):

@@ -50,14 +50,8 @@ class DPTensorFastGradientAdaptiveClipping(DPTensorFastGradientClipping):
         self.initial_clipping_norm = self.optimizer.max_grad_norm
         self.initial_noise_multiplier = initial_noise_multiplier
 
-    def backward(self):
-        if self.loss_reduction == "mean":
-            reduced = torch.mean(self.loss_per_sample, dim=0)
-        elif self.loss_reduction == "sum":
-            reduced = torch.sum(self.loss_per_sample, dim=0)
-        else:
-            raise ValueError(f"loss_reduction = {self.loss_reduction}. Only 'sum' and 'mean' losses are supported")
-        single = getattr(self.module, "single_backward", False) is True
+    def _backward(self, reduced: torch.Tensor, single: bool) -> None:
+        # (the base class's backward() reduces the loss and decides between one pass and two)
         first_pass_backward(self.module, reduced, retain_graph=not single)
         self.optimizer.zero_grad()
 

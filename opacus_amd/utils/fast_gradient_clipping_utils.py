@@ -6,6 +6,7 @@ Mirror of opacus/utils/fast_gradient_clipping_utils.py.
 from __future__ import annotations
 
 import copy
+import warnings
 
 import torch
 
@@ -25,6 +26,22 @@ def first_pass_backward(module, reduced: torch.Tensor, retain_graph: bool = True
         torch.autograd.grad(reduced, list(inputs), retain_graph=retain_graph, allow_unused=True)
     else:
         reduced.backward(retain_graph=retain_graph)
+
+
+_warned_two_passes = False
+
+
+def _warn_two_passes_once() -> None:
+    global _warned_two_passes
+    if not _warned_two_passes:
+        _warned_two_passes = True
+        warnings.warn(
+            "The loss depends on trainable parameters other than through the layers that ghost clipping "
+            "hooks (a regulariser on the weights, a functional use of a layer's weight, a layer that uses "
+            "a parameter more than once per call): such steps run the two backward passes of the reference "
+            "instead of the single pass. Pass single_backward=False to silence this warning.",
+            stacklevel=3,
+        )
 
 
 class DPTensorFastGradientClipping:
@@ -103,6 +120,19 @@ class DPTensorFastGradientClipping:
         else:
             raise ValueError(f"loss_reduction = {self.loss_reduction}. Only 'sum' and 'mean' losses are supported")
         single = getattr(self.module, "single_backward", False) is True
+        if single and not self.module.single_pass_is_exact(reduced):
+            # the loss reaches a trainable parameter other than through a hooked layer: only
+            # autograd's second pass differentiates that term, so this step takes both passes
+            _warn_two_passes_once()
+            self.module.single_backward = False
+            try:
+                self._backward(reduced, single=False)
+            finally:
+                self.module.single_backward = True
+            return
+        self._backward(reduced, single)
+
+    def _backward(self, reduced: torch.Tensor, single: bool) -> None:
         first_pass_backward(self.module, reduced, retain_graph=not single)
         self.optimizer.zero_grad()
         coeff = self.module.get_clipping_coef()

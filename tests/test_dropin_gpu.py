@@ -967,6 +967,56 @@ def test_ghost_single_backward_leaves_the_second_pass_gradients(A, case):
         close(g1 / scale, g2 / scale, 1e-4, 2e-6, f"{case} {name}")
 
 
+@pytest.mark.parametrize("extra", ["regulariser", "functional_use"])
+def test_ghost_loss_terms_outside_the_hooked_layers_keep_their_gradient(A, extra):
+    """A loss with a term that reaches trainable parameters other than through a hooked layer
+    (criterion + regulariser, the ``loss + tensor`` arithmetic of DPTensorFastGradientClipping;
+    a functional use of a layer's weight): the reference's second pass differentiates it with the
+    rest of sum_n coef[n] loss[n] (fast_gradient_clipping_utils.py:193-201). The default
+    (single_backward=True) must leave the same p.grad as single_backward=False: its guard sends
+    such a step through both passes. Checked against fp64 autograd of the weighted loss."""
+    torch.manual_seed(5)
+    net = nn.Sequential(nn.Linear(12, 20), nn.GELU(), nn.Linear(20, 6))
+    x, y = torch.randn(6, 9, 12), torch.randn(6, 9, 6)
+    C = 0.05
+
+    def extra_term(model, xb):
+        if extra == "regulariser":
+            return 0.3 * sum(p.pow(2).sum() for p in model.parameters())
+        inner = model._module if hasattr(model, "_module") else model
+        return 0.2 * F.linear(xb, inner[0].weight).pow(2).flatten(1).mean(1)  # per sample
+
+    def loss_call(model, opt, b):
+        dp_loss = A.DPLossFastGradientClipping(model, opt, PerSampleMSE("mean"), "mean")(model(b[0]), b[1])
+        return dp_loss + extra_term(model, b[0])
+
+    import warnings as _w
+
+    with _w.catch_warnings():
+        _w.simplefilter("ignore")
+        two, _ = _ghost_grads(A, net, (x, y), loss_call, single=False, C=C)
+        one, ghost = _ghost_grads(A, net, (x, y), loss_call, single=True, C=C)
+    assert ghost.single_backward is True and ghost._kept_passes == []
+    # fp64: coefficients from the per-sample norms of the criterion alone (what the hooks see),
+    # then the gradient of sum_n coef[n] * (loss[n] + extra)
+    ref = copy.deepcopy(net).double()
+    gs = per_sample_grads_cpu(ref, x.double(), y.double(), lambda out, t: PerSampleMSE("sum")(out, t))
+    norms = torch.sqrt(sum(g.flatten(1).pow(2).sum(1) for g in gs.values()))
+    coef = (C / (norms + 1e-6)).clamp(max=1.0)
+    ref.zero_grad()
+    per_sample = PerSampleMSE("none")(ref(x.double()), y.double()) + extra_term(ref, x.double())
+    (coef * per_sample).sum().backward()
+    for (name, _), g1, g2, p in zip(ghost.named_parameters(), one, two, ref.parameters()):
+        scale = p.grad.abs().max().item() + 1e-12
+        close(g1 / scale, g2 / scale, 1e-4, 2e-6, f"{extra} {name}: default against two passes")
+        close(g1.double() / scale, p.grad / scale, 1e-4, 1e-5, f"{extra} {name}: against fp64 autograd")
+    # without the extra term the same model takes the single pass (nothing is kept afterwards, no warning)
+    with _w.catch_warnings():
+        _w.simplefilter("error")
+        _ghost_grads(A, net, (x, y), lambda m, o, b: A.DPLossFastGradientClipping(m, o, PerSampleMSE("mean"), "mean")(m(b[0]), b[1]),
+                     single=True, C=C)
+
+
 @pytest.mark.parametrize("bias", [True, False])
 def test_ghost_single_backward_bf16_weighted_contraction(A, bias):
     """A bf16 MLP on sequences whose Linear layers the weighted contraction takes (whole k tiles of

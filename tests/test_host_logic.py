@@ -666,6 +666,72 @@ def test_first_backward_pass_asks_for_the_entry_tensors_only():
     torch.testing.assert_close(w.grad, torch.full((3,), 2.0))
 
 
+def test_single_pass_guard_sees_uses_of_parameters_outside_the_hooked_layers():
+    """The single backward pass rebuilds the clipped sum from the hooked layers alone; the
+    reference's second pass differentiates the whole graph (fast_gradient_clipping_utils.py:193-201).
+    ``single_pass_is_exact`` compares the uses of every trainable parameter that autograd recorded
+    with the layer calls that the forward hooks counted, and ``backward()`` takes two passes when
+    they differ."""
+    torch.manual_seed(0)
+
+    def forget_forward(module):
+        for m in module.modules():
+            m.__dict__.pop("activations", None)
+        for p in module.parameters():
+            p._forward_counter = 0
+
+    class TwoUses(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.fc1, self.ln, self.fc2 = nn.Linear(4, 6), nn.LayerNorm(6), nn.Linear(6, 3)
+
+        def forward(self, x):
+            return self.fc2(self.ln(torch.tanh(self.ln(self.fc1(x)))))  # one layer applied twice
+
+    net = TwoUses()
+    ghost = GradSampleModuleFastGradientClipping(net)
+    x = torch.randn(5, 4)
+    loss = ghost(x).pow(2).sum(1)
+    assert ghost.single_pass_is_exact(loss.mean())
+    # a regulariser on the weights is a use that no hook has seen
+    assert not ghost.single_pass_is_exact((loss + 0.1 * net.fc1.weight.pow(2).sum()).mean())
+    assert not ghost.single_pass_is_exact((loss + 1e-3 * sum(p.pow(2).sum() for p in net.parameters())).mean())
+    # so is a functional use of a hooked layer's weight beside the layer's own call
+    assert not ghost.single_pass_is_exact((loss + F.linear(x, net.fc1.weight).sum(1)).mean())
+    # and a trainable parameter that belongs to no layer of the wrapped module
+    outside = nn.Parameter(torch.ones(()))
+    assert not ghost.single_pass_is_exact((loss * outside).mean())
+    # tensors that are not parameters (an input that requires grad) do not count
+    xg = torch.randn(5, 4, requires_grad=True)
+    forget_forward(net)
+    assert ghost.single_pass_is_exact(ghost(xg).pow(2).sum(1).mean())
+    # a frozen parameter may be used anywhere
+    forget_forward(net)
+    net.fc2.bias.requires_grad_(False)
+    ghost.remove_hooks()
+    ghost = GradSampleModuleFastGradientClipping(net)
+    loss = ghost(x).pow(2).sum(1)
+    assert ghost.single_pass_is_exact((loss + net.fc2.bias.sum()).mean())
+    assert ghost.single_pass_is_exact(torch.zeros(()))  # no graph at all
+
+    # backward(): an inexact step is run with two passes (single_backward is off while its hooks fire)
+    module, optimizer = _mock_pair("sum")
+    module.single_backward = True
+    module.single_pass_is_exact.side_effect = lambda reduced: False
+    seen = []
+    module.get_clipping_coef.side_effect = lambda: (seen.append(module.single_backward), torch.tensor([0.5, 1.0]))[1]
+    w = torch.tensor([1.0, 1.0], requires_grad=True)
+    with pytest.warns(UserWarning, match="two backward passes"):
+        DPTensorFastGradientClipping(module, optimizer, w * torch.tensor([2.0, 3.0]), "sum").backward()
+    assert seen == [False] and module.single_backward is True
+    module.accumulate_clipped_gradients.assert_not_called()
+    torch.testing.assert_close(w.grad, torch.tensor([2.0 + 1.0, 3.0 + 3.0]))  # both passes ran (the mock zeroes nothing)
+    # an exact step takes the single pass
+    module.single_pass_is_exact.side_effect = lambda reduced: True
+    DPTensorFastGradientClipping(module, optimizer, w * torch.tensor([2.0, 3.0]), "sum").backward()
+    module.accumulate_clipped_gradients.assert_called_once()
+
+
 def test_dp_loss_requires_consistent_reductions_and_restores_reduction():
     module, optimizer = _mock_pair("mean")
     crit = nn.CrossEntropyLoss(reduction="mean")
