@@ -104,8 +104,11 @@ int dpk_linear_weighted_sum(const void* b, const void* a, int in_dtype, const fl
 
 /* dpk_linear_weighted_sum for several layers in one call: the block tiles of all layers are
  * one pool of work, so the GPU stays full across layers whose own tile count is not a
- * multiple of what it holds at once (C5: 29 layers, 37 launches -> one). Every layer is
- * contracted in one piece (no workspace); per-layer requirements as above, all results of
+ * multiple of what it holds at once (C5: 29 layers, 37 launches -> one). A pool with too few
+ * tiles to fill the GPU (a two-layer MLP) has every layer's samples cut into 2, 4 or 8 pieces
+ * (dividing every n), whose fp32 sums go to the workspace and are added by one more launch;
+ * dpk_linear_weighted_sum_multi_workspace_bytes says how much the same table will need (0: one
+ * piece). ws must be 256-byte aligned. Per-layer requirements as above, all results of
  * `out_dtype`. `layers` is a host array of any length (32 layers per launch). */
 typedef struct dpk_wsum_layer {
   const void* b;     /* [n,T,out] bf16 */
@@ -115,8 +118,9 @@ typedef struct dpk_wsum_layer {
   int64_t n, T, out, in;
   float scale;
 } dpk_wsum_layer;
+size_t dpk_linear_weighted_sum_multi_workspace_bytes(const dpk_wsum_layer* layers /*host*/, int count);
 int dpk_linear_weighted_sum_multi(const dpk_wsum_layer* layers /*host*/, int count, int in_dtype, int out_dtype,
-                                  dpk_stream_t stream);
+                                  void* ws, size_t ws_bytes, dpk_stream_t stream);
 
 /* gs_bias[n,k] = scale * sum_t b[n,t,k]                   (linear.py:50)
  * sumsq (nullable, float[n]) receives sum_k gs_bias[n,k]^2 of the values as stored, for

@@ -13,7 +13,7 @@ from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "lib" / "libdpsgd_hip.so"
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 DPK_OK = 0
 DPK_F32 = 0
@@ -66,7 +66,8 @@ SIGNATURES = {
     "dpk_linear_weighted_sum": (
         c_int, [_P, _P, c_int, _P, _P, c_int, _I, _I, _I, _I, c_float, c_int, _P, c_size_t, _P]
     ),
-    "dpk_linear_weighted_sum_multi": (c_int, [_P, c_int, c_int, c_int, _P]),
+    "dpk_linear_weighted_sum_multi_workspace_bytes": (c_size_t, [_P, c_int]),
+    "dpk_linear_weighted_sum_multi": (c_int, [_P, c_int, c_int, c_int, _P, c_size_t, _P]),
     "dpk_linear_bias_gs": (c_int, [_P, c_int, _P, c_int, _P, _I, _I, _I, c_float, _P]),
     "dpk_linear_ghost_norm_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
     "dpk_linear_ghost_norm": (c_int, [_P, _P, c_int, _P, _P, _I, _I, _I, _I, c_float, c_int, _P, c_size_t, _P]),

@@ -7,7 +7,7 @@
 
 #include "../../include/dpk.h"
 
-#define DPK_ABI_VERSION 2
+#define DPK_ABI_VERSION 3
 #define DPK_WAVE 64
 
 // ---- host side -------------------------------------------------------------

@@ -119,25 +119,28 @@ __global__ __launch_bounds__(kThreads) void ghost_norm_bf16_kernel(
 //
 // Work units are (sample, tile pair), numbered sample-major. The first nbig units
 // get a block each; when the launch would otherwise end in a thinly filled round
-// of resident blocks, the remaining units are cut into quadrants of 64 x 64 and
-// every quadrant gets a block of its own that splits k over its waves. Unit u
-// writes its partial sums at u * slots (a quadrant at u * slots + quadrant).
-template <class C>
-constexpr bool ghost_cfg_has_quadrants() {
-  return C::BM == 128 && C::BN == 128 && C::BK == 64 && C::kWaves == 4 && C::kStages == 2;
-}
+// of resident blocks, each remaining unit is cut into kGhostPieces pieces that get a
+// block each. A unit cannot be cut along both contractions (it is the sum of the
+// products of two Gram tiles), but it is linear in either Gram alone: piece p forms the
+// longer-contraction Gram over the p-th part of its k range only, the other Gram in
+// full, and the pieces' partial sums add up to the unit's. A piece keeps the 128 x 128
+// tile (the operand bytes per MFMA of a whole unit) and does (K_long / pieces +
+// K_short) / (K_long + K_short) of its work. (Cutting the tile into quadrants of 64 x 64
+// whose waves split k measured worse: a quadrant block alone on a CU took 26 us where
+// the whole unit takes 37.) Unit u writes its partial sums at u * slots (+ piece).
+constexpr int kGhostPieces = 4;
 
-// One work unit: tile pair `pair` of one sample of one layer, as a whole 128 x 128 tile (big) or
-// as quadrant `quad` of it. The partial sums of unit `unit_index` (sample * npairs + pair) go
-// to pw / pb at unit_index * slots (+ quad).
+// One work unit: tile pair `pair` of one sample of one layer, whole (big) or as piece
+// `piece` of it. The partial sums of unit `unit_index` (sample * npairs + pair) go
+// to pw / pb at unit_index * slots (+ piece).
 // TE: bf16_t, or float (a stage row of 128 bytes is then 32 k values).
 template <class C, typename TE>
 __device__ __forceinline__ void ghost_unit(mb16d::Smem<C>& sm, float* red, const TE* __restrict__ bs,
                                            const TE* __restrict__ as, float* __restrict__ pw,
                                            float* __restrict__ pb, int64_t T, int64_t Dout, int64_t Din, int nJ,
-                                           int pair, bool big, uint32_t quad, size_t unit_index, int slots) {
+                                           int pair, bool big, uint32_t piece, size_t unit_index, int slots) {
   constexpr int R = C::BM / C::BN;
-  constexpr bool kQuadrants = ghost_cfg_has_quadrants<C>();
+  constexpr int BKE = C::ROW_BYTES / static_cast<int>(sizeof(TE));  // k values of a stage row
   int I = 0;
   while (pair >= nJ - R * I) {
     pair -= nJ - R * I;
@@ -148,68 +151,55 @@ __device__ __forceinline__ void ghost_unit(mb16d::Smem<C>& sm, float* red, const
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int kh = lane >> 5, l32 = lane & 31;
   float sw = 0.f, sb = 0.f;
-  size_t slot = unit_index * slots;
-  if (big) {
-    const int64_t m0a = static_cast<int64_t>(I) * C::BM, m0b = static_cast<int64_t>(J) * C::BN;
-    const int wm0 = (wave / C::kWaveCols) * 64, wn0 = (wave % C::kWaveCols) * 64;
-    mb16d::Tile tg, ta;
-    tg.clear();
-    ta.clear();
-    mb16d::mainloop<C, TE>(tg, sm, bs, bs, Dout, m0a, m0b, T, Dout, wm0, wn0);
-    if (pw) mb16d::mainloop<C, TE>(ta, sm, as, as, Din, m0a, m0b, T, Din, wm0, wn0);
-    // rows past T hold copies of row T - 1: leave them out
-    const int rmax = static_cast<int>(T - m0a < C::BM ? T - m0a : C::BM);
-    const int cmax = static_cast<int>(T - m0b < C::BN ? T - m0b : C::BN);
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const int row = wm0 + i * 32 + (v >> 2) * 8 + kh * 4 + (v & 3), col = wn0 + j * 32 + l32;
-          if (row < rmax && col < cmax) {
-            const float g = tg.acc[i][j][v];
-            sb += g;
-            sw = fmaf(g, ta.acc[i][j][v], sw);
-          }
-        }
-  } else if constexpr (kQuadrants) {
-    // quadrant (quad >> 1, quad & 1) of the unit's tile; R == 1 on this path
-    const int64_t m0a = static_cast<int64_t>(I) * C::BM + (quad >> 1) * 64;
-    const int64_t m0b = static_cast<int64_t>(J) * C::BN + (quad & 1u) * 64;
-    slot += quad;
-    if (m0a < T && m0b < T) {  // block-uniform
-      mb16d::Tile t;
-      t.clear();
-      mb16d::mainloop_splitk<C, TE>(t, sm, bs, bs, Dout, m0a, m0b, T, Dout);
-      const mb16d::floatx16 g = mb16d::splitk_reduce<C>(t, sm);
-      mb16d::floatx16 h;
-      if (pw) {
-        t.clear();
-        mb16d::mainloop_splitk<C, TE>(t, sm, as, as, Din, m0a, m0b, T, Din);
-        h = mb16d::splitk_reduce<C>(t, sm);
-      }
-      const int rmax = static_cast<int>(T - m0a < 64 ? T - m0a : 64);
-      const int cmax = static_cast<int>(T - m0b < 64 ? T - m0b : 64);
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int row = (wave >> 1) * 32 + (v >> 2) * 8 + kh * 4 + (v & 3), col = (wave & 1) * 32 + l32;
-        if (row < rmax && col < cmax) {
-          sb += g[v];
-          if (pw) sw = fmaf(g[v], h[v], sw);
-        }
-      }
+  const size_t slot = unit_index * slots + (big ? 0u : piece);
+  // the k ranges of the two Grams: whole, or the piece's part of the longer one
+  int64_t kb0 = 0, kb1 = Dout, ka0 = 0, ka1 = Din;
+  bool count_bias = true;
+  if (!big) {
+    const bool split_b = !pw || Dout >= Din;
+    const int64_t nk = (split_b ? Dout : Din) / BKE;
+    const int64_t t0 = nk * piece / kGhostPieces * BKE, t1 = nk * (piece + 1) / kGhostPieces * BKE;
+    if (split_b) {
+      kb0 = t0;
+      kb1 = t1;
+    } else {
+      ka0 = t0;
+      ka1 = t1;
+      count_bias = piece == 0;  // the whole b Gram is formed by every piece: its sum counts once
     }
   }
+  const int64_t m0a = static_cast<int64_t>(I) * C::BM, m0b = static_cast<int64_t>(J) * C::BN;
+  const int wm0 = (wave / C::kWaveCols) * 64, wn0 = (wave % C::kWaveCols) * 64;
+  mb16d::Tile tg, ta;
+  tg.clear();
+  ta.clear();
+  if (kb1 > kb0) mb16d::mainloop<C, TE>(tg, sm, bs + kb0, bs + kb0, Dout, m0a, m0b, T, kb1 - kb0, wm0, wn0);
+  if (pw && ka1 > ka0) mb16d::mainloop<C, TE>(ta, sm, as + ka0, as + ka0, Din, m0a, m0b, T, ka1 - ka0, wm0, wn0);
+  // rows past T hold copies of row T - 1: leave them out
+  const int rmax = static_cast<int>(T - m0a < C::BM ? T - m0a : C::BM);
+  const int cmax = static_cast<int>(T - m0b < C::BN ? T - m0b : C::BN);
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int row = wm0 + i * 32 + (v >> 2) * 8 + kh * 4 + (v & 3), col = wn0 + j * 32 + l32;
+        if (row < rmax && col < cmax) {
+          const float g = tg.acc[i][j][v];
+          sb += g;
+          sw = fmaf(g, ta.acc[i][j][v], sw);
+        }
+      }
   if (pw) {
     const float s = block_sum<C::kWaves>(sw, red);
     if (threadIdx.x == 0) pw[slot] = s * weight;
-    // a whole unit leaves the other quadrant slots empty
+    // a whole unit leaves the other pieces' slots empty
     if (big && slots > 1 && threadIdx.x < slots && threadIdx.x > 0) pw[slot + threadIdx.x] = 0.f;
   }
   if (pb) {
     const float s = block_sum<C::kWaves>(sb, red);
-    if (threadIdx.x == 0) pb[slot] = s * weight;
+    if (threadIdx.x == 0) pb[slot] = count_bias ? s * weight : 0.f;
     if (big && slots > 1 && threadIdx.x < slots && threadIdx.x > 0) pb[slot + threadIdx.x] = 0.f;
   }
 }
@@ -219,18 +209,17 @@ __global__ __launch_bounds__(C::kThreads) void ghost_norm_bf16_dlds_kernel(
     const TE* __restrict__ b, const TE* __restrict__ a, float* __restrict__ pw,
     float* __restrict__ pb, int64_t T, int64_t Dout, int64_t Din, int nJ, int npairs, uint32_t nbig,
     int slots) {
-  constexpr bool kQuadrants = ghost_cfg_has_quadrants<C>();
   __shared__ mb16d::Smem<C> sm;
   __shared__ float red[C::kWaves];
-  const bool big = !kQuadrants || blockIdx.x < nbig;
+  const bool big = blockIdx.x < nbig;
   uint32_t unit, quad = 0;
   if (big) {
     unit = xcd_contiguous_id(blockIdx.x, nbig);
   } else {
     // nbig is a multiple of 8, so the low bits still name the XCD
     const uint32_t sid = xcd_contiguous_id(blockIdx.x - nbig, gridDim.x - nbig);
-    unit = nbig + (sid >> 2);
-    quad = sid & 3u;
+    unit = nbig + sid / kGhostPieces;
+    quad = sid % kGhostPieces;
   }
   const int64_t sample = unit / static_cast<uint32_t>(npairs);
   const int pair = static_cast<int>(unit % static_cast<uint32_t>(npairs));
@@ -242,13 +231,13 @@ __global__ __launch_bounds__(C::kThreads) void ghost_norm_bf16_dlds_kernel(
 // The ghost norms of one layer at a benchmark shape are a launch of a few hundred units on
 // 512 resident blocks: its last round of blocks is mostly empty, and every layer pays that
 // again. Pooled, the units of all layers of a backward pass fill the rounds, and the one
-// tail is cut into quadrant blocks. Layers are given in descending order of feature count,
+// tail is cut into pieces (see above). Layers are given in descending order of feature count,
 // so that every XCD starts with its longest units.
 //
 // Hardware block id i runs on XCD i % 8, and an XCD takes its blocks in id order. XCD x is
 // given the samples [s0[x], s0[x] + cnt[x]) of every layer (units that share a sample's
 // rows share that XCD's L2), layer after layer: `len[x]` units, of which the last `tail[x]`
-// are run as four quadrant blocks each.
+// are run as kGhostPieces blocks each.
 constexpr int kGhostMultiMax = 32;               // layers per launch
 constexpr int kGhostMultiLayers = DPK_GHOST_MULTI_MAX;  // layers per call (several launches)
 
@@ -269,10 +258,10 @@ __global__ __launch_bounds__(C::kThreads) void ghost_norm_multi_kernel(const Gho
   __shared__ float red[C::kWaves];
   const uint32_t x = blockIdx.x & 7u, idx = blockIdx.x >> 3;
   const uint32_t tail = A.tail[x], nbig = A.len[x] - tail;
-  if (idx >= nbig + 4u * tail) return;
+  if (idx >= nbig + kGhostPieces * tail) return;
   const bool big = idx < nbig;
-  const uint32_t u = big ? idx : nbig + ((idx - nbig) >> 2);
-  const uint32_t quad = big ? 0u : ((idx - nbig) & 3u);
+  const uint32_t u = big ? idx : nbig + (idx - nbig) / kGhostPieces;
+  const uint32_t quad = big ? 0u : (idx - nbig) % kGhostPieces;
   const uint32_t cnt = A.cnt[x];
   int l = 0;
   while (l + 1 < A.nlayers && u >= cnt * A.pair_prefix[l + 1]) ++l;
@@ -397,7 +386,7 @@ extern "C" size_t dpk_linear_ghost_norm_workspace_bytes(int64_t n, int64_t T, in
                                                         int64_t in) {
   if (n <= 0 || T <= 1) return 0;
   // Room for any tiling: 64-row tile pairs, or 128-row tile pairs with four
-  // quadrant slots each (2 m^2 + 2 m slots per sample covers both).
+  // piece slots each (2 m^2 + 2 m slots per sample covers both).
   const int64_t m = dpk_cdiv(T, 128);
   const size_t gram = dpk_align_up(static_cast<size_t>(2 * n * (2 * m * m + 2 * m)) * sizeof(float), 256);
   // ... and for the direct route, whichever of the two a call ends up taking
@@ -463,20 +452,19 @@ extern "C" int dpk_linear_ghost_norm(const void* b, const void* a, int dtype, fl
   const bool dlds = dlds_takes(b, a, dtype, norm_w != nullptr, T, out, in);
   const int64_t npairs = dlds ? ghost_pairs(T, GhostCfg::BM, GhostCfg::BN) : nt * (nt + 1) / 2;
   const int64_t blocks = n * npairs;
-  // A last round of resident blocks (two per CU) that is at most a quarter full is
-  // served by quadrant blocks instead, which then fit one round of their own: a lone
-  // tile block per CU runs latency-bound and takes most of a full round's time, a
-  // round of quadrant blocks about a third of it.
+  // The units of a last round of resident blocks (two per CU) that is at most a quarter
+  // full are cut into pieces, which then fit one round of their own: left whole, they
+  // would take a full round's time on a quarter of the CUs.
   int64_t tail = 0;
-  if (dlds && ghost_cfg_has_quadrants<GhostCfg>()) {
+  if (dlds) {
     const int cus = dpk_device_cus();
     DPK_REQUIRE(cus > 0, DPK_E_LAUNCH, "%s: cannot query the device", who);
     const int64_t resident = 2 * static_cast<int64_t>(cus);
     const int64_t r = blocks % resident;
-    if (resident % 8 == 0 && r > 0 && r * 4 <= resident) tail = r;
+    if (resident % 8 == 0 && r > 0 && r * kGhostPieces <= resident) tail = r;
   }
-  const int slots = tail ? 4 : 1;
-  const int64_t grid_blocks = blocks - tail + 4 * tail;
+  const int slots = tail ? kGhostPieces : 1;
+  const int64_t grid_blocks = blocks - tail + kGhostPieces * tail;
   DPK_REQUIRE(nt < 32768 && grid_blocks <= DPK_MAX_GRID_X && blocks * slots <= DPK_MAX_GRID_X, DPK_E_SHAPE,
               "%s: %lld blocks exceed the grid limit", who, (long long)grid_blocks);
   const size_t need = static_cast<size_t>(2 * blocks * slots) * sizeof(float);
@@ -664,12 +652,12 @@ extern "C" int dpk_linear_ghost_norm_multi(const dpk_ghost_layer* layers, int co
       A.cnt[x] = static_cast<uint32_t>((x + 1) * n / 8) - A.s0[x];
       A.len[x] = A.cnt[x] * P;
       const uint32_t r = resident > 0 ? A.len[x] % resident : 0;
-      A.tail[x] = (cus % 8 == 0 && r > 0 && r * 4 <= resident) ? r : 0;
+      A.tail[x] = (cus % 8 == 0 && r > 0 && r * kGhostPieces <= resident) ? r : 0;
       any_tail = any_tail || A.tail[x] > 0;
-      const uint32_t blocks = A.len[x] - A.tail[x] + 4 * A.tail[x];
+      const uint32_t blocks = A.len[x] - A.tail[x] + kGhostPieces * A.tail[x];
       longest = blocks > longest ? blocks : longest;
     }
-    A.slots = any_tail ? 4 : 1;
+    A.slots = any_tail ? kGhostPieces : 1;
     for (int i = 0; i < nl; ++i) {
       const dpk_ghost_layer& L = layers[pooled[c0 + i]];
       float* part = reinterpret_cast<float*>(base + lay_off[pooled[c0 + i]]);

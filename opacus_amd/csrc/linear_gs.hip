@@ -14,6 +14,7 @@
 #include "mfma_f32_dlds.h"
 #include "mfma_f32.h"
 
+#include <cstring>
 #include <type_traits>
 
 namespace {
@@ -369,9 +370,13 @@ struct WsumMultiArgs {
   int32_t unit_rows[kWsumMax];  // T
   int32_t M[kWsumMax], N[kWsumMax];
   int32_t tiles_n[kWsumMax];  // tiles along N, columns of tiles varying fastest; or minus the tiles along M, rows fastest
-  uint32_t tile_prefix[kWsumMax + 1];
+  uint32_t tile_prefix[kWsumMax + 1];  // blocks of the layers before: tiles x pieces
   float scale[kWsumMax];
   int32_t nlayers;
+  // pieces > 1: a layer's samples are cut into that many runs, each with blocks of its own; piece p of
+  // layer l leaves its fp32 sum at part[l] + p * M * N and add_pieces_multi_kernel adds the pieces
+  int32_t pieces;
+  float* part[kWsumMax];
 };
 
 template <class C, typename TOUT>
@@ -385,13 +390,46 @@ __global__ __launch_bounds__(C::kThreads, 2) void linear_wsum_multi_kernel(const
   // Tiles that run at the same time on an XCD should need few operand panels between them: with
   // the shorter tile dimension varying fastest, a CU-count's worth of consecutive tiles is a
   // block of a few rows by a few columns rather than a strip across the wide dimension.
-  const uint32_t rem = bid - A.tile_prefix[l];
+  uint32_t rem = bid - A.tile_prefix[l];
+  const uint32_t per_piece = (A.tile_prefix[l + 1] - A.tile_prefix[l]) / static_cast<uint32_t>(A.pieces);
+  const uint32_t piece = rem / per_piece;  // a piece's tiles are consecutive: its operand rows stay in one L2
+  rem -= piece * per_piece;
   const int32_t tn = A.tiles_n[l];  // negative: rows of tiles vary fastest, -tn rows
   const uint32_t tm_i = tn > 0 ? rem / static_cast<uint32_t>(tn) : rem % static_cast<uint32_t>(-tn);
   const uint32_t tn_i = tn > 0 ? rem % static_cast<uint32_t>(tn) : rem / static_cast<uint32_t>(-tn);
-  linear_dlds_tile<TrBf16, C, TOUT, true>(sm, red, A.b[l], A.a[l], static_cast<TOUT*>(A.out[l]), nullptr, 0u, A.rows[l],
-                                          A.M[l], A.N[l], A.scale[l], static_cast<int64_t>(tm_i) * C::BQ,
-                                          static_cast<int64_t>(tn_i) * C::BP, A.coef[l], A.unit_rows[l]);
+  const int64_t rows = A.rows[l] / A.pieces, row0 = rows * piece;
+  const int64_t M = A.M[l], N = A.N[l];
+  TOUT* out = static_cast<TOUT*>(A.out[l]);
+  if constexpr (std::is_same<TOUT, float>::value) {
+    if (A.pieces > 1) out = A.part[l] + static_cast<int64_t>(piece) * M * N;
+  }
+  linear_dlds_tile<TrBf16, C, TOUT, true>(sm, red, A.b[l] + row0 * M, A.a[l] + row0 * N, out, nullptr, 0u, rows, M, N,
+                                          A.scale[l], static_cast<int64_t>(tm_i) * C::BQ,
+                                          static_cast<int64_t>(tn_i) * C::BP,
+                                          A.coef[l] + row0 / A.unit_rows[l], A.unit_rows[l]);
+}
+
+// out[l][e] = sum_p part[l][p * count + e] for the layers of a pooled launch, four elements per thread.
+struct AddPiecesMultiArgs {
+  const float* part[kWsumMax];
+  void* out[kWsumMax];
+  int64_t count4[kWsumMax];
+  uint32_t block_prefix[kWsumMax + 1];
+  int32_t nlayers, pieces;
+};
+
+template <typename TOUT>
+__global__ __launch_bounds__(kThreads) void add_pieces_multi_kernel(const AddPiecesMultiArgs A) {
+  int l = 0;
+  while (l + 1 < A.nlayers && blockIdx.x >= A.block_prefix[l + 1]) ++l;
+  const int64_t e = static_cast<int64_t>(blockIdx.x - A.block_prefix[l]) * kThreads + threadIdx.x;
+  const int64_t count4 = A.count4[l];
+  if (e >= count4) return;
+  typedef float vf4 __attribute__((ext_vector_type(4)));
+  const vf4* src = reinterpret_cast<const vf4*>(A.part[l]) + e;
+  vf4 sum = __builtin_nontemporal_load(src);
+  for (int p = 1; p < A.pieces; ++p) sum += __builtin_nontemporal_load(src + p * count4);
+  dpk_io<TOUT>::store4(static_cast<TOUT*>(A.out[l]) + 4 * e, make_float4(sum.x, sum.y, sum.z, sum.w));
 }
 
 using DldsF32Cfg = mf32d::Config<2, 2, 2, 2, 4>;  // 128 x 128, 4 waves, 64 KB: two blocks per CU
@@ -811,14 +849,63 @@ extern "C" int dpk_linear_weighted_sum(const void* b, const void* a, int in_dtyp
 }
 
 // The same sums for several layers at once (dpk_wsum_layer records, host array): one launch per
-// group of up to 32 layers whose results share a dtype, every layer in one piece.
+// group of up to 32 layers whose results share a dtype. A pool with too few tiles to fill the GPU
+// in whole rounds of blocks has every layer's samples cut into `pieces` runs (each piece's fp32
+// sum to the workspace, one more launch adds them), so that blocks = tiles x pieces does.
+namespace {
+struct WsumPoolPlan {
+  int tile;    // 128 or 256
+  int pieces;  // 1, 2, 4 or 8, dividing every layer's n
+};
+
+// The pooled launch runs at a rate that hardly depends on how its work is spread once most CUs
+// have a block (measured on two layers of 1024 x 4096, 16384 rows: 64 + 64 tiles of 256 x 256 in one
+// piece 306 us, in two pieces, 256 blocks, 290 us with the pass that adds them, in four 314 us;
+// 512 tiles of 128 x 128 335 us), so pieces are only used to give every CU a block: the smallest
+// count that does. 256 x 256 tiles wherever every layer is at least that wide.
+WsumPoolPlan wsum_pool_plan(const dpk_wsum_layer* layers, int count, int cus) {
+  int64_t tiles256 = 0, tiles128 = 0;
+  bool all_wide = true;
+  int64_t g = 0;  // pieces must divide every n
+  for (int i = 0; i < count; ++i) {
+    const dpk_wsum_layer& L = layers[i];
+    tiles256 += dpk_cdiv(L.out, 256) * dpk_cdiv(L.in, 256);
+    tiles128 += dpk_cdiv(L.out, 128) * dpk_cdiv(L.in, 128);
+    all_wide = all_wide && L.out >= 256 && L.in >= 256;
+    int64_t a = L.n, b = g;
+    while (b) {
+      const int64_t t = a % b;
+      a = b;
+      b = t;
+    }
+    g = a;
+  }
+  WsumPoolPlan best{all_wide ? 256 : 128, 1};
+  const int64_t tiles = all_wide ? tiles256 : tiles128;
+  const int64_t resident = all_wide ? cus : 2 * cus;
+  while (best.pieces < 8 && tiles * best.pieces < resident && g % (2 * best.pieces) == 0) best.pieces *= 2;
+  return best;
+}
+}  // namespace
+
+extern "C" size_t dpk_linear_weighted_sum_multi_workspace_bytes(const dpk_wsum_layer* layers, int count) {
+  if (!layers || count <= 0) return 0;
+  int cus = dpk_device_cus();
+  if (cus <= 0) cus = 256;
+  const WsumPoolPlan plan = wsum_pool_plan(layers, count, cus);
+  if (plan.pieces == 1) return 0;
+  size_t total = 0;
+  for (int i = 0; i < count; ++i)
+    total += dpk_align_up(static_cast<size_t>(plan.pieces) * layers[i].out * layers[i].in * sizeof(float), 256);
+  return total;
+}
+
 extern "C" int dpk_linear_weighted_sum_multi(const dpk_wsum_layer* layers, int count, int in_dtype, int out_dtype,
-                                             dpk_stream_t stream) {
+                                             void* ws, size_t ws_bytes, dpk_stream_t stream) {
   const char* who = "dpk_linear_weighted_sum_multi";
   DPK_REQUIRE(count >= 0 && (layers || count == 0), DPK_E_ARG, "%s: count=%d, layers=%p", who, count, (const void*)layers);
   DPK_REQUIRE(in_dtype == DPK_BF16 && dpk_dtype_ok(out_dtype), DPK_E_DTYPE, "%s: dtypes %d,%d (bf16 input only)", who,
               in_dtype, out_dtype);
-  int64_t tiles256 = 0, tiles128 = 0;
   for (int i = 0; i < count; ++i) {
     const dpk_wsum_layer& L = layers[i];
     DPK_REQUIRE(L.n >= 1 && L.T >= 1 && L.out >= 1 && L.in >= 1, DPK_E_SHAPE, "%s: layer %d: n=%lld T=%lld out=%lld in=%lld",
@@ -830,25 +917,30 @@ extern "C" int dpk_linear_weighted_sum_multi(const dpk_wsum_layer* layers, int c
                     dpk_aligned(L.b, 16) && dpk_aligned(L.a, 16) && dpk_aligned(L.out_sum, 16) && dpk_aligned(L.coef, 4),
                 DPK_E_SHAPE, "%s: layer %d: out=%lld and in=%lld must be multiples of 8 above 64 and the tensors 16-byte aligned",
                 who, i, (long long)L.out, (long long)L.in);
-    tiles256 += dpk_cdiv(L.out, 256) * dpk_cdiv(L.in, 256);
-    tiles128 += dpk_cdiv(L.out, 128) * dpk_cdiv(L.in, 128);
   }
   if (count == 0) return DPK_OK;
-  // the same cost rule as for one layer, on the pool: rounds of resident blocks times work per block
   int cus = dpk_device_cus();
   if (cus <= 0) cus = 256;
-  const double cost_small = static_cast<double>(dpk_cdiv(tiles128, 2 * cus)) * 2.0;
-  const double cost_large = static_cast<double>(dpk_cdiv(tiles256, cus)) * 4.0 * kTrLargeGain;
-  bool all_wide = true;
-  for (int i = 0; i < count; ++i) all_wide = all_wide && layers[i].out >= 256 && layers[i].in >= 256;
-  const int tile = (all_wide && cost_large < cost_small) ? 256 : 128;
+  const WsumPoolPlan plan = wsum_pool_plan(layers, count, cus);
+  const int tile = plan.tile, pieces = plan.pieces;
+  if (pieces > 1) {
+    const size_t need = dpk_linear_weighted_sum_multi_workspace_bytes(layers, count);
+    DPK_REQUIRE(ws && ws_bytes >= need, DPK_E_WORKSPACE, "%s: workspace %zu < %zu bytes", who, ws_bytes, need);
+    DPK_REQUIRE(dpk_aligned(ws, 256), DPK_E_ALIGN, "%s: workspace must be 256-byte aligned", who);
+  }
   hipStream_t s = static_cast<hipStream_t>(stream);
+  char* part = static_cast<char*>(ws);
   for (int lo = 0; lo < count; lo += kWsumMax) {
     const int nl = count - lo < kWsumMax ? count - lo : kWsumMax;
     WsumMultiArgs A;
+    AddPiecesMultiArgs R;
+    memset(&A, 0, sizeof(A));
+    memset(&R, 0, sizeof(R));
     A.nlayers = nl;
-    A.tile_prefix[0] = 0;
-    int64_t total = 0;
+    A.pieces = pieces;
+    R.nlayers = nl;
+    R.pieces = pieces;
+    int64_t total = 0, add_blocks = 0;
     for (int i = 0; i < nl; ++i) {
       const dpk_wsum_layer& L = layers[lo + i];
       A.b[i] = static_cast<const bf16_t*>(L.b);
@@ -862,20 +954,37 @@ extern "C" int dpk_linear_weighted_sum_multi(const dpk_wsum_layer* layers, int c
       const int32_t tm = static_cast<int32_t>(dpk_cdiv(L.out, tile)), tn = static_cast<int32_t>(dpk_cdiv(L.in, tile));
       A.tiles_n[i] = tm < tn ? -tm : tn;  // the shorter dimension varies fastest
       A.scale[i] = L.scale;
-      total += dpk_cdiv(L.out, tile) * dpk_cdiv(L.in, tile);
+      total += dpk_cdiv(L.out, tile) * dpk_cdiv(L.in, tile) * pieces;
       DPK_REQUIRE(total <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: %lld blocks exceed the grid limit", who, (long long)total);
       A.tile_prefix[i + 1] = static_cast<uint32_t>(total);
+      if (pieces > 1) {
+        A.part[i] = reinterpret_cast<float*>(part);
+        R.part[i] = A.part[i];
+        R.out[i] = L.out_sum;
+        R.count4[i] = L.out * L.in / 4;
+        add_blocks += dpk_cdiv(R.count4[i], kThreads);
+        DPK_REQUIRE(add_blocks <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: %lld blocks exceed the grid limit", who, (long long)add_blocks);
+        R.block_prefix[i + 1] = static_cast<uint32_t>(add_blocks);
+        part += dpk_align_up(static_cast<size_t>(pieces) * L.out * L.in * sizeof(float), 256);
+      }
     }
     const dim3 grid(static_cast<unsigned>(total));
-    if (tile == 256 && out_dtype == DPK_BF16)
+    const bool f32 = out_dtype == DPK_F32 || pieces > 1;  // pieces are summed in fp32
+    if (tile == 256 && !f32)
       hipLaunchKernelGGL((linear_wsum_multi_kernel<TrLarge, bf16_t>), grid, dim3(TrLarge::kThreads), 0, s, A);
     else if (tile == 256)
       hipLaunchKernelGGL((linear_wsum_multi_kernel<TrLarge, float>), grid, dim3(TrLarge::kThreads), 0, s, A);
-    else if (out_dtype == DPK_BF16)
+    else if (!f32)
       hipLaunchKernelGGL((linear_wsum_multi_kernel<TrSmall, bf16_t>), grid, dim3(TrSmall::kThreads), 0, s, A);
     else
       hipLaunchKernelGGL((linear_wsum_multi_kernel<TrSmall, float>), grid, dim3(TrSmall::kThreads), 0, s, A);
     DPK_LAUNCH_CHECK(who);
+    if (pieces > 1) {
+      const dim3 g2(static_cast<unsigned>(add_blocks));
+      if (out_dtype == DPK_BF16) hipLaunchKernelGGL(add_pieces_multi_kernel<bf16_t>, g2, dim3(kThreads), 0, s, R);
+      else hipLaunchKernelGGL(add_pieces_multi_kernel<float>, g2, dim3(kThreads), 0, s, R);
+      DPK_LAUNCH_CHECK(who);
+    }
   }
   return DPK_OK;
 }

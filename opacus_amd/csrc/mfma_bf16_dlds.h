@@ -233,6 +233,9 @@ struct Tile {
 // kLoadsPerTile * (NS - 2). abase / bbase must be wave-uniform and every byte
 // offset inside the matrices must fit 32 bits (M * ld * 2 < 2^32).
 // Ma / Mb: rows of the two operand matrices (the same matrix for a Gram).
+// (A diagonal tile of a Gram has the same rows as both operands. Fetching them once and
+// pointing both operand reads at the one image measured 5 % faster on a launch of one
+// round of blocks and 4.5 % slower on a launch of 24 rounds, and was not kept.)
 template <class C, typename T = bf16_t>
 __device__ __forceinline__ void mainloop(Tile& t, Smem<C>& sm, const T* abase,
                                          const T* bbase, int64_t ld, int64_t m0a, int64_t m0b,
@@ -280,116 +283,6 @@ __device__ __forceinline__ void mainloop(Tile& t, Smem<C>& sm, const T* abase,
                                          const T* bbase, int64_t ld, int64_t m0a, int64_t m0b,
                                          int64_t M, int64_t K, int wm0, int wn0) {
   mainloop<C, T>(t, sm, abase, bbase, ld, m0a, m0b, M, M, K, wm0, wn0);
-}
-
-// ---- 64 x 64 tile with the k extent of a stage split over the block's waves -----
-// For work units too small to deserve a whole block tile (the tail of a launch that
-// does not fill the last round of resident blocks): all kWaves waves share one
-// 64 x 64 tile, wave w takes the w-th 16-wide k slice of every stage, and the
-// partial tiles are summed through LDS afterwards. Same swizzle; a stage holds 64 A
-// rows then 64 B rows (16 KB).
-template <class C, typename T = bf16_t>
-__device__ __forceinline__ void mainloop_splitk(Tile& t, Smem<C>& sm, const T* abase,
-                                                const T* bbase, int64_t ld, int64_t m0a,
-                                                int64_t m0b, int64_t M, int64_t K) {
-  static_assert(C::BK == 64 && C::kWaves == 4 && C::kStages == 2,
-                "split-k small tile: one 32-byte k slice per wave, two stages");
-  constexpr int ROW_BYTES = C::ROW_BYTES, ES = sizeof(T);
-  constexpr int BK = ROW_BYTES / ES;  // k values of a stage row: 64 bf16 or 32 floats
-  constexpr bool kF32 = std::is_same<T, float>::value;
-  typedef typename std::conditional<kF32, floatx4, bf16x8>::type frag_t;
-  constexpr int kLoads = 2 * 64 * ROW_BYTES / 1024 / C::kWaves;  // per wave and stage: 4
-  constexpr int kHalf = kLoads / 2;                              // the first half fetch A rows
-  const int64_t nk = K / BK;
-  const uint32_t lds0 = lds_offset(&sm.stage[0][0]);
-  const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  uint32_t off[kLoads];
-#pragma unroll
-  for (int q = 0; q < kLoads; ++q) {
-    // group q * kWaves + wave of the stage image; groups 0..7 are A rows, 8..15 B rows
-    off[q] = q < kHalf ? lane_offset<C, ES>(ld, m0a, M, q) : lane_offset<C, ES>(ld, m0b, M, q - kHalf);
-    asm volatile("" : "+v"(off[q]));
-  }
-  auto issue = [&](int64_t kt, uint32_t st) {
-#pragma unroll
-    for (int q = 0; q < kLoads; ++q)
-      load16_to_lds((q < kHalf ? abase : bbase) + kt * BK, off[q], st + group_lds<C>(q));
-  };
-  // The small stages (16 KB) leave room for a ring of four in the same memory: with
-  // only four MFMAs per wave and stage there is little work to hide a load behind,
-  // so tiles are requested three stages ahead.
-  constexpr int kRing = 4;
-  constexpr uint32_t kSmallStage = 2 * 64 * ROW_BYTES;
-  static_assert(kRing * kSmallStage <= sizeof(Smem<C>), "small-stage ring must fit the stage memory");
-#pragma unroll
-  for (int s = 0; s < kRing - 1; ++s) issue(s < nk ? s : nk - 1, lds0 + s * kSmallStage);
-  const int kh = lane >> 5, l32 = lane & 31;
-  int stage = 0;
-  for (int64_t kt = 0; kt < nk; ++kt) {
-    // tile kt has landed (the two tiles after it may still be in flight) and the stage
-    // read in the previous iteration is free
-    wait_and_barrier<kLoads*(kRing - 2)>();
-    const int64_t kn = kt + kRing - 1 < nk ? kt + kRing - 1 : nk - 1;
-    issue(kn, lds0 + ((stage + kRing - 1) & (kRing - 1)) * kSmallStage);
-    const unsigned char* As = &sm.stage[0][0] + stage * kSmallStage;
-    const unsigned char* Bs = As + 64 * ROW_BYTES;
-    frag_t av[2], bv[2];
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int row = i * 32 + l32;
-      av[i] = *reinterpret_cast<const frag_t*>(As + row * ROW_BYTES + swz<C>(row, wave * 2 + kh) * 16);
-      bv[i] = *reinterpret_cast<const frag_t*>(Bs + row * ROW_BYTES + swz<C>(row, wave * 2 + kh) * 16);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    if constexpr (kF32) {
-#pragma unroll
-      for (int e = 0; e < 4; ++e)
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-          for (int j = 0; j < 2; ++j)
-            t.acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i][e], bv[j][e], t.acc[i][j], 0, 0, 0);
-    } else {
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-          t.acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[i], bv[j], t.acc[i][j], 0, 0, 0);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    stage = (stage + 1) & (kRing - 1);
-  }
-  wait_and_barrier<0>();
-}
-
-// Sums the waves' partial 64 x 64 tiles of mainloop_splitk through the (now idle)
-// stage memory. Returns the 32 x 32 block (wave >> 1, wave & 1) of the sum in the
-// MFMA accumulator layout.
-template <class C>
-__device__ __forceinline__ floatx16 splitk_reduce(const Tile& t, Smem<C>& sm) {
-  static_assert(C::kWaves == 4 && sizeof(Smem<C>) >= 4 * 4 * 16 * 64 * sizeof(float),
-                "four partial tiles of 16 KB must fit the stage memory");
-  float* buf = reinterpret_cast<float*>(&sm.stage[0][0]);
-  const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) buf[((wave * 4 + i * 2 + j) * 16 + v) * 64 + lane] = t.acc[i][j][v];
-  __syncthreads();
-  floatx16 r;
-#pragma unroll
-  for (int v = 0; v < 16; ++v) {
-    float s = 0.f;
-#pragma unroll
-    for (int src = 0; src < 4; ++src) s += buf[((src * 4 + wave) * 16 + v) * 64 + lane];
-    r[v] = s;
-  }
-  __syncthreads();  // the stage memory is free for the next main loop
-  return r;
 }
 
 }  // namespace mb16d

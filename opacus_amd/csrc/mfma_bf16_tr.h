@@ -196,10 +196,20 @@ struct Tile {
 // in units of the current unit's coefficient: at a unit's first tile it is rescaled by
 // coef[u - 1] / coef[u], and by the last coefficient at the end. What it holds is then at most
 // (sum of the weighted terms so far) / coef[u], so it overflows only where the unit's own
-// unweighted product nearly does. A coefficient below kMinCoef counts as kMinCoef (an exact
-// zero would turn the rescaling into a division by zero); a NaN stays a NaN.
+// unweighted product nearly does. No rescaling multiplies by more than 2^40: a coefficient smaller
+// than 2^-40 of the one before it (an exact zero: a masked sample) counts as that fraction of it,
+// and any coefficient below kMinCoef as kMinCoef. Such a unit then enters the sum with a weight
+// of at most 2^-40 of its neighbour's, far below fp32 resolution, where an exact zero would turn
+// the rescaling into a division by zero and a fixed floor alone would let a partial sum above
+// 3e8 overflow. (Leaving the unit's MFMAs out instead, by a second copy of the step or by zeroing
+// one operand's registers under a branch, cost the 256 x 256 kernel 12 % of its rate.)
+// Coefficients are non-negative; a NaN stays a NaN.
 constexpr float kMinCoef = 1e-30f;
-__device__ __forceinline__ float at_least_min_coef(float c) { return c < kMinCoef ? kMinCoef : c; }
+constexpr float kMinRatio = 9.094947017729282e-13f;  // 2^-40
+__device__ __forceinline__ float floored_coef(float c, float prev) {
+  const float floor = prev * kMinRatio > kMinCoef ? prev * kMinRatio : kMinCoef;
+  return c < floor ? floor : c;
+}
 
 template <class C, bool kWeighted = false>
 __device__ __forceinline__ void mainloop(Tile<C>& t, Smem<C>& sm, const bf16_t* P, int64_t ldp, int64_t p0,
@@ -213,7 +223,7 @@ __device__ __forceinline__ void mainloop(Tile<C>& t, Smem<C>& sm, const bf16_t* 
     units = nk / tiles_per_unit;
     boundary = tiles_per_unit;
     // (read one unit ahead and not looked at before its unit begins: nothing waits for the load)
-    c_cur = at_least_min_coef(coef[0]);
+    c_cur = floored_coef(coef[0], 0.f);
     c_nxt = coef[units > 1 ? 1 : 0];
   }
   const int dup = static_cast<int>(nk * BK - K);  // rows the last tile repeats
@@ -278,7 +288,7 @@ __device__ __forceinline__ void mainloop(Tile<C>& t, Smem<C>& sm, const bf16_t* 
     const unsigned char* st = sm.stage[(kt + 1) & (NS - 1)];
     if constexpr (kWeighted) {
       if (kt == boundary) {  // first tile of the next unit (uniform over the block)
-        const float c_new = at_least_min_coef(c_nxt);
+        const float c_new = floored_coef(c_nxt, c_cur);
         const float ratio = c_cur / c_new;
         c_cur = c_new;
         ++unit;

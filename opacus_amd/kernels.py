@@ -240,18 +240,15 @@ def linear_weighted_sum_multi(
     """:func:`linear_weighted_sum` for several layers in one call: each item is ``(backprops,
     activations, coef, scale)`` (every pair one that :func:`linear_weighted_sum_takes`); returns
     the ``[out, in]`` sums in order. The block tiles of all layers are one pool of work, so the
-    GPU stays full across layers whose own tile count does not fill it in whole rounds
-    (``pooled=False``/``True`` overrides the choice between that and layer-by-layer calls)."""
+    GPU stays full across layers whose own tile count does not fill it in whole rounds; a small
+    pool (a two-layer MLP) has its samples cut into pieces inside the call
+    (``pooled=False`` calls layer by layer instead)."""
     if not items:
         return []
     dev = _need_gpu(*[t for it in items for t in it[:3]])
     out_dtype = out_dtype or items[0][0].dtype
-    # a small pool (a two-layer MLP) is better off layer by layer, each cut into pieces along the
-    # samples: the pooled launch contracts every layer in one piece and needs several rounds of
-    # 256 x 256 tiles to keep the GPU busy
-    tiles = sum(-(-it[0].shape[-1] // 256) * -(-it[1].shape[-1] // 256) for it in items)
     if pooled is None:
-        pooled = tiles >= 4 * device_cus()
+        pooled = True
     if not pooled:
         return [linear_weighted_sum(b, a, c, scale=scale, out_dtype=out_dtype) for b, a, c, scale in items]
     table = (_lib.WsumLayer * len(items))()
@@ -270,10 +267,12 @@ def linear_weighted_sum_multi(
         outs.append(out)
         row.b, row.a, row.coef, row.out_sum = b.data_ptr(), a.data_ptr(), c.data_ptr(), out.data_ptr()
         row.n, row.T, row.out, row.inp, row.scale = n, b.shape[1], out_f, in_f, float(scale)
+    L = lib()
+    ws, wsb = _ws(L.dpk_linear_weighted_sum_multi_workspace_bytes(table, len(items)), dev)
     with _timed("linear_weighted_sum", dev):
         check(
             "dpk_linear_weighted_sum_multi",
-            lib().dpk_linear_weighted_sum_multi(table, len(items), DPK_BF16, _code(out_dtype), _stream(dev)),
+            L.dpk_linear_weighted_sum_multi(table, len(items), DPK_BF16, _code(out_dtype), _ptr(ws), wsb, _stream(dev)),
         )
     del keep
     return outs

@@ -507,7 +507,7 @@ WEIGHTED_SUM_CASES = [
 
 
 @pytest.mark.parametrize("n,T,fin,fout,pieces", WEIGHTED_SUM_CASES)
-@pytest.mark.parametrize("coefs", ["spread", "equal", "tiny_and_zero"])
+@pytest.mark.parametrize("coefs", ["spread", "equal", "tiny_and_zero", "zeros_after_large_sums"])
 @pytest.mark.parametrize("out_f32", [False, True])
 def test_linear_weighted_sum(K, n, T, fin, fout, pieces, coefs, out_f32):
     """sum_n coef[n] * b[n]^T a[n] with the coefficients applied to the accumulators, against the
@@ -519,6 +519,15 @@ def test_linear_weighted_sum(K, n, T, fin, fout, pieces, coefs, out_f32):
         c = torch.rand(n) * 0.99 + 0.01
     elif coefs == "equal":
         c = torch.full((n,), 0.37)
+    elif coefs == "zeros_after_large_sums":
+        # masked samples (coefficient exactly 0) after partial sums of 1e10 and more: a sample that
+        # counts zero times must leave the sum alone (dividing the accumulator by a floored
+        # coefficient would overflow here); zeros first, last and in a row as well
+        a, b = (a.float() * 3e4).bfloat16(), (b.float() * 3e5).bfloat16()
+        c = torch.rand(n) * 0.5 + 0.5
+        c[1], c[-1] = 0.0, 0.0
+        if n > 4:
+            c[0], c[3], c[4] = 0.0, 0.0, 1e-38
     else:  # coefficients twelve orders of magnitude apart and an exact zero, at either end too
         c = torch.rand(n) * 0.9 + 0.1
         c[0], c[n // 2], c[-1] = 1e-12, 0.0, 3e-9
