@@ -87,16 +87,23 @@ int dpk_linear_gs(const void* b, const void* a, int in_dtype, void* gs, int gs_d
  * backprops of one backward pass: what the reference's second backward pass of
  * sum_s coef[s] * loss[s] leaves in weight.grad (utils/fast_gradient_clipping_utils.py:193-201,
  * DPTensorFastGradientClipping.backward), without that pass and without a weighted copy of
- * either operand. b: [n,T,out], a: [n,T,in], bf16; coef: float[n]; out: [out,in] of `out_dtype`.
- * One contraction over samples and positions at once: the accumulators are rescaled by
- * coef[s-1]/coef[s] where sample s begins, so no per-sample product is stored anywhere. A
- * coefficient below 1e-30 counts as 1e-30. pieces > 1 cuts the samples into that many runs
- * (more blocks for a layer with few output tiles) whose fp32 sums go through the workspace
- * (dpk_linear_weighted_sum_workspace_bytes) and are added by a second kernel.
- * Requires T % 32 == 0, n % pieces == 0, out and in multiples of 8 above 64, 16-byte aligned
- * tensors; anything else is refused with DPK_E_SHAPE (the caller then weights an operand itself
- * and calls dpk_linear_gs on one "sample" of n*T rows). */
-size_t dpk_linear_weighted_sum_workspace_bytes(int64_t out_features, int64_t in_features, int pieces);
+ * either operand. b: [n,T,out], a: [n,T,in] of `in_dtype`; coef: float[n] (non-negative);
+ * out: [out,in] of `out_dtype`.
+ * bf16 operands with T % 32 == 0, out and in multiples of 8 above 64, n % pieces == 0 and
+ * 16-byte aligned tensors: one bf16 MFMA contraction over samples and positions at once, the
+ * accumulators rescaled by coef[s-1]/coef[s] where sample s begins, so no per-sample product is
+ * stored anywhere. No rescaling multiplies by more than 2^40: a coefficient below 2^-40 of the
+ * one before it (an exact zero) counts as that fraction of it, one below 1e-30 as 1e-30.
+ * pieces > 1 cuts the samples into that many runs (more blocks for a layer with few output
+ * tiles) whose fp32 sums go through the workspace and are added by a second kernel.
+ * fp32 operands with T % 16 == 0, out and in multiples of 4 (in of 8 for a bf16 result) above 64:
+ * the same on the fp32 MFMA with operands loaded straight into LDS.
+ * Everything else (any T, any feature sizes, any alignment): the fp32 MFMA contraction over all
+ * n*T rows with the rows of b multiplied by their coefficients on the way into LDS (bf16 rows
+ * are widened first); pieces are then runs of rows.
+ * ws: dpk_linear_weighted_sum_workspace_bytes bytes, 256-byte aligned. */
+size_t dpk_linear_weighted_sum_workspace_bytes(int64_t n, int64_t T, int64_t out_features, int64_t in_features,
+                                               int in_dtype, int pieces);
 int dpk_linear_weighted_sum(const void* b, const void* a, int in_dtype, const float* coef, void* out,
                             int out_dtype, int64_t n, int64_t T, int64_t out_features,
                             int64_t in_features, float scale, int pieces, void* ws, size_t ws_bytes,
@@ -127,6 +134,16 @@ int dpk_linear_weighted_sum_multi(const dpk_wsum_layer* layers /*host*/, int cou
  * the optimizer's norm pass (optimizers/optimizer.py:444-446). */
 int dpk_linear_bias_gs(const void* b, int in_dtype, void* gs_bias, int gs_dtype, float* sumsq,
                        int64_t n, int64_t T, int64_t out, float scale, dpk_stream_t stream);
+
+/* out[k] = scale * sum_s coef[s] * sum_t b[s,t,k]: the clip-weighted sum of the per-sample bias
+ * gradients (linear.py:50), what the second backward pass leaves in bias.grad
+ * (utils/fast_gradient_clipping_utils.py:193-201). One pass over b in 256 chunks of rows whose
+ * fp32 sums are added in a fixed order. b: [n,T,out] of `in_dtype`; out: [out] of `out_dtype`.
+ * ws: dpk_linear_bias_weighted_sum_workspace_bytes bytes, 256-byte aligned. */
+size_t dpk_linear_bias_weighted_sum_workspace_bytes(int64_t n, int64_t T, int64_t out);
+int dpk_linear_bias_weighted_sum(const void* b, int in_dtype, const float* coef, void* out_sum, int out_dtype,
+                                 int64_t n, int64_t T, int64_t out, float scale, void* ws, size_t ws_bytes,
+                                 dpk_stream_t stream);
 
 /* ------------------------------------------------------------------------- *
  * Ghost-clipping per-sample norms of nn.Linear
@@ -257,6 +274,20 @@ int dpk_embedding_unique_pairs(const int64_t* ids, int64_t n, int64_t T, int64_t
 int dpk_embedding_gs(const int64_t* ids, const void* b, int in_dtype, void* gs, int gs_dtype,
                      int64_t n, int64_t T, int64_t V, int64_t D, float scale, int32_t* status,
                      void* ws, size_t ws_bytes, dpk_stream_t stream);
+
+/* out[v,:] = scale * sum_n coef[n] * sum_{t : ids[n,t]==v} b[n,t,:]
+ * The clip-weighted sum of an Embedding table's per-sample gradients (embedding.py:48-61), what
+ * the reference's second backward pass of sum_n coef[n] * loss[n] leaves in weight.grad
+ * (utils/fast_gradient_clipping_utils.py:193-201), without a weighted copy of the backprops.
+ * Equal ids are linked across the whole batch, every list is summed in fp32 in position order
+ * (each row times its sample's coefficient) and every row of the table is written once: no
+ * atomics, the same bits on every run. out: [V,D] of `out_dtype` (the input's type or fp32),
+ * 16-byte aligned, fully written. ids outside [0,V) and `status` as for dpk_embedding_gs.
+ * ws: dpk_embedding_weighted_sum_workspace_bytes bytes, 256-byte aligned. */
+size_t dpk_embedding_weighted_sum_workspace_bytes(int64_t n, int64_t T, int64_t D);
+int dpk_embedding_weighted_sum(const int64_t* ids, const void* b, int in_dtype, const float* coef, void* out,
+                               int out_dtype, int64_t n, int64_t T, int64_t V, int64_t D, float scale,
+                               int32_t* status, void* ws, size_t ws_bytes, dpk_stream_t stream);
 
 /* nn.EmbeddingBag (embedding.py:67-94): bag i = index[offsets[i] : offsets[i+1]] (the
  * last one runs to L); gs[i, index[j], :] = scale * b[i,:] for every j of bag i, divided

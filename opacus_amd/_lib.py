@@ -62,7 +62,13 @@ SIGNATURES = {
     "dpk_device_cus": (c_int, []),
     "dpk_linear_gs_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
     "dpk_linear_gs": (c_int, [_P, _P, c_int, _P, c_int, _P, _I, _I, _I, _I, c_float, c_int, _P, c_size_t, _P]),
-    "dpk_linear_weighted_sum_workspace_bytes": (c_size_t, [_I, _I, c_int]),
+    "dpk_linear_weighted_sum_workspace_bytes": (c_size_t, [_I, _I, _I, _I, c_int, c_int]),
+    "dpk_linear_bias_weighted_sum_workspace_bytes": (c_size_t, [_I, _I, _I]),
+    "dpk_linear_bias_weighted_sum": (c_int, [_P, c_int, _P, _P, c_int, _I, _I, _I, c_float, _P, c_size_t, _P]),
+    "dpk_embedding_weighted_sum_workspace_bytes": (c_size_t, [_I, _I, _I]),
+    "dpk_embedding_weighted_sum": (
+        c_int, [_P, _P, c_int, _P, _P, c_int, _I, _I, _I, _I, c_float, _P, _P, c_size_t, _P]
+    ),
     "dpk_linear_weighted_sum": (
         c_int, [_P, _P, c_int, _P, _P, c_int, _I, _I, _I, _I, c_float, c_int, _P, c_size_t, _P]
     ),

@@ -379,11 +379,13 @@ __global__ __launch_bounds__(kThreads) void emb_emit_pairs_kernel(
 // grid = n * tch * dch. A block owns kLeadersPerBlock positions and 1024 columns;
 // thread <-> 4 columns. MODE 0: sum of squares of the per-id sums (ghost norm).
 // MODE 1: write scale * sum into gs[sample, id, :].
+// MODE 2: as MODE 1 with every row multiplied by its weight rw[t] before it is added (the
+// clip-weighted sum over a whole batch laid out as one "sample" of n * T positions).
 template <typename TIN, typename TOUT, int MODE, bool VEC>
 __global__ __launch_bounds__(kThreads) void emb_walk_kernel(
     const int64_t* __restrict__ ids, const TIN* __restrict__ b, const int32_t* __restrict__ next,
     const int32_t* __restrict__ leader, int64_t T, int64_t D, int64_t V, int tch, int dch,
-    float scale, float* __restrict__ partials, TOUT* __restrict__ gs) {
+    float scale, float* __restrict__ partials, TOUT* __restrict__ gs, const float* __restrict__ rw = nullptr) {
   __shared__ float red[kWaves];
   int64_t bid = blockIdx.x;
   const int dc = static_cast<int>(bid % dch);
@@ -425,21 +427,31 @@ __global__ __launch_bounds__(kThreads) void emb_walk_kernel(
     const int64_t t = t0 + r;
     if (follow[r] < -1) continue;  // uniform over the block
     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (VEC && d < D) acc = dpk_io<TIN>::unpack4(first[r]);
+    if (VEC && d < D) {
+      acc = dpk_io<TIN>::unpack4(first[r]);
+      if (MODE == 2) {
+        const float c = rw[t];
+        acc.x *= c;
+        acc.y *= c;
+        acc.z *= c;
+        acc.w *= c;
+      }
+    }
     if (d < D) {
       for (int64_t u = VEC ? static_cast<int64_t>(follow[r]) : t; u >= 0; u = nx[u]) {
         const TIN* p = bs + u * D + d;
+        const float c = MODE == 2 ? rw[u] : 1.f;
         if (VEC) {
           const float4 v = dpk_io<TIN>::load4(p);
-          acc.x += v.x;
-          acc.y += v.y;
-          acc.z += v.z;
-          acc.w += v.w;
+          acc.x = fmaf(c, v.x, acc.x);
+          acc.y = fmaf(c, v.y, acc.y);
+          acc.z = fmaf(c, v.z, acc.z);
+          acc.w = fmaf(c, v.w, acc.w);
         } else {
-          acc.x += dpk_io<TIN>::load(p);
-          if (d + 1 < D) acc.y += dpk_io<TIN>::load(p + 1);
-          if (d + 2 < D) acc.z += dpk_io<TIN>::load(p + 2);
-          if (d + 3 < D) acc.w += dpk_io<TIN>::load(p + 3);
+          acc.x = fmaf(c, dpk_io<TIN>::load(p), acc.x);
+          if (d + 1 < D) acc.y = fmaf(c, dpk_io<TIN>::load(p + 1), acc.y);
+          if (d + 2 < D) acc.z = fmaf(c, dpk_io<TIN>::load(p + 2), acc.z);
+          if (d + 3 < D) acc.w = fmaf(c, dpk_io<TIN>::load(p + 3), acc.w);
         }
       }
     }
@@ -572,18 +584,25 @@ bool launch_link(const int64_t* ids, int64_t n, int64_t T, int64_t V, const EmbW
 
 template <typename TIN, typename TOUT, int MODE>
 void launch_walk(bool vec, const int64_t* ids, const void* b, const EmbWs& w, int64_t n, int64_t T,
-                 int64_t D, int64_t V, float scale, void* gs, hipStream_t s) {
+                 int64_t D, int64_t V, float scale, void* gs, hipStream_t s, const float* rw = nullptr) {
   const int tch = static_cast<int>(dpk_cdiv(T, kLeadersPerBlock));
   const int dch = static_cast<int>(dpk_cdiv(D, kThreads * 4));
   const dim3 grid(static_cast<unsigned>(n * tch * dch)), block(kThreads);
   if (vec)
     hipLaunchKernelGGL((emb_walk_kernel<TIN, TOUT, MODE, true>), grid, block, 0, s, ids,
                        static_cast<const TIN*>(b), w.next, w.leader, T, D, V, tch, dch, scale,
-                       w.partials, static_cast<TOUT*>(gs));
+                       w.partials, static_cast<TOUT*>(gs), rw);
   else
     hipLaunchKernelGGL((emb_walk_kernel<TIN, TOUT, MODE, false>), grid, block, 0, s, ids,
                        static_cast<const TIN*>(b), w.next, w.leader, T, D, V, tch, dch, scale,
-                       w.partials, static_cast<TOUT*>(gs));
+                       w.partials, static_cast<TOUT*>(gs), rw);
+}
+
+// rw[r] = coef[r / T]: the weight of position r of the flattened batch.
+__global__ __launch_bounds__(kThreads) void emb_row_weights_kernel(const float* __restrict__ coef, float* __restrict__ rw,
+                                                                     int64_t rows, int64_t T) {
+  const int64_t r = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (r < rows) rw[r] = coef[r / T];
 }
 
 }  // namespace
@@ -686,6 +705,61 @@ extern "C" int dpk_embedding_gs(const int64_t* ids, const void* b, int in_dtype,
                    dpk_aligned(gs, gs_dtype == DPK_BF16 ? 8 : 16);
   if (in_dtype == DPK_F32) launch_walk<float, float, 1>(vec, ids, b, w, n, T, D, V, scale, gs, s);
   else launch_walk<bf16_t, bf16_t, 1>(vec, ids, b, w, n, T, D, V, scale, gs, s);
+  DPK_LAUNCH_CHECK(who);
+  return DPK_OK;
+}
+
+extern "C" size_t dpk_embedding_weighted_sum_workspace_bytes(int64_t n, int64_t T, int64_t D) {
+  if (n <= 0 || T <= 0) return 0;
+  return ws_layout(1, n * T, D, nullptr, nullptr) + dpk_align_up(static_cast<size_t>(n * T) * sizeof(float), 256);
+}
+
+// out[v, :] = scale * sum_n coef[n] * sum_{t : ids[n,t] == v} b[n,t,:]: the clip-weighted sum of the
+// per-sample gradients of an Embedding table (embedding.py:48-61 weighted per sample), what the
+// second backward pass of sum_n coef[n] * loss[n] leaves in weight.grad
+// (utils/fast_gradient_clipping_utils.py:193-201). The batch is taken as one run of n * T
+// positions: equal ids are linked across samples, each list is summed in fp32 in position order
+// with every row times its sample's coefficient, and a row of the table is written once. out is
+// fully written (rows no id names are zero). Ids outside [0, V): as for dpk_embedding_gs.
+extern "C" int dpk_embedding_weighted_sum(const int64_t* ids, const void* b, int in_dtype, const float* coef, void* out,
+                                          int out_dtype, int64_t n, int64_t T, int64_t V, int64_t D, float scale,
+                                          int32_t* status, void* ws, size_t ws_bytes, dpk_stream_t stream) {
+  const char* who = "dpk_embedding_weighted_sum";
+  DPK_REQUIRE(n >= 1 && T >= 1 && V >= 1 && D >= 1, DPK_E_SHAPE, "%s: n=%lld T=%lld V=%lld D=%lld", who, (long long)n,
+              (long long)T, (long long)V, (long long)D);
+  DPK_REQUIRE(b && coef && out, DPK_E_ARG, "%s: NULL tensor", who);
+  DPK_REQUIRE(dpk_dtype_ok(in_dtype) && dpk_dtype_ok(out_dtype) && (in_dtype == out_dtype || out_dtype == DPK_F32),
+              DPK_E_DTYPE, "%s: dtypes %d,%d (the result in the input's type or fp32)", who, in_dtype, out_dtype);
+  DPK_REQUIRE(dpk_aligned(b, dpk_elsize(in_dtype)) && dpk_aligned(out, 16) && dpk_aligned(coef, 4) && dpk_aligned(status, 4),
+              DPK_E_ALIGN, "%s: misaligned tensor (out must be 16-byte aligned)", who);
+  const int64_t L = n * T;
+  DPK_REQUIRE(L < (int64_t{1} << 31), DPK_E_SHAPE, "%s: n * T = %lld positions", who, (long long)L);
+  const size_t lists = ws_layout(1, L, D, nullptr, nullptr);
+  const size_t need = lists + dpk_align_up(static_cast<size_t>(L) * sizeof(float), 256);
+  EmbWs w;
+  int rc = check_common(who, ids, 1, L, D, ws, ws_bytes, &w);
+  if (rc != DPK_OK) return rc;
+  DPK_REQUIRE(ws_bytes >= need, DPK_E_WORKSPACE, "%s: workspace %zu < %zu bytes", who, ws_bytes, need);
+  float* rw = reinterpret_cast<float*>(static_cast<char*>(ws) + lists);
+  const int64_t tch = dpk_cdiv(L, kLeadersPerBlock), dch = dpk_cdiv(D, kThreads * 4);
+  DPK_REQUIRE(tch * dch <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: too many blocks", who);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  hipLaunchKernelGGL(emb_row_weights_kernel, dim3(static_cast<unsigned>(dpk_cdiv(L, kThreads))), dim3(kThreads), 0, s, coef,
+                     rw, L, T);
+  launch_link(ids, 1, L, V, w, status, false, s);
+  DPK_LAUNCH_CHECK(who);
+  const size_t bytes = static_cast<size_t>(V) * D * dpk_elsize(out_dtype);
+  const int64_t n16 = static_cast<int64_t>(bytes / 16);
+  const int64_t ntail = static_cast<int64_t>(bytes - static_cast<size_t>(n16) * 16);
+  int64_t blocks = dpk_cdiv(n16 > 0 ? n16 : 1, kThreads * 4);
+  if (blocks > 65536) blocks = 65536;
+  hipLaunchKernelGGL(zero_fill_kernel, dim3(static_cast<unsigned>(blocks)), dim3(kThreads), 0, s, static_cast<uint4*>(out),
+                     n16, static_cast<unsigned char*>(out) + static_cast<size_t>(n16) * 16, ntail);
+  DPK_LAUNCH_CHECK(who);
+  const bool vec = D % 4 == 0 && dpk_aligned(b, in_dtype == DPK_BF16 ? 8 : 16);
+  if (in_dtype == DPK_F32) launch_walk<float, float, 2>(vec, ids, b, w, 1, L, D, V, scale, out, s, rw);
+  else if (out_dtype == DPK_BF16) launch_walk<bf16_t, bf16_t, 2>(vec, ids, b, w, 1, L, D, V, scale, out, s, rw);
+  else launch_walk<bf16_t, float, 2>(vec, ids, b, w, 1, L, D, V, scale, out, s, rw);
   DPK_LAUNCH_CHECK(who);
   return DPK_OK;
 }

@@ -220,6 +220,7 @@ template <> struct TrOut<float> { static constexpr int kPad = 16, kRows = 64; };
 // main loop of mfma_bf16_tr.h (bf16, transposing LDS reads) or mfma_f32_dlds.h (fp32).
 struct TrBf16 {
   typedef bf16_t elem;
+  static constexpr int kBK = mb16t::BK;
   template <class C> using Smem = mb16t::Smem<C>;
   template <class C> using Tile = mb16t::Tile<C>;
   template <class C, class... A> static __device__ __forceinline__ void mainloop(A&&... args) {
@@ -231,15 +232,19 @@ struct TrBf16 {
 };
 struct DldsF32 {
   typedef float elem;
+  static constexpr int kBK = mf32d::BK;
   template <class C> using Smem = mf32d::Smem<C>;
   template <class C> using Tile = mf32d::Tile<C>;
   template <class C, class... A> static __device__ __forceinline__ void mainloop(A&&... args) {
     mf32d::mainloop<C>(static_cast<A&&>(args)...);
   }
+  template <class C, class... A> static __device__ __forceinline__ void mainloop_weighted(A&&... args) {
+    mf32d::mainloop<C, true>(static_cast<A&&>(args)...);
+  }
 };
 
 //
-// W (bf16 engine only): a "sample" of the launch is a run of T / unit_rows units of unit_rows
+// W: a "sample" of the launch is a run of T / unit_rows units of unit_rows
 // rows each (unit_rows a multiple of the k tile), and unit u of sample s counts
 // coef[s * (T / unit_rows) + u] times: gs[s] = scale * sum_u coef[..] * b_u^T a_u.
 // (Two waves per SIMD asked for, which these kernels reach anyway, caps W at 256 registers: the
@@ -265,7 +270,7 @@ __device__ __forceinline__ void linear_dlds_tile(
   typename E::template Tile<C> tile;
   tile.clear();
   if constexpr (W)
-    E::template mainloop_weighted<C>(tile, sm, a, N, n0, b, M, m0, T, wj0, wi0, coef, unit_rows / mb16t::BK);
+    E::template mainloop_weighted<C>(tile, sm, a, N, n0, b, M, m0, T, wj0, wi0, coef, unit_rows / E::kBK);
   else
     E::template mainloop<C>(tile, sm, a, N, n0, b, M, m0, T, wj0, wi0);
   const int kk = lane >> 5, l32 = lane & 31;
@@ -704,6 +709,147 @@ __global__ __launch_bounds__(kThreads) void add_pieces_kernel(const float* __res
   dpk_io<TOUT>::store4(out + 4 * e, acc);
 }
 
+// ---- clip-weighted sums for the shapes and dtypes the transposing-read kernel does not take ----
+// w[r] = coef[r / T] for the n * T rows of a layer's operands: the weight of a row.
+__global__ __launch_bounds__(kThreads) void row_weights_kernel(const float* __restrict__ coef, float* __restrict__ w,
+                                                                 int64_t rows, int64_t T) {
+  const int64_t r = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (r < rows) w[r] = coef[r / T];
+}
+
+// LoaderMContig whose rows are multiplied by their weights on the way into LDS (in fp32, as the
+// reference multiplies the backprops by the coefficients before its second pass,
+// fast_gradient_clipping_utils.py:193-196; bf16 rows are widened first, which is exact).
+template <int BMN, typename T, bool VEC>
+struct LoaderMContigWeighted : mf32::LoaderMContig<BMN, T, VEC> {
+  typedef mf32::LoaderMContig<BMN, T, VEC> Base;
+  const float* w;
+  __device__ __forceinline__ LoaderMContigWeighted(const T* base_, int64_t ld_, int64_t m0_, int64_t M_, int64_t K_,
+                                                   const float* w_)
+      : Base(base_, ld_, m0_, M_, K_), w(w_) {}
+  __device__ __forceinline__ void fetch(int64_t k0) {
+    Base::fetch(k0);
+#pragma unroll
+    for (int r = 0; r < Base::R; ++r) {
+      const int idx = threadIdx.x + r * mf32::NTHREADS;
+      const int64_t k = k0 + idx / (BMN / 4);
+      const float c = k < this->K ? w[k] : 0.f;
+      this->st[r].x *= c;
+      this->st[r].y *= c;
+      this->st[r].z *= c;
+      this->st[r].w *= c;
+    }
+  }
+};
+
+// out (or piece p's fp32 partial) = scale * sum_r w[r] * b[r, :]^T a[r, :] over the rows of piece p,
+// on the fp32 MFMA whatever the input type: any T, any feature sizes, any alignment.
+template <int BM, int BN, typename TIN, typename TOUT, bool VEC>
+__global__ __launch_bounds__(kThreads) void linear_wsum_generic_kernel(
+    const TIN* __restrict__ b, const TIN* __restrict__ a, const float* __restrict__ w, TOUT* __restrict__ out,
+    int64_t rows, int64_t rows_per_piece, int64_t M, int64_t N, float scale, int64_t tiles_m, int64_t tiles_n) {
+  __shared__ mf32::Smem<BM, BN> sm;
+  const int64_t per_piece = tiles_m * tiles_n;
+  const int64_t piece = blockIdx.x / per_piece;
+  const int64_t rem = blockIdx.x % per_piece;
+  const int64_t m0 = (rem / tiles_n) * BM, n0 = (rem % tiles_n) * BN;
+  const int64_t k0 = piece * rows_per_piece;
+  const int64_t k1 = k0 + rows_per_piece < rows ? k0 + rows_per_piece : rows;
+  LoaderMContigWeighted<BM, TIN, VEC> la(b, M, m0, M, k1, w);
+  mf32::LoaderMContig<BN, TIN, VEC> lb(a, N, n0, N, k1);
+  mf32::Tile<BM, BN> tile;
+  tile.clear();
+  if (k0 < k1) mf32::mainloop<BM, BN>(tile, sm, la, lb, k0, k1);
+  TOUT* dst = out + piece * M * N;
+  tile.for_each([&](int r, int c, float v) {
+    const int64_t i = m0 + r, j = n0 + c;
+    if (i < M && j < N) dpk_io<TOUT>::store(dst + i * N + j, v * scale);
+  });
+}
+
+// part[chunk, k] = sum over the chunk's rows of w[r] * b[r, k]: thread <-> 4 columns (VEC) or one,
+// eight rows of loads in flight.
+template <typename TIN, bool VEC>
+__global__ __launch_bounds__(kThreads) void wcolsum_partial_kernel(const TIN* __restrict__ b, const float* __restrict__ w,
+                                                                     float* __restrict__ part, int64_t rows,
+                                                                     int64_t rows_per_chunk, int64_t Kdim,
+                                                                     int64_t col_blocks) {
+  constexpr int W = VEC ? 4 : 1, U = 8;
+  const int64_t chunk = blockIdx.x / col_blocks;
+  const int64_t k = ((blockIdx.x % col_blocks) * kThreads + threadIdx.x) * W;
+  if (k >= Kdim) return;
+  const int64_t r0 = chunk * rows_per_chunk;
+  const int64_t r1 = r0 + rows_per_chunk < rows ? r0 + rows_per_chunk : rows;
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  const TIN* p = b + k;
+  int64_t r = r0;
+  if (VEC) {
+    for (; r + U <= r1; r += U) {
+      typename dpk_io<TIN>::raw4 x[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) x[u] = dpk_io<TIN>::load4_raw(p + (r + u) * Kdim);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const float4 v = dpk_io<TIN>::unpack4(x[u]);
+        const float c = w[r + u];
+        acc.x = fmaf(c, v.x, acc.x);
+        acc.y = fmaf(c, v.y, acc.y);
+        acc.z = fmaf(c, v.z, acc.z);
+        acc.w = fmaf(c, v.w, acc.w);
+      }
+    }
+  }
+  for (; r < r1; ++r) {
+    const float c = w[r];
+    if (VEC) {
+      const float4 v = dpk_io<TIN>::load4(p + r * Kdim);
+      acc.x = fmaf(c, v.x, acc.x);
+      acc.y = fmaf(c, v.y, acc.y);
+      acc.z = fmaf(c, v.z, acc.z);
+      acc.w = fmaf(c, v.w, acc.w);
+    } else {
+      acc.x = fmaf(c, dpk_io<TIN>::load(p + r * Kdim), acc.x);
+    }
+  }
+  float* o = part + chunk * Kdim + k;
+  if (VEC) {
+    *reinterpret_cast<float4*>(o) = acc;
+  } else {
+    *o = acc.x;
+  }
+}
+
+// out[k] = scale * sum_chunk part[chunk, k]: a block owns 64 columns, its four waves take every fourth
+// chunk each (eight loads in flight) and their sums meet in LDS; the order of addition is fixed.
+template <typename TOUT>
+__global__ __launch_bounds__(kThreads) void wcolsum_final_kernel(const float* __restrict__ part, TOUT* __restrict__ out,
+                                                                   int64_t chunks, int64_t Kdim, float scale) {
+  __shared__ float red[kWaves][DPK_WAVE];
+  const int lane = threadIdx.x & (DPK_WAVE - 1), wave = threadIdx.x / DPK_WAVE;
+  const int64_t k = static_cast<int64_t>(blockIdx.x) * DPK_WAVE + lane;
+  float s = 0.f;
+  if (k < Kdim) {
+    constexpr int U = 8;
+    int64_t c = wave;
+    for (; c + (U - 1) * kWaves < chunks; c += U * kWaves) {
+      float x[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) x[u] = part[(c + u * kWaves) * Kdim + k];
+#pragma unroll
+      for (int u = 0; u < U; ++u) s += x[u];
+    }
+    for (; c < chunks; c += kWaves) s += part[c * Kdim + k];
+  }
+  red[wave][lane] = s;
+  __syncthreads();
+  if (wave == 0 && k < Kdim) {
+    float t = red[0][lane];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) t += red[w][lane];
+    dpk_io<TOUT>::store(out + k, t * scale);
+  }
+}
+
 bool linear_vec(const void* b, const void* a, const void* gs, int in_dtype, int gs_dtype, int64_t M,
                 int64_t N) {
   const size_t ia = in_dtype == DPK_BF16 ? 8 : 16, oa = gs_dtype == DPK_BF16 ? 8 : 16;
@@ -780,15 +926,47 @@ extern "C" int dpk_linear_gs(const void* b, const void* a, int in_dtype, void* g
   return DPK_OK;
 }
 
-extern "C" size_t dpk_linear_weighted_sum_workspace_bytes(int64_t out, int64_t in, int pieces) {
-  if (out <= 0 || in <= 0 || pieces <= 1) return 0;
-  return dpk_align_up(static_cast<size_t>(pieces) * out * in * sizeof(float), 256);
+namespace {
+// Whether the transposing-read bf16 kernel takes the layer (the fast path of dpk_linear_weighted_sum
+// and the only one of dpk_linear_weighted_sum_multi).
+bool wsum_fast_shape(int in_dtype, int64_t T, int64_t out, int64_t in) {
+  return in_dtype == DPK_BF16 && T % mb16t::BK == 0 && out % 8 == 0 && in % 8 == 0 && out > 64 && in > 64 &&
+         out < (1LL << 24) && in < (1LL << 24);
+}
+// ... and the direct-load fp32 kernel with the coefficients on its accumulators
+bool wsum_fast_shape_f32(int in_dtype, int out_dtype, int64_t T, int64_t out, int64_t in) {
+  return in_dtype == DPK_F32 && T % mf32d::BK == 0 && out % 4 == 0 && in % (out_dtype == DPK_BF16 ? 8 : 4) == 0 &&
+         out > 64 && in > 64 && out < (1LL << 24) && in < (1LL << 24);
+}
+
+struct WsumGenericLayout {
+  size_t weights, total;  // [0, weights): float[n * T] row weights; then float[pieces, out, in] when pieces > 1
+};
+WsumGenericLayout wsum_generic_layout(int64_t n, int64_t T, int64_t out, int64_t in, int pieces) {
+  WsumGenericLayout l;
+  l.weights = dpk_align_up(static_cast<size_t>(n * T) * sizeof(float), 256);
+  l.total = l.weights + (pieces > 1 ? dpk_align_up(static_cast<size_t>(pieces) * out * in * sizeof(float), 256) : 0);
+  return l;
+}
+}  // namespace
+
+extern "C" size_t dpk_linear_weighted_sum_workspace_bytes(int64_t n, int64_t T, int64_t out, int64_t in, int in_dtype,
+                                                          int pieces) {
+  if (n <= 0 || T <= 0 || out <= 0 || in <= 0 || pieces < 1) return 0;
+  (void)in_dtype;
+  // room for either path: a shape the fast kernel takes still goes the generic way when a tensor
+  // turns out not to be 16-byte aligned
+  return wsum_generic_layout(n, T, out, in, pieces).total;
 }
 
 // out_sum = scale * sum_s coef[s] * b[s]^T a[s]: the clip-weighted sum of a Linear layer's
-// per-sample gradients, contracted over samples and positions at once. With pieces > 1 piece p
-// (samples p * n / pieces .. + n / pieces - 1) leaves its fp32 sum in the workspace and a
-// second kernel adds the pieces into out_sum.
+// per-sample gradients, contracted over samples and positions at once
+// (what the second backward pass leaves in weight.grad, fast_gradient_clipping_utils.py:193-201).
+// bf16 operands in whole k tiles per sample go to the transposing-read kernel with the coefficients
+// on its accumulators; with pieces > 1 piece p (samples p * n / pieces .. + n / pieces - 1) leaves
+// its fp32 sum in the workspace and a second kernel adds the pieces into out_sum. Everything else
+// (fp32 operands, any T, any feature sizes and alignment) goes to the fp32 MFMA kernel whose loader
+// multiplies the rows of b by their weights; its pieces are runs of rows.
 extern "C" int dpk_linear_weighted_sum(const void* b, const void* a, int in_dtype, const float* coef, void* out_sum,
                                        int out_dtype, int64_t n, int64_t T, int64_t out, int64_t in, float scale,
                                        int pieces, void* ws, size_t ws_bytes, dpk_stream_t stream) {
@@ -797,12 +975,73 @@ extern "C" int dpk_linear_weighted_sum(const void* b, const void* a, int in_dtyp
               "%s: n=%lld T=%lld out=%lld in=%lld pieces=%d", who, (long long)n, (long long)T, (long long)out,
               (long long)in, pieces);
   DPK_REQUIRE(b && a && coef && out_sum, DPK_E_ARG, "%s: NULL tensor", who);
-  DPK_REQUIRE(in_dtype == DPK_BF16 && dpk_dtype_ok(out_dtype), DPK_E_DTYPE, "%s: dtypes %d,%d (bf16 input only)", who,
-              in_dtype, out_dtype);
-  DPK_REQUIRE(T % mb16t::BK == 0 && n % pieces == 0, DPK_E_SHAPE,
-              "%s: T=%lld must be a multiple of %d and n=%lld of pieces=%d", who, (long long)T, mb16t::BK,
-              (long long)n, pieces);
-  DPK_REQUIRE(dpk_aligned(coef, 4), DPK_E_ALIGN, "%s: misaligned coefficients", who);
+  DPK_REQUIRE(dpk_dtype_ok(in_dtype) && dpk_dtype_ok(out_dtype), DPK_E_DTYPE, "%s: dtypes %d,%d", who, in_dtype,
+              out_dtype);
+  DPK_REQUIRE(dpk_aligned(coef, 4) && dpk_aligned(b, dpk_elsize(in_dtype)) && dpk_aligned(a, dpk_elsize(in_dtype)) &&
+                  dpk_aligned(out_sum, dpk_elsize(out_dtype)),
+              DPK_E_ALIGN, "%s: misaligned tensor", who);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int64_t count = out * in;
+  const bool fast = (wsum_fast_shape(in_dtype, T, out, in) || wsum_fast_shape_f32(in_dtype, out_dtype, T, out, in)) &&
+                    n % pieces == 0 && dpk_aligned(b, 16) && dpk_aligned(a, 16) && dpk_aligned(out_sum, 16);
+  if (!fast) {
+    // generic path: row weights, then the fp32 MFMA kernel over all n * T rows (in `pieces` runs of rows)
+    const int64_t rows = n * T;
+    const WsumGenericLayout l = wsum_generic_layout(n, T, out, in, pieces);
+    DPK_REQUIRE(ws && ws_bytes >= l.total, DPK_E_WORKSPACE, "%s: workspace %zu < %zu bytes", who, ws_bytes, l.total);
+    DPK_REQUIRE(dpk_aligned(ws, 256), DPK_E_ALIGN, "%s: workspace must be 256-byte aligned", who);
+    float* w = static_cast<float*>(ws);
+    float* part = reinterpret_cast<float*>(static_cast<char*>(ws) + l.weights);
+    const int64_t rows_per_piece = dpk_cdiv(dpk_cdiv(rows, pieces), mf32::BK) * mf32::BK;
+    const int bm = (out > 64 && in > 64) ? 128 : 64;
+    const int64_t tiles_m = dpk_cdiv(out, bm), tiles_n = dpk_cdiv(in, bm);
+    const int64_t blocks = pieces * tiles_m * tiles_n;
+    DPK_REQUIRE(blocks <= DPK_MAX_GRID_X && dpk_cdiv(rows, kThreads) <= DPK_MAX_GRID_X && (pieces == 1 || count % 4 == 0),
+                DPK_E_SHAPE, "%s: %lld blocks exceed the grid limit, or out * in = %lld is not a multiple of 4 with pieces",
+                who, (long long)blocks, (long long)count);
+    hipLaunchKernelGGL(row_weights_kernel, dim3(static_cast<unsigned>(dpk_cdiv(rows, kThreads))), dim3(kThreads), 0, s,
+                       coef, w, rows, T);
+    DPK_LAUNCH_CHECK(who);
+    const bool vec = out % 4 == 0 && in % 4 == 0 && dpk_aligned(b, 4 * dpk_elsize(in_dtype)) &&
+                     dpk_aligned(a, 4 * dpk_elsize(in_dtype));
+    const dim3 grid(static_cast<unsigned>(blocks));
+    const bool split = pieces > 1;
+#define DPK_WG(BMN, TIN, TOUT, V)                                                                                   \
+  hipLaunchKernelGGL((linear_wsum_generic_kernel<BMN, BMN, TIN, TOUT, V>), grid, dim3(kThreads), 0, s,              \
+                     static_cast<const TIN*>(b), static_cast<const TIN*>(a), w,                                     \
+                     split ? reinterpret_cast<TOUT*>(part) : static_cast<TOUT*>(out_sum), rows, rows_per_piece, out, \
+                     in, scale, tiles_m, tiles_n)
+#define DPK_WG_V(BMN, TIN, TOUT) \
+  do {                           \
+    if (vec) DPK_WG(BMN, TIN, TOUT, true); \
+    else DPK_WG(BMN, TIN, TOUT, false);    \
+  } while (0)
+#define DPK_WG_B(TIN, TOUT)                  \
+  do {                                       \
+    if (bm == 128) DPK_WG_V(128, TIN, TOUT); \
+    else DPK_WG_V(64, TIN, TOUT);            \
+  } while (0)
+    const bool f32_dst = split || out_dtype == DPK_F32;
+    if (in_dtype == DPK_F32 && f32_dst) DPK_WG_B(float, float);
+    else if (in_dtype == DPK_F32) DPK_WG_B(float, bf16_t);
+    else if (f32_dst) DPK_WG_B(bf16_t, float);
+    else DPK_WG_B(bf16_t, bf16_t);
+#undef DPK_WG_B
+#undef DPK_WG_V
+#undef DPK_WG
+    DPK_LAUNCH_CHECK(who);
+    if (split) {
+      const dim3 g2(static_cast<unsigned>(dpk_cdiv(count / 4, kThreads)));
+      if (out_dtype == DPK_BF16)
+        hipLaunchKernelGGL(add_pieces_kernel<bf16_t>, g2, dim3(kThreads), 0, s, part, static_cast<bf16_t*>(out_sum),
+                           count / 4, pieces);
+      else
+        hipLaunchKernelGGL(add_pieces_kernel<float>, g2, dim3(kThreads), 0, s, part, static_cast<float*>(out_sum),
+                           count / 4, pieces);
+      DPK_LAUNCH_CHECK(who);
+    }
+    return DPK_OK;
+  }
   const bool split = pieces > 1;
   if (split) {
     const size_t need = static_cast<size_t>(pieces) * out * in * sizeof(float);
@@ -813,19 +1052,27 @@ extern "C" int dpk_linear_weighted_sum(const void* b, const void* a, int in_dtyp
   const int dst_dtype = split ? DPK_F32 : out_dtype;
   const int64_t rows = (n / pieces) * T;
   Plan p = make_plan(rows, out, in, true);
-  plan_tr(p, b, a, out_sum, pieces, rows, out, in, dpk_device_cus(), DPK_TILE_AUTO);
-  DPK_REQUIRE(p.tr != 0, DPK_E_SHAPE,
-              "%s: out=%lld and in=%lld must be multiples of 8 above 64 and the tensors 16-byte aligned", who,
-              (long long)out, (long long)in);
+  if (in_dtype == DPK_BF16) plan_tr(p, b, a, out_sum, pieces, rows, out, in, dpk_device_cus(), DPK_TILE_AUTO);
+  else plan_dlds_f32(p, b, a, out_sum, dst_dtype, rows, out, in);
+  DPK_REQUIRE(p.tr != 0, DPK_E_SHAPE, "%s: out=%lld in=%lld: no tile plan", who, (long long)out, (long long)in);
   const int64_t blocks = pieces * p.tiles_m * p.tiles_n;
-  const int64_t count4 = out * in / 4;  // out, in multiples of 8
+  const int64_t count4 = out * in / 4;  // out, in multiples of 4
   DPK_REQUIRE(blocks <= DPK_MAX_GRID_X && dpk_cdiv(count4, kThreads) <= DPK_MAX_GRID_X, DPK_E_SHAPE,
               "%s: %lld blocks exceed the grid limit", who, (long long)blocks);
-  hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 grid(static_cast<unsigned>(blocks));
+  float* none = nullptr;
+  if (in_dtype == DPK_F32) {
+    const float* bf = static_cast<const float*>(b);
+    const float* af = static_cast<const float*>(a);
+    if (dst_dtype == DPK_BF16)
+      hipLaunchKernelGGL((linear_dlds_kernel<DldsF32, DldsF32Cfg, bf16_t, true>), grid, dim3(DldsF32Cfg::kThreads), 0, s,
+                         bf, af, static_cast<bf16_t*>(dst), none, rows, out, in, scale, p.tiles_m, p.tiles_n, coef, T);
+    else
+      hipLaunchKernelGGL((linear_dlds_kernel<DldsF32, DldsF32Cfg, float, true>), grid, dim3(DldsF32Cfg::kThreads), 0, s,
+                         bf, af, static_cast<float*>(dst), none, rows, out, in, scale, p.tiles_m, p.tiles_n, coef, T);
+  } else {
   const bf16_t* bp = static_cast<const bf16_t*>(b);
   const bf16_t* ap = static_cast<const bf16_t*>(a);
-  float* none = nullptr;
 #define DPK_WSUM(CFG, TOUT)                                                                                    \
   hipLaunchKernelGGL((linear_dlds_kernel<TrBf16, CFG, TOUT, true>), grid, dim3(CFG::kThreads), 0, s, bp, ap, \
                      static_cast<TOUT*>(dst), none, rows, out, in, scale, p.tiles_m, p.tiles_n, coef, T)
@@ -834,6 +1081,7 @@ extern "C" int dpk_linear_weighted_sum(const void* b, const void* a, int in_dtyp
   else if (dst_dtype == DPK_BF16) DPK_WSUM(TrSmall, bf16_t);
   else DPK_WSUM(TrSmall, float);
 #undef DPK_WSUM
+  }
   DPK_LAUNCH_CHECK(who);
   if (split) {
     const dim3 g2(static_cast<unsigned>(dpk_cdiv(count4, kThreads)));
@@ -845,6 +1093,77 @@ extern "C" int dpk_linear_weighted_sum(const void* b, const void* a, int in_dtyp
                          static_cast<float*>(out_sum), count4, pieces);
     DPK_LAUNCH_CHECK(who);
   }
+  return DPK_OK;
+}
+
+// out_sum[k] = scale * sum_s coef[s] * sum_t b[s, t, k]: the clip-weighted sum of a Linear layer's
+// per-sample bias gradients (linear.py:50 weighted as fast_gradient_clipping_utils.py:193-201
+// weights the loss), one pass over b in chunks of rows and a fixed-order sum of the chunks.
+namespace {
+constexpr int64_t kWcolChunks = 256;
+struct WcolLayout {
+  size_t weights, total;
+  int64_t chunks, rows_per_chunk;
+};
+WcolLayout wcol_layout(int64_t n, int64_t T, int64_t out) {
+  WcolLayout l;
+  const int64_t rows = n * T;
+  l.chunks = rows < kWcolChunks ? rows : kWcolChunks;
+  l.rows_per_chunk = dpk_cdiv(rows, l.chunks);
+  l.chunks = dpk_cdiv(rows, l.rows_per_chunk);
+  l.weights = dpk_align_up(static_cast<size_t>(rows) * sizeof(float), 256);
+  l.total = l.weights + dpk_align_up(static_cast<size_t>(l.chunks) * out * sizeof(float), 256);
+  return l;
+}
+}  // namespace
+
+extern "C" size_t dpk_linear_bias_weighted_sum_workspace_bytes(int64_t n, int64_t T, int64_t out) {
+  if (n <= 0 || T <= 0 || out <= 0) return 0;
+  return wcol_layout(n, T, out).total;
+}
+
+extern "C" int dpk_linear_bias_weighted_sum(const void* b, int in_dtype, const float* coef, void* out_sum, int out_dtype,
+                                            int64_t n, int64_t T, int64_t out, float scale, void* ws, size_t ws_bytes,
+                                            dpk_stream_t stream) {
+  const char* who = "dpk_linear_bias_weighted_sum";
+  DPK_REQUIRE(n >= 1 && T >= 1 && out >= 1, DPK_E_SHAPE, "%s: n=%lld T=%lld out=%lld", who, (long long)n, (long long)T,
+              (long long)out);
+  DPK_REQUIRE(b && coef && out_sum, DPK_E_ARG, "%s: NULL tensor", who);
+  DPK_REQUIRE(dpk_dtype_ok(in_dtype) && dpk_dtype_ok(out_dtype), DPK_E_DTYPE, "%s: dtypes %d,%d", who, in_dtype, out_dtype);
+  DPK_REQUIRE(dpk_aligned(coef, 4) && dpk_aligned(b, dpk_elsize(in_dtype)) && dpk_aligned(out_sum, dpk_elsize(out_dtype)),
+              DPK_E_ALIGN, "%s: misaligned tensor", who);
+  const WcolLayout l = wcol_layout(n, T, out);
+  DPK_REQUIRE(ws && ws_bytes >= l.total, DPK_E_WORKSPACE, "%s: workspace %zu < %zu bytes", who, ws_bytes, l.total);
+  DPK_REQUIRE(dpk_aligned(ws, 256), DPK_E_ALIGN, "%s: workspace must be 256-byte aligned", who);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int64_t rows = n * T;
+  float* w = static_cast<float*>(ws);
+  float* part = reinterpret_cast<float*>(static_cast<char*>(ws) + l.weights);
+  const bool vec = out % 4 == 0 && dpk_aligned(b, 4 * dpk_elsize(in_dtype));
+  const int64_t col_blocks = dpk_cdiv(out, kThreads * (vec ? 4 : 1));
+  DPK_REQUIRE(l.chunks * col_blocks <= DPK_MAX_GRID_X && dpk_cdiv(rows, kThreads) <= DPK_MAX_GRID_X, DPK_E_SHAPE,
+              "%s: too many blocks", who);
+  hipLaunchKernelGGL(row_weights_kernel, dim3(static_cast<unsigned>(dpk_cdiv(rows, kThreads))), dim3(kThreads), 0, s, coef,
+                     w, rows, T);
+  DPK_LAUNCH_CHECK(who);
+  const dim3 grid(static_cast<unsigned>(l.chunks * col_blocks));
+#define DPK_WCOL(TIN, V)                                                                                        \
+  hipLaunchKernelGGL((wcolsum_partial_kernel<TIN, V>), grid, dim3(kThreads), 0, s, static_cast<const TIN*>(b), w, \
+                     part, rows, l.rows_per_chunk, out, col_blocks)
+  if (in_dtype == DPK_F32 && vec) DPK_WCOL(float, true);
+  else if (in_dtype == DPK_F32) DPK_WCOL(float, false);
+  else if (vec) DPK_WCOL(bf16_t, true);
+  else DPK_WCOL(bf16_t, false);
+#undef DPK_WCOL
+  DPK_LAUNCH_CHECK(who);
+  const dim3 g2(static_cast<unsigned>(dpk_cdiv(out, DPK_WAVE)));
+  if (out_dtype == DPK_BF16)
+    hipLaunchKernelGGL(wcolsum_final_kernel<bf16_t>, g2, dim3(kThreads), 0, s, part, static_cast<bf16_t*>(out_sum),
+                       l.chunks, out, scale);
+  else
+    hipLaunchKernelGGL(wcolsum_final_kernel<float>, g2, dim3(kThreads), 0, s, part, static_cast<float*>(out_sum), l.chunks,
+                       out, scale);
+  DPK_LAUNCH_CHECK(who);
   return DPK_OK;
 }
 

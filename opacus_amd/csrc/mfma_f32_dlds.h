@@ -24,6 +24,7 @@
 
 #include "dpk_common.h"
 #include "mfma_bf16_dlds.h"
+#include "mfma_bf16_tr.h"
 
 namespace mf32d {
 
@@ -116,6 +117,15 @@ struct Tile {
         for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
   }
 
+  __device__ __forceinline__ void scale(float f) {
+#pragma unroll
+    for (int i = 0; i < C::TP; ++i)
+#pragma unroll
+      for (int j = 0; j < C::TQ; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] *= f;
+  }
+
   // The MFMAs of the tile in `cur`, with the LDS reads of the next tile (into `nxt`) and the
   // global -> LDS loads of a later one (issue(q), q < kLoads) dealt out evenly between them.
   template <class IssueFn>
@@ -141,12 +151,25 @@ struct Tile {
 // (with tile kt + NS) as soon as every wave holds tile kt in registers. Every step issues
 // exactly one tile's loads (past the end the last tile again), so kLoads * (NS - 2) loads may
 // stay in flight while a tile is awaited.
-template <class C>
+//
+// kWeighted: as in mfma_bf16_tr.h. The K rows are units of tiles_per_unit k tiles each and unit u
+// counts coef[u] times; the accumulator is kept in units of the current unit's coefficient,
+// rescaled by coef[u - 1] / coef[u] at a unit's first tile (an fp32 tile's 64 MFMAs of 64 cycles
+// each dwarf the 64 multiplications) and by the last coefficient at the end, with the same floors.
+template <class C, bool kWeighted = false>
 __device__ __forceinline__ void mainloop(Tile<C>& t, Smem<C>& sm, const float* P, int64_t ldp, int64_t p0,
                                          const float* Q, int64_t ldq, int64_t q0, int64_t K, int wp0,
-                                         int wq0) {
+                                         int wq0, const float* coef = nullptr, int64_t tiles_per_unit = 0) {
   constexpr int NS = C::NS;
   const int64_t nk = (K + BK - 1) / BK;
+  int64_t boundary = 0, unit = 0, units = 0;
+  float c_cur = 1.f, c_nxt = 1.f;
+  if constexpr (kWeighted) {
+    units = nk / tiles_per_unit;
+    boundary = tiles_per_unit;
+    c_cur = mb16t::floored_coef(coef[0], 0.f);
+    c_nxt = coef[units > 1 ? 1 : 0];
+  }
   const int dup = static_cast<int>(nk * BK - K);  // rows the last tile repeats
   const uint32_t lds0 = lds_offset(&sm.stage[0][0]);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -205,6 +228,16 @@ __device__ __forceinline__ void mainloop(Tile<C>& t, Smem<C>& sm, const float* P
     wait_and_barrier<C::kLoads*(NS - 2)>();
     zero_repeated_rows(kt + 1);
     const unsigned char* st = sm.stage[(kt + 1) & (NS - 1)];
+    if constexpr (kWeighted) {
+      if (kt == boundary) {  // first tile of the next unit (uniform over the block)
+        const float c_new = mb16t::floored_coef(c_nxt, c_cur);
+        t.scale(c_cur / c_new);
+        c_cur = c_new;
+        ++unit;
+        boundary += tiles_per_unit;
+        c_nxt = coef[unit + 1 < units ? unit + 1 : units - 1];
+      }
+    }
     t.mma(cur, nxt, st, st + C::SUBP * SUB_BYTES, fp, fq, [&](int q) { issue_q(kt + NS, q); });
   };
   int64_t kt = 0;
@@ -215,6 +248,7 @@ __device__ __forceinline__ void mainloop(Tile<C>& t, Smem<C>& sm, const float* P
   if (kt < nk) step(kt, f0, f1);
   __builtin_amdgcn_s_waitcnt(kWaitLgkm0);
   wait_and_barrier<0>();  // the stage memory is the caller's again
+  if constexpr (kWeighted) t.scale(c_cur);
 }
 
 }  // namespace mf32d

@@ -14,9 +14,11 @@ their two ghost norms plus twice a cross term, ``kernels.tied_embedding_cross_te
 
 ``single_backward=True`` (the default) replaces the second backward pass: the hooks keep every
 layer's (activations, backprops) of the first pass, and once the clipping coefficients are known the
-clipped gradient sum of each layer is formed from them directly: one GEMM
-``(coef * b)^T a`` for a Linear layer, the weighted embedding backward for an Embedding, the
-layer's grad sampler and the clip-weighted sum for anything else. The sum is the one the
+clipped gradient sum of each layer is formed from them directly: one contraction over samples
+and positions with the coefficients applied inside the kernel for a Linear layer
+(``kernels.linear_weighted_sum[_multi]``, ``linear_bias_weighted_sum``), the per-id sum of the
+weighted backprop rows for an Embedding (``kernels.embedding_weighted_sum``), the layer's grad
+sampler and the clip-weighted sum for anything else. The sum is the one the
 second pass would have left in ``p.grad`` (the gradient of ``sum_n coef[n] loss[n]`` is linear
 in the per-sample backprops); what is saved is the pass's walk back through the activations,
 at the price of keeping the backprops alive until the coefficients exist (the first pass no
@@ -443,27 +445,43 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
             sums_w = kernels.linear_weighted_sum_multi([(b, a, c, scale) for _, a, b, scale in items])
             for (module, a, backprops, scale), total in zip(items, sums_w):
                 add(module.weight, total)
-                if module.bias is not None:
-                    per_sample = backprops.sum(dim=tuple(range(1, backprops.dim() - 1)), dtype=torch.float32)
-                    add(module.bias, ((c * scale) @ per_sample).to(backprops.dtype))
+                if module.bias is not None and module.bias.requires_grad:
+                    add(module.bias, kernels.linear_bias_weighted_sum(backprops, c, scale=scale))
         del pooled, by_device
         for module, activations, backprops, scale, grad_samples in rest:
             n = backprops.shape[0]
             c = coef.to(device=backprops.device, dtype=torch.float32)
             if n == 0:
                 continue
-            if self._sampler_for(module) is linear_grad_sampler:  # nn.Linear itself and RNNLinear, not a subclass with a forward of its own
+            if self._sampler_for(module) is linear_grad_sampler and kernels.native_dtype(backprops.dtype) and backprops.is_cuda:
+                # nn.Linear itself and RNNLinear (not a subclass with a forward of its own) in the shapes and
+                # dtypes the pooled contraction does not take: fp32, positions that are not whole k tiles,
+                # odd feature sizes. One contraction over all rows with the rows of the backprops weighted
+                # on their way into the kernel's LDS tiles: no weighted copy, no library GEMM.
+                if module.weight.requires_grad:
+                    add(module.weight, kernels.linear_weighted_sum(backprops, activations[0], c, scale=scale))
+                if module.bias is not None and module.bias.requires_grad:
+                    add(module.bias, kernels.linear_bias_weighted_sum(backprops, c, scale=scale))
+            elif self._sampler_for(module) is linear_grad_sampler:  # float16: widened operands, torch's GEMM
                 a = activations[0].to(backprops.dtype)
                 w = (c * scale).to(backprops.dtype).view(n, *([1] * (backprops.dim() - 1)))
-                if module.bias is None and a.shape[-1] < backprops.shape[-1]:
-                    # (coef * b)^T a == b^T (coef * a): weight the narrower of the two
-                    rows, cols = backprops, a * w
-                else:
-                    rows, cols = backprops * w, a
-                rows = rows.reshape(-1, rows.shape[-1])
-                add(module.weight, _rows_t_cols(rows, cols.reshape(-1, cols.shape[-1])))
+                rows = (backprops * w).reshape(-1, backprops.shape[-1])
+                add(module.weight, rows.t().mm(a.reshape(-1, a.shape[-1])))
                 if module.bias is not None:
                     add(module.bias, rows.sum(dim=0))
+            elif (
+                type(module) is nn.Embedding
+                and module.max_norm is None
+                and not module.scale_grad_by_freq
+                and kernels.native_dtype(backprops.dtype)
+                and backprops.is_cuda
+            ):
+                # every table row is the fp32 sum, over the whole batch, of the weighted backprop rows of
+                # the positions that name it, written once
+                total = kernels.embedding_weighted_sum(activations[0], backprops, c, module.num_embeddings, scale=scale)
+                if module.padding_idx is not None:
+                    total[module.padding_idx].zero_()  # autograd's embedding backward leaves that row at zero
+                add(module.weight, total)
             elif type(module) is nn.Embedding and module.max_norm is None:
                 ids = activations[0]
                 weighted = backprops * (c * scale).to(backprops.dtype).view(n, *([1] * (backprops.dim() - 1)))
@@ -535,36 +553,6 @@ class GradSampleHooksFastGradientClipping(GradSampleHooks):
     @per_sample_gradient_norms.setter
     def per_sample_gradient_norms(self, value):
         self._per_sample_gradient_norms = value
-
-
-def _rows_t_cols(rows: torch.Tensor, cols: torch.Tensor) -> torch.Tensor:
-    """``rows^T cols`` for ``rows [K, out]`` and ``cols [K, in]``: the clip-weighted sum of a Linear
-    layer's per-sample gradients, one contraction over all samples and positions. Both operands
-    have the contracted dimension as their slow one, which is the layout the library's bf16
-    Linear contraction is built for (``dpk_linear_gs`` on one "sample" of K rows): on the
-    benchmark shapes it runs at 0.83-1.1 PFLOP/s against 0.74-1.04 for ``torch.mm`` on the
-    transposed view, and a thin layer (few output tiles) is cut into four pieces along K whose
-    fp32 partial products are added (2048 x 512: 50 against 111 us). Other dtypes and shapes go
-    to ``torch.mm``."""
-    K_, out_f, in_f = rows.shape[0], rows.shape[1], cols.shape[1]
-    if (
-        rows.is_cuda
-        and rows.dtype == torch.bfloat16
-        and cols.dtype == torch.bfloat16
-        and out_f % 64 == 0
-        and in_f % 64 == 0
-        and K_ % 256 == 0
-        and K_ >= 2048
-    ):
-        pieces = 4 if (out_f // 128) * (in_f // 128) < 128 else 1
-        if pieces == 1:
-            return kernels.linear_grad_sample(rows.view(1, K_, out_f), cols.view(1, K_, in_f), want_sumsq=False)[0][0]
-        part, _ = kernels.linear_grad_sample(
-            rows.view(pieces, K_ // pieces, out_f), cols.view(pieces, K_ // pieces, in_f), want_sumsq=False,
-            out_dtype=torch.float32,
-        )
-        return part.sum(0).to(rows.dtype)
-    return rows.t().mm(cols)
 
 
 class GradSampleModuleFastGradientClipping(GradSampleHooksFastGradientClipping, AbstractGradSampleModule):

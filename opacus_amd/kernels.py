@@ -179,9 +179,10 @@ def linear_grad_sample(
 
 
 def linear_weighted_sum_takes(backprops: torch.Tensor, activations: torch.Tensor) -> bool:
-    """Whether :func:`linear_weighted_sum` takes the pair (the shapes ``dpk_linear_weighted_sum``
-    accepts): bf16 on the GPU, whole k tiles of 32 positions per sample, feature counts that are
-    multiples of 8 above 64."""
+    """Whether the pair goes to the bf16 contraction with the coefficients on its accumulators
+    (and may be pooled by :func:`linear_weighted_sum_multi`): bf16 on the GPU, whole k tiles of 32
+    positions per sample, feature counts that are multiples of 8 above 64. Any other pair
+    :func:`linear_weighted_sum` sends to the fp32 MFMA kernel with weighted rows."""
     if not (backprops.is_cuda and backprops.dtype == torch.bfloat16 and activations.dtype == torch.bfloat16):
         return False
     if backprops.dim() < 3 or backprops.shape[0] == 0 or backprops.shape[:-1] != activations.shape[:-1]:
@@ -200,12 +201,16 @@ def linear_weighted_sum(
     out_dtype: Optional[torch.dtype] = None,
 ) -> torch.Tensor:
     """``sum_n coef[n] * scale * b[n]^T a[n]`` as ``[out, in]``: the clip-weighted sum of a Linear
-    layer's per-sample gradients in one contraction over samples and positions, the weights
-    applied to the accumulators where a sample begins. ``pieces`` cuts the samples into that
-    many runs whose fp32 sums a second kernel adds (default: 4 for a layer with at most
-    256 output tiles of 128 x 128, which alone would not fill the GPU twice over, when n allows;
-    else 1)."""
+    layer's per-sample gradients in one contraction over samples and positions, for fp32 and
+    bf16 operands of any shape (see :func:`linear_weighted_sum_takes` for the two kernels behind
+    it). ``pieces`` cuts the samples (or rows) into that many runs whose fp32 sums a second kernel
+    adds (default: 4 for a layer with at most 256 output tiles of 128 x 128, which alone would not
+    fill the GPU twice over, when n allows; else 1)."""
     dev = _need_gpu(backprops, activations, coef)
+    if activations.dtype != backprops.dtype:
+        activations = activations.to(backprops.dtype)
+    if not native_dtype(backprops.dtype):
+        raise TypeError(f"linear_weighted_sum takes float32 and bfloat16, not {backprops.dtype}")
     n, out_f, in_f = backprops.shape[0], backprops.shape[-1], activations.shape[-1]
     b = _dense(backprops).reshape(n, -1, out_f)
     a = _dense(activations).reshape(n, -1, in_f)
@@ -217,10 +222,15 @@ def linear_weighted_sum(
         raise ValueError(f"{c.numel()} coefficients for {n} samples")
     if pieces is None:
         few_tiles = -(-out_f // 128) * -(-in_f // 128) <= 256
-        pieces = 4 if few_tiles and n % 4 == 0 else 1
+        # the kernels with the coefficients on the accumulators cut along whole samples, the one with
+        # weighted rows anywhere
+        per_sample = linear_weighted_sum_takes(b, a) or (
+            b.dtype == torch.float32 and T % 16 == 0 and out_f % 4 == 0 and in_f % 8 == 0 and out_f > 64 and in_f > 64
+        )
+        pieces = 4 if few_tiles and (out_f * in_f) % 4 == 0 and (n % 4 == 0 or not per_sample) and n * T >= 256 else 1
     out = torch.empty((out_f, in_f), dtype=out_dtype or backprops.dtype, device=dev)
     L = lib()
-    ws, wsb = _ws(L.dpk_linear_weighted_sum_workspace_bytes(out_f, in_f, int(pieces)), dev)
+    ws, wsb = _ws(L.dpk_linear_weighted_sum_workspace_bytes(n, T, out_f, in_f, _code(b), int(pieces)), dev)
     with _timed("linear_weighted_sum", dev):
         check(
             "dpk_linear_weighted_sum",
@@ -276,6 +286,33 @@ def linear_weighted_sum_multi(
         )
     del keep
     return outs
+
+
+def linear_bias_weighted_sum(
+    backprops: torch.Tensor, coef: torch.Tensor, scale: float = 1.0, out_dtype: Optional[torch.dtype] = None
+) -> torch.Tensor:
+    """``scale * sum_n coef[n] * sum_t b[n, t, :]`` as ``[out]``: the clip-weighted sum of a Linear
+    layer's per-sample bias gradients, one pass over the backprops."""
+    dev = _need_gpu(backprops, coef)
+    if not native_dtype(backprops.dtype):
+        raise TypeError(f"linear_bias_weighted_sum takes float32 and bfloat16, not {backprops.dtype}")
+    n, out_f = backprops.shape[0], backprops.shape[-1]
+    b = _dense(backprops).reshape(n, -1, out_f)
+    T = b.shape[1]
+    c = _dense(coef.to(torch.float32)).reshape(-1)
+    if c.numel() != n:
+        raise ValueError(f"{c.numel()} coefficients for {n} samples")
+    out = torch.empty((out_f,), dtype=out_dtype or backprops.dtype, device=dev)
+    L = lib()
+    ws, wsb = _ws(L.dpk_linear_bias_weighted_sum_workspace_bytes(n, T, out_f), dev)
+    with _timed("linear_bias_weighted_sum", dev):
+        check(
+            "dpk_linear_bias_weighted_sum",
+            L.dpk_linear_bias_weighted_sum(
+                _ptr(b), _code(b), _ptr(c), _ptr(out), _code(out), n, T, out_f, float(scale), _ptr(ws), wsb, _stream(dev)
+            ),
+        )
+    return out
 
 
 def _with_sumsq(gs: torch.Tensor, sumsq: torch.Tensor) -> torch.Tensor:
@@ -602,6 +639,47 @@ def embedding_grad_sample(
     if VALIDATE_EMBEDDING_INDICES:
         check_embedding_indices(dev)
     return gs
+
+
+def embedding_weighted_sum(
+    ids: torch.Tensor,
+    backprops: torch.Tensor,
+    coef: torch.Tensor,
+    num_embeddings: int,
+    scale: float = 1.0,
+    out_dtype: Optional[torch.dtype] = None,
+) -> torch.Tensor:
+    """``out[v, :] = scale * sum_n coef[n] * sum_{t: ids[n,t]==v} b[n,t,:]`` as ``[V, D]``: the
+    clip-weighted sum of an Embedding table's per-sample gradients, summed per id in fp32 over the
+    whole batch in a fixed order. ``out_dtype``: the backprops' dtype (default) or float32."""
+    dev = _need_gpu(ids, backprops, coef)
+    if not native_dtype(backprops.dtype):
+        raise TypeError(f"embedding_weighted_sum takes float32 and bfloat16, not {backprops.dtype}")
+    ids2 = _ids_2d(ids)
+    n, T = ids2.shape
+    D = backprops.shape[-1]
+    out = torch.empty((num_embeddings, D), dtype=out_dtype or backprops.dtype, device=dev)
+    if n == 0 or T == 0:
+        return out.zero_()
+    b = _dense(backprops).reshape(n, -1, D)
+    if b.shape[1] != T:
+        raise ValueError(f"ids {tuple(ids.shape)} and backprops {tuple(backprops.shape)} disagree")
+    c = _dense(coef.to(torch.float32)).reshape(-1)
+    if c.numel() != n:
+        raise ValueError(f"{c.numel()} coefficients for {n} samples")
+    L = lib()
+    ws, wsb = _ws(L.dpk_embedding_weighted_sum_workspace_bytes(n, T, D), dev)
+    with _timed("embedding_weighted_sum", dev):
+        check(
+            "dpk_embedding_weighted_sum",
+            L.dpk_embedding_weighted_sum(
+                _ptr(ids2), _ptr(b), _code(b), _ptr(c), _ptr(out), _code(out), n, T, num_embeddings, D, float(scale),
+                _ptr(_emb_status(dev)), _ptr(ws), wsb, _stream(dev),
+            ),
+        )
+    if VALIDATE_EMBEDDING_INDICES:
+        check_embedding_indices(dev)
+    return out
 
 
 def embedding_ghost_norm(ids: torch.Tensor, backprops: torch.Tensor, scale: float = 1.0) -> torch.Tensor:

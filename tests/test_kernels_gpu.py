@@ -572,7 +572,7 @@ def test_linear_weighted_sum_multi(K, count):
         K.linear_weighted_sum_multi([(b[:, :16].contiguous(), a[:, :16].contiguous(), c, 1.0)], pooled=True)
 
 
-def test_linear_weighted_sum_keeps_a_nan_and_refuses_other_shapes(K):
+def test_linear_weighted_sum_keeps_a_nan_and_multi_refuses_other_shapes(K):
     torch.manual_seed(5)
     a, b = dev(torch.randn(4, 32, 128).bfloat16()), dev(torch.randn(4, 32, 128).bfloat16())
     c = torch.tensor([0.5, float("nan"), 0.25, 1.0])
@@ -580,10 +580,119 @@ def test_linear_weighted_sum_keeps_a_nan_and_refuses_other_shapes(K):
     assert not K.linear_weighted_sum_takes(b[:, :16], a[:, :16])  # half a k tile per sample
     assert not K.linear_weighted_sum_takes(b.float(), a.float())
     assert not K.linear_weighted_sum_takes(b[..., :64], a)
+    with pytest.raises(RuntimeError, match="dpk_linear_weighted_sum_multi"):  # the pool takes the bf16 kernel's shapes only
+        K.linear_weighted_sum_multi([(b[:, :16].contiguous(), a[:, :16].contiguous(), dev(c), 1.0)])
     with pytest.raises(RuntimeError, match="dpk_linear_weighted_sum"):
-        K.linear_weighted_sum(b[:, :16].contiguous(), a[:, :16].contiguous(), dev(c))
-    with pytest.raises(RuntimeError, match="dpk_linear_weighted_sum"):
-        K.linear_weighted_sum(b, a, dev(c), pieces=3)
+        K.linear_weighted_sum(b, a, dev(c), pieces=0)
+    with pytest.raises(TypeError):
+        K.linear_weighted_sum(b.half(), a.half(), dev(c))
+
+
+# fp32 operands, positions that are not whole k tiles, odd feature sizes, misaligned tensors: the fp32
+# MFMA kernel with weighted rows
+GENERIC_WSUM_CASES = [
+    # (n, mid, in, out, dtype, pieces)
+    (5, (7,), 24, 40, torch.float32, 1),
+    (6, (33,), 136, 200, torch.float32, None),
+    (3, (4, 5), 30, 18, torch.float32, 1),  # odd sizes: element-wise loads
+    (8, (64,), 256, 128, torch.float32, 4),
+    (4, (50,), 128, 256, torch.bfloat16, None),  # bf16, 50 positions per sample
+    (2, (31,), 72, 100, torch.bfloat16, 2),
+    (7, (1,), 64, 32, torch.float32, 1),  # one position per sample
+    (3, (), 48, 16, torch.float32, 1),  # 2-d input
+    # fp32 with whole k tiles of 16 positions: the direct-load fp32 kernel, coefficients on its accumulators
+    (8, (16,), 128, 128, torch.float32, 1),  # one k tile per sample: a rescaling before every tile
+    (6, (48,), 136, 200, torch.float32, 2),  # ragged block tiles
+    (16, (128,), 512, 256, torch.float32, None),
+    (4, (80,), 1024, 1024, torch.float32, 1),
+]
+
+
+@pytest.mark.parametrize("n,mid,fin,fout,dtype,pieces", GENERIC_WSUM_CASES)
+@pytest.mark.parametrize("coefs", ["spread", "tiny_and_zero"])
+def test_linear_weighted_sum_generic_shapes(K, n, mid, fin, fout, dtype, pieces, coefs):
+    """sum_n coef[n] * b[n]^T a[n] and the bias sum for everything the bf16 tile kernel does not
+    take, against (coef * gs).sum(0) of the oracle's per-sample gradients in fp64: fp32 1e-5, bf16
+    inputs exact products with fp32 accumulation (1e-5 into an fp32 result, one rounding into bf16)."""
+    torch.manual_seed(n * 31 + fin)
+    a = torch.randn(n, *mid, fin).to(dtype)
+    b = (torch.randn(n, *mid, fout) * 0.3).to(dtype)
+    c = torch.rand(n) * 0.99 + 0.01
+    if coefs == "tiny_and_zero":
+        c[0], c[n // 2], c[-1] = 1e-12, 0.0, 3e-9
+    assert not K.linear_weighted_sum_takes(dev(b), dev(a))
+    gs_w, gs_b = O.linear_grad_sample(a.double(), b.double())
+    want_w = (c.double().view(n, 1, 1) * gs_w).sum(0) * 1.5
+    want_b = (c.double().view(n, 1) * gs_b).sum(0) * 1.5
+    for out_dtype in (None, torch.float32):
+        got = K.linear_weighted_sum(dev(b), dev(a), dev(c), scale=1.5, pieces=pieces, out_dtype=out_dtype)
+        assert got.shape == (fout, fin) and got.dtype == (out_dtype or dtype)
+        bar = BF16_REL if (out_dtype or dtype) == torch.bfloat16 else FP32_REL
+        assert_rel(got[None], want_w[None], bar, f"weighted sum {dtype} -> {got.dtype}")
+        got_b = K.linear_bias_weighted_sum(dev(b), dev(c), scale=1.5, out_dtype=out_dtype)
+        assert got_b.shape == (fout,) and got_b.dtype == (out_dtype or dtype)
+        assert_rel(got_b, want_b, bar, f"bias weighted sum {dtype} -> {got_b.dtype}")
+    if dtype == torch.bfloat16:
+        # operands two bytes off a 16-byte boundary take the same path
+        odd_b = torch.empty(b.numel() + 1, dtype=dtype, device="cuda")[1:].view(b.shape).copy_(b)
+        got = K.linear_weighted_sum(odd_b, dev(a), dev(c), scale=1.5, pieces=pieces, out_dtype=torch.float32)
+        assert_rel(got[None], want_w[None], FP32_REL, "misaligned backprops")
+
+
+def test_linear_bias_weighted_sum_at_benchmark_width(K):
+    """C3's first layer: 32 x 512 rows of 4096 bf16 columns, 64 chunks of rows."""
+    torch.manual_seed(2)
+    n, T, D = 32, 512, 4096
+    b = (torch.randn(n, T, D) * 0.02).bfloat16()
+    c = torch.rand(n) * 0.9 + 0.1
+    want = (c.double().view(n, 1, 1) * b.double()).sum((0, 1))
+    assert_rel(K.linear_bias_weighted_sum(dev(b), dev(c), out_dtype=torch.float32), want, 1e-5, "bias weighted sum")
+    assert_rel(K.linear_bias_weighted_sum(dev(b), dev(c)), want, BF16_REL, "bias weighted sum bf16")
+
+
+@pytest.mark.parametrize(
+    "n,Tshape,V,D,dtype",
+    [(5, (3, 2), 9, 4, torch.float32), (3, (40,), 7, 17, torch.float32), (4, (300,), 50, 64, torch.bfloat16),
+     (2, (64,), 10, 1030, torch.float32), (6, (1000,), 3000, 128, torch.bfloat16), (3, (2000,), 11, 8, torch.float32),
+     (1, (1,), 1, 4, torch.float32)],
+)
+def test_embedding_weighted_sum(K, n, Tshape, V, D, dtype):
+    """out[v] = sum_n coef[n] sum_{t: ids[n,t]==v} b[n,t]: the clip-weighted sum of the Embedding
+    per-sample gradients, against the oracle's [n, V, D] gradients weighted and added in fp64
+    (ids repeated inside a sample and across samples; the batch as one run of up to 6000 positions:
+    lists by sorting below 4096, by the pairwise scan above). Which rows are written is index work:
+    exact. Two runs give the same bits."""
+    torch.manual_seed(V * 7 + D)
+    ids = torch.randint(0, V, (n, *Tshape))
+    b = torch.randn(n, *Tshape, D).to(dtype)
+    c = torch.rand(n) * 0.9 + 0.1
+    if n > 2:
+        c[1] = 0.0
+    gs = O.embedding_grad_sample(ids, b.double(), V)
+    want = (c.double().view(n, 1, 1) * gs).sum(0) * 0.5
+    K.check_embedding_indices("cuda")
+    for out_dtype in (None, torch.float32):
+        got = K.embedding_weighted_sum(dev(ids), dev(b), dev(c), V, scale=0.5, out_dtype=out_dtype)
+        assert got.shape == (V, D) and got.dtype == (out_dtype or dtype)
+        # rows as the groups of the comparison: every table row is held to its own size
+        assert_rel(got, want, BF16_REL if got.dtype == torch.bfloat16 else FP32_REL, f"embedding weighted sum -> {got.dtype}")
+        named = torch.zeros(V, dtype=torch.bool)
+        named[ids.reshape(-1)] = True
+        assert not got.cpu()[~named].any(), "a row no id names was written"
+        again = K.embedding_weighted_sum(dev(ids), dev(b), dev(c), V, scale=0.5, out_dtype=out_dtype)
+        assert torch.equal(got, again)
+    K.check_embedding_indices("cuda")
+    # an id outside the table contributes nothing and raises the flag
+    bad = ids.clone()
+    bad.view(-1)[0] = V
+    got = K.embedding_weighted_sum(dev(bad), dev(b), dev(c), V, out_dtype=torch.float32)
+    with pytest.raises(IndexError, match="outside"):
+        K.check_embedding_indices("cuda")
+    keep = torch.ones(ids.numel(), dtype=torch.bool)
+    keep[0] = False
+    want2 = torch.zeros(V, D, dtype=torch.float64)
+    want2.index_add_(0, ids.reshape(-1)[keep], (c.double().repeat_interleave(ids[0].numel()).view(-1, 1) * b.double().reshape(-1, D))[keep])
+    assert_rel(got, want2, FP32_REL if dtype == torch.float32 else 1e-4, "with one id out of range")
 
 
 def test_linear_ghost_norm_2d_inputs(K):
