@@ -232,17 +232,24 @@ struct SortMem {
   int32_t wide;  // some id of the sample does not fit the packed form
 };
 
+// total: ids holds this many entries in all (the last "sample" may be shorter than T: a run of
+// positions of a flattened batch). sorted_ids / sorted_pos (nullable): the sample's sorted (id,
+// position) pairs, entry i of sample s at s * T + i, for a merge across samples.
 template <int E>
 __device__ __forceinline__ void sort_link_sample(SortMem<E>& m, int64_t sample, const int64_t* __restrict__ ids, int T,
                                                  int64_t V, int32_t* __restrict__ next, int32_t* __restrict__ leader,
                                                  int32_t* __restrict__ rank, int32_t* __restrict__ count,
-                                                 int32_t* __restrict__ flag) {
+                                                 int32_t* __restrict__ flag, int64_t total = INT64_MAX,
+                                                 int64_t* __restrict__ sorted_ids = nullptr,
+                                                 int32_t* __restrict__ sorted_pos = nullptr) {
   constexpr int64_t kPackLimit = int64_t{1} << 51;
   int64_t* key = m.key;
   int32_t* pos = m.pos;
   int32_t* runs = m.runs;
   int32_t& wide = m.wide;
   const int64_t* row = ids + sample * T;
+  // entries of this sample (a short last run of a flattened batch: what lies past it is padding)
+  const int len = total - sample * T < T ? static_cast<int>(total - sample * T) : T;
   const int tid = threadIdx.x;
   if (tid == 0) wide = 0;
   __syncthreads();
@@ -251,9 +258,9 @@ __device__ __forceinline__ void sort_link_sample(SortMem<E>& m, int64_t sample, 
 #pragma unroll
   for (int e = 0; e < E; ++e) {
     const int i = tid * E + e;
-    const bool live = i < T;
+    const bool live = i < len;
     v[e].key = live ? row[i] : INT64_MAX;
-    v[e].pos = live ? i : T + i;  // padding sorts behind every real pair, whatever its id
+    v[e].pos = live ? i : T + i;  // padding sorts behind every real pair, whatever its id (positions < T are real)
     bad = bad || (live && V > 0 && (v[e].key < 0 || v[e].key >= V));
     big = big || (live && (v[e].key < 0 || v[e].key >= kPackLimit));
   }
@@ -283,13 +290,19 @@ __device__ __forceinline__ void sort_link_sample(SortMem<E>& m, int64_t sample, 
     pos[tid * E + e] = v[e].pos;
   }
   __syncthreads();
-  const int lo = tid * E, hi = lo + E < T ? lo + E : T;
+  const int lo = tid * E, hi = lo + E < len ? lo + E : len;
+  if (sorted_ids) {  // uniform
+    for (int i = lo; i < hi; ++i) {
+      sorted_ids[sample * T + i] = key[i];
+      sorted_pos[sample * T + i] = pos[i];
+    }
+  }
   int32_t mine = 0;
   for (int i = lo; i < hi; ++i) {
     const bool lead = i == 0 || key[i - 1] != key[i];
     mine += lead ? 1 : 0;
     const int p = pos[i];
-    next[sample * T + p] = (i + 1 < T && key[i + 1] == key[i]) ? pos[i + 1] : -1;
+    next[sample * T + p] = (i + 1 < len && key[i + 1] == key[i]) ? pos[i + 1] : -1;
     leader[sample * T + p] = lead ? 1 : 0;
   }
   if (!rank) return;  // uniform
@@ -313,6 +326,91 @@ __global__ __launch_bounds__(kThreads) void emb_sort_link_kernel(const int64_t* 
                                                                   int32_t* __restrict__ flag) {
   __shared__ SortMem<E> m;
   sort_link_sample<E>(m, blockIdx.x, ids, T, V, next, leader, rank, count, flag);
+}
+
+// ---- lists across a whole batch: sorted runs, then a merge by binary search ------------------
+// The L positions of a flattened batch are cut into runs of R <= kSortMax positions; one block
+// sorts each run (the kernel above, which also leaves the run's sorted (id, position) pairs),
+// and the kernel below links equal ids across runs: a position's successor is the next entry of
+// its run when that has the same id, else the first entry with that id of the nearest later run
+// that has one; it leads its list when no earlier entry of its run and no earlier run has the id.
+// Lists are therefore in increasing position, as a single scan over the batch would build them.
+template <int E>
+__global__ __launch_bounds__(kThreads) void emb_sort_runs_kernel(const int64_t* __restrict__ ids, int R, int64_t V,
+                                                                  int64_t total, int32_t* __restrict__ next,
+                                                                  int32_t* __restrict__ leader,
+                                                                  int64_t* __restrict__ sorted_ids,
+                                                                  int32_t* __restrict__ sorted_pos,
+                                                                  int32_t* __restrict__ flag) {
+  __shared__ SortMem<E> m;
+  sort_link_sample<E>(m, blockIdx.x, ids, R, V, next, leader, nullptr, nullptr, flag, total, sorted_ids, sorted_pos);
+}
+
+// One thread per sorted entry (run r, index i). The searches of a group of eight other runs advance
+// together, so that eight loads are in flight per step instead of one.
+__global__ __launch_bounds__(kThreads) void emb_merge_runs_kernel(const int64_t* __restrict__ sorted_ids,
+                                                                   const int32_t* __restrict__ sorted_pos, int R,
+                                                                   int64_t total, int nruns,
+                                                                   int32_t* __restrict__ next,
+                                                                   int32_t* __restrict__ leader) {
+  const int64_t e = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  const int r = static_cast<int>(e / R), i = static_cast<int>(e % R);
+  auto run_len = [&](int q) { return static_cast<int>(total - static_cast<int64_t>(q) * R < R ? total - static_cast<int64_t>(q) * R : R); };
+  if (r >= nruns || i >= run_len(r)) return;
+  const int64_t* mine = sorted_ids + static_cast<int64_t>(r) * R;
+  const int64_t sid = mine[i];
+  const int len = run_len(r);
+  const bool first = i == 0 || mine[i - 1] != sid;
+  const bool last = i + 1 == len || mine[i + 1] != sid;
+  const int64_t g = static_cast<int64_t>(r) * R + sorted_pos[static_cast<int64_t>(r) * R + i];
+  int64_t succ = last ? -1 : static_cast<int64_t>(r) * R + sorted_pos[static_cast<int64_t>(r) * R + i + 1];
+  bool earlier = false;
+  int best = nruns;
+  if (first || last) {
+    constexpr int G = 8;
+    for (int q0 = 0; q0 < nruns; q0 += G) {
+      int lo[G], left[G];
+#pragma unroll
+      for (int j = 0; j < G; ++j) {
+        const int q = q0 + j;
+        const bool want = q < nruns && ((q > r && last && q < best) || (q < r && first && !earlier));
+        lo[j] = 0;
+        left[j] = want ? run_len(q) : 0;
+      }
+      // lower bound of sid in every wanted run: at most 13 halvings of 4096 entries
+#pragma unroll 1
+      for (int step = 0; step < 13; ++step) {
+#pragma unroll
+        for (int j = 0; j < G; ++j) {
+          if (left[j] > 0) {
+            const int half = left[j] >> 1, mid = lo[j] + half;
+            const int64_t v = sorted_ids[static_cast<int64_t>(q0 + j) * R + mid];
+            if (v < sid) {
+              lo[j] = mid + 1;
+              left[j] -= half + 1;
+            } else {
+              left[j] = half;
+            }
+          }
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < G; ++j) {
+        const int q = q0 + j;
+        const bool want = q < nruns && ((q > r && last && q < best) || (q < r && first && !earlier));
+        if (want && lo[j] < run_len(q) && sorted_ids[static_cast<int64_t>(q) * R + lo[j]] == sid) {
+          if (q > r) {
+            best = q;
+            succ = static_cast<int64_t>(q) * R + sorted_pos[static_cast<int64_t>(q) * R + lo[j]];
+          } else {
+            earlier = true;
+          }
+        }
+      }
+    }
+  }
+  next[g] = static_cast<int32_t>(succ);
+  leader[g] = first && !earlier ? 1 : 0;
 }
 
 // rank[t] = #{leaders t' of the sample with ids[t'] < ids[t]}; count[sample] = #leaders.
@@ -709,9 +807,30 @@ extern "C" int dpk_embedding_gs(const int64_t* ids, const void* b, int in_dtype,
   return DPK_OK;
 }
 
+namespace {
+// Run length of the batch-wide sort: short runs sort faster and give more blocks, long runs keep the
+// number of runs (searches per entry in the merge) down.
+int batch_run_length(int64_t L) { return L <= 1024 ? static_cast<int>(L <= 256 ? 256 : (L <= 512 ? 512 : 1024)) : (L <= 32768 ? 1024 : kSortMax); }
+
+struct EmbBatchLayout {
+  size_t lists, weights, sorted_ids, sorted_pos, total;
+};
+EmbBatchLayout batch_layout(int64_t L, int64_t D) {
+  EmbBatchLayout l;
+  const int R = batch_run_length(L);
+  const int64_t padded = dpk_cdiv(L, R) * R;
+  l.lists = ws_layout(1, L, D, nullptr, nullptr);
+  l.weights = l.lists;
+  l.sorted_ids = l.weights + dpk_align_up(static_cast<size_t>(L) * sizeof(float), 256);
+  l.sorted_pos = l.sorted_ids + dpk_align_up(static_cast<size_t>(padded) * sizeof(int64_t), 256);
+  l.total = l.sorted_pos + dpk_align_up(static_cast<size_t>(padded) * sizeof(int32_t), 256);
+  return l;
+}
+}  // namespace
+
 extern "C" size_t dpk_embedding_weighted_sum_workspace_bytes(int64_t n, int64_t T, int64_t D) {
   if (n <= 0 || T <= 0) return 0;
-  return ws_layout(1, n * T, D, nullptr, nullptr) + dpk_align_up(static_cast<size_t>(n * T) * sizeof(float), 256);
+  return batch_layout(n * T, D).total;
 }
 
 // out[v, :] = scale * sum_n coef[n] * sum_{t : ids[n,t] == v} b[n,t,:]: the clip-weighted sum of the
@@ -734,19 +853,36 @@ extern "C" int dpk_embedding_weighted_sum(const int64_t* ids, const void* b, int
               DPK_E_ALIGN, "%s: misaligned tensor (out must be 16-byte aligned)", who);
   const int64_t L = n * T;
   DPK_REQUIRE(L < (int64_t{1} << 31), DPK_E_SHAPE, "%s: n * T = %lld positions", who, (long long)L);
-  const size_t lists = ws_layout(1, L, D, nullptr, nullptr);
-  const size_t need = lists + dpk_align_up(static_cast<size_t>(L) * sizeof(float), 256);
+  const EmbBatchLayout lay = batch_layout(L, D);
   EmbWs w;
   int rc = check_common(who, ids, 1, L, D, ws, ws_bytes, &w);
   if (rc != DPK_OK) return rc;
-  DPK_REQUIRE(ws_bytes >= need, DPK_E_WORKSPACE, "%s: workspace %zu < %zu bytes", who, ws_bytes, need);
-  float* rw = reinterpret_cast<float*>(static_cast<char*>(ws) + lists);
+  DPK_REQUIRE(ws_bytes >= lay.total, DPK_E_WORKSPACE, "%s: workspace %zu < %zu bytes", who, ws_bytes, lay.total);
+  char* base = static_cast<char*>(ws);
+  float* rw = reinterpret_cast<float*>(base + lay.weights);
+  int64_t* sorted_ids = reinterpret_cast<int64_t*>(base + lay.sorted_ids);
+  int32_t* sorted_pos = reinterpret_cast<int32_t*>(base + lay.sorted_pos);
   const int64_t tch = dpk_cdiv(L, kLeadersPerBlock), dch = dpk_cdiv(D, kThreads * 4);
-  DPK_REQUIRE(tch * dch <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: too many blocks", who);
+  const int R = batch_run_length(L);
+  const int64_t nruns = dpk_cdiv(L, R);
+  DPK_REQUIRE(tch * dch <= DPK_MAX_GRID_X && nruns <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: too many blocks", who);
   hipStream_t s = static_cast<hipStream_t>(stream);
   hipLaunchKernelGGL(emb_row_weights_kernel, dim3(static_cast<unsigned>(dpk_cdiv(L, kThreads))), dim3(kThreads), 0, s, coef,
                      rw, L, T);
-  launch_link(ids, 1, L, V, w, status, false, s);
+  // lists of equal ids over the whole batch: sorted runs, merged by binary search
+  {
+    const dim3 grid(static_cast<unsigned>(nruns)), block(kThreads);
+#define DPK_RUNS(E_) \
+  hipLaunchKernelGGL(emb_sort_runs_kernel<E_>, grid, block, 0, s, ids, R, V, L, w.next, w.leader, sorted_ids, sorted_pos, status)
+    if (R <= 256) DPK_RUNS(1);
+    else if (R <= 512) DPK_RUNS(2);
+    else if (R <= 1024) DPK_RUNS(4);
+    else DPK_RUNS(16);
+#undef DPK_RUNS
+    DPK_LAUNCH_CHECK(who);
+    hipLaunchKernelGGL(emb_merge_runs_kernel, dim3(static_cast<unsigned>(dpk_cdiv(nruns * R, kThreads))), dim3(kThreads), 0,
+                       s, sorted_ids, sorted_pos, R, L, static_cast<int>(nruns), w.next, w.leader);
+  }
   DPK_LAUNCH_CHECK(who);
   const size_t bytes = static_cast<size_t>(V) * D * dpk_elsize(out_dtype);
   const int64_t n16 = static_cast<int64_t>(bytes / 16);

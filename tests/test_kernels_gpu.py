@@ -654,13 +654,14 @@ def test_linear_bias_weighted_sum_at_benchmark_width(K):
     "n,Tshape,V,D,dtype",
     [(5, (3, 2), 9, 4, torch.float32), (3, (40,), 7, 17, torch.float32), (4, (300,), 50, 64, torch.bfloat16),
      (2, (64,), 10, 1030, torch.float32), (6, (1000,), 3000, 128, torch.bfloat16), (3, (2000,), 11, 8, torch.float32),
-     (1, (1,), 1, 4, torch.float32)],
+     (1, (1,), 1, 4, torch.float32), (40, (1000,), 50000, 8, torch.float32), (9, (4097,), 300, 4, torch.float32),
+     (5, (1023,), 2, 4, torch.float32)],
 )
 def test_embedding_weighted_sum(K, n, Tshape, V, D, dtype):
     """out[v] = sum_n coef[n] sum_{t: ids[n,t]==v} b[n,t]: the clip-weighted sum of the Embedding
     per-sample gradients, against the oracle's [n, V, D] gradients weighted and added in fp64
-    (ids repeated inside a sample and across samples; the batch as one run of up to 6000 positions:
-    lists by sorting below 4096, by the pairwise scan above). Which rows are written is index work:
+    (ids repeated inside a sample and across samples; the batch of up to 40000 positions is sorted in
+    runs of 1024 or 4096 that are merged by binary search). Which rows are written is index work:
     exact. Two runs give the same bits."""
     torch.manual_seed(V * 7 + D)
     ids = torch.randint(0, V, (n, *Tshape))
