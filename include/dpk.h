@@ -430,6 +430,21 @@ int dpk_add_noise_multi(const void* const* summed /*host*/, void* const* grad /*
                         const int64_t* P /*host*/, int64_t K, int in_dtype, int out_dtype, float std,
                         float denom, uint64_t seed, uint64_t offset, int draws, dpk_stream_t stream);
 
+/* The whole DPOptimizer step of a small model in one launch: clip factors
+ * min(1, C / (sqrt(sum_k sumsq[k][i]) + 1e-6)) (optimizer.py:444-455), the clip-weighted sum over
+ * the batch (:456-475), the noise and the division (:477-504). Replaces the loop of
+ * DPOptimizer.clip_and_accumulate + add_noise + scale_grad for K <= DPK_MULTI_MAX parameters of
+ * 64 <= n <= 1024 samples. gs[k]: [n, P[k]] of `gs_dtype`; sumsq[k]: float[n], the squared norms of
+ * the rows of gs[k] (the samplers leave them); grad[k] (written) and summed[k] (nullable; the clipped
+ * sum before the noise) of `out_dtype`. Host arrays of K device pointers and sizes. Every block
+ * recomputes the n factors; sums, factors and noise are bit-identical to dpk_clip_factor on the
+ * stacked squared norms, dpk_clip_accumulate_multi in its small-tensor shape and
+ * dpk_add_noise_multi with the same (std, denom, seed, offset, draws), in that order. */
+int dpk_clip_noise_step(const void* const* gs /*host*/, const float* const* sumsq /*host*/, void* const* grad /*host*/,
+                        void* const* summed /*host, nullable*/, const int64_t* P /*host*/, int64_t K, int gs_dtype,
+                        int out_dtype, int64_t n, float max_grad_norm, float std, float denom, uint64_t seed,
+                        uint64_t offset, int draws, dpk_stream_t stream);
+
 /* out[p] = std * z[p]: the bare generator, for statistical tests. */
 int dpk_fill_normal(float* out, int64_t P, float std, uint64_t seed, uint64_t offset,
                     dpk_stream_t stream);

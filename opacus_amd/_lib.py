@@ -122,6 +122,9 @@ SIGNATURES = {
     "dpk_add_noise": (c_int, [_P, c_int, _P, c_int, _I, c_float, c_float, c_uint64, c_uint64, c_int, _P]),
     "dpk_clip_factor_per_layer": (c_int, [_P, _I, _I, c_int, _P, _P, _P]),
     "dpk_clip_accumulate_per_layer": (c_int, [_P, _P, _P, _I, c_int, c_int, _P, _I, c_int, _P]),
+    "dpk_clip_noise_step": (
+        c_int, [_P, _P, _P, _P, _P, _I, c_int, c_int, _I, c_float, c_float, c_float, c_uint64, c_uint64, c_int, _P]
+    ),
     "dpk_add_noise_multi": (
         c_int,
         [_P, _P, _P, _I, c_int, c_int, c_float, c_float, c_uint64, c_uint64, c_int, _P],

@@ -3,7 +3,10 @@
 // factor, and the clip-weighted sum over the batch. All HBM-bound; each reads
 // the n x P per-sample gradient tensor exactly once, with 16-byte accesses that
 // are contiguous across a wavefront, and reduces in a fixed order.
+#include <cstring>
+
 #include "dpk_common.h"
+#include "philox_normal.h"
 
 namespace {
 
@@ -219,6 +222,145 @@ __global__ __launch_bounds__(NT) void clip_accumulate_kernel(ClipArgs a, int64_t
     if (accumulate) acc.x += dpk_io<TO>::load(out);
     dpk_io<TO>::store(out, acc.x);
   }
+}
+
+// ---- a whole DPOptimizer step for a small model in one launch -------------------------------
+// clip factors from the per-parameter squared norms, the clip-weighted sum over the batch, the
+// noise and the division by the batch size (optimizer.py:444-504), for up to DPK_MULTI_MAX
+// tensors of at most kStepMaxN samples: every block recomputes the n factors into LDS (K * n
+// floats out of the cache), sums its columns exactly as clip_accumulate_kernel does with RS = 16
+// (same loop, same order of additions: the same bits), and carries them on through the noise add
+// of add_noise_kernel (noise.hip: the same Philox group per four elements, the same arithmetic)
+// into grad. The clipped sum itself is also stored when the caller wants it (summed[k] != NULL).
+// For a model of a few ten thousand parameters the step is bound by launches and host work:
+// this is one launch where there were four (stacked norms, factors, sum, noise).
+constexpr int kStepMaxN = 1024;
+constexpr int kStepRS = 16, kStepU = 8;
+
+struct StepArgs {
+  const void* gs[DPK_MULTI_MAX];
+  const float* sumsq[DPK_MULTI_MAX];  // float[n] per tensor
+  void* grad[DPK_MULTI_MAX];
+  void* summed[DPK_MULTI_MAX];        // nullable
+  int64_t P[DPK_MULTI_MAX];
+  int64_t gprefix[DPK_MULTI_MAX + 1];  // Philox groups before tensor k
+  uint32_t bprefix[DPK_MULTI_MAX + 1];  // blocks before tensor k
+  uint8_t vec[DPK_MULTI_MAX];           // tensor k in 4-element chunks
+  int K;
+};
+
+template <typename TG, typename TO, bool VEC>
+__device__ __forceinline__ void step_columns(const StepArgs& a, int k, int64_t n, const float* clip, float4* part,
+                                             float std, float denom, uint64_t seed, uint64_t offset, int draws) {
+  constexpr int W = VEC ? 4 : 1, RS = kStepRS, U = kStepU, CX = kThreads / RS;
+  const int64_t P = a.P[k];
+  const int64_t blk = blockIdx.x - a.bprefix[k];
+  const int cx = threadIdx.x % CX;
+  const int ry = threadIdx.x / CX;
+  const int64_t col = (blk * CX + cx) * W;
+  const bool live = col < P;
+  const TG* base = static_cast<const TG*>(a.gs[k]) + col;
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (live) {
+    int64_t r = ry;
+    for (; r + (U - 1) * RS < n; r += U * RS) {
+      float4 v[U];
+      float c[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const TG* p = base + (r + u * RS) * P;
+        if (VEC) {
+          v[u] = dpk_io<TG>::load4_nt(p);
+        } else {
+          v[u] = make_float4(dpk_io<TG>::load(p), 0.f, 0.f, 0.f);
+        }
+        c[u] = clip[r + u * RS];
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        acc.x = fmaf(c[u], v[u].x, acc.x);
+        if (VEC) {
+          acc.y = fmaf(c[u], v[u].y, acc.y);
+          acc.z = fmaf(c[u], v[u].z, acc.z);
+          acc.w = fmaf(c[u], v[u].w, acc.w);
+        }
+      }
+    }
+    for (; r < n; r += RS) {
+      const TG* p = base + r * P;
+      const float c = clip[r];
+      if (VEC) {
+        float4 v = dpk_io<TG>::load4(p);
+        acc.x = fmaf(c, v.x, acc.x);
+        acc.y = fmaf(c, v.y, acc.y);
+        acc.z = fmaf(c, v.z, acc.z);
+        acc.w = fmaf(c, v.w, acc.w);
+      } else {
+        acc.x = fmaf(c, dpk_io<TG>::load(p), acc.x);
+      }
+    }
+  }
+  part[threadIdx.x] = acc;
+  __syncthreads();
+  if (ry != 0 || !live) return;
+#pragma unroll
+  for (int j = 1; j < RS; ++j) {
+    float4 o = part[j * CX + cx];
+    acc.x += o.x;
+    acc.y += o.y;
+    acc.z += o.z;
+    acc.w += o.w;
+  }
+  // what summed_grad would hold: the sum rounded to the parameter's type
+  TO* summed = static_cast<TO*>(a.summed[k]);
+  TO* grad = static_cast<TO*>(a.grad[k]) + col;
+  const float inv = 1.0f / denom;
+  const bool exact_div = std == 0.f;
+  const uint64_t group = static_cast<uint64_t>(a.gprefix[k]) + static_cast<uint64_t>(col >> 2);
+  float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (std != 0.f) {
+    z = dpk_noise::noise4(group, seed, offset, draws);
+    z.x *= std;
+    z.y *= std;
+    z.z *= std;
+    z.w *= std;
+  }
+  if (VEC) {
+    if (sizeof(TO) == 2) {  // one rounding, as the stored sum has
+      acc.x = bf16_to_f32(f32_to_bf16(acc.x));
+      acc.y = bf16_to_f32(f32_to_bf16(acc.y));
+      acc.z = bf16_to_f32(f32_to_bf16(acc.z));
+      acc.w = bf16_to_f32(f32_to_bf16(acc.w));
+    }
+    if (summed) dpk_io<TO>::store4(summed + col, acc);
+    float4 v;
+    if (exact_div) v = make_float4(acc.x / denom, acc.y / denom, acc.z / denom, acc.w / denom);
+    else v = make_float4((acc.x + z.x) * inv, (acc.y + z.y) * inv, (acc.z + z.z) * inv, (acc.w + z.w) * inv);
+    dpk_io<TO>::store4(grad, v);
+  } else {
+    if (sizeof(TO) == 2) acc.x = bf16_to_f32(f32_to_bf16(acc.x));
+    if (summed) dpk_io<TO>::store(summed + col, acc.x);
+    const int e = static_cast<int>(col & 3);
+    const float ze = e == 0 ? z.x : e == 1 ? z.y : e == 2 ? z.z : z.w;
+    dpk_io<TO>::store(grad, exact_div ? acc.x / denom : (acc.x + ze) * inv);
+  }
+}
+
+template <typename TG, typename TO>
+__global__ __launch_bounds__(kThreads) void clip_noise_step_kernel(StepArgs a, int64_t n, float C, float std, float denom,
+                                                                    uint64_t seed, uint64_t offset, int draws) {
+  __shared__ float clip[kStepMaxN];
+  __shared__ float4 part[kThreads];
+  for (int64_t r = threadIdx.x; r < n; r += kThreads) {
+    float s = 0.f;
+    for (int k = 0; k < a.K; ++k) s += a.sumsq[k][r];  // (as clip_factor_kernel adds the rows of the stacked table)
+    clip[r] = fminf(C / (sqrtf(s) + 1e-6f), 1.0f);
+  }
+  __syncthreads();
+  int k = 0;
+  while (k + 1 < a.K && blockIdx.x >= a.bprefix[k + 1]) ++k;
+  if (a.vec[k]) step_columns<TG, TO, true>(a, k, n, clip, part, std, denom, seed, offset, draws);
+  else step_columns<TG, TO, false>(a, k, n, clip, part, std, denom, seed, offset, draws);
 }
 
 // The shape for very large tensors: a block owns kWideChunks * 256 consecutive 16-byte
@@ -591,4 +733,55 @@ extern "C" int dpk_clip_accumulate(const void* gs, int gs_dtype, const float* cl
                                    dpk_stream_t stream) {
   return dpk_clip_accumulate_multi(&gs, &summed, &P, 1, gs_dtype, out_dtype, clip, n, accumulate,
                                    stream);
+}
+
+// The whole step of a small model in one launch (see clip_noise_step_kernel): K <= DPK_MULTI_MAX
+// tensors, 64 <= n <= 1024 samples. Results are bit-identical to dpk_clip_factor on the stacked
+// sumsq rows + dpk_clip_accumulate_multi (in its small-tensor shape) + dpk_add_noise_multi.
+extern "C" int dpk_clip_noise_step(const void* const* gs, const float* const* sumsq, void* const* grad,
+                                   void* const* summed, const int64_t* P, int64_t K, int gs_dtype, int out_dtype,
+                                   int64_t n, float max_grad_norm, float std, float denom, uint64_t seed,
+                                   uint64_t offset, int draws, dpk_stream_t stream) {
+  const char* who = "dpk_clip_noise_step";
+  DPK_REQUIRE(gs && sumsq && grad && P, DPK_E_ARG, "%s: NULL pointer table", who);
+  DPK_REQUIRE(K >= 1 && K <= DPK_MULTI_MAX, DPK_E_SHAPE, "%s: K=%lld not in [1,%d]", who, (long long)K, DPK_MULTI_MAX);
+  DPK_REQUIRE(n >= 64 && n <= kStepMaxN, DPK_E_SHAPE, "%s: n=%lld not in [64,%d]", who, (long long)n, kStepMaxN);
+  DPK_REQUIRE(dpk_dtype_ok(gs_dtype) && dpk_dtype_ok(out_dtype), DPK_E_DTYPE, "%s: dtypes %d,%d", who, gs_dtype, out_dtype);
+  DPK_REQUIRE(draws == 1 || draws == 4, DPK_E_ARG, "%s: draws=%d (1 or 4)", who, draws);
+  DPK_REQUIRE(std >= 0.f && denom != 0.f, DPK_E_ARG, "%s: std=%g denom=%g", who, (double)std, (double)denom);
+  StepArgs a;
+  memset(&a, 0, sizeof(a));
+  a.K = static_cast<int>(K);
+  const size_t gneed = gs_dtype == DPK_BF16 ? 8 : 16, oneed = out_dtype == DPK_BF16 ? 8 : 16;
+  int64_t blocks = 0;
+  for (int k = 0; k < K; ++k) {
+    DPK_REQUIRE(P[k] >= 1, DPK_E_SHAPE, "%s: P[%d]=%lld", who, k, (long long)P[k]);
+    DPK_REQUIRE(gs[k] && sumsq[k] && grad[k], DPK_E_ARG, "%s: tensor %d is NULL", who, k);
+    DPK_REQUIRE(dpk_aligned(gs[k], dpk_elsize(gs_dtype)) && dpk_aligned(grad[k], dpk_elsize(out_dtype)) &&
+                    dpk_aligned(summed ? summed[k] : nullptr, dpk_elsize(out_dtype)) && dpk_aligned(sumsq[k], 4),
+                DPK_E_ALIGN, "%s: tensor %d misaligned", who, k);
+    a.gs[k] = gs[k];
+    a.sumsq[k] = sumsq[k];
+    a.grad[k] = grad[k];
+    a.summed[k] = summed ? summed[k] : nullptr;
+    a.P[k] = P[k];
+    const bool vec = P[k] % 4 == 0 && dpk_aligned(gs[k], gneed) && dpk_aligned(grad[k], oneed) &&
+                     dpk_aligned(a.summed[k], oneed);
+    a.vec[k] = vec ? 1 : 0;
+    a.gprefix[k + 1] = a.gprefix[k] + dpk_cdiv(P[k], 4);
+    blocks += dpk_cdiv(P[k], (kThreads / kStepRS) * (vec ? 4 : 1));
+    DPK_REQUIRE(blocks <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: too many blocks", who);
+    a.bprefix[k + 1] = static_cast<uint32_t>(blocks);
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
+#define DPK_STEP(TG, TO) \
+  hipLaunchKernelGGL((clip_noise_step_kernel<TG, TO>), grid, block, 0, s, a, n, max_grad_norm, std, denom, seed, offset, draws)
+  if (gs_dtype == DPK_F32 && out_dtype == DPK_F32) DPK_STEP(float, float);
+  else if (gs_dtype == DPK_BF16 && out_dtype == DPK_F32) DPK_STEP(bf16_t, float);
+  else if (gs_dtype == DPK_F32 && out_dtype == DPK_BF16) DPK_STEP(float, bf16_t);
+  else DPK_STEP(bf16_t, bf16_t);
+#undef DPK_STEP
+  DPK_LAUNCH_CHECK(who);
+  return DPK_OK;
 }

@@ -1009,8 +1009,11 @@ extern "C" size_t dpk_conv2d_gs_workspace_bytes(int64_t n, int64_t C, int64_t O,
   const int64_t Og = O / groups, Pg = (C / groups) * KH * KW;
   // the pieces of a split contraction (decided at call time from the device's size) need room
   // for their raw tiles; Q <= 0: the caller does not want the split
+  // (the current device's CU count, as the call will use it: ask on the device the call is made on)
   const Plan p = make_plan(Og, Pg, false);
-  const int pieces = Q > 0 ? split_pieces(n * groups * p.tiles_m * p.tiles_n, Q, 256) : 1;
+  int cus = dpk_device_cus();
+  if (cus <= 0) cus = 256;
+  const int pieces = Q > 0 ? split_pieces(n * groups * p.tiles_m * p.tiles_n, Q, cus) : 1;
   return conv_ws(n, Og, Pg, groups, O, pieces > 1 ? kSplitMax : 1).total;
 }
 
@@ -1080,9 +1083,14 @@ int conv_gs(const char* who, const void* x, const void* b, int in_dtype, void* g
   const int64_t blocks = n * groups * p.tiles_m * p.tiles_n;
   // few long blocks on the gather kernel: cut the contraction over the positions into pieces,
   // if the caller's workspace has room for their raw tiles
-  int ksplit = patch_bytes > 0 ? 1 : split_pieces(blocks, Q, dpk_device_cus());
-  const ConvWs wl = conv_ws(n, O / groups, Pg, groups, O, ksplit);
-  if (ksplit > 1 && !(ws && ws_bytes >= wl.total && dpk_aligned(ws, 256))) ksplit = 1;
+  int cus = dpk_device_cus();
+  if (cus <= 0) cus = 256;
+  int ksplit = patch_bytes > 0 ? 1 : split_pieces(blocks, Q, cus);
+  ConvWs wl = conv_ws(n, O / groups, Pg, groups, O, ksplit);
+  if (ksplit > 1 && !(ws && ws_bytes >= wl.total && dpk_aligned(ws, 256))) {
+    ksplit = 1;  // no room for the pieces: one piece, and the (smaller) layout that goes with it
+    wl = conv_ws(n, O / groups, Pg, groups, O, 1);
+  }
   const int kchunk = ksplit > 1 ? static_cast<int>(dpk_cdiv(dpk_cdiv(Q, ksplit), mf32::BK) * mf32::BK) : static_cast<int>(Q);
   DPK_REQUIRE(blocks * ksplit <= DPK_MAX_GRID_X, DPK_E_SHAPE, "%s: %lld blocks exceed the grid limit", who,
               (long long)(blocks * ksplit));

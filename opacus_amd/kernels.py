@@ -1090,6 +1090,45 @@ def add_noise_multi(
     return used
 
 
+CLIP_NOISE_STEP_MIN_N, CLIP_NOISE_STEP_MAX_N = 64, 1024
+
+
+def clip_noise_step(
+    gs_list: Sequence[torch.Tensor],
+    sumsq_list: Sequence[torch.Tensor],
+    grad_list: Sequence[torch.Tensor],
+    summed_list: Optional[Sequence[torch.Tensor]],
+    max_grad_norm: float,
+    std: float,
+    denom: float,
+    seed: int,
+    offset: int,
+    draws: int = 1,
+) -> None:
+    """The whole step of a small model in one launch: clip factors from the per-parameter squared
+    norms ``sumsq_list`` (``float32[n]`` each), ``summed_k = sum_n clip[n] * gs_k[n]`` (stored when
+    ``summed_list`` is given) and ``grad_k = (summed_k + std * z) / denom`` with the noise stream of
+    :func:`add_noise_multi`. At most ``DPK_MULTI_MAX`` tensors of 64 to 1024 samples; the results
+    are the bits that :func:`clip_factor`, :func:`clip_accumulate` and :func:`add_noise_multi` give."""
+    K = len(gs_list)
+    dev = _need_gpu(*gs_list, *sumsq_list, *grad_list)
+    n = gs_list[0].shape[0]
+    gdt, odt = gs_list[0].dtype, grad_list[0].dtype
+    gptrs = (ctypes.c_void_p * K)(*[t.data_ptr() for t in gs_list])
+    qptrs = (ctypes.c_void_p * K)(*[t.data_ptr() for t in sumsq_list])
+    optrs = (ctypes.c_void_p * K)(*[t.data_ptr() for t in grad_list])
+    sptrs = (ctypes.c_void_p * K)(*[t.data_ptr() for t in summed_list]) if summed_list is not None else None
+    sizes = (ctypes.c_int64 * K)(*[t.numel() for t in grad_list])
+    with _timed("clip_noise_step", dev):
+        check(
+            "dpk_clip_noise_step",
+            lib().dpk_clip_noise_step(
+                gptrs, qptrs, optrs, sptrs, sizes, K, _code(gdt), _code(odt), n, float(max_grad_norm), float(std),
+                float(denom), seed & 0xFFFFFFFFFFFFFFFF, offset & 0xFFFFFFFFFFFFFFFF, draws, _stream(dev),
+            ),
+        )
+
+
 def fill_normal(out: torch.Tensor, std: float, seed: int, offset: int) -> None:
     dev = _need_gpu(out)
     if out.dtype != torch.float32 or not out.is_contiguous():

@@ -355,6 +355,87 @@ class DPOptimizer(Optimizer):
             self.add_noise()
             self.scale_grad()
 
+    # ---- the whole step of a small model as one launch ----------------------------------------
+    FUSED_STEP_MAX_ELEMENTS = 1 << 20  # columns (in units of 4 where all tensors allow it) up to which it is used
+
+    def _fused_small_step(self) -> bool:
+        """clip_and_accumulate + add_noise + scale_grad as one kernel launch, when nothing about this
+        step needs them apart: flat clipping by this class's own rule, no virtual step pending or
+        behind, one device and dtype, per-sample gradients that still carry the squared norms their
+        samplers left, 64 to 1024 samples and few enough columns that the sum runs in its
+        small-tensor shape. ``p.grad`` and ``p.summed_grad`` hold the bits the three methods leave
+        (same kernels' arithmetic in the same order, same noise stream); they are views of two flat
+        buffers, one allocation each instead of one per parameter. Returns False when the step has
+        to take the separate methods."""
+        cls = type(self)
+        if (
+            cls.clip_and_accumulate is not DPOptimizer.clip_and_accumulate
+            or cls._clip_factors is not DPOptimizer._clip_factors
+            or cls.add_noise is not DPOptimizer.add_noise
+            or cls.scale_grad is not DPOptimizer.scale_grad
+            or self._check_skip_next_step(pop_next=False)
+        ):
+            return False
+        plist = self.params
+        if not plist or len(plist) > kernels.DPK_MULTI_MAX:
+            return False
+        flats, sumsqs = [], []
+        first = plist[0].grad_sample if hasattr(plist[0], "grad_sample") else None
+        if not isinstance(first, torch.Tensor) or not first.is_cuda:
+            return False
+        n, dev, gdt, odt = first.shape[0], first.device, first.dtype, plist[0].dtype
+        if not (kernels.CLIP_NOISE_STEP_MIN_N <= n <= kernels.CLIP_NOISE_STEP_MAX_N):
+            return False
+        if not (kernels.native_dtype(gdt) and kernels.native_dtype(odt)):
+            return False
+        total, vec = 0, True
+        for p in plist:
+            g = getattr(p, "grad_sample", None)
+            if (
+                not isinstance(g, torch.Tensor) or p.summed_grad is not None or hasattr(g, "_processed")
+                or g.device != dev or g.dtype != gdt or p.dtype != odt or g.shape[0] != n or not g.is_contiguous()
+                or g.numel() == 0
+            ):
+                return False
+            ss = cached_sumsq(g)
+            if ss is None or ss.device != dev:
+                return False
+            flats.append(g)
+            sumsqs.append(ss)
+            P = g.numel() // n
+            total += P
+            vec = vec and P % 4 == 0
+        if total // (4 if vec else 1) >= min(self.FUSED_STEP_MAX_ELEMENTS, 256 * 1024):
+            return False  # the separate kernels stream tensors of this size
+        # one buffer for the sums and one for the gradients, every parameter's piece at a multiple of 16 bytes
+        offs, at = [], 0
+        for g in flats:
+            offs.append(at)
+            at += -(-(g.numel() // n) // 8) * 8
+        flat_sum = torch.empty(at, device=dev, dtype=odt)
+        flat_grad = torch.empty(at, device=dev, dtype=odt)
+        summed = [flat_sum[o : o + g.numel() // n] for o, g in zip(offs, flats)]
+        grads = [flat_grad[o : o + g.numel() // n] for o, g in zip(offs, flats)]
+        if self._step_skip_queue:
+            self._step_skip_queue.pop(0)  # (False: checked above) this step's entry of the queue
+        std = self._noise_std()
+        denom = 1.0
+        if self.loss_reduction == "mean":
+            denom = float(self.expected_batch_size * self.accumulated_iterations)
+        if std == 0:
+            seed = offset = 0  # nothing is drawn and the generator stays where it is
+        else:
+            seed, offset = philox_stream(self.generator, dev, calls=1, secure=self.secure_mode)
+        kernels.clip_noise_step(
+            flats, sumsqs, grads, summed, float(self.max_grad_norm), std, denom, seed, offset, draws=4 if self.secure_mode else 1
+        )
+        for p, g, sm, gr in zip(plist, flats, summed, grads):
+            p.summed_grad = sm.view(p.shape)
+            p.grad = gr.view(p.shape)
+            _mark_as_processed(g)
+            _mark_as_processed(p.summed_grad)
+        return True
+
     def zero_grad(self, set_to_none: bool = False):
         """Clears ``p.grad``, ``p.grad_sample`` and, unless the last step was a skipped
         (virtual) one, ``p.summed_grad`` (optimizer.py:506-537)."""
@@ -369,11 +450,12 @@ class DPOptimizer(Optimizer):
         a skipped one that only accumulated (optimizer.py:539-563)."""
         if len(self.params) == 0:
             return True
-        self.clip_and_accumulate()
-        if self._check_skip_next_step():
-            self._is_last_step_skipped = True
-            return False
-        self._noise_and_scale()
+        if not self._fused_small_step():
+            self.clip_and_accumulate()
+            if self._check_skip_next_step():
+                self._is_last_step_skipped = True
+                return False
+            self._noise_and_scale()
         if self.step_hook:
             self.step_hook(self)
         self._is_last_step_skipped = False

@@ -62,10 +62,26 @@ class StepRecorder:
 class PrivacyEngine:
     """Attaches DP-SGD to a (module, optimizer, data loader) triple (privacy_engine.py:36-98)."""
 
-    def __init__(self, *, accountant: str = "prv", secure_mode: bool = False):
+    SECURE_MODE_URANDOM_PHILOX = "urandom-philox"
+
+    def __init__(self, *, accountant: str = "prv", secure_mode: Union[bool, str] = False):
         self.accountant = StepRecorder()
         self.accountant_mechanism = accountant
-        self.secure_mode = secure_mode
+        if secure_mode is True:
+            # The reference's secure mode is a cryptographically secure generator (torchcsprng) and it
+            # refuses to run without one (privacy_engine.py:86-96). None is available here, so the
+            # flag is refused too rather than honoured with something weaker; what this build can
+            # offer instead has to be asked for by name.
+            raise ImportError(
+                "secure_mode=True asks for a cryptographically secure random number generator (the reference "
+                "uses torchcsprng), which this build does not have. "
+                f"secure_mode={self.SECURE_MODE_URANDOM_PHILOX!r} selects what it does have: noise keys and the "
+                "sampling generator seeded from os.urandom (no seed reproduces them) and four summed draws per "
+                "value, on statistical generators (Philox4x32-10, MT19937)."
+            )
+        if secure_mode not in (False, self.SECURE_MODE_URANDOM_PHILOX):
+            raise ValueError(f"secure_mode must be False or {self.SECURE_MODE_URANDOM_PHILOX!r}, not {secure_mode!r}")
+        self.secure_mode = bool(secure_mode)
         self.secure_rng = None
         self.dataset = None
         if self.secure_mode:

@@ -57,6 +57,72 @@ def close(got, want, rtol, atol, msg=""):
     torch.testing.assert_close(got.detach().float().cpu(), want.detach().float().cpu(), rtol=rtol, atol=atol, msg=lambda m: f"{msg}: {m}")
 
 
+def test_small_model_step_in_one_launch_leaves_the_same_bits(A, monkeypatch):
+    """DPOptimizer.step of a small model runs clip factors, clipped sum, noise and scaling as one kernel
+    (optimizer.py:444-504 in one pass). p.grad and p.summed_grad must be bit for bit what the
+    separate kernels leave, with and without noise (same generator seed: same Philox stream), for a
+    parameter list with sizes that are and are not multiples of four; and virtual steps, which
+    need the sum kept apart from the noise, must still take the separate kernels."""
+    from opacus_amd.optimizers.optimizer import DPOptimizer
+
+    class Net(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.conv = nn.Conv2d(1, 6, 5, stride=2)
+            self.fc1 = nn.Linear(6 * 12 * 12, 33)
+            self.fc2 = nn.Linear(33, 10)
+
+        def forward(self, x):
+            return self.fc2(F.relu(self.fc1(F.relu(self.conv(x)).flatten(1))))
+
+    torch.manual_seed(11)
+    net = Net()
+    n = 96
+    x, y = torch.randn(n, 1, 28, 28).to(DEV), torch.randint(0, 10, (n,)).to(DEV)
+    used = []
+    real = DPOptimizer._fused_small_step
+
+    def run(sigma, fused, skip_first=False):
+        model = A.GradSampleModule(copy.deepcopy(net).to(DEV))
+        g = torch.Generator(device=DEV).manual_seed(1234)
+        opt = A.DPOptimizer(torch.optim.SGD(model.parameters(), lr=0.1), noise_multiplier=sigma, max_grad_norm=0.7,
+                            expected_batch_size=n, generator=g)
+        monkeypatch.setattr(DPOptimizer, "_fused_small_step", (lambda self: (used.append(real(self)), used[-1])[1]) if fused else (lambda self: False))
+        out = []
+        for step in range(2):
+            opt.zero_grad()
+            F.cross_entropy(model(x), y).backward()
+            if skip_first and step == 0:
+                opt.signal_skip_step(True)
+            else:
+                opt.signal_skip_step(False)
+            opt.step()
+            out.append([(p.grad.clone() if p.grad is not None else None, p.summed_grad.clone()) for p in model.parameters()])
+        return out, g.get_offset()
+
+    for sigma in (0.0, 1.3):
+        used.clear()
+        one, off1 = run(sigma, True)
+        assert used == [True, True]
+        sep, off2 = run(sigma, False)
+        assert off1 == off2  # the generator moved by the same amount
+        for s1, s2 in zip(one, sep):
+            for (g1, sm1), (g2, sm2) in zip(s1, s2):
+                assert torch.equal(g1, g2) and torch.equal(sm1, sm2)
+        if sigma:
+            assert not torch.equal(one[0][0][0], one[1][0][0])  # fresh noise every step
+    # a skipped (virtual) step and the step that follows it keep the sum apart: separate kernels
+    used.clear()
+    one, _ = run(1.3, True, skip_first=True)
+    assert used == [False, False]
+    sep, _ = run(1.3, False, skip_first=True)
+    for step, (s1, s2) in enumerate(zip(one, sep)):
+        for (g1, sm1), (g2, sm2) in zip(s1, s2):
+            assert torch.equal(sm1, sm2)
+            if step == 1:  # (after the skipped step p.grad is whatever autograd's own pass left)
+                assert torch.equal(g1, g2)
+
+
 # ---- models (down-scaled versions of the benchmark configurations) -----------------------------
 class SmallCNN(nn.Module):
     """Config 1: Conv(1,16,8,2,3) ReLU MaxPool Conv(16,32,4,2) ReLU MaxPool Linear(512,32) ReLU Linear(32,10)."""

@@ -837,10 +837,16 @@ def test_secure_mode_is_not_reproducible_from_any_seed():
     k2 = philox_stream(torch.Generator().manual_seed(3), dev)
     assert k1 == k2 and _NOISE_KEY_DOMAIN != 0
 
+    # the reference's flag asks for a CSPRNG, which is not there: refused as the reference refuses
+    # without torchcsprng (privacy_engine.py:86-96); the weaker mode has to be named
+    with pytest.raises(ImportError, match="urandom-philox"):
+        PrivacyEngine(secure_mode=True)
+    with pytest.raises(ValueError):
+        PrivacyEngine(secure_mode="yes")
     with pytest.warns(UserWarning, match="not cryptographically secure"):
-        e1 = PrivacyEngine(secure_mode=True)
+        e1 = PrivacyEngine(secure_mode="urandom-philox")
     with pytest.warns(UserWarning, match="os.urandom"):
-        e2 = PrivacyEngine(secure_mode=True)
+        e2 = PrivacyEngine(secure_mode=PrivacyEngine.SECURE_MODE_URANDOM_PHILOX)
     assert e1.secure_rng is not None and e1.secure_rng.initial_seed() != e2.secure_rng.initial_seed()
     net = nn.Linear(4, 2)
     sgd = torch.optim.SGD(net.parameters(), lr=0.1)
