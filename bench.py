@@ -732,6 +732,26 @@ def kernel_table(dev, iters: int = 10, warm: int = 3, with_cpu: bool = True):
     yield row("linear_weighted_sum_multi", "a9", "C5 all 29 Linear layers pooled, n=16 T=1024 bf16",
               timed(lambda: K.linear_weighted_sum_multi(items)), "mfma_bf16", sum(2.0 * n * T * i * o for i, o in layers))
     del items
+    # ... and C3's two layers pooled: too few tiles for the GPU, so the samples are cut into pieces inside the call
+    n, T = 32, 512
+    c = torch.rand(n, device=dev) * 0.9 + 0.1
+    items = [((torch.randn(n, T, o, device=dev) * 0.02).bfloat16(), torch.randn(n, T, i, device=dev).bfloat16(), c, 1.0)
+             for i, o in ((1024, 4096), (4096, 1024))]
+    yield row("linear_weighted_sum_multi", "a9", "C3 fc1 + fc2 pooled (two pieces), n=32 T=512 bf16",
+              timed(lambda: K.linear_weighted_sum_multi(items)), "mfma_bf16", 2 * 2.0 * n * T * 1024 * 4096)
+    yield row("linear_bias_weighted_sum", "a9", "C3 fc1 bias n=32 T=512 out=4096 bf16",
+              timed(lambda: K.linear_bias_weighted_sum(items[0][0], c)), "hbm", n * T * 4096 * 2)
+    del items
+    # fp32 operands: the direct-load fp32 kernel with the coefficients on its accumulators, and the weighted-row
+    # kernel for a sequence length that is not a whole number of k tiles
+    c = torch.rand(16, device=dev) * 0.9 + 0.1
+    a, b = torch.randn(16, 256, 1024, device=dev), torch.randn(16, 256, 1024, device=dev)
+    yield row("linear_weighted_sum (fp32)", "a9", "n=16 T=256 1024x1024 f32",
+              timed(lambda: K.linear_weighted_sum(b, a, c)), "mfma_fp32", 2.0 * 16 * 256 * 1024 * 1024)
+    a, b = torch.randn(16, 250, 1024, device=dev), torch.randn(16, 250, 1024, device=dev)
+    yield row("linear_weighted_sum (fp32, weighted rows)", "a9", "n=16 T=250 1024x1024 f32",
+              timed(lambda: K.linear_weighted_sum(b, a, c)), "mfma_fp32", 2.0 * 16 * 250 * 1024 * 1024)
+    del a, b
     # the same kernel on fp32 operands
     tri, full = tri_tiles(1024)
     a = torch.randn(16, 1024, 2048, device=dev)
@@ -757,6 +777,9 @@ def kernel_table(dev, iters: int = 10, warm: int = 3, with_cpu: bool = True):
     yield row("embedding_ghost_norm", "a5", "C5 n=16 T=1024 D=2048 bf16", timed(lambda: K.embedding_ghost_norm(ids, b)),
               "hbm", b.numel() * 2 + ids.numel() * 8,
               cpu(lambda: O.embedding_norm_sample(cids, cb), 4, "4 of 16 samples"))
+    cw = torch.rand(n, device=dev) * 0.9 + 0.1
+    yield row("embedding_weighted_sum", "a9", "C5 n=16 T=1024 V=32000 D=2048 bf16",
+              timed(lambda: K.embedding_weighted_sum(ids, b, cw, V)), "hbm", b.numel() * 2 + V * D * 2 + ids.numel() * 8)
     yield row("rms_norm_gs", "a6", "C5 n=16 T=1024 D=2048 bf16", timed(lambda: K.rms_norm_grad_sample(x, b, D, 1e-5)),
               "hbm", 2 * b.numel() * 2, cpu(lambda: O.rms_norm_grad_sample(cx, cb, (D,), 1e-5), 4, "4 of 16 samples"))
     ah = torch.randn(n, T, D, device=dev).bfloat16()
@@ -812,6 +835,14 @@ def kernel_table(dev, iters: int = 10, warm: int = 3, with_cpu: bool = True):
     yield row("conv2d_gs", "a3", "C1 conv2 n=256 16->32 k4 s2 f32",
               timed(lambda: K.conv2d_grad_sample(x, b, (4, 4), (2, 2), (0, 0, 0, 0), (1, 1), 1)), "mfma_fp32",
               2.0 * n * 32 * 256 * 25)
+    # ---- C1: the whole optimizer step of the small CNN as one launch (factors, clipped sum, noise, scaling)
+    sizes = [1024, 16, 8192, 32, 16384, 32, 320, 10]
+    gsl = [torch.randn(n, P, device=dev) for P in sizes]
+    ssl = [g.pow(2).sum(1) for g in gsl]
+    grl = [torch.empty(P, device=dev) for P in sizes]
+    sml = [torch.empty(P, device=dev) for P in sizes]
+    yield row("clip_noise_step", "a10+a11", "C1 n=256 P=26010 (8 tensors) f32",
+              timed(lambda: K.clip_noise_step(gsl, ssl, grl, sml, 1.0, 1.1, 256.0, 1, 0)), "hbm", (n + 2) * sum(sizes) * 4)
 
 
 def run_workload(name: str, dev, steps: int, warmup: int, all_timers: bool = False, calibrate_copy: bool = False,
