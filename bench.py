@@ -261,12 +261,12 @@ def workload_c1(dev, autograd_weight_grads=False):
     return _hooks_workload(
         dev, SmallCNN(), torch.randn(n, 1, 28, 28), torch.randint(0, 10, (n,)), n, 1.1,
         "Small CNN (conv 1->16 k8 s2 p3, conv 16->32 k4 s2, fc 512->32, fc 32->10) fp32, batch 256, hooks, C=1, sigma=1.1",
-        dict(kernel="clip_accumulate_kernel<float,float,*,RS=16> (8 tensors, one launch)", timer="clip_accumulate",
-             bound="hbm", work_per_launch=float(n * P * 4 + P * 4), unit="GB/s", peak=HBM_PEAK_GBS,
-             # scaled with the copy kernel's factor (FETCH_SIZE x 2.000); this kernel's short row pieces may be
-             # fetched in requests the counter sizes correctly, in which case the true figure is half
-             traffic=53396593,
-             traffic_source="recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of bench.py --workload c1, profiles/clip_accumulate_small_cnn_b256_hbm_traffic.txt (not re-measured by this run)"),
+        # the optimizer's whole step on the eight parameter tensors as one launch: reads every per-sample
+        # gradient once (n*P*4), writes the noised gradient and the clipped sum (2*P*4)
+        dict(kernel="clip_noise_step_kernel<float,float> (clip factors, clipped sum, noise and scaling of all 8 tensors, one launch)",
+             timer="clip_noise_step", bound="hbm", work_per_launch=float(n * P * 4 + 2 * P * 4), unit="GB/s", peak=HBM_PEAK_GBS,
+             traffic=26995456,
+             traffic_source="recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of bench.py --workload c1, profiles/clip_noise_step_small_cnn_b256_hbm_traffic.txt (not re-measured by this run)"),
         autograd_weight_grads=autograd_weight_grads,
     )
 
@@ -281,7 +281,7 @@ def workload_c4(dev, autograd_weight_grads=False):
         dict(kernel="conv2d_gs_patch_kernel<64,64,float,float>", timer="conv2d_gs", bound="mfma",
              work_per_launch=flops, unit="TFLOP/s", peak=MFMA_FP32_PEAK_TFLOPS,
              # inputs 134.2 MB + per-sample gradients 37.7 MB = 172.0 MB must move once
-             traffic=174364893,
+             traffic=174340597,
              traffic_source="recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of bench.py --workload c4, profiles/conv2d_gs_resblock_b256_hbm_traffic.txt (not re-measured by this run)"),
         autograd_weight_grads=autograd_weight_grads,
     )
@@ -317,8 +317,9 @@ def _ghost_workload(dev, net, make_inputs, loss_call, n, T, sigma, desc, single=
         return plain_step
 
     flops = ghost_executed_flops(net, n, T)
-    ghost = dict(kernel="ghost_norm_multi_kernel<128x128, 2 stages> (all Linear layers of a step pooled into one launch; thin layers by linear_dlds_kernel; "
-                        "ghost_norm_bf16_dlds_kernel layer by layer with two backward passes)",
+    ghost = dict(kernel="ghost_norm_multi_kernel<128x128, 2 stages> (all Linear layers of a step pooled into one launch, the units "
+                        "past the last whole round of resident blocks each cut into four pieces along the contraction; thin layers "
+                        "by linear_dlds_kernel; ghost_norm_bf16_dlds_kernel layer by layer with two backward passes)",
                  timer="linear_ghost_norm", bound="mfma", work_per_step=flops, unit="TFLOP/s",
                  peak=MFMA_BF16_PEAK_TFLOPS, traffic=traffic, **({"traffic_source": traffic_source} if traffic else {}))
     out = dict(
@@ -330,8 +331,9 @@ def _ghost_workload(dev, net, make_inputs, loss_call, n, T, sigma, desc, single=
         # with one backward pass the clipped sums are this library's kernel too, and the longer of the two
         wsum_flops = sum(2.0 * n * T * m.in_features * m.out_features for m in net.modules() if isinstance(m, nn.Linear))
         out["roofline"] = dict(
-            kernel="linear_wsum_multi_kernel<256x256> (clip-weighted sums of all Linear layers in one pooled launch; "
-                   "linear_dlds_kernel<.., weighted> layer by layer, cut into pieces, for a small pool)",
+            kernel="linear_wsum_multi_kernel<256x256> (clip-weighted sums of all Linear layers in one pooled launch; a pool "
+                   "with fewer tiles than resident blocks is cut into pieces of samples whose fp32 partial sums "
+                   "add_pieces_multi_kernel adds, and the time covers both kernels)",
             timer="linear_weighted_sum", bound="mfma", work_per_step=wsum_flops, unit="TFLOP/s", peak=MFMA_BF16_PEAK_TFLOPS,
             traffic=wsum_traffic, **({"traffic_source": wsum_traffic_source} if wsum_traffic else {}))
         out["roofline_also"] = {"roofline_ghost_norm": ghost}
@@ -357,11 +359,12 @@ def workload_c3(dev, single=True):
         "MLP Linear(1024->4096) GELU Linear(4096->1024), bf16, batch 32, T=512, ghost clipping, C=1, sigma=1",
         single=single, plain_loss=lambda ref, x: PerSampleMSE("mean")(ref(x)),
         # HBM bytes of the pooled launch (operands of both layers: 335.5 MB must be read once)
-        traffic=367683253 if single else None,
+        traffic=367228187 if single else None,
         traffic_source="recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of bench.py --workload c3, profiles/ghost_norm_multi_mlp_b32_t512_hbm_traffic.txt (not re-measured by this run)",
-        # per launch (one layer: 167.8 MB of operands read once, 67.1 MB of fp32 piece sums written)
-        wsum_traffic=319111020,
-        wsum_traffic_source="recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of bench.py --workload c3, profiles/weighted_sum_mlp_b32_t512_hbm_traffic.txt (not re-measured by this run)",
+        # the pooled launch and the kernel that adds its pieces: 335.5 MB of operands read once, 67.1 MB of
+        # fp32 piece sums written and read again, 16.8 MB of bf16 results written
+        wsum_traffic=553920016,
+        wsum_traffic_source="recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of bench.py --workload c3, profiles/weighted_sum_multi_mlp_b32_t512_hbm_traffic.txt (not re-measured by this run)",
     )
 
 
@@ -388,13 +391,13 @@ def workload_c5(dev, tied=False, single=True):
         # HBM bytes of the pooled launch (21 layers by the Gram route; their operands, 5.21 GB, must be
         # read once; a unit streams two 128-row blocks of both operands and the 4 MB L2 of an XCD does not
         # hold a sample's rows of the wide layers, so the units re-fetch from the last-level cache)
-        traffic=11823073150 if single and not tied else None,
+        traffic=11340730370 if single and not tied else None,
         traffic_source="recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of bench.py --workload c5, "
                        "profiles/ghost_norm_multi_llama_b16_t1024_hbm_traffic.txt (not re-measured by this run)",
         # the pooled launch: 5.88 GB of operands and 0.49 GB of results must move once; a tile streams 256
         # columns of both operands over all 16384 rows, and the narrow operand of a layer (67 MB, which
         # stays in the 256 MB last-level cache) is fetched again by every row of tiles
-        wsum_traffic=14198920269 if not tied else None,
+        wsum_traffic=14199424257 if not tied else None,
         wsum_traffic_source="recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of bench.py --workload c5, "
                             "profiles/weighted_sum_multi_llama_b16_t1024_hbm_traffic.txt (not re-measured by this run)",
     )
