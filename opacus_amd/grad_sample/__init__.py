@@ -9,6 +9,7 @@ from .grad_sample_module_fast_gradient_clipping import (
     GradSampleModuleFastGradientClipping,
 )
 from .gsm_base import AbstractGradSampleHooks, AbstractGradSampleModule
+from .lazy import LazyLinearGradSample
 from .utils import (
     get_gsm_class,
     get_hooks_class,
@@ -38,6 +39,7 @@ __all__ = [
     "GradSampleHooksFastGradientClipping",
     "AbstractGradSampleModule",
     "AbstractGradSampleHooks",
+    "LazyLinearGradSample",
     "register_grad_sampler",
     "register_norm_sampler",
     "create_or_accumulate_grad_sample",

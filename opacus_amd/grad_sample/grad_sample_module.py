@@ -33,6 +33,7 @@ from ..utils.module_utils import (
 )
 from .. import kernels
 from ._common import tag_sumsq
+from .lazy import LazyLinearGradSample, lazy_linear_grad_sample
 from .functorch import ft_compute_per_sample_gradient, prepare_layer
 from .gsm_base import AbstractGradSampleHooks, AbstractGradSampleModule
 
@@ -94,7 +95,16 @@ def create_or_accumulate_grad_sample(
     """
     if not param.requires_grad:
         return
+    if isinstance(grad_sample, LazyLinearGradSample):
+        # kept as factors only as the pass's one full-batch result for this parameter
+        if not hasattr(param, "_current_grad_sample") and grad_sample.shape[0] == max_batch_len:
+            param._current_grad_sample = grad_sample
+            return
+        grad_sample = grad_sample.materialize()
+        adopt = True  # the tensor was formed for this parameter alone
     if hasattr(param, "_current_grad_sample"):
+        if isinstance(param._current_grad_sample, LazyLinearGradSample):
+            param._current_grad_sample = param._current_grad_sample.materialize()
         param._current_grad_sample[: grad_sample.shape[0]] += grad_sample
     elif adopt and grad_sample.shape[0] == max_batch_len:
         param._current_grad_sample = grad_sample
@@ -175,7 +185,15 @@ class GradSampleHooks(AbstractGradSampleHooks):
     such a layer stays as it was (``None`` after ``zero_grad``), which a caller that reads
     ``p.grad`` between ``backward()`` and ``step()`` must know; the switch also changes
     ``requires_grad`` inside forward, so it is not for models whose forward runs concurrently
-    from several threads."""
+    from several threads.
+
+    ``lazy_linear_grad_sample=True`` (off by default; the reference has no such option) leaves
+    ``weight.grad_sample`` of every ``nn.Linear`` served by the library's own sampler as a
+    :class:`~opacus_amd.grad_sample.lazy.LazyLinearGradSample`: the layer's activations and
+    backprops instead of the ``[n, out, in]`` tensor they define (grad_sample/linear.py:41-48).
+    ``DPOptimizer`` takes the per-sample norms and the clipped sum from the factors; whoever else
+    reads the attribute gets the tensor, formed at that moment. ``isinstance(p.grad_sample,
+    torch.Tensor)`` is false for such a parameter until then."""
 
     GRAD_SAMPLERS = {}
     # ghost clipping needs autograd's weight gradients in its second pass
@@ -192,8 +210,10 @@ class GradSampleHooks(AbstractGradSampleHooks):
         strict: bool = True,
         force_functorch=False,
         autograd_weight_grads: Optional[bool] = None,
+        lazy_linear_grad_sample: bool = False,
     ):
         super().__init__(m, batch_first=batch_first, loss_reduction=loss_reduction)
+        self.lazy_linear_grad_sample = bool(lazy_linear_grad_sample)
         errors = self.validate(module=m, strict=strict)
         if errors and not strict:
             logger.info(f"Validation found the following errors: {errors}. Using non-strict mode, continuing")
@@ -364,7 +384,10 @@ class GradSampleHooks(AbstractGradSampleHooks):
             activations, backprops = stacked
             for p in trainable_parameter_list(module):
                 p._forward_counter += 1  # taken off again below, as for a module used once
-        grad_samples = call_sampler(sampler, module, activations, backprops, scale)
+        if self._keeps_factors(module, sampler, backprops):
+            grad_samples = lazy_linear_grad_sample(module, activations, backprops, scale)
+        else:
+            grad_samples = call_sampler(sampler, module, activations, backprops, scale)
         adopt = getattr(sampler, "owns_output", False)
         for param, gs in grad_samples.items():
             create_or_accumulate_grad_sample(
@@ -383,6 +406,20 @@ class GradSampleHooks(AbstractGradSampleHooks):
                     )
         if len(module.activations) == 0:
             module.__dict__.pop("max_batch_len", None)
+
+    def _keeps_factors(self, module: nn.Module, sampler: Callable, backprops: torch.Tensor) -> bool:
+        """Whether this use of ``module`` is filed as activations and backprops
+        (``lazy_linear_grad_sample``): an ``nn.Linear`` itself, served by the library's sampler
+        (a sampler the user registered for it must run), in a dtype the kernels contract."""
+        return (
+            getattr(self, "lazy_linear_grad_sample", False)
+            and type(module) is nn.Linear
+            and not self.force_functorch
+            and _runs_on_kernels(sampler)
+            and backprops.is_cuda
+            and kernels.native_dtype(backprops.dtype)
+            and backprops.shape[0] > 0
+        )
 
     def _stack_uses(self, module: nn.Module, activations: List[torch.Tensor], backprops: torch.Tensor):
         """For a module applied many times per forward pass (``stack_uses``, the RNNLinear
@@ -492,6 +529,7 @@ class GradSampleModule(GradSampleHooks, AbstractGradSampleModule):
         strict: bool = True,
         force_functorch=False,
         autograd_weight_grads: Optional[bool] = None,
+        lazy_linear_grad_sample: bool = False,
     ):
         nn.Module.__init__(self)
         GradSampleHooks.__init__(
@@ -502,6 +540,7 @@ class GradSampleModule(GradSampleHooks, AbstractGradSampleModule):
             strict=strict,
             force_functorch=force_functorch,
             autograd_weight_grads=autograd_weight_grads,
+            lazy_linear_grad_sample=lazy_linear_grad_sample,
         )
         self.grad_accumulation_hook = None
 

@@ -27,6 +27,7 @@ from torch.optim import Optimizer
 
 from .. import kernels
 from ..grad_sample._common import cached_sumsq
+from ..grad_sample.lazy import LazyLinearGradSample
 from .utils import params
 
 logger = logging.getLogger(__name__)
@@ -38,7 +39,7 @@ _OFFSET_PER_CALL = 4
 
 def _mark_as_processed(obj: Union[torch.Tensor, List[torch.Tensor]]):
     """Flags gradients as consumed by a step so that using them twice is caught (optimizer.py:32-58)."""
-    if isinstance(obj, torch.Tensor):
+    if isinstance(obj, (torch.Tensor, LazyLinearGradSample)):
         obj._processed = True
     elif isinstance(obj, list):
         for x in obj:
@@ -46,7 +47,7 @@ def _mark_as_processed(obj: Union[torch.Tensor, List[torch.Tensor]]):
 
 
 def _check_processed_flag_tensor(x: torch.Tensor):
-    if hasattr(x, "_processed"):
+    if "_processed" in getattr(x, "__dict__", ()):
         raise ValueError(
             "Gradients haven't been cleared since the last optimizer step. "
             "In order to obtain privacy guarantees you must call optimizer.zero_grad()"
@@ -55,7 +56,7 @@ def _check_processed_flag_tensor(x: torch.Tensor):
 
 
 def _check_processed_flag(obj: Union[torch.Tensor, List[torch.Tensor]]):
-    if isinstance(obj, torch.Tensor):
+    if isinstance(obj, (torch.Tensor, LazyLinearGradSample)):
         _check_processed_flag_tensor(obj)
     elif isinstance(obj, list):
         for x in obj:
@@ -150,15 +151,19 @@ class DPOptimizer(Optimizer):
             p.summed_grad = None
 
     # ---- per-sample gradient access -----------------------------------------------------
-    def _get_flat_grad_sample(self, p: torch.Tensor):
+    def _get_flat_grad_sample(self, p: torch.Tensor, factors_ok: bool = False):
         """``p.grad_sample`` as one tensor; a list from several backward passes is
-        concatenated along the batch (optimizer.py:252-292)."""
+        concatenated along the batch (optimizer.py:252-292). A Linear weight's gradient that is
+        still held as its two factors (``lazy_linear_grad_sample``) is returned as it is to a caller
+        that says it can work from them, and formed for any other."""
         if not hasattr(p, "grad_sample"):
             raise ValueError("Per sample gradient not found. Are you using GradSampleModule?")
         if p.grad_sample is None:
             raise ValueError("Per sample gradient is not initialized. Not updated in backward pass?")
         if isinstance(p.grad_sample, torch.Tensor):
             return p.grad_sample
+        if isinstance(p.grad_sample, LazyLinearGradSample):
+            return p.grad_sample if factors_ok else p.grad_sample.materialize()
         if isinstance(p.grad_sample, list):
             return torch.cat(p.grad_sample, dim=0)
         raise ValueError(f"Unexpected grad_sample type: {type(p.grad_sample)}")
@@ -189,7 +194,7 @@ class DPOptimizer(Optimizer):
         for p in self.params:
             if not hasattr(p, "grad_sample"):
                 raise ValueError("Per sample gradient not found. Are you using GradSampleModule?")
-            if isinstance(p.grad_sample, torch.Tensor):
+            if isinstance(p.grad_sample, (torch.Tensor, LazyLinearGradSample)):
                 vals.add(1)
             elif isinstance(p.grad_sample, list):
                 vals.add(len(p.grad_sample))
@@ -237,7 +242,10 @@ class DPOptimizer(Optimizer):
         rows: List[Optional[torch.Tensor]] = []
         missing: Dict[Tuple[torch.dtype, torch.device], List[int]] = {}
         for k, (p, g) in enumerate(zip(plist, flats)):
-            ss = cached_sumsq(p.grad_sample) if isinstance(p.grad_sample, torch.Tensor) else None
+            if isinstance(g, LazyLinearGradSample):
+                ss = g.sumsq  # closed form or Gram contraction of the factors
+            else:
+                ss = cached_sumsq(p.grad_sample) if isinstance(p.grad_sample, torch.Tensor) else None
             rows.append(ss)
             if ss is None:
                 missing.setdefault((g.dtype, g.device), []).append(k)
@@ -264,7 +272,7 @@ class DPOptimizer(Optimizer):
         flats = []
         for p in plist:
             _check_processed_flag(p.grad_sample)
-            g = self._get_flat_grad_sample(p)
+            g = self._get_flat_grad_sample(p, factors_ok=True)
             if not kernels.supported_dtype(g.dtype):
                 raise TypeError(f"per-sample gradients must be float32 or bfloat16 on this path, got {g.dtype}")
             flats.append(g)
@@ -274,6 +282,15 @@ class DPOptimizer(Optimizer):
         groups: Dict[tuple, List[int]] = {}
         for k, (p, g) in enumerate(zip(plist, flats)):
             out_dtype = p.dtype if kernels.supported_dtype(p.dtype) else torch.float32
+            if isinstance(g, LazyLinearGradSample):
+                # a Linear weight held as activations and backprops: its clipped sum is one
+                # contraction over samples and positions with the clip factors as coefficients
+                total = g.weighted_sum((clip[k] if per_layer else clip).to(g.device), out_dtype=out_dtype)
+                if p.summed_grad is None:
+                    p.summed_grad = total
+                else:
+                    p.summed_grad += total
+                continue
             if p.summed_grad is None:
                 p.summed_grad = torch.empty(g.shape[1:], device=g.device, dtype=out_dtype)
                 fresh = True

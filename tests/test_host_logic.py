@@ -1025,3 +1025,51 @@ def test_bench_refuses_more_than_one_gpu():
     done = subprocess.run([sys.executable, str(bench), "--gpus", "2"], capture_output=True, text=True, timeout=120)
     assert done.returncode != 0
     assert "one GPU" in (done.stdout + done.stderr)
+
+
+def test_lazy_linear_grad_sample_answers_what_it_can_without_the_tensor(monkeypatch):
+    """The stand-in for a Linear weight's per-sample gradient (grad_sample/linear.py:41-48 kept as its
+    two factors): shape questions, the optimizer's processed flag and the hooks' filing must not
+    form the [n, out, in] tensor; a second result for the same parameter in one pass must."""
+    from opacus_amd.grad_sample import grad_sample_module as gsm
+    from opacus_amd.grad_sample.lazy import LazyLinearGradSample
+    from opacus_amd.optimizers import optimizer as optmod
+
+    formed = []
+
+    def fake_materialize(self):
+        formed.append(self)
+        if self._gs is None:
+            self._gs = self._scale * torch.einsum("n...i,n...j->nij", self._b, self._a)
+        return self._gs
+
+    monkeypatch.setattr(LazyLinearGradSample, "materialize", fake_materialize)
+    b, a = torch.randn(5, 3, 4), torch.randn(5, 3, 6)
+    lz = LazyLinearGradSample(b, a, scale=2.0)
+    assert lz.shape == (5, 4, 6) and len(lz) == 5 and lz.dim() == 3 and lz.numel() == 120 and lz.size(1) == 4
+    assert lz.dtype == torch.float32 and lz.device.type == "cpu" and "factors only" in repr(lz)
+    optmod._check_processed_flag(lz)
+    optmod._mark_as_processed(lz)
+    with pytest.raises(ValueError, match="haven't been cleared"):
+        optmod._check_processed_flag(lz)
+    p = nn.Parameter(torch.zeros(4, 6))
+    gsm.create_or_accumulate_grad_sample(param=p, grad_sample=lz, max_batch_len=5)
+    assert p._current_grad_sample is lz and not formed
+    # everything else is the tensor's business
+    want = 2.0 * torch.einsum("nti,ntj->nij", b, a)
+    torch.testing.assert_close(torch.stack([lz])[0], want)
+    assert formed
+    torch.testing.assert_close(lz.flatten(1).sum(1), want.flatten(1).sum(1))
+    torch.testing.assert_close((lz * 2)[1], 2 * want[1])
+    # a second use of the layer in the same pass adds into the first: both formed
+    other = LazyLinearGradSample(torch.randn(5, 3, 4), torch.randn(5, 3, 6))
+    first = LazyLinearGradSample(b, a, scale=2.0)
+    q = nn.Parameter(torch.zeros(4, 6))
+    gsm.create_or_accumulate_grad_sample(param=q, grad_sample=first, max_batch_len=5)
+    gsm.create_or_accumulate_grad_sample(param=q, grad_sample=other, max_batch_len=5)
+    assert isinstance(q._current_grad_sample, torch.Tensor)
+    torch.testing.assert_close(q._current_grad_sample, want + torch.einsum("nti,ntj->nij", other._b, other._a))
+    # a batch shorter than the longest of the pass goes into the zero-filled buffer as before
+    r = nn.Parameter(torch.zeros(4, 6))
+    gsm.create_or_accumulate_grad_sample(param=r, grad_sample=LazyLinearGradSample(b[:3], a[:3]), max_batch_len=5)
+    assert r._current_grad_sample.shape == (5, 4, 6) and not r._current_grad_sample[3:].any()
