@@ -179,6 +179,18 @@ def test_noise_stream_virtual_steps_and_per_layer_clipping(A):
     for k in pe:
         assert_rel(pl[k], pe[k], 1e-5, f"per-layer clipping, {k}")
 
+    from functools import partial
+
+    from opacus_amd.optimizers import AdaClipDPOptimizer
+
+    ada = partial(AdaClipDPOptimizer, target_unclipped_quantile=0.5, clipbound_learning_rate=0.2, max_clipbound=10.0,
+                  min_clipbound=0.01, unclipped_num_std=1.0)
+    me, _, ae, _ = one_step(A, net, x, loss_of, lazy=False, opt_cls=ada, C=0.4)
+    ml, kept, al, _ = one_step(A, net, x, loss_of, lazy=True, opt_cls=ada, C=0.4)
+    assert not kept["fc1.weight"].is_materialized
+    for k in ae:
+        assert_rel(al[k], ae[k], 1e-5, f"adaptive clipping, {k}")
+
 
 def test_layers_the_option_does_not_take(A):
     """A Linear used twice in one forward pass sums its uses (grad_sample_module.py:58-59): formed at
