@@ -383,7 +383,7 @@ GHOST_ROUTES = [0, 1, 2]  # DPK_ROUTE_AUTO, DPK_ROUTE_GRAM, DPK_ROUTE_DIRECT
     + [(3, 200, 256, 16), (2, 130, 8, 520)]  # thin layers: the direct route by choice
     # feature sizes that are multiples of 32: the direct-load kernel on fp32 operands (route "gram")
     + [(3, 200, 64, 96), (2, 300, 160, 288), (5, 1000, 32, 64)]
-    # ... with a tail of quadrant blocks: few units (all quadrants), 576 units (512 whole tiles + 256 quadrants)
+    # ... with a tail cut into pieces along k: few units (all in pieces), 576 units (512 whole tiles + 64 units in 4 pieces each)
     + [(2, 256, 512, 256), (3, 150, 64, 64), (16, 1000, 64, 128)],
 )
 @pytest.mark.parametrize("scale", [1.0, 4.0])
@@ -417,13 +417,13 @@ def test_linear_ghost_norm_f32(K, n, T, fin, fout, scale, route):
         (16, [(1000, 64, 128, True, True), (1000, 128, 64, True, True), (520, 192, 64, True, False)]),
         # 5 samples: XCDs with one sample and XCDs with none
         (5, [(256, 128, 128, True, True), (256, 64, 256, True, True)]),
-        # 32 samples, 10 + 10 tile pairs each: 80 units per XCD = one round of 64 and a tail of 16 cut into quadrants
+        # 32 samples, 10 + 10 tile pairs each: 80 units per XCD = one round of 64 and a tail of 16 cut into pieces along k
         (32, [(512, 64, 128, True, True), (512, 128, 64, True, True)]),
     ],
 )
 def test_linear_ghost_norm_multi_matches_layer_by_layer(K, dtype, n, layers):
     """All layers of a pass in one call (the tile pairs of every layer share the launch, longest
-    first, the tail in quadrant blocks) against the float64 oracle and against one call per layer."""
+    first, the tail as pieces along k) against the float64 oracle and against one call per layer."""
     torch.manual_seed(n * 31 + len(layers))
     items, wants, singles = [], [], []
     for T, fin, fout, want_w, want_b in layers:
@@ -711,12 +711,12 @@ def test_linear_ghost_norm_2d_inputs(K):
         (3, 2, 8, 16),
         (2, 70, 40, 24),
         (2, 200, 136, 264),
-        (2, 256, 1024, 512),  # direct-to-LDS kernel, few units: every unit cut into quadrant blocks
+        (2, 256, 1024, 512),  # direct-to-LDS kernel, few units: every unit cut into pieces along k
         (3, 33, 30, 18),
-        (3, 150, 64, 64),  # quadrants that start beyond T
-        (3, 200, 64, 128),  # quadrants with a few valid rows
+        (3, 150, 64, 64),  # tail pieces of tiles that reach beyond T
+        (3, 200, 64, 128),  # tail pieces with a few valid rows
         (20, 640, 64, 64),  # 300 units on a 256-CU device: whole-tile blocks only
-        (16, 1000, 64, 128),  # 576 units: 512 whole-tile blocks and a tail of quadrant blocks, ragged T
+        (16, 1000, 64, 128),  # 576 units: 512 whole-tile blocks and a tail in pieces, ragged T
         (4, 512, 1024, 16),  # a low-rank adapter: thin on one side
         (4, 512, 16, 1024),
     ],

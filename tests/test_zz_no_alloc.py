@@ -14,7 +14,7 @@ pytestmark = pytest.mark.gpu
 
 FP32_REL = 1e-5
 
-# (n, T, out, in, dtype, route): Gram route with whole-tile and quadrant blocks, the direct
+# (n, T, out, in, dtype, route): Gram route with whole-tile blocks and tail pieces, the direct
 # route (which also keeps the column sums of b in the buffer), fp32 and bf16, T == 1
 FIRST_THEN_SMALLER = [
     ((16, 1000, 64, 128, torch.bfloat16, 0), (3, 150, 64, 64, torch.bfloat16, 0)),
