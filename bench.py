@@ -757,17 +757,25 @@ def kernel_table(dev, iters: int = 10, warm: int = 3, with_cpu: bool = True):
     c = torch.rand(n, device=dev) * 0.9 + 0.1
     items = [((torch.randn(n, T, o, device=dev) * 0.02).bfloat16(), torch.randn(n, T, i, device=dev).bfloat16(), c, 1.0)
              for i, o in ((1024, 4096), (4096, 1024))]
+    cpu_items = [(bb[:1].cpu().float(), aa[:1].cpu().float()) for bb, aa, _, _ in items]
+    cc = c[:1].cpu()
     yield row("linear_weighted_sum_multi", "a9", "C3 fc1 + fc2 pooled (two pieces), n=32 T=512 bf16",
-              timed(lambda: K.linear_weighted_sum_multi(items)), "mfma_bf16", 2 * 2.0 * n * T * 1024 * 4096)
+              timed(lambda: K.linear_weighted_sum_multi(items)), "mfma_bf16", 2 * 2.0 * n * T * 1024 * 4096,
+              cpu(lambda: [torch.einsum("n,nij->ij", cc, O.linear_grad_sample(aa, bb)[0]) for bb, aa in cpu_items], n,
+                  f"1 of {n} samples, both layers, fp32 einsum + weighted sum"))
     yield row("linear_bias_weighted_sum", "a9", "C3 fc1 bias n=32 T=512 out=4096 bf16",
-              timed(lambda: K.linear_bias_weighted_sum(items[0][0], c)), "hbm", n * T * 4096 * 2)
+              timed(lambda: K.linear_bias_weighted_sum(items[0][0], c)), "hbm", n * T * 4096 * 2,
+              cpu(lambda: torch.einsum("n,ni->i", cc, O.linear_grad_sample(cpu_items[0][1], cpu_items[0][0])[1]), n,
+                  f"1 of {n} samples, fp32 sum over positions + weighted sum"))
     del items
     # fp32 operands: the direct-load fp32 kernel with the coefficients on its accumulators, and the weighted-row
     # kernel for a sequence length that is not a whole number of k tiles
     c = torch.rand(16, device=dev) * 0.9 + 0.1
     a, b = torch.randn(16, 256, 1024, device=dev), torch.randn(16, 256, 1024, device=dev)
+    ca, cb, cc = a[:4].cpu(), b[:4].cpu(), c[:4].cpu()
     yield row("linear_weighted_sum (fp32)", "a9", "n=16 T=256 1024x1024 f32",
-              timed(lambda: K.linear_weighted_sum(b, a, c)), "mfma_fp32", 2.0 * 16 * 256 * 1024 * 1024)
+              timed(lambda: K.linear_weighted_sum(b, a, c)), "mfma_fp32", 2.0 * 16 * 256 * 1024 * 1024,
+              cpu(lambda: torch.einsum("n,nij->ij", cc, O.linear_grad_sample(ca, cb)[0]), 4, "4 of 16 samples, einsum + weighted sum"))
     a, b = torch.randn(16, 250, 1024, device=dev), torch.randn(16, 250, 1024, device=dev)
     yield row("linear_weighted_sum (fp32, weighted rows)", "a9", "n=16 T=250 1024x1024 f32",
               timed(lambda: K.linear_weighted_sum(b, a, c)), "mfma_fp32", 2.0 * 16 * 250 * 1024 * 1024)
@@ -798,8 +806,11 @@ def kernel_table(dev, iters: int = 10, warm: int = 3, with_cpu: bool = True):
               "hbm", b.numel() * 2 + ids.numel() * 8,
               cpu(lambda: O.embedding_norm_sample(cids, cb), 4, "4 of 16 samples"))
     cw = torch.rand(n, device=dev) * 0.9 + 0.1
+    ccw = cw[:1].cpu()
     yield row("embedding_weighted_sum", "a9", "C5 n=16 T=1024 V=32000 D=2048 bf16",
-              timed(lambda: K.embedding_weighted_sum(ids, b, cw, V)), "hbm", b.numel() * 2 + V * D * 2 + ids.numel() * 8)
+              timed(lambda: K.embedding_weighted_sum(ids, b, cw, V)), "hbm", b.numel() * 2 + V * D * 2 + ids.numel() * 8,
+              cpu(lambda: torch.einsum("n,nvd->vd", ccw, O.embedding_grad_sample(cids[:1], cb[:1].float(), V)), n,
+                  f"1 of {n} samples, per-sample table + weighted sum"))
     yield row("rms_norm_gs", "a6", "C5 n=16 T=1024 D=2048 bf16", timed(lambda: K.rms_norm_grad_sample(x, b, D, 1e-5)),
               "hbm", 2 * b.numel() * 2, cpu(lambda: O.rms_norm_grad_sample(cx, cb, (D,), 1e-5), 4, "4 of 16 samples"))
     ah = torch.randn(n, T, D, device=dev).bfloat16()
