@@ -251,3 +251,40 @@ def test_full_size_headline_layer(A):
         want = ((coef[:, None] * b.double()).t() @ x.double()) / n
     assert_rel(model._module.weight.grad, want, 1e-5, "weight.grad at full size")
     assert_rel(gs.sumsq, b.double().pow(2).sum(1) * x.double().pow(2).sum(1), 1e-5, "closed-form squared norms")
+
+
+def test_through_make_private_with_poisson_batches(A):
+    """A module wrapped by the caller with the option on goes through ``PrivacyEngine.make_private``
+    as any pre-wrapped module does (privacy_engine.py:171-183); Poisson batches of varying and zero
+    length train, and the weights end up where the materialising run leaves them (same seeds, sigma 0)."""
+    from torch.utils.data import DataLoader, TensorDataset
+
+    def run(lazy):
+        torch.manual_seed(21)
+        net = MLP().to(DEV)
+        wrapped = A.GradSampleModule(net, lazy_linear_grad_sample=lazy)
+        ds = TensorDataset(torch.randn(40, 96), torch.randint(0, 10, (40,)))
+        dl = DataLoader(ds, batch_size=4)
+        engine = A.PrivacyEngine()
+        model, opt, loader = engine.make_private(
+            module=wrapped, optimizer=torch.optim.SGD(net.parameters(), lr=0.1), data_loader=dl, noise_multiplier=0.0,
+            max_grad_norm=0.5, poisson_sampling=True,
+        )
+        assert model is wrapped
+        torch.manual_seed(22)  # the sampler's draws
+        sizes = []
+        for x, y in loader:
+            opt.zero_grad()
+            if len(x):
+                F.cross_entropy(model(x.to(DEV)), y.to(DEV)).backward()
+            else:
+                model(x.to(DEV)).sum().backward()
+            sizes.append(len(x))
+            opt.step()
+        return sizes, [p.detach().clone() for p in net.parameters()]
+
+    sizes_e, we = run(False)
+    sizes_l, wl = run(True)
+    assert sizes_e == sizes_l and len(set(sizes_e)) > 1
+    for a, b in zip(wl, we):
+        assert_rel(a, b, 1e-5, "weights after an epoch of Poisson batches")
